@@ -1,0 +1,257 @@
+#!/usr/bin/env python3
+"""Benchmark of the int8 quantized-GEMM inference path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only gemm|gemv|ln|softmax]
+
+One "step" is one pass of the path over the north-star workload: activations A fp16
+[1,4096,4096] ~N(0,1) and weights W fp16 [1,10240,4096] ~N(0,0.02) (seed 1000, generated on
+the CPU and resident in HBM before timing) through ``bmm(A, False, W, True, int8=True)`` --
+row-absmax scales and int8 rounding of both operands, int8 MFMA GEMM with int32 accumulation,
+fp16 dequantisation -- exactly what the reference's GEMMInt8.forward does per call.
+
+Prints ONE JSON line.  `value` is 2*M*N*K / step time in TOP/s for that whole step; the
+`roofline` object is the GEMM kernel alone against the dense int8 MFMA peak; `components`
+carries the decode GEMV, layernorm and softmax kernels against the HBM peak; `cpu_baseline`
+is the torch formulation of the same step timed on the host cores (a reported baseline).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_INT8_TOPS = 5000.0      # MI355X dense int8 MFMA, published
+PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, published
+M, K, N = 4096, 4096, 10240  # north-star GEMM
+
+
+def parse():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=50)
+    p.add_argument("--warmup", type=int, default=10)
+    p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    p.add_argument("--only", default="", help="run only one kernel loop (for profiling): gemm|gemv|ln|softmax|pipeline")
+    p.add_argument("--reps", type=int, default=200, help="launches per timed batch in the per-kernel loops")
+    return p.parse_args()
+
+
+def event_ms(fn, reps, warmup=3):
+    """Average milliseconds per call of fn over `reps` back-to-back calls, from HIP events on
+    torch's current stream (the stream every launcher is given)."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / reps
+
+
+def graph_ms(launches, reps):
+    """Capture the list of launch closures once into a HIP graph (no host launch overhead
+    between kernels) and time `reps` replays; returns ms per launch.  Falls back to eager
+    timing if capture is unavailable."""
+    import torch
+    try:
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            for f in launches:
+                f()
+        torch.cuda.current_stream().wait_stream(s)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for f in launches:
+                f()
+        g.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / (reps * len(launches)), "hipgraph"
+    except Exception as ex:   # pragma: no cover
+        sys.stderr.write("graph capture failed (%s); eager timing\n" % ex)
+        i = [0]
+
+        def one():
+            launches[i[0] % len(launches)]()
+            i[0] += 1
+        return event_ms(one, reps * len(launches)), "eager"
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        sys.stderr.write("bench.py measures one GPU: the path has no collectives and every GPU box of this "
+                         "build has a single MI355X; --gpus %d is not supported\n" % args.gpus)
+        sys.exit(2)
+    import torch
+    from cpm_kernels_amd.build import library_path, build_library
+    if not os.path.exists(library_path()):
+        build_library(verbose=False)
+    from cpm_kernels_amd.library import cpmk
+    import cpm_kernels_amd.kernels as ck
+    import cpm_kernels_amd.torch as ct
+    assert cpmk.lib.loaded, "libcpmk_hip.so missing"
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    dev = torch.device("cuda:0")
+    st = lambda: torch.cuda.current_stream().cuda_stream   # noqa: E731
+    only = args.only
+    result = {}
+
+    # ---- north-star workload ---------------------------------------------------------------
+    g = torch.Generator().manual_seed(1000)
+    A_cpu = torch.randn(1, M, K, generator=g).half()
+    W_cpu = (torch.randn(1, N, K, generator=g) * 0.02).half()
+    A, W = A_cpu.to(dev), W_cpu.to(dev)
+    ops = 2.0 * M * N * K
+
+    step_ms = None
+    if only in ("", "pipeline"):
+        def step():
+            return ct.bmm(A, False, W, True, int8=True)
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            step()
+        e1.record()
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        step_ms = max(e0.elapsed_time(e1) / args.steps, 0.0)
+        result["wall_ms_per_step"] = round(wall_ms, 4)
+
+    # ---- GEMM kernel alone (roofline) ------------------------------------------------------
+    roofline = None
+    if only in ("", "gemm"):
+        sA = torch.empty((1, M), dtype=torch.half, device=dev); qA = torch.empty((1, M, K), dtype=torch.int8, device=dev)
+        sW = torch.empty((1, N), dtype=torch.half, device=dev); qW = torch.empty((1, N, K), dtype=torch.int8, device=dev)
+        ck.gemm_quantize(1, M, K, A.data_ptr(), sA.data_ptr(), qA.data_ptr(), False, st())
+        ck.gemm_quantize(1, N, K, W.data_ptr(), sW.data_ptr(), qW.data_ptr(), False, st())
+        out16 = torch.empty((1, M, N), dtype=torch.half, device=dev)
+
+        def gemm():
+            ck.gemm_int8_scale(N, K, M, 1, 1, True, False, qW.data_ptr(), qA.data_ptr(), sA.data_ptr(), sW.data_ptr(),
+                               True, True, out16.data_ptr(), st())
+        ms = event_ms(gemm, max(20, args.steps), warmup=max(3, args.warmup))
+        tops = ops / (ms * 1e-3) / 1e12
+        roofline = {"kernel": "k_gemm_kmajor (int8 MFMA GEMM + fused fp16 dequant), M=%d K=%d N=%d" % (M, K, N),
+                    "bound": "mfma", "achieved": round(tops, 2), "peak": PEAK_INT8_TOPS, "unit": "TFLOP/s",
+                    "ops": "int8 multiply-accumulates counted as 2 ops (TOP/s)",
+                    "frac": round(tops / PEAK_INT8_TOPS, 4), "avg_kernel_us": round(ms * 1e3, 2), "traffic": None}
+        out32 = torch.empty((1, M, N), dtype=torch.int32, device=dev)
+
+        def gemm32():
+            ck.gemm_int8(N, K, M, 1, 1, True, False, qW.data_ptr(), qA.data_ptr(), out32.data_ptr(), st())
+        ms32 = event_ms(gemm32, max(20, args.steps), warmup=3)
+        roofline["int32_out_tops"] = round(ops / (ms32 * 1e-3) / 1e12, 2)
+        del out32
+
+    # ---- HBM-bound components ---------------------------------------------------------------
+    components = {}
+    reps = args.reps
+
+    def hbm(name, nbytes, ms, how, shape):
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        components[name] = {"shape": shape, "algorithmic_bytes": int(nbytes), "avg_us": round(ms * 1e3, 3),
+                            "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                            "frac": round(gbs / PEAK_HBM_GBS, 4), "timing": how}
+
+    if only in ("", "gemv"):
+        # config 2: W int8 [10240,4096], 32 vectors; 8 weight copies (336 MB) rotate so every
+        # launch streams its matrix from HBM, not from the 256 MB Infinity Cache
+        gg = torch.Generator().manual_seed(1002)
+        nrot = 8
+        mats = [torch.randint(-127, 128, (10240, 4096), generator=gg, dtype=torch.int8).to(dev) for _ in range(nrot)]
+        smat = (torch.rand(10240, generator=gg) * 0.009 + 0.001).half().to(dev)
+        v = torch.randn(32, 4096, generator=gg).half().to(dev)
+        sv = torch.empty((32,), dtype=torch.half, device=dev); qv = torch.empty((32, 4096), dtype=torch.int8, device=dev)
+        ck.gemv_calc_scale(32, 4096, v.data_ptr(), sv.data_ptr(), st())
+        ck.gemv_round(32, 4096, v.data_ptr(), sv.data_ptr(), qv.data_ptr(), st())
+        o = torch.empty((32, 10240), dtype=torch.half, device=dev)
+        launches = [(lambda m_=m_: ck.gemv_broadcast_mat_int8(32, 10240, 4096, smat.data_ptr(), m_.data_ptr(), sv.data_ptr(),
+                                                               qv.data_ptr(), o.data_ptr(), st())) for m_ in mats]
+        ms, how = graph_ms(launches, max(5, reps // nrot))
+        hbm("gemv_broadcast_mat_int8", 10240 * 4096 + 32 * 4096 + 2 * 32 * 10240 + 2 * 10240 + 2 * 32, ms, how,
+            "W int8 [10240,4096] x 32 vectors")
+        del mats
+
+    if only in ("", "ln"):
+        gg = torch.Generator().manual_seed(1003)
+        nrot = 10    # 10 x 33.5 MB inputs
+        xs = [torch.randn(8, 4096, 512, generator=gg).half().to(dev) for _ in range(nrot)]
+        y = torch.empty_like(xs[0])
+        launches = [(lambda x_=x_: ck.layernorm_forward(8, 4096, 512, x_.data_ptr(), y.data_ptr(), 1e-5, True, st()))
+                    for x_ in xs]
+        ms, how = graph_ms(launches, max(5, reps // nrot))
+        hbm("layernorm_forward", 4 * 8 * 4096 * 512, ms, how, "[8,4096,512] fp16, dim 1")
+        del xs
+
+    if only in ("", "softmax"):
+        gg = torch.Generator().manual_seed(1003)
+        s = (torch.randn(64, 1024, 1024, generator=gg) * 4).half()
+        kk = torch.arange(1024)[:, None]; qq = torch.arange(1024)[None, :]
+        s.masked_fill_((kk > qq)[None], float("-inf"))
+        sd = s.to(dev).repeat(8, 1, 1).contiguous()          # [512,1024,1024], 1.07 GB
+        del s
+        so = torch.empty_like(sd)
+        launches = [lambda: ck.softmax_forward(512, 1024, 1024, sd.data_ptr(), so.data_ptr(), st())]
+        ms, how = graph_ms(launches, max(3, reps // 20))
+        hbm("softmax_forward", 4 * 512 * 1024 * 1024, ms, how, "[512,1024,1024] fp16 causal, dim 1")
+        del sd, so
+
+    # ---- CPU baseline: torch formulation of the same step on the host cores ------------------
+    cpu = None
+    if not args.no_cpu and only == "":
+        from oracle.formulations import quant_bmm_rowwise
+        ncores = os.cpu_count() or 1
+        torch.set_num_threads(ncores)
+        quant_bmm_rowwise(A_cpu[:, :256], W_cpu[:, :256])      # warm the thread pool
+        times = []
+        t_begin = time.perf_counter()
+        while len(times) < 3 and time.perf_counter() - t_begin < 25.0:
+            t0 = time.perf_counter()
+            quant_bmm_rowwise(A_cpu, W_cpu)
+            times.append(time.perf_counter() - t0)
+        best = sorted(times)[len(times) // 2]
+        cpu = {"value": round(ops / best / 1e12, 4), "unit": "TOP/s", "cores": torch.get_num_threads(),
+               "kind": "port", "seconds_per_step": round(best, 3),
+               "sample": "full north-star step (fp32 fake-quant of A and W + fp32 matmul), median of %d runs" % len(times)}
+
+    value = ops / (step_ms * 1e-3) / 1e12 if step_ms else None
+    line = {
+        "metric": "int8 quant-GEMM TOPS + GEMV/LN/softmax HBM GB/s (frac of peak) at 1 GPU",
+        "value": round(value, 2) if value else None, "unit": "TOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(step_ms, 4) if step_ms else None,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8 (int32 accumulate, fp16 in/out)", "data": "synthetic",
+        "config": {"workload": "north-star int8 quant-GEMM M=4096 K=4096 N=10240: bmm(A[1,4096,4096] fp16, "
+                               "W[1,10240,4096] fp16, int8=True) = quantise A and W, int8 MFMA GEMM, fp16 dequant",
+                   "seed": 1000},
+        "roofline": roofline, "cpu_baseline": cpu, "components": components,
+        "device": torch.cuda.get_device_name(0),
+    }
+    line.update(result)
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

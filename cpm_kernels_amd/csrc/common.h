@@ -1,0 +1,123 @@
+// Shared device/host helpers for the gfx950 kernels of libcpmk_hip.so.
+// Everything here assumes 64-wide wavefronts (CDNA); nothing is written for 32-lane warps.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "../../include/cpmk.h"
+
+namespace cpmk {
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef int32_t int4_t __attribute__((ext_vector_type(4)));
+typedef int32_t int2_t __attribute__((ext_vector_type(2)));
+typedef int32_t int16_tv __attribute__((ext_vector_type(16)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+
+__host__ __device__ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---- wave64 reductions (butterfly over all 6 lane bits) -----------------------------
+__device__ inline float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+    return v;
+}
+__device__ inline float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    return v;
+}
+__device__ inline int32_t wave_sum_i32(int32_t v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    return v;
+}
+
+// Block-wide reductions for blocks of NWAVES*64 threads.  `red` is LDS scratch of at least
+// NWAVES floats.  Every thread returns the reduced value.  Contains two barriers so the
+// scratch can be reused by the next call.
+template <int NWAVES>
+__device__ inline float block_max(float v, float* red) {
+    v = wave_max(v);
+    if (NWAVES == 1) return v;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    if (lane == 0) red[w] = v;
+    __syncthreads();
+    float r = red[0];
+#pragma unroll
+    for (int i = 1; i < NWAVES; ++i) r = fmaxf(r, red[i]);
+    __syncthreads();
+    return r;
+}
+template <int NWAVES>
+__device__ inline float block_sum(float v, float* red) {
+    v = wave_sum(v);
+    if (NWAVES == 1) return v;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    if (lane == 0) red[w] = v;
+    __syncthreads();
+    float r = red[0];
+#pragma unroll
+    for (int i = 1; i < NWAVES; ++i) r += red[i];
+    __syncthreads();
+    return r;
+}
+
+// ---- quantisation arithmetic ---------------------------------------------------------
+// absmax/127 rounded to fp16.  The reference divides in double and converts
+// double->float->half (cuda/gemm.cu:74); for every fp16 magnitude that equals the
+// correctly rounded fp32 divide used here (checked exhaustively by the CPU tests).
+__device__ inline half_t scale_from_absmax(float mx) { return (half_t)(mx / 127.0f); }
+
+// int8( rint( x / s ) ): IEEE fp32 divide, round-half-even (cuda/gemm.cu:16).  Values that do
+// not fit int8 (reachable only with a subnormal fp16 scale) saturate and NaN (0/0 for an
+// all-zero row) gives 0; the reference's float->int8_t cast is undefined behaviour there.
+__device__ inline int32_t quant_i8(float x, float s) {
+    const float d = x / s;
+    float q = __builtin_rintf(d);
+    q = fminf(fmaxf(q, -128.0f), 127.0f);   // fmaxf/fminf drop a NaN operand ...
+    return (d != d) ? 0 : (int32_t)q;       // ... so map NaN to 0 explicitly
+}
+
+__device__ inline uint32_t pack4_i8(int32_t a, int32_t b, int32_t c, int32_t d) {
+    return (uint32_t)(a & 0xff) | ((uint32_t)(b & 0xff) << 8) | ((uint32_t)(c & 0xff) << 16) |
+           ((uint32_t)d << 24);
+}
+
+// fp32 -> fp16 of a value that must first exist as a rounded fp32 number.  Without the
+// register barrier the compiler folds "convert(multiply)" into v_fma_mixlo_f16, which rounds
+// the exact product once, straight to fp16; the reference rounds to fp32 and then to fp16
+// (cuda/gemm.cu:55), and the two differ on about one product in 10^4.
+__device__ inline half_t round_f16(float v) {
+    asm("" : "+v"(v));
+    return (half_t)v;
+}
+
+// dequantising epilogue of cu_gemm_scale (cuda/gemm.cu:55): two fp32 multiplies in this order.
+__device__ inline half_t dequant(int32_t acc, float sx, float sy) {
+    return round_f16(((float)acc * sx) * sy);
+}
+
+// ---- host-side launch helpers ----------------------------------------------------------
+inline int launch_status() { return (int)hipGetLastError(); }
+
+// Map a linear workgroup index so that consecutive logical tiles land on the same XCD.
+// Workgroups are dealt round-robin to the 8 XCDs of an MI355X (workgroup i -> XCD i % 8),
+// each XCD has its own L2; tiles that share cache lines should therefore share an XCD.
+__device__ inline uint32_t xcd_remap(uint32_t bid, uint32_t nblocks) {
+    constexpr uint32_t kXcd = 8;
+    const uint32_t per = nblocks / kXcd;          // tiles per XCD in the remappable part
+    const uint32_t lim = per * kXcd;
+    if (bid >= lim) return bid;                   // ragged tail keeps its index
+    return (bid % kXcd) * per + bid / kXcd;
+}
+
+}  // namespace cpmk

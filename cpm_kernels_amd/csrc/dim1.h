@@ -1,0 +1,92 @@
+// Register-resident column tiles for reductions over dim 1 of a (batch, n, m) fp16 tensor.
+//
+// The reference walks such tensors with 32x32 thread blocks, 64-byte row segments and two or
+// three passes over global memory (cuda/layernorm.cu:6-71, cuda/softmax.cu:6-43).  Here one
+// workgroup of NT threads owns all n rows of LPR*8 adjacent columns and keeps them in
+// registers, so HBM is read once and written once:
+//   lane -> (cg = tid % LPR, rg = tid / LPR); pass p covers rows p*(NT/LPR) + rg;
+//   each lane holds R 16-byte pieces (8 columns of R rows).
+// Reductions run per lane, then over the lanes of a wave that share cg (xor butterflies on
+// the lane bits above log2(LPR)), then over waves through a few hundred bytes of LDS.
+#pragma once
+#include "common.h"
+
+namespace cpmk {
+
+template <int NT, int LPR, int R>
+struct ColTile {
+    static constexpr int RPP = NT / LPR;       // rows per pass
+    static constexpr int ROWS = RPP * R;       // rows the tile can hold
+    static constexpr int COLS = LPR * 8;
+    static constexpr int NW = NT / 64;
+    // LDS floats needed by reduce<NV>: (NW + 1) * COLS * NV
+};
+
+// Load the tile; rows >= n and columns >= m are left as `fill` in every half.
+template <int NT, int LPR, int R>
+__device__ inline void coltile_load(half8_t (&v)[R], const half_t* base, int32_t n, int32_t m, int32_t col0,
+                                    half_t fill) {
+    constexpr int RPP = NT / LPR;
+    const int rg = threadIdx.x / LPR;
+#pragma unroll
+    for (int p = 0; p < R; ++p) {
+        const int32_t row = p * RPP + rg;
+        half8_t x;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = fill;
+        if (row < n && col0 < m)
+            x = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(base + (int64_t)row * m + col0));
+        v[p] = x;
+    }
+}
+
+template <int NT, int LPR, int R>
+__device__ inline void coltile_store(const half8_t (&v)[R], half_t* base, int32_t n, int32_t m, int32_t col0) {
+    constexpr int RPP = NT / LPR;
+    const int rg = threadIdx.x / LPR;
+#pragma unroll
+    for (int p = 0; p < R; ++p) {
+        const int32_t row = p * RPP + rg;
+        if (row < n && col0 < m)
+            __builtin_nontemporal_store(v[p], reinterpret_cast<half8_t*>(base + (int64_t)row * m + col0));
+    }
+}
+
+// Reduce NV groups of 8 per-lane column partials over all rows of the tile.  On return every
+// lane holds the totals of its own 8 columns.  `lds` must hold (NT/64 + 1) * LPR*8 * NV floats.
+template <int NT, int LPR, int NV, bool IS_MAX>
+__device__ inline void coltile_reduce(float (&v)[NV * 8], float* lds) {
+    constexpr int NW = NT / 64, COLS = LPR * 8, W = COLS * NV;
+#pragma unroll
+    for (int o = LPR; o < 64; o <<= 1) {
+#pragma unroll
+        for (int e = 0; e < NV * 8; ++e) {
+            const float t = __shfl_xor(v[e], o, kWave);
+            v[e] = IS_MAX ? fmaxf(v[e], t) : v[e] + t;
+        }
+    }
+    if (NW == 1) return;
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    if (lane < LPR) {
+#pragma unroll
+        for (int g = 0; g < NV; ++g)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) lds[w * W + g * COLS + lane * 8 + e] = v[g * 8 + e];
+    }
+    __syncthreads();
+    if (tid < W) {
+        float r = lds[tid];
+#pragma unroll
+        for (int i = 1; i < NW; ++i) r = IS_MAX ? fmaxf(r, lds[i * W + tid]) : r + lds[i * W + tid];
+        lds[NW * W + tid] = r;
+    }
+    __syncthreads();
+    const int cg = tid % LPR;
+#pragma unroll
+    for (int g = 0; g < NV; ++g)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[g * 8 + e] = lds[NW * W + g * COLS + cg * 8 + e];
+    __syncthreads();
+}
+
+}  // namespace cpmk

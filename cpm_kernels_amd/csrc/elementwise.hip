@@ -1,0 +1,168 @@
+// Streaming fp16 kernels: GELU, per-channel affine, residual add, padding mask.
+// One 16-byte load/store per lane wherever the shape allows it.
+#include "common.h"
+
+namespace cpmk {
+
+// cuda/gelu.cu:14 evaluates, with double-precision literals,
+//   0.5 * x * (1.0 + tanhf(0.7978845608028654 * x * (1.0 + 0.044715 * x * x)))
+// i.e. the tanh argument and the final product are formed in double, tanhf in float.
+__device__ inline half_t gelu1(half_t h) {
+    const float x = (float)h;
+    const double xd = (double)x;
+    const float u = (float)(0.7978845608028654 * xd * (1.0 + 0.044715 * xd * xd));
+    const float r = (float)(0.5 * xd * (1.0 + (double)tanhf(u)));
+    return (half_t)r;
+}
+
+__global__ __launch_bounds__(256) void k_gelu(int64_t total, const half_t* mat, half_t* out, int vec) {
+    const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (vec) {
+        const int64_t e0 = gid * 8;
+        if (e0 + 8 <= total) {
+            half8_t v = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(mat + e0));
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = gelu1(v[e]);
+            __builtin_nontemporal_store(v, reinterpret_cast<half8_t*>(out + e0));
+        } else {
+            for (int64_t i = e0; i < total; ++i) out[i] = gelu1(mat[i]);
+        }
+    } else if (gid < total) {
+        out[gid] = gelu1(mat[gid]);
+    }
+}
+
+// out[b,i,:] = fma(x, alpha[i], beta[i]) (HAS_BETA) or x * alpha[i], fp16 arithmetic
+// (cuda/arith.cu:97-127).  rows = batch*n, channel = row % n.
+template <bool HAS_BETA>
+__global__ __launch_bounds__(256) void k_ln_affine(int64_t total, int32_t n, int32_t m, const half_t* x,
+                                                   const half_t* __restrict__ alpha,
+                                                   const half_t* __restrict__ beta, half_t* out, int vec) {
+    const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t e0 = vec ? gid * 8 : gid * 2;       // m % 2 == 0 (vec: m % 8 == 0)
+    if (e0 >= total) return;
+    const int32_t ch = (int32_t)((e0 / m) % n);
+    const half_t a = alpha[ch];
+    const half_t b = HAS_BETA ? beta[ch] : (half_t)0.0f;
+    if (vec) {
+        half8_t v = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(x + e0));
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = HAS_BETA ? __builtin_fmaf16(v[e], a, b) : (half_t)(v[e] * a);
+        __builtin_nontemporal_store(v, reinterpret_cast<half8_t*>(out + e0));
+    } else {
+        half2_t v = *reinterpret_cast<const half2_t*>(x + e0);
+#pragma unroll
+        for (int e = 0; e < 2; ++e) v[e] = HAS_BETA ? __builtin_fmaf16(v[e], a, b) : (half_t)(v[e] * a);
+        *reinterpret_cast<half2_t*>(out + e0) = v;
+    }
+}
+
+__global__ __launch_bounds__(256) void k_add(int64_t total, const half_t* x, const half_t* y, half_t* out, int vec) {
+    const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (vec) {
+        const int64_t e0 = gid * 8;
+        if (e0 + 8 <= total) {
+            half8_t a = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(x + e0));
+            half8_t b = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(y + e0));
+            __builtin_nontemporal_store(a + b, reinterpret_cast<half8_t*>(out + e0));
+        } else {
+            for (int64_t i = e0; i < total; ++i) out[i] = x[i] + y[i];
+        }
+    } else if (gid < total) {
+        out[gid] = x[gid] + y[gid];
+    }
+}
+
+// out[b,i,j] = mask[b,j] == 0 ? value : x[b,i,j]      (cuda/mask.cu:6-23)
+__global__ __launch_bounds__(256) void k_mask(int64_t total, int32_t n, int32_t m, const half_t* x,
+                                              const int8_t* __restrict__ mask, half_t value, half_t* out, int vec) {
+    const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t e0 = vec ? gid * 8 : gid;
+    if (e0 >= total) return;
+    const int64_t row = e0 / m;
+    const int32_t j = (int32_t)(e0 - row * m);
+    const int8_t* mp = mask + (row / n) * m + j;
+    if (vec) {
+        half8_t v = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(x + e0));
+        const uint2_t mk = *reinterpret_cast<const uint2_t*>(mp);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const uint32_t byte = ((e < 4 ? mk.x : mk.y) >> ((e & 3) * 8)) & 0xffu;
+            if (byte == 0) v[e] = value;
+        }
+        __builtin_nontemporal_store(v, reinterpret_cast<half8_t*>(out + e0));
+    } else {
+        out[e0] = (mp[0] == 0) ? value : x[e0];
+    }
+}
+
+}  // namespace cpmk
+
+using namespace cpmk;
+
+extern "C" {
+
+int cpmk_gelu_forward(int32_t batch, int32_t n, const void* mat, void* out, void* stream) {
+    if (batch < 0 || n < 0) return CPMK_EBADARG;
+    const int64_t total = (int64_t)batch * n;
+    if (total == 0) return 0;
+    const int vec = aligned16(mat) && aligned16(out);
+    const int64_t g = ceil_div(vec ? ceil_div(total, 8) : total, 256);
+    hipLaunchKernelGGL(k_gelu, dim3((unsigned)g), dim3(256), 0, (hipStream_t)stream, total, (const half_t*)mat,
+                       (half_t*)out, vec);
+    return launch_status();
+}
+
+static int ln_affine(int32_t batch, int32_t n, int32_t m, const void* inp, const void* alpha, const void* beta,
+                     void* out, hipStream_t st) {
+    if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
+    if (m % 2) return CPMK_EALIGN;   // kernels/arith.py:146,200
+    const int64_t total = (int64_t)batch * n * m;
+    if (total == 0) return 0;
+    const int vec = (m % 8 == 0) && aligned16(inp) && aligned16(out);
+    const int64_t g = ceil_div(total / (vec ? 8 : 2), 256);
+    if (beta)
+        hipLaunchKernelGGL((k_ln_affine<true>), dim3((unsigned)g), dim3(256), 0, st, total, n, m, (const half_t*)inp,
+                           (const half_t*)alpha, (const half_t*)beta, (half_t*)out, vec);
+    else
+        hipLaunchKernelGGL((k_ln_affine<false>), dim3((unsigned)g), dim3(256), 0, st, total, n, m, (const half_t*)inp,
+                           (const half_t*)alpha, (const half_t*)nullptr, (half_t*)out, vec);
+    return launch_status();
+}
+
+int cpmk_arith_ln_mul_add(int32_t batch, int32_t n, int32_t m, const void* inp, const void* alpha,
+                          const void* beta, void* out, void* stream) {
+    if (beta == nullptr) return CPMK_EBADARG;
+    return ln_affine(batch, n, m, inp, alpha, beta, out, (hipStream_t)stream);
+}
+
+int cpmk_arith_ln_mul(int32_t batch, int32_t n, int32_t m, const void* inp, const void* alpha, void* out,
+                      void* stream) {
+    return ln_affine(batch, n, m, inp, alpha, nullptr, out, (hipStream_t)stream);
+}
+
+int cpmk_arith_element_add(int32_t batch, int32_t n, const void* x, const void* y, void* out, void* stream) {
+    if (batch < 0 || n < 0) return CPMK_EBADARG;
+    if (n % 2) return CPMK_EALIGN;   // kernels/arith.py:53
+    const int64_t total = (int64_t)batch * n;
+    if (total == 0) return 0;
+    const int vec = aligned16(x) && aligned16(y) && aligned16(out);
+    const int64_t g = ceil_div(vec ? ceil_div(total, 8) : total, 256);
+    hipLaunchKernelGGL(k_add, dim3((unsigned)g), dim3(256), 0, (hipStream_t)stream, total, (const half_t*)x,
+                       (const half_t*)y, (half_t*)out, vec);
+    return launch_status();
+}
+
+int cpmk_mask(int32_t batch, int32_t n, int32_t m, const void* inp, const void* mask, float value, void* out,
+              void* stream) {
+    if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
+    const int64_t total = (int64_t)batch * n * m;
+    if (total == 0) return 0;
+    const int vec = (m % 8 == 0) && aligned16(inp) && aligned16(out) && ((reinterpret_cast<uintptr_t>(mask) & 7u) == 0);
+    const int64_t g = ceil_div(vec ? total / 8 : total, 256);
+    hipLaunchKernelGGL(k_mask, dim3((unsigned)g), dim3(256), 0, (hipStream_t)stream, total, n, m, (const half_t*)inp,
+                       (const int8_t*)mask, (half_t)value, (half_t*)out, vec);
+    return launch_status();
+}
+
+}  // extern "C"

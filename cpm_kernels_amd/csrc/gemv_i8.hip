@@ -1,0 +1,179 @@
+// Decode GEMV with a broadcast int8 weight matrix:
+//   out[b,o] = fp16( (f32(sum_k mat[o,k]*vec[b,k]) * f32(scale_vec[b])) * f32(scale_mat[o]) )
+// (cuda/gemv.cu:57-76 of the reference, which launches one 1024-thread block per output
+// scalar and re-reads the weight row once per batch element).
+//
+// Here the weight matrix is streamed from HBM exactly once: the batch of quantised vectors
+// is the second operand of v_mfma_i32_16x16x64_i8, so one pass over a 16-row slab of the
+// matrix serves up to 128 vectors.  The sum over k is an exact integer sum, so splitting k
+// over waves and reordering it inside the MFMA cannot change the int32 result.
+#include "common.h"
+
+namespace cpmk {
+
+// Workgroup = NW waves, RG*16 consecutive matrix rows, all of k.  k is cut into 256-byte
+// chunks dealt round-robin to the waves; within a chunk lane (r = l%16, q = l/16) owns the
+// 64 contiguous bytes [q*64, q*64+64) of row r as four 16-byte pieces, one MFMA each.  The
+// vector operand uses the same lane -> k assignment, which is all the MFMA needs.
+template <int NW, int RG, int NB>
+__global__ __launch_bounds__(NW * 64) void k_gemv_mfma(int32_t batch, int32_t dim_out, int32_t dim_in,
+                                                       const half_t* __restrict__ scale_mat,
+                                                       const int8_t* __restrict__ mat,
+                                                       const half_t* __restrict__ scale_vec,
+                                                       const int8_t* __restrict__ vec,
+                                                       half_t* __restrict__ out) {
+    __shared__ int32_t part[RG * NB][256];   // cross-wave sums (LDS integer atomics)
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int r = lane & 15, q = lane >> 4;
+    const int32_t row0 = blockIdx.x * (RG * 16);
+
+    int4_t acc[RG][NB];
+#pragma unroll
+    for (int g = 0; g < RG; ++g)
+#pragma unroll
+        for (int t = 0; t < NB; ++t) acc[g][t] = int4_t{0, 0, 0, 0};
+
+    const int nchunks = (dim_in + 255) >> 8;
+    for (int c = w; c < nchunks; c += NW) {
+        const int32_t kb = c * 256 + q * 64;
+        int4_t wv[RG][4], vv[NB][4];
+#pragma unroll
+        for (int g = 0; g < RG; ++g) {
+            const int32_t row = row0 + g * 16 + r;
+            const int8_t* p = mat + (int64_t)row * dim_in + kb;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                int4_t v = {0, 0, 0, 0};
+                if (row < dim_out && kb + j * 16 < dim_in)
+                    v = __builtin_nontemporal_load(reinterpret_cast<const int4_t*>(p) + j);
+                wv[g][j] = v;
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < NB; ++t) {
+            const int32_t b = t * 16 + r;
+            const int8_t* p = vec + (int64_t)b * dim_in + kb;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                int4_t v = {0, 0, 0, 0};
+                if (b < batch && kb + j * 16 < dim_in) v = *(reinterpret_cast<const int4_t*>(p) + j);
+                vv[t][j] = v;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int g = 0; g < RG; ++g)
+#pragma unroll
+                for (int t = 0; t < NB; ++t)
+                    acc[g][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wv[g][j], vv[t][j], acc[g][t], 0, 0, 0);
+    }
+
+    for (int idx = tid; idx < RG * NB * 256; idx += NW * 64) (&part[0][0])[idx] = 0;
+    __syncthreads();
+    // accumulator e of lane l: matrix row (l/16)*4 + e, vector l%16 of the 16x16 tile
+#pragma unroll
+    for (int g = 0; g < RG; ++g)
+#pragma unroll
+        for (int t = 0; t < NB; ++t)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) atomicAdd(&part[g * NB + t][(q * 4 + e) * 16 + r], acc[g][t][e]);
+    __syncthreads();
+
+    // part[tile][row_in_tile*16 + b_in_tile]; thread -> (b, row) with row fastest so a
+    // vector's outputs are stored contiguously.
+    for (int idx = tid; idx < RG * NB * 256; idx += NW * 64) {
+        const int rr = idx % (RG * 16), bb = idx / (RG * 16);
+        const int g = rr >> 4, t = bb >> 4;
+        const int32_t s = part[g * NB + t][(rr & 15) * 16 + (bb & 15)];
+        const int32_t row = row0 + rr;
+        if (row < dim_out && bb < batch)
+            out[(int64_t)bb * dim_out + row] = dequant(s, (float)scale_vec[bb], (float)scale_mat[row]);
+    }
+}
+
+// Generic path (any dim_in % 4 == 0, any alignment): one wave per matrix row, dword loads,
+// v_dot4_i32_i8, up to 8 vectors per pass so the row is read from HBM once per 8 vectors.
+__global__ __launch_bounds__(256) void k_gemv_dot4(int32_t batch, int32_t dim_out, int32_t dim_in,
+                                                   const half_t* __restrict__ scale_mat,
+                                                   const int8_t* __restrict__ mat,
+                                                   const half_t* __restrict__ scale_vec,
+                                                   const int8_t* __restrict__ vec,
+                                                   half_t* __restrict__ out) {
+    const int lane = threadIdx.x & 63;
+    const int32_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= dim_out) return;
+    const int32_t* mrow = reinterpret_cast<const int32_t*>(mat + (int64_t)row * dim_in);
+    const int32_t k4 = dim_in >> 2;
+    const float sm = (float)scale_mat[row];
+    for (int32_t b0 = 0; b0 < batch; b0 += 8) {
+        int32_t acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        for (int32_t i = lane; i < k4; i += 64) {
+            const int32_t wv = mrow[i];
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                if (b0 + t < batch) {
+                    const int32_t vv = reinterpret_cast<const int32_t*>(vec + (int64_t)(b0 + t) * dim_in)[i];
+                    acc[t] = __builtin_amdgcn_sdot4(wv, vv, acc[t], false);
+                }
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const int32_t s = wave_sum_i32(acc[t]);
+            if (lane == 0 && b0 + t < batch)
+                out[(int64_t)(b0 + t) * dim_out + row] = dequant(s, (float)scale_vec[b0 + t], sm);
+        }
+    }
+}
+
+template <int NB>
+static void launch_mfma(int32_t batch, int32_t dim_out, int32_t dim_in, const half_t* sm, const int8_t* mat,
+                        const half_t* sv, const int8_t* vec, half_t* out, hipStream_t st) {
+    // 32 rows per workgroup halves the L2 traffic for the vectors; keep 16 when that
+    // would leave compute units without a workgroup.
+    if (dim_out >= 32 * 256) {
+        hipLaunchKernelGGL((k_gemv_mfma<8, 2, NB>), dim3((unsigned)ceil_div(dim_out, 32)), dim3(512), 0, st,
+                           batch, dim_out, dim_in, sm, mat, sv, vec, out);
+    } else {
+        hipLaunchKernelGGL((k_gemv_mfma<8, 1, NB>), dim3((unsigned)ceil_div(dim_out, 16)), dim3(512), 0, st,
+                           batch, dim_out, dim_in, sm, mat, sv, vec, out);
+    }
+}
+
+}  // namespace cpmk
+
+using namespace cpmk;
+
+extern "C" int cpmk_gemv_broadcast_mat_int8(int32_t batch, int32_t dim_out, int32_t dim_in,
+                                            const void* scale_mat, const void* mat, const void* scale_vec,
+                                            const void* vec, void* out, void* stream) {
+    if (batch < 0 || dim_out < 0 || dim_in < 0) return CPMK_EBADARG;
+    if (dim_in % 4) return CPMK_EALIGN;   // kernels/gemv.py:65
+    if (batch == 0 || dim_out == 0) return 0;
+    hipStream_t st = (hipStream_t)stream;
+    const half_t* sm = (const half_t*)scale_mat;
+    const half_t* sv = (const half_t*)scale_vec;
+    const int8_t* M = (const int8_t*)mat;
+    const int8_t* V = (const int8_t*)vec;
+    half_t* O = (half_t*)out;
+    const bool fast = dim_in > 0 && (dim_in % 16 == 0) && aligned16(mat) && aligned16(vec);
+    if (!fast) {
+        hipLaunchKernelGGL(k_gemv_dot4, dim3((unsigned)ceil_div(dim_out, 4)), dim3(256), 0, st, batch, dim_out,
+                           dim_in, sm, M, sv, V, O);
+        return launch_status();
+    }
+    // up to 128 vectors per pass over the matrix
+    for (int32_t b0 = 0; b0 < batch; b0 += 128) {
+        const int32_t nb = batch - b0 < 128 ? batch - b0 : 128;
+        const int8_t* v = V + (int64_t)b0 * dim_in;
+        half_t* o = O + (int64_t)b0 * dim_out;
+        const half_t* s = sv + b0;
+        if (nb <= 16) launch_mfma<1>(nb, dim_out, dim_in, sm, M, s, v, o, st);
+        else if (nb <= 32) launch_mfma<2>(nb, dim_out, dim_in, sm, M, s, v, o, st);
+        else if (nb <= 64) launch_mfma<4>(nb, dim_out, dim_in, sm, M, s, v, o, st);
+        else launch_mfma<8>(nb, dim_out, dim_in, sm, M, s, v, o, st);
+        if (int e = launch_status()) return e;
+    }
+    return 0;
+}

@@ -1,0 +1,112 @@
+// T5-style relative position buckets and the bias gather built on them
+// (cuda/position_bucket.cu:6-54, :105-133 of the reference).
+#include "common.h"
+
+namespace cpmk {
+
+// int32 table of max_distance entries.  Same float formulation as cu_init_position_mapping:
+// note that max_distance / exact_buckets is an integer division there (.cu:16).
+__global__ __launch_bounds__(256) void k_position_init(int32_t num_buckets, int32_t max_distance, int32_t* out,
+                                                       int bidirectional) {
+    const int32_t part = num_buckets / (bidirectional ? 2 : 1);
+    const int32_t exact = part / 2;
+    const int32_t log_buckets = part - exact;
+    const float v = logf((float)(max_distance / exact));
+    for (int32_t i = blockIdx.x * 256 + threadIdx.x; i < max_distance; i += gridDim.x * 256) {
+        if (i < exact) out[i] = i;
+        else out[i] = (int32_t)(logf((float)i / (float)exact) / v * (float)log_buckets) + exact;
+    }
+}
+
+__device__ inline int32_t bucket_of(int32_t rel, int32_t num_buckets, int32_t max_distance,
+                                    const int32_t* __restrict__ table, int bidirectional) {
+    int32_t off = 0;
+    if (rel < 0) {
+        if (bidirectional) { rel = -rel; off = num_buckets / 2; }
+        else rel = 0;
+    }
+    if (rel >= max_distance) rel = max_distance - 1;
+    return table[rel] + off;
+}
+
+// out[h, k, q] = weight[h, bucket(q - k)].  The bias is Toeplitz: for one head it depends on
+// q - k only.  A workgroup builds that head's diagonal vector d[r], r = q - k + (key_len-1),
+// for the q - k range of its KR key rows in LDS and then streams the rows out.
+// grid = (ceil(key_len / KR), num_heads)
+constexpr int KR = 16;
+__global__ __launch_bounds__(256) void k_position_forward(int32_t query_len, int32_t key_len, int32_t num_buckets,
+                                                          int32_t max_distance, const int32_t* __restrict__ table,
+                                                          const half_t* __restrict__ weight, half_t* out,
+                                                          int bidirectional) {
+    extern __shared__ half_t diag[];          // query_len + KR - 1 entries
+    const int32_t k0 = blockIdx.x * KR;
+    const int32_t h = blockIdx.y;
+    const int32_t kend = min(k0 + KR, key_len);
+    // diag[t] holds rel = t - (kend - 1 - k0) + ... : rel ranges over [-(kend-1), query_len-1-k0]
+    const int32_t rel_min = -(kend - 1);
+    const int32_t nd = query_len + (kend - k0) - 1;
+    const half_t* wh = weight + (int64_t)h * num_buckets;
+    for (int32_t t = threadIdx.x; t < nd; t += 256)
+        diag[t] = wh[bucket_of(rel_min + t, num_buckets, max_distance, table, bidirectional)];
+    __syncthreads();
+    for (int32_t k = k0; k < kend; ++k) {
+        half_t* orow = out + ((int64_t)h * key_len + k) * query_len;
+        const int32_t shift = -k - rel_min;    // q - k - rel_min = q + shift
+        for (int32_t q = threadIdx.x; q < query_len; q += 256) orow[q] = diag[q + shift];
+    }
+}
+
+// out[h, k] for one query position (decode step).
+__global__ __launch_bounds__(256) void k_position_step(int32_t query_pos, int32_t key_len, int32_t num_buckets,
+                                                       int32_t max_distance, int32_t num_heads,
+                                                       const int32_t* __restrict__ table,
+                                                       const half_t* __restrict__ weight, half_t* out,
+                                                       int bidirectional) {
+    const int32_t k = blockIdx.x * 256 + threadIdx.x;
+    if (k >= key_len) return;
+    const int32_t bucket = bucket_of(query_pos - k, num_buckets, max_distance, table, bidirectional);
+    for (int32_t h = 0; h < num_heads; ++h) out[(int64_t)h * key_len + k] = weight[(int64_t)h * num_buckets + bucket];
+}
+
+}  // namespace cpmk
+
+using namespace cpmk;
+
+extern "C" {
+
+int cpmk_position_embedding_init(int32_t num_buckets, int32_t max_distance, void* out, int bidirectional,
+                                 void* stream) {
+    if (num_buckets < (bidirectional ? 4 : 2) || max_distance < 0) return CPMK_EBADARG;
+    if (max_distance == 0) return 0;
+    hipLaunchKernelGGL(k_position_init, dim3((unsigned)ceil_div(max_distance, 256)), dim3(256), 0,
+                       (hipStream_t)stream, num_buckets, max_distance, (int32_t*)out, bidirectional);
+    return launch_status();
+}
+
+int cpmk_position_embedding_forward(int32_t query_len, int32_t key_len, int32_t num_buckets, int32_t max_distance,
+                                    int32_t num_heads, const void* position_mapping, const void* weight, void* out,
+                                    int bidirectional, void* stream) {
+    if (query_len < 0 || key_len < 0 || num_heads < 0 || num_buckets <= 0 || max_distance <= 0) return CPMK_EBADARG;
+    if ((int64_t)query_len * key_len * num_heads == 0) return 0;
+    if (num_heads > 65535) return CPMK_ETOOBIG;
+    const size_t smem = (size_t)(query_len + KR - 1) * sizeof(half_t);
+    if (smem > 64 * 1024) return CPMK_ETOOBIG;     // query_len up to 32752
+    dim3 grid((unsigned)ceil_div(key_len, KR), (unsigned)num_heads);
+    hipLaunchKernelGGL(k_position_forward, grid, dim3(256), smem, (hipStream_t)stream, query_len, key_len,
+                       num_buckets, max_distance, (const int32_t*)position_mapping, (const half_t*)weight,
+                       (half_t*)out, bidirectional);
+    return launch_status();
+}
+
+int cpmk_position_embedding_step(int32_t query_pos, int32_t key_len, int32_t num_buckets, int32_t max_distance,
+                                 int32_t num_heads, const void* position_mapping, const void* weight, void* out,
+                                 int bidirectional, void* stream) {
+    if (key_len < 0 || num_heads < 0 || num_buckets <= 0 || max_distance <= 0) return CPMK_EBADARG;
+    if ((int64_t)key_len * num_heads == 0) return 0;
+    hipLaunchKernelGGL(k_position_step, dim3((unsigned)ceil_div(key_len, 256)), dim3(256), 0, (hipStream_t)stream,
+                       query_pos, key_len, num_buckets, max_distance, num_heads, (const int32_t*)position_mapping,
+                       (const half_t*)weight, (half_t*)out, bidirectional);
+    return launch_status();
+}
+
+}  // extern "C"

@@ -1,0 +1,377 @@
+// Row/column absmax scales, fp16 -> int8 rounding and int32 -> fp16 dequantisation.
+// All of these are single-pass HBM-bound streaming kernels: 16-byte loads per lane,
+// wave64 butterfly reductions, no 32-lane geometry.
+// Arithmetic follows cuda/gemm.cu:6-98,176-205 and cuda/gemv.cu:26-54 of the reference.
+#include "common.h"
+
+namespace cpmk {
+
+// ---------------------------------------------------------------------------------------
+// absmax over contiguous rows: out[row] = fp16(max_j |mat[row, j]| / 127)
+// TPR threads cooperate on one row (64 = one wave, 256 = whole block).
+// ---------------------------------------------------------------------------------------
+template <int TPR, bool VEC>
+__global__ __launch_bounds__(256) void k_row_absmax(int64_t rows, int32_t m,
+                                                    const half_t* __restrict__ mat,
+                                                    half_t* __restrict__ out) {
+    __shared__ float red[4];
+    constexpr int RPB = 256 / TPR;
+    const int t = threadIdx.x % TPR;
+    const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / TPR;
+    float mx = 0.0f;
+    if (row < rows) {
+        const half_t* p = mat + row * m;
+        if (VEC) {
+            const half8_t* p8 = reinterpret_cast<const half8_t*>(p);
+            const int m8 = m >> 3;
+            for (int j = t; j < m8; j += TPR) {
+                half8_t v = __builtin_nontemporal_load(p8 + j);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) mx = fmaxf(fabsf((float)v[e]), mx);
+            }
+        } else {
+            for (int j = t; j < m; j += TPR) mx = fmaxf(fabsf((float)p[j]), mx);
+        }
+    }
+    if (TPR == 64) {
+        mx = wave_max(mx);
+    } else {
+        mx = block_max<4>(mx, red);
+    }
+    if (t == 0 && row < rows) out[row] = scale_from_absmax(mx);
+}
+
+// ---------------------------------------------------------------------------------------
+// absmax over dim 1 of (b, n, m): out[b, j] = fp16(max_i |mat[b,i,j]| / 127)
+// Block = 256 threads = 32 row groups x 8 lanes; each lane owns 8 adjacent columns
+// (one 16-byte load per row), the 32 row groups stride over n and are combined in LDS.
+// gridDim = (ceil(m/64), batch).
+// ---------------------------------------------------------------------------------------
+template <bool VEC>
+__global__ __launch_bounds__(256) void k_col_absmax(int32_t n, int32_t m,
+                                                    const half_t* __restrict__ mat,
+                                                    half_t* __restrict__ out) {
+    __shared__ float red[32][65];
+    const int lane8 = threadIdx.x & 7, rg = threadIdx.x >> 3;
+    const int col0 = blockIdx.x * 64 + lane8 * 8;
+    const half_t* base = mat + (int64_t)blockIdx.y * n * m;
+    float mx[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) mx[e] = 0.0f;
+    if (VEC) {
+        if (col0 < m) {
+            for (int i = rg; i < n; i += 32) {
+                half8_t v = *reinterpret_cast<const half8_t*>(base + (int64_t)i * m + col0);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) mx[e] = fmaxf(fabsf((float)v[e]), mx[e]);
+            }
+        }
+    } else {
+        for (int i = rg; i < n; i += 32) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (col0 + e < m) mx[e] = fmaxf(fabsf((float)base[(int64_t)i * m + col0 + e]), mx[e]);
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) red[rg][lane8 * 8 + e] = mx[e];
+    __syncthreads();
+    if (threadIdx.x < 64) {
+        float r = 0.0f;
+#pragma unroll 8
+        for (int g = 0; g < 32; ++g) r = fmaxf(r, red[g][threadIdx.x]);
+        const int col = blockIdx.x * 64 + threadIdx.x;
+        if (col < m) out[(int64_t)blockIdx.y * m + col] = scale_from_absmax(r);
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// rounding: out = int8(rint(x / scale)).  MODE 0: scale per row (index = element / m),
+// MODE 1: scale per (batch, column) (index = b*m + j).  VEC: 16 elements per thread.
+// ---------------------------------------------------------------------------------------
+template <int MODE, bool VEC>
+__global__ __launch_bounds__(256) void k_round(int64_t total, int32_t n, int32_t m,
+                                               const half_t* __restrict__ mat,
+                                               const half_t* __restrict__ scale,
+                                               int8_t* __restrict__ out) {
+    const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (VEC) {
+        const int64_t e0 = gid * 16;
+        if (e0 >= total) return;
+        const int64_t row = e0 / m;            // m % 16 == 0: the 16 elements share a row
+        const int32_t j0 = (int32_t)(e0 - row * m);
+        const half8_t* p = reinterpret_cast<const half8_t*>(mat + e0);
+        half8_t a = __builtin_nontemporal_load(p), b = __builtin_nontemporal_load(p + 1);
+        float s[16];
+        if (MODE == 0) {
+            const float sr = (float)scale[row];
+#pragma unroll
+            for (int e = 0; e < 16; ++e) s[e] = sr;
+        } else {
+            const int64_t bidx = row / n;
+            const half8_t* sp = reinterpret_cast<const half8_t*>(scale + bidx * m + j0);
+            half8_t s0 = sp[0], s1 = sp[1];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) { s[e] = (float)s0[e]; s[8 + e] = (float)s1[e]; }
+        }
+        int32_t q[16];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            q[e] = quant_i8((float)a[e], s[e]);
+            q[8 + e] = quant_i8((float)b[e], s[8 + e]);
+        }
+        uint4_t w;
+        w.x = pack4_i8(q[0], q[1], q[2], q[3]);
+        w.y = pack4_i8(q[4], q[5], q[6], q[7]);
+        w.z = pack4_i8(q[8], q[9], q[10], q[11]);
+        w.w = pack4_i8(q[12], q[13], q[14], q[15]);
+        *reinterpret_cast<uint4_t*>(out + e0) = w;
+    } else {
+        if (gid >= total) return;
+        const int64_t row = gid / m;
+        float s;
+        if (MODE == 0) s = (float)scale[row];
+        else s = (float)scale[(row / n) * m + (gid - row * m)];
+        out[gid] = (int8_t)quant_i8((float)mat[gid], s);
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// dequantisation: out = fp16((f32(acc) * sx) * sy)
+// MODE 0: both scales (cu_gemm_scale), MODE 1: scale_x only, MODE 2: scale_y only.
+// VEC: 8 elements per thread (two 16-byte loads, one 16-byte store), m % 8 == 0.
+// ---------------------------------------------------------------------------------------
+template <int MODE, bool VEC>
+__global__ __launch_bounds__(256) void k_dequant(int64_t total, int32_t n, int32_t m,
+                                                 const int32_t* __restrict__ mat,
+                                                 const half_t* __restrict__ scale_x,
+                                                 const half_t* __restrict__ scale_y,
+                                                 half_t* __restrict__ out, int bcx, int bcy) {
+    const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t e0 = VEC ? gid * 8 : gid;
+    if (e0 >= total) return;
+    const int64_t row = e0 / m;                // = b*n + i
+    const int32_t j0 = (int32_t)(e0 - row * m);
+    const int64_t b = row / n;
+    const int32_t i = (int32_t)(row - b * n);
+    float sx = 1.0f;
+    if (MODE != 2) sx = (float)scale_x[bcx ? i : row];
+    const half_t* sy = (MODE != 1) ? scale_y + (bcy ? 0 : b * m) + j0 : nullptr;
+    if (VEC) {
+        const int4_t* p = reinterpret_cast<const int4_t*>(mat + e0);
+        int4_t a0 = __builtin_nontemporal_load(p), a1 = __builtin_nontemporal_load(p + 1);
+        half8_t syv;
+        if (MODE != 1) syv = *reinterpret_cast<const half8_t*>(sy);
+        half8_t o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int32_t acc = e < 4 ? a0[e] : a1[e - 4];
+            if (MODE == 0) o[e] = dequant(acc, sx, (float)syv[e]);
+            else if (MODE == 1) o[e] = round_f16(sx * (float)acc);
+            else o[e] = round_f16((float)acc * (float)syv[e]);
+        }
+        *reinterpret_cast<half8_t*>(out + e0) = o;
+    } else {
+        const int32_t acc = mat[e0];
+        if (MODE == 0) out[e0] = dequant(acc, sx, (float)sy[0]);
+        else if (MODE == 1) out[e0] = round_f16(sx * (float)acc);
+        else out[e0] = round_f16((float)acc * (float)sy[0]);
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// fused absmax + round over contiguous rows (one wave per row, the row stays in
+// registers between the two phases): rows up to 64 lanes x NV x 8 halves.
+// ---------------------------------------------------------------------------------------
+template <int NV>
+__global__ __launch_bounds__(256) void k_row_quantize(int64_t rows, int32_t m,
+                                                      const half_t* __restrict__ mat,
+                                                      half_t* __restrict__ scale,
+                                                      int8_t* __restrict__ out) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const half8_t* p8 = reinterpret_cast<const half8_t*>(mat + row * m);
+    const int m8 = m >> 3;
+    half8_t v[NV];
+    float mx = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int j = lane + i * 64;
+        if (j < m8) {
+            v[i] = __builtin_nontemporal_load(p8 + j);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) mx = fmaxf(fabsf((float)v[i][e]), mx);
+        }
+    }
+    mx = wave_max(mx);
+    const half_t sh = scale_from_absmax(mx);
+    if (lane == 0) scale[row] = sh;
+    const float s = (float)sh;
+    uint2_t* o8 = reinterpret_cast<uint2_t*>(out + row * m);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int j = lane + i * 64;
+        if (j < m8) {
+            int32_t q[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) q[e] = quant_i8((float)v[i][e], s);
+            uint2_t w;
+            w.x = pack4_i8(q[0], q[1], q[2], q[3]);
+            w.y = pack4_i8(q[4], q[5], q[6], q[7]);
+            o8[j] = w;
+        }
+    }
+}
+
+static int check3(int32_t batch, int32_t n, int32_t m) {
+    if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
+    return 0;
+}
+
+static int row_absmax(int64_t rows, int32_t m, const void* mat, void* out, hipStream_t st) {
+    if (rows == 0) return 0;
+    const bool vec = (m % 8 == 0) && aligned16(mat);
+    const half_t* p = (const half_t*)mat;
+    half_t* o = (half_t*)out;
+    // few long rows: a whole block per row; otherwise a wave per row
+    const bool wide = rows < 2048 && m >= 2048;
+    if (wide) {
+        if (vec) hipLaunchKernelGGL((k_row_absmax<256, true>), dim3((unsigned)rows), dim3(256), 0, st, rows, m, p, o);
+        else hipLaunchKernelGGL((k_row_absmax<256, false>), dim3((unsigned)rows), dim3(256), 0, st, rows, m, p, o);
+    } else {
+        const unsigned g = (unsigned)ceil_div(rows, 4);
+        if (vec) hipLaunchKernelGGL((k_row_absmax<64, true>), dim3(g), dim3(256), 0, st, rows, m, p, o);
+        else hipLaunchKernelGGL((k_row_absmax<64, false>), dim3(g), dim3(256), 0, st, rows, m, p, o);
+    }
+    return launch_status();
+}
+
+template <int MODE>
+static int round_launch(int32_t batch, int32_t n, int32_t m, const void* mat, const void* scale,
+                        void* out, hipStream_t st) {
+    const int64_t total = (int64_t)batch * n * m;
+    if (total == 0) return 0;
+    const bool vec = (m % 16 == 0) && aligned16(mat) && aligned16(out) && (MODE == 0 || aligned16(scale));
+    const half_t* p = (const half_t*)mat;
+    const half_t* s = (const half_t*)scale;
+    int8_t* o = (int8_t*)out;
+    if (vec) {
+        const int64_t g = ceil_div(total / 16, 256);
+        hipLaunchKernelGGL((k_round<MODE, true>), dim3((unsigned)g), dim3(256), 0, st, total, n, m, p, s, o);
+    } else {
+        const int64_t g = ceil_div(total, 256);
+        hipLaunchKernelGGL((k_round<MODE, false>), dim3((unsigned)g), dim3(256), 0, st, total, n, m, p, s, o);
+    }
+    return launch_status();
+}
+
+template <int MODE>
+static int dequant_launch(int32_t batch, int32_t n, int32_t m, const void* mat, const void* sx,
+                          const void* sy, void* out, int bcx, int bcy, hipStream_t st) {
+    const int64_t total = (int64_t)batch * n * m;
+    if (total == 0) return 0;
+    const bool vec = (m % 8 == 0) && aligned16(mat) && aligned16(out) && (MODE == 1 || aligned16(sy));
+    if (vec) {
+        const int64_t g = ceil_div(total / 8, 256);
+        hipLaunchKernelGGL((k_dequant<MODE, true>), dim3((unsigned)g), dim3(256), 0, st, total, n, m,
+                           (const int32_t*)mat, (const half_t*)sx, (const half_t*)sy, (half_t*)out, bcx, bcy);
+    } else {
+        const int64_t g = ceil_div(total, 256);
+        hipLaunchKernelGGL((k_dequant<MODE, false>), dim3((unsigned)g), dim3(256), 0, st, total, n, m,
+                           (const int32_t*)mat, (const half_t*)sx, (const half_t*)sy, (half_t*)out, bcx, bcy);
+    }
+    return launch_status();
+}
+
+}  // namespace cpmk
+
+using namespace cpmk;
+
+extern "C" {
+
+int cpmk_gemm_calc_scale(int32_t batch, int32_t n, int32_t m, const void* mat, void* out, void* stream) {
+    if (int e = check3(batch, n, m)) return e;
+    return row_absmax((int64_t)batch * n, m, mat, out, (hipStream_t)stream);
+}
+
+int cpmk_gemv_calc_scale(int32_t batch, int32_t n, const void* vec, void* out, void* stream) {
+    if (batch < 0 || n < 0) return CPMK_EBADARG;
+    return row_absmax(batch, n, vec, out, (hipStream_t)stream);
+}
+
+int cpmk_gemm_calc_scale_transpose(int32_t batch, int32_t n, int32_t m, const void* mat, void* out,
+                                   void* stream) {
+    if (int e = check3(batch, n, m)) return e;
+    if (batch == 0 || m == 0) return 0;
+    const bool vec = (m % 8 == 0) && aligned16(mat);
+    dim3 grid((unsigned)ceil_div(m, 64), (unsigned)batch);
+    if (vec) hipLaunchKernelGGL((k_col_absmax<true>), grid, dim3(256), 0, (hipStream_t)stream, n, m, (const half_t*)mat, (half_t*)out);
+    else hipLaunchKernelGGL((k_col_absmax<false>), grid, dim3(256), 0, (hipStream_t)stream, n, m, (const half_t*)mat, (half_t*)out);
+    return launch_status();
+}
+
+int cpmk_gemm_round(int32_t batch, int32_t n, int32_t m, const void* mat, const void* scale, void* out,
+                    void* stream) {
+    if (int e = check3(batch, n, m)) return e;
+    return round_launch<0>(batch, n, m, mat, scale, out, (hipStream_t)stream);
+}
+
+int cpmk_gemv_round(int32_t batch, int32_t n, const void* vec, const void* scale, void* out, void* stream) {
+    if (batch < 0 || n < 0) return CPMK_EBADARG;
+    return round_launch<0>(1, batch, n, vec, scale, out, (hipStream_t)stream);
+}
+
+int cpmk_gemm_round_transpose(int32_t batch, int32_t n, int32_t m, const void* mat, const void* scale,
+                              void* out, void* stream) {
+    if (int e = check3(batch, n, m)) return e;
+    return round_launch<1>(batch, n, m, mat, scale, out, (hipStream_t)stream);
+}
+
+int cpmk_gemm_scale(int32_t batch, int32_t n, int32_t m, const void* mat, const void* scale_x,
+                    const void* scale_y, void* out, int bcx, int bcy, void* stream) {
+    if (int e = check3(batch, n, m)) return e;
+    return dequant_launch<0>(batch, n, m, mat, scale_x, scale_y, out, bcx, bcy, (hipStream_t)stream);
+}
+
+int cpmk_gemm_scale_x(int32_t batch, int32_t n, int32_t m, const void* mat, const void* scale_x, void* out,
+                      void* stream) {
+    if (int e = check3(batch, n, m)) return e;
+    return dequant_launch<1>(batch, n, m, mat, scale_x, nullptr, out, 0, 0, (hipStream_t)stream);
+}
+
+int cpmk_gemm_scale_y(int32_t batch, int32_t n, int32_t m, const void* mat, const void* scale_y, void* out,
+                      void* stream) {
+    if (int e = check3(batch, n, m)) return e;
+    return dequant_launch<2>(batch, n, m, mat, nullptr, scale_y, out, 0, 0, (hipStream_t)stream);
+}
+
+int cpmk_gemm_quantize(int32_t batch, int32_t n, int32_t m, const void* mat, void* scale, void* out,
+                       int transpose, void* stream) {
+    if (int e = check3(batch, n, m)) return e;
+    hipStream_t st = (hipStream_t)stream;
+    if (!transpose) {
+        const int64_t rows = (int64_t)batch * n;
+        if (rows == 0) return 0;
+        const bool vec = (m % 8 == 0) && aligned16(mat) && ((reinterpret_cast<uintptr_t>(out) & 7u) == 0);
+        if (vec && m <= 64 * 8 * 16) {
+            const unsigned g = (unsigned)ceil_div(rows, 4);
+            const int nv = (int)ceil_div(m, 512);
+            const half_t* p = (const half_t*)mat;
+            half_t* s = (half_t*)scale;
+            int8_t* o = (int8_t*)out;
+            if (nv <= 1) hipLaunchKernelGGL((k_row_quantize<1>), dim3(g), dim3(256), 0, st, rows, m, p, s, o);
+            else if (nv <= 2) hipLaunchKernelGGL((k_row_quantize<2>), dim3(g), dim3(256), 0, st, rows, m, p, s, o);
+            else if (nv <= 4) hipLaunchKernelGGL((k_row_quantize<4>), dim3(g), dim3(256), 0, st, rows, m, p, s, o);
+            else if (nv <= 8) hipLaunchKernelGGL((k_row_quantize<8>), dim3(g), dim3(256), 0, st, rows, m, p, s, o);
+            else hipLaunchKernelGGL((k_row_quantize<16>), dim3(g), dim3(256), 0, st, rows, m, p, s, o);
+            return launch_status();
+        }
+        if (int e = cpmk_gemm_calc_scale(batch, n, m, mat, scale, stream)) return e;
+        return cpmk_gemm_round(batch, n, m, mat, scale, out, stream);
+    }
+    if (int e = cpmk_gemm_calc_scale_transpose(batch, n, m, mat, scale, stream)) return e;
+    return cpmk_gemm_round_transpose(batch, n, m, mat, scale, out, stream);
+}
+
+}  // extern "C"

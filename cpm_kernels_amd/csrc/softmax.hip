@@ -1,0 +1,162 @@
+// Softmax over dim 1 of (batch, n, m) fp16 and over contiguous rows (decode step):
+//   M = max(max_i x, -1e6);  S = sum_i exp(x - M) + 1e-10;  out = fp16(exp(x - M) / S)
+// (cuda/softmax.cu:6-43, :117-159).  A column that is entirely -inf therefore yields 0, not
+// NaN.  The reference reads the input three times and evaluates expf twice per element; the
+// tile kernel below reads once, evaluates exp once and keeps the results in registers.
+#include "dim1.h"
+
+namespace cpmk {
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+// exp(x - M) as one fma and one v_exp_f32: exp2(x*log2e - M*log2e).
+__device__ inline float exp_shift(float x, float mlog2e) { return __builtin_amdgcn_exp2f(__builtin_fmaf(x, kLog2e, -mlog2e)); }
+
+template <int NT, int LPR, int R>
+__global__ __launch_bounds__(NT) void k_softmax_tile(int32_t n, int32_t m, int32_t tiles_per_batch,
+                                                     const half_t* inp, half_t* out) {
+    using T = ColTile<NT, LPR, R>;
+    __shared__ float lds[(T::NW + 1) * T::COLS];
+    const uint32_t t = xcd_remap(blockIdx.x, gridDim.x);
+    const uint32_t b = t / tiles_per_batch, ct = t - b * tiles_per_batch;
+    const int32_t col0 = ct * T::COLS + (threadIdx.x % LPR) * 8;
+    const int64_t boff = (int64_t)b * n * m;
+
+    half8_t v[R];
+    coltile_load<NT, LPR, R>(v, inp + boff, n, m, col0, (half_t)(-__builtin_inff()));
+
+    float mx[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) mx[e] = -__builtin_inff();
+#pragma unroll
+    for (int p = 0; p < R; ++p)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) mx[e] = fmaxf(mx[e], (float)v[p][e]);
+    coltile_reduce<NT, LPR, 1, true>(mx, lds);
+
+    float ex[R][8], s[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        mx[e] = fmaxf(mx[e], -1e6f) * kLog2e;
+        s[e] = 0.0f;
+    }
+#pragma unroll
+    for (int p = 0; p < R; ++p)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            ex[p][e] = exp_shift((float)v[p][e], mx[e]);   // rows >= n hold -inf -> 0
+            s[e] += ex[p][e];
+        }
+    coltile_reduce<NT, LPR, 1, false>(s, lds);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s[e] = 1.0f / (s[e] + 1e-10f);
+#pragma unroll
+    for (int p = 0; p < R; ++p)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[p][e] = round_f16(ex[p][e] * s[e]);
+    coltile_store<NT, LPR, R>(v, out + boff, n, m, col0);
+}
+
+// Generic fallback: 64 columns x 4 row groups, three passes (max, sum, write).  All reads of
+// a column by other threads finish before the barrier that precedes the first store, and
+// the last pass re-reads each element in the thread that overwrites it: out may alias inp.
+__global__ __launch_bounds__(256) void k_softmax_generic(int32_t n, int32_t m, const half_t* inp, half_t* out) {
+    __shared__ float red[4][64];
+    const int c = threadIdx.x & 63, rg = threadIdx.x >> 6;
+    const int32_t col = blockIdx.x * 64 + c;
+    const int64_t boff = (int64_t)blockIdx.y * n * m;
+    float mx = -__builtin_inff();
+    if (col < m)
+        for (int32_t i = rg; i < n; i += 4) mx = fmaxf(mx, (float)inp[boff + (int64_t)i * m + col]);
+    red[rg][c] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(red[0][c], red[1][c]), fmaxf(red[2][c], red[3][c]));
+    mx = fmaxf(mx, -1e6f) * kLog2e;
+    __syncthreads();
+    float s = 0.0f;
+    if (col < m)
+        for (int32_t i = rg; i < n; i += 4) s += exp_shift((float)inp[boff + (int64_t)i * m + col], mx);
+    red[rg][c] = s;
+    __syncthreads();
+    s = 1.0f / (red[0][c] + red[1][c] + red[2][c] + red[3][c] + 1e-10f);
+    if (col < m)
+        for (int32_t i = rg; i < n; i += 4) {
+            const int64_t o = boff + (int64_t)i * m + col;
+            out[o] = round_f16(exp_shift((float)inp[o], mx) * s);
+        }
+}
+
+// Contiguous rows (batch, n), in place capable: one 256-thread workgroup per row.
+__global__ __launch_bounds__(256) void k_softmax_rows(int32_t n, const half_t* inp, half_t* out) {
+    __shared__ float red[4];
+    const half_t* p = inp + (int64_t)blockIdx.x * n;
+    half_t* o = out + (int64_t)blockIdx.x * n;
+    float mx = -__builtin_inff();
+    for (int32_t i = threadIdx.x; i < n; i += 256) mx = fmaxf(mx, (float)p[i]);
+    mx = fmaxf(block_max<4>(mx, red), -1e6f) * kLog2e;
+    float s = 0.0f;
+    for (int32_t i = threadIdx.x; i < n; i += 256) s += exp_shift((float)p[i], mx);
+    s = 1.0f / (block_sum<4>(s, red) + 1e-10f);
+    for (int32_t i = threadIdx.x; i < n; i += 256) o[i] = round_f16(exp_shift((float)p[i], mx) * s);
+}
+
+template <int NT, int LPR, int R>
+static void launch_tile(int32_t batch, int32_t n, int32_t m, const half_t* inp, half_t* out, hipStream_t st) {
+    const int32_t tiles = (int32_t)ceil_div(m, LPR * 8);
+    hipLaunchKernelGGL((k_softmax_tile<NT, LPR, R>), dim3((unsigned)((int64_t)tiles * batch)), dim3(NT), 0, st, n, m,
+                       tiles, inp, out);
+}
+
+template <int NT, int LPR>
+static bool launch_tile_r(int r, int32_t batch, int32_t n, int32_t m, const half_t* inp, half_t* out,
+                          hipStream_t st) {
+    if (r <= 1) launch_tile<NT, LPR, 1>(batch, n, m, inp, out, st);
+    else if (r <= 2) launch_tile<NT, LPR, 2>(batch, n, m, inp, out, st);
+    else if (r <= 4) launch_tile<NT, LPR, 4>(batch, n, m, inp, out, st);
+    else if (r <= 8) launch_tile<NT, LPR, 8>(batch, n, m, inp, out, st);
+    else return false;
+    return true;
+}
+
+static int softmax_dispatch(int32_t batch, int32_t n, int32_t m, const void* inp, void* out, hipStream_t st) {
+    if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
+    if ((int64_t)batch * n * m == 0) return 0;
+    const half_t* x = (const half_t*)inp;
+    half_t* y = (half_t*)out;
+    if (m == 1) {
+        hipLaunchKernelGGL(k_softmax_rows, dim3((unsigned)batch), dim3(256), 0, st, n, x, y);
+        return launch_status();
+    }
+    if (m % 8 == 0 && aligned16(inp) && aligned16(out)) {
+        bool ok = false;
+        if (n <= 64 * 8 && m >= 64) ok = launch_tile_r<512, 8>((int)ceil_div(n, 64), batch, n, m, x, y, st);
+        else if (n <= 128 * 8 && m >= 64) ok = launch_tile_r<1024, 8>((int)ceil_div(n, 128), batch, n, m, x, y, st);
+        else if (n <= 256 * 8 && m >= 32) ok = launch_tile_r<1024, 4>((int)ceil_div(n, 256), batch, n, m, x, y, st);
+        else if (n <= 512 * 8) ok = launch_tile_r<1024, 2>((int)ceil_div(n, 512), batch, n, m, x, y, st);
+        if (ok) return launch_status();
+    }
+    if (batch > 65535) return CPMK_ETOOBIG;
+    dim3 grid((unsigned)ceil_div(m, 64), (unsigned)batch);
+    hipLaunchKernelGGL(k_softmax_generic, grid, dim3(256), 0, st, n, m, x, y);
+    return launch_status();
+}
+
+}  // namespace cpmk
+
+using namespace cpmk;
+
+extern "C" {
+
+int cpmk_softmax_forward(int32_t batch, int32_t n, int32_t m, const void* inp, void* out, void* stream) {
+    return softmax_dispatch(batch, n, m, inp, out, (hipStream_t)stream);
+}
+
+int cpmk_softmax_step_inplace(int32_t batch, int32_t n, void* x, void* stream) {
+    if (batch < 0 || n < 0) return CPMK_EBADARG;
+    if ((int64_t)batch * n == 0) return 0;
+    hipLaunchKernelGGL(k_softmax_rows, dim3((unsigned)batch), dim3(256), 0, (hipStream_t)stream, n,
+                       (const half_t*)x, (half_t*)x);
+    return launch_status();
+}
+
+}  // extern "C"

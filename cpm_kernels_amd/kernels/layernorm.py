@@ -1,0 +1,57 @@
+"""Normalisation launchers with the signatures of cpm_kernels/kernels/layernorm.py."""
+from ..library import cpmk
+from .base import DevicePointer, CUDAStream, _stream, not_on_path
+
+
+def layernorm_forward(batch: int, n: int, m: int,
+                      mat: DevicePointer,    # (batch, n, m)
+                      out: DevicePointer,    # (batch, n, m)
+                      eps: float, rd_mean: bool,
+                      stream: CUDAStream):
+    """reference: kernels/layernorm.py:18-38"""
+    cpmk.layernorm_forward(batch, n, m, mat, out, eps, int(bool(rd_mean)), _stream(stream))
+
+
+def layernorm_inplace_forward(batch: int, n: int, m: int,
+                              mat: DevicePointer,    # (batch, n, m)
+                              eps: float, rd_mean: bool,
+                              stream: CUDAStream):
+    """reference: kernels/layernorm.py:40-58"""
+    cpmk.layernorm_forward(batch, n, m, mat, mat, eps, int(bool(rd_mean)), _stream(stream))
+
+
+def layernorm_affine_forward(batch: int, n: int, m: int,
+                             mat: DevicePointer,      # (batch, n, m)
+                             alpha: DevicePointer,    # (n)
+                             beta,                    # (n) or None / 0
+                             out: DevicePointer,      # (batch, n, m)
+                             eps: float, rd_mean: bool,
+                             stream: CUDAStream):
+    """layernorm_forward + arith_ln_mul_add / arith_ln_mul in one launch, bit-identical to the
+    two-launch sequence of torch/layernorm.py:9-29,88-111."""
+    cpmk.layernorm_affine_forward(batch, n, m, mat, alpha, beta or None, out, eps, int(bool(rd_mean)),
+                                  _stream(stream))
+
+
+def layernorm_step(batch: int, n: int,
+                   mat: DevicePointer,    # (batch, n)  fp16
+                   out: DevicePointer,    # (batch, n)  fp16
+                   eps: float, rd_mean: bool,
+                   stream: CUDAStream):
+    """reference: kernels/layernorm.py:152-171"""
+    cpmk.layernorm_step(batch, n, mat, out, eps, int(bool(rd_mean)), _stream(stream))
+
+
+def layernorm_step_inplace(batch: int, n: int,
+                           mat: DevicePointer,    # (batch, n)  fp16
+                           eps: float, rd_mean: bool,
+                           stream: CUDAStream):
+    """reference: kernels/layernorm.py:173-190"""
+    cpmk.layernorm_step(batch, n, mat, mat, eps, int(bool(rd_mean)), _stream(stream))
+
+
+_w = "training, kernels/layernorm.py:60-150"
+layernorm_forward_v = not_on_path("layernorm_forward_v", _w)
+layernorm_forward_mv = not_on_path("layernorm_forward_mv", _w)
+layernorm_backward_v = not_on_path("layernorm_backward_v", _w)
+layernorm_backward_mv = not_on_path("layernorm_backward_mv", _w)

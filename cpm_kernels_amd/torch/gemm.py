@@ -1,0 +1,110 @@
+"""``bmm(A, aT, B, bT, int8)`` with the interface of cpm_kernels/torch/gemm.py:233-239.
+
+int8=True is the hot path: row-wise absmax quantisation of both operands, int8 GEMM with
+int32 accumulation, fp16 dequantisation (GEMMInt8.forward, torch/gemm.py:84-113).  The
+reference does that in six launches with an int32 round trip; here the default is three
+(two fused quantise launches and one GEMM with the dequantising epilogue), bit-identical to
+the six-launch sequence, which ``fused=False`` still runs through the kernel-level API.
+"""
+import torch
+from ..kernels import gemm_calc_scale, gemm_calc_scale_transpose, gemm_round, gemm_round_transpose, \
+    gemm_scale, gemm_int8, gemm_int8_scale, gemm_quantize
+from ._common import cur_stream, InferenceOnly
+
+
+def calc_scale(mat: torch.Tensor, transpose: bool) -> torch.Tensor:
+    """reference: torch/gemm.py:5-19"""
+    assert mat.is_contiguous() and mat.is_cuda
+    b, n, m = mat.size()
+    out = torch.empty((b, m if transpose else n), dtype=torch.half, device=mat.device)
+    fn = gemm_calc_scale_transpose if transpose else gemm_calc_scale
+    fn(b, n, m, mat.data_ptr(), out.data_ptr(), cur_stream())
+    return out
+
+
+def round_i8(mat: torch.Tensor, scale: torch.Tensor, transpose: bool) -> torch.Tensor:
+    """reference: torch/gemm.py:21-38"""
+    assert mat.is_contiguous() and mat.is_cuda
+    assert scale.is_contiguous() and scale.is_cuda
+    b, n, m = mat.size()
+    out = torch.empty(mat.size(), dtype=torch.int8, device=mat.device)
+    fn = gemm_round_transpose if transpose else gemm_round
+    fn(b, n, m, mat.data_ptr(), scale.data_ptr(), out.data_ptr(), cur_stream())
+    return out
+
+
+def quantize(mat: torch.Tensor, transpose: bool):
+    """calc_scale + round_i8 in one launch; returns (scale, int8 tensor)."""
+    assert mat.is_contiguous() and mat.is_cuda and mat.dtype == torch.half
+    b, n, m = mat.size()
+    scale = torch.empty((b, m if transpose else n), dtype=torch.half, device=mat.device)
+    out = torch.empty(mat.size(), dtype=torch.int8, device=mat.device)
+    gemm_quantize(b, n, m, mat.data_ptr(), scale.data_ptr(), out.data_ptr(), transpose, cur_stream())
+    return scale, out
+
+
+def _dims(quantA, quantB, aT, bT):
+    M = quantA.size(2) if aT else quantA.size(1)
+    K = quantA.size(1) if aT else quantA.size(2)
+    N = quantB.size(1) if bT else quantB.size(2)
+    return M, K, N
+
+
+def gemm_and_scale(quantA, scaleA, quantB, scaleB, aT, bT, fused=True) -> torch.Tensor:
+    """reference: torch/gemm.py:40-82 (both scales present).  The operands are swapped in
+    the kernel call exactly as there (:45-52) so the (M, N) product comes out row-major."""
+    M, K, N = _dims(quantA, quantB, aT, bT)
+    batch = max(quantA.size(0), quantB.size(0))
+    result_fp = torch.empty((batch, M, N), dtype=torch.float16, device=quantA.device)
+    if fused:
+        gemm_int8_scale(N, K, M, quantB.size(0), quantA.size(0), bT, aT,
+                        quantB.data_ptr(), quantA.data_ptr(),
+                        scaleA.data_ptr(), scaleB.data_ptr(),
+                        quantA.size(0) == 1, quantB.size(0) == 1,
+                        result_fp.data_ptr(), cur_stream())
+        return result_fp
+    result_i32 = torch.empty((batch, M, N), dtype=torch.int32, device=quantA.device)
+    gemm_int8(N, K, M, quantB.size(0), quantA.size(0), bT, aT,
+              quantB.data_ptr(), quantA.data_ptr(), result_i32.data_ptr(), cur_stream())
+    gemm_scale(batch, M, N, result_i32.data_ptr(), scaleA.data_ptr(), scaleB.data_ptr(),
+               result_fp.data_ptr(), quantA.size(0) == 1, quantB.size(0) == 1, cur_stream())
+    return result_fp
+
+
+class GEMMInt8(InferenceOnly):
+    @staticmethod
+    def forward(ctx, A: torch.Tensor, aT: bool, B: torch.Tensor, bT: bool, fused: bool = True):
+        """A: (batchA, M, K) [(batchA, K, M) if aT], B: (batchB, K, N) [(batchB, N, K) if bT]
+        -> (batch, M, N) fp16.  reference: torch/gemm.py:84-113"""
+        assert A.is_cuda and B.is_cuda and A.device == B.device
+        assert A.is_contiguous() and B.is_contiguous()
+        assert A.dtype == torch.half and B.dtype == torch.half
+        if fused:
+            scale_A, quantized_A = quantize(A, aT)
+            scale_B, quantized_B = quantize(B, not bT)
+        else:
+            scale_A = calc_scale(A, aT)
+            scale_B = calc_scale(B, not bT)
+            quantized_A = round_i8(A, scale_A, aT)
+            quantized_B = round_i8(B, scale_B, not bT)
+        return gemm_and_scale(quantized_A, scale_A, quantized_B, scale_B, aT, bT, fused)
+
+
+class GEMMFloat(InferenceOnly):
+    @staticmethod
+    def forward(ctx, A: torch.Tensor, aT: bool, B: torch.Tensor, bT: bool):
+        """fp16 product through the vendor BLAS (the reference calls cuBLASLt here,
+        torch/gemm.py:159-231); not a hand-written kernel and not on the int8 path."""
+        assert A.is_cuda and B.is_cuda and A.device == B.device
+        assert A.dtype == B.dtype
+        a = A.transpose(-1, -2) if aT else A
+        b = B.transpose(-1, -2) if bT else B
+        return torch.matmul(a, b)
+
+
+def bmm(A: torch.Tensor, aT: bool, B: torch.Tensor, bT: bool, int8: bool = False, fused: bool = True) -> torch.Tensor:
+    assert A.ndim == 3
+    assert B.ndim == 3
+    if int8:
+        return GEMMInt8.apply(A, aT, B, bT, fused)
+    return GEMMFloat.apply(A, aT, B, bT)

@@ -1,0 +1,34 @@
+"""Padding mask with the interface of cpm_kernels/torch/mask.py (forward only)."""
+import torch
+from ..kernels import mask as mask_kernel
+from ._common import cur_stream, check_half, InferenceOnly
+
+
+def _check(x, mask):
+    check_half(x, 3)
+    assert mask.is_contiguous() and mask.is_cuda and mask.dtype == torch.bool and mask.ndim == 2
+    assert x.device == mask.device
+    assert mask.size() == (x.size(0), x.size(2))
+
+
+class OpMask(InferenceOnly):
+    @staticmethod
+    def forward(ctx, x: torch.Tensor, mask: torch.Tensor, value: float) -> torch.Tensor:
+        _check(x, mask)
+        out = torch.empty(x.size(), dtype=torch.float16, device=x.device)
+        mask_kernel(x.size(0), x.size(1), x.size(2), x.data_ptr(), mask.data_ptr(), value, out.data_ptr(),
+                    cur_stream())
+        return out
+
+
+def mask(x: torch.Tensor, mask: torch.Tensor, value: float) -> torch.Tensor:
+    return OpMask.apply(x, mask, value)
+
+
+def mask_inplace(x: torch.Tensor, mask: torch.Tensor, value: float) -> None:
+    _check(x, mask)
+    mask_kernel(x.size(0), x.size(1), x.size(2), x.data_ptr(), mask.data_ptr(), value, x.data_ptr(), cur_stream())
+
+
+def maskTH(x: torch.Tensor, mask: torch.Tensor, value: float) -> torch.Tensor:
+    return torch.where(mask[:, None, :], x, torch.scalar_tensor(value, device=x.device, dtype=x.dtype))

@@ -1,0 +1,497 @@
+"""GPU parity: every HIP kernel, called through the C ABI (cpm_kernels_amd.kernels -> ctypes ->
+libcpmk_hip.so), against the CPU oracle on the same seeded inputs.
+
+Bars (from the path's contract): bit-exact for scales, int8 rounding, int32 accumulators,
+dequantised outputs (the multiplication order is fixed, so they can be), position buckets,
+bias gather and the fp16 elementwise helpers; |a-e| <= 1e-3*|e| + atol for layernorm, softmax
+and gelu, with atol stated at each test.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import cpm_kernels_amd.kernels as ck
+from util import stream, to_gpu, to_np, assert_bits_equal, assert_close_fp16, rand_half
+
+pytestmark = pytest.mark.gpu
+
+
+def _name(*a):
+    print("case", *a, flush=True)
+
+
+# ---------------------------------------------------------------------------------------------
+# quantisation
+# ---------------------------------------------------------------------------------------------
+def adversarial_rows(rng, n, m):
+    """Rows that stress the rounding contract: zeros, one huge value, subnormal-scale rows,
+    exact .5 ties, constant rows, +-max fp16."""
+    x = rand_half(rng, (n, m))
+    if n >= 8 and m >= 8:
+        x[0] = 0
+        x[1] = 0; x[1, m // 2] = 65504
+        x[2] = (rng.standard_normal(m) * 1e-5).astype(np.float16)          # absmax < 9e-4 -> subnormal scale
+        x[3] = np.float16(6e-8)                                            # scale underflows to 0
+        # ties: scale = 1/127*127 ... choose absmax 127 -> scale 1.0 exactly, values k+0.5
+        x[4] = (rng.integers(-126, 126, m) + 0.5).astype(np.float16); x[4, 0] = 127
+        x[5] = np.float16(-3.0)
+        x[6] = rand_half(rng, (m,), 100.0); x[6, -1] = -65504
+        x[7] = rand_half(rng, (m,), 0.02)
+    return x
+
+
+QUANT_SHAPES = [(1, 512, 4096), (3, 17, 1000), (2, 5, 7), (1, 1, 8), (2, 64, 48), (1, 9, 8200), (4, 33, 16),
+                (1, 2100, 128), (1, 3, 20480)]
+
+
+@pytest.mark.parametrize("shape", QUANT_SHAPES)
+def test_calc_scale_and_round(gpu, shape):
+    _name("calc_scale/round", shape)
+    b, n, m = shape
+    rng = np.random.default_rng(b * 1000003 + n * 1009 + m)
+    x = np.stack([adversarial_rows(rng, n, m) for _ in range(b)])
+    xd = to_gpu(x)
+    sd = torch.empty((b, n), dtype=torch.half, device=gpu)
+    ck.gemm_calc_scale(b, n, m, xd.data_ptr(), sd.data_ptr(), stream())
+    s_ref = oracle.gemm_calc_scale(x)
+    assert_bits_equal(to_np(sd), s_ref, "gemm_calc_scale %s" % (shape,))
+    qd = torch.empty((b, n, m), dtype=torch.int8, device=gpu)
+    ck.gemm_round(b, n, m, xd.data_ptr(), sd.data_ptr(), qd.data_ptr(), stream())
+    assert_bits_equal(to_np(qd), oracle.gemm_round(x, s_ref), "gemm_round %s" % (shape,))
+    # fused launcher == the two launches
+    s2 = torch.empty_like(sd); q2 = torch.empty_like(qd)
+    ck.gemm_quantize(b, n, m, xd.data_ptr(), s2.data_ptr(), q2.data_ptr(), False, stream())
+    assert_bits_equal(to_np(s2), s_ref, "gemm_quantize scale")
+    assert_bits_equal(to_np(q2), to_np(qd), "gemm_quantize int8")
+    # gemv forms are the same arithmetic on (batch*n, m)
+    sv = torch.empty((b * n,), dtype=torch.half, device=gpu)
+    ck.gemv_calc_scale(b * n, m, xd.data_ptr(), sv.data_ptr(), stream())
+    assert_bits_equal(to_np(sv), s_ref.reshape(-1), "gemv_calc_scale")
+    qv = torch.empty((b * n, m), dtype=torch.int8, device=gpu)
+    ck.gemv_round(b * n, m, xd.data_ptr(), sv.data_ptr(), qv.data_ptr(), stream())
+    assert_bits_equal(to_np(qv).reshape(b, n, m), to_np(qd), "gemv_round")
+
+
+@pytest.mark.parametrize("shape", QUANT_SHAPES)
+def test_calc_scale_and_round_transpose(gpu, shape):
+    _name("calc_scale_transpose/round_transpose", shape)
+    b, n, m = shape
+    rng = np.random.default_rng(7 + b * 1000003 + n * 1009 + m)
+    # adversarial columns: build on the transposed view
+    x = np.stack([np.ascontiguousarray(adversarial_rows(rng, m, n).T) for _ in range(b)])
+    xd = to_gpu(x)
+    sd = torch.empty((b, m), dtype=torch.half, device=gpu)
+    ck.gemm_calc_scale_transpose(b, n, m, xd.data_ptr(), sd.data_ptr(), stream())
+    s_ref = oracle.gemm_calc_scale_transpose(x)
+    assert_bits_equal(to_np(sd), s_ref, "gemm_calc_scale_transpose %s" % (shape,))
+    qd = torch.empty((b, n, m), dtype=torch.int8, device=gpu)
+    ck.gemm_round_transpose(b, n, m, xd.data_ptr(), sd.data_ptr(), qd.data_ptr(), stream())
+    assert_bits_equal(to_np(qd), oracle.gemm_round_transpose(x, s_ref), "gemm_round_transpose %s" % (shape,))
+    s2 = torch.empty_like(sd); q2 = torch.empty_like(qd)
+    ck.gemm_quantize(b, n, m, xd.data_ptr(), s2.data_ptr(), q2.data_ptr(), True, stream())
+    assert_bits_equal(to_np(s2), s_ref, "gemm_quantize(T) scale")
+    assert_bits_equal(to_np(q2), to_np(qd), "gemm_quantize(T) int8")
+    # invariant: transposed forms == row forms on the transposed tensor
+    xt = np.ascontiguousarray(x.transpose(0, 2, 1))
+    assert_bits_equal(s_ref, oracle.gemm_calc_scale(xt), "transpose invariant (scale)")
+
+
+def test_round_unaligned_views(gpu):
+    """Pointers that are only 2-byte aligned take the scalar kernels."""
+    _name("round unaligned")
+    rng = np.random.default_rng(5)
+    x = rand_half(rng, (1, 6, 40))
+    buf = torch.empty(x.size + 1, dtype=torch.half, device=gpu)
+    buf[1:] = to_gpu(x).reshape(-1)
+    sd = torch.empty((1, 6), dtype=torch.half, device=gpu)
+    ck.gemm_calc_scale(1, 6, 40, buf.data_ptr() + 2, sd.data_ptr(), stream())
+    assert_bits_equal(to_np(sd), oracle.gemm_calc_scale(x), "unaligned calc_scale")
+    qd = torch.empty((1, 6, 40), dtype=torch.int8, device=gpu)
+    ck.gemm_round(1, 6, 40, buf.data_ptr() + 2, sd.data_ptr(), qd.data_ptr(), stream())
+    assert_bits_equal(to_np(qd), oracle.gemm_round(x, oracle.gemm_calc_scale(x)), "unaligned round")
+
+
+@pytest.mark.parametrize("shape,bcx,bcy", [((1, 512, 4096), True, True), ((3, 20, 44), False, False),
+                                          ((3, 20, 44), True, False), ((2, 7, 13), False, True),
+                                          ((4, 128, 256), False, True)])
+def test_gemm_scale(gpu, shape, bcx, bcy):
+    _name("gemm_scale", shape, bcx, bcy)
+    b, n, m = shape
+    rng = np.random.default_rng(11 + n + m)
+    acc = rng.integers(-2 ** 27, 2 ** 27, shape, dtype=np.int64).astype(np.int32)   # > 2^24: int->float rounds
+    acc[0, 0, :4] = [0, 1, -1, 2 ** 31 - 1]
+    sx = (rng.random((n if bcx else b * n,)) * 0.05 + 1e-4).astype(np.float16)
+    sy = (rng.random((m if bcy else b * m,)) * 0.01 + 1e-5).astype(np.float16)
+    accd, sxd, syd = to_gpu(acc), to_gpu(sx), to_gpu(sy)
+    out = torch.empty(shape, dtype=torch.half, device=gpu)
+    ck.gemm_scale(b, n, m, accd.data_ptr(), sxd.data_ptr(), syd.data_ptr(), out.data_ptr(), bcx, bcy, stream())
+    assert_bits_equal(to_np(out), oracle.gemm_scale(acc, sx, sy, bcx, bcy), "gemm_scale")
+    if not bcx:
+        ck.gemm_scale_x(b, n, m, accd.data_ptr(), sxd.data_ptr(), out.data_ptr(), stream())
+        assert_bits_equal(to_np(out), oracle.gemm_scale_x(acc, sx), "gemm_scale_x")
+    if not bcy:
+        ck.gemm_scale_y(b, n, m, accd.data_ptr(), syd.data_ptr(), out.data_ptr(), stream())
+        assert_bits_equal(to_np(out), oracle.gemm_scale_y(acc, sy), "gemm_scale_y")
+
+
+# ---------------------------------------------------------------------------------------------
+# int8 GEMM: shapes of the reference's TEST_CASES (tests/test_gemm.py:43-60), every transpose
+# combination, broadcast on either side; plus tile-boundary shapes.
+# ---------------------------------------------------------------------------------------------
+GEMM_CASES = [  # (batch, M, K, N) in the reference's bmm naming: kernel m = N, n = M
+    (1, 4, 4, 4), (2, 4, 4, 4), (1, 8, 8, 8), (3, 12, 12, 12), (1, 16, 16, 16), (1, 32, 32, 32),
+    (1, 64, 64, 64), (1, 128, 128, 128), (4, 128, 128, 128), (8, 112, 224, 112),
+    (2, 512, 1024, 2048), (2, 500, 1024, 1996), (2, 512, 2560, 1024), (2, 1024, 512, 1024),
+    (1, 260, 80, 132), (1, 256, 4096, 128), (1, 36, 16, 292),
+]
+
+
+def _gemm_case(gpu, m, k, n, bA, bB, aT, bT, rng, fused_too=True):
+    A = rng.integers(-127, 128, (bA, m, k) if aT else (bA, k, m), dtype=np.int8)
+    B = rng.integers(-127, 128, (bB, k, n) if bT else (bB, n, k), dtype=np.int8)
+    if m * n * k * max(bA, bB) <= 2 ** 22:
+        ref = oracle.gemm_int8(m, k, n, aT, bT, A, B)
+    else:
+        ref = oracle.gemm_int8_blas(m, k, n, aT, bT, A, B)
+    batch = max(bA, bB)
+    Ad, Bd = to_gpu(A), to_gpu(B)
+    out = torch.full((batch, n, m), 12345, dtype=torch.int32, device=gpu)
+    ck.gemm_int8(m, k, n, bA, bB, aT, bT, Ad.data_ptr(), Bd.data_ptr(), out.data_ptr(), stream())
+    what = "gemm_int8 m=%d k=%d n=%d bA=%d bB=%d aT=%d bT=%d" % (m, k, n, bA, bB, aT, bT)
+    assert_bits_equal(to_np(out), ref, what)
+    if fused_too:
+        bcr, bcc = bB == 1, bA == 1
+        srow = (rng.random((n if bcr else batch * n,)) * 0.05 + 1e-4).astype(np.float16)
+        scol = (rng.random((m if bcc else batch * m,)) * 0.01 + 1e-5).astype(np.float16)
+        sr, sc = to_gpu(srow), to_gpu(scol)
+        o16 = torch.empty((batch, n, m), dtype=torch.half, device=gpu)
+        ck.gemm_int8_scale(m, k, n, bA, bB, aT, bT, Ad.data_ptr(), Bd.data_ptr(), sr.data_ptr(), sc.data_ptr(),
+                           bcr, bcc, o16.data_ptr(), stream())
+        assert_bits_equal(to_np(o16), oracle.gemm_scale(ref, srow, scol, bcr, bcc), what + " fused epilogue")
+
+
+@pytest.mark.parametrize("case", GEMM_CASES)
+def test_gemm_int8(gpu, case):
+    batch, M, K, N = case
+    rng = np.random.default_rng(M * 7919 + K * 31 + N)
+    for aT in (False, True):
+        for bT in (False, True):
+            for (bA, bB) in {(batch, batch), (1, batch), (batch, 1)}:
+                _name("gemm_int8", case, aT, bT, bA, bB)
+                _gemm_case(gpu, N, K, M, bA, bB, aT, bT, rng)
+
+
+def test_gemm_int8_extreme_values(gpu):
+    """All operands -128 / 127: largest accumulators the int8 product can produce."""
+    _name("gemm_int8 extremes")
+    m, k, n = 256, 4096, 128
+    for va, vb in ((-128, -128), (127, -128), (127, 127)):
+        A = np.full((1, m, k), va, np.int8); B = np.full((1, n, k), vb, np.int8)
+        out = torch.empty((1, n, m), dtype=torch.int32, device=gpu)
+        Ad, Bd = to_gpu(A), to_gpu(B)
+        ck.gemm_int8(m, k, n, 1, 1, True, False, Ad.data_ptr(), Bd.data_ptr(), out.data_ptr(), stream())
+        assert (to_np(out) == va * vb * k).all()
+
+
+def test_gemm_int8_config1_full(gpu):
+    """BASELINE config 1 at full size (A [1,512,4096], W [1,4096,4096]) through the whole
+    kernel-level pipeline, every stage bit-exact against the oracle."""
+    _name("config1 full pipeline")
+    g = torch.Generator().manual_seed(1001)
+    A = torch.randn(1, 512, 4096, generator=g).half().numpy()
+    W = (torch.randn(1, 4096, 4096, generator=g) * 0.02).half().numpy()
+    sA, sW = oracle.gemm_calc_scale(A), oracle.gemm_calc_scale(W)
+    qA, qW = oracle.gemm_round(A, sA), oracle.gemm_round(W, sW)
+    acc = oracle.gemm_int8_blas(4096, 4096, 512, True, False, qW, qA)
+    ref = oracle.gemm_scale(acc, sA, sW, True, True)
+    Ad, Wd = to_gpu(A), to_gpu(W)
+    sAd = torch.empty((1, 512), dtype=torch.half, device=gpu); sWd = torch.empty((1, 4096), dtype=torch.half, device=gpu)
+    ck.gemm_calc_scale(1, 512, 4096, Ad.data_ptr(), sAd.data_ptr(), stream())
+    ck.gemm_calc_scale(1, 4096, 4096, Wd.data_ptr(), sWd.data_ptr(), stream())
+    qAd = torch.empty((1, 512, 4096), dtype=torch.int8, device=gpu); qWd = torch.empty((1, 4096, 4096), dtype=torch.int8, device=gpu)
+    ck.gemm_round(1, 512, 4096, Ad.data_ptr(), sAd.data_ptr(), qAd.data_ptr(), stream())
+    ck.gemm_round(1, 4096, 4096, Wd.data_ptr(), sWd.data_ptr(), qWd.data_ptr(), stream())
+    assert_bits_equal(to_np(qAd), qA, "qA"); assert_bits_equal(to_np(qWd), qW, "qW")
+    accd = torch.empty((1, 512, 4096), dtype=torch.int32, device=gpu)
+    ck.gemm_int8(4096, 4096, 512, 1, 1, True, False, qWd.data_ptr(), qAd.data_ptr(), accd.data_ptr(), stream())
+    assert_bits_equal(to_np(accd), acc, "int32 accumulators")
+    outd = torch.empty((1, 512, 4096), dtype=torch.half, device=gpu)
+    ck.gemm_scale(1, 512, 4096, accd.data_ptr(), sAd.data_ptr(), sWd.data_ptr(), outd.data_ptr(), True, True, stream())
+    assert_bits_equal(to_np(outd), ref, "dequantised output")
+    # loose check against the fp32 fake-quant formulation of the reference's test (tol 0.5 there)
+    from oracle.formulations import quant_bmm_rowwise
+    loose = quant_bmm_rowwise(torch.from_numpy(A), torch.from_numpy(W)).numpy()
+    assert np.abs(to_np(outd).astype(np.float32) - loose).max() < 0.05
+
+
+def test_gemm_int8_north_star_checksums(gpu):
+    """M=4096, K=4096, N=10240 at full size: the int32 result must reproduce the exact row and
+    column checksums  sum_i out[j,i] = P[j,:] . (sum_i Q[i,:])  and the transpose of that, which
+    any wrong, missing or duplicated tile breaks; plus a random sample of entries."""
+    _name("north-star checksums")
+    M, K, N = 4096, 4096, 10240
+    rng = np.random.default_rng(1000)
+    qA = rng.integers(-127, 128, (1, M, K), dtype=np.int8)      # activations (rows of out)
+    qW = rng.integers(-127, 128, (1, N, K), dtype=np.int8)      # weights (columns of out)
+    out = torch.empty((1, M, N), dtype=torch.int32, device=gpu)
+    qWd, qAd = to_gpu(qW), to_gpu(qA)
+    ck.gemm_int8(N, K, M, 1, 1, True, False, qWd.data_ptr(), qAd.data_ptr(), out.data_ptr(), stream())
+    o = to_np(out)[0].astype(np.int64)
+    a64, w64 = qA[0].astype(np.int64), qW[0].astype(np.int64)
+    assert np.array_equal(o.sum(axis=1), a64 @ w64.sum(axis=0))
+    assert np.array_equal(o.sum(axis=0), w64 @ a64.sum(axis=0))
+    jj = rng.integers(0, M, 2000); ii = rng.integers(0, N, 2000)
+    assert np.array_equal(o[jj, ii], (a64[jj] * w64[ii]).sum(axis=1))
+
+
+# ---------------------------------------------------------------------------------------------
+# decode GEMV
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("batch,dim_out,dim_in", [(32, 10240, 4096), (16, 4444, 8888), (1, 48, 256), (33, 100, 4096),
+                                                  (130, 64, 512), (5, 17, 12), (128, 1000, 1040), (8, 40, 16)])
+def test_gemv_broadcast_mat_int8(gpu, batch, dim_out, dim_in):
+    _name("gemv", batch, dim_out, dim_in)
+    rng = np.random.default_rng(1002 + dim_out)
+    mat = rng.integers(-127, 128, (dim_out, dim_in), dtype=np.int8)
+    vec = rng.integers(-127, 128, (batch, dim_in), dtype=np.int8)
+    sm = (rng.random(dim_out) * 0.009 + 0.001).astype(np.float16)
+    sv = (rng.random(batch) * 0.05 + 0.001).astype(np.float16)
+    # exact reference: fp64 BLAS dot products are exact here, dequant via the oracle's gemm_scale
+    acc = (vec.astype(np.float64) @ mat.astype(np.float64).T).astype(np.int32)[None]     # (1, batch, dim_out)
+    ref = oracle.gemm_scale(acc, sv, sm, True, True)[0]
+    if batch * dim_out * dim_in <= 2 ** 24:
+        assert_bits_equal(oracle.gemv_broadcast_mat_int8(sm, mat, sv, vec), ref, "oracle gemv == gemm path")
+    out = torch.empty((batch, dim_out), dtype=torch.half, device=gpu)
+    md, vd, smd, svd = to_gpu(mat), to_gpu(vec), to_gpu(sm), to_gpu(sv)
+    ck.gemv_broadcast_mat_int8(batch, dim_out, dim_in, smd.data_ptr(), md.data_ptr(), svd.data_ptr(), vd.data_ptr(),
+                               out.data_ptr(), stream())
+    assert_bits_equal(to_np(out), ref, "gemv_broadcast_mat_int8")
+    # the invariant the reference tests (tests/test_gemv.py:49-59): GEMV == GEMM path
+    if batch % 4 or dim_out % 4:
+        return
+    o2 = torch.empty((1, batch, dim_out), dtype=torch.half, device=gpu)
+    ck.gemm_int8_scale(dim_out, dim_in, batch, 1, 1, True, False, md.data_ptr(), vd.data_ptr(), svd.data_ptr(),
+                       smd.data_ptr(), True, True, o2.data_ptr(), stream())
+    assert_bits_equal(to_np(o2)[0], to_np(out), "gemv == gemm_int8_scale")
+
+
+# ---------------------------------------------------------------------------------------------
+# layernorm / softmax / gelu (tolerance ops)
+# ---------------------------------------------------------------------------------------------
+LN_SHAPES = [(8, 4096, 512), (16, 768, 512), (4, 1024, 512), (3, 100, 40), (2, 33, 24), (2, 777, 123), (5, 4096, 1),
+             (1, 5000, 64), (2, 2048, 32), (1, 1536, 8), (2, 64, 72)]
+
+
+@pytest.mark.parametrize("shape", LN_SHAPES)
+@pytest.mark.parametrize("rd_mean", [True, False])
+def test_layernorm_forward(gpu, shape, rd_mean):
+    _name("layernorm", shape, rd_mean)
+    b, n, m = shape
+    rng = np.random.default_rng(1003 + n + m)
+    x = (rng.standard_normal(shape) * rng.uniform(0.5, 3.0) + (0.7 if rd_mean else 0.0)).astype(np.float16)
+    for eps in (1e-5, 1e-3):
+        ref = oracle.layernorm_forward(x, eps, rd_mean)
+        xd = to_gpu(x)
+        out = torch.empty_like(xd)
+        ck.layernorm_forward(b, n, m, xd.data_ptr(), out.data_ptr(), eps, rd_mean, stream())
+        # outputs are O(1); atol 2e-4 covers values next to zero where x - mean cancels
+        assert_close_fp16(to_np(out), ref, rtol=1e-3, atol=2e-4, what="layernorm_forward %s" % (shape,))
+        ck.layernorm_inplace_forward(b, n, m, xd.data_ptr(), eps, rd_mean, stream())
+        assert_bits_equal(to_np(xd), to_np(out), "in place == out of place")
+    if m == 1:   # the reference pins step == forward(m=1) (tests/test_layernorm.py:115-152)
+        xd = to_gpu(x); o2 = torch.empty_like(xd)
+        ck.layernorm_step(b, n, xd.data_ptr(), o2.data_ptr(), 1e-3, rd_mean, stream())
+        assert_bits_equal(to_np(o2), to_np(out), "layernorm_step == forward(m=1)")
+
+
+@pytest.mark.parametrize("shape", [(8, 4096, 512), (3, 100, 40), (2, 777, 124), (2, 1024, 64)])
+@pytest.mark.parametrize("bias", [True, False])
+def test_layernorm_affine_fused(gpu, shape, bias):
+    """Fused norm+affine == layernorm_forward then arith_ln_mul_add / arith_ln_mul, bit for bit."""
+    _name("layernorm affine", shape, bias)
+    b, n, m = shape
+    rng = np.random.default_rng(17 + n)
+    x = rand_half(rng, shape)
+    gamma = (1 + 0.1 * rng.standard_normal(n)).astype(np.float16)
+    beta = (0.1 * rng.standard_normal(n)).astype(np.float16)
+    xd, gd, bd = to_gpu(x), to_gpu(gamma), to_gpu(beta)
+    two = torch.empty_like(xd)
+    ck.layernorm_forward(b, n, m, xd.data_ptr(), two.data_ptr(), 1e-5, bias, stream())
+    normed = to_np(two).copy()
+    if bias:
+        ck.arith_ln_mul_add(b, n, m, two.data_ptr(), gd.data_ptr(), bd.data_ptr(), two.data_ptr(), stream())
+        assert_bits_equal(to_np(two), oracle.arith_ln_mul_add(normed, gamma, beta), "arith_ln_mul_add")
+    else:
+        ck.arith_ln_mul(b, n, m, two.data_ptr(), gd.data_ptr(), two.data_ptr(), stream())
+        assert_bits_equal(to_np(two), oracle.arith_ln_mul(normed, gamma), "arith_ln_mul")
+    one = torch.empty_like(xd)
+    ck.layernorm_affine_forward(b, n, m, xd.data_ptr(), gd.data_ptr(), bd.data_ptr() if bias else None,
+                                one.data_ptr(), 1e-5, bias, stream())
+    assert_bits_equal(to_np(one), to_np(two), "fused == two launches")
+
+
+SOFTMAX_SHAPES = [(1, 2, 32), (4, 128, 128), (4, 128, 16), (4, 123, 16), (16, 1024, 320), (7, 1024, 321),
+                  (3, 512, 64), (2, 2000, 48), (2, 4096, 16), (1, 5000, 24), (6, 333, 1), (2, 64, 200)]
+
+
+@pytest.mark.parametrize("shape", SOFTMAX_SHAPES)
+def test_softmax_forward(gpu, shape):
+    _name("softmax", shape)
+    b, n, m = shape
+    rng = np.random.default_rng(1004 + n + m)
+    x = rand_half(rng, shape, 4.0)
+    if n >= 8 and m >= 4:
+        x[0, : n // 2, 0] = -np.inf              # partially masked column
+        x[0, :, 1] = -np.inf                     # fully masked column -> zeros, not NaN
+        x[0, :, 2] = -np.inf; x[0, n // 3, 2] = 3.0     # one-hot -> exactly 1
+        x[0, :, 3] = np.float16(2.5)             # constant -> 1/n
+    ref = oracle.softmax_forward(x)
+    xd = to_gpu(x); out = torch.empty_like(xd)
+    ck.softmax_forward(b, n, m, xd.data_ptr(), out.data_ptr(), stream())
+    got = to_np(out)
+    # atol 1e-7: about two steps of the fp16 subnormal grid, where tiny probabilities live
+    assert_close_fp16(got, ref, rtol=1e-3, atol=1e-7, max_ulp=2, what="softmax_forward %s" % (shape,))
+    if n >= 8 and m >= 4:
+        assert (got[0, :, 1] == 0).all()
+        assert got[0, n // 3, 2] == 1.0 and got[0, :, 2].sum() == 1.0
+    ck.softmax_inplace_forward(b, n, m, xd.data_ptr(), stream())
+    assert_bits_equal(to_np(xd), got, "in place == out of place")
+    if m == 1:   # tests/test_softmax.py:51-76 of the reference: step == forward(m=1)
+        xs = to_gpu(x)
+        ck.softmax_step_inplace(b, n, xs.data_ptr(), stream())
+        assert_bits_equal(to_np(xs), got, "softmax_step_inplace == forward(m=1)")
+
+
+def test_softmax_causal_full_size_properties(gpu):
+    """Config 3 size, (64, 1024, 1024) slice count reduced to keep the CPU side in seconds:
+    causal -inf above the diagonal; columns sum to 1, masked entries are exactly 0, and a
+    sample of columns matches the oracle."""
+    _name("softmax causal")
+    b, n, m = 64, 1024, 1024
+    g = torch.Generator().manual_seed(1003)
+    s = (torch.randn(b, n, m, generator=g) * 4).half()
+    kk = torch.arange(n)[:, None]; qq = torch.arange(m)[None, :]
+    s.masked_fill_((kk > qq)[None], float("-inf"))
+    xd = s.cuda(); out = torch.empty_like(xd)
+    ck.softmax_forward(b, n, m, xd.data_ptr(), out.data_ptr(), stream())
+    o = out.float()
+    assert torch.all(o.masked_select((kk > qq)[None].cuda()) == 0)
+    assert torch.allclose(o.sum(dim=1), torch.ones(b, m, device=gpu), atol=2e-3)
+    ref = oracle.softmax_forward(s[:2].numpy())
+    assert_close_fp16(to_np(out[:2]), ref, rtol=1e-3, atol=1e-7, max_ulp=2, what="softmax causal sample")
+
+
+def test_gelu_all_fp16_inputs(gpu):
+    _name("gelu exhaustive")
+    x = np.arange(65536, dtype=np.uint16).view(np.float16).reshape(4, 16384)
+    ref = oracle.gelu_forward(x)
+    xd = to_gpu(x); out = torch.empty_like(xd)
+    ck.gelu_forward(4, 16384, xd.data_ptr(), out.data_ptr(), stream())
+    got = to_np(out)
+    # atol 6e-8 = one step of the fp16 subnormal grid (tanhf differs by an ulp between libraries)
+    assert_close_fp16(got, ref, rtol=1e-3, atol=6e-8, max_ulp=1, what="gelu_forward all inputs")
+    ck.gelu_inplace_forward(4, 16384, xd.data_ptr(), stream())
+    assert_bits_equal(to_np(xd), got, "in place == out of place")
+    # odd length / unaligned tail
+    y = x.reshape(-1)[1000:1000 + 1237].copy().reshape(1, 1237)
+    yd = to_gpu(y); o2 = torch.empty_like(yd)
+    ck.gelu_forward(1, 1237, yd.data_ptr(), o2.data_ptr(), stream())
+    assert_bits_equal(to_np(o2), got.reshape(-1)[1000:1000 + 1237].reshape(1, 1237), "gelu odd length")
+
+
+# ---------------------------------------------------------------------------------------------
+# position bias
+# ---------------------------------------------------------------------------------------------
+POS_CONFIGS = [(32, 12, 128, False), (32, 12, 128, True), (32, 24, 256, True), (128, 64, 128, True),
+               (16, 64, 256, False), (16, 16, 512, True), (32, 64, 128, True)]
+
+
+@pytest.mark.parametrize("cfg", POS_CONFIGS)
+def test_position_embedding(gpu, cfg):
+    _name("position", cfg)
+    num_buckets, heads, max_distance, bidi = cfg
+    table = torch.empty((max_distance,), dtype=torch.int32, device=gpu)
+    ck.position_embedding_init(num_buckets, max_distance, table.data_ptr(), bidi, stream())
+    t_ref = oracle.position_embedding_init(num_buckets, max_distance, bidi)
+    assert_bits_equal(to_np(table), t_ref, "bucket table %s" % (cfg,))
+    rng = np.random.default_rng(1005)
+    w = rand_half(rng, (heads, num_buckets))
+    wd = to_gpu(w)
+    for (ql, kl) in ((128, 128), (77, 200), (1024, 16), (5, 3)):
+        out = torch.empty((heads, kl, ql), dtype=torch.half, device=gpu)
+        ck.position_embedding_forward(ql, kl, num_buckets, max_distance, heads, table.data_ptr(), wd.data_ptr(),
+                                      out.data_ptr(), bidi, stream())
+        ref = oracle.position_embedding_forward(ql, kl, num_buckets, max_distance, t_ref, w, bidi)
+        assert_bits_equal(to_np(out), ref, "position_embedding_forward %s %d %d" % (cfg, ql, kl))
+    o = torch.empty((heads, 300), dtype=torch.half, device=gpu)
+    ck.position_embedding_step(150, 300, num_buckets, max_distance, heads, table.data_ptr(), wd.data_ptr(),
+                               o.data_ptr(), bidi, stream())
+    assert_bits_equal(to_np(o), oracle.position_embedding_step(150, 300, num_buckets, max_distance, t_ref, w, bidi),
+                      "position_embedding_step")
+
+
+def test_position_embedding_config5_size(gpu):
+    """64 heads, 1024 x 1024, 32 buckets, max_distance 128, bidirectional: Toeplitz property at
+    full size plus equality with the oracle."""
+    _name("position config5")
+    table = torch.empty((128,), dtype=torch.int32, device=gpu)
+    ck.position_embedding_init(32, 128, table.data_ptr(), True, stream())
+    g = torch.Generator().manual_seed(1005)
+    w = (torch.randn(64, 32, generator=g) * 0.02).half()
+    out = torch.empty((64, 1024, 1024), dtype=torch.half, device=gpu)
+    wd = w.cuda()
+    ck.position_embedding_forward(1024, 1024, 32, 128, 64, table.data_ptr(), wd.data_ptr(), out.data_ptr(), True,
+                                  stream())
+    torch.cuda.synchronize()
+    assert torch.equal(out[:, 1:, 1:], out[:, :-1, :-1])          # depends on q - k only
+    ref = oracle.position_embedding_forward(1024, 1024, 32, 128, oracle.position_embedding_init(32, 128, True),
+                                            w.numpy(), True)
+    assert_bits_equal(to_np(out), ref, "config 5 bias")
+
+
+# ---------------------------------------------------------------------------------------------
+# elementwise helpers
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("shape", [(8, 4096, 512), (3, 33, 10), (2, 5, 1232)])
+def test_elementwise(gpu, shape):
+    _name("elementwise", shape)
+    b, n, m = shape
+    rng = np.random.default_rng(23 + m)
+    x = rand_half(rng, shape, 30.0); y = rand_half(rng, shape, 0.01)
+    alpha = rand_half(rng, (n,), 2.0); beta = rand_half(rng, (n,), 5.0)
+    xd, yd, ad, bd = to_gpu(x), to_gpu(y), to_gpu(alpha), to_gpu(beta)
+    out = torch.empty_like(xd)
+    ck.arith_ln_mul_add(b, n, m, xd.data_ptr(), ad.data_ptr(), bd.data_ptr(), out.data_ptr(), stream())
+    assert_bits_equal(to_np(out), oracle.arith_ln_mul_add(x, alpha, beta), "arith_ln_mul_add")
+    ck.arith_ln_mul(b, n, m, xd.data_ptr(), ad.data_ptr(), out.data_ptr(), stream())
+    assert_bits_equal(to_np(out), oracle.arith_ln_mul(x, alpha), "arith_ln_mul")
+    ck.arith_element_add(b, n * m, xd.data_ptr(), yd.data_ptr(), out.data_ptr(), stream())
+    assert_bits_equal(to_np(out), oracle.arith_element_add(x, y), "arith_element_add")
+    msk = rng.random((b, m)) < 0.7
+    md = to_gpu(msk)
+    for value in (float("-inf"), 0.0, 1.5):
+        ck.mask(b, n, m, xd.data_ptr(), md.data_ptr(), value, out.data_ptr(), stream())
+        assert_bits_equal(to_np(out), oracle.mask(x, msk, value), "mask value=%r" % value)
+
+
+def test_error_codes(gpu):
+    """Bad arguments come back as RuntimeError from the C ABI / AssertionError from the asserts
+    the reference has (kernels/gemm.py:139-140, gemv.py:65, arith.py:53,146)."""
+    _name("errors")
+    from cpm_kernels_amd.library import cpmk
+    t = torch.zeros(64, dtype=torch.int8, device=gpu)
+    with pytest.raises(AssertionError):
+        ck.gemm_int8(6, 4, 4, 1, 1, False, False, t.data_ptr(), t.data_ptr(), t.data_ptr(), stream())
+    with pytest.raises(AssertionError):
+        ck.gemm_int8(4, 4, 4, 2, 3, False, False, t.data_ptr(), t.data_ptr(), t.data_ptr(), stream())
+    with pytest.raises(AssertionError):
+        ck.gemv_broadcast_mat_int8(1, 4, 6, 0, 0, 0, 0, 0, stream())
+    with pytest.raises(RuntimeError, match="divisibility"):
+        cpmk.gemm_int8(6, 4, 4, 1, 1, 0, 0, t.data_ptr(), t.data_ptr(), t.data_ptr(), None)
+    with pytest.raises(RuntimeError, match="invalid argument"):
+        cpmk.gemm_calc_scale(-1, 4, 4, t.data_ptr(), t.data_ptr(), None)
+    # empty problems are no-ops
+    ck.gemm_calc_scale(0, 4, 4, 0, 0, stream())
+    ck.softmax_forward(2, 0, 4, 0, 0, stream())
+    ck.gelu_forward(0, 16, 0, 0, stream())
