@@ -107,6 +107,10 @@ __device__ inline half_t dequant(int32_t acc, float sx, float sy) {
 }
 
 // ---- host-side launch helpers ----------------------------------------------------------
+// hipGetLastError() is sticky per host thread: an error left behind by an unrelated runtime
+// call (for instance a failed device probe of another library) would otherwise be reported
+// by the first launcher that asks.  Every launcher therefore clears it on entry.
+inline void clear_stale_error() { (void)hipGetLastError(); }
 inline int launch_status() { return (int)hipGetLastError(); }
 
 // Map a linear workgroup index so that consecutive logical tiles land on the same XCD.

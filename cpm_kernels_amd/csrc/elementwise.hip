@@ -103,6 +103,7 @@ using namespace cpmk;
 extern "C" {
 
 int cpmk_gelu_forward(int32_t batch, int32_t n, const void* mat, void* out, void* stream) {
+    clear_stale_error();
     if (batch < 0 || n < 0) return CPMK_EBADARG;
     const int64_t total = (int64_t)batch * n;
     if (total == 0) return 0;
@@ -132,16 +133,19 @@ static int ln_affine(int32_t batch, int32_t n, int32_t m, const void* inp, const
 
 int cpmk_arith_ln_mul_add(int32_t batch, int32_t n, int32_t m, const void* inp, const void* alpha,
                           const void* beta, void* out, void* stream) {
+    clear_stale_error();
     if (beta == nullptr) return CPMK_EBADARG;
     return ln_affine(batch, n, m, inp, alpha, beta, out, (hipStream_t)stream);
 }
 
 int cpmk_arith_ln_mul(int32_t batch, int32_t n, int32_t m, const void* inp, const void* alpha, void* out,
                       void* stream) {
+    clear_stale_error();
     return ln_affine(batch, n, m, inp, alpha, nullptr, out, (hipStream_t)stream);
 }
 
 int cpmk_arith_element_add(int32_t batch, int32_t n, const void* x, const void* y, void* out, void* stream) {
+    clear_stale_error();
     if (batch < 0 || n < 0) return CPMK_EBADARG;
     if (n % 2) return CPMK_EALIGN;   // kernels/arith.py:53
     const int64_t total = (int64_t)batch * n;
@@ -155,6 +159,7 @@ int cpmk_arith_element_add(int32_t batch, int32_t n, const void* x, const void* 
 
 int cpmk_mask(int32_t batch, int32_t n, int32_t m, const void* inp, const void* mask, float value, void* out,
               void* stream) {
+    clear_stale_error();
     if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
     const int64_t total = (int64_t)batch * n * m;
     if (total == 0) return 0;

@@ -300,6 +300,7 @@ extern "C" {
 
 int cpmk_gemm_int8(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_t batchB, int aT, int bT,
                    const void* A, const void* B, void* out, void* stream) {
+    clear_stale_error();
     return gemm_dispatch<false>(m, k, n, batchA, batchB, aT, bT, A, B, nullptr, nullptr, 0, 0, out,
                                 (hipStream_t)stream);
 }
@@ -307,6 +308,7 @@ int cpmk_gemm_int8(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_t batc
 int cpmk_gemm_int8_scale(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_t batchB, int aT, int bT,
                          const void* A, const void* B, const void* scale_row, const void* scale_col,
                          int broad_cast_row, int broad_cast_col, void* out, void* stream) {
+    clear_stale_error();
     return gemm_dispatch<true>(m, k, n, batchA, batchB, aT, bT, A, B, scale_row, scale_col, broad_cast_row,
                                broad_cast_col, out, (hipStream_t)stream);
 }

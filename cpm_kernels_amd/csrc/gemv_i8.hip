@@ -148,6 +148,7 @@ using namespace cpmk;
 extern "C" int cpmk_gemv_broadcast_mat_int8(int32_t batch, int32_t dim_out, int32_t dim_in,
                                             const void* scale_mat, const void* mat, const void* scale_vec,
                                             const void* vec, void* out, void* stream) {
+    clear_stale_error();
     if (batch < 0 || dim_out < 0 || dim_in < 0) return CPMK_EBADARG;
     if (dim_in % 4) return CPMK_EALIGN;   // kernels/gemv.py:65
     if (batch == 0 || dim_out == 0) return 0;

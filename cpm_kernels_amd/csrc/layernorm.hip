@@ -152,7 +152,6 @@ static bool launch_tile_r(int r, int32_t batch, int32_t n, int32_t m, const half
     else if (r <= 2) launch_tile<LPR, 2>(batch, n, m, mat, out, alpha, beta, eps, rd_mean, st);
     else if (r <= 4) launch_tile<LPR, 4>(batch, n, m, mat, out, alpha, beta, eps, rd_mean, st);
     else if (r <= 8) launch_tile<LPR, 8>(batch, n, m, mat, out, alpha, beta, eps, rd_mean, st);
-    else if (r <= 16) launch_tile<LPR, 16>(batch, n, m, mat, out, alpha, beta, eps, rd_mean, st);
     else return false;
     return true;
 }
@@ -170,7 +169,7 @@ static int layernorm_dispatch(int32_t batch, int32_t n, int32_t m, const void* m
         return launch_status();
     }
     if (m % 8 == 0 && aligned16(mat) && aligned16(out)) {
-        // widest row segment whose tile still fits the register budget (R <= 8 preferred)
+        // widest row segment whose tile still fits the register budget (at most 8 pieces per lane)
         bool ok = false;
         if (n <= 128 * 8 && m >= 64) ok = launch_tile_r<8>((int)ceil_div(n, 128), batch, n, m, x, y, al, be, eps, rd_mean, st);
         else if (n <= 256 * 8 && m >= 32) ok = launch_tile_r<4>((int)ceil_div(n, 256), batch, n, m, x, y, al, be, eps, rd_mean, st);
@@ -191,17 +190,20 @@ extern "C" {
 
 int cpmk_layernorm_forward(int32_t batch, int32_t n, int32_t m, const void* mat, void* out, float eps,
                            int rd_mean, void* stream) {
+    clear_stale_error();
     return layernorm_dispatch(batch, n, m, mat, out, nullptr, nullptr, eps, rd_mean, (hipStream_t)stream);
 }
 
 int cpmk_layernorm_affine_forward(int32_t batch, int32_t n, int32_t m, const void* mat, const void* alpha,
                                   const void* beta, void* out, float eps, int rd_mean, void* stream) {
+    clear_stale_error();
     if (alpha == nullptr) return CPMK_EBADARG;
     return layernorm_dispatch(batch, n, m, mat, out, alpha, beta, eps, rd_mean, (hipStream_t)stream);
 }
 
 int cpmk_layernorm_step(int32_t batch, int32_t n, const void* mat, void* out, float eps, int rd_mean,
                         void* stream) {
+    clear_stale_error();
     if (batch < 0 || n < 0) return CPMK_EBADARG;
     if ((int64_t)batch * n == 0) return 0;
     hipLaunchKernelGGL(k_layernorm_rows, dim3((unsigned)batch), dim3(256), 0, (hipStream_t)stream, n,

@@ -76,6 +76,7 @@ extern "C" {
 
 int cpmk_position_embedding_init(int32_t num_buckets, int32_t max_distance, void* out, int bidirectional,
                                  void* stream) {
+    clear_stale_error();
     if (num_buckets < (bidirectional ? 4 : 2) || max_distance < 0) return CPMK_EBADARG;
     if (max_distance == 0) return 0;
     hipLaunchKernelGGL(k_position_init, dim3((unsigned)ceil_div(max_distance, 256)), dim3(256), 0,
@@ -86,6 +87,7 @@ int cpmk_position_embedding_init(int32_t num_buckets, int32_t max_distance, void
 int cpmk_position_embedding_forward(int32_t query_len, int32_t key_len, int32_t num_buckets, int32_t max_distance,
                                     int32_t num_heads, const void* position_mapping, const void* weight, void* out,
                                     int bidirectional, void* stream) {
+    clear_stale_error();
     if (query_len < 0 || key_len < 0 || num_heads < 0 || num_buckets <= 0 || max_distance <= 0) return CPMK_EBADARG;
     if ((int64_t)query_len * key_len * num_heads == 0) return 0;
     if (num_heads > 65535) return CPMK_ETOOBIG;
@@ -101,6 +103,7 @@ int cpmk_position_embedding_forward(int32_t query_len, int32_t key_len, int32_t 
 int cpmk_position_embedding_step(int32_t query_pos, int32_t key_len, int32_t num_buckets, int32_t max_distance,
                                  int32_t num_heads, const void* position_mapping, const void* weight, void* out,
                                  int bidirectional, void* stream) {
+    clear_stale_error();
     if (key_len < 0 || num_heads < 0 || num_buckets <= 0 || max_distance <= 0) return CPMK_EBADARG;
     if ((int64_t)key_len * num_heads == 0) return 0;
     hipLaunchKernelGGL(k_position_step, dim3((unsigned)ceil_div(key_len, 256)), dim3(256), 0, (hipStream_t)stream,

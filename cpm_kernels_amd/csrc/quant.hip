@@ -291,17 +291,20 @@ using namespace cpmk;
 extern "C" {
 
 int cpmk_gemm_calc_scale(int32_t batch, int32_t n, int32_t m, const void* mat, void* out, void* stream) {
+    clear_stale_error();
     if (int e = check3(batch, n, m)) return e;
     return row_absmax((int64_t)batch * n, m, mat, out, (hipStream_t)stream);
 }
 
 int cpmk_gemv_calc_scale(int32_t batch, int32_t n, const void* vec, void* out, void* stream) {
+    clear_stale_error();
     if (batch < 0 || n < 0) return CPMK_EBADARG;
     return row_absmax(batch, n, vec, out, (hipStream_t)stream);
 }
 
 int cpmk_gemm_calc_scale_transpose(int32_t batch, int32_t n, int32_t m, const void* mat, void* out,
                                    void* stream) {
+    clear_stale_error();
     if (int e = check3(batch, n, m)) return e;
     if (batch == 0 || m == 0) return 0;
     const bool vec = (m % 8 == 0) && aligned16(mat);
@@ -313,41 +316,48 @@ int cpmk_gemm_calc_scale_transpose(int32_t batch, int32_t n, int32_t m, const vo
 
 int cpmk_gemm_round(int32_t batch, int32_t n, int32_t m, const void* mat, const void* scale, void* out,
                     void* stream) {
+    clear_stale_error();
     if (int e = check3(batch, n, m)) return e;
     return round_launch<0>(batch, n, m, mat, scale, out, (hipStream_t)stream);
 }
 
 int cpmk_gemv_round(int32_t batch, int32_t n, const void* vec, const void* scale, void* out, void* stream) {
+    clear_stale_error();
     if (batch < 0 || n < 0) return CPMK_EBADARG;
     return round_launch<0>(1, batch, n, vec, scale, out, (hipStream_t)stream);
 }
 
 int cpmk_gemm_round_transpose(int32_t batch, int32_t n, int32_t m, const void* mat, const void* scale,
                               void* out, void* stream) {
+    clear_stale_error();
     if (int e = check3(batch, n, m)) return e;
     return round_launch<1>(batch, n, m, mat, scale, out, (hipStream_t)stream);
 }
 
 int cpmk_gemm_scale(int32_t batch, int32_t n, int32_t m, const void* mat, const void* scale_x,
                     const void* scale_y, void* out, int bcx, int bcy, void* stream) {
+    clear_stale_error();
     if (int e = check3(batch, n, m)) return e;
     return dequant_launch<0>(batch, n, m, mat, scale_x, scale_y, out, bcx, bcy, (hipStream_t)stream);
 }
 
 int cpmk_gemm_scale_x(int32_t batch, int32_t n, int32_t m, const void* mat, const void* scale_x, void* out,
                       void* stream) {
+    clear_stale_error();
     if (int e = check3(batch, n, m)) return e;
     return dequant_launch<1>(batch, n, m, mat, scale_x, nullptr, out, 0, 0, (hipStream_t)stream);
 }
 
 int cpmk_gemm_scale_y(int32_t batch, int32_t n, int32_t m, const void* mat, const void* scale_y, void* out,
                       void* stream) {
+    clear_stale_error();
     if (int e = check3(batch, n, m)) return e;
     return dequant_launch<2>(batch, n, m, mat, nullptr, scale_y, out, 0, 0, (hipStream_t)stream);
 }
 
 int cpmk_gemm_quantize(int32_t batch, int32_t n, int32_t m, const void* mat, void* scale, void* out,
                        int transpose, void* stream) {
+    clear_stale_error();
     if (int e = check3(batch, n, m)) return e;
     hipStream_t st = (hipStream_t)stream;
     if (!transpose) {

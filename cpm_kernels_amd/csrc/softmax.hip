@@ -148,10 +148,12 @@ using namespace cpmk;
 extern "C" {
 
 int cpmk_softmax_forward(int32_t batch, int32_t n, int32_t m, const void* inp, void* out, void* stream) {
+    clear_stale_error();
     return softmax_dispatch(batch, n, m, inp, out, (hipStream_t)stream);
 }
 
 int cpmk_softmax_step_inplace(int32_t batch, int32_t n, void* x, void* stream) {
+    clear_stale_error();
     if (batch < 0 || n < 0) return CPMK_EBADARG;
     if ((int64_t)batch * n == 0) return 0;
     hipLaunchKernelGGL(k_softmax_rows, dim3((unsigned)batch), dim3(256), 0, (hipStream_t)stream, n,

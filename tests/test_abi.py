@@ -1,0 +1,160 @@
+"""CPU-only checks of the drop-in boundary: the C-ABI library loads and exports every symbol
+include/cpmk.h declares, the Python layers keep the reference's names and error behaviour, and
+nothing in the product path imports the oracle.  No compute calls (no GPU here)."""
+import ctypes
+import os
+import re
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def header_symbols():
+    text = open(os.path.join(ROOT, "include", "cpmk.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(cpmk_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from cpm_kernels_amd.build import library_path, build_library
+    if not os.path.exists(library_path()):
+        build_library(verbose=False)
+    lib = ctypes.CDLL(library_path())
+    syms = header_symbols()
+    assert len(syms) >= 30
+    for s in syms:
+        assert hasattr(lib, s), "libcpmk_hip.so does not export %s" % s
+    from cpm_kernels_amd.library import cpmk
+    assert sorted(cpmk.EXPORTED_SYMBOLS) == syms, "python binding and header disagree"
+    assert cpmk.version == 10000
+    assert "divisibility" in cpmk.error_string(10002) and cpmk.error_string(0) == "success"
+
+
+# cpm_kernels/kernels/__init__.py:1-14 of the reference exports these names
+REFERENCE_KERNEL_NAMES = """
+embedding_forward embedding_backward_stage1 embedding_backward_stage2 embedding_step
+gelu_forward gelu_backward gelu_inplace_forward
+gemm_calc_scale gemm_calc_scale_transpose gemm_round gemm_round_transpose gemm_scale gemm_fp16 gemm_int8
+gemm_backward_round_scale gemm_backward_scale_round gemm_scale_x gemm_scale_y
+gemv_fp16 gemv_broadcast_mat_int8 gemv_fp16_transpose gemv_broadcast_mat_fp16 gemv_calc_scale gemv_round
+gemv_broadcast_mat_fp16_light gemv_fp16_light gemv_fp16_transpose_light
+mask
+arith_batch_add_backward arith_batch_add_forward arith_element_add arith_ln_add_backward arith_ln_div arith_ln_mul
+arith_ln_mul_add arith_ln_mul_backward arith_ln_sub_div arith_element_mul arith_ln_add arith_batch_mul
+arith_batch_mul_add arith_global_scale
+layernorm_forward layernorm_inplace_forward layernorm_forward_v layernorm_forward_mv layernorm_backward_v
+layernorm_backward_mv layernorm_step layernorm_step_inplace
+position_embedding_init position_embedding_forward position_embedding_backward position_embedding_step
+softmax_forward softmax_backward softmax_inplace_forward softmax_step_inplace
+transpose copy_data_to_kv has_nan_inf
+""".split()
+
+ON_PATH = """gelu_forward gelu_inplace_forward gemm_calc_scale gemm_calc_scale_transpose gemm_round
+gemm_round_transpose gemm_scale gemm_int8 gemm_scale_x gemm_scale_y gemv_broadcast_mat_int8 gemv_calc_scale
+gemv_round mask arith_element_add arith_ln_mul arith_ln_mul_add layernorm_forward layernorm_inplace_forward
+layernorm_step layernorm_step_inplace position_embedding_init position_embedding_forward position_embedding_step
+softmax_forward softmax_inplace_forward softmax_step_inplace""".split()
+
+
+def test_kernel_layer_keeps_reference_names_and_signatures():
+    import inspect
+    import cpm_kernels.kernels as ck
+    import cpm_kernels_amd.kernels as ck2
+    assert ck is ck2
+    for name in REFERENCE_KERNEL_NAMES:
+        assert callable(getattr(ck, name)), name
+    for name in ("array_add", "adjustify_logits", "copy_extend_buffer", "copy_pos_hidden"):
+        assert callable(getattr(ck.utils, name))
+    sig = lambda f: list(inspect.signature(f).parameters)   # noqa: E731
+    assert sig(ck.gemm_int8) == ["m", "k", "n", "batchA", "batchB", "aT", "bT", "A", "B", "out", "stream"]
+    assert sig(ck.gemm_scale) == ["batch", "n", "m", "mat", "scale_x", "scale_y", "out", "broad_cast_x", "broad_cast_y", "stream"]
+    assert sig(ck.gemm_round) == ["batch", "n", "m", "mat", "scale", "out", "stream"]
+    assert sig(ck.gemm_calc_scale) == ["batch", "n", "m", "mat", "out", "stream"]
+    assert sig(ck.gemv_broadcast_mat_int8) == ["batch", "dim_out", "dim_in", "scale_mat", "mat", "scale_vec", "vec", "out", "stream"]
+    assert sig(ck.layernorm_forward) == ["batch", "n", "m", "mat", "out", "eps", "rd_mean", "stream"]
+    assert sig(ck.softmax_forward) == ["batch", "n", "m", "inp", "out", "stream"]
+    assert sig(ck.gelu_forward) == ["batch", "n", "mat", "out", "stream"]
+    assert sig(ck.position_embedding_forward) == ["query_len", "key_len", "num_buckets", "max_distance", "num_heads",
+                                                  "position_mapping", "weight", "out", "bidirectional", "stream"]
+    assert sig(ck.mask) == ["batch", "n", "m", "inp", "mask", "value", "out", "stream"]
+    assert sig(ck.arith_ln_mul_add) == ["batch", "n", "m", "inp", "alpha", "beta", "out", "stream"]
+    # off-path names raise loudly, never no-op
+    for name in sorted(set(REFERENCE_KERNEL_NAMES) - set(ON_PATH)):
+        with pytest.raises(NotImplementedError):
+            getattr(ck, name)()
+
+
+def test_reference_asserts_are_kept():
+    import cpm_kernels_amd.kernels as ck
+    with pytest.raises(AssertionError):          # kernels/gemm.py:139
+        ck.gemm_int8(6, 4, 4, 1, 1, False, False, 0, 0, 0, None)
+    with pytest.raises(AssertionError):          # kernels/gemm.py:140
+        ck.gemm_int8(4, 4, 4, 2, 3, False, False, 0, 0, 0, None)
+    with pytest.raises(AssertionError):          # kernels/gemv.py:65
+        ck.gemv_broadcast_mat_int8(1, 4, 6, 0, 0, 0, 0, 0, None)
+    with pytest.raises(AssertionError):          # kernels/arith.py:53
+        ck.arith_element_add(1, 3, 0, 0, 0, None)
+    with pytest.raises(AssertionError):          # kernels/arith.py:146
+        ck.arith_ln_mul_add(1, 2, 3, 0, 0, 0, 0, None)
+
+
+def test_argument_errors_from_the_c_abi_without_a_gpu():
+    """Argument checks happen before any launch, so they can be exercised on a GPU-less host."""
+    from cpm_kernels_amd.library import cpmk
+    with pytest.raises(RuntimeError, match="HIP Error: cpmk: invalid argument"):
+        cpmk.gemm_calc_scale(-1, 4, 4, None, None, None)
+    with pytest.raises(RuntimeError, match="divisibility"):
+        cpmk.gemv_broadcast_mat_int8(1, 4, 6, None, None, None, None, None, None)
+    with pytest.raises(RuntimeError, match="invalid argument"):
+        cpmk.gemm_int8(4, 4, 4, 2, 3, 0, 0, None, None, None, None)
+    # empty problems return before touching the device
+    cpmk.gemm_round(0, 4, 4, None, None, None, None)
+    cpmk.softmax_forward(1, 0, 4, None, None, None)
+    cpmk.position_embedding_forward(0, 4, 32, 128, 2, None, None, None, 1, None)
+
+
+def test_missing_library_gives_stubs_not_import_errors():
+    """cpm_kernels/library/base.py:67-74 of the reference: an absent library leaves the package
+    importable and every bound call raises RuntimeError('Library ... is not initialized')."""
+    code = ("import cpm_kernels_amd.kernels as ck\n"
+            "from cpm_kernels_amd.library import cpmk\n"
+            "from cpm_kernels_amd.device import num_devices\n"
+            "assert cpmk.version == 0 and not cpmk.lib.loaded and num_devices() == 0\n"
+            "try:\n    ck.gemm_calc_scale(1, 4, 4, 0, 0, None)\n"
+            "except RuntimeError as e:\n    assert 'is not initialized' in str(e); print('STUB-OK')\n")
+    env = dict(os.environ, CPMK_LIBRARY="/nonexistent/libcpmk_hip.so", PYTHONPATH=ROOT)
+    out = subprocess.run([sys.executable, "-c", code], env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert "STUB-OK" in out.stdout, out.stdout
+
+
+def test_product_code_never_touches_the_oracle():
+    bad = []
+    for base, _, files in os.walk(os.path.join(ROOT, "cpm_kernels_amd")):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp")):
+                text = open(os.path.join(base, f)).read()
+                if re.search(r"^\s*(from|import)\s+oracle\b", text, flags=re.M) or "cpmk_oracle" in text:
+                    bad.append(os.path.join(base, f))
+    assert not bad, bad
+    for f in os.listdir(os.path.join(ROOT, "cpm_kernels")):
+        if f.endswith(".py"):
+            assert "oracle" not in open(os.path.join(ROOT, "cpm_kernels", f)).read()
+
+
+def test_torch_layer_imports_and_exports():
+    import cpm_kernels.torch as ct
+    for name in ("bmm", "LayerNorm", "LayerNormTH", "normalize_inplace", "normalizeTH", "softmax", "softmaxTH",
+                 "softmax_inplace", "gelu", "geluTH", "gelu_inplace", "PositionEmbedding", "PositionEmbeddingTH",
+                 "mask", "mask_inplace", "maskTH", "ln_mul_add", "ln_mul", "element_add"):
+        assert hasattr(ct, name), name
+
+
+def test_device_module_without_gpu():
+    from cpm_kernels_amd import device
+    n = device.num_devices()
+    assert n >= 0
+    with pytest.raises(ValueError):
+        device.Device(n)          # one past the end is out of range (the reference accepts it by an off-by-one)
