@@ -11,6 +11,12 @@
 #pragma once
 #include "common.h"
 
+// Column tiles touch row segments shorter than a cache line that neighbouring workgroups
+// complete, so their loads and stores must allocate in L2 (no non-temporal hint).
+#ifndef CPMK_COLTILE_NT
+#define CPMK_COLTILE_NT 0
+#endif
+
 namespace cpmk {
 
 template <int NT, int LPR, int R>
@@ -22,20 +28,26 @@ struct ColTile {
     // LDS floats needed by reduce<NV>: (NW + 1) * COLS * NV
 };
 
-// Load the tile; rows >= n and columns >= m are left as `fill` in every half.
+// Load the tile; rows >= n and columns >= m are left as `fill` in every half.  `base` is the
+// (wave-uniform) start of this batch entry; element offsets inside it are 32-bit, which lets
+// the compiler address with a scalar base plus one VGPR offset instead of holding R 64-bit
+// pointers across the reduction phases (callers guarantee n*m < 2^31).
 template <int NT, int LPR, int R>
 __device__ inline void coltile_load(half8_t (&v)[R], const half_t* base, int32_t n, int32_t m, int32_t col0,
                                     half_t fill) {
     constexpr int RPP = NT / LPR;
     const int rg = threadIdx.x / LPR;
+    const uint32_t off0 = (uint32_t)rg * (uint32_t)m + (uint32_t)col0, stride = (uint32_t)RPP * (uint32_t)m;
 #pragma unroll
     for (int p = 0; p < R; ++p) {
         const int32_t row = p * RPP + rg;
         half8_t x;
 #pragma unroll
         for (int e = 0; e < 8; ++e) x[e] = fill;
-        if (row < n && col0 < m)
-            x = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(base + (int64_t)row * m + col0));
+        if (row < n && col0 < m) {
+            const half8_t* src = reinterpret_cast<const half8_t*>(base + (off0 + p * stride));
+            x = CPMK_COLTILE_NT ? __builtin_nontemporal_load(src) : *src;
+        }
         v[p] = x;
     }
 }
@@ -44,11 +56,15 @@ template <int NT, int LPR, int R>
 __device__ inline void coltile_store(const half8_t (&v)[R], half_t* base, int32_t n, int32_t m, int32_t col0) {
     constexpr int RPP = NT / LPR;
     const int rg = threadIdx.x / LPR;
+    const uint32_t off0 = (uint32_t)rg * (uint32_t)m + (uint32_t)col0, stride = (uint32_t)RPP * (uint32_t)m;
 #pragma unroll
     for (int p = 0; p < R; ++p) {
         const int32_t row = p * RPP + rg;
-        if (row < n && col0 < m)
-            __builtin_nontemporal_store(v[p], reinterpret_cast<half8_t*>(base + (int64_t)row * m + col0));
+        if (row < n && col0 < m) {
+            half8_t* dst = reinterpret_cast<half8_t*>(base + (off0 + p * stride));
+            if (CPMK_COLTILE_NT) __builtin_nontemporal_store(v[p], dst);
+            else *dst = v[p];
+        }
     }
 }
 

@@ -9,14 +9,17 @@
 // the one indexed by the output COLUMN i is called Q; each is either "K-major" (kk
 // contiguous) or "MN-major" (j resp. i contiguous).
 //
-// Fast kernel (k_gemm_kmajor): both operands K-major, k % 16 == 0.  256-thread workgroups,
-// 64-byte K slices staged through double-buffered, XOR-swizzled LDS, v_mfma_i32_32x32x32_i8
-// with the output row operand as MFMA "A" and the output column operand as MFMA "B" so that
-// 32 lanes store 32 consecutive output columns.  Integer accumulation is exact, so any
-// summation order gives the reference's int32 result bit for bit.
-//
-// Generic kernel (k_gemm_generic): any layout, any sizes; LDS tiles + v_dot4_i32_i8.
+// Three kernels, all exact (integer accumulation is order-independent, so the int32 result
+// equals the reference's bit for bit):
+//   k_gemm_dma     both operands K-major, k % 128 == 0: persistent workgroups walk the output
+//                  tiles; global memory goes straight into a two-stage, XOR-swizzled LDS ring
+//                  (global_load_lds_dwordx4), one barrier per 128-byte K slab, fragment double
+//                  buffering, v_mfma_i32_32x32x32_i8 with the operands swapped so that a lane
+//                  owns 4 consecutive output columns (8/16-byte stores).
+//   k_gemm_kmajor  both operands K-major, k % 16 == 0: register-staged 64-byte K slabs.
+//   k_gemm_generic any layout and size: LDS tiles + v_dot4_i32_i8.
 #include "common.h"
+#include <type_traits>
 
 namespace cpmk {
 
@@ -170,6 +173,214 @@ __global__ __launch_bounds__(WAVES_R* WAVES_C * 64) void k_gemm_kmajor(GemmArgs 
 }
 
 // ---------------------------------------------------------------------------------------
+// Persistent LDS-DMA kernel
+// ---------------------------------------------------------------------------------------
+template <int X, int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (X < N) {
+        f(std::integral_constant<int, X>{});
+        static_for<X + 1, N>(f);
+    }
+}
+
+// 16 bytes per lane from global memory straight into LDS.  The LDS address is m0 + lane*16,
+// so one wave instruction fills 1 KB of contiguous LDS; the swizzle is applied by choosing
+// which global chunk each lane fetches.  Inline asm because the compiler would otherwise
+// guard every later LDS read with vmcnt(0), which serialises the prefetch.
+__device__ __forceinline__ void lds_dma16(uint32_t voff, const int8_t* sbase, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr)
+                 : "memory");
+}
+// s_waitcnt vmcnt(N) only (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14)
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+struct DmaArgs {
+    GemmArgs g;
+    int32_t batch;
+    int32_t ntiles;    // tiles per batch entry
+};
+
+// Workgroup = WR x WC waves, wave tile = TR x TC MFMA tiles of 32x32, K slab = BKB bytes.
+// Pipeline per K slab `it` (stage cur = it & 1):
+//   k-steps 0 .. KS-2 : MFMAs of step s while the fragments of step s+1 are read from LDS
+//   s_waitcnt vmcnt(0); barrier     -> slab it+1 has landed in stage nxt for every wave and
+//                                      nobody reads stage cur any more
+//   k-step KS-1       : MFMAs while the step-0 fragments of slab it+1 are read and the DMA of
+//                       slab it+2 is issued into stage cur
+// Past the end of K the slab index is clamped (a redundant load nobody reads), which keeps the
+// loop body free of branches; the compiler then keeps all accumulators in AGPRs.
+template <int WR, int WC, int TR, int TC, int BKB, bool FUSED>
+__global__ __launch_bounds__(WR* WC * 64) void k_gemm_dma(DmaArgs da) {
+    const GemmArgs& a = da.g;
+    constexpr int KS = BKB / 32, CPR = BKB / 16;
+    constexpr int NW = WR * WC, BR = WR * TR * 32, BC = WC * TC * 32;
+    constexpr int STAGE = (BR + BC) * BKB;
+    constexpr int RPI = 1024 / BKB;                // rows per DMA instruction
+    constexpr int NDMA = (BR + BC) / RPI;
+    static_assert(NDMA % NW == 0, "stage must split evenly over the waves");
+    constexpr int CNT = NDMA / NW;
+    constexpr int NM = TR * TC;
+    constexpr int RPW = 256 / BKB;                 // rows per 256-byte bank wrap
+    extern __shared__ __attribute__((aligned(16))) int8_t smem[];
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) int8_t*)smem;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wr = wave / WC, wc = wave % WC;
+    const int lrow = lane & 31, lk = lane >> 5;
+    const int32_t K = a.k;
+    const int nk = K / BKB;
+    auto swz = [](int r) __attribute__((always_inline)) { return (r / RPW) & (CPR - 1); };
+    // fragment offsets for k-step 0; step s reads logical chunk 2s + lk: xor (2s << 4) commutes with the swizzle
+    int offP[TR], offQ[TC];
+#pragma unroll
+    for (int i = 0; i < TR; ++i) {
+        const int r = wr * TR * 32 + i * 32 + lrow;
+        offP[i] = r * BKB + ((lk ^ swz(r)) << 4);
+    }
+#pragma unroll
+    for (int j = 0; j < TC; ++j) {
+        const int r = wc * TC * 32 + j * 32 + lrow;
+        offQ[j] = BR * BKB + r * BKB + ((lk ^ swz(r)) << 4);
+    }
+    const uint32_t total = (uint32_t)da.ntiles * da.batch;
+
+    for (uint32_t round = 0;; ++round) {
+        // workgroup w of G takes item round*G + (w%8)*(G/8) + w/8: the workgroups of one XCD
+        // (w % 8) work on adjacent tiles and share operand slabs in that XCD's L2
+        const uint32_t G = gridDim.x;
+        const uint32_t L = round * G + ((G % 8 == 0) ? (blockIdx.x % 8) * (G / 8) + blockIdx.x / 8 : blockIdx.x);
+        if (L >= total) break;
+        const uint32_t b = L / da.ntiles, t = L - b * da.ntiles;
+        constexpr uint32_t GRP = 4;                // row tiles per raster group
+        const uint32_t group_sz = GRP * a.tiles_c;
+        const uint32_t g = t / group_sz;
+        const uint32_t rows_in_group = min(GRP, (uint32_t)a.tiles_r - g * GRP);
+        const uint32_t tin = t - g * group_sz;
+        const uint32_t tile_r = g * GRP + tin % rows_in_group, tile_c = tin / rows_in_group;
+        const int32_t j0 = tile_r * BR, i0 = tile_c * BC;
+        const int8_t* Pb = a.P + (int64_t)b * a.strideP;
+        const int8_t* Qb = a.Q + (int64_t)b * a.strideQ;
+
+        // this wave's DMA instructions: d -> stage rows [RPI*dd, RPI*dd + RPI), dd = wave + d*NW;
+        // rows past the matrix are clamped (they only feed outputs that are never stored)
+        uint32_t voff[CNT], ldst[CNT];
+        bool isq[CNT];
+#pragma unroll
+        for (int d = 0; d < CNT; ++d) {
+            const int dd = wave + d * NW;
+            const int r = dd * RPI + lane / CPR;
+            const int c = (lane % CPR) ^ swz(r);
+            const bool q = dd * RPI >= BR;
+            isq[d] = q;
+            const int32_t grow = q ? min(i0 + (r - BR), a.m - 1) : min(j0 + r, a.n - 1);
+            voff[d] = (uint32_t)grow * (uint32_t)K + c * 16;
+            ldst[d] = lds_base + dd * 1024;
+        }
+        auto dma1 = [&](auto dc, int kt, int stage) __attribute__((always_inline)) {
+            constexpr int d = decltype(dc)::value;
+            lds_dma16(voff[d], (isq[d] ? Qb : Pb) + (int64_t)kt * BKB, ldst[d] + stage * STAGE);
+        };
+
+        int16_tv acc[TR][TC];
+#pragma unroll
+        for (int i = 0; i < TR; ++i)
+#pragma unroll
+            for (int j = 0; j < TC; ++j)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+        int4_t fp[2][TR], fq[2][TC];
+        auto lfrag1 = [&](auto xc, auto bufc, int stage, int ks) __attribute__((always_inline)) {
+            constexpr int x = decltype(xc)::value, buf = decltype(bufc)::value;
+            if constexpr (x < TR)
+                fp[buf][x] = *reinterpret_cast<const int4_t*>(smem + stage * STAGE + (offP[x] ^ (ks << 5)));
+            else
+                fq[buf][x - TR] = *reinterpret_cast<const int4_t*>(smem + stage * STAGE + (offQ[x - TR] ^ (ks << 5)));
+        };
+        // one k-step: NM MFMAs with NMEM memory operations spread evenly between them, order pinned
+        auto kstep = [&](auto bufc, auto&& memop, auto nmem_c) __attribute__((always_inline)) {
+            constexpr int NMEM = decltype(nmem_c)::value, buf = decltype(bufc)::value;
+            static_for<0, NM>([&](auto xc) __attribute__((always_inline)) {
+                constexpr int x = decltype(xc)::value;
+                constexpr int i = x / TC, j = x % TC;
+                // MFMA "A" = column-operand rows, "B" = row-operand rows: lane l, register e of the
+                // result is output row l%32, column (e/4)*8 + (l/32)*4 + e%4 of the 32x32 tile
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fq[buf][j], fp[buf][i], acc[i][j], 0, 0, 0);
+                constexpr int lo = (x * NMEM) / NM, hi = ((x + 1) * NMEM) / NM;
+                static_for<lo, hi>([&](auto yc) __attribute__((always_inline)) { memop(yc); });
+                __builtin_amdgcn_sched_barrier(0);
+            });
+        };
+        using C0 = std::integral_constant<int, 0>;
+
+        __syncthreads();                 // every wave is done with the ring of the previous tile
+        static_for<0, CNT>([&](auto dc) __attribute__((always_inline)) { dma1(dc, 0, 0); });
+        wait_vmcnt<0>();
+        __syncthreads();
+        static_for<0, CNT>([&](auto dc) __attribute__((always_inline)) { dma1(dc, min(1, nk - 1), 1); });
+        static_for<0, TR + TC>([&](auto xc) __attribute__((always_inline)) { lfrag1(xc, C0{}, 0, 0); });
+
+        for (int it = 0; it < nk; ++it) {
+            const int cur = it & 1, nxt = cur ^ 1;
+            static_for<0, KS - 1>([&](auto ksc) __attribute__((always_inline)) {
+                constexpr int ks = decltype(ksc)::value;
+                kstep(std::integral_constant<int, (ks & 1)>{},
+                      [&](auto xc) __attribute__((always_inline)) {
+                          lfrag1(xc, std::integral_constant<int, ((ks + 1) & 1)>{}, cur, ks + 1);
+                      },
+                      std::integral_constant<int, TR + TC>{});
+            });
+            __builtin_amdgcn_sched_barrier(0);
+            wait_vmcnt<0>();
+            __syncthreads();
+            __builtin_amdgcn_sched_barrier(0);
+            const int kt2 = min(it + 2, nk - 1);
+            kstep(std::integral_constant<int, ((KS - 1) & 1)>{},
+                  [&](auto xc) __attribute__((always_inline)) {
+                      constexpr int x = decltype(xc)::value;
+                      if constexpr (x < TR + TC) lfrag1(xc, std::integral_constant<int, (KS & 1)>{}, nxt, 0);
+                      else dma1(std::integral_constant<int, x - (TR + TC)>{}, kt2, cur);
+                  },
+                  std::integral_constant<int, TR + TC + CNT>{});
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        wait_vmcnt<0>();                 // drain the clamped loads before the ring is reused
+
+        const int64_t obase = (int64_t)b * a.n * a.m;
+#pragma unroll
+        for (int i = 0; i < TR; ++i) {
+            const int32_t row = j0 + wr * TR * 32 + i * 32 + lrow;
+            float sx = 0.0f;
+            if (FUSED && row < a.n) sx = (float)a.srow[a.bc_row ? row : (int64_t)b * a.n + row];
+#pragma unroll
+            for (int j = 0; j < TC; ++j) {
+#pragma unroll
+                for (int g4 = 0; g4 < 4; ++g4) {
+                    const int32_t col = i0 + wc * TC * 32 + j * 32 + g4 * 8 + lk * 4;
+                    if (row < a.n && col < a.m) {      // m % 4 == 0: the four columns are in or out together
+                        const int64_t o = obase + (int64_t)row * a.m + col;
+                        if (FUSED) {
+                            const half4_t sy =
+                                *reinterpret_cast<const half4_t*>(a.scol + (a.bc_col ? 0 : (int64_t)b * a.m) + col);
+                            half4_t h;
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) h[e] = dequant(acc[i][j][g4 * 4 + e], sx, (float)sy[e]);
+                            *reinterpret_cast<half4_t*>(reinterpret_cast<half_t*>(a.out) + o) = h;
+                        } else {
+                            const int4_t v = {acc[i][j][g4 * 4], acc[i][j][g4 * 4 + 1], acc[i][j][g4 * 4 + 2],
+                                              acc[i][j][g4 * 4 + 3]};
+                            *reinterpret_cast<int4_t*>(reinterpret_cast<int32_t*>(a.out) + o) = v;
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
 // Generic path: 64x64 output tile, 32 bytes of K per stage, 256 threads each computing a
 // 4x4 block with v_dot4_i32_i8.  Element-wise guarded loads handle every layout and size.
 // ---------------------------------------------------------------------------------------
@@ -261,6 +472,45 @@ static int launch_kmajor(GemmArgs& a, int batch, hipStream_t st) {
     return launch_status();
 }
 
+static int compute_units() {
+    static int cus[64] = {0};          // per device ordinal, filled on first use
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cus[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cus[dev] = n;
+    }
+    return cus[dev];
+}
+
+template <int WR, int WC, int TR, int TC, int BKB, bool FUSED>
+static int launch_dma(GemmArgs& a, int batch, hipStream_t st) {
+    constexpr int BR = WR * TR * 32, BC = WC * TC * 32;
+    constexpr int smem = 2 * (BR + BC) * BKB;
+    a.tiles_r = (int32_t)ceil_div(a.n, BR);
+    a.tiles_c = (int32_t)ceil_div(a.m, BC);
+    DmaArgs da;
+    da.g = a;
+    da.batch = batch;
+    da.ntiles = a.tiles_r * a.tiles_c;
+    auto kern = k_gemm_dma<WR, WC, TR, TC, BKB, FUSED>;
+    static bool attr_set[64] = {false};       // dynamic LDS above 64 KB must be enabled per device
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    if (dev >= 0 && dev < 64 && !attr_set[dev]) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+        if (e != hipSuccess) return (int)e;
+        attr_set[dev] = true;
+    }
+    const int64_t total = (int64_t)da.ntiles * batch;
+    const int cus = compute_units();
+    dim3 grid((unsigned)(total < cus ? total : cus));
+    hipLaunchKernelGGL(kern, grid, dim3(WR * WC * 64), smem, st, da);
+    return launch_status();
+}
+
 template <bool FUSED>
 static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_t batchB, int aT, int bT,
                          const void* A, const void* B, const void* srow, const void* scol, int bcr,
@@ -280,8 +530,13 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
     a.tiles_r = a.tiles_c = 0;
     const bool p_kmajor = !bT, q_kmajor = aT != 0;
     const bool fast = p_kmajor && q_kmajor && k > 0 && (k % 16 == 0) && aligned16(A) && aligned16(B);
+    if (fast && (k % 128 == 0) && (int64_t)n * k < (1ll << 32) && (int64_t)m * k < (1ll << 32)) {
+        // 256x256 tiles when they give most compute units a tile, else 128x128
+        const int64_t big = ceil_div(n, 256) * ceil_div(m, 256) * batch;
+        if (big * 4 >= compute_units() * 3) return launch_dma<2, 4, 4, 2, 128, FUSED>(a, batch, st);
+        return launch_dma<2, 2, 2, 2, 128, FUSED>(a, batch, st);
+    }
     if (fast) {
-        // tile choice: large tiles when they still give every CU work, else smaller ones
         const int64_t t256 = ceil_div(n, 256) * ceil_div(m, 128) * batch;
         if (t256 >= 256) return launch_kmajor<2, 2, 4, 2, FUSED>(a, batch, st);
         return launch_kmajor<2, 2, 2, 2, FUSED>(a, batch, st);

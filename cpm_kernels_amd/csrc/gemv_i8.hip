@@ -7,14 +7,28 @@
 // is the second operand of v_mfma_i32_16x16x64_i8, so one pass over a 16-row slab of the
 // matrix serves up to 128 vectors.  The sum over k is an exact integer sum, so splitting k
 // over waves and reordering it inside the MFMA cannot change the int32 result.
+//
+// Loading the matrix directly in the MFMA register layout (lane = row) would make every lane of
+// a load instruction touch a different cache line: 64 L1 lookups per instruction, and the vector
+// L1 becomes the bottleneck at about a quarter of the HBM rate.  The fast kernel therefore loads
+// 4 rows x 256 contiguous bytes per instruction (8 cache lines) and transposes 16-row groups
+// into the MFMA layout through 4 KB of wave-private, XOR-swizzled LDS.
 #include "common.h"
+#include <type_traits>
+
+#ifndef CPMK_GEMV_NT
+#define CPMK_GEMV_NT 0
+#endif
 
 namespace cpmk {
 
+// Predicated MFMA kernel for dim_in % 16 == 0 that is not a multiple of 256 (loads in the MFMA
+// layout, zero-filled past the end of k).
 // Workgroup = NW waves, RG*16 consecutive matrix rows, all of k.  k is cut into 256-byte
-// chunks dealt round-robin to the waves; within a chunk lane (r = l%16, q = l/16) owns the
-// 64 contiguous bytes [q*64, q*64+64) of row r as four 16-byte pieces, one MFMA each.  The
-// vector operand uses the same lane -> k assignment, which is all the MFMA needs.
+// chunks dealt round-robin to the waves; a chunk is four 64-byte pieces, one MFMA each, and
+// in piece j lane (r = l%16, q = l/16) reads bytes [j*64 + q*16, +16) of row r -- the four
+// lanes of a row read one contiguous 64-byte sector per instruction.  The vector operand uses
+// the same lane -> k assignment, which is all the MFMA needs.
 template <int NW, int RG, int NB>
 __global__ __launch_bounds__(NW * 64) void k_gemv_mfma(int32_t batch, int32_t dim_out, int32_t dim_in,
                                                        const half_t* __restrict__ scale_mat,
@@ -35,7 +49,7 @@ __global__ __launch_bounds__(NW * 64) void k_gemv_mfma(int32_t batch, int32_t di
 
     const int nchunks = (dim_in + 255) >> 8;
     for (int c = w; c < nchunks; c += NW) {
-        const int32_t kb = c * 256 + q * 64;
+        const int32_t kb = c * 256 + q * 16;
         int4_t wv[RG][4], vv[NB][4];
 #pragma unroll
         for (int g = 0; g < RG; ++g) {
@@ -44,8 +58,9 @@ __global__ __launch_bounds__(NW * 64) void k_gemv_mfma(int32_t batch, int32_t di
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 int4_t v = {0, 0, 0, 0};
-                if (row < dim_out && kb + j * 16 < dim_in)
-                    v = __builtin_nontemporal_load(reinterpret_cast<const int4_t*>(p) + j);
+                if (row < dim_out && kb + j * 64 < dim_in)
+                    v = CPMK_GEMV_NT ? __builtin_nontemporal_load(reinterpret_cast<const int4_t*>(p + j * 64))
+                                     : *reinterpret_cast<const int4_t*>(p + j * 64);
                 wv[g][j] = v;
             }
         }
@@ -56,7 +71,7 @@ __global__ __launch_bounds__(NW * 64) void k_gemv_mfma(int32_t batch, int32_t di
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 int4_t v = {0, 0, 0, 0};
-                if (b < batch && kb + j * 16 < dim_in) v = *(reinterpret_cast<const int4_t*>(p) + j);
+                if (b < batch && kb + j * 64 < dim_in) v = *reinterpret_cast<const int4_t*>(p + j * 64);
                 vv[t][j] = v;
             }
         }
@@ -82,6 +97,108 @@ __global__ __launch_bounds__(NW * 64) void k_gemv_mfma(int32_t batch, int32_t di
 
     // part[tile][row_in_tile*16 + b_in_tile]; thread -> (b, row) with row fastest so a
     // vector's outputs are stored contiguously.
+    for (int idx = tid; idx < RG * NB * 256; idx += NW * 64) {
+        const int rr = idx % (RG * 16), bb = idx / (RG * 16);
+        const int g = rr >> 4, t = bb >> 4;
+        const int32_t s = part[g * NB + t][(rr & 15) * 16 + (bb & 15)];
+        const int32_t row = row0 + rr;
+        if (row < dim_out && bb < batch)
+            out[(int64_t)bb * dim_out + row] = dequant(s, (float)scale_vec[bb], (float)scale_mat[row]);
+    }
+}
+
+// Fast kernel: dim_in % 256 == 0.  Workgroup = NW waves and RG*16 matrix rows; the 256-byte K
+// chunks are dealt round-robin to the waves.  Per chunk a wave loads, fully coalesced,
+// RG*16 matrix rows and NB*16 vectors (lane l: 16-byte chunk l%16 of row l/16 + 4i), then turns
+// each 16-row group into four MFMA operands (piece j: lane (r = l%16, q = l/16) holds bytes
+// [j*64 + q*16, +16) of row r) by writing it to LDS at row*256 + ((chunk ^ row) << 4) and reading
+// it back transposed; both directions are bank-conflict free.  LDS executes one wave's
+// operations in order, so the 4 KB buffer is reused without waits.  Rows and vectors past the
+// end are clamped: they only feed outputs that are never stored.
+template <int NW, int RG, int NB>
+__global__ __launch_bounds__(NW * 64) void k_gemv_coalesced(int32_t batch, int32_t dim_out, int32_t dim_in,
+                                                            const half_t* __restrict__ scale_mat,
+                                                            const int8_t* __restrict__ mat,
+                                                            const half_t* __restrict__ scale_vec,
+                                                            const int8_t* __restrict__ vec,
+                                                            half_t* __restrict__ out) {
+    __shared__ __attribute__((aligned(16))) int8_t tbuf[NW][4096];
+    __shared__ int32_t part[RG * NB][256];
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int r = lane & 15, q = lane >> 4;      // MFMA layout
+    const int x = lane & 15, y4 = lane >> 4;     // load layout
+    const int32_t row0 = blockIdx.x * (RG * 16);
+    int8_t* tb = tbuf[w];
+    int woff[4], roff[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int yy = i * 4 + y4;
+        woff[i] = yy * 256 + ((x ^ yy) << 4);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) roff[j] = r * 256 + (((j * 4 + q) ^ r) << 4);
+    const int8_t* wp[RG][4];
+    const int8_t* vp[NB][4];
+#pragma unroll
+    for (int g = 0; g < RG; ++g)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            wp[g][i] = mat + (int64_t)min(row0 + g * 16 + i * 4 + y4, dim_out - 1) * dim_in + x * 16;
+#pragma unroll
+    for (int t = 0; t < NB; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) vp[t][i] = vec + (int64_t)min(t * 16 + i * 4 + y4, batch - 1) * dim_in + x * 16;
+
+    int4_t acc[RG][NB];
+#pragma unroll
+    for (int g = 0; g < RG; ++g)
+#pragma unroll
+        for (int t = 0; t < NB; ++t) acc[g][t] = int4_t{0, 0, 0, 0};
+
+    const int nchunks = dim_in >> 8;
+    for (int c = w; c < nchunks; c += NW) {
+        int4_t wr[RG][4], vr[NB][4];
+#pragma unroll
+        for (int g = 0; g < RG; ++g)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) wr[g][i] = *reinterpret_cast<const int4_t*>(wp[g][i] + c * 256);
+#pragma unroll
+        for (int t = 0; t < NB; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) vr[t][i] = *reinterpret_cast<const int4_t*>(vp[t][i] + c * 256);
+#pragma unroll
+        for (int g = 0; g < RG; ++g) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) *reinterpret_cast<int4_t*>(tb + woff[i]) = wr[g][i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) wr[g][j] = *reinterpret_cast<const int4_t*>(tb + roff[j]);
+        }
+#pragma unroll
+        for (int t = 0; t < NB; ++t) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) *reinterpret_cast<int4_t*>(tb + woff[i]) = vr[t][i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) vr[t][j] = *reinterpret_cast<const int4_t*>(tb + roff[j]);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int g = 0; g < RG; ++g)
+#pragma unroll
+                for (int t = 0; t < NB; ++t)
+                    acc[g][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wr[g][j], vr[t][j], acc[g][t], 0, 0, 0);
+    }
+
+    for (int idx = tid; idx < RG * NB * 256; idx += NW * 64) (&part[0][0])[idx] = 0;
+    __syncthreads();
+    // accumulator e of lane l: matrix row (l/16)*4 + e, vector l%16 of the 16x16 tile
+#pragma unroll
+    for (int g = 0; g < RG; ++g)
+#pragma unroll
+        for (int t = 0; t < NB; ++t)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) atomicAdd(&part[g * NB + t][(q * 4 + e) * 16 + r], acc[g][t][e]);
+    __syncthreads();
     for (int idx = tid; idx < RG * NB * 256; idx += NW * 64) {
         const int rr = idx % (RG * 16), bb = idx / (RG * 16);
         const int g = rr >> 4, t = bb >> 4;
@@ -127,11 +244,48 @@ __global__ __launch_bounds__(256) void k_gemv_dot4(int32_t batch, int32_t dim_ou
     }
 }
 
+static int gemv_compute_units() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+        cus = n;
+    }
+    return cus;
+}
+
+// Rows per workgroup: as few workgroups as there are compute units when the matrix allows it,
+// because every workgroup re-reads all the vectors (from L2); at most 64 rows.
+template <int NB, int MAXRG>
+static void launch_coalesced(int32_t batch, int32_t dim_out, int32_t dim_in, const half_t* sm, const int8_t* mat,
+                             const half_t* sv, const int8_t* vec, half_t* out, hipStream_t st) {
+    const int64_t groups = ceil_div(dim_out, 16);
+    int rg = (int)ceil_div(groups, gemv_compute_units());
+    if (rg > MAXRG) rg = MAXRG;
+    if (rg < 1) rg = 1;
+    const dim3 grid((unsigned)ceil_div(groups, rg));
+    auto go = [&](auto rgc) {
+        hipLaunchKernelGGL((k_gemv_coalesced<8, decltype(rgc)::value, NB>), grid, dim3(512), 0, st, batch, dim_out, dim_in,
+                           sm, mat, sv, vec, out);
+    };
+    if constexpr (MAXRG >= 4) { if (rg == 4) return go(std::integral_constant<int, 4>{}); }
+    if constexpr (MAXRG >= 3) { if (rg == 3) return go(std::integral_constant<int, 3>{}); }
+    if constexpr (MAXRG >= 2) { if (rg == 2) return go(std::integral_constant<int, 2>{}); }
+    go(std::integral_constant<int, 1>{});
+}
+
 template <int NB>
 static void launch_mfma(int32_t batch, int32_t dim_out, int32_t dim_in, const half_t* sm, const int8_t* mat,
                         const half_t* sv, const int8_t* vec, half_t* out, hipStream_t st) {
     // 32 rows per workgroup halves the L2 traffic for the vectors; keep 16 when that
     // would leave compute units without a workgroup.
+#ifdef CPMK_GEMV_NW
+    hipLaunchKernelGGL((k_gemv_mfma<CPMK_GEMV_NW, CPMK_GEMV_RG, NB>), dim3((unsigned)ceil_div(dim_out, 16 * CPMK_GEMV_RG)),
+                       dim3(64 * CPMK_GEMV_NW), 0, st, batch, dim_out, dim_in, sm, mat, sv, vec, out);
+    return;
+#endif
     if (dim_out >= 32 * 256) {
         hipLaunchKernelGGL((k_gemv_mfma<8, 2, NB>), dim3((unsigned)ceil_div(dim_out, 32)), dim3(512), 0, st,
                            batch, dim_out, dim_in, sm, mat, sv, vec, out);
@@ -170,7 +324,12 @@ extern "C" int cpmk_gemv_broadcast_mat_int8(int32_t batch, int32_t dim_out, int3
         const int8_t* v = V + (int64_t)b0 * dim_in;
         half_t* o = O + (int64_t)b0 * dim_out;
         const half_t* s = sv + b0;
-        if (nb <= 16) launch_mfma<1>(nb, dim_out, dim_in, sm, M, s, v, o, st);
+        if (dim_in % 256 == 0) {
+            if (nb <= 16) launch_coalesced<1, 4>(nb, dim_out, dim_in, sm, M, s, v, o, st);
+            else if (nb <= 32) launch_coalesced<2, 4>(nb, dim_out, dim_in, sm, M, s, v, o, st);
+            else if (nb <= 64) launch_coalesced<4, 2>(nb, dim_out, dim_in, sm, M, s, v, o, st);
+            else launch_coalesced<8, 1>(nb, dim_out, dim_in, sm, M, s, v, o, st);
+        } else if (nb <= 16) launch_mfma<1>(nb, dim_out, dim_in, sm, M, s, v, o, st);
         else if (nb <= 32) launch_mfma<2>(nb, dim_out, dim_in, sm, M, s, v, o, st);
         else if (nb <= 64) launch_mfma<4>(nb, dim_out, dim_in, sm, M, s, v, o, st);
         else launch_mfma<8>(nb, dim_out, dim_in, sm, M, s, v, o, st);

@@ -71,6 +71,93 @@ __global__ __launch_bounds__(NT) void k_layernorm_tile(int32_t n, int32_t m, int
     coltile_store<NT, LPR, R>(v, out + boff, n, m, col0);
 }
 
+// Tall columns (n up to 16 * 1024 with 128-byte row segments).  A register tile can hold
+// 1024 rows of 64 columns; narrower tiles would hold more rows but touch only part of every
+// cache line, and the partial lines cost more L2 bandwidth than HBM has.  So the n rows of a
+// 64-column tile are split over PARTS = ceil(n / 1024) workgroups that run side by side on one
+// XCD: each keeps its own 1024 rows in registers and streams the other parts' rows once, only
+// to accumulate the column statistics (those reads are L2 hits: a sibling fetched or is
+// fetching the same lines).  No workgroup waits for another, so there is nothing to deadlock.
+template <int NT, int R>
+__global__ __launch_bounds__(NT) void k_layernorm_tall(int32_t n, int32_t m, int32_t tiles_per_batch, int32_t parts,
+                                                       const half_t* mat, half_t* out,
+                                                       const half_t* __restrict__ alpha,
+                                                       const half_t* __restrict__ beta, float eps, int rd_mean) {
+    constexpr int LPR = 8;
+    using T = ColTile<NT, LPR, R>;
+    __shared__ float lds[(T::NW + 1) * T::COLS * 2];
+    const uint32_t t = xcd_remap(blockIdx.x, gridDim.x);
+    const uint32_t part = t % parts, tile = t / parts;
+    const uint32_t b = tile / tiles_per_batch, ct = tile - b * tiles_per_batch;
+    const int32_t col0 = ct * T::COLS + (threadIdx.x % LPR) * 8;
+    const int64_t boff = (int64_t)b * n * m;
+    const int32_t own0 = part * T::ROWS;                 // first row this workgroup normalises
+    const int32_t own_n = min(T::ROWS, n - own0);        // > 0 by construction
+
+    half8_t v[R];
+    coltile_load<NT, LPR, R>(v, mat + boff + (int64_t)own0 * m, own_n, m, col0, (half_t)0.0f);
+    float s[16];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) s[e] = 0.0f;
+    // the other parts' rows: statistics only
+    const int rg = threadIdx.x / LPR;
+    if (col0 < m) {
+        for (int32_t r0 = 0; r0 < n; r0 += T::RPP * 4) {
+            half8_t w[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int32_t row = r0 + u * T::RPP + rg;
+                const bool mine = row >= own0 && row < own0 + T::ROWS;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) w[u][e] = (half_t)0.0f;
+                if (row < n && !mine) w[u] = *reinterpret_cast<const half8_t*>(mat + boff + ((uint32_t)row * (uint32_t)m + (uint32_t)col0));
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float x = (float)w[u][e];
+                    s[e] += x;
+                    s[8 + e] += x * x;
+                }
+        }
+    }
+#pragma unroll
+    for (int p = 0; p < R; ++p)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float x = (float)v[p][e];
+            s[e] += x;
+            s[8 + e] += x * x;
+        }
+    coltile_reduce<NT, LPR, 2, false>(s, lds);
+
+    float mean[8], rstd[8];
+    const float fn = (float)n;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        float var = s[8 + e] / fn;
+        mean[e] = 0.0f;
+        if (rd_mean) {
+            mean[e] = s[e] / fn;
+            var -= mean[e] * mean[e];
+        }
+        rstd[e] = rsqrtf(var + eps);
+    }
+#pragma unroll
+    for (int p = 0; p < R; ++p) {
+        half8_t y;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) y[e] = round_f16(((float)v[p][e] - mean[e]) * rstd[e]);
+        if (alpha != nullptr) {
+            const int32_t row = own0 + p * T::RPP + rg;
+            if (row < n) y = affine8(y, alpha[row], beta ? beta[row] : (half_t)0.0f, beta != nullptr);
+        }
+        v[p] = y;
+    }
+    coltile_store<NT, LPR, R>(v, out + boff + (int64_t)own0 * m, own_n, m, col0);
+}
+
 // Generic fallback (any n, m, alignment): 64 columns x 4 row groups per workgroup, two
 // passes over global memory; the statistics are complete before the first store, and each
 // element is re-read by the thread that overwrites it, so out may alias mat.
@@ -168,9 +255,17 @@ static int layernorm_dispatch(int32_t batch, int32_t n, int32_t m, const void* m
         hipLaunchKernelGGL(k_layernorm_rows, dim3((unsigned)batch), dim3(256), 0, st, n, x, y, eps, rd_mean);
         return launch_status();
     }
-    if (m % 8 == 0 && aligned16(mat) && aligned16(out)) {
+    if (m % 8 == 0 && aligned16(mat) && aligned16(out) && (int64_t)n * m < (1ll << 31)) {
         // widest row segment whose tile still fits the register budget (at most 8 pieces per lane)
         bool ok = false;
+        if (n > 128 * 8 && n <= 16 * 1024 && m >= 64 && (const void*)x != (const void*)y) {
+            // tall columns: 64-column tiles, n split over side-by-side workgroups.  Not for in-place
+            // calls: a workgroup would overwrite rows that a sibling still reads for its statistics.
+            const int32_t parts = (int32_t)ceil_div(n, 1024), tiles = (int32_t)ceil_div(m, 64);
+            hipLaunchKernelGGL((k_layernorm_tall<1024, 8>), dim3((unsigned)((int64_t)tiles * batch * parts)), dim3(1024), 0,
+                               st, n, m, tiles, parts, x, y, al, be, eps, rd_mean);
+            return launch_status();
+        }
         if (n <= 128 * 8 && m >= 64) ok = launch_tile_r<8>((int)ceil_div(n, 128), batch, n, m, x, y, al, be, eps, rd_mean, st);
         else if (n <= 256 * 8 && m >= 32) ok = launch_tile_r<4>((int)ceil_div(n, 256), batch, n, m, x, y, al, be, eps, rd_mean, st);
         else ok = launch_tile_r<2>((int)ceil_div(n, 512), batch, n, m, x, y, al, be, eps, rd_mean, st);

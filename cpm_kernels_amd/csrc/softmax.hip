@@ -12,6 +12,12 @@ constexpr float kLog2e = 1.4426950408889634f;
 // exp(x - M) as one fma and one v_exp_f32: exp2(x*log2e - M*log2e).
 __device__ inline float exp_shift(float x, float mlog2e) { return __builtin_amdgcn_exp2f(__builtin_fmaf(x, kLog2e, -mlog2e)); }
 
+// Register-resident column tile: HBM is read once and exp is evaluated once per element.  The
+// kernel is co-limited by HBM and by the VALU (v_exp_f32 is a quarter-rate instruction), so the
+// arithmetic is kept lean: column maxima on the packed fp16 inputs (exact), one fused
+// multiply-add and one exp2 per element, and a 16-byte piece whose 8 inputs are all -inf for
+// every lane of the wave (whole rows masked out, as in causal attention) is skipped -- its
+// exponentials are exactly 0.
 template <int NT, int LPR, int R>
 __global__ __launch_bounds__(NT) void k_softmax_tile(int32_t n, int32_t m, int32_t tiles_per_batch,
                                                      const half_t* inp, half_t* out) {
@@ -25,13 +31,12 @@ __global__ __launch_bounds__(NT) void k_softmax_tile(int32_t n, int32_t m, int32
     half8_t v[R];
     coltile_load<NT, LPR, R>(v, inp + boff, n, m, col0, (half_t)(-__builtin_inff()));
 
+    half8_t hm = v[0];
+#pragma unroll
+    for (int p = 1; p < R; ++p) hm = __builtin_elementwise_max(hm, v[p]);
     float mx[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) mx[e] = -__builtin_inff();
-#pragma unroll
-    for (int p = 0; p < R; ++p)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) mx[e] = fmaxf(mx[e], (float)v[p][e]);
+    for (int e = 0; e < 8; ++e) mx[e] = (float)hm[e];
     coltile_reduce<NT, LPR, 1, true>(mx, lds);
 
     float ex[R][8], s[8];
@@ -41,12 +46,20 @@ __global__ __launch_bounds__(NT) void k_softmax_tile(int32_t n, int32_t m, int32
         s[e] = 0.0f;
     }
 #pragma unroll
-    for (int p = 0; p < R; ++p)
+    for (int p = 0; p < R; ++p) {
+        const uint4_t raw = __builtin_bit_cast(uint4_t, v[p]);
+        const bool all_ninf = (raw.x == 0xfc00fc00u) & (raw.y == 0xfc00fc00u) & (raw.z == 0xfc00fc00u) & (raw.w == 0xfc00fc00u);
+        if (__builtin_amdgcn_ballot_w64(!all_ninf) == 0) {      // wave-uniform: nothing but -inf here
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            ex[p][e] = exp_shift((float)v[p][e], mx[e]);   // rows >= n hold -inf -> 0
-            s[e] += ex[p][e];
+            for (int e = 0; e < 8; ++e) ex[p][e] = 0.0f;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                ex[p][e] = exp_shift((float)v[p][e], mx[e]);   // rows >= n hold -inf -> 0
+                s[e] += ex[p][e];
+            }
         }
+    }
     coltile_reduce<NT, LPR, 1, false>(s, lds);
 #pragma unroll
     for (int e = 0; e < 8; ++e) s[e] = 1.0f / (s[e] + 1e-10f);
@@ -127,7 +140,7 @@ static int softmax_dispatch(int32_t batch, int32_t n, int32_t m, const void* inp
         hipLaunchKernelGGL(k_softmax_rows, dim3((unsigned)batch), dim3(256), 0, st, n, x, y);
         return launch_status();
     }
-    if (m % 8 == 0 && aligned16(inp) && aligned16(out)) {
+    if (m % 8 == 0 && aligned16(inp) && aligned16(out) && (int64_t)n * m < (1ll << 31)) {
         bool ok = false;
         if (n <= 64 * 8 && m >= 64) ok = launch_tile_r<512, 8>((int)ceil_div(n, 64), batch, n, m, x, y, st);
         else if (n <= 128 * 8 && m >= 64) ok = launch_tile_r<1024, 8>((int)ceil_div(n, 128), batch, n, m, x, y, st);

@@ -8,11 +8,20 @@
 
 Search order: ``$CPMK_LIBRARY`` (explicit file), the in-tree build
 ``cpm_kernels_amd/lib/libcpmk_hip.so``, then the system linker path.
+
+One process must use one HIP runtime: a ``hipStream_t`` or device pointer made by one copy of
+``libamdhip64`` means nothing to another, and a second copy that initialises after the first
+finds no usable device.  PyTorch-ROCm wheels ship their own ``libamdhip64.so`` and load it by
+path, so if this library were loaded first it would pull in the system copy and the two would
+coexist.  ``preload_torch_hip_runtime()`` therefore maps PyTorch's copy first (when PyTorch is
+installed and ships one); the ``NEEDED libamdhip64.so.N`` of ``libcpmk_hip.so`` then binds to it
+by soname, and a later ``import torch`` finds the very same file already loaded.
 """
 import ctypes
 import ctypes.util
 import logging
 import os
+import sys
 from functools import wraps
 from typing import Callable, TypeVar
 
@@ -20,6 +29,34 @@ logger = logging.getLogger(__name__)
 LibCall = TypeVar("LibCall")
 
 _PKG_DIR = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+_preloaded = False
+
+
+def preload_torch_hip_runtime():
+    """Map the HIP runtime bundled with PyTorch (if any) before anything links the system one."""
+    global _preloaded
+    if _preloaded or "torch" in sys.modules:      # torch imported: its runtime is already mapped
+        _preloaded = True
+        return None
+    _preloaded = True
+    try:
+        import importlib.util
+        spec = importlib.util.find_spec("torch")
+    except (ImportError, ValueError):
+        return None
+    if spec is None or not spec.submodule_search_locations:
+        return None
+    cand = os.path.join(list(spec.submodule_search_locations)[0], "lib", "libamdhip64.so")
+    if not os.path.exists(cand):
+        return None
+    try:
+        ctypes.CDLL(cand, mode=ctypes.RTLD_GLOBAL)
+        return cand
+    except OSError as e:
+        logger.warning("Could not preload %s: %s", cand, e)
+        return None
 
 
 def find_lib(name: str):
@@ -39,6 +76,7 @@ class Lib:
         self._lib = None
         self._load_error = None
         if self._path is not None:
+            preload_torch_hip_runtime()
             try:
                 self._lib = ctypes.CDLL(self._path)
             except OSError as e:          # e.g. libamdhip64.so missing on this host

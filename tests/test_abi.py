@@ -158,3 +158,15 @@ def test_device_module_without_gpu():
     assert n >= 0
     with pytest.raises(ValueError):
         device.Device(n)          # one past the end is out of range (the reference accepts it by an off-by-one)
+
+
+def test_single_hip_runtime_whichever_is_imported_first():
+    """libcpmk_hip.so must bind to the HIP runtime PyTorch ships, also when this package is
+    imported before torch: two copies of libamdhip64 in one process do not share streams,
+    pointers or the device."""
+    code = ("import cpm_kernels_amd, torch\n"
+            "libs = sorted(set(l.split()[-1] for l in open('/proc/self/maps') if 'libamdhip64' in l))\n"
+            "print('HIPLIBS', len(libs), libs)\n")
+    out = subprocess.run([sys.executable, "-c", code], env=dict(os.environ, PYTHONPATH=ROOT), stdout=subprocess.PIPE,
+                         stderr=subprocess.STDOUT, text=True)
+    assert "HIPLIBS 1 " in out.stdout, out.stdout
