@@ -298,7 +298,10 @@ def test_layernorm_forward(gpu, shape, rd_mean):
         # outputs are O(1); atol 2e-4 covers values next to zero where x - mean cancels
         assert_close_fp16(to_np(out), ref, rtol=1e-3, atol=2e-4, what="layernorm_forward %s" % (shape,))
         ck.layernorm_inplace_forward(b, n, m, xd.data_ptr(), eps, rd_mean, stream())
-        assert_bits_equal(to_np(xd), to_np(out), "in place == out of place")
+        # tall columns take a different kernel in place (another summation order), so the two
+        # agree to the last fp16 bit only up to the rounding of the statistics
+        assert_close_fp16(to_np(xd), ref, rtol=1e-3, atol=2e-4, what="layernorm_inplace_forward %s" % (shape,))
+        assert_close_fp16(to_np(xd), to_np(out), rtol=1e-3, atol=2e-4, what="in place vs out of place")
     if m == 1:   # the reference pins step == forward(m=1) (tests/test_layernorm.py:115-152)
         xd = to_gpu(x); o2 = torch.empty_like(xd)
         ck.layernorm_step(b, n, xd.data_ptr(), o2.data_ptr(), 1e-3, rd_mean, stream())
