@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the int8 quantized-GEMM inference path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only gemm|gemv|ln|softmax]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only gemm|gemv|ln|softmax|pipeline|calib]
 
 One "step" is one pass of the path over the north-star workload: activations A fp16
 [1,4096,4096] ~N(0,1) and weights W fp16 [1,10240,4096] ~N(0,0.02) (seed 1000, generated on
@@ -28,6 +28,17 @@ PEAK_INT8_TOPS = 5000.0      # MI355X dense int8 MFMA, published
 PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, published
 M, K, N = 4096, 4096, 10240  # north-star GEMM
 
+# HBM bytes per launch of each kernel, measured offline with hardware counters (they cannot be
+# read from inside this process): `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` over
+# `python3 bench.py --no-cpu --only <workload>`, each counter scaled by what it reads for the
+# 256 MiB device copy of `--only calib` (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000 on MI355X).
+TRAFFIC_BYTES = {
+    "gemm_fused": 341.8e6,     # 252.3 MB fetched (operand tiles re-read across the 8 L2s) + 89.4 MB written
+    "gemv": 43.7e6,
+    "layernorm": 67.3e6,
+    "softmax": 2147.5e6,
+}
+
 
 def parse():
     p = argparse.ArgumentParser()
@@ -35,7 +46,8 @@ def parse():
     p.add_argument("--steps", type=int, default=50)
     p.add_argument("--warmup", type=int, default=10)
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    p.add_argument("--only", default="", help="run only one kernel loop (for profiling): gemm|gemv|ln|softmax|pipeline")
+    p.add_argument("--only", default="", help="run only one kernel loop (for profiling): gemm|gemv|ln|softmax|pipeline|calib "
+                        "(calib = a plain 256 MiB device copy, the known-size kernel that scales the HBM counters)")
     p.add_argument("--reps", type=int, default=200, help="launches per timed batch in the per-kernel loops")
     return p.parse_args()
 
@@ -113,6 +125,16 @@ def main():
     only = args.only
     result = {}
 
+    if only == "calib":
+        # a copy of known size: FETCH_SIZE / WRITE_SIZE read for it give the counters' scale
+        src = torch.randint(-128, 128, (256 << 20,), dtype=torch.int8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calib": "5 device copies of %d bytes (read + write each)" % src.numel()}), flush=True)
+        return
+
     # ---- north-star workload ---------------------------------------------------------------
     g = torch.Generator().manual_seed(1000)
     A_cpu = torch.randn(1, M, K, generator=g).half()
@@ -152,10 +174,12 @@ def main():
                                True, True, out16.data_ptr(), st())
         ms = event_ms(gemm, max(20, args.steps), warmup=max(3, args.warmup))
         tops = ops / (ms * 1e-3) / 1e12
-        roofline = {"kernel": "k_gemm_kmajor (int8 MFMA GEMM + fused fp16 dequant), M=%d K=%d N=%d" % (M, K, N),
+        roofline = {"kernel": "k_gemm_dma<2,4,4,2,128,true> (int8 MFMA GEMM + fused fp16 dequant), M=%d K=%d N=%d" % (M, K, N),
                     "bound": "mfma", "achieved": round(tops, 2), "peak": PEAK_INT8_TOPS, "unit": "TFLOP/s",
                     "ops": "int8 multiply-accumulates counted as 2 ops (TOP/s)",
-                    "frac": round(tops / PEAK_INT8_TOPS, 4), "avg_kernel_us": round(ms * 1e3, 2), "traffic": None}
+                    "frac": round(tops / PEAK_INT8_TOPS, 4), "avg_kernel_us": round(ms * 1e3, 2),
+                    "traffic": TRAFFIC_BYTES["gemm_fused"], "traffic_unit": "bytes per launch (HBM fetch + write counters)",
+                    "algorithmic_bytes": M * K + N * K + 2 * M * N}
         out32 = torch.empty((1, M, N), dtype=torch.int32, device=dev)
 
         def gemm32():
@@ -168,11 +192,11 @@ def main():
     components = {}
     reps = args.reps
 
-    def hbm(name, nbytes, ms, how, shape):
+    def hbm(name, nbytes, ms, how, shape, traffic):
         gbs = nbytes / (ms * 1e-3) / 1e9
-        components[name] = {"shape": shape, "algorithmic_bytes": int(nbytes), "avg_us": round(ms * 1e3, 3),
+        components[name] = {"shape": shape, "bound": "hbm", "algorithmic_bytes": int(nbytes), "avg_us": round(ms * 1e3, 3),
                             "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                            "frac": round(gbs / PEAK_HBM_GBS, 4), "timing": how}
+                            "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": traffic, "timing": how}
 
     if only in ("", "gemv"):
         # config 2: W int8 [10240,4096], 32 vectors; 8 weight copies (336 MB) rotate so every
@@ -190,7 +214,7 @@ def main():
                                                                qv.data_ptr(), o.data_ptr(), st())) for m_ in mats]
         ms, how = graph_ms(launches, max(5, reps // nrot))
         hbm("gemv_broadcast_mat_int8", 10240 * 4096 + 32 * 4096 + 2 * 32 * 10240 + 2 * 10240 + 2 * 32, ms, how,
-            "W int8 [10240,4096] x 32 vectors")
+            "W int8 [10240,4096] x 32 vectors", TRAFFIC_BYTES["gemv"])
         del mats
 
     if only in ("", "ln"):
@@ -201,7 +225,7 @@ def main():
         launches = [(lambda x_=x_: ck.layernorm_forward(8, 4096, 512, x_.data_ptr(), y.data_ptr(), 1e-5, True, st()))
                     for x_ in xs]
         ms, how = graph_ms(launches, max(5, reps // nrot))
-        hbm("layernorm_forward", 4 * 8 * 4096 * 512, ms, how, "[8,4096,512] fp16, dim 1")
+        hbm("layernorm_forward", 4 * 8 * 4096 * 512, ms, how, "[8,4096,512] fp16, dim 1", TRAFFIC_BYTES["layernorm"])
         del xs
 
     if only in ("", "softmax"):
@@ -214,7 +238,7 @@ def main():
         so = torch.empty_like(sd)
         launches = [lambda: ck.softmax_forward(512, 1024, 1024, sd.data_ptr(), so.data_ptr(), st())]
         ms, how = graph_ms(launches, max(3, reps // 20))
-        hbm("softmax_forward", 4 * 512 * 1024 * 1024, ms, how, "[512,1024,1024] fp16 causal, dim 1")
+        hbm("softmax_forward", 4 * 512 * 1024 * 1024, ms, how, "[512,1024,1024] fp16 causal, dim 1", TRAFFIC_BYTES["softmax"])
         del sd, so
 
     # ---- CPU baseline: torch formulation of the same step on the host cores ------------------
