@@ -87,6 +87,22 @@ __device__ inline int32_t quant_i8(float x, float s) {
     return (d != d) ? 0 : (int32_t)q;       // ... so map NaN to 0 explicitly
 }
 
+// The same result from the row's reciprocal y = 1/s (one IEEE divide per row instead of one per
+// element): a residual step restores the quotient closely enough that rint() lands on the same
+// integer, ties included; when the residual is not finite (infinite operands, zero scale) the
+// plain product already has the sign and size the divide would give.  Equality with quant_i8
+// holds for every (fp16 value, fp16 scale) pair; tests/native/recip_round_check.c proves it by
+// enumeration.
+__device__ inline int32_t quant_i8_rcp(float x, float s, float y) {
+    const float q0 = x * y;
+    const float r = __builtin_fmaf(-s, q0, x);
+    const float q1 = __builtin_fmaf(r, y, q0);
+    const float d = (r - r == 0.0f) ? q1 : q0;
+    float q = __builtin_rintf(d);
+    q = fminf(fmaxf(q, -128.0f), 127.0f);
+    return (d != d) ? 0 : (int32_t)q;
+}
+
 __device__ inline uint32_t pack4_i8(int32_t a, int32_t b, int32_t c, int32_t d) {
     return (uint32_t)(a & 0xff) | ((uint32_t)(b & 0xff) << 8) | ((uint32_t)(c & 0xff) << 16) |
            ((uint32_t)d << 24);

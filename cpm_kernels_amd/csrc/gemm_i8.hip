@@ -200,21 +200,55 @@ __device__ __forceinline__ void wait_vmcnt() {
 struct DmaArgs {
     GemmArgs g;
     int32_t batch;
-    int32_t ntiles;    // tiles per batch entry
+    int32_t ntiles;    // full-size tiles per batch entry (tiles_r x tiles_c)
+    uint32_t nfull;    // work items [0, nfull) are whole tiles in walk order ...
+    uint32_t nhalf;    // ... items [nfull, nfull + nhalf) are column halves of the tiles that follow
 };
 
-// Workgroup = WR x WC waves, wave tile = TR x TC MFMA tiles of 32x32, K slab = BKB bytes.
+// One work item of the persistent kernel: a whole BR x BC tile, or its left/right half.
+struct GemmItem {
+    uint32_t b;        // batch entry
+    int32_t j0, i0;    // first output row / column
+    bool half;
+    bool valid;
+};
+
+// Tiles are walked in groups of GRP row tiles, column-major inside a group, so neighbours in the
+// walk share operand slabs in L2.
+template <int BR, int BC>
+__device__ __forceinline__ GemmItem gemm_item(uint32_t L, const DmaArgs& da) {
+    GemmItem it;
+    it.valid = L < da.nfull + da.nhalf;
+    it.half = L >= da.nfull;
+    const uint32_t h = it.half ? L - da.nfull : 0;
+    const uint32_t id = it.half ? da.nfull + (h >> 1) : L;
+    it.b = id / (uint32_t)da.ntiles;
+    const uint32_t t = id - it.b * (uint32_t)da.ntiles;
+    constexpr uint32_t GRP = 4;
+    const uint32_t group_sz = GRP * (uint32_t)da.g.tiles_c;
+    const uint32_t g = t / group_sz;
+    const uint32_t rows_in_group = min(GRP, (uint32_t)da.g.tiles_r - g * GRP);
+    const uint32_t tin = t - g * group_sz;
+    it.j0 = (int32_t)((g * GRP + tin % rows_in_group) * BR);
+    it.i0 = (int32_t)((tin / rows_in_group) * BC + (h & 1) * (BC / 2));
+    return it;
+}
+
+// One output tile of BR x BC = (WR*TR*32) x (WC*TC*32), K slab = BKB bytes.
 // Pipeline per K slab `it` (stage cur = it & 1):
 //   k-steps 0 .. KS-2 : MFMAs of step s while the fragments of step s+1 are read from LDS
 //   s_waitcnt vmcnt(0); barrier     -> slab it+1 has landed in stage nxt for every wave and
 //                                      nobody reads stage cur any more
 //   k-step KS-1       : MFMAs while the step-0 fragments of slab it+1 are read and the DMA of
 //                       slab it+2 is issued into stage cur
-// Past the end of K the slab index is clamped (a redundant load nobody reads), which keeps the
-// loop body free of branches; the compiler then keeps all accumulators in AGPRs.
+// Past the end of K the DMA fetches slabs 0 and 1 of the NEXT tile of this workgroup (when it
+// has the same shape), so that tile starts with its operands already in LDS and the loads
+// overlap this tile's stores; otherwise the slab index is clamped (a redundant load nobody
+// reads).  Either way the loop body has no branches, which lets the compiler keep the
+// accumulators in place.  Returns true if the next tile's first two slabs are on their way.
 template <int WR, int WC, int TR, int TC, int BKB, bool FUSED>
-__global__ __launch_bounds__(WR* WC * 64) void k_gemm_dma(DmaArgs da) {
-    const GemmArgs& a = da.g;
+__device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, uint32_t lds_base, const GemmItem cur_item,
+                                              const GemmItem nxt_item, const bool have_slabs) {
     constexpr int KS = BKB / 32, CPR = BKB / 16;
     constexpr int NW = WR * WC, BR = WR * TR * 32, BC = WC * TC * 32;
     constexpr int STAGE = (BR + BC) * BKB;
@@ -224,8 +258,6 @@ __global__ __launch_bounds__(WR* WC * 64) void k_gemm_dma(DmaArgs da) {
     constexpr int CNT = NDMA / NW;
     constexpr int NM = TR * TC;
     constexpr int RPW = 256 / BKB;                 // rows per 256-byte bank wrap
-    extern __shared__ __attribute__((aligned(16))) int8_t smem[];
-    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) int8_t*)smem;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wr = wave / WC, wc = wave % WC;
@@ -245,138 +277,169 @@ __global__ __launch_bounds__(WR* WC * 64) void k_gemm_dma(DmaArgs da) {
         const int r = wc * TC * 32 + j * 32 + lrow;
         offQ[j] = BR * BKB + r * BKB + ((lk ^ swz(r)) << 4);
     }
-    const uint32_t total = (uint32_t)da.ntiles * da.batch;
+    const uint32_t b = cur_item.b;
+    const int32_t j0 = cur_item.j0, i0 = cur_item.i0;
+    const int8_t* Pb = a.P + (int64_t)b * a.strideP;
+    const int8_t* Qb = a.Q + (int64_t)b * a.strideQ;
+    // the next tile is fetched ahead only if its LDS layout is this one's and the ring parity works out
+    const bool ahead = nxt_item.valid && nxt_item.half == cur_item.half && nk >= 2 && (nk & 1) == 0;
+    const int8_t* Pn = a.P + (int64_t)nxt_item.b * a.strideP;
+    const int8_t* Qn = a.Q + (int64_t)nxt_item.b * a.strideQ;
 
-    for (uint32_t round = 0;; ++round) {
-        // workgroup w of G takes item round*G + (w%8)*(G/8) + w/8: the workgroups of one XCD
-        // (w % 8) work on adjacent tiles and share operand slabs in that XCD's L2
-        const uint32_t G = gridDim.x;
-        const uint32_t L = round * G + ((G % 8 == 0) ? (blockIdx.x % 8) * (G / 8) + blockIdx.x / 8 : blockIdx.x);
-        if (L >= total) break;
-        const uint32_t b = L / da.ntiles, t = L - b * da.ntiles;
-        constexpr uint32_t GRP = 4;                // row tiles per raster group
-        const uint32_t group_sz = GRP * a.tiles_c;
-        const uint32_t g = t / group_sz;
-        const uint32_t rows_in_group = min(GRP, (uint32_t)a.tiles_r - g * GRP);
-        const uint32_t tin = t - g * group_sz;
-        const uint32_t tile_r = g * GRP + tin % rows_in_group, tile_c = tin / rows_in_group;
-        const int32_t j0 = tile_r * BR, i0 = tile_c * BC;
-        const int8_t* Pb = a.P + (int64_t)b * a.strideP;
-        const int8_t* Qb = a.Q + (int64_t)b * a.strideQ;
+    // this wave's DMA instructions: d -> stage rows [RPI*dd, RPI*dd + RPI), dd = wave + d*NW;
+    // rows past the matrix are clamped (they only feed outputs that are never stored)
+    uint32_t voff[CNT], voffn[CNT], ldst[CNT];
+    bool isq[CNT];
+#pragma unroll
+    for (int d = 0; d < CNT; ++d) {
+        const int dd = wave + d * NW;
+        const int r = dd * RPI + lane / CPR;
+        const int c = (lane % CPR) ^ swz(r);
+        const bool q = dd * RPI >= BR;
+        isq[d] = q;
+        const int32_t grow = q ? min(i0 + (r - BR), a.m - 1) : min(j0 + r, a.n - 1);
+        const int32_t grown = q ? min(nxt_item.i0 + (r - BR), a.m - 1) : min(nxt_item.j0 + r, a.n - 1);
+        voff[d] = (uint32_t)grow * (uint32_t)K + c * 16;
+        voffn[d] = (uint32_t)grown * (uint32_t)K + c * 16;
+        ldst[d] = lds_base + dd * 1024;
+    }
+    // slab kt of this tile, or slab kt - nk of the next one (nx)
+    auto dma1 = [&](auto dc, int kt, bool nx, int stage) __attribute__((always_inline)) {
+        constexpr int d = decltype(dc)::value;
+        // read every candidate first and select values, never addresses of the captured variables
+        const int8_t *pb = Pb, *qb = Qb, *pn = Pn, *qn = Qn;
+        const uint32_t v0 = voff[d], v1 = voffn[d];
+        const bool q = isq[d];
+        const int8_t* b0 = q ? qb : pb;
+        const int8_t* b1 = q ? qn : pn;
+        lds_dma16(nx ? v1 : v0, (nx ? b1 : b0) + (int64_t)kt * BKB, ldst[d] + stage * STAGE);
+    };
 
-        // this wave's DMA instructions: d -> stage rows [RPI*dd, RPI*dd + RPI), dd = wave + d*NW;
-        // rows past the matrix are clamped (they only feed outputs that are never stored)
-        uint32_t voff[CNT], ldst[CNT];
-        bool isq[CNT];
+    int16_tv acc[TR][TC];
 #pragma unroll
-        for (int d = 0; d < CNT; ++d) {
-            const int dd = wave + d * NW;
-            const int r = dd * RPI + lane / CPR;
-            const int c = (lane % CPR) ^ swz(r);
-            const bool q = dd * RPI >= BR;
-            isq[d] = q;
-            const int32_t grow = q ? min(i0 + (r - BR), a.m - 1) : min(j0 + r, a.n - 1);
-            voff[d] = (uint32_t)grow * (uint32_t)K + c * 16;
-            ldst[d] = lds_base + dd * 1024;
-        }
-        auto dma1 = [&](auto dc, int kt, int stage) __attribute__((always_inline)) {
-            constexpr int d = decltype(dc)::value;
-            lds_dma16(voff[d], (isq[d] ? Qb : Pb) + (int64_t)kt * BKB, ldst[d] + stage * STAGE);
-        };
+    for (int i = 0; i < TR; ++i)
+#pragma unroll
+        for (int j = 0; j < TC; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+    int4_t fp[2][TR], fq[2][TC];
+    auto lfrag1 = [&](auto xc, auto bufc, int stage, int ks) __attribute__((always_inline)) {
+        constexpr int x = decltype(xc)::value, buf = decltype(bufc)::value;
+        if constexpr (x < TR)
+            fp[buf][x] = *reinterpret_cast<const int4_t*>(smem + stage * STAGE + (offP[x] ^ (ks << 5)));
+        else
+            fq[buf][x - TR] = *reinterpret_cast<const int4_t*>(smem + stage * STAGE + (offQ[x - TR] ^ (ks << 5)));
+    };
+    // one k-step: NM MFMAs with NMEM memory operations spread evenly between them, order pinned
+    auto kstep = [&](auto bufc, auto&& memop, auto nmem_c) __attribute__((always_inline)) {
+        constexpr int NMEM = decltype(nmem_c)::value, buf = decltype(bufc)::value;
+        static_for<0, NM>([&](auto xc) __attribute__((always_inline)) {
+            constexpr int x = decltype(xc)::value;
+            constexpr int i = x / TC, j = x % TC;
+            // MFMA "A" = column-operand rows, "B" = row-operand rows: lane l, register e of the
+            // result is output row l%32, column (e/4)*8 + (l/32)*4 + e%4 of the 32x32 tile
+            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fq[buf][j], fp[buf][i], acc[i][j], 0, 0, 0);
+            constexpr int lo = (x * NMEM) / NM, hi = ((x + 1) * NMEM) / NM;
+            static_for<lo, hi>([&](auto yc) __attribute__((always_inline)) { memop(yc); });
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+    using C0 = std::integral_constant<int, 0>;
 
-        int16_tv acc[TR][TC];
-#pragma unroll
-        for (int i = 0; i < TR; ++i)
-#pragma unroll
-            for (int j = 0; j < TC; ++j)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
-        int4_t fp[2][TR], fq[2][TC];
-        auto lfrag1 = [&](auto xc, auto bufc, int stage, int ks) __attribute__((always_inline)) {
-            constexpr int x = decltype(xc)::value, buf = decltype(bufc)::value;
-            if constexpr (x < TR)
-                fp[buf][x] = *reinterpret_cast<const int4_t*>(smem + stage * STAGE + (offP[x] ^ (ks << 5)));
-            else
-                fq[buf][x - TR] = *reinterpret_cast<const int4_t*>(smem + stage * STAGE + (offQ[x - TR] ^ (ks << 5)));
-        };
-        // one k-step: NM MFMAs with NMEM memory operations spread evenly between them, order pinned
-        auto kstep = [&](auto bufc, auto&& memop, auto nmem_c) __attribute__((always_inline)) {
-            constexpr int NMEM = decltype(nmem_c)::value, buf = decltype(bufc)::value;
-            static_for<0, NM>([&](auto xc) __attribute__((always_inline)) {
-                constexpr int x = decltype(xc)::value;
-                constexpr int i = x / TC, j = x % TC;
-                // MFMA "A" = column-operand rows, "B" = row-operand rows: lane l, register e of the
-                // result is output row l%32, column (e/4)*8 + (l/32)*4 + e%4 of the 32x32 tile
-                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fq[buf][j], fp[buf][i], acc[i][j], 0, 0, 0);
-                constexpr int lo = (x * NMEM) / NM, hi = ((x + 1) * NMEM) / NM;
-                static_for<lo, hi>([&](auto yc) __attribute__((always_inline)) { memop(yc); });
-                __builtin_amdgcn_sched_barrier(0);
-            });
-        };
-        using C0 = std::integral_constant<int, 0>;
-
+    if (!have_slabs) {
         __syncthreads();                 // every wave is done with the ring of the previous tile
-        static_for<0, CNT>([&](auto dc) __attribute__((always_inline)) { dma1(dc, 0, 0); });
+        static_for<0, CNT>([&](auto dc) __attribute__((always_inline)) { dma1(dc, 0, false, 0); });
         wait_vmcnt<0>();
         __syncthreads();
-        static_for<0, CNT>([&](auto dc) __attribute__((always_inline)) { dma1(dc, min(1, nk - 1), 1); });
-        static_for<0, TR + TC>([&](auto xc) __attribute__((always_inline)) { lfrag1(xc, C0{}, 0, 0); });
+        static_for<0, CNT>([&](auto dc) __attribute__((always_inline)) { dma1(dc, min(1, nk - 1), false, 1); });
+    } else {
+        wait_vmcnt<0>();                 // slabs 0 and 1 were requested during the previous tile
+        __syncthreads();
+    }
+    static_for<0, TR + TC>([&](auto xc) __attribute__((always_inline)) { lfrag1(xc, C0{}, 0, 0); });
 
-        for (int it = 0; it < nk; ++it) {
-            const int cur = it & 1, nxt = cur ^ 1;
-            static_for<0, KS - 1>([&](auto ksc) __attribute__((always_inline)) {
-                constexpr int ks = decltype(ksc)::value;
-                kstep(std::integral_constant<int, (ks & 1)>{},
-                      [&](auto xc) __attribute__((always_inline)) {
-                          lfrag1(xc, std::integral_constant<int, ((ks + 1) & 1)>{}, cur, ks + 1);
-                      },
-                      std::integral_constant<int, TR + TC>{});
-            });
-            __builtin_amdgcn_sched_barrier(0);
-            wait_vmcnt<0>();
-            __syncthreads();
-            __builtin_amdgcn_sched_barrier(0);
-            const int kt2 = min(it + 2, nk - 1);
-            kstep(std::integral_constant<int, ((KS - 1) & 1)>{},
+    for (int it = 0; it < nk; ++it) {
+        const int cur = it & 1, nxt = cur ^ 1;
+        static_for<0, KS - 1>([&](auto ksc) __attribute__((always_inline)) {
+            constexpr int ks = decltype(ksc)::value;
+            kstep(std::integral_constant<int, (ks & 1)>{},
                   [&](auto xc) __attribute__((always_inline)) {
-                      constexpr int x = decltype(xc)::value;
-                      if constexpr (x < TR + TC) lfrag1(xc, std::integral_constant<int, (KS & 1)>{}, nxt, 0);
-                      else dma1(std::integral_constant<int, x - (TR + TC)>{}, kt2, cur);
+                      lfrag1(xc, std::integral_constant<int, ((ks + 1) & 1)>{}, cur, ks + 1);
                   },
-                  std::integral_constant<int, TR + TC + CNT>{});
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        wait_vmcnt<0>();                 // drain the clamped loads before the ring is reused
+                  std::integral_constant<int, TR + TC>{});
+        });
+        __builtin_amdgcn_sched_barrier(0);
+        wait_vmcnt<0>();
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        const bool nx = ahead && it + 2 >= nk;
+        const int kt2 = nx ? it + 2 - nk : min(it + 2, nk - 1);
+        kstep(std::integral_constant<int, ((KS - 1) & 1)>{},
+              [&](auto xc) __attribute__((always_inline)) {
+                  constexpr int x = decltype(xc)::value;
+                  if constexpr (x < TR + TC) lfrag1(xc, std::integral_constant<int, (KS & 1)>{}, nxt, 0);
+                  else dma1(std::integral_constant<int, x - (TR + TC)>{}, kt2, nx, cur);
+              },
+              std::integral_constant<int, TR + TC + CNT>{});
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    if (!ahead) wait_vmcnt<0>();         // drain the clamped loads before the ring is reused
 
-        const int64_t obase = (int64_t)b * a.n * a.m;
+    const int64_t obase = (int64_t)b * a.n * a.m;
 #pragma unroll
-        for (int i = 0; i < TR; ++i) {
-            const int32_t row = j0 + wr * TR * 32 + i * 32 + lrow;
-            float sx = 0.0f;
-            if (FUSED && row < a.n) sx = (float)a.srow[a.bc_row ? row : (int64_t)b * a.n + row];
+    for (int i = 0; i < TR; ++i) {
+        const int32_t row = j0 + wr * TR * 32 + i * 32 + lrow;
+        float sx = 0.0f;
+        if (FUSED && row < a.n) sx = (float)a.srow[a.bc_row ? row : (int64_t)b * a.n + row];
 #pragma unroll
-            for (int j = 0; j < TC; ++j) {
+        for (int j = 0; j < TC; ++j) {
 #pragma unroll
-                for (int g4 = 0; g4 < 4; ++g4) {
-                    const int32_t col = i0 + wc * TC * 32 + j * 32 + g4 * 8 + lk * 4;
-                    if (row < a.n && col < a.m) {      // m % 4 == 0: the four columns are in or out together
-                        const int64_t o = obase + (int64_t)row * a.m + col;
-                        if (FUSED) {
-                            const half4_t sy =
-                                *reinterpret_cast<const half4_t*>(a.scol + (a.bc_col ? 0 : (int64_t)b * a.m) + col);
-                            half4_t h;
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const int32_t col = i0 + wc * TC * 32 + j * 32 + g4 * 8 + lk * 4;
+                if (row < a.n && col < a.m) {      // m % 4 == 0: the four columns are in or out together
+                    const int64_t o = obase + (int64_t)row * a.m + col;
+                    if (FUSED) {
+                        const half4_t sy =
+                            *reinterpret_cast<const half4_t*>(a.scol + (a.bc_col ? 0 : (int64_t)b * a.m) + col);
+                        half4_t h;
 #pragma unroll
-                            for (int e = 0; e < 4; ++e) h[e] = dequant(acc[i][j][g4 * 4 + e], sx, (float)sy[e]);
-                            *reinterpret_cast<half4_t*>(reinterpret_cast<half_t*>(a.out) + o) = h;
-                        } else {
-                            const int4_t v = {acc[i][j][g4 * 4], acc[i][j][g4 * 4 + 1], acc[i][j][g4 * 4 + 2],
-                                              acc[i][j][g4 * 4 + 3]};
-                            *reinterpret_cast<int4_t*>(reinterpret_cast<int32_t*>(a.out) + o) = v;
-                        }
+                        for (int e = 0; e < 4; ++e) h[e] = dequant(acc[i][j][g4 * 4 + e], sx, (float)sy[e]);
+                        *reinterpret_cast<half4_t*>(reinterpret_cast<half_t*>(a.out) + o) = h;
+                    } else {
+                        const int4_t v = {acc[i][j][g4 * 4], acc[i][j][g4 * 4 + 1], acc[i][j][g4 * 4 + 2],
+                                          acc[i][j][g4 * 4 + 3]};
+                        *reinterpret_cast<int4_t*>(reinterpret_cast<int32_t*>(a.out) + o) = v;
                     }
                 }
             }
         }
+    }
+    return ahead;
+}
+
+// Persistent kernel: WR x WC waves, wave tile = TR x TC MFMA tiles of 32x32.  Workgroup w of G
+// takes items round*G + (w%8)*(G/8) + w/8: the workgroups of one XCD (w % 8) work on adjacent
+// tiles and share operand slabs in that XCD's L2.  When the tile count leaves a last round
+// that at most half the workgroups could join, those tiles are issued as column halves
+// (HALVES), one per workgroup, so the round takes half as long.
+template <int WR, int WC, int TR, int TC, int BKB, bool FUSED, bool HALVES>
+__global__ __launch_bounds__(WR* WC * 64) void k_gemm_dma(DmaArgs da) {
+    constexpr int BR = WR * TR * 32, BC = WC * TC * 32;
+    extern __shared__ __attribute__((aligned(16))) int8_t smem[];
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) int8_t*)smem;
+    const uint32_t G = gridDim.x;
+    const uint32_t w = (G % 8 == 0) ? (blockIdx.x % 8) * (G / 8) + blockIdx.x / 8 : blockIdx.x;
+    bool have_slabs = false;
+    GemmItem cur = gemm_item<BR, BC>(w, da);
+    for (uint32_t L = w; cur.valid; L += G) {
+        const GemmItem nxt = gemm_item<BR, BC>(L + G, da);
+        if (HALVES && cur.half) {
+            if constexpr (HALVES)
+                have_slabs = gemm_dma_tile<WR, WC, TR, TC / 2, BKB, FUSED>(da.g, smem, lds_base, cur, nxt, have_slabs);
+        } else {
+            have_slabs = gemm_dma_tile<WR, WC, TR, TC, BKB, FUSED>(da.g, smem, lds_base, cur, nxt, have_slabs);
+        }
+        cur = nxt;
     }
 }
 
@@ -484,17 +547,16 @@ static int compute_units() {
     return cus[dev];
 }
 
-template <int WR, int WC, int TR, int TC, int BKB, bool FUSED>
-static int launch_dma(GemmArgs& a, int batch, hipStream_t st) {
+// waves (rows x cols), MFMA tiles per wave (rows x cols), K bytes per slab of the large-shape kernel
+#ifndef CPMK_GEMM_BIG
+#define CPMK_GEMM_BIG 2, 4, 4, 2, 128
+#endif
+
+template <int WR, int WC, int TR, int TC, int BKB, bool FUSED, bool HALVES>
+static int launch_dma_kernel(const DmaArgs& da, unsigned grid, hipStream_t st) {
     constexpr int BR = WR * TR * 32, BC = WC * TC * 32;
     constexpr int smem = 2 * (BR + BC) * BKB;
-    a.tiles_r = (int32_t)ceil_div(a.n, BR);
-    a.tiles_c = (int32_t)ceil_div(a.m, BC);
-    DmaArgs da;
-    da.g = a;
-    da.batch = batch;
-    da.ntiles = a.tiles_r * a.tiles_c;
-    auto kern = k_gemm_dma<WR, WC, TR, TC, BKB, FUSED>;
+    auto kern = k_gemm_dma<WR, WC, TR, TC, BKB, FUSED, HALVES>;
     static bool attr_set[64] = {false};       // dynamic LDS above 64 KB must be enabled per device
     int dev = 0;
     (void)hipGetDevice(&dev);
@@ -504,11 +566,32 @@ static int launch_dma(GemmArgs& a, int batch, hipStream_t st) {
         if (e != hipSuccess) return (int)e;
         attr_set[dev] = true;
     }
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(WR * WC * 64), smem, st, da);
+    return launch_status();
+}
+
+template <int WR, int WC, int TR, int TC, int BKB, bool FUSED>
+static int launch_dma(GemmArgs& a, int batch, hipStream_t st) {
+    constexpr int BR = WR * TR * 32, BC = WC * TC * 32;
+    a.tiles_r = (int32_t)ceil_div(a.n, BR);
+    a.tiles_c = (int32_t)ceil_div(a.m, BC);
+    DmaArgs da;
+    da.g = a;
+    da.batch = batch;
+    da.ntiles = a.tiles_r * a.tiles_c;
     const int64_t total = (int64_t)da.ntiles * batch;
     const int cus = compute_units();
-    dim3 grid((unsigned)(total < cus ? total : cus));
-    hipLaunchKernelGGL(kern, grid, dim3(WR * WC * 64), smem, st, da);
-    return launch_status();
+    const int64_t grid = total < cus ? total : cus;
+    // a last round of r <= grid/2 tiles is issued as 2r half tiles
+    const int64_t r = total % grid;
+    da.nfull = (uint32_t)total;
+    da.nhalf = 0;
+    if (TC % 2 == 0 && r > 0 && 2 * r <= grid) {
+        da.nfull = (uint32_t)(total - r);
+        da.nhalf = (uint32_t)(2 * r);
+        return launch_dma_kernel<WR, WC, TR, TC, BKB, FUSED, (TC % 2 == 0)>(da, (unsigned)grid, st);
+    }
+    return launch_dma_kernel<WR, WC, TR, TC, BKB, FUSED, false>(da, (unsigned)grid, st);
 }
 
 template <bool FUSED>
@@ -533,7 +616,7 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
     if (fast && (k % 128 == 0) && (int64_t)n * k < (1ll << 32) && (int64_t)m * k < (1ll << 32)) {
         // 256x256 tiles when they give most compute units a tile, else 128x128
         const int64_t big = ceil_div(n, 256) * ceil_div(m, 256) * batch;
-        if (big * 4 >= compute_units() * 3) return launch_dma<2, 4, 4, 2, 128, FUSED>(a, batch, st);
+        if (big * 4 >= compute_units() * 3) return launch_dma<CPMK_GEMM_BIG, FUSED>(a, batch, st);
         return launch_dma<2, 2, 2, 2, 128, FUSED>(a, batch, st);
     }
     if (fast) {

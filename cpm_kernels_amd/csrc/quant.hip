@@ -115,10 +115,19 @@ __global__ __launch_bounds__(256) void k_round(int64_t total, int32_t n, int32_t
             for (int e = 0; e < 8; ++e) { s[e] = (float)s0[e]; s[8 + e] = (float)s1[e]; }
         }
         int32_t q[16];
+        if (MODE == 0) {
+            const float y = 1.0f / s[0];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            q[e] = quant_i8((float)a[e], s[e]);
-            q[8 + e] = quant_i8((float)b[e], s[8 + e]);
+            for (int e = 0; e < 8; ++e) {
+                q[e] = quant_i8_rcp((float)a[e], s[0], y);
+                q[8 + e] = quant_i8_rcp((float)b[e], s[0], y);
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                q[e] = quant_i8((float)a[e], s[e]);
+                q[8 + e] = quant_i8((float)b[e], s[8 + e]);
+            }
         }
         uint4_t w;
         w.x = pack4_i8(q[0], q[1], q[2], q[3]);
@@ -207,7 +216,7 @@ __global__ __launch_bounds__(256) void k_row_quantize(int64_t rows, int32_t m,
     mx = wave_max(mx);
     const half_t sh = scale_from_absmax(mx);
     if (lane == 0) scale[row] = sh;
-    const float s = (float)sh;
+    const float s = (float)sh, y = 1.0f / s;
     uint2_t* o8 = reinterpret_cast<uint2_t*>(out + row * m);
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
@@ -215,7 +224,7 @@ __global__ __launch_bounds__(256) void k_row_quantize(int64_t rows, int32_t m,
         if (j < m8) {
             int32_t q[8];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) q[e] = quant_i8((float)v[i][e], s);
+            for (int e = 0; e < 8; ++e) q[e] = quant_i8_rcp((float)v[i][e], s, y);
             uint2_t w;
             w.x = pack4_i8(q[0], q[1], q[2], q[3]);
             w.y = pack4_i8(q[4], q[5], q[6], q[7]);

@@ -368,3 +368,18 @@ def test_oracle_reproduces_golden_fixtures():
     assert_close_fp16(oracle.layernorm_forward(g["x"], 1e-5, True), g["ln"], rtol=1e-3, atol=1e-4, what="golden ln")
     assert_close_fp16(oracle.softmax_forward(g["x"]), g["softmax"], rtol=1e-3, atol=1e-7, what="golden softmax")
     assert_close_fp16(oracle.gelu_forward(g["x"]), g["gelu"], rtol=1e-3, atol=1e-6, what="golden gelu")
+
+
+def test_reciprocal_rounding_equals_divide_rounding_exhaustively(tmp_path):
+    """The device rounds rows through y = 1/s and one residual step; tests/native/
+    recip_round_check.c enumerates all 2^32 (fp16 value, fp16 scale) pairs against the
+    divide-then-round of cuda/gemm.cu:16 with the same IEEE operations on the host."""
+    import os, shutil, subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    src = os.path.join(os.path.dirname(os.path.abspath(__file__)), "native", "recip_round_check.c")
+    exe = str(tmp_path / "recip_round_check")
+    subprocess.run(["gcc", "-O2", "-ffp-contract=off", "-mfma", "-msse4.1", "-fopenmp", src, "-o", exe, "-lm"], check=True)
+    r = subprocess.run([exe], capture_output=True, text=True)       # the whole grid: seconds on a few cores
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert r.stdout.startswith("4294967296 pairs, 0 mismatches"), r.stdout

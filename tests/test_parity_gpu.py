@@ -112,6 +112,37 @@ def test_round_unaligned_views(gpu):
     assert_bits_equal(to_np(qd), oracle.gemm_round(x, oracle.gemm_calc_scale(x)), "unaligned round")
 
 
+def test_round_every_value_scale_pair(gpu):
+    """gemm_round over ALL 65536 x 65536 (fp16 value, fp16 scale) pairs: the row kernels round
+    through the row's reciprocal, which must equal divide-then-round everywhere.  The whole grid
+    is checked on the device against gemm_round_transpose (per-element IEEE divide) on the
+    transposed problem, and sampled scale rows against the oracle on the host."""
+    _name("round all pairs")
+    allh = torch.arange(65536, dtype=torch.int32, device=gpu).to(torch.int16).view(torch.half)   # every bit pattern
+    x_row = allh.contiguous()
+    rng = np.random.default_rng(11)
+    CH = 4096                                           # scale patterns per chunk
+    for c0 in range(0, 65536, CH):
+        sc = allh[c0:c0 + CH].contiguous()              # (CH,)   row scales
+        mat = x_row[None, :].expand(CH, 65536).contiguous()          # (CH, 65536): row i = all values
+        out = torch.empty((CH, 65536), dtype=torch.int8, device=gpu)
+        ck.gemm_round(1, CH, 65536, mat.data_ptr(), sc.data_ptr(), out.data_ptr(), stream())
+        # same numbers with the roles of rows and columns swapped: element (j, i) = value j, scale i
+        mat_t = x_row[:, None].expand(65536, CH).contiguous()
+        out_t = torch.empty((65536, CH), dtype=torch.int8, device=gpu)
+        ck.gemm_round_transpose(1, 65536, CH, mat_t.data_ptr(), sc.data_ptr(), out_t.data_ptr(), stream())
+        assert torch.equal(out, out_t.t()), "reciprocal rounding differs from divide rounding, scales %d..%d" % (c0, c0 + CH)
+        # the fused quantiser's rounding stage is the same code; pin sampled rows to the oracle
+        rows = rng.integers(0, CH, 4)
+        got = out[rows].cpu().numpy()
+        xs = np.arange(65536, dtype=np.uint16).view(np.float16)
+        for k, r in enumerate(rows):
+            sr = np.array([[c0 + r]], dtype=np.uint16).view(np.float16)
+            ref = oracle.gemm_round(xs[None, None, :], sr)
+            assert_bits_equal(got[k], ref[0, 0], "oracle row, scale pattern %d" % (c0 + r))
+        del mat, mat_t, out, out_t
+
+
 @pytest.mark.parametrize("shape,bcx,bcy", [((1, 512, 4096), True, True), ((3, 20, 44), False, False),
                                           ((3, 20, 44), True, False), ((2, 7, 13), False, True),
                                           ((4, 128, 256), False, True)])
