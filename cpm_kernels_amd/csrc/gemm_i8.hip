@@ -197,6 +197,10 @@ __device__ __forceinline__ void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
+#ifndef CPMK_GEMM_MPM
+#define CPMK_GEMM_MPM 0     // >0: that many memory operations after each MFMA from the start of a k-step; 0: spread evenly
+#endif
+
 struct DmaArgs {
     GemmArgs g;
     int32_t batch;
@@ -315,6 +319,25 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, u
         lds_dma16(nx ? v1 : v0, (nx ? b1 : b0) + (int64_t)kt * BKB, ldst[d] + stage * STAGE);
     };
 
+    // the dequantisation scales of this lane's outputs, fetched now so that the epilogue does
+    // not wait on memory between its stores
+    half_t sxh[TR];
+    half4_t syh[TC][4];
+    if (FUSED) {
+#pragma unroll
+        for (int i = 0; i < TR; ++i) {
+            const int32_t row = min(j0 + wr * TR * 32 + i * 32 + lrow, a.n - 1);
+            sxh[i] = a.srow[a.bc_row ? row : (int64_t)b * a.n + row];
+        }
+#pragma unroll
+        for (int j = 0; j < TC; ++j)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const int32_t col = min(i0 + wc * TC * 32 + j * 32 + g4 * 8 + lk * 4, a.m - 4);   // m % 4 == 0
+                syh[j][g4] = *reinterpret_cast<const half4_t*>(a.scol + (a.bc_col ? 0 : (int64_t)b * a.m) + col);
+            }
+    }
+
     int16_tv acc[TR][TC];
 #pragma unroll
     for (int i = 0; i < TR; ++i)
@@ -339,7 +362,12 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, u
             // MFMA "A" = column-operand rows, "B" = row-operand rows: lane l, register e of the
             // result is output row l%32, column (e/4)*8 + (l/32)*4 + e%4 of the 32x32 tile
             acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fq[buf][j], fp[buf][i], acc[i][j], 0, 0, 0);
+#if CPMK_GEMM_MPM
+            constexpr int lo = x * CPMK_GEMM_MPM < NMEM ? x * CPMK_GEMM_MPM : NMEM;
+            constexpr int hi = (x == NM - 1 || (x + 1) * CPMK_GEMM_MPM > NMEM) ? NMEM : (x + 1) * CPMK_GEMM_MPM;
+#else
             constexpr int lo = (x * NMEM) / NM, hi = ((x + 1) * NMEM) / NM;
+#endif
             static_for<lo, hi>([&](auto yc) __attribute__((always_inline)) { memop(yc); });
             __builtin_amdgcn_sched_barrier(0);
         });
@@ -355,6 +383,14 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, u
     } else {
         wait_vmcnt<0>();                 // slabs 0 and 1 were requested during the previous tile
         __syncthreads();
+    }
+    if (FUSED) {     // pin the scale loads above the K loop (the waits just above cover them)
+#pragma unroll
+        for (int i = 0; i < TR; ++i) asm volatile("" : "+v"(sxh[i]));
+#pragma unroll
+        for (int j = 0; j < TC; ++j)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) asm volatile("" : "+v"(syh[j][g4]));
     }
     static_for<0, TR + TC>([&](auto xc) __attribute__((always_inline)) { lfrag1(xc, C0{}, 0, 0); });
 
@@ -390,7 +426,7 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, u
     for (int i = 0; i < TR; ++i) {
         const int32_t row = j0 + wr * TR * 32 + i * 32 + lrow;
         float sx = 0.0f;
-        if (FUSED && row < a.n) sx = (float)a.srow[a.bc_row ? row : (int64_t)b * a.n + row];
+        if (FUSED) sx = (float)sxh[i];
 #pragma unroll
         for (int j = 0; j < TC; ++j) {
 #pragma unroll
@@ -399,8 +435,7 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, u
                 if (row < a.n && col < a.m) {      // m % 4 == 0: the four columns are in or out together
                     const int64_t o = obase + (int64_t)row * a.m + col;
                     if (FUSED) {
-                        const half4_t sy =
-                            *reinterpret_cast<const half4_t*>(a.scol + (a.bc_col ? 0 : (int64_t)b * a.m) + col);
+                        const half4_t sy = syh[j][g4];
                         half4_t h;
 #pragma unroll
                         for (int e = 0; e < 4; ++e) h[e] = dequant(acc[i][j][g4 * 4 + e], sx, (float)sy[e]);
