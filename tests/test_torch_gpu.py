@@ -1,0 +1,191 @@
+"""GPU tests of the torch-level wrappers (cpm_kernels_amd.torch), modelled on the reference's own
+test-suite: each wrapper against the torch formulation the reference compares it with
+(tests/test_gemm.py, test_layernorm.py, test_softmax.py, test_gelu.py, test_position_embedding.py,
+test_mask.py, test_arith.py of the reference), evaluated in fp32 on the CPU, plus the stricter
+relations this build adds (fused == kernel-by-kernel, bit for bit).
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle import formulations as F
+import cpm_kernels_amd.torch as ct
+from util import assert_bits_equal, assert_close_fp16, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True)
+def _inference_only():
+    """The wrappers are forward-only; run every test without autograd bookkeeping."""
+    with torch.no_grad():
+        yield
+
+
+def _name(*a):
+    print("case", *a, flush=True)
+
+
+# shapes after the reference's TEST_CASES (tests/test_gemm.py:43-60): (batch, M, K, N), scaled down
+BMM_CASES = [(1, 4, 4, 4), (2, 4, 8, 4), (3, 12, 16, 8), (4, 36, 128, 4), (2, 512, 256, 300),
+             (1, 20, 4096, 260), (3, 260, 384, 132)]
+
+
+@pytest.mark.parametrize("case", BMM_CASES)
+@pytest.mark.parametrize("aT", [False, True])
+@pytest.mark.parametrize("bT", [False, True])
+def test_bmm_int8(gpu, case, aT, bT):
+    _name("bmm int8", case, aT, bT)
+    batch, M, K, N = case
+    g = torch.Generator().manual_seed(M * 31 + K * 7 + N + aT * 2 + bT)
+    for bA, bB in ((batch, batch), (1, batch), (batch, 1)):
+        A = torch.randn((bA, K, M) if aT else (bA, M, K), generator=g).half()
+        B = (torch.randn((bB, N, K) if bT else (bB, K, N), generator=g) * 0.05).half()
+        out = ct.bmm(A.cuda(), aT, B.cuda(), bT, int8=True)
+        out_unfused = ct.bmm(A.cuda(), aT, B.cuda(), bT, int8=True, fused=False)
+        assert out.shape == (batch, M, N) and out.dtype == torch.half
+        # the three-launch path equals the reference's six-launch sequence bit for bit
+        assert_bits_equal(to_np(out), to_np(out_unfused), "fused bmm == kernel-by-kernel bmm")
+        # against the CPU oracle of the same sequence (exact) ...
+        Ap = A.transpose(1, 2).contiguous() if aT else A          # (bA, M, K)
+        Bp = B.contiguous() if bT else B.transpose(1, 2).contiguous()   # (bB, N, K)
+        a_np, b_np = Ap.numpy(), Bp.numpy()
+        sa, sb = oracle.gemm_calc_scale(a_np), oracle.gemm_calc_scale(b_np)
+        qa, qb = oracle.gemm_round(a_np, sa), oracle.gemm_round(b_np, sb)
+        acc = np.einsum("bmk,bnk->bmn", np.broadcast_to(qa, (batch, M, K)).astype(np.float64),
+                        np.broadcast_to(qb, (batch, N, K)).astype(np.float64)).astype(np.int32)
+        ref = oracle.gemm_scale(acc, np.broadcast_to(sa, (batch, M)).copy(), np.broadcast_to(sb, (batch, N)).copy(),
+                                False, False)
+        assert_bits_equal(to_np(out), ref, "bmm int8 == oracle sequence")
+        # ... and, loosely, against the fp32 fake-quant formulation the reference's test uses
+        # (tests/test_gemm.py:87-98 accepts 0.5 absolute; quantising along K as the kernels do)
+        loose = F.quant_bmm_rowwise(Ap, Bp).numpy()
+        err = np.abs(to_np(out).astype(np.float32) - loose).max()
+        assert err < 0.5 and err <= 2e-2 * max(1.0, np.abs(loose).max()), err
+
+
+def test_bmm_fp16_goes_to_the_vendor_blas(gpu):
+    """int8=False is outside the hand-written path: the wrapper hands it to torch.matmul."""
+    g = torch.Generator().manual_seed(1)
+    A = torch.randn(2, 8, 16, generator=g).half().cuda()
+    B = torch.randn(2, 16, 12, generator=g).half().cuda()
+    assert torch.equal(ct.bmm(A, False, B, False, int8=False), torch.matmul(A, B))
+
+
+@pytest.mark.parametrize("shape", [(4, 512, 64), (3, 100, 40), (2, 4096, 128)])
+@pytest.mark.parametrize("bias", [True, False])
+def test_layernorm_module(gpu, shape, bias):
+    _name("LayerNorm", shape, bias)
+    b, n, m = shape
+    g = torch.Generator().manual_seed(n + m)
+    x = torch.randn(shape, generator=g).half()
+    for fused in (True, False):
+        ln = ct.LayerNorm(n, eps=1e-5, bias=bias, fused=fused).half().cuda()     # fp16 parameters, as the reference tests use it
+        with torch.no_grad():
+            ln.weight.copy_((1 + 0.1 * torch.randn(n, generator=g)).half())
+            if bias:
+                ln.bias.copy_((0.1 * torch.randn(n, generator=g)).half())
+        out = ln(x.cuda())
+        ref = F.layernorm_dim1(x, ln.weight.cpu(), ln.bias.cpu() if bias else None, 1e-5)
+        # reference bar: 5e-3 (tests/test_layernorm.py:100-113); here 1e-3 relative + the fp16
+        # rounding of the intermediate (one ulp of an O(1) value) that both implementations carry
+        assert_close_fp16(to_np(out), ref.numpy(), rtol=2e-3, atol=2e-3, what="LayerNorm fused=%s" % fused)
+        th = ct.LayerNormTH(n, eps=1e-5, bias=bias).half().cuda()
+        th.load_state_dict(ln.state_dict())
+        assert_close_fp16(to_np(out), to_np(th(x.cuda())), rtol=5e-3, atol=5e-3, what="LayerNorm vs LayerNormTH")
+    xi = x.cuda().clone()
+    ct.normalize_inplace(xi, 1e-5, True)
+    assert_close_fp16(to_np(xi), to_np(ct.normalizeTH(x.cuda(), 1e-5, True)), rtol=2e-3, atol=2e-3, what="normalize_inplace")
+
+
+@pytest.mark.parametrize("shape", [(8, 128, 256), (3, 77, 40), (2, 1024, 64)])
+def test_softmax_wrapper(gpu, shape):
+    _name("softmax", shape)
+    g = torch.Generator().manual_seed(shape[1])
+    x = (torch.randn(shape, generator=g) * 4).half()
+    x[:, shape[1] // 2:, 0] = float("-inf")
+    out = ct.softmax(x.cuda())
+    assert_close_fp16(to_np(out), F.softmax_dim1(x).numpy(), rtol=1e-3, atol=1e-6, what="softmax")
+    assert_close_fp16(to_np(out), to_np(ct.softmaxTH(x.cuda())), rtol=2e-3, atol=1e-6, what="softmax vs softmaxTH")
+    xi = x.cuda().clone()
+    ct.softmax_inplace(xi)
+    assert_bits_equal(to_np(xi), to_np(out), "softmax_inplace")
+
+
+def test_gelu_wrapper(gpu):
+    _name("gelu")
+    x = (torch.randn(4, 33, 20, generator=torch.Generator().manual_seed(5)) * 3).half()
+    out = ct.gelu(x.cuda())
+    assert_close_fp16(to_np(out), F.gelu_tanh(x).numpy(), rtol=1e-3, atol=1e-4, what="gelu")
+    xi = x.cuda().clone()
+    ct.gelu_inplace(xi)
+    assert_bits_equal(to_np(xi), to_np(out), "gelu_inplace")
+
+
+@pytest.mark.parametrize("cfg", [(32, 128, True), (32, 128, False), (64, 256, True), (32, 64, False)])
+def test_position_embedding_module(gpu, cfg):
+    _name("PositionEmbedding", cfg)
+    num_buckets, max_distance, bidi = cfg
+    heads = 12
+    pe = ct.PositionEmbedding(heads, num_buckets, max_distance, bidi).half().cuda()
+    with torch.no_grad():
+        pe.weight.copy_((torch.randn(heads, num_buckets, generator=torch.Generator().manual_seed(9)) * 0.02).half())
+    out = pe(128, 96)            # (key_len, query_len) as in the reference's forward
+    ref = F.position_bias(pe.weight.detach().cpu(), 96, 128, bidi, num_buckets, max_distance)
+    assert out.shape == (heads, 128, 96)
+    assert_bits_equal(to_np(out), ref.numpy(), "PositionEmbedding")
+    th = ct.PositionEmbeddingTH(heads, num_buckets, max_distance, bidi).half().cuda()
+    th.load_state_dict(pe.state_dict())
+    assert_bits_equal(to_np(th(128, 96)), ref.numpy(), "PositionEmbeddingTH")
+
+
+def test_mask_and_arith_wrappers(gpu):
+    _name("mask/arith")
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(3, 16, 40, generator=g).half()
+    y = torch.randn(3, 16, 40, generator=g).half()
+    mk = torch.rand(3, 40, generator=g) > 0.4
+    out = ct.mask(x.cuda(), mk.cuda(), float("-inf"))
+    assert_bits_equal(to_np(out), to_np(ct.maskTH(x.cuda(), mk.cuda(), float("-inf"))), "mask")
+    assert_bits_equal(to_np(ct.element_add(x.cuda(), y.cuda())), (x + y).numpy(), "element_add")
+    al = torch.randn(16, generator=g).half()
+    be = torch.randn(16, generator=g).half()
+    ref = (x.double() * al.double()[None, :, None] + be.double()[None, :, None]).half()     # fp16 FMA = one rounding
+    assert_bits_equal(to_np(ct.ln_mul_add(x.cuda(), al.cuda(), be.cuda())), ref.numpy(), "ln_mul_add")
+    assert_bits_equal(to_np(ct.ln_mul(x.cuda(), al.cuda())), (x.double() * al.double()[None, :, None]).half().numpy(), "ln_mul")
+
+
+def test_ffn_block_composition(gpu):
+    """CPM-2-style FFN block at reduced size: layernorm -> int8 GEMM -> gelu -> int8 GEMM -> residual,
+    through the wrappers in the reference's native (batch, hidden, seq) layout, against the fp32
+    formulations chained on the CPU.  The tolerance is the int8 quantisation noise of two GEMMs."""
+    _name("ffn block")
+    g = torch.Generator().manual_seed(1004)
+    b, d, dff, s = 2, 256, 640, 64
+    x = torch.randn(b, d, s, generator=g).half()
+    W1 = (torch.randn(1, dff, d, generator=g) * 0.02).half()
+    W2 = (torch.randn(1, d, dff, generator=g) * 0.02).half()
+    ln = ct.LayerNorm(d, eps=1e-5, bias=True).half().cuda()
+    with torch.no_grad():
+        ln.weight.copy_((1 + 0.1 * torch.randn(d, generator=g)).half())
+        ln.bias.copy_((0.1 * torch.randn(d, generator=g)).half())
+    xd = x.cuda()
+    h = ln(xd)
+    h = ct.bmm(W1.cuda(), False, h, False, int8=True)          # (b, dff, s)
+    h = ct.gelu(h)
+    h = ct.bmm(W2.cuda(), False, h, False, int8=True)          # (b, d, s)
+    out = ct.element_add(h, xd)
+    # CPU chain in fp32 with the same quantisation axes (weights along K = last dim, activations along K = dim 1)
+    r = F.layernorm_dim1(x, ln.weight.cpu(), ln.bias.cpu(), 1e-5).float()
+    def qmm(W, act):   # W (1, N, K), act (b, K, S)
+        Wq = F.fake_quant_rows(W.float())
+        aq = F.fake_quant_rows(act.transpose(1, 2)).transpose(1, 2)      # per (b, s) column, along K
+        return torch.matmul(Wq, aq)
+    r = qmm(W1, r).half().float()
+    r = F.gelu_tanh(r).half().float()
+    r = qmm(W2, r)
+    ref = (r + x.float())
+    got = to_np(out).astype(np.float32)
+    err = np.abs(got - ref.numpy())
+    assert err.max() < 3e-2 and err.mean() < 3e-3, (err.max(), err.mean())

@@ -13,7 +13,7 @@ def to_gpu(a: np.ndarray) -> torch.Tensor:
 
 def to_np(t: torch.Tensor) -> np.ndarray:
     torch.cuda.synchronize()
-    return t.cpu().numpy()
+    return t.detach().cpu().numpy()
 
 
 def bits(a: np.ndarray) -> np.ndarray:
