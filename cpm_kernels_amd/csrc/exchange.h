@@ -1,0 +1,83 @@
+// Exchange of per-column partial statistics between the workgroups of a team.
+//
+// A column reduction whose rows do not fit one workgroup's registers is split over the P
+// workgroups of a team (workgroups t*P .. t*P+P-1 of the launch, dispatched side by side).  Each
+// posts its partials as 8-byte packets {value, launch tag} with device-scope atomic stores and
+// collects its team mates' packets by polling until the tag matches; a packet is valid as a
+// whole or not at all, so no fence and no separate flag is needed, and the packets of an older
+// launch can never be mistaken for this one's.
+//
+// The team member that finishes collecting last wipes the team's packets, so a launch that is
+// replayed with the same arguments (a captured graph) starts from a clean slate as well.
+//
+// The packets live in a fixed pool in device memory owned by the library (nothing is allocated
+// per call).  Consecutive launches rotate over kXchRegions regions of the pool, so launches that
+// overlap in time on different streams do not share packets unless more than kXchRegions of
+// them are in flight at once.  A launch may use at most kXchSlots (team, part) pairs.
+//
+// Progress: a workgroup only ever waits for workgroups of its own team, whose indices differ by
+// less than P <= kXchMaxParts; workgroups start in index order, so all members of the oldest
+// unfinished team are resident and that team completes.  Should a packet nevertheless not arrive
+// within about a second the wait gives up and the caller writes NaN: a visible failure instead
+// of a hung GPU.
+#pragma once
+#include "common.h"
+
+namespace cpmk {
+
+constexpr int kXchRegions = 4;
+constexpr int kXchSlots = 8192;      // (team, part) pairs per launch
+constexpr int kXchVals = 128;        // packets per slot: 64 columns x 2 statistics
+constexpr int kXchMaxParts = 8;
+
+constexpr size_t kXchRegionWords = (size_t)kXchSlots * kXchVals + kXchSlots;   // packets, then one counter per team
+
+struct XchLaunch {
+    uint64_t* region;   // kXchRegionWords 8-byte words in device memory
+    uint32_t tag;       // never 0, differs from the tags of the launches that used this region before
+};
+
+// Host: region and tag for the next launch on the current device.  Returns 0 or a HIP error code.
+int xch_begin(XchLaunch* out);
+
+__device__ inline void xch_post(uint64_t* slot, int idx, float v, uint32_t tag) {
+    const uint64_t pkt = ((uint64_t)tag << 32) | (uint64_t)__builtin_bit_cast(uint32_t, v);
+    __hip_atomic_store(slot + idx, pkt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Poll one packet; false if it has not arrived by `deadline` (wall_clock64 ticks).
+__device__ inline bool xch_wait(const uint64_t* p, uint32_t tag, uint64_t deadline, float& v) {
+    for (;;) {
+        const uint64_t pkt = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if ((uint32_t)(pkt >> 32) == tag) {
+            v = __builtin_bit_cast(float, (uint32_t)pkt);
+            return true;
+        }
+        if (wall_clock64() > deadline) {
+            v = 0.0f;
+            return false;
+        }
+        __builtin_amdgcn_s_sleep(2);
+    }
+}
+
+// To be called by the first wave of a workgroup once the whole workgroup has collected its
+// packets (i.e. after the barrier that follows the xch_wait calls): counts the team members that
+// are done and lets the last one clear the team's `parts` slots and the counter.
+__device__ inline void xch_retire(uint64_t* region, uint32_t team, int parts) {
+    uint64_t* counter = region + (size_t)kXchSlots * kXchVals + team;
+    uint64_t* team_slots = region + (size_t)team * parts * kXchVals;
+    const int lane = threadIdx.x & 63;
+    uint64_t old = 0;
+    if (lane == 0) old = __hip_atomic_fetch_add(counter, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const uint32_t seen = __builtin_amdgcn_readfirstlane((uint32_t)old);
+    if ((int)seen == parts - 1) {
+        for (int i = lane; i < parts * kXchVals; i += 64)
+            __hip_atomic_store(team_slots + i, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (lane == 0) __hip_atomic_store(counter, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+constexpr uint64_t kXchTimeoutTicks = 100000000ull;   // wall_clock64 counts at 100 MHz: one second
+
+}  // namespace cpmk

@@ -4,6 +4,7 @@
 // optionally followed, on the fp16-rounded y, by the affine of cu_arith_ln_mul_add /
 // cu_arith_ln_mul (cuda/arith.cu:97-127): fp16 fma(y, alpha[i], beta[i]) or y * alpha[i].
 #include "dim1.h"
+#include "exchange.h"
 
 namespace cpmk {
 
@@ -71,57 +72,47 @@ __global__ __launch_bounds__(NT) void k_layernorm_tile(int32_t n, int32_t m, int
     coltile_store<NT, LPR, R>(v, out + boff, n, m, col0);
 }
 
-// Tall columns (n up to 16 * 1024 with 128-byte row segments).  A register tile can hold
-// 1024 rows of 64 columns; narrower tiles would hold more rows but touch only part of every
-// cache line, and the partial lines cost more L2 bandwidth than HBM has.  So the n rows of a
-// 64-column tile are split over PARTS = ceil(n / 1024) workgroups that run side by side on one
-// XCD: each keeps its own 1024 rows in registers and streams the other parts' rows once, only
-// to accumulate the column statistics (those reads are L2 hits: a sibling fetched or is
-// fetching the same lines).  No workgroup waits for another, so there is nothing to deadlock.
+// Tall columns.  A register tile holds T::ROWS rows of 64 columns (128-byte row segments, whole
+// cache lines); narrower tiles would hold more rows but touch only part of every line.  The n
+// rows of a 64-column tile are therefore split over a team of `parts` workgroups (exchange.h):
+// each keeps its own rows in registers, posts its partial column sums, adds up the team's
+// partials in part order (so the result does not depend on timing) and normalises its rows.
+// A workgroup reads and writes only its own rows: out may alias mat.
 template <int NT, int R>
-__global__ __launch_bounds__(NT) void k_layernorm_tall(int32_t n, int32_t m, int32_t tiles_per_batch, int32_t parts,
+__global__ __launch_bounds__(NT) void k_layernorm_team(int32_t n, int32_t m, int32_t tiles_per_batch, int32_t parts,
                                                        const half_t* mat, half_t* out,
                                                        const half_t* __restrict__ alpha,
-                                                       const half_t* __restrict__ beta, float eps, int rd_mean) {
+                                                       const half_t* __restrict__ beta, float eps, int rd_mean,
+                                                       uint64_t* xch, uint32_t tag) {
     constexpr int LPR = 8;
     using T = ColTile<NT, LPR, R>;
+    static_assert(T::COLS * 2 == kXchVals, "slot layout");
     __shared__ float lds[(T::NW + 1) * T::COLS * 2];
-    const uint32_t t = xcd_remap(blockIdx.x, gridDim.x);
-    const uint32_t part = t % parts, tile = t / parts;
-    const uint32_t b = tile / tiles_per_batch, ct = tile - b * tiles_per_batch;
-    const int32_t col0 = ct * T::COLS + (threadIdx.x % LPR) * 8;
-    const int64_t boff = (int64_t)b * n * m;
+    __shared__ float tot[kXchVals];
+    __shared__ int failed;
+    const int tid = threadIdx.x;
+    const uint32_t part = blockIdx.x % parts, team = blockIdx.x / parts;
+    const uint32_t b = team / tiles_per_batch, ct = team - b * tiles_per_batch;
+    const int32_t col0 = ct * T::COLS + (tid % LPR) * 8;
     const int32_t own0 = part * T::ROWS;                 // first row this workgroup normalises
     const int32_t own_n = min(T::ROWS, n - own0);        // > 0 by construction
+    const int64_t boff = (int64_t)b * n * m + (int64_t)own0 * m;
+    if (tid == 0) failed = 0;
 
     half8_t v[R];
-    coltile_load<NT, LPR, R>(v, mat + boff + (int64_t)own0 * m, own_n, m, col0, (half_t)0.0f);
+    coltile_load<NT, LPR, R>(v, mat + boff, own_n, m, col0, (half_t)0.0f);
+    // the affine coefficients of this lane's rows, requested now so that they arrive during the exchange
+    const int rg = tid / LPR;
+    half_t al[R], be[R];
+#pragma unroll
+    for (int p = 0; p < R; ++p) {
+        const int32_t row = min(own0 + p * T::RPP + rg, n - 1);
+        al[p] = alpha != nullptr ? alpha[row] : (half_t)1.0f;
+        be[p] = beta != nullptr ? beta[row] : (half_t)0.0f;
+    }
     float s[16];
 #pragma unroll
     for (int e = 0; e < 16; ++e) s[e] = 0.0f;
-    // the other parts' rows: statistics only
-    const int rg = threadIdx.x / LPR;
-    if (col0 < m) {
-        for (int32_t r0 = 0; r0 < n; r0 += T::RPP * 4) {
-            half8_t w[4];
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const int32_t row = r0 + u * T::RPP + rg;
-                const bool mine = row >= own0 && row < own0 + T::ROWS;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) w[u][e] = (half_t)0.0f;
-                if (row < n && !mine) w[u] = *reinterpret_cast<const half8_t*>(mat + boff + ((uint32_t)row * (uint32_t)m + (uint32_t)col0));
-            }
-#pragma unroll
-            for (int u = 0; u < 4; ++u)
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const float x = (float)w[u][e];
-                    s[e] += x;
-                    s[8 + e] += x * x;
-                }
-        }
-    }
 #pragma unroll
     for (int p = 0; p < R; ++p)
 #pragma unroll
@@ -130,7 +121,32 @@ __global__ __launch_bounds__(NT) void k_layernorm_tall(int32_t n, int32_t m, int
             s[e] += x;
             s[8 + e] += x * x;
         }
-    coltile_reduce<NT, LPR, 2, false>(s, lds);
+    coltile_reduce<NT, LPR, 2, false>(s, lds);      // every lane: this part's sums of its 8 columns
+
+    // packet g*64 + c of a slot: statistic g (0 sum, 1 sum of squares) of tile column c
+    uint64_t* team_slots = xch + (size_t)team * parts * kXchVals;
+    if (tid < LPR) {
+        uint64_t* slot = team_slots + (size_t)part * kXchVals;
+#pragma unroll
+        for (int k = 0; k < 16; ++k) xch_post(slot, (k >> 3) * T::COLS + tid * 8 + (k & 7), s[k], tag);
+    }
+    if (tid < kXchVals) {
+        const uint64_t deadline = wall_clock64() + kXchTimeoutTicks;
+        float acc = 0.0f;
+        bool ok = true;
+        for (int32_t q = 0; q < parts; ++q) {
+            float x;
+            ok &= xch_wait(team_slots + (size_t)q * kXchVals + tid, tag, deadline, x);
+            acc += x;
+        }
+        tot[tid] = acc;
+        if (!ok) failed = 1;
+    }
+    __syncthreads();
+    const int cg = tid % LPR;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) s[k] = tot[(k >> 3) * T::COLS + cg * 8 + (k & 7)];
+    const bool bad = failed != 0;
 
     float mean[8], rstd[8];
     const float fn = (float)n;
@@ -142,20 +158,18 @@ __global__ __launch_bounds__(NT) void k_layernorm_tall(int32_t n, int32_t m, int
             mean[e] = s[e] / fn;
             var -= mean[e] * mean[e];
         }
-        rstd[e] = rsqrtf(var + eps);
+        rstd[e] = bad ? __builtin_nanf("") : rsqrtf(var + eps);
     }
 #pragma unroll
     for (int p = 0; p < R; ++p) {
         half8_t y;
 #pragma unroll
         for (int e = 0; e < 8; ++e) y[e] = round_f16(((float)v[p][e] - mean[e]) * rstd[e]);
-        if (alpha != nullptr) {
-            const int32_t row = own0 + p * T::RPP + rg;
-            if (row < n) y = affine8(y, alpha[row], beta ? beta[row] : (half_t)0.0f, beta != nullptr);
-        }
+        if (alpha != nullptr) y = affine8(y, al[p], be[p], beta != nullptr);
         v[p] = y;
     }
-    coltile_store<NT, LPR, R>(v, out + boff + (int64_t)own0 * m, own_n, m, col0);
+    coltile_store<NT, LPR, R>(v, out + boff, own_n, m, col0);
+    if (tid < 64) xch_retire(xch, team, parts);     // after the barrier above: this workgroup holds all it needs
 }
 
 // Generic fallback (any n, m, alignment): 64 columns x 4 row groups per workgroup, two
@@ -258,13 +272,24 @@ static int layernorm_dispatch(int32_t batch, int32_t n, int32_t m, const void* m
     if (m % 8 == 0 && aligned16(mat) && aligned16(out) && (int64_t)n * m < (1ll << 31)) {
         // widest row segment whose tile still fits the register budget (at most 8 pieces per lane)
         bool ok = false;
-        if (n > 128 * 8 && n <= 16 * 1024 && m >= 64 && (const void*)x != (const void*)y) {
-            // tall columns: 64-column tiles, n split over side-by-side workgroups.  Not for in-place
-            // calls: a workgroup would overwrite rows that a sibling still reads for its statistics.
-            const int32_t parts = (int32_t)ceil_div(n, 1024), tiles = (int32_t)ceil_div(m, 64);
-            hipLaunchKernelGGL((k_layernorm_tall<1024, 8>), dim3((unsigned)((int64_t)tiles * batch * parts)), dim3(1024), 0,
-                               st, n, m, tiles, parts, x, y, al, be, eps, rd_mean);
-            return launch_status();
+        if (n > 128 * 8 && m >= 64) {
+            // tall columns: 64-column tiles, the rows split over a team of workgroups
+            const int64_t tiles = ceil_div(m, 64);
+            const bool big = n >= 2048;                       // 1024 rows a part, else 512
+            const int64_t parts = ceil_div(n, big ? 1024 : 512);
+            if (parts <= kXchMaxParts && tiles * batch * parts <= kXchSlots) {
+                XchLaunch xl;
+                const int rc = xch_begin(&xl);
+                if (rc != 0) return rc;
+                const dim3 grid((unsigned)(tiles * batch * parts));
+                if (big)
+                    hipLaunchKernelGGL((k_layernorm_team<1024, 8>), grid, dim3(1024), 0, st, n, m, (int32_t)tiles,
+                                       (int32_t)parts, x, y, al, be, eps, rd_mean, xl.region, xl.tag);
+                else
+                    hipLaunchKernelGGL((k_layernorm_team<512, 8>), grid, dim3(512), 0, st, n, m, (int32_t)tiles,
+                                       (int32_t)parts, x, y, al, be, eps, rd_mean, xl.region, xl.tag);
+                return launch_status();
+            }
         }
         if (n <= 128 * 8 && m >= 64) ok = launch_tile_r<8>((int)ceil_div(n, 128), batch, n, m, x, y, al, be, eps, rd_mean, st);
         else if (n <= 256 * 8 && m >= 32) ok = launch_tile_r<4>((int)ceil_div(n, 256), batch, n, m, x, y, al, be, eps, rd_mean, st);

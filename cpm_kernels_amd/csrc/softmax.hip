@@ -4,6 +4,7 @@
 // NaN.  The reference reads the input three times and evaluates expf twice per element; the
 // tile kernel below reads once, evaluates exp once and keeps the results in registers.
 #include "dim1.h"
+#include "exchange.h"
 
 namespace cpmk {
 
@@ -70,6 +71,110 @@ __global__ __launch_bounds__(NT) void k_softmax_tile(int32_t n, int32_t m, int32
     coltile_store<NT, LPR, R>(v, out + boff, n, m, col0);
 }
 
+// Columns too tall for one workgroup's registers at 128-byte row segments: the n rows of a
+// 64-column tile are split over a team of `parts` workgroups (exchange.h).  Each computes, for its own rows, the column maximum m_p (floored at
+// -1e6 like M itself) and the exponentials and their sum s_p relative to m_p, posts (m_p, s_p),
+// and rescales by exp(m_p - M) / S with M = max_p m_p and S = sum_p s_p exp(m_p - M) + 1e-10,
+// which is the single-workgroup result up to two extra fp32 roundings.
+template <int NT, int R>
+__global__ __launch_bounds__(NT) void k_softmax_team(int32_t n, int32_t m, int32_t tiles_per_batch, int32_t parts,
+                                                     const half_t* inp, half_t* out, uint64_t* xch, uint32_t tag) {
+    constexpr int LPR = 8;
+    using T = ColTile<NT, LPR, R>;
+    static_assert(T::COLS * 2 == kXchVals, "slot layout");
+    __shared__ float lds[(T::NW + 1) * T::COLS];
+    __shared__ float tot[kXchVals];
+    __shared__ int failed;
+    const int tid = threadIdx.x;
+    const uint32_t part = blockIdx.x % parts, team = blockIdx.x / parts;
+    const uint32_t b = team / tiles_per_batch, ct = team - b * tiles_per_batch;
+    const int32_t col0 = ct * T::COLS + (tid % LPR) * 8;
+    const int32_t own0 = part * T::ROWS;
+    const int32_t own_n = min(T::ROWS, n - own0);
+    const int64_t boff = (int64_t)b * n * m + (int64_t)own0 * m;
+    if (tid == 0) failed = 0;
+
+    half8_t v[R];
+    coltile_load<NT, LPR, R>(v, inp + boff, own_n, m, col0, (half_t)(-__builtin_inff()));
+
+    half8_t hm = v[0];
+#pragma unroll
+    for (int p = 1; p < R; ++p) hm = __builtin_elementwise_max(hm, v[p]);
+    float mx[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) mx[e] = (float)hm[e];
+    coltile_reduce<NT, LPR, 1, true>(mx, lds);
+
+    float ex[R][8], s[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        mx[e] = fmaxf(mx[e], -1e6f) * kLog2e;       // m_p, in units of log2(e)
+        s[e] = 0.0f;
+    }
+#pragma unroll
+    for (int p = 0; p < R; ++p) {
+        const uint4_t raw = __builtin_bit_cast(uint4_t, v[p]);
+        const bool all_ninf = (raw.x == 0xfc00fc00u) & (raw.y == 0xfc00fc00u) & (raw.z == 0xfc00fc00u) & (raw.w == 0xfc00fc00u);
+        if (__builtin_amdgcn_ballot_w64(!all_ninf) == 0) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) ex[p][e] = 0.0f;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                ex[p][e] = exp_shift((float)v[p][e], mx[e]);
+                s[e] += ex[p][e];
+            }
+        }
+    }
+    coltile_reduce<NT, LPR, 1, false>(s, lds);
+
+    // packet c: m_p of tile column c; packet 64 + c: s_p
+    uint64_t* team_slots = xch + (size_t)team * parts * kXchVals;
+    if (tid < LPR) {
+        uint64_t* slot = team_slots + (size_t)part * kXchVals;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            xch_post(slot, tid * 8 + e, mx[e], tag);
+            xch_post(slot, T::COLS + tid * 8 + e, s[e], tag);
+        }
+    }
+    if (tid < T::COLS) {
+        const uint64_t deadline = wall_clock64() + kXchTimeoutTicks;
+        float mp[kXchMaxParts], sp[kXchMaxParts];
+        bool ok = true;
+        float M = -__builtin_inff();
+#pragma unroll
+        for (int q = 0; q < kXchMaxParts; ++q) {
+            mp[q] = -__builtin_inff();
+            sp[q] = 0.0f;
+            if (q < parts) {
+                ok &= xch_wait(team_slots + (size_t)q * kXchVals + tid, tag, deadline, mp[q]);
+                ok &= xch_wait(team_slots + (size_t)q * kXchVals + T::COLS + tid, tag, deadline, sp[q]);
+                M = fmaxf(M, mp[q]);
+            }
+        }
+        float S = 0.0f;
+#pragma unroll
+        for (int q = 0; q < kXchMaxParts; ++q)
+            if (q < parts) S += sp[q] * __builtin_amdgcn_exp2f(mp[q] - M);
+        tot[tid] = M;
+        tot[T::COLS + tid] = ok ? 1.0f / (S + 1e-10f) : __builtin_nanf("");
+        if (!ok) failed = 1;
+    }
+    __syncthreads();
+    const int cg = tid % LPR;
+    float f[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+        f[e] = __builtin_amdgcn_exp2f(mx[e] - tot[cg * 8 + e]) * tot[T::COLS + cg * 8 + e];     // exp(m_p - M) / S
+#pragma unroll
+    for (int p = 0; p < R; ++p)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[p][e] = round_f16(ex[p][e] * f[e]);
+    coltile_store<NT, LPR, R>(v, out + boff, own_n, m, col0);
+    if (tid < 64) xch_retire(xch, team, parts);     // after the barrier above: this workgroup holds all it needs
+}
+
 // Generic fallback: 64 columns x 4 row groups, three passes (max, sum, write).  All reads of
 // a column by other threads finish before the barrier that precedes the first store, and
 // the last pass re-reads each element in the thread that overwrites it: out may alias inp.
@@ -131,6 +236,11 @@ static bool launch_tile_r(int r, int32_t batch, int32_t n, int32_t m, const half
     return true;
 }
 
+// columns taller than this go to the team kernel (single workgroups hold up to 2048 rows at 64-byte row segments)
+#ifndef CPMK_SOFTMAX_TEAM_MIN
+#define CPMK_SOFTMAX_TEAM_MIN 2048
+#endif
+
 static int softmax_dispatch(int32_t batch, int32_t n, int32_t m, const void* inp, void* out, hipStream_t st) {
     if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
     if ((int64_t)batch * n * m == 0) return 0;
@@ -142,6 +252,24 @@ static int softmax_dispatch(int32_t batch, int32_t n, int32_t m, const void* inp
     }
     if (m % 8 == 0 && aligned16(inp) && aligned16(out) && (int64_t)n * m < (1ll << 31)) {
         bool ok = false;
+        if (n > CPMK_SOFTMAX_TEAM_MIN && m >= 64) {
+            const int64_t tiles = ceil_div(m, 64);
+            const bool big = n >= 2048;                       // 1024 rows a part, else 512
+            const int64_t parts = ceil_div(n, big ? 1024 : 512);
+            if (parts <= kXchMaxParts && tiles * batch * parts <= kXchSlots) {
+                XchLaunch xl;
+                const int rc = xch_begin(&xl);
+                if (rc != 0) return rc;
+                const dim3 grid((unsigned)(tiles * batch * parts));
+                if (big)
+                    hipLaunchKernelGGL((k_softmax_team<1024, 8>), grid, dim3(1024), 0, st, n, m, (int32_t)tiles,
+                                       (int32_t)parts, x, y, xl.region, xl.tag);
+                else
+                    hipLaunchKernelGGL((k_softmax_team<512, 8>), grid, dim3(512), 0, st, n, m, (int32_t)tiles,
+                                       (int32_t)parts, x, y, xl.region, xl.tag);
+                return launch_status();
+            }
+        }
         if (n <= 64 * 8 && m >= 64) ok = launch_tile_r<512, 8>((int)ceil_div(n, 64), batch, n, m, x, y, st);
         else if (n <= 128 * 8 && m >= 64) ok = launch_tile_r<1024, 8>((int)ceil_div(n, 128), batch, n, m, x, y, st);
         else if (n <= 256 * 8 && m >= 32) ok = launch_tile_r<1024, 4>((int)ceil_div(n, 256), batch, n, m, x, y, st);

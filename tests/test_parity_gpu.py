@@ -311,7 +311,7 @@ def test_gemv_broadcast_mat_int8(gpu, batch, dim_out, dim_in):
 # layernorm / softmax / gelu (tolerance ops)
 # ---------------------------------------------------------------------------------------------
 LN_SHAPES = [(8, 4096, 512), (16, 768, 512), (4, 1024, 512), (3, 100, 40), (2, 33, 24), (2, 777, 123), (5, 4096, 1),
-             (1, 5000, 64), (2, 2048, 32), (1, 1536, 8), (2, 64, 72)]
+             (1, 5000, 64), (2, 2048, 32), (1, 1536, 8), (2, 64, 72), (2, 1100, 64), (1, 8192, 128), (1, 9000, 64)]
 
 
 @pytest.mark.parametrize("shape", LN_SHAPES)
@@ -337,6 +337,81 @@ def test_layernorm_forward(gpu, shape, rd_mean):
         xd = to_gpu(x); o2 = torch.empty_like(xd)
         ck.layernorm_step(b, n, xd.data_ptr(), o2.data_ptr(), 1e-3, rd_mean, stream())
         assert_bits_equal(to_np(o2), to_np(out), "layernorm_step == forward(m=1)")
+
+
+def test_team_kernels_repeated_and_concurrent(gpu):
+    """Tall columns are reduced by teams of workgroups that exchange partial results through a
+    packet pool inside the library.  Back-to-back launches reuse the pool's regions, launches on
+    two streams overlap in time, and in-place calls alias input and output: every result must
+    equal the first one bit for bit (the team sums in part order, so results do not depend on
+    timing) and match the oracle."""
+    _name("team kernels")
+    rng = np.random.default_rng(77)
+    x = (rng.standard_normal((2, 3000, 192)) * 2 + 0.3).astype(np.float16)
+    xs = (rng.standard_normal((2, 2500, 128)) * 4).astype(np.float16)
+    xs[:, 1500:, :40] = -np.inf
+    ln_ref = oracle.layernorm_forward(x, 1e-5, True)
+    sm_ref = oracle.softmax_forward(xs)
+    xd, xsd = to_gpu(x), to_gpu(xs)
+    first_ln = torch.empty_like(xd); first_sm = torch.empty_like(xsd)
+    ck.layernorm_forward(2, 3000, 192, xd.data_ptr(), first_ln.data_ptr(), 1e-5, True, stream())
+    ck.softmax_forward(2, 2500, 128, xsd.data_ptr(), first_sm.data_ptr(), stream())
+    assert_close_fp16(to_np(first_ln), ln_ref, rtol=1e-3, atol=2e-4, what="team layernorm")
+    assert_close_fp16(to_np(first_sm), sm_ref, rtol=1e-3, atol=1e-7, what="team softmax")
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    outs = []
+    torch.cuda.synchronize()
+    for it in range(24):
+        for s_ in (s1, s2):
+            with torch.cuda.stream(s_):
+                o1 = torch.empty_like(xd); o2 = xsd.clone()
+                ck.layernorm_forward(2, 3000, 192, xd.data_ptr(), o1.data_ptr(), 1e-5, True, s_.cuda_stream)
+                ck.softmax_inplace_forward(2, 2500, 128, o2.data_ptr(), s_.cuda_stream)
+                outs.append((o1, o2))
+    torch.cuda.synchronize()
+    a, b = to_np(first_ln), to_np(first_sm)
+    for k, (o1, o2) in enumerate(outs):
+        assert_bits_equal(to_np(o1), a, "layernorm launch %d" % k)
+        assert_bits_equal(to_np(o2), b, "softmax launch %d" % k)
+
+
+def test_team_kernels_in_a_replayed_graph(gpu):
+    """A captured launch is replayed with the same kernel arguments, packet pool region and tag
+    included; each replay gets new input data and must give that data's result, not a mix with
+    partial sums a previous replay left behind."""
+    _name("team kernels, graph replay")
+    rng = np.random.default_rng(78)
+    shape_ln, shape_sm = (2, 2600, 128), (1, 4096, 192)
+    xin = torch.empty(shape_ln, dtype=torch.half, device=gpu); xout = torch.empty_like(xin)
+    sin = torch.empty(shape_sm, dtype=torch.half, device=gpu); sout = torch.empty_like(sin)
+
+    def launches():
+        ck.layernorm_forward(*shape_ln, xin.data_ptr(), xout.data_ptr(), 1e-5, True, stream())
+        ck.softmax_forward(*shape_sm, sin.data_ptr(), sout.data_ptr(), stream())
+
+    xin.normal_(); sin.normal_()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        launches()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        launches()
+    for it in range(5):
+        x = (rng.standard_normal(shape_ln) * (1 + it) + it).astype(np.float16)
+        sx = (rng.standard_normal(shape_sm) * 4).astype(np.float16)
+        xin.copy_(to_gpu(x)); sin.copy_(to_gpu(sx))
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        got_ln, got_sm = to_np(xout).copy(), to_np(sout).copy()
+        launches()                                   # eager, same inputs
+        assert_bits_equal(got_ln, to_np(xout), "layernorm replay %d == eager" % it)
+        assert_bits_equal(got_sm, to_np(sout), "softmax replay %d == eager" % it)
+        assert_close_fp16(got_ln, oracle.layernorm_forward(x, 1e-5, True), rtol=1e-3, atol=2e-4, what="replay %d layernorm" % it)
+        assert_close_fp16(got_sm, oracle.softmax_forward(sx), rtol=1e-3, atol=1e-7, what="replay %d softmax" % it)
 
 
 @pytest.mark.parametrize("shape", [(8, 4096, 512), (3, 100, 40), (2, 777, 124), (2, 1024, 64)])
@@ -366,7 +441,8 @@ def test_layernorm_affine_fused(gpu, shape, bias):
 
 
 SOFTMAX_SHAPES = [(1, 2, 32), (4, 128, 128), (4, 128, 16), (4, 123, 16), (16, 1024, 320), (7, 1024, 321),
-                  (3, 512, 64), (2, 2000, 48), (2, 4096, 16), (1, 5000, 24), (6, 333, 1), (2, 64, 200)]
+                  (3, 512, 64), (2, 2000, 48), (2, 4096, 16), (1, 5000, 24), (6, 333, 1), (2, 64, 200), (2, 2100, 64),
+                  (1, 4096, 192), (1, 8192, 64), (1, 9000, 64)]
 
 
 @pytest.mark.parametrize("shape", SOFTMAX_SHAPES)
