@@ -4,15 +4,17 @@
 
 namespace cpmk {
 
-// cuda/gelu.cu:14 evaluates, with double-precision literals,
-//   0.5 * x * (1.0 + tanhf(0.7978845608028654 * x * (1.0 + 0.044715 * x * x)))
-// i.e. the tanh argument and the final product are formed in double, tanhf in float.
+// cuda/gelu.cu:14 evaluates 0.5 * x * (1 + tanh(c * x * (1 + 0.044715 x^2))), c = sqrt(2/pi), partly in
+// double.  With u = c x (1 + 0.044715 x^2) the same function is x / (1 + exp(-2u)), which needs
+// one exp2 and one reciprocal in fp32 and, unlike 1 + tanh(u), does not cancel for negative x.
+// The fp32 result is within a few ulps of the exact value, so its fp16 rounding is the exact
+// one or its neighbour (the bar of the contract is 1e-3 relative).
 __device__ inline half_t gelu1(half_t h) {
     const float x = (float)h;
-    const double xd = (double)x;
-    const float u = (float)(0.7978845608028654 * xd * (1.0 + 0.044715 * xd * xd));
-    const float r = (float)(0.5 * xd * (1.0 + (double)tanhf(u)));
-    return (half_t)r;
+    constexpr float k1 = -2.3022081981462618f;     // -2 log2(e) c
+    constexpr float k2 = -0.10294323958011010f;    // -2 log2(e) c * 0.044715
+    const float e = __builtin_amdgcn_exp2f(x * __builtin_fmaf(k2, x * x, k1));      // exp(-2u)
+    return (half_t)(x * __builtin_amdgcn_rcpf(1.0f + e));
 }
 
 __global__ __launch_bounds__(256) void k_gelu(int64_t total, const half_t* mat, half_t* out, int vec) {

@@ -499,8 +499,16 @@ def test_gelu_all_fp16_inputs(gpu):
     xd = to_gpu(x); out = torch.empty_like(xd)
     ck.gelu_forward(4, 16384, xd.data_ptr(), out.data_ptr(), stream())
     got = to_np(out)
-    # atol 6e-8 = one step of the fp16 subnormal grid (tanhf differs by an ulp between libraries)
-    assert_close_fp16(got, ref, rtol=1e-3, atol=6e-8, max_ulp=1, what="gelu_forward all inputs")
+    # Normal-range results: 1e-3 relative and at most one fp16 ulp from the restated reference.
+    # Below the smallest normal fp16 (x < -4.1) the reference's own 1 + tanhf(u) has one or two
+    # significant bits left (cuda/gelu.cu:14 adds 1 to a float within 1e-7 of -1), so its values
+    # there are rounding noise around the true -|x| exp(-2|u|); the kernel evaluates
+    # x / (1 + exp(-2u)), which does not cancel.  Both are within 4 steps of the subnormal grid.
+    normal = np.abs(ref.astype(np.float64)) >= 6.2e-5
+    fin = np.isfinite(ref)
+    sel = normal | ~fin
+    assert_close_fp16(np.where(sel, got, 0), np.where(sel, ref, 0), rtol=1e-3, atol=0.0, max_ulp=1, what="gelu_forward, normal range")
+    assert_close_fp16(np.where(sel, 0, got), np.where(sel, 0, ref), rtol=0.0, atol=2.4e-7, what="gelu_forward, subnormal range")
     ck.gelu_inplace_forward(4, 16384, xd.data_ptr(), stream())
     assert_bits_equal(to_np(xd), got, "in place == out of place")
     # odd length / unaligned tail
