@@ -97,10 +97,11 @@ __device__ inline int32_t quant_i8_rcp(float x, float s, float y) {
     const float q0 = x * y;
     const float r = __builtin_fmaf(-s, q0, x);
     const float q1 = __builtin_fmaf(r, y, q0);
-    const float d = (r - r == 0.0f) ? q1 : q0;
-    float q = __builtin_rintf(d);
-    q = fminf(fmaxf(q, -128.0f), 127.0f);
-    return (d != d) ? 0 : (int32_t)q;
+    const float d = __builtin_amdgcn_classf(r, 0x1f8) ? q1 : q0;      // 0x1f8: zero, subnormal or normal
+    int32_t n;
+    // v_cvt_i32_f32 saturates to the int32 range and turns NaN into 0
+    asm("v_cvt_i32_f32 %0, %1" : "=v"(n) : "v"(__builtin_rintf(d)));
+    return min(max(n, -128), 127);
 }
 
 __device__ inline uint32_t pack4_i8(int32_t a, int32_t b, int32_t c, int32_t d) {
@@ -138,6 +139,19 @@ __device__ inline uint32_t xcd_remap(uint32_t bid, uint32_t nblocks) {
     const uint32_t lim = per * kXcd;
     if (bid >= lim) return bid;                   // ragged tail keeps its index
     return (bid % kXcd) * per + bid / kXcd;
+}
+
+// Compute units of the current device (cached per device ordinal; 256 if the query fails).
+inline int compute_units() {
+    static int cus[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cus[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cus[dev] = n;
+    }
+    return cus[dev];
 }
 
 }  // namespace cpmk

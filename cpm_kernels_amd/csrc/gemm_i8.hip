@@ -570,18 +570,6 @@ static int launch_kmajor(GemmArgs& a, int batch, hipStream_t st) {
     return launch_status();
 }
 
-static int compute_units() {
-    static int cus[64] = {0};          // per device ordinal, filled on first use
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-    if (cus[dev] == 0) {
-        int n = 0;
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-        cus[dev] = n;
-    }
-    return cus[dev];
-}
-
 // waves (rows x cols), MFMA tiles per wave (rows x cols), K bytes per slab of the large-shape kernel
 #ifndef CPMK_GEMM_BIG
 #define CPMK_GEMM_BIG 2, 4, 4, 2, 128

@@ -244,25 +244,13 @@ __global__ __launch_bounds__(256) void k_gemv_dot4(int32_t batch, int32_t dim_ou
     }
 }
 
-static int gemv_compute_units() {
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) != hipSuccess ||
-            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-            n = 256;
-        cus = n;
-    }
-    return cus;
-}
-
 // Rows per workgroup: as few workgroups as there are compute units when the matrix allows it,
 // because every workgroup re-reads all the vectors (from L2); at most 64 rows.
 template <int NB, int MAXRG>
 static void launch_coalesced(int32_t batch, int32_t dim_out, int32_t dim_in, const half_t* sm, const int8_t* mat,
                              const half_t* sv, const int8_t* vec, half_t* out, hipStream_t st) {
     const int64_t groups = ceil_div(dim_out, 16);
-    int rg = (int)ceil_div(groups, gemv_compute_units());
+    int rg = (int)ceil_div(groups, compute_units());
     if (rg > MAXRG) rg = MAXRG;
     if (rg < 1) rg = 1;
     const dim3 grid((unsigned)ceil_div(groups, rg));

@@ -189,48 +189,88 @@ __global__ __launch_bounds__(256) void k_dequant(int64_t total, int32_t n, int32
 }
 
 // ---------------------------------------------------------------------------------------
-// fused absmax + round over contiguous rows (one wave per row, the row stays in
-// registers between the two phases): rows up to 64 lanes x NV x 8 halves.
+// Contiguous rows of up to 64 lanes x NV x 8 halves, one wave per row, the row in registers:
+// absmax -> scale (QUANT false: cu_gemm_calc_scale) and, fused, the rounding of the same
+// registers (QUANT true: calc_scale + round in one pass over HBM).  Waves stride over the rows;
+// the launcher picks the wave count so that every wave gets the same number of rows when the
+// row count allows.  Many resident waves, each with one row in flight, hide the memory latency
+// better here than fewer waves that prefetch their next row (measured).
 // ---------------------------------------------------------------------------------------
-template <int NV>
-__global__ __launch_bounds__(256) void k_row_quantize(int64_t rows, int32_t m,
-                                                      const half_t* __restrict__ mat,
-                                                      half_t* __restrict__ scale,
-                                                      int8_t* __restrict__ out) {
+template <int NV, bool QUANT>
+__global__ __launch_bounds__(256) void k_rows(int64_t rows, int32_t m, const half_t* __restrict__ mat,
+                                              half_t* __restrict__ scale, int8_t* __restrict__ out) {
     const int lane = threadIdx.x & 63;
-    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t nw = (int64_t)gridDim.x * 4;
+    int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= rows) return;
-    const half8_t* p8 = reinterpret_cast<const half8_t*>(mat + row * m);
     const int m8 = m >> 3;
-    half8_t v[NV];
-    float mx = 0.0f;
+    half8_t cur[NV];
+    auto load = [&](half8_t (&v)[NV], int64_t r) __attribute__((always_inline)) {
+        const half8_t* p8 = reinterpret_cast<const half8_t*>(mat + r * m);
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
-        const int j = lane + i * 64;
-        if (j < m8) {
-            v[i] = __builtin_nontemporal_load(p8 + j);
+        for (int i = 0; i < NV; ++i) {
+            const int j = lane + i * 64;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) mx = fmaxf(fabsf((float)v[i][e]), mx);
+            for (int e = 0; e < 8; ++e) v[i][e] = (half_t)0.0f;
+            if (j < m8) v[i] = __builtin_nontemporal_load(p8 + j);
         }
-    }
-    mx = wave_max(mx);
-    const half_t sh = scale_from_absmax(mx);
-    if (lane == 0) scale[row] = sh;
-    const float s = (float)sh, y = 1.0f / s;
-    uint2_t* o8 = reinterpret_cast<uint2_t*>(out + row * m);
+    };
+    load(cur, row);
+    while (true) {
+        const int64_t next = row + nw;
+        // |x| maxima on the packed halves (exact), then across the wave
+        half8_t hm;
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
-        const int j = lane + i * 64;
-        if (j < m8) {
-            int32_t q[8];
+        for (int e = 0; e < 8; ++e) hm[e] = (half_t)0.0f;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) q[e] = quant_i8_rcp((float)v[i][e], s, y);
-            uint2_t w;
-            w.x = pack4_i8(q[0], q[1], q[2], q[3]);
-            w.y = pack4_i8(q[4], q[5], q[6], q[7]);
-            o8[j] = w;
+        for (int i = 0; i < NV; ++i) hm = __builtin_elementwise_max(hm, __builtin_elementwise_abs(cur[i]));
+        float mx = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) mx = fmaxf((float)hm[e], mx);
+        mx = wave_max(mx);
+        const half_t sh = scale_from_absmax(mx);
+        if (lane == 0) scale[row] = sh;
+        if (QUANT) {
+            const float s = (float)sh, y = 1.0f / s;
+            uint2_t* o8 = reinterpret_cast<uint2_t*>(out + row * m);
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                const int j = lane + i * 64;
+                if (j < m8) {
+                    int32_t q[8];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) q[e] = quant_i8_rcp((float)cur[i][e], s, y);
+                    uint2_t w;
+                    w.x = pack4_i8(q[0], q[1], q[2], q[3]);
+                    w.y = pack4_i8(q[4], q[5], q[6], q[7]);
+                    o8[j] = w;
+                }
+            }
         }
+        if (next >= rows) break;
+        load(cur, next);
+        row = next;
     }
+}
+
+// Workgroups (4 waves each) for k_rows: between 1 and max_k per compute unit (what the register
+// budget lets be resident at once), the count that wastes the fewest wave-rows; more workgroups
+// on a tie.
+static unsigned rows_grid(int64_t rows, int cus, int nv) {
+    const int max_k = nv <= 8 ? 8 : 4;
+    const int64_t need = ceil_div(rows, 4);
+    if (need <= (int64_t)cus) return (unsigned)need;
+    int64_t best = cus;
+
+    double best_eff = 0.0;
+    for (int k = 1; k <= max_k; ++k) {
+        const int64_t g = (int64_t)cus * k;
+        if (g > need) break;
+        const int64_t per = ceil_div(rows, g * 4);
+        const double eff = (double)rows / (double)(per * g * 4);
+        if (eff >= best_eff) { best_eff = eff; best = g; }
+    }
+    return (unsigned)best;
 }
 
 static int check3(int32_t batch, int32_t n, int32_t m) {
@@ -249,6 +289,16 @@ static int row_absmax(int64_t rows, int32_t m, const void* mat, void* out, hipSt
         if (vec) hipLaunchKernelGGL((k_row_absmax<256, true>), dim3((unsigned)rows), dim3(256), 0, st, rows, m, p, o);
         else hipLaunchKernelGGL((k_row_absmax<256, false>), dim3((unsigned)rows), dim3(256), 0, st, rows, m, p, o);
     } else {
+        const int nv = (int)ceil_div(m, 512);
+        if (vec && nv <= 16) {
+            const unsigned g = rows_grid(rows, compute_units(), nv);
+            if (nv <= 1) hipLaunchKernelGGL((k_rows<1, false>), dim3(g), dim3(256), 0, st, rows, m, p, o, (int8_t*)nullptr);
+            else if (nv <= 2) hipLaunchKernelGGL((k_rows<2, false>), dim3(g), dim3(256), 0, st, rows, m, p, o, (int8_t*)nullptr);
+            else if (nv <= 4) hipLaunchKernelGGL((k_rows<4, false>), dim3(g), dim3(256), 0, st, rows, m, p, o, (int8_t*)nullptr);
+            else if (nv <= 8) hipLaunchKernelGGL((k_rows<8, false>), dim3(g), dim3(256), 0, st, rows, m, p, o, (int8_t*)nullptr);
+            else hipLaunchKernelGGL((k_rows<16, false>), dim3(g), dim3(256), 0, st, rows, m, p, o, (int8_t*)nullptr);
+            return launch_status();
+        }
         const unsigned g = (unsigned)ceil_div(rows, 4);
         if (vec) hipLaunchKernelGGL((k_row_absmax<64, true>), dim3(g), dim3(256), 0, st, rows, m, p, o);
         else hipLaunchKernelGGL((k_row_absmax<64, false>), dim3(g), dim3(256), 0, st, rows, m, p, o);
@@ -374,16 +424,16 @@ int cpmk_gemm_quantize(int32_t batch, int32_t n, int32_t m, const void* mat, voi
         if (rows == 0) return 0;
         const bool vec = (m % 8 == 0) && aligned16(mat) && ((reinterpret_cast<uintptr_t>(out) & 7u) == 0);
         if (vec && m <= 64 * 8 * 16) {
-            const unsigned g = (unsigned)ceil_div(rows, 4);
             const int nv = (int)ceil_div(m, 512);
+            const unsigned g = rows_grid(rows, compute_units(), nv);
             const half_t* p = (const half_t*)mat;
             half_t* s = (half_t*)scale;
             int8_t* o = (int8_t*)out;
-            if (nv <= 1) hipLaunchKernelGGL((k_row_quantize<1>), dim3(g), dim3(256), 0, st, rows, m, p, s, o);
-            else if (nv <= 2) hipLaunchKernelGGL((k_row_quantize<2>), dim3(g), dim3(256), 0, st, rows, m, p, s, o);
-            else if (nv <= 4) hipLaunchKernelGGL((k_row_quantize<4>), dim3(g), dim3(256), 0, st, rows, m, p, s, o);
-            else if (nv <= 8) hipLaunchKernelGGL((k_row_quantize<8>), dim3(g), dim3(256), 0, st, rows, m, p, s, o);
-            else hipLaunchKernelGGL((k_row_quantize<16>), dim3(g), dim3(256), 0, st, rows, m, p, s, o);
+            if (nv <= 1) hipLaunchKernelGGL((k_rows<1, true>), dim3(g), dim3(256), 0, st, rows, m, p, s, o);
+            else if (nv <= 2) hipLaunchKernelGGL((k_rows<2, true>), dim3(g), dim3(256), 0, st, rows, m, p, s, o);
+            else if (nv <= 4) hipLaunchKernelGGL((k_rows<4, true>), dim3(g), dim3(256), 0, st, rows, m, p, s, o);
+            else if (nv <= 8) hipLaunchKernelGGL((k_rows<8, true>), dim3(g), dim3(256), 0, st, rows, m, p, s, o);
+            else hipLaunchKernelGGL((k_rows<16, true>), dim3(g), dim3(256), 0, st, rows, m, p, s, o);
             return launch_status();
         }
         if (int e = cpmk_gemm_calc_scale(batch, n, m, mat, scale, stream)) return e;
