@@ -107,16 +107,18 @@ __global__ __launch_bounds__(NW * 64) void k_gemv_mfma(int32_t batch, int32_t di
     }
 }
 
-// Fast kernel: dim_in % 256 == 0.  Workgroup = NW waves and RG*16 matrix rows; the 256-byte K
-// chunks are dealt round-robin to the waves.  Per chunk a wave loads, fully coalesced,
-// RG*16 matrix rows and NB*16 vectors (lane l: 16-byte chunk l%16 of row l/16 + 4i), then turns
-// each 16-row group into four MFMA operands (piece j: lane (r = l%16, q = l/16) holds bytes
-// [j*64 + q*16, +16) of row r) by writing it to LDS at row*256 + ((chunk ^ row) << 4) and reading
-// it back transposed; both directions are bank-conflict free.  LDS executes one wave's
-// operations in order, so the 4 KB buffer is reused without waits.  Rows and vectors past the
-// end are clamped: they only feed outputs that are never stored.
+// Fast kernel: dim_in % 256 == 0.  Workgroup = NW waves and 4*r4 consecutive matrix rows (r4 <=
+// 4*RG; the launcher sizes r4 so that every compute unit gets one workgroup); the 256-byte K
+// chunks are dealt round-robin to the waves, two per trip so that a wave has both chunks' loads
+// in flight before it touches either.  Per chunk a wave loads, fully coalesced, its rows and
+// NB*16 vectors (lane l: 16-byte chunk l%16 of row l/16 + 4i), then turns each 16-row group into
+// four MFMA operands (piece j: lane (r = l%16, q = l/16) holds bytes [j*64 + q*16, +16) of row r)
+// by writing it to LDS at row*256 + ((chunk ^ row) << 4) and reading it back transposed; both
+// directions are bank-conflict free.  LDS executes one wave's operations in order, so the 4 KB
+// buffer is reused without waits.  Vectors past the end are clamped and row steps past r4 are
+// not loaded (the MFMA then sees stale LDS bytes): both only feed outputs that are never stored.
 template <int NW, int RG, int NB>
-__global__ __launch_bounds__(NW * 64) void k_gemv_coalesced(int32_t batch, int32_t dim_out, int32_t dim_in,
+__global__ __launch_bounds__(NW * 64) void k_gemv_coalesced(int32_t batch, int32_t dim_out, int32_t dim_in, int32_t r4,
                                                             const half_t* __restrict__ scale_mat,
                                                             const int8_t* __restrict__ mat,
                                                             const half_t* __restrict__ scale_vec,
@@ -127,7 +129,8 @@ __global__ __launch_bounds__(NW * 64) void k_gemv_coalesced(int32_t batch, int32
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int r = lane & 15, q = lane >> 4;      // MFMA layout
     const int x = lane & 15, y4 = lane >> 4;     // load layout
-    const int32_t row0 = blockIdx.x * (RG * 16);
+    const int32_t rpb = r4 * 4;                  // rows of this workgroup
+    const int32_t row0 = blockIdx.x * rpb;
     int8_t* tb = tbuf[w];
     int woff[4], roff[4];
 #pragma unroll
@@ -137,17 +140,21 @@ __global__ __launch_bounds__(NW * 64) void k_gemv_coalesced(int32_t batch, int32
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) roff[j] = r * 256 + (((j * 4 + q) ^ r) << 4);
-    const int8_t* wp[RG][4];
-    const int8_t* vp[NB][4];
+    // 32-bit byte offsets from the two base pointers (the launcher checks that they fit)
+    uint32_t wo[RG][4], vo[NB][4];
+    bool wok[RG][4];
 #pragma unroll
     for (int g = 0; g < RG; ++g)
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            wp[g][i] = mat + (int64_t)min(row0 + g * 16 + i * 4 + y4, dim_out - 1) * dim_in + x * 16;
+        for (int i = 0; i < 4; ++i) {
+            const int32_t row = row0 + (g * 4 + i) * 4 + y4;
+            wok[g][i] = (g * 4 + i) < r4;
+            wo[g][i] = (uint32_t)min(row, dim_out - 1) * (uint32_t)dim_in + x * 16;
+        }
 #pragma unroll
     for (int t = 0; t < NB; ++t)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) vp[t][i] = vec + (int64_t)min(t * 16 + i * 4 + y4, batch - 1) * dim_in + x * 16;
+        for (int i = 0; i < 4; ++i) vo[t][i] = (uint32_t)min(t * 16 + i * 4 + y4, batch - 1) * (uint32_t)dim_in + x * 16;
 
     int4_t acc[RG][NB];
 #pragma unroll
@@ -155,17 +162,20 @@ __global__ __launch_bounds__(NW * 64) void k_gemv_coalesced(int32_t batch, int32
 #pragma unroll
         for (int t = 0; t < NB; ++t) acc[g][t] = int4_t{0, 0, 0, 0};
 
-    const int nchunks = dim_in >> 8;
-    for (int c = w; c < nchunks; c += NW) {
-        int4_t wr[RG][4], vr[NB][4];
+    auto load_chunk = [&](int4_t (&wr)[RG][4], int4_t (&vr)[NB][4], int c) __attribute__((always_inline)) {
 #pragma unroll
         for (int g = 0; g < RG; ++g)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) wr[g][i] = *reinterpret_cast<const int4_t*>(wp[g][i] + c * 256);
+            for (int i = 0; i < 4; ++i) {
+                wr[g][i] = int4_t{0, 0, 0, 0};
+                if (wok[g][i]) wr[g][i] = *reinterpret_cast<const int4_t*>(mat + (wo[g][i] + (uint32_t)c * 256u));
+            }
 #pragma unroll
         for (int t = 0; t < NB; ++t)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) vr[t][i] = *reinterpret_cast<const int4_t*>(vp[t][i] + c * 256);
+            for (int i = 0; i < 4; ++i) vr[t][i] = *reinterpret_cast<const int4_t*>(vec + (vo[t][i] + (uint32_t)c * 256u));
+    };
+    auto mac_chunk = [&](int4_t (&wr)[RG][4], int4_t (&vr)[NB][4]) __attribute__((always_inline)) {
 #pragma unroll
         for (int g = 0; g < RG; ++g) {
 #pragma unroll
@@ -187,6 +197,23 @@ __global__ __launch_bounds__(NW * 64) void k_gemv_coalesced(int32_t batch, int32
 #pragma unroll
                 for (int t = 0; t < NB; ++t)
                     acc[g][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wr[g][j], vr[t][j], acc[g][t], 0, 0, 0);
+    };
+
+    const int nchunks = dim_in >> 8;
+    int c = w;
+    if constexpr (RG + NB <= 5) {      // two chunks in flight where the registers allow it
+        for (; c + NW < nchunks; c += 2 * NW) {
+            int4_t wa[RG][4], va[NB][4], wb[RG][4], vb[NB][4];
+            load_chunk(wa, va, c);
+            load_chunk(wb, vb, c + NW);
+            mac_chunk(wa, va);
+            mac_chunk(wb, vb);
+        }
+    }
+    for (; c < nchunks; c += NW) {
+        int4_t wa[RG][4], va[NB][4];
+        load_chunk(wa, va, c);
+        mac_chunk(wa, va);
     }
 
     for (int idx = tid; idx < RG * NB * 256; idx += NW * 64) (&part[0][0])[idx] = 0;
@@ -199,8 +226,9 @@ __global__ __launch_bounds__(NW * 64) void k_gemv_coalesced(int32_t batch, int32
 #pragma unroll
             for (int e = 0; e < 4; ++e) atomicAdd(&part[g * NB + t][(q * 4 + e) * 16 + r], acc[g][t][e]);
     __syncthreads();
-    for (int idx = tid; idx < RG * NB * 256; idx += NW * 64) {
-        const int rr = idx % (RG * 16), bb = idx / (RG * 16);
+    // thread -> (vector, row) with the row fastest, so a vector's outputs are stored contiguously
+    for (int idx = tid; idx < rpb * NB * 16; idx += NW * 64) {
+        const int rr = idx % rpb, bb = idx / rpb;
         const int g = rr >> 4, t = bb >> 4;
         const int32_t s = part[g * NB + t][(rr & 15) * 16 + (bb & 15)];
         const int32_t row = row0 + rr;
@@ -244,19 +272,20 @@ __global__ __launch_bounds__(256) void k_gemv_dot4(int32_t batch, int32_t dim_ou
     }
 }
 
-// Rows per workgroup: as few workgroups as there are compute units when the matrix allows it,
-// because every workgroup re-reads all the vectors (from L2); at most 64 rows.
+// Rows per workgroup, in steps of 4: one workgroup per compute unit when the matrix allows it
+// (every workgroup re-reads all the vectors from L2, so fewer and larger ones are better), at
+// most 16*MAXRG rows.
 template <int NB, int MAXRG>
 static void launch_coalesced(int32_t batch, int32_t dim_out, int32_t dim_in, const half_t* sm, const int8_t* mat,
                              const half_t* sv, const int8_t* vec, half_t* out, hipStream_t st) {
-    const int64_t groups = ceil_div(dim_out, 16);
-    int rg = (int)ceil_div(groups, compute_units());
-    if (rg > MAXRG) rg = MAXRG;
-    if (rg < 1) rg = 1;
-    const dim3 grid((unsigned)ceil_div(groups, rg));
+    int64_t r4 = ceil_div(ceil_div(dim_out, compute_units()), 4);
+    if (r4 > 4 * MAXRG) r4 = 4 * MAXRG;
+    if (r4 < 1) r4 = 1;
+    const int rg = (int)ceil_div(r4, 4);
+    const dim3 grid((unsigned)ceil_div(dim_out, r4 * 4));
     auto go = [&](auto rgc) {
         hipLaunchKernelGGL((k_gemv_coalesced<8, decltype(rgc)::value, NB>), grid, dim3(512), 0, st, batch, dim_out, dim_in,
-                           sm, mat, sv, vec, out);
+                           (int32_t)r4, sm, mat, sv, vec, out);
     };
     if constexpr (MAXRG >= 4) { if (rg == 4) return go(std::integral_constant<int, 4>{}); }
     if constexpr (MAXRG >= 3) { if (rg == 3) return go(std::integral_constant<int, 3>{}); }
@@ -312,7 +341,7 @@ extern "C" int cpmk_gemv_broadcast_mat_int8(int32_t batch, int32_t dim_out, int3
         const int8_t* v = V + (int64_t)b0 * dim_in;
         half_t* o = O + (int64_t)b0 * dim_out;
         const half_t* s = sv + b0;
-        if (dim_in % 256 == 0) {
+        if (dim_in % 256 == 0 && (int64_t)dim_out * dim_in < (1ll << 32) && (int64_t)nb * dim_in < (1ll << 32)) {
             if (nb <= 16) launch_coalesced<1, 4>(nb, dim_out, dim_in, sm, M, s, v, o, st);
             else if (nb <= 32) launch_coalesced<2, 4>(nb, dim_out, dim_in, sm, M, s, v, o, st);
             else if (nb <= 64) launch_coalesced<4, 2>(nb, dim_out, dim_in, sm, M, s, v, o, st);
