@@ -1,0 +1,167 @@
+// Per-column absmax scales and rounding of a (batch, n, m) fp16 tensor in one pass over HBM:
+//   scale[b, j] = fp16(max_i |mat[b,i,j]| / 127),   q = int8(rint(mat[b,i,j] / scale[b,j]))
+// i.e. cu_gemm_calc_scale_transpose followed by cu_gemm_round_transpose (cuda/gemm.cu:22-33,
+// 79-98), with q written either in place (b, n, m) or transposed (b, m, n).  The transposed form
+// is what lets torch-level bmm feed operands given as (batch, K, N) to the K-major int8 GEMM
+// (the reference's GEMMInt8.forward, torch/gemm.py:84-113, quantises such an operand along
+// dim 1 and leaves the transposition to cuBLASLt).
+#include "dim1.h"
+#include "exchange.h"
+
+namespace cpmk {
+
+// 64 columns x 512 rows per workgroup; taller columns are shared by a team (exchange.h) that
+// exchanges the per-column maxima.  Lane (cg = tid % 8, rg = tid / 8) holds 8 columns of the 8
+// consecutive rows rg*8 .. rg*8+7, so that its int8 results are 8 contiguous bytes in either
+// output layout.
+template <int NT>
+__global__ __launch_bounds__(NT) void k_col_quantize_team(int32_t n, int32_t m, int32_t tiles_per_batch, int32_t parts,
+                                                          const half_t* __restrict__ mat, half_t* __restrict__ scale,
+                                                          int8_t* __restrict__ out, int transposed, uint64_t* xch,
+                                                          uint32_t tag) {
+    constexpr int LPR = 8, R = 8, COLS = 64, ROWS = NT / LPR * R;
+    __shared__ float lds[(NT / 64 + 1) * COLS];
+    __shared__ float tot[COLS];
+    __shared__ int failed;
+    const int tid = threadIdx.x, cg = tid % LPR, rg = tid / LPR;
+    const uint32_t part = blockIdx.x % parts, team = blockIdx.x / parts;
+    const uint32_t b = team / tiles_per_batch, ct = team - b * tiles_per_batch;
+    const int32_t col0 = ct * COLS + cg * 8;
+    const int32_t row0 = part * ROWS + rg * 8;           // this lane's first row
+    const int64_t boff = (int64_t)b * n * m;
+    if (tid == 0) failed = 0;
+
+    half8_t v[R];
+#pragma unroll
+    for (int p = 0; p < R; ++p) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[p][e] = (half_t)0.0f;
+        if (row0 + p < n && col0 < m)
+            v[p] = *reinterpret_cast<const half8_t*>(mat + boff + ((uint32_t)(row0 + p) * (uint32_t)m + (uint32_t)col0));
+    }
+    half8_t hm = __builtin_elementwise_abs(v[0]);
+#pragma unroll
+    for (int p = 1; p < R; ++p) hm = __builtin_elementwise_max(hm, __builtin_elementwise_abs(v[p]));
+    float mx[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) mx[e] = (float)hm[e];
+    coltile_reduce<NT, LPR, 1, true>(mx, lds);           // every lane: this part's maxima of its 8 columns
+
+    if (parts > 1) {
+        uint64_t* team_slots = xch + (size_t)team * parts * kXchVals;
+        if (tid < LPR) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) xch_post(team_slots + (size_t)part * kXchVals, tid * 8 + e, mx[e], tag);
+        }
+        if (tid < COLS) {
+            const uint64_t deadline = wall_clock64() + kXchTimeoutTicks;
+            float M = 0.0f;
+            bool ok = true;
+            for (int32_t q = 0; q < parts; ++q) {
+                float x;
+                ok &= xch_wait(team_slots + (size_t)q * kXchVals + tid, tag, deadline, x);
+                M = fmaxf(M, x);
+            }
+            tot[tid] = ok ? M : __builtin_nanf("");
+            if (!ok) failed = 1;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int e = 0; e < 8; ++e) mx[e] = tot[cg * 8 + e];
+    }
+
+    half8_t sh;
+    float s[8], y[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        sh[e] = scale_from_absmax(mx[e]);
+        s[e] = (float)sh[e];
+        y[e] = 1.0f / s[e];
+    }
+    if (part == 0 && rg == 0 && col0 < m) *reinterpret_cast<half8_t*>(scale + (int64_t)b * m + col0) = sh;
+
+    uint32_t q[R][2];       // [row p][columns 0-3 | 4-7], one byte each
+#pragma unroll
+    for (int p = 0; p < R; ++p) {
+        int32_t t[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) t[e] = quant_i8_rcp((float)v[p][e], s[e], y[e]);
+        q[p][0] = pack4_i8(t[0], t[1], t[2], t[3]);
+        q[p][1] = pack4_i8(t[4], t[5], t[6], t[7]);
+    }
+    if (col0 < m) {
+        if (!transposed) {
+#pragma unroll
+            for (int p = 0; p < R; ++p)
+                if (row0 + p < n)
+                    *reinterpret_cast<uint2_t*>(out + boff + ((uint32_t)(row0 + p) * (uint32_t)m + (uint32_t)col0)) =
+                        uint2_t{q[p][0], q[p][1]};
+        } else if (row0 < n) {     // n % 8 == 0: the lane's 8 rows are in or out together
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                uint32_t lo = 0, hi = 0;       // byte p = row p of column e
+#pragma unroll
+                for (int p = 0; p < 4; ++p) {
+                    lo |= ((q[p][e >> 2] >> ((e & 3) * 8)) & 0xffu) << (p * 8);
+                    hi |= ((q[p + 4][e >> 2] >> ((e & 3) * 8)) & 0xffu) << (p * 8);
+                }
+                *reinterpret_cast<uint2_t*>(out + boff + ((uint32_t)(col0 + e) * (uint32_t)n + (uint32_t)row0)) = uint2_t{lo, hi};
+            }
+        }
+    }
+    if (parts > 1 && tid < 64) xch_retire(xch, team, parts);
+}
+
+// Any shape: rounding with per-column scales into the transposed layout, one element per thread.
+__global__ __launch_bounds__(256) void k_round_cols_transposed(int64_t total, int32_t n, int32_t m,
+                                                               const half_t* __restrict__ mat,
+                                                               const half_t* __restrict__ scale,
+                                                               int8_t* __restrict__ out) {
+    const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (gid >= total) return;
+    const int64_t bi = gid / m;                 // b*n + i
+    const int32_t j = (int32_t)(gid - bi * m);
+    const int64_t b = bi / n;
+    const int32_t i = (int32_t)(bi - b * n);
+    out[(b * m + j) * n + i] = (int8_t)quant_i8((float)mat[gid], (float)scale[b * m + j]);
+}
+
+}  // namespace cpmk
+
+using namespace cpmk;
+
+extern "C" {
+
+int cpmk_gemm_calc_scale_transpose(int32_t, int32_t, int32_t, const void*, void*, void*);
+int cpmk_gemm_round_transpose(int32_t, int32_t, int32_t, const void*, const void*, void*, void*);
+
+int cpmk_gemm_quantize_cols(int32_t batch, int32_t n, int32_t m, const void* mat, void* scale, void* out,
+                            int out_transposed, void* stream) {
+    clear_stale_error();
+    if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
+    if ((int64_t)batch * n * m == 0) return 0;
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t tiles = ceil_div(m, 64), parts = ceil_div(n, 512);
+    const bool team_ok = (m % 8 == 0) && (!out_transposed || n % 8 == 0) && aligned16(mat) && aligned16(scale) &&
+                         ((reinterpret_cast<uintptr_t>(out) & 7u) == 0) && (int64_t)n * m < (1ll << 31) &&
+                         parts <= kXchMaxParts && tiles * batch * parts <= kXchSlots;
+    if (team_ok) {
+        XchLaunch xl = {nullptr, 0};
+        if (parts > 1) {
+            const int rc = xch_begin(&xl);
+            if (rc != 0) return rc;
+        }
+        hipLaunchKernelGGL((k_col_quantize_team<512>), dim3((unsigned)(tiles * batch * parts)), dim3(512), 0, st, n, m,
+                           (int32_t)tiles, (int32_t)parts, (const half_t*)mat, (half_t*)scale, (int8_t*)out,
+                           out_transposed, xl.region, xl.tag);
+        return launch_status();
+    }
+    if (int e = cpmk_gemm_calc_scale_transpose(batch, n, m, mat, scale, stream)) return e;
+    if (!out_transposed) return cpmk_gemm_round_transpose(batch, n, m, mat, scale, out, stream);
+    const int64_t total = (int64_t)batch * n * m;
+    hipLaunchKernelGGL(k_round_cols_transposed, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, st, total, n, m,
+                       (const half_t*)mat, (const half_t*)scale, (int8_t*)out);
+    return launch_status();
+}
+
+}  // extern "C"

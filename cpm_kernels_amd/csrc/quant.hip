@@ -349,6 +349,8 @@ using namespace cpmk;
 
 extern "C" {
 
+int cpmk_gemm_quantize_cols(int32_t, int32_t, int32_t, const void*, void*, void*, int, void*);   // colquant.hip
+
 int cpmk_gemm_calc_scale(int32_t batch, int32_t n, int32_t m, const void* mat, void* out, void* stream) {
     clear_stale_error();
     if (int e = check3(batch, n, m)) return e;
@@ -439,8 +441,7 @@ int cpmk_gemm_quantize(int32_t batch, int32_t n, int32_t m, const void* mat, voi
         if (int e = cpmk_gemm_calc_scale(batch, n, m, mat, scale, stream)) return e;
         return cpmk_gemm_round(batch, n, m, mat, scale, out, stream);
     }
-    if (int e = cpmk_gemm_calc_scale_transpose(batch, n, m, mat, scale, stream)) return e;
-    return cpmk_gemm_round_transpose(batch, n, m, mat, scale, out, stream);
+    return cpmk_gemm_quantize_cols(batch, n, m, mat, scale, out, 0, stream);
 }
 
 }  // extern "C"

@@ -91,6 +91,18 @@ def gemm_quantize(batch: int, n: int, m: int,
     cpmk.gemm_quantize(batch, n, m, mat, scale, out, int(bool(transpose)), _stream(stream))
 
 
+def gemm_quantize_cols(batch: int, n: int, m: int,
+                       mat: DevicePointer,      # (b, n, m) fp16
+                       scale: DevicePointer,    # (b, m) fp16
+                       out: DevicePointer,      # (b, n, m) int8, or (b, m, n) if out_transposed
+                       out_transposed: bool,
+                       stream: CUDAStream):
+    """gemm_calc_scale_transpose + gemm_round_transpose in one pass (fuses torch/gemm.py:5-38 for
+    an operand quantised along dim 1), optionally writing the int8 tensor transposed so that it
+    is K-major for gemm_int8."""
+    cpmk.gemm_quantize_cols(batch, n, m, mat, scale, out, int(bool(out_transposed)), _stream(stream))
+
+
 def gemm_scale_x(batch: int, n: int, m: int,
                  mat: DevicePointer,        # (b, n, m)  int32
                  scale_x: DevicePointer,    # (b, n)     fp16

@@ -8,7 +8,7 @@ the six-launch sequence, which ``fused=False`` still runs through the kernel-lev
 """
 import torch
 from ..kernels import gemm_calc_scale, gemm_calc_scale_transpose, gemm_round, gemm_round_transpose, \
-    gemm_scale, gemm_int8, gemm_int8_scale, gemm_quantize
+    gemm_scale, gemm_int8, gemm_int8_scale, gemm_quantize, gemm_quantize_cols
 from ._common import cur_stream, InferenceOnly
 
 
@@ -40,6 +40,21 @@ def quantize(mat: torch.Tensor, transpose: bool):
     scale = torch.empty((b, m if transpose else n), dtype=torch.half, device=mat.device)
     out = torch.empty(mat.size(), dtype=torch.int8, device=mat.device)
     gemm_quantize(b, n, m, mat.data_ptr(), scale.data_ptr(), out.data_ptr(), transpose, cur_stream())
+    return scale, out
+
+
+def quantize_k_major(mat: torch.Tensor, k_is_dim1: bool):
+    """Quantise along K and return (scale, int8 tensor with K as the last, contiguous dim):
+    for an operand stored (b, rows, K) that is `quantize(mat, False)`; for one stored (b, K, cols)
+    the per-column quantisation of `quantize(mat, True)` with the result written transposed,
+    (b, cols, K).  Same scales and int8 values either way."""
+    if not k_is_dim1:
+        return quantize(mat, False)
+    assert mat.is_contiguous() and mat.is_cuda and mat.dtype == torch.half
+    b, k, cols = mat.size()
+    scale = torch.empty((b, cols), dtype=torch.half, device=mat.device)
+    out = torch.empty((b, cols, k), dtype=torch.int8, device=mat.device)
+    gemm_quantize_cols(b, k, cols, mat.data_ptr(), scale.data_ptr(), out.data_ptr(), True, cur_stream())
     return scale, out
 
 
@@ -80,8 +95,11 @@ class GEMMInt8(InferenceOnly):
         assert A.is_contiguous() and B.is_contiguous()
         assert A.dtype == torch.half and B.dtype == torch.half
         if fused:
-            scale_A, quantized_A = quantize(A, aT)
-            scale_B, quantized_B = quantize(B, not bT)
+            # both operands are brought to K-major int8 while they are quantised, so every
+            # layout runs on the fast GEMM kernel: A (bA, M, K) and B (bB, N, K)
+            scale_A, quantized_A = quantize_k_major(A, aT)
+            scale_B, quantized_B = quantize_k_major(B, not bT)
+            return gemm_and_scale(quantized_A, scale_A, quantized_B, scale_B, False, True, True)
         else:
             scale_A = calc_scale(A, aT)
             scale_B = calc_scale(B, not bT)

@@ -111,6 +111,15 @@ int cpmk_gemm_int8_scale(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
 int cpmk_gemm_quantize(int32_t batch, int32_t n, int32_t m, const void* mat,
                        void* scale, void* out, int transpose, void* stream);
 
+/* Per-column scales (b,m) and rounding in one pass, as cpmk_gemm_quantize with transpose = 1
+ * (cpm_kernels/torch/gemm.py:98-102 for an operand given as (b, K, N)), with the int8 result
+ * written in place (b,n,m) when out_transposed = 0 or transposed (b,m,n) when 1.  The transposed
+ * form has no counterpart in the reference, where cuBLASLt consumes the operand as it lies; here
+ * it turns such an operand into the K-major layout of the fast int8 GEMM.  Values are
+ * bit-identical to calc_scale_transpose + round_transpose. */
+int cpmk_gemm_quantize_cols(int32_t batch, int32_t n, int32_t m, const void* mat,
+                            void* scale, void* out, int out_transposed, void* stream);
+
 /* ---- decode GEMV (kernels/gemv.py, cuda/gemv.cu) --------------------------------- */
 /* out[b] = fp16( max_j |vec[b,j]| / 127 )                gemv.py:18-33 / gemv.cu:26-40 */
 int cpmk_gemv_calc_scale(int32_t batch, int32_t n, const void* vec, void* out, void* stream);

@@ -42,7 +42,7 @@ def adversarial_rows(rng, n, m):
 
 
 QUANT_SHAPES = [(1, 512, 4096), (3, 17, 1000), (2, 5, 7), (1, 1, 8), (2, 64, 48), (1, 9, 8200), (4, 33, 16),
-                (1, 2100, 128), (1, 3, 20480)]
+                (1, 2100, 128), (1, 3, 20480), (2, 4096, 192), (1, 1032, 72), (3, 520, 8)]
 
 
 @pytest.mark.parametrize("shape", QUANT_SHAPES)
@@ -95,6 +95,14 @@ def test_calc_scale_and_round_transpose(gpu, shape):
     # invariant: transposed forms == row forms on the transposed tensor
     xt = np.ascontiguousarray(x.transpose(0, 2, 1))
     assert_bits_equal(s_ref, oracle.gemm_calc_scale(xt), "transpose invariant (scale)")
+    # one-pass column quantiser, int8 in place and transposed (K-major for the GEMM)
+    for tr in (False, True):
+        s3 = torch.zeros_like(sd)
+        q3 = torch.zeros((b, m, n) if tr else (b, n, m), dtype=torch.int8, device=gpu)
+        ck.gemm_quantize_cols(b, n, m, xd.data_ptr(), s3.data_ptr(), q3.data_ptr(), tr, stream())
+        assert_bits_equal(to_np(s3), s_ref, "gemm_quantize_cols scale (transposed=%s)" % tr)
+        want = to_np(qd).transpose(0, 2, 1) if tr else to_np(qd)
+        assert_bits_equal(to_np(q3), np.ascontiguousarray(want), "gemm_quantize_cols int8 (transposed=%s)" % tr)
 
 
 def test_round_unaligned_views(gpu):
