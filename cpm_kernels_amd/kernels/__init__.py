@@ -1,7 +1,7 @@
 """Same export list as cpm_kernels/kernels/__init__.py:1-14 of the reference, plus the three
 fused launchers this build adds (gemm_int8_scale, gemm_quantize, gemm_quantize_cols,
 layernorm_affine_forward)."""
-from .offpath import embedding_forward, embedding_backward_stage1, embedding_backward_stage2, embedding_step
+from .embedding import embedding_forward, embedding_backward_stage1, embedding_backward_stage2, embedding_step
 from .gelu import gelu_forward, gelu_backward, gelu_inplace_forward
 from .gemm import gemm_calc_scale, gemm_calc_scale_transpose, gemm_round, gemm_round_transpose, gemm_scale, \
     gemm_fp16, gemm_int8, gemm_backward_round_scale, gemm_backward_scale_round, gemm_scale_x, gemm_scale_y, \
@@ -18,5 +18,5 @@ from .position_bucket import position_embedding_init, position_embedding_forward
     position_embedding_step
 from .softmax import softmax_forward, softmax_backward, softmax_inplace_forward, softmax_step_inplace
 from .offpath import transpose
-from .offpath import copy_data_to_kv, has_nan_inf
+from .utils import copy_data_to_kv, has_nan_inf
 from . import utils

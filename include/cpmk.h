@@ -120,6 +120,19 @@ int cpmk_gemm_quantize(int32_t batch, int32_t n, int32_t m, const void* mat,
 int cpmk_gemm_quantize_cols(int32_t batch, int32_t n, int32_t m, const void* mat,
                             void* scale, void* out, int out_transposed, void* stream);
 
+/* ---- callers either side of the path in a decode loop ----------------------------- */
+/* out[b,i,j] = weights[ids[b,j], i];  ids (b, seq) int32, weights (vocab, hidden) fp16,
+ * out (b, hidden, seq) fp16                    kernels/embedding.py:14-34 / embedding.cu:6-37 */
+int cpmk_embedding_forward(int32_t batch, int32_t hidden_size, int32_t seq_len, const void* ids,
+                           const void* weights, void* out, void* stream);
+/* out[b,:] = weights[ids[b],:]                 kernels/embedding.py:88-105 / embedding.cu:90-103 */
+int cpmk_embedding_step(int32_t batch, int32_t embedding_size, const void* ids,
+                        const void* weights, void* out, void* stream);
+/* out[b,pos,:] = inp[b,:];  out (b, buffer_len, n) fp16, n % 2 == 0
+ *                                              kernels/utils.py:18-37 / utils.cu:13-29 */
+int cpmk_copy_data_to_kv(int32_t batch, int32_t buffer_len, int32_t n, const void* inp,
+                         void* out, int32_t pos, void* stream);
+
 /* ---- decode GEMV (kernels/gemv.py, cuda/gemv.cu) --------------------------------- */
 /* out[b] = fp16( max_j |vec[b,j]| / 127 )                gemv.py:18-33 / gemv.cu:26-40 */
 int cpmk_gemv_calc_scale(int32_t batch, int32_t n, const void* vec, void* out, void* stream);

@@ -56,7 +56,8 @@ ON_PATH = """gelu_forward gelu_inplace_forward gemm_calc_scale gemm_calc_scale_t
 gemm_round_transpose gemm_scale gemm_int8 gemm_scale_x gemm_scale_y gemv_broadcast_mat_int8 gemv_calc_scale
 gemv_round mask arith_element_add arith_ln_mul arith_ln_mul_add layernorm_forward layernorm_inplace_forward
 layernorm_step layernorm_step_inplace position_embedding_init position_embedding_forward position_embedding_step
-softmax_forward softmax_inplace_forward softmax_step_inplace""".split()
+softmax_forward softmax_inplace_forward softmax_step_inplace embedding_forward embedding_step
+copy_data_to_kv""".split()
 
 
 def test_kernel_layer_keeps_reference_names_and_signatures():
@@ -81,6 +82,10 @@ def test_kernel_layer_keeps_reference_names_and_signatures():
                                                   "position_mapping", "weight", "out", "bidirectional", "stream"]
     assert sig(ck.mask) == ["batch", "n", "m", "inp", "mask", "value", "out", "stream"]
     assert sig(ck.arith_ln_mul_add) == ["batch", "n", "m", "inp", "alpha", "beta", "out", "stream"]
+    assert sig(ck.embedding_forward) == ["batch", "hidden_size", "seq_len", "ids", "weights", "out", "stream"]
+    assert sig(ck.embedding_step) == ["batch", "embedding_size", "ids", "weights", "out", "stream"]
+    assert sig(ck.copy_data_to_kv) == ["batch", "buffer_len", "n", "inp", "out", "pos", "stream"]
+    assert ck.utils.copy_data_to_kv is ck.copy_data_to_kv
     # off-path names raise loudly, never no-op
     for name in sorted(set(REFERENCE_KERNEL_NAMES) - set(ON_PATH)):
         with pytest.raises(NotImplementedError):

@@ -601,6 +601,33 @@ def test_elementwise(gpu, shape):
         assert_bits_equal(to_np(out), oracle.mask(x, msk, value), "mask value=%r" % value)
 
 
+@pytest.mark.parametrize("shape", [(2, 64, 128), (3, 100, 77), (1, 4096, 33), (4, 24, 1)])
+def test_embedding_and_kv_copy(gpu, shape):
+    """Pure data movement next to the path: gathers from the embedding table and the copy of a
+    decode step's hidden state into the key/value buffer (cuda/embedding.cu:6-37,90-103,
+    cuda/utils.cu:13-29), against numpy indexing."""
+    _name("embedding / copy_data_to_kv", shape)
+    b, hidden, seq = shape
+    rng = np.random.default_rng(hidden + seq)
+    vocab = 211
+    w = rand_half(rng, (vocab, hidden))
+    ids = rng.integers(0, vocab, (b, seq)).astype(np.int32)
+    wd, idd = to_gpu(w), to_gpu(ids)
+    out = torch.empty((b, hidden, seq), dtype=torch.half, device=gpu)
+    ck.embedding_forward(b, hidden, seq, idd.data_ptr(), wd.data_ptr(), out.data_ptr(), stream())
+    assert_bits_equal(to_np(out), np.ascontiguousarray(w[ids].transpose(0, 2, 1)), "embedding_forward")
+    step_ids = to_gpu(ids[:, 0].copy())
+    o2 = torch.empty((b, hidden), dtype=torch.half, device=gpu)
+    ck.embedding_step(b, hidden, step_ids.data_ptr(), wd.data_ptr(), o2.data_ptr(), stream())
+    assert_bits_equal(to_np(o2), w[ids[:, 0]], "embedding_step")
+    if hidden % 2 == 0:
+        buf = rand_half(rng, (b, 9, hidden))
+        bd = to_gpu(buf)
+        ck.copy_data_to_kv(b, 9, hidden, o2.data_ptr(), bd.data_ptr(), 5, stream())
+        want = buf.copy(); want[:, 5, :] = w[ids[:, 0]]
+        assert_bits_equal(to_np(bd), want, "copy_data_to_kv")
+
+
 def test_error_codes(gpu):
     """Bad arguments come back as RuntimeError from the C ABI / AssertionError from the asserts
     the reference has (kernels/gemm.py:139-140, gemv.py:65, arith.py:53,146)."""
