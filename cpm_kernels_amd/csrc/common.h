@@ -15,6 +15,7 @@ typedef float float4_t __attribute__((ext_vector_type(4)));
 typedef int32_t int4_t __attribute__((ext_vector_type(4)));
 typedef int32_t int2_t __attribute__((ext_vector_type(2)));
 typedef int32_t int16_tv __attribute__((ext_vector_type(16)));
+typedef float float16_tv __attribute__((ext_vector_type(16)));
 typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
 

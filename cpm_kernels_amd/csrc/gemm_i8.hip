@@ -18,6 +18,8 @@
 //                  owns 4 consecutive output columns (8/16-byte stores).
 //   k_gemm_kmajor  both operands K-major, k % 16 == 0: register-staged 64-byte K slabs.
 //   k_gemm_generic any layout and size: LDS tiles + v_dot4_i32_i8.
+// The tile kernel also serves the fp16 product of kernels/gemm.py:188-256 (cpmk_gemm_fp16): the
+// same bytes of K per lane feed v_mfma_f32_32x32x16_f16, with fp32 accumulators.
 #include "common.h"
 #include <type_traits>
 
@@ -201,6 +203,11 @@ __device__ __forceinline__ void wait_vmcnt() {
 #define CPMK_GEMM_MPM 0     // >0: that many memory operations after each MFMA from the start of a k-step; 0: spread evenly
 #endif
 
+// What the tile kernel does with its accumulators.
+constexpr int kEpiInt32 = 0;     // int8 product, int32 out
+constexpr int kEpiDequant = 1;   // int8 product, fp16( (f32(acc) * s_row) * s_col ) out
+constexpr int kEpiF16 = 2;       // fp16 product with fp32 accumulation, fp16 out
+
 struct DmaArgs {
     GemmArgs g;
     int32_t batch;
@@ -250,9 +257,11 @@ __device__ __forceinline__ GemmItem gemm_item(uint32_t L, const DmaArgs& da) {
 // overlap this tile's stores; otherwise the slab index is clamped (a redundant load nobody
 // reads).  Either way the loop body has no branches, which lets the compiler keep the
 // accumulators in place.  Returns true if the next tile's first two slabs are on their way.
-template <int WR, int WC, int TR, int TC, int BKB, bool FUSED>
+template <int WR, int WC, int TR, int TC, int BKB, int EPI>
 __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, uint32_t lds_base, const GemmItem cur_item,
                                               const GemmItem nxt_item, const bool have_slabs) {
+    constexpr bool FUSED = EPI == kEpiDequant, F16 = EPI == kEpiF16;
+    using acc_t = std::conditional_t<F16, float16_tv, int16_tv>;
     constexpr int KS = BKB / 32, CPR = BKB / 16;
     constexpr int NW = WR * WC, BR = WR * TR * 32, BC = WC * TC * 32;
     constexpr int STAGE = (BR + BC) * BKB;
@@ -338,7 +347,7 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, u
             }
     }
 
-    int16_tv acc[TR][TC];
+    acc_t acc[TR][TC];
 #pragma unroll
     for (int i = 0; i < TR; ++i)
 #pragma unroll
@@ -361,7 +370,11 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, u
             constexpr int i = x / TC, j = x % TC;
             // MFMA "A" = column-operand rows, "B" = row-operand rows: lane l, register e of the
             // result is output row l%32, column (e/4)*8 + (l/32)*4 + e%4 of the 32x32 tile
-            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fq[buf][j], fp[buf][i], acc[i][j], 0, 0, 0);
+            if constexpr (F16)      // 32 bytes of K are 16 halves: same lane -> byte assignment as the int8 MFMA
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, fq[buf][j]),
+                                                                   __builtin_bit_cast(half8_t, fp[buf][i]), acc[i][j], 0, 0, 0);
+            else
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fq[buf][j], fp[buf][i], acc[i][j], 0, 0, 0);
 #if CPMK_GEMM_MPM
             constexpr int lo = x * CPMK_GEMM_MPM < NMEM ? x * CPMK_GEMM_MPM : NMEM;
             constexpr int hi = (x == NM - 1 || (x + 1) * CPMK_GEMM_MPM > NMEM) ? NMEM : (x + 1) * CPMK_GEMM_MPM;
@@ -434,15 +447,20 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, u
                 const int32_t col = i0 + wc * TC * 32 + j * 32 + g4 * 8 + lk * 4;
                 if (row < a.n && col < a.m) {      // m % 4 == 0: the four columns are in or out together
                     const int64_t o = obase + (int64_t)row * a.m + col;
-                    if (FUSED) {
+                    if constexpr (F16) {
+                        half4_t h;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) h[e] = (half_t)acc[i][j][g4 * 4 + e];
+                        *reinterpret_cast<half4_t*>(reinterpret_cast<half_t*>(a.out) + o) = h;
+                    } else if constexpr (FUSED) {
                         const half4_t sy = syh[j][g4];
                         half4_t h;
 #pragma unroll
                         for (int e = 0; e < 4; ++e) h[e] = dequant(acc[i][j][g4 * 4 + e], sx, (float)sy[e]);
                         *reinterpret_cast<half4_t*>(reinterpret_cast<half_t*>(a.out) + o) = h;
                     } else {
-                        const int4_t v = {acc[i][j][g4 * 4], acc[i][j][g4 * 4 + 1], acc[i][j][g4 * 4 + 2],
-                                          acc[i][j][g4 * 4 + 3]};
+                        const int4_t v = {(int32_t)acc[i][j][g4 * 4], (int32_t)acc[i][j][g4 * 4 + 1],
+                                          (int32_t)acc[i][j][g4 * 4 + 2], (int32_t)acc[i][j][g4 * 4 + 3]};
                         *reinterpret_cast<int4_t*>(reinterpret_cast<int32_t*>(a.out) + o) = v;
                     }
                 }
@@ -457,7 +475,7 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, u
 // tiles and share operand slabs in that XCD's L2.  When the tile count leaves a last round
 // that at most half the workgroups could join, those tiles are issued as column halves
 // (HALVES), one per workgroup, so the round takes half as long.
-template <int WR, int WC, int TR, int TC, int BKB, bool FUSED, bool HALVES>
+template <int WR, int WC, int TR, int TC, int BKB, int EPI, bool HALVES>
 __global__ __launch_bounds__(WR* WC * 64) void k_gemm_dma(DmaArgs da) {
     constexpr int BR = WR * TR * 32, BC = WC * TC * 32;
     extern __shared__ __attribute__((aligned(16))) int8_t smem[];
@@ -470,9 +488,9 @@ __global__ __launch_bounds__(WR* WC * 64) void k_gemm_dma(DmaArgs da) {
         const GemmItem nxt = gemm_item<BR, BC>(L + G, da);
         if (HALVES && cur.half) {
             if constexpr (HALVES)
-                have_slabs = gemm_dma_tile<WR, WC, TR, TC / 2, BKB, FUSED>(da.g, smem, lds_base, cur, nxt, have_slabs);
+                have_slabs = gemm_dma_tile<WR, WC, TR, TC / 2, BKB, EPI>(da.g, smem, lds_base, cur, nxt, have_slabs);
         } else {
-            have_slabs = gemm_dma_tile<WR, WC, TR, TC, BKB, FUSED>(da.g, smem, lds_base, cur, nxt, have_slabs);
+            have_slabs = gemm_dma_tile<WR, WC, TR, TC, BKB, EPI>(da.g, smem, lds_base, cur, nxt, have_slabs);
         }
         cur = nxt;
     }
@@ -575,11 +593,11 @@ static int launch_kmajor(GemmArgs& a, int batch, hipStream_t st) {
 #define CPMK_GEMM_BIG 2, 4, 4, 2, 128
 #endif
 
-template <int WR, int WC, int TR, int TC, int BKB, bool FUSED, bool HALVES>
+template <int WR, int WC, int TR, int TC, int BKB, int EPI, bool HALVES>
 static int launch_dma_kernel(const DmaArgs& da, unsigned grid, hipStream_t st) {
     constexpr int BR = WR * TR * 32, BC = WC * TC * 32;
     constexpr int smem = 2 * (BR + BC) * BKB;
-    auto kern = k_gemm_dma<WR, WC, TR, TC, BKB, FUSED, HALVES>;
+    auto kern = k_gemm_dma<WR, WC, TR, TC, BKB, EPI, HALVES>;
     static bool attr_set[64] = {false};       // dynamic LDS above 64 KB must be enabled per device
     int dev = 0;
     (void)hipGetDevice(&dev);
@@ -593,7 +611,7 @@ static int launch_dma_kernel(const DmaArgs& da, unsigned grid, hipStream_t st) {
     return launch_status();
 }
 
-template <int WR, int WC, int TR, int TC, int BKB, bool FUSED>
+template <int WR, int WC, int TR, int TC, int BKB, int EPI>
 static int launch_dma(GemmArgs& a, int batch, hipStream_t st) {
     constexpr int BR = WR * TR * 32, BC = WC * TC * 32;
     a.tiles_r = (int32_t)ceil_div(a.n, BR);
@@ -612,9 +630,9 @@ static int launch_dma(GemmArgs& a, int batch, hipStream_t st) {
     if (TC % 2 == 0 && r > 0 && 2 * r <= grid) {
         da.nfull = (uint32_t)(total - r);
         da.nhalf = (uint32_t)(2 * r);
-        return launch_dma_kernel<WR, WC, TR, TC, BKB, FUSED, (TC % 2 == 0)>(da, (unsigned)grid, st);
+        return launch_dma_kernel<WR, WC, TR, TC, BKB, EPI, (TC % 2 == 0)>(da, (unsigned)grid, st);
     }
-    return launch_dma_kernel<WR, WC, TR, TC, BKB, FUSED, false>(da, (unsigned)grid, st);
+    return launch_dma_kernel<WR, WC, TR, TC, BKB, EPI, false>(da, (unsigned)grid, st);
 }
 
 template <bool FUSED>
@@ -639,8 +657,8 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
     if (fast && (k % 128 == 0) && (int64_t)n * k < (1ll << 32) && (int64_t)m * k < (1ll << 32)) {
         // 256x256 tiles when they give most compute units a tile, else 128x128
         const int64_t big = ceil_div(n, 256) * ceil_div(m, 256) * batch;
-        if (big * 4 >= compute_units() * 3) return launch_dma<CPMK_GEMM_BIG, FUSED>(a, batch, st);
-        return launch_dma<2, 2, 2, 2, 128, FUSED>(a, batch, st);
+        if (big * 4 >= compute_units() * 3) return launch_dma<CPMK_GEMM_BIG, FUSED ? kEpiDequant : kEpiInt32>(a, batch, st);
+        return launch_dma<2, 2, 2, 2, 128, FUSED ? kEpiDequant : kEpiInt32>(a, batch, st);
     }
     if (fast) {
         const int64_t t256 = ceil_div(n, 256) * ceil_div(m, 128) * batch;
@@ -650,6 +668,99 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
     dim3 grid((unsigned)ceil_div(m, 64), (unsigned)ceil_div(n, 64), (unsigned)batch);
     if (grid.y > 65535) return CPMK_ETOOBIG;
     hipLaunchKernelGGL((k_gemm_generic<FUSED>), grid, dim3(256), 0, st, a, (int)p_kmajor, (int)q_kmajor);
+    return launch_status();
+}
+
+// ---------------------------------------------------------------------------------------
+// fp16 product (fp32 accumulation), any layout and size: 64x64 output tile, 16 halves of K per
+// stage, 256 threads each computing a 4x4 block.  The K-major, k % 64 == 0 case runs on the
+// tile kernel above with the fp16 MFMA instead.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_gemm_f16_generic(GemmArgs a, int p_kmajor, int q_kmajor) {
+    constexpr int T = 64, GK = 16, LD = GK + 2;
+    __shared__ half_t sP[T * LD];
+    __shared__ half_t sQ[T * LD];
+    const int b = blockIdx.z;
+    const int32_t k = a.k >> 1;                        // a.k is the row length in bytes
+    const half_t* P = reinterpret_cast<const half_t*>(a.P + (int64_t)b * a.strideP);
+    const half_t* Q = reinterpret_cast<const half_t*>(a.Q + (int64_t)b * a.strideQ);
+    const int32_t j0 = blockIdx.y * T, i0 = blockIdx.x * T;
+    const int tid = threadIdx.x, ty = tid >> 4, tx = tid & 15;
+    float acc[4][4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[r][c] = 0.0f;
+    for (int32_t k0 = 0; k0 < k; k0 += GK) {
+#pragma unroll
+        for (int s = 0; s < T * GK / 256; ++s) {
+            const int q = tid + s * 256;
+            int r, kk;
+            if (p_kmajor) { r = q / GK; kk = q % GK; } else { r = q % T; kk = q / T; }
+            const int32_t row = j0 + r, kg = k0 + kk;
+            half_t v = (half_t)0.0f;
+            if (row < a.n && kg < k) v = p_kmajor ? P[(int64_t)row * k + kg] : P[(int64_t)kg * a.n + row];
+            sP[r * LD + kk] = v;
+            if (q_kmajor) { r = q / GK; kk = q % GK; } else { r = q % T; kk = q / T; }
+            const int32_t col = i0 + r;
+            const int32_t kg2 = k0 + kk;
+            v = (half_t)0.0f;
+            if (col < a.m && kg2 < k) v = q_kmajor ? Q[(int64_t)col * k + kg2] : Q[(int64_t)kg2 * a.m + col];
+            sQ[r * LD + kk] = v;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < GK; ++kk) {
+            float pa[4], qb[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) pa[r] = (float)sP[(ty * 4 + r) * LD + kk];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) qb[c] = (float)sQ[(tx + c * 16) * LD + kk];
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int c = 0; c < 4; ++c) acc[r][c] = __builtin_fmaf(pa[r], qb[c], acc[r][c]);
+        }
+        __syncthreads();
+    }
+    const int64_t obase = (int64_t)b * a.n * a.m;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int32_t row = j0 + ty * 4 + r;
+        if (row >= a.n) continue;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int32_t col = i0 + tx + c * 16;
+            if (col < a.m) reinterpret_cast<half_t*>(a.out)[obase + (int64_t)row * a.m + col] = (half_t)acc[r][c];
+        }
+    }
+}
+
+static int gemm_f16_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_t batchB, int aT, int bT,
+                             const void* A, const void* B, void* out, hipStream_t st) {
+    if (m < 0 || n < 0 || k < 0 || batchA < 1 || batchB < 1) return CPMK_EBADARG;
+    if ((m % 2) || (n % 2) || (k % 2)) return CPMK_EALIGN;      // kernels/gemm.py:200
+    if (!(batchA == batchB || batchA == 1 || batchB == 1)) return CPMK_EBADARG;   // :201
+    const int batch = batchA > batchB ? batchA : batchB;
+    if (m == 0 || n == 0) return 0;
+    if (batch > 65535 || k > (1 << 30)) return CPMK_ETOOBIG;
+    GemmArgs a;
+    a.P = (const int8_t*)B; a.Q = (const int8_t*)A; a.out = out;
+    a.srow = nullptr; a.scol = nullptr;
+    a.strideP = batchB == 1 ? 0 : (int64_t)n * k * 2;          // bytes
+    a.strideQ = batchA == 1 ? 0 : (int64_t)m * k * 2;
+    a.n = n; a.m = m; a.k = k * 2; a.bc_row = 0; a.bc_col = 0;
+    a.tiles_r = a.tiles_c = 0;
+    const bool p_kmajor = !bT, q_kmajor = aT != 0;
+    if (p_kmajor && q_kmajor && k > 0 && (k % 64 == 0) && (m % 4 == 0) && aligned16(A) && aligned16(B) &&
+        (int64_t)n * k * 2 < (1ll << 32) && (int64_t)m * k * 2 < (1ll << 32)) {
+        const int64_t big = ceil_div(n, 256) * ceil_div(m, 256) * batch;
+        if (big * 4 >= compute_units() * 3) return launch_dma<CPMK_GEMM_BIG, kEpiF16>(a, batch, st);
+        return launch_dma<2, 2, 2, 2, 128, kEpiF16>(a, batch, st);
+    }
+    dim3 grid((unsigned)ceil_div(m, 64), (unsigned)ceil_div(n, 64), (unsigned)batch);
+    if (grid.y > 65535) return CPMK_ETOOBIG;
+    hipLaunchKernelGGL(k_gemm_f16_generic, grid, dim3(256), 0, st, a, (int)p_kmajor, (int)q_kmajor);
     return launch_status();
 }
 
@@ -672,6 +783,12 @@ int cpmk_gemm_int8_scale(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
     clear_stale_error();
     return gemm_dispatch<true>(m, k, n, batchA, batchB, aT, bT, A, B, scale_row, scale_col, broad_cast_row,
                                broad_cast_col, out, (hipStream_t)stream);
+}
+
+int cpmk_gemm_fp16(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_t batchB, int aT, int bT,
+                   const void* A, const void* B, void* out, void* stream) {
+    clear_stale_error();
+    return gemm_f16_dispatch(m, k, n, batchA, batchB, aT, bT, A, B, out, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -1,0 +1,141 @@
+// fp16 matrix-vector products of the decode loop (cuda/gemv.cu:78-175 and the cuBLASLt calls
+// of kernels/gemv.py:82-283), fp32 accumulation, fp16 result:
+//   gemv_fp16               out[b,o] = sum_k mat[b,o,k] * vec[b,k]
+//   gemv_fp16_transpose     out[b,o] = sum_k mat[b,k,o] * vec[b,k]
+//   gemv_broadcast_mat_fp16 out[b,o] = sum_k mat[o,k]   * vec[b,k]    (one matrix for all vectors)
+// All three stream the matrix from HBM once.
+#include "common.h"
+
+namespace cpmk {
+
+// One wave per (batch, row): 16-byte loads of the row and of the vector, wave reduction.
+// mat_bstride = 0 shares the matrix over the batch (then the rows of all vectors are done by one
+// wave, so the matrix is still read once).
+template <int NB>
+__global__ __launch_bounds__(256) void k_gemv_f16_rows(int32_t batch, int32_t dim_out, int32_t dim_in, int64_t mat_bstride,
+                                                       const half_t* __restrict__ mat, const half_t* __restrict__ vec,
+                                                       half_t* __restrict__ out, int vec8) {
+    const int lane = threadIdx.x & 63;
+    const int64_t item = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    // private matrices: item = b*dim_out + row; shared matrix: item = row, all NB vectors of a pass
+    const int64_t b0 = mat_bstride ? item / dim_out : (int64_t)blockIdx.y * NB;
+    const int32_t row = (int32_t)(mat_bstride ? item - b0 * dim_out : item);
+    if (row >= dim_out || b0 >= batch) return;
+    const half_t* mrow = mat + b0 * mat_bstride + (int64_t)row * dim_in;
+    float acc[NB];
+#pragma unroll
+    for (int t = 0; t < NB; ++t) acc[t] = 0.0f;
+    if (vec8) {
+        for (int32_t i = lane; i < (dim_in >> 3); i += 64) {
+            const half8_t w = reinterpret_cast<const half8_t*>(mrow)[i];
+#pragma unroll
+            for (int t = 0; t < NB; ++t) {
+                if (b0 + t < batch) {
+                    const half8_t v = reinterpret_cast<const half8_t*>(vec + (b0 + t) * dim_in)[i];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) acc[t] = __builtin_fmaf((float)w[e], (float)v[e], acc[t]);
+                }
+            }
+        }
+    } else {
+        for (int32_t i = lane; i < dim_in; i += 64) {
+            const float w = (float)mrow[i];
+#pragma unroll
+            for (int t = 0; t < NB; ++t)
+                if (b0 + t < batch) acc[t] = __builtin_fmaf(w, (float)vec[(b0 + t) * dim_in + i], acc[t]);
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < NB; ++t) {
+        const float s = wave_sum(acc[t]);
+        if (lane == 0 && b0 + t < batch) out[(b0 + t) * dim_out + row] = (half_t)s;
+    }
+}
+
+// mat (batch, dim_in, dim_out): 256 threads = 32 row groups x 8 lanes of 8 adjacent columns; the
+// row groups stride over dim_in and are combined in LDS.  gridDim = (ceil(dim_out/64), batch).
+__global__ __launch_bounds__(256) void k_gemv_f16_transpose(int32_t dim_out, int32_t dim_in, const half_t* __restrict__ mat,
+                                                            const half_t* __restrict__ vec, half_t* __restrict__ out,
+                                                            int vec8) {
+    __shared__ float red[32][65];
+    const int lane8 = threadIdx.x & 7, rg = threadIdx.x >> 3;
+    const int32_t col0 = blockIdx.x * 64 + lane8 * 8;
+    const int64_t b = blockIdx.y;
+    const half_t* base = mat + b * dim_in * dim_out;
+    const half_t* v = vec + b * dim_in;
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
+    for (int32_t i = rg; i < dim_in; i += 32) {
+        const float x = (float)v[i];
+        if (vec8) {
+            if (col0 < dim_out) {
+                const half8_t w = *reinterpret_cast<const half8_t*>(base + (int64_t)i * dim_out + col0);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(x, (float)w[e], acc[e]);
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (col0 + e < dim_out) acc[e] = __builtin_fmaf(x, (float)base[(int64_t)i * dim_out + col0 + e], acc[e]);
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) red[rg][lane8 * 8 + e] = acc[e];
+    __syncthreads();
+    if (threadIdx.x < 64) {
+        float r = 0.0f;
+#pragma unroll 8
+        for (int g = 0; g < 32; ++g) r += red[g][threadIdx.x];
+        const int32_t col = blockIdx.x * 64 + threadIdx.x;
+        if (col < dim_out) out[b * dim_out + col] = (half_t)r;
+    }
+}
+
+}  // namespace cpmk
+
+using namespace cpmk;
+
+extern "C" {
+
+int cpmk_gemv_fp16(int32_t batch, int32_t dim_out, int32_t dim_in, const void* mat, const void* vec, void* out,
+                   void* stream) {
+    clear_stale_error();
+    if (batch < 0 || dim_out < 0 || dim_in < 0) return CPMK_EBADARG;
+    if ((int64_t)batch * dim_out == 0) return 0;
+    const int vec8 = (dim_in % 8 == 0) && aligned16(mat) && aligned16(vec);
+    const int64_t items = (int64_t)batch * dim_out;
+    hipLaunchKernelGGL((k_gemv_f16_rows<1>), dim3((unsigned)ceil_div(items, 4)), dim3(256), 0, (hipStream_t)stream, batch,
+                       dim_out, dim_in, (int64_t)dim_out * dim_in, (const half_t*)mat, (const half_t*)vec, (half_t*)out, vec8);
+    return launch_status();
+}
+
+int cpmk_gemv_fp16_transpose(int32_t batch, int32_t dim_out, int32_t dim_in, const void* mat, const void* vec, void* out,
+                             void* stream) {
+    clear_stale_error();
+    if (batch < 0 || dim_out < 0 || dim_in < 0) return CPMK_EBADARG;
+    if ((int64_t)batch * dim_out == 0) return 0;
+    if (batch > 65535) return CPMK_ETOOBIG;
+    const int vec8 = (dim_out % 8 == 0) && aligned16(mat);
+    dim3 grid((unsigned)ceil_div(dim_out, 64), (unsigned)batch);
+    hipLaunchKernelGGL(k_gemv_f16_transpose, grid, dim3(256), 0, (hipStream_t)stream, dim_out, dim_in, (const half_t*)mat,
+                       (const half_t*)vec, (half_t*)out, vec8);
+    return launch_status();
+}
+
+int cpmk_gemv_broadcast_mat_fp16(int32_t batch, int32_t dim_out, int32_t dim_in, const void* mat, const void* vec,
+                                 void* out, void* stream) {
+    clear_stale_error();
+    if (batch < 0 || dim_out < 0 || dim_in < 0) return CPMK_EBADARG;
+    if ((int64_t)batch * dim_out == 0) return 0;
+    const int vec8 = (dim_in % 8 == 0) && aligned16(mat) && aligned16(vec);
+    constexpr int NB = 8;               // vectors per pass over a matrix row
+    const int64_t passes = ceil_div(batch, NB);
+    if (passes > 65535) return CPMK_ETOOBIG;
+    dim3 grid((unsigned)ceil_div(dim_out, 4), (unsigned)passes);
+    hipLaunchKernelGGL((k_gemv_f16_rows<NB>), grid, dim3(256), 0, (hipStream_t)stream, batch, dim_out, dim_in, (int64_t)0,
+                       (const half_t*)mat, (const half_t*)vec, (half_t*)out, vec8);
+    return launch_status();
+}
+
+}  // extern "C"

@@ -121,6 +121,18 @@ def gemm_scale_y(batch: int, n: int, m: int,
     cpmk.gemm_scale_y(batch, n, m, mat, scale_y, out, _stream(stream))
 
 
-gemm_fp16 = not_on_path("gemm_fp16", "fp16 cuBLASLt GEMM, kernels/gemm.py:188-256")
+def gemm_fp16(m: int, k: int, n: int,
+              batchA: int, batchB: int,
+              aT: bool, bT: bool,
+              A: DevicePointer,      # (bA, k, m) fp16   [(bA, m, k) if aT]
+              B: DevicePointer,      # (bB, n, k) fp16   [(bB, k, n) if bT]
+              out: DevicePointer,    # (max(bA, bB), n, m) fp16
+              stream: CUDAStream):
+    """reference: kernels/gemm.py:188-256 (cuBLASLt); same asserts (:200-201).  fp32 accumulation."""
+    assert m % 2 == 0 and n % 2 == 0 and k % 2 == 0
+    assert batchA == batchB or batchA == 1 or batchB == 1
+    cpmk.gemm_fp16(m, k, n, batchA, batchB, int(bool(aT)), int(bool(bT)), A, B, out, _stream(stream))
+
+
 gemm_backward_round_scale = not_on_path("gemm_backward_round_scale", "training, kernels/gemm.py:258-281")
 gemm_backward_scale_round = not_on_path("gemm_backward_scale_round", "training, kernels/gemm.py:283-307")

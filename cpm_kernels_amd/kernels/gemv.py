@@ -1,6 +1,6 @@
 """Decode GEMV launchers with the signatures of cpm_kernels/kernels/gemv.py."""
 from ..library import cpmk
-from .base import DevicePointer, CUDAStream, _stream, not_on_path
+from .base import DevicePointer, CUDAStream, _stream
 
 
 def gemv_calc_scale(batch: int, n: int,
@@ -32,10 +32,48 @@ def gemv_broadcast_mat_int8(batch: int, dim_out: int, dim_in: int,
     cpmk.gemv_broadcast_mat_int8(batch, dim_out, dim_in, scale_mat, mat, scale_vec, vec, out, _stream(stream))
 
 
-_w = "fp16 GEMV, kernels/gemv.py:82-283"
-gemv_fp16 = not_on_path("gemv_fp16", _w)
-gemv_fp16_light = not_on_path("gemv_fp16_light", _w)
-gemv_fp16_transpose = not_on_path("gemv_fp16_transpose", _w)
-gemv_fp16_transpose_light = not_on_path("gemv_fp16_transpose_light", _w)
-gemv_broadcast_mat_fp16 = not_on_path("gemv_broadcast_mat_fp16", _w)
-gemv_broadcast_mat_fp16_light = not_on_path("gemv_broadcast_mat_fp16_light", _w)
+def gemv_fp16(batch: int, dim_out: int, dim_in: int,
+              mat: DevicePointer,     # (batch, dim_out, dim_in) fp16
+              vec: DevicePointer,     # (batch, dim_in)   fp16
+              out: DevicePointer,     # (batch, dim_out)  fp16
+              stream: CUDAStream):
+    """reference: kernels/gemv.py:82-127 (cuBLASLt)"""
+    cpmk.gemv_fp16(batch, dim_out, dim_in, mat, vec, out, _stream(stream))
+
+
+def gemv_fp16_light(batch: int, dim_out: int, dim_in: int, mat: DevicePointer, vec: DevicePointer,
+                    out: DevicePointer, stream: CUDAStream):
+    """reference: kernels/gemv.py:129-149 (the reference's own kernel instead of cuBLASLt)"""
+    assert dim_in % 2 == 0
+    cpmk.gemv_fp16(batch, dim_out, dim_in, mat, vec, out, _stream(stream))
+
+
+def gemv_fp16_transpose(batch: int, dim_out: int, dim_in: int,
+                        mat: DevicePointer,     # (batch, dim_in, dim_out) fp16
+                        vec: DevicePointer,     # (batch, dim_in)   fp16
+                        out: DevicePointer,     # (batch, dim_out)  fp16
+                        stream: CUDAStream):
+    """reference: kernels/gemv.py:151-196 (cuBLASLt)"""
+    cpmk.gemv_fp16_transpose(batch, dim_out, dim_in, mat, vec, out, _stream(stream))
+
+
+def gemv_fp16_transpose_light(batch: int, dim_out: int, dim_in: int, mat: DevicePointer, vec: DevicePointer,
+                              out: DevicePointer, stream: CUDAStream):
+    """reference: kernels/gemv.py:198-216"""
+    cpmk.gemv_fp16_transpose(batch, dim_out, dim_in, mat, vec, out, _stream(stream))
+
+
+def gemv_broadcast_mat_fp16(batch: int, dim_out: int, dim_in: int,
+                            mat: DevicePointer,     # (dim_out, dim_in) fp16
+                            vec: DevicePointer,     # (batch, dim_in)   fp16
+                            out: DevicePointer,     # (batch, dim_out)  fp16
+                            stream: CUDAStream):
+    """reference: kernels/gemv.py:218-262 (cuBLASLt)"""
+    cpmk.gemv_broadcast_mat_fp16(batch, dim_out, dim_in, mat, vec, out, _stream(stream))
+
+
+def gemv_broadcast_mat_fp16_light(batch: int, dim_out: int, dim_in: int, mat: DevicePointer, vec: DevicePointer,
+                                  out: DevicePointer, stream: CUDAStream):
+    """reference: kernels/gemv.py:264-283"""
+    assert dim_in % 2 == 0
+    cpmk.gemv_broadcast_mat_fp16(batch, dim_out, dim_in, mat, vec, out, _stream(stream))

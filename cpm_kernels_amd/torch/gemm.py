@@ -8,7 +8,7 @@ the six-launch sequence, which ``fused=False`` still runs through the kernel-lev
 """
 import torch
 from ..kernels import gemm_calc_scale, gemm_calc_scale_transpose, gemm_round, gemm_round_transpose, \
-    gemm_scale, gemm_int8, gemm_int8_scale, gemm_quantize, gemm_quantize_cols
+    gemm_scale, gemm_int8, gemm_int8_scale, gemm_quantize, gemm_quantize_cols, gemm_fp16
 from ._common import cur_stream, InferenceOnly
 
 
@@ -111,13 +111,17 @@ class GEMMInt8(InferenceOnly):
 class GEMMFloat(InferenceOnly):
     @staticmethod
     def forward(ctx, A: torch.Tensor, aT: bool, B: torch.Tensor, bT: bool):
-        """fp16 product through the vendor BLAS (the reference calls cuBLASLt here,
-        torch/gemm.py:159-231); not a hand-written kernel and not on the int8 path."""
+        """fp16 product with fp32 accumulation.  reference: torch/gemm.py:159-231 (cuBLASLt there);
+        operands are passed swapped to the kernel exactly as in :170-183 so that the (M, N)
+        result comes out row-major."""
         assert A.is_cuda and B.is_cuda and A.device == B.device
-        assert A.dtype == B.dtype
-        a = A.transpose(-1, -2) if aT else A
-        b = B.transpose(-1, -2) if bT else B
-        return torch.matmul(a, b)
+        assert A.is_contiguous() and B.is_contiguous()
+        assert A.dtype == torch.half and B.dtype == torch.half
+        M, K, N = _dims(A, B, aT, bT)
+        batch = max(A.size(0), B.size(0))
+        out = torch.empty((batch, M, N), dtype=torch.half, device=A.device)
+        gemm_fp16(N, K, M, B.size(0), A.size(0), bT, aT, B.data_ptr(), A.data_ptr(), out.data_ptr(), cur_stream())
+        return out
 
 
 def bmm(A: torch.Tensor, aT: bool, B: torch.Tensor, bT: bool, int8: bool = False, fused: bool = True) -> torch.Tensor:

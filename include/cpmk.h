@@ -120,6 +120,22 @@ int cpmk_gemm_quantize(int32_t batch, int32_t n, int32_t m, const void* mat,
 int cpmk_gemm_quantize_cols(int32_t batch, int32_t n, int32_t m, const void* mat,
                             void* scale, void* out, int out_transposed, void* stream);
 
+/* ---- fp16 products next to the path (attention scores, fp16 decode) ---------------- */
+/* Same operand convention as cpmk_gemm_int8 with fp16 operands and fp16 output, fp32
+ * accumulation (the reference asks cuBLASLt for fp16 accumulation where the device has it).
+ * Requires m, n, k even as the reference asserts.        kernels/gemm.py:188-256 (cuBLASLt) */
+int cpmk_gemm_fp16(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_t batchB,
+                   int aT, int bT, const void* A, const void* B, void* out, void* stream);
+/* out[b,o] = sum_k mat[b,o,k] vec[b,k]      kernels/gemv.py:82-149 / cuda/gemv.cu:78-107 */
+int cpmk_gemv_fp16(int32_t batch, int32_t dim_out, int32_t dim_in, const void* mat,
+                   const void* vec, void* out, void* stream);
+/* out[b,o] = sum_k mat[b,k,o] vec[b,k]      kernels/gemv.py:151-216 / cuda/gemv.cu:109-140 */
+int cpmk_gemv_fp16_transpose(int32_t batch, int32_t dim_out, int32_t dim_in, const void* mat,
+                             const void* vec, void* out, void* stream);
+/* out[b,o] = sum_k mat[o,k] vec[b,k]        kernels/gemv.py:218-283 / cuda/gemv.cu:142-175 */
+int cpmk_gemv_broadcast_mat_fp16(int32_t batch, int32_t dim_out, int32_t dim_in, const void* mat,
+                                 const void* vec, void* out, void* stream);
+
 /* ---- callers either side of the path in a decode loop ----------------------------- */
 /* out[b,i,j] = weights[ids[b,j], i];  ids (b, seq) int32, weights (vocab, hidden) fp16,
  * out (b, hidden, seq) fp16                    kernels/embedding.py:14-34 / embedding.cu:6-37 */

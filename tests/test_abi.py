@@ -57,7 +57,8 @@ gemm_round_transpose gemm_scale gemm_int8 gemm_scale_x gemm_scale_y gemv_broadca
 gemv_round mask arith_element_add arith_ln_mul arith_ln_mul_add layernorm_forward layernorm_inplace_forward
 layernorm_step layernorm_step_inplace position_embedding_init position_embedding_forward position_embedding_step
 softmax_forward softmax_inplace_forward softmax_step_inplace embedding_forward embedding_step
-copy_data_to_kv""".split()
+copy_data_to_kv gemm_fp16 gemv_fp16 gemv_fp16_light gemv_fp16_transpose gemv_fp16_transpose_light
+gemv_broadcast_mat_fp16 gemv_broadcast_mat_fp16_light""".split()
 
 
 def test_kernel_layer_keeps_reference_names_and_signatures():

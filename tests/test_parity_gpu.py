@@ -601,6 +601,60 @@ def test_elementwise(gpu, shape):
         assert_bits_equal(to_np(out), oracle.mask(x, msk, value), "mask value=%r" % value)
 
 
+# ---------------------------------------------------------------------------------------------
+# fp16 products next to the path (fp32 accumulation; the bar is the 1e-3 of fp16 outputs)
+# ---------------------------------------------------------------------------------------------
+F16_GEMM_CASES = [  # (batch, n, k, m) in the kernel's convention: out (batch, n, m)
+    (1, 4, 4, 4), (2, 6, 10, 8), (3, 34, 64, 20), (2, 256, 128, 260), (1, 512, 1024, 384), (2, 130, 192, 70)]
+
+
+@pytest.mark.parametrize("case", F16_GEMM_CASES)
+@pytest.mark.parametrize("aT", [False, True])
+@pytest.mark.parametrize("bT", [False, True])
+def test_gemm_fp16(gpu, case, aT, bT):
+    _name("gemm_fp16", case, aT, bT)
+    batch, n, k, m = case
+    rng = np.random.default_rng(n * 7 + k * 3 + m + aT * 2 + bT)
+    for bA, bB in ((batch, batch), (1, batch), (batch, 1)):
+        A = rng.standard_normal((bA, m, k) if aT else (bA, k, m)).astype(np.float16)
+        B = (rng.standard_normal((bB, k, n) if bT else (bB, n, k)) / np.sqrt(k)).astype(np.float16)
+        Ad, Bd = to_gpu(A), to_gpu(B)
+        out = torch.empty((batch, n, m), dtype=torch.half, device=gpu)
+        ck.gemm_fp16(m, k, n, bA, bB, aT, bT, Ad.data_ptr(), Bd.data_ptr(), out.data_ptr(), stream())
+        Aop = A.astype(np.float64) if aT else A.astype(np.float64).transpose(0, 2, 1)      # (bA, m, k)
+        Bop = B.astype(np.float64).transpose(0, 2, 1) if bT else B.astype(np.float64)      # (bB, n, k)
+        ref = np.einsum("bnk,bmk->bnm", np.broadcast_to(Bop, (batch, n, k)), np.broadcast_to(Aop, (batch, m, k)))
+        # one fp16 rounding of an fp32-accumulated sum; atol covers sums that cancel to near zero
+        assert_close_fp16(to_np(out), ref.astype(np.float16), rtol=1e-3, atol=1e-3, what="gemm_fp16 %s" % (case,))
+
+
+@pytest.mark.parametrize("shape", [(4, 64, 256), (3, 33, 100), (2, 1000, 4096), (1, 7, 6)])
+def test_gemv_fp16_family(gpu, shape):
+    _name("gemv fp16", shape)
+    batch, dim_out, dim_in = shape
+    rng = np.random.default_rng(dim_out + dim_in)
+    vec = rng.standard_normal((batch, dim_in)).astype(np.float16)
+    mat = (rng.standard_normal((batch, dim_out, dim_in)) / np.sqrt(dim_in)).astype(np.float16)
+    vd, md = to_gpu(vec), to_gpu(mat)
+    out = torch.empty((batch, dim_out), dtype=torch.half, device=gpu)
+    ref = np.einsum("bok,bk->bo", mat.astype(np.float64), vec.astype(np.float64)).astype(np.float16)
+    for fn in (ck.gemv_fp16, ck.gemv_fp16_light):
+        out.zero_()
+        fn(batch, dim_out, dim_in, md.data_ptr(), vd.data_ptr(), out.data_ptr(), stream())
+        assert_close_fp16(to_np(out), ref, rtol=1e-3, atol=1e-3, what=fn.__name__)
+    mt = to_gpu(np.ascontiguousarray(mat.transpose(0, 2, 1)))                # (batch, dim_in, dim_out)
+    for fn in (ck.gemv_fp16_transpose, ck.gemv_fp16_transpose_light):
+        out.zero_()
+        fn(batch, dim_out, dim_in, mt.data_ptr(), vd.data_ptr(), out.data_ptr(), stream())
+        assert_close_fp16(to_np(out), ref, rtol=1e-3, atol=1e-3, what=fn.__name__)
+    m0 = to_gpu(mat[0])
+    ref0 = np.einsum("ok,bk->bo", mat[0].astype(np.float64), vec.astype(np.float64)).astype(np.float16)
+    for fn in (ck.gemv_broadcast_mat_fp16, ck.gemv_broadcast_mat_fp16_light):
+        out.zero_()
+        fn(batch, dim_out, dim_in, m0.data_ptr(), vd.data_ptr(), out.data_ptr(), stream())
+        assert_close_fp16(to_np(out), ref0, rtol=1e-3, atol=1e-3, what=fn.__name__)
+
+
 @pytest.mark.parametrize("shape", [(2, 64, 128), (3, 100, 77), (1, 4096, 33), (4, 24, 1)])
 def test_embedding_and_kv_copy(gpu, shape):
     """Pure data movement next to the path: gathers from the embedding table and the copy of a

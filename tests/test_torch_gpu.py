@@ -65,12 +65,20 @@ def test_bmm_int8(gpu, case, aT, bT):
         assert err < 0.5 and err <= 2e-2 * max(1.0, np.abs(loose).max()), err
 
 
-def test_bmm_fp16_goes_to_the_vendor_blas(gpu):
-    """int8=False is outside the hand-written path: the wrapper hands it to torch.matmul."""
-    g = torch.Generator().manual_seed(1)
-    A = torch.randn(2, 8, 16, generator=g).half().cuda()
-    B = torch.randn(2, 16, 12, generator=g).half().cuda()
-    assert torch.equal(ct.bmm(A, False, B, False, int8=False), torch.matmul(A, B))
+@pytest.mark.parametrize("aT", [False, True])
+@pytest.mark.parametrize("bT", [False, True])
+def test_bmm_fp16(gpu, aT, bT):
+    """int8=False: fp16 product with fp32 accumulation (tests/test_gemm.py:62-85 of the reference
+    compares with torch.matmul at 5e-2; here 1e-3 against float64)."""
+    _name("bmm fp16", aT, bT)
+    g = torch.Generator().manual_seed(1 + aT * 2 + bT)
+    for (b, M, K, N) in [(2, 8, 16, 12), (3, 130, 256, 64), (1, 512, 512, 260)]:
+        A = torch.randn((b, K, M) if aT else (b, M, K), generator=g).half()
+        B = (torch.randn((b, N, K) if bT else (b, K, N), generator=g) / K ** 0.5).half()
+        out = ct.bmm(A.cuda(), aT, B.cuda(), bT, int8=False)
+        ref = F.real_bmm(A.double(), aT, B.double(), bT, False).half()
+        assert out.shape == (b, M, N)
+        assert_close_fp16(to_np(out), ref.numpy(), rtol=1e-3, atol=1e-3, what="bmm fp16")
 
 
 @pytest.mark.parametrize("shape", [(4, 512, 64), (3, 100, 40), (2, 4096, 128)])
