@@ -197,3 +197,69 @@ def test_ffn_block_composition(gpu):
     got = to_np(out).astype(np.float32)
     err = np.abs(got - ref.numpy())
     assert err.max() < 3e-2 and err.mean() < 3e-3, (err.max(), err.mean())
+
+
+def test_transformer_layer_composition(gpu):
+    """A CPM-2-shaped transformer layer at reduced size through the wrappers only, in the
+    reference's (batch, hidden, seq) layout: LayerNorm -> int8 Q/K/V projections -> fp16 scores
+    (B*H, len_k, len_q) + T5 relative bias -> padding mask (-inf on padded queries) -> softmax
+    over dim 1 -> fp16 PV -> int8 output projection -> residual -> LayerNorm -> int8 FFN with
+    gelu -> residual; against the same chain of fp32 formulations on the CPU.  The tolerance is
+    the int8 quantisation noise of four chained quantised products."""
+    _name("transformer layer")
+    g = torch.Generator().manual_seed(1005)
+    b, d, H, dh, dff, s = 2, 256, 4, 64, 640, 96
+    x = torch.randn(b, d, s, generator=g).half()
+    W = {k: (torch.randn(1, o, i, generator=g) * 0.04).half()
+         for k, (o, i) in {"q": (d, d), "k": (d, d), "v": (d, d), "o": (d, d), "w1": (dff, d), "w2": (d, dff)}.items()}
+    lens = torch.tensor([s, s - 29])
+    pad = (torch.arange(s)[None, :] < lens[:, None])                     # (b, s) True = real token
+    ln1 = ct.LayerNorm(d, bias=True).half().cuda(); ln2 = ct.LayerNorm(d, bias=True).half().cuda()
+    pe = ct.PositionEmbedding(H, 32, 128, True).half().cuda()
+    for mod in (ln1, ln2):
+        mod.weight.copy_((1 + 0.1 * torch.randn(d, generator=g)).half()); mod.bias.copy_((0.1 * torch.randn(d, generator=g)).half())
+    pe.weight.copy_((torch.randn(H, 32, generator=g) * 0.02).half())
+    Wd = {k: v.cuda() for k, v in W.items()}
+    xd, padd = x.cuda(), pad.cuda()
+
+    # ---- device, wrappers only ----
+    h = ln1(xd)
+    q, k, v = (ct.bmm(Wd[n], False, h, False, int8=True).view(b * H, dh, s) for n in "qkv")
+    scores = ct.bmm(k, True, q, False, int8=False)                       # (b*H, s_k, s_q)
+    scores = (scores.float() / dh ** 0.5).half()
+    bias = pe(s, s)                                                      # (H, s_k, s_q)
+    scores = ct.element_add(scores.view(b, H * s * s).contiguous(), bias.reshape(1, -1).expand(b, -1).contiguous())
+    scores = ct.mask(scores.view(b, H * s, s), padd, float("-inf"))      # padded queries -> -inf columns
+    probs = ct.softmax(scores.view(b * H, s, s))                         # all -inf column -> 0
+    ctx = ct.bmm(v, False, probs, False, int8=False).view(b, d, s)       # (b*H, dh, s_q)
+    y = ct.element_add(ct.bmm(Wd["o"], False, ctx, False, int8=True), xd)
+    h2 = ln2(y)
+    f = ct.gelu(ct.bmm(Wd["w1"], False, h2, False, int8=True))
+    out = ct.element_add(ct.bmm(Wd["w2"], False, f, False, int8=True), y)
+
+    # ---- CPU, fp32 formulations ----
+    def qmm(Wm, act):       # Wm (1, N, K) along K; act (b, K, S) quantised per (b, s) column along K
+        # an all-zero column (a padded query after attention) has scale 0: 0/0 in the fp32
+        # formulation, 0 in the kernels (NaN -> 0 in the rounding)
+        aq = torch.nan_to_num(F.fake_quant_rows(act.float().transpose(1, 2)), nan=0.0).transpose(1, 2)
+        return torch.matmul(F.fake_quant_rows(Wm.float()), aq)
+    r = F.layernorm_dim1(x, ln1.weight.cpu(), ln1.bias.cpu(), 1e-5)
+    rq, rk, rv = (qmm(W[n], r).half().view(b * H, dh, s).float() for n in "qkv")
+    sc = (torch.matmul(rk.transpose(1, 2), rq).half().float() / dh ** 0.5).half().float()
+    rb = F.position_bias(pe.weight.cpu(), s, s, True, 32, 128).float()   # (H, s_k, s_q)
+    sc = (sc.view(b, H, s, s) + rb[None]).half().float()
+    sc = sc.masked_fill(~pad[:, None, None, :], float("-inf")).view(b * H, s, s)
+    pr = torch.softmax(sc, dim=1)
+    pr = torch.where(torch.isnan(pr), torch.zeros_like(pr), pr).half().float()    # all -inf column -> 0
+    rc = torch.matmul(rv, pr).half().view(b, d, s).float()
+    ry = (qmm(W["o"], rc).half().float() + x.float()).half()
+    r2 = F.layernorm_dim1(ry, ln2.weight.cpu(), ln2.bias.cpu(), 1e-5)
+    rf = F.gelu_tanh(qmm(W["w1"], r2).half()).float()
+    ref = (qmm(W["w2"], rf).half().float() + ry.float())
+
+    got = to_np(out).astype(np.float32)
+    err = np.abs(got - ref.numpy())
+    assert np.isfinite(got).all()
+    assert err.max() < 6e-2 and err.mean() < 4e-3, (err.max(), err.mean())
+    # padded query positions received exactly zero attention
+    assert float(probs.view(b, H, s, s)[1, :, :, s - 29:].abs().max()) == 0.0
