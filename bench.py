@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the int8 quantized-GEMM inference path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only gemm|gemv|ln|softmax|pipeline|calib]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only gemm|gemv|ln|softmax|other|pipeline|calib]
 
 One "step" is one pass of the path over the north-star workload: activations A fp16
 [1,4096,4096] ~N(0,1) and weights W fp16 [1,10240,4096] ~N(0,0.02) (seed 1000, generated on
@@ -11,7 +11,8 @@ fp16 dequantisation -- exactly what the reference's GEMMInt8.forward does per ca
 
 Prints ONE JSON line.  `value` is 2*M*N*K / step time in TOP/s for that whole step; the
 `roofline` object is the GEMM kernel alone against the dense int8 MFMA peak; `components`
-carries the decode GEMV, layernorm and softmax kernels against the HBM peak; `cpu_baseline`
+carries the decode GEMV, layernorm and softmax kernels (and, after them, every other kernel of
+the path) against the HBM peak; `cpu_baseline`
 is the torch formulation of the same step timed on the host cores (a reported baseline).
 """
 import argparse
@@ -46,7 +47,7 @@ def parse():
     p.add_argument("--steps", type=int, default=50)
     p.add_argument("--warmup", type=int, default=10)
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    p.add_argument("--only", default="", help="run only one kernel loop (for profiling): gemm|gemv|ln|softmax|pipeline|calib "
+    p.add_argument("--only", default="", help="run only one kernel loop (for profiling): gemm|gemv|ln|softmax|other|pipeline|calib "
                         "(calib = a plain 256 MiB device copy, the known-size kernel that scales the HBM counters)")
     p.add_argument("--reps", type=int, default=200, help="launches per timed batch in the per-kernel loops")
     return p.parse_args()
@@ -240,6 +241,89 @@ def main():
         ms, how = graph_ms(launches, max(3, reps // 20))
         hbm("softmax_forward", 4 * 512 * 1024 * 1024, ms, how, "[512,1024,1024] fp16 causal, dim 1", TRAFFIC_BYTES["softmax"])
         del sd, so
+
+    if only in ("", "other"):
+        # the other kernels of the path, each at the size its config gives it
+        gg = torch.Generator().manual_seed(1004)
+
+        def rot(shape, count, scale=1.0, dtype=torch.half):
+            return [(torch.randn(*shape, generator=gg) * scale).to(dtype).to(dev) for _ in range(count)]
+        Ws = rot((1, N, K), 3, 0.02)                              # 3 x 84 MB
+        sW = torch.empty((1, N), dtype=torch.half, device=dev); qW = torch.empty((1, N, K), dtype=torch.int8, device=dev)
+        ms, how = graph_ms([(lambda w=w: ck.gemm_quantize(1, N, K, w.data_ptr(), sW.data_ptr(), qW.data_ptr(), False, st())) for w in Ws], max(3, reps // 12))
+        hbm("gemm_quantize (calc_scale+round) W", 3 * N * K + 2 * N, ms, how, "[10240,4096] fp16 -> int8 + row scales", None)
+        ms, how = graph_ms([(lambda w=w: ck.gemm_calc_scale(1, N, K, w.data_ptr(), sW.data_ptr(), st())) for w in Ws], max(3, reps // 12))
+        hbm("gemm_calc_scale W", 2 * N * K + 2 * N, ms, how, "[10240,4096] fp16", None)
+        ms, how = graph_ms([(lambda w=w: ck.gemm_round(1, N, K, w.data_ptr(), sW.data_ptr(), qW.data_ptr(), st())) for w in Ws], max(3, reps // 12))
+        hbm("gemm_round W", 3 * N * K + 2 * N, ms, how, "[10240,4096] fp16 -> int8", None)
+        del Ws, qW
+        accs = [torch.randint(-3000000, 3000000, (1, M, N), generator=gg, dtype=torch.int32).to(dev) for _ in range(2)]
+        sA = (torch.rand(M, generator=gg) * 0.03).half().to(dev); sN = (torch.rand(N, generator=gg) * 0.001).half().to(dev)
+        o16 = torch.empty((1, M, N), dtype=torch.half, device=dev)
+        ms, how = graph_ms([(lambda a_=a_: ck.gemm_scale(1, M, N, a_.data_ptr(), sA.data_ptr(), sN.data_ptr(), o16.data_ptr(), True, True, st())) for a_ in accs], max(3, reps // 8))
+        hbm("gemm_scale", 6 * M * N + 2 * (M + N), ms, how, "[4096,10240] int32 -> fp16", None)
+        del accs, o16
+        xs = rot((8, 4096, 512), 10)                              # C3 / C4 activations, 10 x 33.5 MB
+        y = torch.empty_like(xs[0])
+        al = (1 + 0.1 * torch.randn(4096, generator=gg)).half().to(dev); be = (0.1 * torch.randn(4096, generator=gg)).half().to(dev)
+        ms, how = graph_ms([(lambda x_=x_: ck.layernorm_affine_forward(8, 4096, 512, x_.data_ptr(), al.data_ptr(), be.data_ptr(), y.data_ptr(), 1e-5, True, st())) for x_ in xs], max(5, reps // 10))
+        hbm("layernorm + gamma/beta (fused)", 4 * 8 * 4096 * 512, ms, how, "[8,4096,512] fp16", None)
+        ms, how = graph_ms([(lambda x_=x_: ck.arith_ln_mul_add(8, 4096, 512, x_.data_ptr(), al.data_ptr(), be.data_ptr(), y.data_ptr(), st())) for x_ in xs], max(5, reps // 10))
+        hbm("arith_ln_mul_add", 4 * 8 * 4096 * 512, ms, how, "[8,4096,512] fp16", None)
+        ms, how = graph_ms([(lambda i=i: ck.arith_element_add(8, 4096 * 512, xs[i].data_ptr(), xs[(i + 1) % 10].data_ptr(), y.data_ptr(), st())) for i in range(10)], max(5, reps // 10))
+        hbm("arith_element_add", 6 * 8 * 4096 * 512, ms, how, "[8, 4096*512] fp16", None)
+        mk = (torch.rand(8, 512, generator=gg) > 0.3).to(dev)
+        ms, how = graph_ms([(lambda x_=x_: ck.mask(8, 4096, 512, x_.data_ptr(), mk.data_ptr(), float("-inf"), y.data_ptr(), st())) for x_ in xs], max(5, reps // 10))
+        hbm("mask", 4 * 8 * 4096 * 512 + 8 * 512, ms, how, "[8,4096,512] fp16", None)
+        sX = torch.empty((8, 512), dtype=torch.half, device=dev); qX = torch.empty((8, 512, 4096), dtype=torch.int8, device=dev)
+        ms, how = graph_ms([(lambda x_=x_: ck.gemm_quantize_cols(8, 4096, 512, x_.data_ptr(), sX.data_ptr(), qX.data_ptr(), True, st())) for x_ in xs], max(5, reps // 10))
+        hbm("gemm_quantize_cols (transposed int8 out)", 3 * 8 * 4096 * 512 + 2 * 8 * 512, ms, how, "[8,4096,512] fp16, per-column scales", None)
+        del xs, y, qX
+        gs = rot((8, 10240 * 512), 3)                             # C4 gelu input, 3 x 84 MB
+        go = torch.empty_like(gs[0])
+        ms, how = graph_ms([(lambda x_=x_: ck.gelu_forward(8, 10240 * 512, x_.data_ptr(), go.data_ptr(), st())) for x_ in gs], max(3, reps // 12))
+        hbm("gelu_forward", 4 * 8 * 10240 * 512, ms, how, "[8, 10240*512] fp16", None)
+        del gs, go
+        tbl = torch.empty(128, dtype=torch.int32, device=dev)
+        ck.position_embedding_init(32, 128, tbl.data_ptr(), True, st())
+        pw = (torch.randn(64, 32, generator=gg) * 0.02).half().to(dev)
+        pos = [torch.empty((64, 1024, 1024), dtype=torch.half, device=dev) for _ in range(3)]
+        ms, how = graph_ms([(lambda o_=o_: ck.position_embedding_forward(1024, 1024, 32, 128, 64, tbl.data_ptr(), pw.data_ptr(), o_.data_ptr(), True, st())) for o_ in pos], max(3, reps // 12))
+        hbm("position_embedding_forward", 2 * 64 * 1024 * 1024 + 2 * 64 * 32 + 4 * 128, ms, how, "64 heads x 1024 x 1024 fp16 written", None)
+        del pos
+        # config 4 up-projection in the reference's native layout: bmm(W1[1,10240,4096], x[8,4096,512], int8)
+        W1 = (torch.randn(1, 10240, 4096, generator=gg) * 0.02).half().to(dev)
+        xa = torch.randn(8, 4096, 512, generator=gg).half().to(dev)
+        ms = event_ms(lambda: ct.bmm(W1, False, xa, False, int8=True), 20)
+        components["ffn up-projection bmm(int8), native layout"] = {
+            "shape": "W1 [1,10240,4096] x act [8,4096,512]", "bound": "mfma", "avg_us": round(ms * 1e3, 2),
+            "achieved": round(2.0 * 10240 * 4096 * 4096 / (ms * 1e-3) / 1e12, 1), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
+            "frac": round(2.0 * 10240 * 4096 * 4096 / (ms * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4), "timing": "events, whole bmm"}
+        del W1, xa
+
+    # per-op CPU timings beside the three headline components (torch formulations, host cores)
+    if not args.no_cpu and only == "":
+        from oracle import formulations as F
+        torch.set_num_threads(os.cpu_count() or 1)
+
+        def cpu_us(fn, n=3):
+            fn()
+            ts = []
+            for _ in range(n):
+                t0 = time.perf_counter(); fn(); ts.append(time.perf_counter() - t0)
+            return round(sorted(ts)[len(ts) // 2] * 1e6, 1)
+        gg = torch.Generator().manual_seed(7)
+        Wq = torch.randint(-127, 128, (10240, 4096), generator=gg).float(); vq = torch.randint(-127, 128, (32, 4096), generator=gg).float()
+        if "gemv_broadcast_mat_int8" in components:
+            components["gemv_broadcast_mat_int8"]["cpu_us"] = cpu_us(lambda: torch.matmul(vq, Wq.t()))
+        xl = torch.randn(8, 4096, 512, generator=gg).half(); wl = torch.ones(4096); bl = torch.zeros(4096)
+        if "layernorm_forward" in components:
+            components["layernorm_forward"]["cpu_us"] = cpu_us(lambda: F.layernorm_dim1(xl, wl, bl, 1e-5))
+        xsm = (torch.randn(16, 1024, 1024, generator=gg) * 4).half()
+        if "softmax_forward" in components:
+            components["softmax_forward"]["cpu_us"] = round(cpu_us(lambda: F.softmax_dim1(xsm)) * 32, 1)
+            components["softmax_forward"]["cpu_sample"] = "1/32 of the tensor timed, scaled"
+        del Wq, vq, xl, xsm
 
     # ---- CPU baseline: torch formulation of the same step on the host cores ------------------
     cpu = None
