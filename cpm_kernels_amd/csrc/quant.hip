@@ -196,17 +196,27 @@ __global__ __launch_bounds__(256) void k_dequant(int64_t total, int32_t n, int32
 // row count allows.  Many resident waves, each with one row in flight, hide the memory latency
 // better here than fewer waves that prefetch their next row (measured).
 // ---------------------------------------------------------------------------------------
+// One or two tensors with rows of the same length per launch (the two operands of a product):
+// virtual row r < rows0 is row r of the first, otherwise row r - rows0 of the second.
+struct RowsArgs {
+    const half_t* mat0; half_t* scale0; int8_t* out0; int64_t rows0;
+    const half_t* mat1; half_t* scale1; int8_t* out1; int64_t rows1;
+    int32_t m;
+};
+
 template <int NV, bool QUANT>
-__global__ __launch_bounds__(256) void k_rows(int64_t rows, int32_t m, const half_t* __restrict__ mat,
-                                              half_t* __restrict__ scale, int8_t* __restrict__ out) {
+__global__ __launch_bounds__(256) void k_rows(RowsArgs a) {
     const int lane = threadIdx.x & 63;
     const int64_t nw = (int64_t)gridDim.x * 4;
+    const int64_t rows = a.rows0 + a.rows1;
+    const int32_t m = a.m;
     int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= rows) return;
     const int m8 = m >> 3;
     half8_t cur[NV];
     auto load = [&](half8_t (&v)[NV], int64_t r) __attribute__((always_inline)) {
-        const half8_t* p8 = reinterpret_cast<const half8_t*>(mat + r * m);
+        const half_t* mat = r < a.rows0 ? a.mat0 + r * m : a.mat1 + (r - a.rows0) * m;
+        const half8_t* p8 = reinterpret_cast<const half8_t*>(mat);
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int j = lane + i * 64;
@@ -229,10 +239,12 @@ __global__ __launch_bounds__(256) void k_rows(int64_t rows, int32_t m, const hal
         for (int e = 0; e < 8; ++e) mx = fmaxf((float)hm[e], mx);
         mx = wave_max(mx);
         const half_t sh = scale_from_absmax(mx);
-        if (lane == 0) scale[row] = sh;
+        const bool second = row >= a.rows0;
+        const int64_t lrow = second ? row - a.rows0 : row;
+        if (lane == 0) (second ? a.scale1 : a.scale0)[lrow] = sh;
         if (QUANT) {
             const float s = (float)sh, y = 1.0f / s;
-            uint2_t* o8 = reinterpret_cast<uint2_t*>(out + row * m);
+            uint2_t* o8 = reinterpret_cast<uint2_t*>((second ? a.out1 : a.out0) + lrow * m);
 #pragma unroll
             for (int i = 0; i < NV; ++i) {
                 const int j = lane + i * 64;
@@ -273,6 +285,16 @@ static unsigned rows_grid(int64_t rows, int cus, int nv) {
     return (unsigned)best;
 }
 
+template <bool QUANT>
+static void launch_rows(const RowsArgs& ra, int nv, hipStream_t st) {
+    const dim3 g(rows_grid(ra.rows0 + ra.rows1, compute_units(), nv));
+    if (nv <= 1) hipLaunchKernelGGL((k_rows<1, QUANT>), g, dim3(256), 0, st, ra);
+    else if (nv <= 2) hipLaunchKernelGGL((k_rows<2, QUANT>), g, dim3(256), 0, st, ra);
+    else if (nv <= 4) hipLaunchKernelGGL((k_rows<4, QUANT>), g, dim3(256), 0, st, ra);
+    else if (nv <= 8) hipLaunchKernelGGL((k_rows<8, QUANT>), g, dim3(256), 0, st, ra);
+    else hipLaunchKernelGGL((k_rows<16, QUANT>), g, dim3(256), 0, st, ra);
+}
+
 static int check3(int32_t batch, int32_t n, int32_t m) {
     if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
     return 0;
@@ -291,12 +313,8 @@ static int row_absmax(int64_t rows, int32_t m, const void* mat, void* out, hipSt
     } else {
         const int nv = (int)ceil_div(m, 512);
         if (vec && nv <= 16) {
-            const unsigned g = rows_grid(rows, compute_units(), nv);
-            if (nv <= 1) hipLaunchKernelGGL((k_rows<1, false>), dim3(g), dim3(256), 0, st, rows, m, p, o, (int8_t*)nullptr);
-            else if (nv <= 2) hipLaunchKernelGGL((k_rows<2, false>), dim3(g), dim3(256), 0, st, rows, m, p, o, (int8_t*)nullptr);
-            else if (nv <= 4) hipLaunchKernelGGL((k_rows<4, false>), dim3(g), dim3(256), 0, st, rows, m, p, o, (int8_t*)nullptr);
-            else if (nv <= 8) hipLaunchKernelGGL((k_rows<8, false>), dim3(g), dim3(256), 0, st, rows, m, p, o, (int8_t*)nullptr);
-            else hipLaunchKernelGGL((k_rows<16, false>), dim3(g), dim3(256), 0, st, rows, m, p, o, (int8_t*)nullptr);
+            const RowsArgs ra = {p, o, nullptr, rows, nullptr, nullptr, nullptr, 0, m};
+            launch_rows<false>(ra, nv, st);
             return launch_status();
         }
         const unsigned g = (unsigned)ceil_div(rows, 4);
@@ -426,22 +444,33 @@ int cpmk_gemm_quantize(int32_t batch, int32_t n, int32_t m, const void* mat, voi
         if (rows == 0) return 0;
         const bool vec = (m % 8 == 0) && aligned16(mat) && ((reinterpret_cast<uintptr_t>(out) & 7u) == 0);
         if (vec && m <= 64 * 8 * 16) {
-            const int nv = (int)ceil_div(m, 512);
-            const unsigned g = rows_grid(rows, compute_units(), nv);
-            const half_t* p = (const half_t*)mat;
-            half_t* s = (half_t*)scale;
-            int8_t* o = (int8_t*)out;
-            if (nv <= 1) hipLaunchKernelGGL((k_rows<1, true>), dim3(g), dim3(256), 0, st, rows, m, p, s, o);
-            else if (nv <= 2) hipLaunchKernelGGL((k_rows<2, true>), dim3(g), dim3(256), 0, st, rows, m, p, s, o);
-            else if (nv <= 4) hipLaunchKernelGGL((k_rows<4, true>), dim3(g), dim3(256), 0, st, rows, m, p, s, o);
-            else if (nv <= 8) hipLaunchKernelGGL((k_rows<8, true>), dim3(g), dim3(256), 0, st, rows, m, p, s, o);
-            else hipLaunchKernelGGL((k_rows<16, true>), dim3(g), dim3(256), 0, st, rows, m, p, s, o);
+            const RowsArgs ra = {(const half_t*)mat, (half_t*)scale, (int8_t*)out, rows, nullptr, nullptr, nullptr, 0, m};
+            launch_rows<true>(ra, (int)ceil_div(m, 512), st);
             return launch_status();
         }
         if (int e = cpmk_gemm_calc_scale(batch, n, m, mat, scale, stream)) return e;
         return cpmk_gemm_round(batch, n, m, mat, scale, out, stream);
     }
     return cpmk_gemm_quantize_cols(batch, n, m, mat, scale, out, 0, stream);
+}
+
+int cpmk_gemm_quantize_pair(int64_t rows0, const void* mat0, void* scale0, void* out0, int64_t rows1, const void* mat1,
+                            void* scale1, void* out1, int32_t m, void* stream) {
+    clear_stale_error();
+    if (rows0 < 0 || rows1 < 0 || m < 0 || rows0 > 0x7fffffff || rows1 > 0x7fffffff) return CPMK_EBADARG;
+    if (m == 0 || rows0 + rows1 == 0) return 0;
+    const bool vec = (m % 8 == 0) && m <= 64 * 8 * 16 && (rows0 == 0 || (aligned16(mat0) && (reinterpret_cast<uintptr_t>(out0) & 7u) == 0)) &&
+                     (rows1 == 0 || (aligned16(mat1) && (reinterpret_cast<uintptr_t>(out1) & 7u) == 0));
+    if (vec) {
+        const RowsArgs ra = {(const half_t*)mat0, (half_t*)scale0, (int8_t*)out0, rows0,
+                             (const half_t*)mat1, (half_t*)scale1, (int8_t*)out1, rows1, m};
+        launch_rows<true>(ra, (int)ceil_div(m, 512), (hipStream_t)stream);
+        return launch_status();
+    }
+    if (rows0 > 0)
+        if (int e = cpmk_gemm_quantize(1, (int32_t)rows0, m, mat0, scale0, out0, 0, stream)) return e;
+    if (rows1 > 0) return cpmk_gemm_quantize(1, (int32_t)rows1, m, mat1, scale1, out1, 0, stream);
+    return 0;
 }
 
 }  // extern "C"

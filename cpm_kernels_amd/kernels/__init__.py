@@ -1,11 +1,11 @@
 """Same export list as cpm_kernels/kernels/__init__.py:1-14 of the reference, plus the three
-fused launchers this build adds (gemm_int8_scale, gemm_quantize, gemm_quantize_cols,
+fused launchers this build adds (gemm_int8_scale, gemm_quantize, gemm_quantize_cols, gemm_quantize_pair,
 layernorm_affine_forward)."""
 from .embedding import embedding_forward, embedding_backward_stage1, embedding_backward_stage2, embedding_step
 from .gelu import gelu_forward, gelu_backward, gelu_inplace_forward
 from .gemm import gemm_calc_scale, gemm_calc_scale_transpose, gemm_round, gemm_round_transpose, gemm_scale, \
     gemm_fp16, gemm_int8, gemm_backward_round_scale, gemm_backward_scale_round, gemm_scale_x, gemm_scale_y, \
-    gemm_int8_scale, gemm_quantize, gemm_quantize_cols
+    gemm_int8_scale, gemm_quantize, gemm_quantize_cols, gemm_quantize_pair
 from .gemv import gemv_fp16, gemv_broadcast_mat_int8, gemv_fp16_transpose, gemv_broadcast_mat_fp16, \
     gemv_calc_scale, gemv_round, gemv_broadcast_mat_fp16_light, gemv_fp16_light, gemv_fp16_transpose_light
 from .mask import mask

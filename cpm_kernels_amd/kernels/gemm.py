@@ -91,6 +91,14 @@ def gemm_quantize(batch: int, n: int, m: int,
     cpmk.gemm_quantize(batch, n, m, mat, scale, out, int(bool(transpose)), _stream(stream))
 
 
+def gemm_quantize_pair(rows0: int, mat0: DevicePointer, scale0: DevicePointer, out0: DevicePointer,
+                       rows1: int, mat1: DevicePointer, scale1: DevicePointer, out1: DevicePointer,
+                       m: int, stream: CUDAStream):
+    """gemm_quantize(transpose=False) of two tensors with rows of length m (rows0 x m fp16 at
+    mat0, rows1 x m at mat1) in one launch."""
+    cpmk.gemm_quantize_pair(rows0, mat0, scale0, out0, rows1, mat1, scale1, out1, m, _stream(stream))
+
+
 def gemm_quantize_cols(batch: int, n: int, m: int,
                        mat: DevicePointer,      # (b, n, m) fp16
                        scale: DevicePointer,    # (b, m) fp16

@@ -8,7 +8,7 @@ the six-launch sequence, which ``fused=False`` still runs through the kernel-lev
 """
 import torch
 from ..kernels import gemm_calc_scale, gemm_calc_scale_transpose, gemm_round, gemm_round_transpose, \
-    gemm_scale, gemm_int8, gemm_int8_scale, gemm_quantize, gemm_quantize_cols, gemm_fp16
+    gemm_scale, gemm_int8, gemm_int8_scale, gemm_quantize, gemm_quantize_cols, gemm_quantize_pair, gemm_fp16
 from ._common import cur_stream, InferenceOnly
 
 
@@ -97,8 +97,18 @@ class GEMMInt8(InferenceOnly):
         if fused:
             # both operands are brought to K-major int8 while they are quantised, so every
             # layout runs on the fast GEMM kernel: A (bA, M, K) and B (bB, N, K)
-            scale_A, quantized_A = quantize_k_major(A, aT)
-            scale_B, quantized_B = quantize_k_major(B, not bT)
+            if not aT and bT and A.size(2) == B.size(2):
+                # both already K-major: one launch quantises the two of them
+                scale_A = torch.empty(A.shape[:2], dtype=torch.half, device=A.device)
+                scale_B = torch.empty(B.shape[:2], dtype=torch.half, device=A.device)
+                quantized_A = torch.empty(A.shape, dtype=torch.int8, device=A.device)
+                quantized_B = torch.empty(B.shape, dtype=torch.int8, device=A.device)
+                gemm_quantize_pair(A.size(0) * A.size(1), A.data_ptr(), scale_A.data_ptr(), quantized_A.data_ptr(),
+                                   B.size(0) * B.size(1), B.data_ptr(), scale_B.data_ptr(), quantized_B.data_ptr(),
+                                   A.size(2), cur_stream())
+            else:
+                scale_A, quantized_A = quantize_k_major(A, aT)
+                scale_B, quantized_B = quantize_k_major(B, not bT)
             return gemm_and_scale(quantized_A, scale_A, quantized_B, scale_B, False, True, True)
         else:
             scale_A = calc_scale(A, aT)

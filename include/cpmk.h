@@ -111,6 +111,14 @@ int cpmk_gemm_int8_scale(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
 int cpmk_gemm_quantize(int32_t batch, int32_t n, int32_t m, const void* mat,
                        void* scale, void* out, int transpose, void* stream);
 
+/* cpmk_gemm_quantize(transpose = 0) of two tensors with rows of the same length m in one
+ * launch: rows0 x m at mat0 and rows1 x m at mat1 (batch and row dimensions flattened), each
+ * with its own scale and int8 output.  What torch-level bmm needs for its two operands; no
+ * counterpart in the reference. */
+int cpmk_gemm_quantize_pair(int64_t rows0, const void* mat0, void* scale0, void* out0,
+                            int64_t rows1, const void* mat1, void* scale1, void* out1,
+                            int32_t m, void* stream);
+
 /* Per-column scales (b,m) and rounding in one pass, as cpmk_gemm_quantize with transpose = 1
  * (cpm_kernels/torch/gemm.py:98-102 for an operand given as (b, K, N)), with the int8 result
  * written in place (b,n,m) when out_transposed = 0 or transposed (b,m,n) when 1.  The transposed

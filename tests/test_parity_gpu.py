@@ -105,6 +105,24 @@ def test_calc_scale_and_round_transpose(gpu, shape):
         assert_bits_equal(to_np(q3), np.ascontiguousarray(want), "gemm_quantize_cols int8 (transposed=%s)" % tr)
 
 
+@pytest.mark.parametrize("rows0,rows1,m", [(512, 4096, 4096), (3, 0, 1000), (0, 7, 24), (5, 9, 30), (33, 17, 8200)])
+def test_quantize_pair(gpu, rows0, rows1, m):
+    """Two tensors with rows of one length quantised by one launch == each by itself."""
+    _name("quantize_pair", rows0, rows1, m)
+    rng = np.random.default_rng(rows0 * 31 + rows1 * 7 + m)
+    xs = [adversarial_rows(rng, r, m) if r else np.zeros((0, m), np.float16) for r in (rows0, rows1)]
+    d = [to_gpu(x) for x in xs]
+    sc = [torch.empty((r,), dtype=torch.half, device=gpu) for r in (rows0, rows1)]
+    q = [torch.empty((r, m), dtype=torch.int8, device=gpu) for r in (rows0, rows1)]
+    ck.gemm_quantize_pair(rows0, d[0].data_ptr(), sc[0].data_ptr(), q[0].data_ptr(),
+                          rows1, d[1].data_ptr(), sc[1].data_ptr(), q[1].data_ptr(), m, stream())
+    for i, r in enumerate((rows0, rows1)):
+        if r:
+            s_ref = oracle.gemm_calc_scale(xs[i][None])
+            assert_bits_equal(to_np(sc[i]), s_ref[0], "pair scale %d" % i)
+            assert_bits_equal(to_np(q[i]), oracle.gemm_round(xs[i][None], s_ref)[0], "pair int8 %d" % i)
+
+
 def test_round_unaligned_views(gpu):
     """Pointers that are only 2-byte aligned take the scalar kernels."""
     _name("round unaligned")
