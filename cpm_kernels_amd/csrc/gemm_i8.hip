@@ -657,8 +657,12 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
     if (fast && (k % 128 == 0) && (int64_t)n * k < (1ll << 32) && (int64_t)m * k < (1ll << 32)) {
         // 256x256 tiles when they give most compute units a tile, else 128x128
         const int64_t big = ceil_div(n, 256) * ceil_div(m, 256) * batch;
-        if (big * 4 >= compute_units() * 3) return launch_dma<CPMK_GEMM_BIG, FUSED ? kEpiDequant : kEpiInt32>(a, batch, st);
-        return launch_dma<2, 2, 2, 2, 128, FUSED ? kEpiDequant : kEpiInt32>(a, batch, st);
+        constexpr int EPI = FUSED ? kEpiDequant : kEpiInt32;
+        if (big * 4 >= compute_units() * 3) return launch_dma<CPMK_GEMM_BIG, EPI>(a, batch, st);
+        // 128x128 tiles, or 128x64 when even those leave a quarter of the compute units idle
+        const int64_t mid = ceil_div(n, 128) * ceil_div(m, 128) * batch;
+        if (mid * 4 >= compute_units() * 3) return launch_dma<2, 2, 2, 2, 128, EPI>(a, batch, st);
+        return launch_dma<2, 2, 2, 1, 128, EPI>(a, batch, st);
     }
     if (fast) {
         const int64_t t256 = ceil_div(n, 256) * ceil_div(m, 128) * batch;
