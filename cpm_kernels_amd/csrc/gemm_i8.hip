@@ -576,12 +576,14 @@ static int launch_kmajor(GemmArgs& a, int batch, hipStream_t st) {
     a.tiles_r = (int32_t)ceil_div(a.n, BR);
     a.tiles_c = (int32_t)ceil_div(a.m, BC);
     auto kern = k_gemm_kmajor<WAVES_R, WAVES_C, TR, TC, FUSED>;
-    static bool attr_set = false;   // raising the dynamic LDS limit is idempotent
-    if (!attr_set && smem > 48 * 1024) {
+    static bool attr_set[64] = {false};   // per device; raising the dynamic LDS limit is idempotent
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    if (smem > 48 * 1024 && dev >= 0 && dev < 64 && !attr_set[dev]) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, smem);
         if (e != hipSuccess) return (int)e;
-        attr_set = true;
+        attr_set[dev] = true;
     }
     dim3 grid((unsigned)(a.tiles_r * a.tiles_c), 1, (unsigned)batch);
     hipLaunchKernelGGL(kern, grid, dim3(WAVES_R * WAVES_C * 64), smem, st, a);
