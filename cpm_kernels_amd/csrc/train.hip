@@ -1,0 +1,466 @@
+// Training-side and remaining elementwise kernels of the reference, forward results and
+// gradients (cuda/arith.cu, cuda/gelu.cu:18-45, cuda/gemm.cu:100-172, cuda/layernorm.cu:142-339,
+// cuda/softmax.cu:86-114, cuda/position_bucket.cu:56-103, cuda/embedding.cu:38-88).  None of
+// them is on the inference hot path; they are written for coalesced 16-byte access and fp32
+// accumulation but not tuned further.
+#include "common.h"
+
+namespace cpmk {
+
+// ---------------------------------------------------------------------------------------
+// fp16 elementwise family.  BC selects what the second/third operand is indexed by:
+//   0 same element, 1 column (idx % n) -- the "batch_*" ops, 2 channel ((idx / m) % n) -- "ln_*".
+// The arithmetic is the reference's: one fp16 rounding per __hadd2/__hmul2/__hfma2.
+// ---------------------------------------------------------------------------------------
+enum : int { kAdd = 0, kMul = 1, kFma = 2, kDiv = 3, kSubDiv = 4 };
+
+__device__ inline half_t ew_apply(int op, half_t x, half_t a, half_t b) {
+    switch (op) {
+        case kAdd: return (half_t)(x + a);
+        case kMul: return (half_t)(x * a);
+        case kFma: return __builtin_fmaf16(x, a, b);
+        case kDiv: return (half_t)(x * (half_t)(1.0f / (float)a));     // __hmul2(x, __hdiv(1, alpha)); fp32 quotient -> fp16 rounds once
+        default: {                                                                   // cu_arith_ln_sub_div
+            const float ra = (float)(1.0 / (double)(float)a);
+            const float nb = -(float)b * ra;
+            return __builtin_fmaf16(x, (half_t)ra, round_f16(nb));
+        }
+    }
+}
+
+template <int OP, int BC>
+__global__ __launch_bounds__(256) void k_ew(int64_t total, int64_t n, int64_t m, const half_t* x, const half_t* __restrict__ a,
+                                            const half_t* __restrict__ b, half_t* out) {
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 2;      // element counts are even (reference asserts)
+    if (i >= total) return;
+    half2_t v = *reinterpret_cast<const half2_t*>(x + i);
+    half2_t r;
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+        const int64_t idx = i + e;
+        const int64_t k = BC == 0 ? idx : (BC == 1 ? idx % n : (idx / m) % n);
+        r[e] = ew_apply(OP, v[e], a[k], b ? b[k] : (half_t)0.0f);
+    }
+    *reinterpret_cast<half2_t*>(out + i) = r;
+}
+
+__global__ __launch_bounds__(256) void k_global_scale(int64_t n, const half_t* inp, float scale, half_t* out) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) out[i] = round_f16((float)inp[i] * scale);
+}
+
+// cu_gelu_backward: grad = gelu'(x) * grad_out with the reference's constants and cut-off at |x| >= 5.
+__global__ __launch_bounds__(256) void k_gelu_backward(int64_t total, const half_t* grad_out, const half_t* mat, half_t* grad) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const float v = (float)grad_out[i], x = (float)mat[i];
+    float g;
+    if (-5.0f < x && x < 5.0f) {
+        const float x3 = x * x * x;
+        const float u = 0.797885f * x + 0.0356774f * x3;
+        float sech = 1.0f / coshf(u);
+        sech *= sech;
+        g = 0.5f + (0.398942f * x + 0.0535161f * x3) * sech + 0.5f * tanhf(u);
+    } else {
+        g = x < 0.0f ? 0.0f : 1.0f;
+    }
+    grad[i] = round_f16(g * v);
+}
+
+// ---------------------------------------------------------------------------------------
+// Sums over everything but one index (fp32 accumulation, one workgroup per output).
+// ---------------------------------------------------------------------------------------
+// grad[j] = sum_b grad_out[b, j]                                            cu_arith_batch_add_backward
+__global__ __launch_bounds__(256) void k_batch_add_backward(int64_t batch, int64_t n, const half_t* __restrict__ grad_out,
+                                                            half_t* __restrict__ grad) {
+    // 64 columns per workgroup, 4 row groups
+    __shared__ float red[4][64];
+    const int c = threadIdx.x & 63, rg = threadIdx.x >> 6;
+    const int64_t col = (int64_t)blockIdx.x * 64 + c;
+    float s = 0.0f;
+    if (col < n)
+        for (int64_t i = rg; i < batch; i += 4) s += (float)grad_out[i * n + col];
+    red[rg][c] = s;
+    __syncthreads();
+    if (rg == 0 && col < n) grad[col] = round_f16(red[0][c] + red[1][c] + red[2][c] + red[3][c]);
+}
+
+// grad[i] = sum_{b, j} (WITH_X ? x[b,i,j] : 1) * grad_out[b,i,j]            cu_arith_ln_mul_backward / _ln_add_backward
+template <bool WITH_X>
+__global__ __launch_bounds__(256) void k_ln_backward(int64_t batch, int64_t n, int64_t m, const half_t* __restrict__ x,
+                                                     const half_t* __restrict__ grad_out, half_t* __restrict__ grad) {
+    __shared__ float red[4];
+    const int64_t ch = blockIdx.x;
+    float s = 0.0f;
+    for (int64_t b = 0; b < batch; ++b) {
+        const int64_t base = (b * n + ch) * m;
+        for (int64_t j = threadIdx.x; j < m; j += 256)
+            s += WITH_X ? (float)x[base + j] * (float)grad_out[base + j] : (float)grad_out[base + j];
+    }
+    s = block_sum<4>(s, red);
+    if (threadIdx.x == 0) grad[ch] = (half_t)s;
+}
+
+// ---------------------------------------------------------------------------------------
+// Reductions over dim 1 of (batch, n, m) followed by an elementwise pass.  Workgroup = 64
+// columns x 4 row groups; gridDim = (ceil(m/64), batch).
+// ---------------------------------------------------------------------------------------
+enum : int { kLnFwdV = 0, kLnFwdMV = 1, kLnBwdV = 2, kLnBwdMV = 3, kSoftmaxBwd = 4, kScaleRound = 5 };
+
+struct ColArgs {
+    int32_t n, m;
+    const half_t* a;       // mat / out (softmax)
+    const half_t* g;       // grad_in (backward kinds)
+    const half_t* mean;    // (batch, m)
+    const half_t* var;     // (batch, m)  (reciprocal standard deviation, as the forward kernels write it)
+    const half_t* sx;      // row scales for kScaleRound
+    half_t* out;           // elementwise result (fp16 kinds)
+    int8_t* out_i8;        // kScaleRound
+    half_t* out_mean;
+    half_t* out_var;       // also scale_y for kScaleRound
+    float eps;
+    int bc;                // kScaleRound: row scales shared by the batch
+};
+
+template <int KIND>
+__global__ __launch_bounds__(256) void k_col(ColArgs p) {
+    __shared__ float red[2][4][64];
+    __shared__ float tot[2][64];
+    const int c = threadIdx.x & 63, rg = threadIdx.x >> 6;      // 64 columns x 4 row groups
+    const int32_t col = blockIdx.x * 64 + c;
+    const int64_t b = blockIdx.y;
+    const int64_t boff = b * p.n * p.m;
+    const bool live = col < p.m;
+    float mean = 0.0f, var = 0.0f;
+    if (live && (KIND == kLnBwdV || KIND == kLnBwdMV)) var = (float)p.var[b * p.m + col];
+    if (live && KIND == kLnBwdMV) mean = (float)p.mean[b * p.m + col];
+    const float c3 = -0.5f * var * var * var;
+    float s0 = 0.0f, s1 = 0.0f;
+    if (live) {
+        for (int32_t i = rg; i < p.n; i += 4) {
+            const int64_t o = boff + (int64_t)i * p.m + col;
+            const float x = (float)p.a[o];
+            if (KIND == kLnFwdV) s1 += x * x;
+            else if (KIND == kLnFwdMV) { s0 += x; s1 += x * x; }
+            else if (KIND == kLnBwdV) s0 += (float)p.g[o] * c3 * x;
+            else if (KIND == kLnBwdMV) { const float gi = (float)p.g[o]; s0 += gi * c3 * (x - mean); s1 += -gi * var; }
+            else if (KIND == kSoftmaxBwd) s0 += x * (float)p.g[o];
+            else s0 = fmaxf(s0, fabsf(x * (float)p.sx[(p.bc ? 0 : b * p.n) + i]));
+        }
+    }
+    red[0][rg][c] = s0;
+    red[1][rg][c] = s1;
+    __syncthreads();
+    if (rg == 0) {
+        if (KIND == kScaleRound) tot[0][c] = fmaxf(fmaxf(red[0][0][c], red[0][1][c]), fmaxf(red[0][2][c], red[0][3][c]));
+        else tot[0][c] = red[0][0][c] + red[0][1][c] + red[0][2][c] + red[0][3][c];
+        tot[1][c] = red[1][0][c] + red[1][1][c] + red[1][2][c] + red[1][3][c];
+    }
+    __syncthreads();
+    s0 = tot[0][c];
+    s1 = tot[1][c];
+    if (!live) return;
+    const float fn = (float)p.n;
+    float k0 = 0.0f, k1 = 0.0f;        // per-column constants of the elementwise pass
+    if (KIND == kLnFwdV) {
+        k1 = rsqrtf(s1 / fn + p.eps);
+        if (rg == 0) p.out_var[b * p.m + col] = (half_t)k1;
+    } else if (KIND == kLnFwdMV) {
+        k0 = s0 / fn;
+        k1 = rsqrtf(s1 / fn - k0 * k0 + p.eps);
+        if (rg == 0) { p.out_var[b * p.m + col] = (half_t)k1; p.out_mean[b * p.m + col] = (half_t)k0; }
+    } else if (KIND == kLnBwdMV) {
+        s1 -= 2.0f * s0 * mean;        // local_grad_mean -= 2 * local_grad_var * local_mean
+    } else if (KIND == kScaleRound) {
+        k0 = (float)((double)s0 / 127.0);        // float / double constant, as the reference writes it
+        if (rg == 0) p.out_var[b * p.m + col] = (half_t)k0;
+    }
+    for (int32_t i = rg; i < p.n; i += 4) {
+        const int64_t o = boff + (int64_t)i * p.m + col;
+        const float x = (float)p.a[o];
+        if (KIND == kLnFwdV) p.out[o] = round_f16(x * k1);
+        else if (KIND == kLnFwdMV) p.out[o] = round_f16((x - k0) * k1);
+        else if (KIND == kLnBwdV) p.out[o] = round_f16((float)p.g[o] * var + (s0 * x * 2.0f) / fn);
+        else if (KIND == kLnBwdMV) p.out[o] = round_f16((float)p.g[o] * var + (s1 + s0 * x * 2.0f) / fn);
+        else if (KIND == kSoftmaxBwd) p.out[o] = round_f16(x * ((float)p.g[o] - s0));
+        else p.out_i8[o] = (int8_t)quant_i8(x * (float)p.sx[(p.bc ? 0 : b * p.n) + i], k0);
+    }
+}
+
+// cu_gemm_backward_round_scale: per-row absmax of mat * scale_y[col] -> scale_x, then rounding.
+__global__ __launch_bounds__(256) void k_round_scale_rows(int32_t n, int32_t m, const half_t* __restrict__ mat,
+                                                          const half_t* __restrict__ scale_y, int8_t* __restrict__ out,
+                                                          half_t* __restrict__ scale_x, int bc) {
+    __shared__ float red[4];
+    const int64_t row = blockIdx.x;                    // b*n + i
+    const int64_t b = row / n;
+    const half_t* x = mat + row * m;
+    const half_t* sy = scale_y + (bc ? 0 : b * m);
+    float mx = 0.0f;
+    for (int32_t j = threadIdx.x; j < m; j += 256) mx = fmaxf(fabsf((float)x[j] * (float)sy[j]), mx);
+    mx = block_max<4>(mx, red);
+    const float s = (float)((double)mx / 127.0);
+    if (threadIdx.x == 0) scale_x[row] = (half_t)s;
+    for (int32_t j = threadIdx.x; j < m; j += 256) out[row * m + j] = (int8_t)quant_i8((float)x[j] * (float)sy[j], s);
+}
+
+// ---------------------------------------------------------------------------------------
+// Gradient of the relative-position bias: grad[h, bucket] = sum of grad_out[h, k, q] over the
+// (k, q) that map to the bucket.  One workgroup per head, a bucket histogram in LDS.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_position_backward(int32_t query_len, int32_t key_len, int32_t num_buckets,
+                                                           int32_t max_distance, const int32_t* __restrict__ mapping,
+                                                           const half_t* __restrict__ grad_out, half_t* __restrict__ grad,
+                                                           int bidirectional) {
+    extern __shared__ float hist[];
+    const int h = blockIdx.x;
+    for (int i = threadIdx.x; i < num_buckets; i += 256) hist[i] = 0.0f;
+    __syncthreads();
+    const int64_t total = (int64_t)key_len * query_len;
+    const half_t* g = grad_out + (int64_t)h * total;
+    for (int64_t i = threadIdx.x; i < total; i += 256) {
+        int32_t rel = (int32_t)(i % query_len) - (int32_t)(i / query_len);
+        int32_t off = 0;
+        if (rel < 0) {
+            if (bidirectional) { rel = -rel; off = num_buckets / 2; }
+            else rel = 0;
+        }
+        if (rel >= max_distance) rel = max_distance - 1;
+        atomicAdd(&hist[mapping[rel] + off], (float)g[i]);
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < num_buckets; i += 256) grad[(int64_t)h * num_buckets + i] = (half_t)hist[i];
+}
+
+// ---------------------------------------------------------------------------------------
+// Embedding gradient in two stages over ids sorted per batch entry (cuda/embedding.cu:38-88):
+// stage 1 sums runs of equal ids inside one batch entry, writes complete runs to grad and the
+// last (possibly continuing) run to aux_grad; stage 2 adds the aux rows into grad, merging equal
+// neighbours.  One thread per hidden column, sequential over the ids as in the reference, so
+// sums are formed in the same order.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_embedding_backward1(int32_t n, int32_t m, const half_t* __restrict__ grad_out,
+                                                             const int32_t* __restrict__ argsort_ids,
+                                                             const int32_t* __restrict__ sorted_ids, half_t* grad,
+                                                             half_t* __restrict__ aux_grad, int32_t* __restrict__ aux_idx) {
+    const int64_t b = blockIdx.x;
+    const int32_t col = blockIdx.y * 256 + threadIdx.x;
+    if (col >= m) return;
+    const int64_t base = b * n;
+    float sum = 0.0f;
+    for (int32_t i = 0; i < n; ++i) {
+        sum += (float)grad_out[(int64_t)argsort_ids[base + i] * m + col];
+        if (i + 1 == n) {
+            aux_grad[b * m + col] = (half_t)sum;
+            if (col == 0) aux_idx[b] = sorted_ids[base + i];
+        } else if (sorted_ids[base + i] != sorted_ids[base + i + 1]) {
+            grad[(int64_t)sorted_ids[base + i] * m + col] = (half_t)sum;
+            sum = 0.0f;
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void k_embedding_backward2(int32_t batch, int32_t m, const half_t* __restrict__ aux_grad,
+                                                             const int32_t* __restrict__ aux_idx, half_t* grad) {
+    const int32_t col = blockIdx.x * 256 + threadIdx.x;
+    if (col >= m) return;
+    float sum = 0.0f;
+    for (int32_t i = 0; i < batch; ++i) {
+        sum += (float)aux_grad[(int64_t)i * m + col];
+        if (i + 1 == batch || aux_idx[i] != aux_idx[i + 1]) {
+            half_t* gp = grad + (int64_t)aux_idx[i] * m + col;
+            *gp = round_f16((float)*gp + sum);
+            sum = 0.0f;
+        }
+    }
+}
+
+template <int OP, int BC>
+static int launch_ew(int64_t total, int64_t n, int64_t m, const void* x, const void* a, const void* b, void* out, void* stream) {
+    if (total < 0) return CPMK_EBADARG;
+    if (total == 0) return 0;
+    if (total % 2) return CPMK_EALIGN;
+    hipLaunchKernelGGL((k_ew<OP, BC>), dim3((unsigned)ceil_div(total / 2, 256)), dim3(256), 0, (hipStream_t)stream, total, n, m,
+                       (const half_t*)x, (const half_t*)a, (const half_t*)b, (half_t*)out);
+    return launch_status();
+}
+
+template <int KIND>
+static int launch_col(int32_t batch, const ColArgs& p, void* stream) {
+    if (batch < 0 || p.n < 0 || p.m < 0) return CPMK_EBADARG;
+    if ((int64_t)batch * p.n * p.m == 0) return 0;
+    if (batch > 65535) return CPMK_ETOOBIG;
+    hipLaunchKernelGGL((k_col<KIND>), dim3((unsigned)ceil_div(p.m, 64), (unsigned)batch), dim3(256), 0, (hipStream_t)stream, p);
+    return launch_status();
+}
+
+}  // namespace cpmk
+
+using namespace cpmk;
+
+extern "C" {
+
+int cpmk_arith_global_scale(int64_t n, const void* inp, float scale, void* out, void* stream) {
+    clear_stale_error();
+    if (n < 0) return CPMK_EBADARG;
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(k_global_scale, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, (hipStream_t)stream, n, (const half_t*)inp,
+                       scale, (half_t*)out);
+    return launch_status();
+}
+int cpmk_arith_element_mul(int32_t batch, int32_t n, const void* x, const void* y, void* out, void* stream) {
+    clear_stale_error();
+    if (n % 2) return CPMK_EALIGN;
+    return launch_ew<kMul, 0>((int64_t)batch * n, n, 1, x, y, nullptr, out, stream);
+}
+int cpmk_arith_batch_add_forward(int32_t batch, int32_t n, const void* x, const void* y, void* out, void* stream) {
+    clear_stale_error();
+    if (n % 2) return CPMK_EALIGN;
+    return launch_ew<kAdd, 1>((int64_t)batch * n, n, 1, x, y, nullptr, out, stream);
+}
+int cpmk_arith_batch_mul_add(int32_t batch, int32_t n, const void* x, const void* alpha, const void* beta, void* out, void* stream) {
+    clear_stale_error();
+    if (n % 2) return CPMK_EALIGN;
+    return launch_ew<kFma, 1>((int64_t)batch * n, n, 1, x, alpha, beta, out, stream);
+}
+int cpmk_arith_batch_mul(int32_t batch, int32_t n, const void* x, const void* alpha, void* out, void* stream) {
+    clear_stale_error();
+    if (n % 2) return CPMK_EALIGN;
+    return launch_ew<kMul, 1>((int64_t)batch * n, n, 1, x, alpha, nullptr, out, stream);
+}
+int cpmk_arith_ln_add(int32_t batch, int32_t n, int32_t m, const void* inp, const void* beta, void* out, void* stream) {
+    clear_stale_error();
+    if (m % 2) return CPMK_EALIGN;
+    return launch_ew<kAdd, 2>((int64_t)batch * n * m, n, m, inp, beta, nullptr, out, stream);
+}
+int cpmk_arith_ln_div(int32_t batch, int32_t n, int32_t m, const void* inp, const void* alpha, void* out, void* stream) {
+    clear_stale_error();
+    if (m % 2) return CPMK_EALIGN;
+    return launch_ew<kDiv, 2>((int64_t)batch * n * m, n, m, inp, alpha, nullptr, out, stream);
+}
+int cpmk_arith_ln_sub_div(int32_t batch, int32_t n, int32_t m, const void* inp, const void* alpha, const void* beta, void* out,
+                          void* stream) {
+    clear_stale_error();
+    if (m % 2) return CPMK_EALIGN;
+    return launch_ew<kSubDiv, 2>((int64_t)batch * n * m, n, m, inp, alpha, beta, out, stream);
+}
+int cpmk_arith_batch_add_backward(int32_t batch, int32_t n, const void* grad_out, void* grad, void* stream) {
+    clear_stale_error();
+    if (batch < 0 || n < 0) return CPMK_EBADARG;
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(k_batch_add_backward, dim3((unsigned)ceil_div(n, 64)), dim3(256), 0, (hipStream_t)stream, (int64_t)batch,
+                       (int64_t)n, (const half_t*)grad_out, (half_t*)grad);
+    return launch_status();
+}
+int cpmk_arith_ln_mul_backward(int32_t batch, int32_t n, int32_t m, const void* inp, const void* grad_out, void* grad, void* stream) {
+    clear_stale_error();
+    if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
+    if (n == 0) return 0;
+    hipLaunchKernelGGL((k_ln_backward<true>), dim3((unsigned)n), dim3(256), 0, (hipStream_t)stream, (int64_t)batch, (int64_t)n,
+                       (int64_t)m, (const half_t*)inp, (const half_t*)grad_out, (half_t*)grad);
+    return launch_status();
+}
+int cpmk_arith_ln_add_backward(int32_t batch, int32_t n, int32_t m, const void* grad_out, void* grad, void* stream) {
+    clear_stale_error();
+    if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
+    if (n == 0) return 0;
+    hipLaunchKernelGGL((k_ln_backward<false>), dim3((unsigned)n), dim3(256), 0, (hipStream_t)stream, (int64_t)batch, (int64_t)n,
+                       (int64_t)m, (const half_t*)nullptr, (const half_t*)grad_out, (half_t*)grad);
+    return launch_status();
+}
+
+int cpmk_gelu_backward(int32_t batch, int32_t n, const void* grad_out, const void* mat, void* grad, void* stream) {
+    clear_stale_error();
+    if (batch < 0 || n < 0) return CPMK_EBADARG;
+    const int64_t total = (int64_t)batch * n;
+    if (total == 0) return 0;
+    hipLaunchKernelGGL(k_gelu_backward, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, (hipStream_t)stream, total,
+                       (const half_t*)grad_out, (const half_t*)mat, (half_t*)grad);
+    return launch_status();
+}
+
+int cpmk_layernorm_forward_v(int32_t batch, int32_t n, int32_t m, const void* mat, void* out, void* out_var, float eps, void* stream) {
+    clear_stale_error();
+    ColArgs p = {n, m, (const half_t*)mat, nullptr, nullptr, nullptr, nullptr, (half_t*)out, nullptr, nullptr, (half_t*)out_var, eps, 0};
+    return launch_col<kLnFwdV>(batch, p, stream);
+}
+int cpmk_layernorm_forward_mv(int32_t batch, int32_t n, int32_t m, const void* mat, void* out, void* out_mean, void* out_var,
+                              float eps, void* stream) {
+    clear_stale_error();
+    ColArgs p = {n, m, (const half_t*)mat, nullptr, nullptr, nullptr, nullptr, (half_t*)out, nullptr, (half_t*)out_mean,
+                 (half_t*)out_var, eps, 0};
+    return launch_col<kLnFwdMV>(batch, p, stream);
+}
+int cpmk_layernorm_backward_v(int32_t batch, int32_t n, int32_t m, const void* mat, const void* grad_out, const void* var, void* grad,
+                              void* stream) {
+    clear_stale_error();
+    ColArgs p = {n, m, (const half_t*)mat, (const half_t*)grad_out, nullptr, (const half_t*)var, nullptr, (half_t*)grad, nullptr,
+                 nullptr, nullptr, 0.0f, 0};
+    return launch_col<kLnBwdV>(batch, p, stream);
+}
+int cpmk_layernorm_backward_mv(int32_t batch, int32_t n, int32_t m, const void* mat, const void* grad_out, const void* mean,
+                               const void* var, void* grad, void* stream) {
+    clear_stale_error();
+    ColArgs p = {n, m, (const half_t*)mat, (const half_t*)grad_out, (const half_t*)mean, (const half_t*)var, nullptr, (half_t*)grad,
+                 nullptr, nullptr, nullptr, 0.0f, 0};
+    return launch_col<kLnBwdMV>(batch, p, stream);
+}
+int cpmk_softmax_backward(int32_t batch, int32_t n, int32_t m, const void* out, const void* grad_out, void* grad, void* stream) {
+    clear_stale_error();
+    ColArgs p = {n, m, (const half_t*)out, (const half_t*)grad_out, nullptr, nullptr, nullptr, (half_t*)grad, nullptr, nullptr, nullptr,
+                 0.0f, 0};
+    return launch_col<kSoftmaxBwd>(batch, p, stream);
+}
+int cpmk_gemm_backward_scale_round(int32_t batch, int32_t n, int32_t m, const void* mat, const void* scale_x, void* out, void* scale_y,
+                                   int broad_cast_x, void* stream) {
+    clear_stale_error();
+    ColArgs p = {n, m, (const half_t*)mat, nullptr, nullptr, nullptr, (const half_t*)scale_x, nullptr, (int8_t*)out, nullptr,
+                 (half_t*)scale_y, 0.0f, broad_cast_x};
+    return launch_col<kScaleRound>(batch, p, stream);
+}
+int cpmk_gemm_backward_round_scale(int32_t batch, int32_t n, int32_t m, const void* mat, const void* scale_y, void* out, void* scale_x,
+                                   int broad_cast_y, void* stream) {
+    clear_stale_error();
+    if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
+    const int64_t rows = (int64_t)batch * n;
+    if (rows == 0) return 0;
+    if (rows > 0x7fffffff) return CPMK_ETOOBIG;
+    hipLaunchKernelGGL(k_round_scale_rows, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, n, m, (const half_t*)mat,
+                       (const half_t*)scale_y, (int8_t*)out, (half_t*)scale_x, broad_cast_y);
+    return launch_status();
+}
+
+int cpmk_position_embedding_backward(int32_t query_len, int32_t key_len, int32_t num_buckets, int32_t max_distance, int32_t num_heads,
+                                     const void* position_mapping, const void* grad_out, void* grad, int bidirectional, void* stream) {
+    clear_stale_error();
+    if (query_len < 0 || key_len < 0 || num_buckets <= 0 || max_distance <= 0 || num_heads < 0) return CPMK_EBADARG;
+    if (num_heads == 0) return 0;
+    if (num_buckets > 8192) return CPMK_ETOOBIG;
+    hipLaunchKernelGGL(k_position_backward, dim3((unsigned)num_heads), dim3(256), num_buckets * sizeof(float), (hipStream_t)stream,
+                       query_len, key_len, num_buckets, max_distance, (const int32_t*)position_mapping, (const half_t*)grad_out,
+                       (half_t*)grad, bidirectional);
+    return launch_status();
+}
+
+int cpmk_embedding_backward_stage1(int32_t batch, int32_t seq_len, int32_t hidden_size, const void* grad_out, const void* argsort_ids,
+                                   const void* sorted_ids, void* grad, void* aux_grad, void* aux_grad_idx, void* stream) {
+    clear_stale_error();
+    if (batch < 0 || seq_len < 0 || hidden_size < 0) return CPMK_EBADARG;
+    if ((int64_t)batch * seq_len * hidden_size == 0) return 0;
+    if (ceil_div(hidden_size, 256) > 65535) return CPMK_ETOOBIG;
+    hipLaunchKernelGGL(k_embedding_backward1, dim3((unsigned)batch, (unsigned)ceil_div(hidden_size, 256)), dim3(256), 0,
+                       (hipStream_t)stream, seq_len, hidden_size, (const half_t*)grad_out, (const int32_t*)argsort_ids,
+                       (const int32_t*)sorted_ids, (half_t*)grad, (half_t*)aux_grad, (int32_t*)aux_grad_idx);
+    return launch_status();
+}
+int cpmk_embedding_backward_stage2(int32_t batch, int32_t hidden_size, const void* aux_grad, const void* aux_grad_idx, void* grad,
+                                   void* stream) {
+    clear_stale_error();
+    if (batch < 0 || hidden_size < 0) return CPMK_EBADARG;
+    if ((int64_t)batch * hidden_size == 0) return 0;
+    hipLaunchKernelGGL(k_embedding_backward2, dim3((unsigned)ceil_div(hidden_size, 256)), dim3(256), 0, (hipStream_t)stream, batch,
+                       hidden_size, (const half_t*)aux_grad, (const int32_t*)aux_grad_idx, (half_t*)grad);
+    return launch_status();
+}
+
+}  // extern "C"

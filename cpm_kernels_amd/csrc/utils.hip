@@ -1,0 +1,123 @@
+// Small utilities of the reference's kernels layer: transpose (cuda/transpose.cu:6-24) and the
+// generation helpers of cuda/utils.cu:31-101 (array_add, adjustify_logits, copy_extend_buffer,
+// has_nan_inf, copy_pos_hidden).
+#include "common.h"
+
+namespace cpmk {
+
+// (batch, n, m) -> (batch, m, n) through a 64x64 LDS tile: each wave reads 128-byte row pieces
+// and writes 128-byte row pieces of the transposed tensor.
+__global__ __launch_bounds__(256) void k_transpose(int32_t n, int32_t m, const half_t* __restrict__ in, half_t* __restrict__ out) {
+    __shared__ half_t tile[64][66];
+    const int64_t boff = (int64_t)blockIdx.z * n * m;
+    const int32_t r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (int r = ty; r < 64; r += 4)
+        if (r0 + r < n && c0 + tx < m) tile[r][tx] = in[boff + (int64_t)(r0 + r) * m + c0 + tx];
+    __syncthreads();
+    for (int c = ty; c < 64; c += 4)
+        if (c0 + c < m && r0 + tx < n) out[boff + (int64_t)(c0 + c) * n + r0 + tx] = tile[tx][c];
+}
+
+__global__ void k_array_add(int32_t* arr, int32_t pos, int32_t val) {
+    if (threadIdx.x == 0) arr[pos] += val;
+}
+
+__global__ __launch_bounds__(256) void k_adjustify_logits(int64_t total, half_t* logits, float temperature, float frequency_penalty,
+                                                          float presence_penalty, const int32_t* __restrict__ frequency) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    float v = (float)logits[i];
+    const int32_t freq = frequency[i];
+    v /= temperature;
+    v -= frequency_penalty * (float)freq;
+    v -= presence_penalty * (freq > 0 ? 1.0f : 0.0f);
+    logits[i] = round_f16(v);
+}
+
+__global__ __launch_bounds__(256) void k_copy_extend(int32_t old_size, int32_t nw_size, const half_t* __restrict__ old_buf,
+                                                     half_t* __restrict__ nw_buf) {
+    const int32_t col = blockIdx.x * 256 + threadIdx.x;
+    if (col < old_size) nw_buf[(int64_t)blockIdx.y * nw_size + col] = old_buf[(int64_t)blockIdx.y * old_size + col];
+}
+
+// out[0] = 1 when any element is +-inf or NaN; out is left untouched otherwise (the caller clears it).
+__global__ __launch_bounds__(256) void k_has_nan_inf(int64_t n, const uint16_t* __restrict__ inp, int8_t* out) {
+    bool bad = false;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
+        bad |= (inp[i] & 0x7c00u) == 0x7c00u;       // exponent all ones: inf or NaN
+    if (__ballot(bad) != 0 && (threadIdx.x & 63) == 0) out[0] = 1;
+}
+
+__global__ __launch_bounds__(256) void k_copy_pos_hidden(int32_t hidden_size, int32_t seq_len, int32_t pos,
+                                                         const half_t* __restrict__ inp, half_t* __restrict__ out) {
+    const int32_t col = blockIdx.x * 256 + threadIdx.x;
+    if (col < hidden_size)
+        out[(int64_t)blockIdx.y * hidden_size + col] = inp[((int64_t)blockIdx.y * hidden_size + col) * seq_len + pos];
+}
+
+}  // namespace cpmk
+
+using namespace cpmk;
+
+extern "C" {
+
+int cpmk_transpose(int32_t batch, int32_t n, int32_t m, const void* inp, void* out, void* stream) {
+    clear_stale_error();
+    if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
+    if ((int64_t)batch * n * m == 0) return 0;
+    if (batch > 65535 || ceil_div(n, 64) > 65535) return CPMK_ETOOBIG;
+    hipLaunchKernelGGL(k_transpose, dim3((unsigned)ceil_div(m, 64), (unsigned)ceil_div(n, 64), (unsigned)batch), dim3(256), 0,
+                       (hipStream_t)stream, n, m, (const half_t*)inp, (half_t*)out);
+    return launch_status();
+}
+
+int cpmk_array_add(void* array, int32_t pos, int32_t val, void* stream) {
+    clear_stale_error();
+    if (pos < 0 || !array) return CPMK_EBADARG;
+    hipLaunchKernelGGL(k_array_add, dim3(1), dim3(64), 0, (hipStream_t)stream, (int32_t*)array, pos, val);
+    return launch_status();
+}
+
+int cpmk_adjustify_logits(int32_t batch, int32_t n, void* logits, float temperature, float frequency_penalty, float presence_penalty,
+                          const void* frequency, void* stream) {
+    clear_stale_error();
+    if (batch < 0 || n < 0) return CPMK_EBADARG;
+    const int64_t total = (int64_t)batch * n;
+    if (total == 0) return 0;
+    hipLaunchKernelGGL(k_adjustify_logits, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, (hipStream_t)stream, total,
+                       (half_t*)logits, temperature, frequency_penalty, presence_penalty, (const int32_t*)frequency);
+    return launch_status();
+}
+
+int cpmk_copy_extend_buffer(int32_t batch, int32_t old_size, int32_t nw_size, const void* old_buffer, void* new_buffer, void* stream) {
+    clear_stale_error();
+    if (batch < 0 || old_size < 0 || nw_size < old_size) return CPMK_EBADARG;
+    if ((int64_t)batch * old_size == 0) return 0;
+    if (batch > 65535) return CPMK_ETOOBIG;
+    hipLaunchKernelGGL(k_copy_extend, dim3((unsigned)ceil_div(old_size, 256), (unsigned)batch), dim3(256), 0, (hipStream_t)stream,
+                       old_size, nw_size, (const half_t*)old_buffer, (half_t*)new_buffer);
+    return launch_status();
+}
+
+int cpmk_has_nan_inf(int64_t n, const void* inp, void* out, void* stream) {
+    clear_stale_error();
+    if (n < 0) return CPMK_EBADARG;
+    if (n == 0) return 0;
+    const int64_t blocks = ceil_div(n, 256 * 16);
+    hipLaunchKernelGGL(k_has_nan_inf, dim3((unsigned)(blocks > 2048 ? 2048 : blocks)), dim3(256), 0, (hipStream_t)stream, n,
+                       (const uint16_t*)inp, (int8_t*)out);
+    return launch_status();
+}
+
+int cpmk_copy_pos_hidden(int32_t batch, int32_t hidden_size, int32_t seq_len, int32_t pos, const void* inp, void* out, void* stream) {
+    clear_stale_error();
+    if (batch < 0 || hidden_size < 0 || seq_len < 0 || pos < 0 || (seq_len > 0 && pos >= seq_len)) return CPMK_EBADARG;
+    if ((int64_t)batch * hidden_size * seq_len == 0) return 0;
+    if (batch > 65535) return CPMK_ETOOBIG;
+    hipLaunchKernelGGL(k_copy_pos_hidden, dim3((unsigned)ceil_div(hidden_size, 256), (unsigned)batch), dim3(256), 0,
+                       (hipStream_t)stream, hidden_size, seq_len, pos, (const half_t*)inp, (half_t*)out);
+    return launch_status();
+}
+
+}  // extern "C"

@@ -1,7 +1,6 @@
-"""Token-embedding gathers with the signatures of cpm_kernels/kernels/embedding.py (forward and
-decode step; the backward stages are outside the inference path)."""
+"""Token-embedding gathers with the signatures of cpm_kernels/kernels/embedding.py ."""
 from ..library import cpmk
-from .base import DevicePointer, CUDAStream, _stream, not_on_path
+from .base import DevicePointer, CUDAStream, _stream
 
 
 def embedding_forward(batch: int,
@@ -24,6 +23,23 @@ def embedding_step(batch: int, embedding_size: int,
     cpmk.embedding_step(batch, embedding_size, ids, weights, out, _stream(stream))
 
 
-_e = "token embedding backward, kernels/embedding.py"
-embedding_backward_stage1 = not_on_path("embedding_backward_stage1", _e)
-embedding_backward_stage2 = not_on_path("embedding_backward_stage2", _e)
+def embedding_backward_stage1(batch: int, seq_len: int, hidden_size: int,
+                              grad_out: DevicePointer,        # (batch * n, m)
+                              argsort_ids: DevicePointer,     # (batch, n)
+                              sorted_ids: DevicePointer,      # (batch, n)
+                              grad: DevicePointer,            # (vocab_size, m)
+                              aux_grad: DevicePointer,        # (batch, m)
+                              aux_grad_idx: DevicePointer,    # (batch)
+                              stream: CUDAStream):
+    """Sums runs of equal sorted ids inside each batch entry.  reference: kernels/embedding.py:36-65"""
+    cpmk.embedding_backward_stage1(batch, seq_len, hidden_size, grad_out, argsort_ids, sorted_ids, grad, aux_grad,
+                                   aux_grad_idx, _stream(stream))
+
+
+def embedding_backward_stage2(batch: int, hidden_size: int,
+                              aux_grad: DevicePointer,        # (batch, m)
+                              aux_grad_idx: DevicePointer,    # (batch)
+                              grad: DevicePointer,            # (vocab_size, m)
+                              stream: CUDAStream):
+    """Adds the per-entry tail runs into grad.  reference: kernels/embedding.py:67-86"""
+    cpmk.embedding_backward_stage2(batch, hidden_size, aux_grad, aux_grad_idx, grad, _stream(stream))

@@ -1,6 +1,6 @@
 """GELU launchers with the signatures of cpm_kernels/kernels/gelu.py."""
 from ..library import cpmk
-from .base import DevicePointer, CUDAStream, _stream, not_on_path
+from .base import DevicePointer, CUDAStream, _stream
 
 
 def gelu_forward(batch: int, n: int,
@@ -17,4 +17,8 @@ def gelu_inplace_forward(batch: int, n: int,
     cpmk.gelu_forward(batch, n, mat, mat, _stream(stream))
 
 
-gelu_backward = not_on_path("gelu_backward", "training, kernels/gelu.py:50-69")
+def gelu_backward(batch: int, n: int,
+                  grad_out: DevicePointer, mat: DevicePointer, grad: DevicePointer,
+                  stream: CUDAStream):
+    """grad = gelu'(mat) * grad_out.  reference: kernels/gelu.py:50-69"""
+    cpmk.gelu_backward(batch, n, grad_out, mat, grad, _stream(stream))

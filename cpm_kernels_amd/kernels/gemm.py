@@ -1,7 +1,7 @@
 """Quantisation, int8 GEMM and dequantisation launchers with the signatures of
 cpm_kernels/kernels/gemm.py.  Arithmetic contracts are stated in include/cpmk.h."""
 from ..library import cpmk
-from .base import DevicePointer, CUDAStream, _stream, not_on_path
+from .base import DevicePointer, CUDAStream, _stream
 
 
 def gemm_round(batch: int, n: int, m: int,
@@ -142,5 +142,23 @@ def gemm_fp16(m: int, k: int, n: int,
     cpmk.gemm_fp16(m, k, n, batchA, batchB, int(bool(aT)), int(bool(bT)), A, B, out, _stream(stream))
 
 
-gemm_backward_round_scale = not_on_path("gemm_backward_round_scale", "training, kernels/gemm.py:258-281")
-gemm_backward_scale_round = not_on_path("gemm_backward_scale_round", "training, kernels/gemm.py:283-307")
+def gemm_backward_round_scale(batch: int, n: int, m: int,
+                              mat: DevicePointer,        # (batch, n, m) fp16
+                              scale_y: DevicePointer,    # (batch, m)    fp16
+                              out: DevicePointer,        # (batch, n, m) int8
+                              scale_x: DevicePointer,    # (batch, n)    fp16
+                              broad_cast_y: bool,
+                              stream: CUDAStream):
+    """Row scales and int8 rounding of mat * scale_y.  reference: kernels/gemm.py:261-283"""
+    cpmk.gemm_backward_round_scale(batch, n, m, mat, scale_y, out, scale_x, int(bool(broad_cast_y)), _stream(stream))
+
+
+def gemm_backward_scale_round(batch: int, n: int, m: int,
+                              mat: DevicePointer,        # (batch, n, m) fp16
+                              scale_x: DevicePointer,    # (batch, n)    fp16
+                              out: DevicePointer,        # (batch, n, m) int8
+                              scale_y: DevicePointer,    # (batch, m)    fp16
+                              broad_cast_x: bool,
+                              stream: CUDAStream):
+    """Column scales and int8 rounding of mat * scale_x.  reference: kernels/gemm.py:285-307"""
+    cpmk.gemm_backward_scale_round(batch, n, m, mat, scale_x, out, scale_y, int(bool(broad_cast_x)), _stream(stream))

@@ -1,6 +1,6 @@
 """Normalisation launchers with the signatures of cpm_kernels/kernels/layernorm.py."""
 from ..library import cpmk
-from .base import DevicePointer, CUDAStream, _stream, not_on_path
+from .base import DevicePointer, CUDAStream, _stream
 
 
 def layernorm_forward(batch: int, n: int, m: int,
@@ -50,8 +50,44 @@ def layernorm_step_inplace(batch: int, n: int,
     cpmk.layernorm_step(batch, n, mat, mat, eps, int(bool(rd_mean)), _stream(stream))
 
 
-_w = "training, kernels/layernorm.py:60-150"
-layernorm_forward_v = not_on_path("layernorm_forward_v", _w)
-layernorm_forward_mv = not_on_path("layernorm_forward_mv", _w)
-layernorm_backward_v = not_on_path("layernorm_backward_v", _w)
-layernorm_backward_mv = not_on_path("layernorm_backward_mv", _w)
+def layernorm_forward_v(batch: int, n: int, m: int,
+                        mat: DevicePointer,        # (batch, n, m)
+                        out: DevicePointer,        # (batch, n, m)
+                        out_var: DevicePointer,    # (batch, m)
+                        eps: float,
+                        stream: CUDAStream):
+    """RMS norm over dim 1 that keeps rsqrt(mean(x^2) + eps) for the backward pass.
+    reference: kernels/layernorm.py:60-80"""
+    cpmk.layernorm_forward_v(batch, n, m, mat, out, out_var, eps, _stream(stream))
+
+
+def layernorm_forward_mv(batch: int, n: int, m: int,
+                         mat: DevicePointer,         # (batch, n, m)
+                         out: DevicePointer,         # (batch, n, m)
+                         out_mean: DevicePointer,    # (batch, m)
+                         out_var: DevicePointer,     # (batch, m)
+                         eps: float,
+                         stream: CUDAStream):
+    """reference: kernels/layernorm.py:82-104"""
+    cpmk.layernorm_forward_mv(batch, n, m, mat, out, out_mean, out_var, eps, _stream(stream))
+
+
+def layernorm_backward_v(batch: int, n: int, m: int,
+                         mat: DevicePointer,         # (batch, n, m)
+                         grad_out: DevicePointer,    # (batch, n, m)
+                         var: DevicePointer,         # (batch, m)
+                         grad: DevicePointer,        # (batch, n, m)
+                         stream: CUDAStream):
+    """reference: kernels/layernorm.py:106-126"""
+    cpmk.layernorm_backward_v(batch, n, m, mat, grad_out, var, grad, _stream(stream))
+
+
+def layernorm_backward_mv(batch: int, n: int, m: int,
+                          mat: DevicePointer,         # (batch, n, m)
+                          grad_out: DevicePointer,    # (batch, n, m)
+                          mean: DevicePointer,        # (batch, m)
+                          var: DevicePointer,         # (batch, m)
+                          grad: DevicePointer,        # (batch, n, m)
+                          stream: CUDAStream):
+    """reference: kernels/layernorm.py:128-150"""
+    cpmk.layernorm_backward_mv(batch, n, m, mat, grad_out, mean, var, grad, _stream(stream))

@@ -1,6 +1,6 @@
 """Softmax launchers with the signatures of cpm_kernels/kernels/softmax.py."""
 from ..library import cpmk
-from .base import DevicePointer, CUDAStream, _stream, not_on_path
+from .base import DevicePointer, CUDAStream, _stream
 
 
 def softmax_forward(batch: int, n: int, m: int,
@@ -25,4 +25,10 @@ def softmax_step_inplace(batch: int, n: int,
     cpmk.softmax_step_inplace(batch, n, x, _stream(stream))
 
 
-softmax_backward = not_on_path("softmax_backward", "training, kernels/softmax.py:48-66")
+def softmax_backward(batch: int, n: int, m: int,
+                     out: DevicePointer,         # (batch, n, m)
+                     grad_out: DevicePointer,    # (batch, n, m)
+                     grad: DevicePointer,        # (batch, n, m)
+                     stream: CUDAStream):
+    """grad = out * (grad_out - (out * grad_out).sum(1)).  reference: kernels/softmax.py:48-66"""
+    cpmk.softmax_backward(batch, n, m, out, grad_out, grad, _stream(stream))

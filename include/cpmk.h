@@ -235,6 +235,102 @@ int cpmk_arith_element_add(int32_t batch, int32_t n, const void* x, const void* 
 int cpmk_mask(int32_t batch, int32_t n, int32_t m, const void* inp,
               const void* mask /* (b,m) int8 */, float value, void* out, void* stream);
 
+/* ---- training side and remaining helpers of the kernels layer ---------------------------------
+ * Not on the inference hot path; same arithmetic as the reference (fp16 ops round once, sums
+ * accumulate in fp32; the order of fp32 summation differs, so sums agree to rounding only). */
+
+/* out = fp16(float(x) * scale) over n elements; n % 2 == 0 asserted by the reference wrapper.
+ *                                                     kernels/arith.py:24-41 / arith.cu:6-16 */
+int cpmk_arith_global_scale(int64_t n, const void* inp, float scale, void* out, void* stream);
+/* out = x * y (fp16); n % 2 == 0.                     kernels/arith.py:68-91 / arith.cu:33-44 */
+int cpmk_arith_element_mul(int32_t batch, int32_t n, const void* x, const void* y, void* out, void* stream);
+/* out[b,j] = x[b,j] + y[j]; n % 2 == 0.               kernels/arith.py:93-116 / arith.cu:47-58 */
+int cpmk_arith_batch_add_forward(int32_t batch, int32_t n, const void* x, const void* y, void* out, void* stream);
+/* grad[j] = sum_b grad_out[b,j].                      kernels/arith.py:118-133 / arith.cu:61-77 */
+int cpmk_arith_batch_add_backward(int32_t batch, int32_t n, const void* grad_out, void* grad, void* stream);
+/* out[b,i,j] = x[b,i,j] + beta[i]; m % 2 == 0.        kernels/arith.py:163-188 / arith.cu:80-94 */
+int cpmk_arith_ln_add(int32_t batch, int32_t n, int32_t m, const void* inp, const void* beta, void* out, void* stream);
+/* out[b,i,j] = x * fp16(1 / alpha[i]); m % 2 == 0.    kernels/arith.py:216-240 / arith.cu:131-143 */
+int cpmk_arith_ln_div(int32_t batch, int32_t n, int32_t m, const void* inp, const void* alpha, void* out, void* stream);
+/* out = fp16_fma(x, fp16(1/alpha[i]), fp16(-beta[i]/alpha[i])); m % 2 == 0.
+ *                                                     kernels/arith.py:242-269 / arith.cu:146-165 */
+int cpmk_arith_ln_sub_div(int32_t batch, int32_t n, int32_t m, const void* inp, const void* alpha, const void* beta,
+                          void* out, void* stream);
+/* grad[i] = sum_{b,j} x[b,i,j] * grad_out[b,i,j].     kernels/arith.py:271-289 / arith.cu:168-214 */
+int cpmk_arith_ln_mul_backward(int32_t batch, int32_t n, int32_t m, const void* inp, const void* grad_out, void* grad,
+                               void* stream);
+/* grad[i] = sum_{b,j} grad_out[b,i,j].                kernels/arith.py:291-307 / arith.cu:217-261 */
+int cpmk_arith_ln_add_backward(int32_t batch, int32_t n, int32_t m, const void* grad_out, void* grad, void* stream);
+/* out[b,j] = fp16_fma(x[b,j], alpha[j], beta[j]); n % 2 == 0.   kernels/arith.py:309-331 / arith.cu:264-275 */
+int cpmk_arith_batch_mul_add(int32_t batch, int32_t n, const void* x, const void* alpha, const void* beta, void* out,
+                             void* stream);
+/* out[b,j] = x[b,j] * alpha[j]; n % 2 == 0.           kernels/arith.py:333-354 / arith.cu:278-288 */
+int cpmk_arith_batch_mul(int32_t batch, int32_t n, const void* x, const void* alpha, void* out, void* stream);
+
+/* grad = gelu'(mat) * grad_out (tanh form, derivative 0/1 outside |x| < 5).
+ *                                                     kernels/gelu.py:50-69 / gelu.cu:20-45 */
+int cpmk_gelu_backward(int32_t batch, int32_t n, const void* grad_out, const void* mat, void* grad, void* stream);
+
+/* grad[b,i,j] = out[b,i,j] * (grad_out[b,i,j] - sum_i out*grad_out).   kernels/softmax.py:48-66 / softmax.cu:86-114 */
+int cpmk_softmax_backward(int32_t batch, int32_t n, int32_t m, const void* out, const void* grad_out, void* grad,
+                          void* stream);
+
+/* RMS-norm over dim 1 that also returns out_var[b,j] = rsqrt(mean(x^2) + eps) as fp16.
+ *                                                     kernels/layernorm.py:60-80 / layernorm.cu:142-184 */
+int cpmk_layernorm_forward_v(int32_t batch, int32_t n, int32_t m, const void* mat, void* out, void* out_var, float eps,
+                             void* stream);
+/* Mean-subtracting norm that also returns out_mean and out_var (reciprocal std), both (batch, m) fp16.
+ *                                                     kernels/layernorm.py:82-104 / layernorm.cu:187-241 */
+int cpmk_layernorm_forward_mv(int32_t batch, int32_t n, int32_t m, const void* mat, void* out, void* out_mean,
+                              void* out_var, float eps, void* stream);
+/* Gradient of forward_v given its out_var.            kernels/layernorm.py:106-126 / layernorm.cu:244-282 */
+int cpmk_layernorm_backward_v(int32_t batch, int32_t n, int32_t m, const void* mat, const void* grad_out,
+                              const void* var, void* grad, void* stream);
+/* Gradient of forward_mv given its out_mean/out_var.  kernels/layernorm.py:128-150 / layernorm.cu:285-339 */
+int cpmk_layernorm_backward_mv(int32_t batch, int32_t n, int32_t m, const void* mat, const void* grad_out,
+                               const void* mean, const void* var, void* grad, void* stream);
+
+/* scale_x[b,i] = max_j |mat*scale_y| / 127 (fp16 out), out = int8(rint(mat*scale_y / that quotient in fp32)).
+ *                                                     kernels/gemm.py:261-283 / gemm.cu:102-133 */
+int cpmk_gemm_backward_round_scale(int32_t batch, int32_t n, int32_t m, const void* mat, const void* scale_y,
+                                   void* out, void* scale_x, int broad_cast_y, void* stream);
+/* The same along dim 1: scale_y[b,j] from max_i |mat*scale_x|.   kernels/gemm.py:285-307 / gemm.cu:136-172 */
+int cpmk_gemm_backward_scale_round(int32_t batch, int32_t n, int32_t m, const void* mat, const void* scale_x,
+                                   void* out, void* scale_y, int broad_cast_x, void* stream);
+
+/* grad[h, bucket] = sum of grad_out[h,k,q] over the (k,q) of the bucket; num_buckets <= 8192.
+ *                                                     kernels/position_bucket.py:60-86 / position_bucket.cu:57-103 */
+int cpmk_position_embedding_backward(int32_t query_len, int32_t key_len, int32_t num_buckets, int32_t max_distance,
+                                     int32_t num_heads, const void* position_mapping, const void* grad_out,
+                                     void* grad, int bidirectional, void* stream);
+
+/* Embedding gradient, stage 1: per batch entry, runs of equal sorted ids summed; complete runs to grad,
+ * the last run to aux_grad/aux_grad_idx.              kernels/embedding.py:36-65 / embedding.cu:36-64 */
+int cpmk_embedding_backward_stage1(int32_t batch, int32_t seq_len, int32_t hidden_size, const void* grad_out,
+                                   const void* argsort_ids, const void* sorted_ids, void* grad, void* aux_grad,
+                                   void* aux_grad_idx, void* stream);
+/* Stage 2: aux rows added into grad, equal neighbours merged first.   kernels/embedding.py:67-86 / embedding.cu:67-88 */
+int cpmk_embedding_backward_stage2(int32_t batch, int32_t hidden_size, const void* aux_grad, const void* aux_grad_idx,
+                                   void* grad, void* stream);
+
+/* (batch, n, m) -> (batch, m, n), fp16.               kernels/transpose.py:11-29 / transpose.cu:6-24 */
+int cpmk_transpose(int32_t batch, int32_t n, int32_t m, const void* inp, void* out, void* stream);
+/* array[pos] += val (int32).                          kernels/utils.py:39-53 / utils.cu:31-35 */
+int cpmk_array_add(void* array, int32_t pos, int32_t val, void* stream);
+/* logits = logits / temperature - frequency_penalty*freq - presence_penalty*(freq > 0), in place.
+ *                                                     kernels/utils.py:55-77 / utils.cu:38-54 */
+int cpmk_adjustify_logits(int32_t batch, int32_t n, void* logits, float temperature, float frequency_penalty,
+                          float presence_penalty, const void* frequency, void* stream);
+/* new[b, :old_size] = old[b, :]; the rest of new untouched.   kernels/utils.py:79-96 / utils.cu:57-67 */
+int cpmk_copy_extend_buffer(int32_t batch, int32_t old_size, int32_t nw_size, const void* old_buffer,
+                            void* new_buffer, void* stream);
+/* out[0] = 1 if any fp16 of inp is inf or NaN, otherwise out is left as it was.
+ *                                                     kernels/utils.py:98-112 / utils.cu:70-88 */
+int cpmk_has_nan_inf(int64_t n, const void* inp, void* out, void* stream);
+/* out[b,h] = inp[b,h,pos] for inp (batch, hidden, seq_len).   kernels/utils.py:114-134 / utils.cu:91-101 */
+int cpmk_copy_pos_hidden(int32_t batch, int32_t hidden_size, int32_t seq_len, int32_t pos, const void* inp,
+                         void* out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
