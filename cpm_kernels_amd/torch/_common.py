@@ -10,12 +10,3 @@ def check_half(x: torch.Tensor, ndim=None):
     assert x.is_cuda and x.is_contiguous() and x.dtype == torch.float16
     if ndim is not None:
         assert x.ndim == ndim
-
-
-class InferenceOnly(torch.autograd.Function):
-    """Base for the wrappers: the int8 inference path has no backward kernels in this build
-    (the reference's backward passes are training-only)."""
-
-    @staticmethod
-    def backward(ctx, *grads):
-        raise NotImplementedError("cpm_kernels_amd implements the inference (forward) path only")

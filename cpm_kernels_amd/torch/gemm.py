@@ -8,8 +8,9 @@ the six-launch sequence, which ``fused=False`` still runs through the kernel-lev
 """
 import torch
 from ..kernels import gemm_calc_scale, gemm_calc_scale_transpose, gemm_round, gemm_round_transpose, \
-    gemm_scale, gemm_int8, gemm_int8_scale, gemm_quantize, gemm_quantize_cols, gemm_quantize_pair, gemm_fp16
-from ._common import cur_stream, InferenceOnly
+    gemm_scale, gemm_scale_x, gemm_scale_y, gemm_int8, gemm_int8_scale, gemm_quantize, gemm_quantize_cols, \
+    gemm_quantize_pair, gemm_fp16, gemm_backward_round_scale, gemm_backward_scale_round
+from ._common import cur_stream
 
 
 def calc_scale(mat: torch.Tensor, transpose: bool) -> torch.Tensor:
@@ -66,12 +67,13 @@ def _dims(quantA, quantB, aT, bT):
 
 
 def gemm_and_scale(quantA, scaleA, quantB, scaleB, aT, bT, fused=True) -> torch.Tensor:
-    """reference: torch/gemm.py:40-82 (both scales present).  The operands are swapped in
-    the kernel call exactly as there (:45-52) so the (M, N) product comes out row-major."""
+    """reference: torch/gemm.py:40-82.  The operands are swapped in the kernel call exactly as
+    there (:45-52) so the (M, N) product comes out row-major.  One of the scales may be None
+    (the backward products): the accumulator is then scaled along the other side only."""
     M, K, N = _dims(quantA, quantB, aT, bT)
     batch = max(quantA.size(0), quantB.size(0))
     result_fp = torch.empty((batch, M, N), dtype=torch.float16, device=quantA.device)
-    if fused:
+    if fused and scaleA is not None and scaleB is not None:
         gemm_int8_scale(N, K, M, quantB.size(0), quantA.size(0), bT, aT,
                         quantB.data_ptr(), quantA.data_ptr(),
                         scaleA.data_ptr(), scaleB.data_ptr(),
@@ -81,12 +83,18 @@ def gemm_and_scale(quantA, scaleA, quantB, scaleB, aT, bT, fused=True) -> torch.
     result_i32 = torch.empty((batch, M, N), dtype=torch.int32, device=quantA.device)
     gemm_int8(N, K, M, quantB.size(0), quantA.size(0), bT, aT,
               quantB.data_ptr(), quantA.data_ptr(), result_i32.data_ptr(), cur_stream())
-    gemm_scale(batch, M, N, result_i32.data_ptr(), scaleA.data_ptr(), scaleB.data_ptr(),
-               result_fp.data_ptr(), quantA.size(0) == 1, quantB.size(0) == 1, cur_stream())
+    if scaleA is not None and scaleB is not None:
+        gemm_scale(batch, M, N, result_i32.data_ptr(), scaleA.data_ptr(), scaleB.data_ptr(),
+                   result_fp.data_ptr(), quantA.size(0) == 1, quantB.size(0) == 1, cur_stream())
+    elif scaleA is not None:
+        gemm_scale_x(batch, M, N, result_i32.data_ptr(), scaleA.data_ptr(), result_fp.data_ptr(), cur_stream())
+    else:
+        assert scaleB is not None
+        gemm_scale_y(batch, M, N, result_i32.data_ptr(), scaleB.data_ptr(), result_fp.data_ptr(), cur_stream())
     return result_fp
 
 
-class GEMMInt8(InferenceOnly):
+class GEMMInt8(torch.autograd.Function):
     @staticmethod
     def forward(ctx, A: torch.Tensor, aT: bool, B: torch.Tensor, bT: bool, fused: bool = True):
         """A: (batchA, M, K) [(batchA, K, M) if aT], B: (batchB, K, N) [(batchB, N, K) if bT]
@@ -109,29 +117,94 @@ class GEMMInt8(InferenceOnly):
             else:
                 scale_A, quantized_A = quantize_k_major(A, aT)
                 scale_B, quantized_B = quantize_k_major(B, not bT)
-            return gemm_and_scale(quantized_A, scale_A, quantized_B, scale_B, False, True, True)
+            # the int8 tensors are held as (bA, M, K) and (bB, N, K) whatever the operand layout was
+            ctx.stored = (False, True)
         else:
             scale_A = calc_scale(A, aT)
             scale_B = calc_scale(B, not bT)
             quantized_A = round_i8(A, scale_A, aT)
             quantized_B = round_i8(B, scale_B, not bT)
-        return gemm_and_scale(quantized_A, scale_A, quantized_B, scale_B, aT, bT, fused)
+            ctx.stored = (aT, bT)
+        ctx.save_for_backward(scale_A, quantized_A, scale_B, quantized_B)
+        ctx.layout = (aT, bT)
+        return gemm_and_scale(quantized_A, scale_A, quantized_B, scale_B, ctx.stored[0], ctx.stored[1], fused)
+
+    @staticmethod
+    def backward(ctx, grad_f: torch.Tensor):
+        """reference: torch/gemm.py:115-186.  grad_A = int8(grad * scale_B, row scales) x quantized_B and
+        grad_B = int8(grad * scale_A, column scales)^T x quantized_A, each dequantised by the new
+        scales only (the other operand's scales went into the gradient before rounding)."""
+        assert grad_f.is_contiguous() and grad_f.is_cuda and grad_f.dtype == torch.float16
+        scale_A, quantized_A, scale_B, quantized_B = ctx.saved_tensors
+        aT, bT = ctx.stored
+        batch, m, n = grad_f.size()
+        st = cur_stream()
+
+        scale_G_a = torch.empty((batch, m), dtype=torch.half, device=grad_f.device)
+        quant_G_a = torch.empty((batch, m, n), dtype=torch.int8, device=grad_f.device)
+        gemm_backward_round_scale(batch, m, n, grad_f.data_ptr(), scale_B.data_ptr(), quant_G_a.data_ptr(),
+                                  scale_G_a.data_ptr(), scale_B.size(0) == 1, st)
+        if aT:
+            grad_A = gemm_and_scale(quantized_B, None, quant_G_a, scale_G_a, bT, True)
+        else:
+            grad_A = gemm_and_scale(quant_G_a, scale_G_a, quantized_B, None, False, not bT)
+        del scale_G_a, quant_G_a
+
+        scale_G_b = torch.empty((batch, n), dtype=torch.half, device=grad_f.device)
+        quant_G_b = torch.empty((batch, m, n), dtype=torch.int8, device=grad_f.device)
+        gemm_backward_scale_round(batch, m, n, grad_f.data_ptr(), scale_A.data_ptr(), quant_G_b.data_ptr(),
+                                  scale_G_b.data_ptr(), scale_A.size(0) == 1, st)
+        if bT:
+            grad_B = gemm_and_scale(quant_G_b, scale_G_b, quantized_A, None, True, aT)
+        else:
+            grad_B = gemm_and_scale(quantized_A, None, quant_G_b, scale_G_b, not aT, False)
+
+        if scale_A.size(0) == 1 and grad_A.size(0) > 1:
+            grad_A = grad_A.sum(dim=0, keepdim=True)
+        if scale_B.size(0) == 1 and grad_B.size(0) > 1:
+            grad_B = grad_B.sum(dim=0, keepdim=True)
+        # back to the layout the operands came in
+        if ctx.layout[0] != aT:
+            grad_A = grad_A.transpose(1, 2).contiguous()
+        if ctx.layout[1] != bT:
+            grad_B = grad_B.transpose(1, 2).contiguous()
+        return grad_A, None, grad_B, None, None
 
 
-class GEMMFloat(InferenceOnly):
+def gemm_pth_fp16(A: torch.Tensor, aT: bool, B: torch.Tensor, bT: bool) -> torch.Tensor:
+    """reference: torch/gemm.py:189-203; operands are passed swapped to the kernel so that the
+    (M, N) result comes out row-major."""
+    M, K, N = _dims(A, B, aT, bT)
+    out = torch.empty((max(A.size(0), B.size(0)), M, N), dtype=torch.half, device=A.device)
+    gemm_fp16(N, K, M, B.size(0), A.size(0), bT, aT, B.data_ptr(), A.data_ptr(), out.data_ptr(), cur_stream())
+    return out
+
+
+class GEMMFloat(torch.autograd.Function):
     @staticmethod
     def forward(ctx, A: torch.Tensor, aT: bool, B: torch.Tensor, bT: bool):
-        """fp16 product with fp32 accumulation.  reference: torch/gemm.py:159-231 (cuBLASLt there);
-        operands are passed swapped to the kernel exactly as in :170-183 so that the (M, N)
-        result comes out row-major."""
+        """fp16 product with fp32 accumulation.  reference: torch/gemm.py:205-217 (cuBLASLt there)."""
         assert A.is_cuda and B.is_cuda and A.device == B.device
         assert A.is_contiguous() and B.is_contiguous()
         assert A.dtype == torch.half and B.dtype == torch.half
-        M, K, N = _dims(A, B, aT, bT)
-        batch = max(A.size(0), B.size(0))
-        out = torch.empty((batch, M, N), dtype=torch.half, device=A.device)
-        gemm_fp16(N, K, M, B.size(0), A.size(0), bT, aT, B.data_ptr(), A.data_ptr(), out.data_ptr(), cur_stream())
-        return out
+        ctx.save_for_backward(A, B)
+        ctx.aT = aT
+        ctx.bT = bT
+        return gemm_pth_fp16(A, aT, B, bT)
+
+    @staticmethod
+    def backward(ctx, grad_f):
+        """reference: torch/gemm.py:219-239"""
+        assert grad_f.is_cuda and grad_f.is_contiguous() and grad_f.dtype == torch.float16
+        aT, bT = ctx.aT, ctx.bT
+        A, B = ctx.saved_tensors
+        grad_A = gemm_pth_fp16(B, bT, grad_f, True) if aT else gemm_pth_fp16(grad_f, False, B, not bT)
+        grad_B = gemm_pth_fp16(grad_f, True, A, aT) if bT else gemm_pth_fp16(A, not aT, grad_f, False)
+        if A.size(0) == 1 and grad_A.size(0) > 1:
+            grad_A = grad_A.sum(dim=0, keepdim=True)
+        if B.size(0) == 1 and grad_B.size(0) > 1:
+            grad_B = grad_B.sum(dim=0, keepdim=True)
+        return grad_A, None, grad_B, None
 
 
 def bmm(A: torch.Tensor, aT: bool, B: torch.Tensor, bT: bool, int8: bool = False, fused: bool = True) -> torch.Tensor:

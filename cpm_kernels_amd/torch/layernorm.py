@@ -1,12 +1,13 @@
 """LayerNorm over dim 1 of (batch, hidden, seq) with the interface of
-cpm_kernels/torch/layernorm.py (forward only)."""
+cpm_kernels/torch/layernorm.py."""
 import torch
 from ..kernels import layernorm_forward, layernorm_inplace_forward, layernorm_affine_forward, \
-    arith_ln_mul_add, arith_ln_mul
-from ._common import cur_stream, check_half, InferenceOnly
+    layernorm_forward_v, layernorm_forward_mv, layernorm_backward_v, layernorm_backward_mv, \
+    arith_ln_mul_add, arith_ln_mul, arith_ln_add_backward, arith_ln_mul_backward
+from ._common import cur_stream, check_half
 
 
-class OpLayerNorm(InferenceOnly):
+class OpLayerNorm(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x: torch.Tensor, eps: float, weight: torch.Tensor, bias, fused: bool = True):
         """bias given: mean-subtracting norm then y*weight+bias (OpLayerNormMean,
@@ -16,6 +17,9 @@ class OpLayerNorm(InferenceOnly):
         b, n, m = x.size()
         out = torch.empty((b, n, m), device=x.device, dtype=torch.float16)
         rd_mean = bias is not None
+        ctx.save_for_backward(x, weight)
+        ctx.eps = eps
+        ctx.rd_mean = rd_mean
         if fused:
             layernorm_affine_forward(b, n, m, x.data_ptr(), weight.data_ptr(),
                                      bias.data_ptr() if rd_mean else None, out.data_ptr(), eps, rd_mean,
@@ -27,6 +31,38 @@ class OpLayerNorm(InferenceOnly):
         else:
             arith_ln_mul(b, n, m, out.data_ptr(), weight.data_ptr(), out.data_ptr(), cur_stream())
         return out
+
+    @staticmethod
+    def backward(ctx, grad_output: torch.Tensor):
+        """The reference's sequence (torch/layernorm.py:31-86, 113-156): the normalised tensor and its
+        statistics are recomputed, the affine gradients are two channel sums, and the input
+        gradient is the norm's backward kernel applied to grad_output * weight."""
+        check_half(grad_output, 3)
+        x, weight = ctx.saved_tensors
+        b, n, m = x.size()
+        st = cur_stream()
+        half = dict(device=x.device, dtype=torch.float16)
+        layer_out = torch.empty((b, n, m), **half)
+        var = torch.empty((b, m), **half)
+        mean = torch.empty((b, m), **half) if ctx.rd_mean else None
+        if ctx.rd_mean:
+            layernorm_forward_mv(b, n, m, x.data_ptr(), layer_out.data_ptr(), mean.data_ptr(), var.data_ptr(), ctx.eps, st)
+        else:
+            layernorm_forward_v(b, n, m, x.data_ptr(), layer_out.data_ptr(), var.data_ptr(), ctx.eps, st)
+        grad_bias = None
+        if ctx.rd_mean:
+            grad_bias = torch.empty((n,), **half)
+            arith_ln_add_backward(b, n, m, grad_output.data_ptr(), grad_bias.data_ptr(), st)
+        grad_weight = torch.empty((n,), **half)
+        arith_ln_mul_backward(b, n, m, layer_out.data_ptr(), grad_output.data_ptr(), grad_weight.data_ptr(), st)
+        grad_x = layer_out                     # its contents are no longer needed
+        arith_ln_mul(b, n, m, grad_output.data_ptr(), weight.data_ptr(), grad_x.data_ptr(), st)
+        grad = torch.empty_like(x)
+        if ctx.rd_mean:
+            layernorm_backward_mv(b, n, m, x.data_ptr(), grad_x.data_ptr(), mean.data_ptr(), var.data_ptr(), grad.data_ptr(), st)
+        else:
+            layernorm_backward_v(b, n, m, x.data_ptr(), grad_x.data_ptr(), var.data_ptr(), grad.data_ptr(), st)
+        return grad, None, grad_weight, grad_bias, None
 
 
 class LayerNorm(torch.nn.Module):

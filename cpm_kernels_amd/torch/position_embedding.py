@@ -1,13 +1,15 @@
 """T5-style relative position bias with the interface of
-cpm_kernels/torch/position_embedding.py (forward only)."""
+cpm_kernels/torch/position_embedding.py ."""
 import math
 import torch
 import torch.nn.functional as F
-from ..kernels import position_embedding_init, position_embedding_forward
-from ._common import cur_stream, check_half, InferenceOnly
+from ..kernels import position_embedding_init, position_embedding_forward, position_embedding_backward
+from ._common import cur_stream, check_half
 
 
-class OpPositionEmbedding(InferenceOnly):
+class OpPositionEmbedding(torch.autograd.Function):
+    """reference: torch/position_embedding.py:6-55"""
+
     @staticmethod
     def forward(ctx, query_len, key_len, num_buckets, max_distance, num_heads, weight: torch.Tensor,
                 bidirectional: bool):
@@ -18,7 +20,19 @@ class OpPositionEmbedding(InferenceOnly):
         out = torch.empty((num_heads, key_len, query_len), device=device, dtype=torch.float16)
         position_embedding_forward(query_len, key_len, num_buckets, max_distance, num_heads, mapping.data_ptr(),
                                    weight.data_ptr(), out.data_ptr(), bidirectional, cur_stream())
+        ctx.save_for_backward(mapping)
+        ctx.input_args = (query_len, key_len, num_buckets, max_distance, num_heads, bidirectional)
         return out
+
+    @staticmethod
+    def backward(ctx, grad_output: torch.Tensor):
+        check_half(grad_output)
+        query_len, key_len, num_buckets, max_distance, num_heads, bidirectional = ctx.input_args
+        mapping = ctx.saved_tensors[0]
+        grad = torch.empty((num_heads, num_buckets), device=grad_output.device, dtype=torch.float16)
+        position_embedding_backward(query_len, key_len, num_buckets, max_distance, num_heads, mapping.data_ptr(),
+                                    grad_output.data_ptr(), grad.data_ptr(), bidirectional, cur_stream())
+        return None, None, None, None, None, grad, None
 
 
 class PositionEmbedding(torch.nn.Module):
