@@ -164,13 +164,11 @@ def test_mask_and_arith_wrappers(gpu):
     assert_bits_equal(to_np(ct.ln_mul(x.cuda(), al.cuda())), (x.double() * al.double()[None, :, None]).half().numpy(), "ln_mul")
 
 
-def test_ffn_block_composition(gpu):
-    """CPM-2-style FFN block at reduced size: layernorm -> int8 GEMM -> gelu -> int8 GEMM -> residual,
-    through the wrappers in the reference's native (batch, hidden, seq) layout, against the fp32
-    formulations chained on the CPU.  The tolerance is the int8 quantisation noise of two GEMMs."""
-    _name("ffn block")
+def _ffn_block(b, d, dff, s, check):
+    """layernorm -> int8 GEMM -> gelu -> int8 GEMM -> residual through the wrappers in the
+    reference's native (batch, hidden, seq) layout; the fp32 formulations chained on the CPU for
+    the batch entries in `check`.  Returns (device output, reference) restricted to `check`."""
     g = torch.Generator().manual_seed(1004)
-    b, d, dff, s = 2, 256, 640, 64
     x = torch.randn(b, d, s, generator=g).half()
     W1 = (torch.randn(1, dff, d, generator=g) * 0.02).half()
     W2 = (torch.randn(1, d, dff, generator=g) * 0.02).half()
@@ -185,7 +183,8 @@ def test_ffn_block_composition(gpu):
     h = ct.bmm(W2.cuda(), False, h, False, int8=True)          # (b, d, s)
     out = ct.element_add(h, xd)
     # CPU chain in fp32 with the same quantisation axes (weights along K = last dim, activations along K = dim 1)
-    r = F.layernorm_dim1(x, ln.weight.cpu(), ln.bias.cpu(), 1e-5).float()
+    xc = x[check]
+    r = F.layernorm_dim1(xc, ln.weight.cpu(), ln.bias.cpu(), 1e-5).float()
     def qmm(W, act):   # W (1, N, K), act (b, K, S)
         Wq = F.fake_quant_rows(W.float())
         aq = F.fake_quant_rows(act.transpose(1, 2)).transpose(1, 2)      # per (b, s) column, along K
@@ -193,26 +192,43 @@ def test_ffn_block_composition(gpu):
     r = qmm(W1, r).half().float()
     r = F.gelu_tanh(r).half().float()
     r = qmm(W2, r)
-    ref = (r + x.float())
-    got = to_np(out).astype(np.float32)
-    err = np.abs(got - ref.numpy())
+    ref = (r + xc.float())
+    return to_np(out[check]).astype(np.float32), ref.numpy()
+
+
+def test_ffn_block_composition(gpu):
+    """CPM-2-style FFN block at reduced size against the fp32 formulations.  The tolerance is the
+    int8 quantisation noise of two GEMMs."""
+    _name("ffn block")
+    got, ref = _ffn_block(2, 256, 640, 64, [0, 1])
+    err = np.abs(got - ref)
     assert err.max() < 3e-2 and err.mean() < 3e-3, (err.max(), err.mean())
 
 
-def test_transformer_layer_composition(gpu):
-    """A CPM-2-shaped transformer layer at reduced size through the wrappers only, in the
-    reference's (batch, hidden, seq) layout: LayerNorm -> int8 Q/K/V projections -> fp16 scores
-    (B*H, len_k, len_q) + T5 relative bias -> padding mask (-inf on padded queries) -> softmax
-    over dim 1 -> fp16 PV -> int8 output projection -> residual -> LayerNorm -> int8 FFN with
-    gelu -> residual; against the same chain of fp32 formulations on the CPU.  The tolerance is
-    the int8 quantisation noise of four chained quantised products."""
-    _name("transformer layer")
+def test_ffn_block_full_size(gpu):
+    """The same block at its full size (tokens 8 x 512, 4096 -> 10240 -> 4096); two of the eight
+    batch entries are followed on the CPU (entries are independent of each other).  With K = 4096
+    and 10240 the quantisation noise of the second product is about 1 % of its output's rms
+    (~0.5), hence the absolute bars."""
+    _name("ffn block, full size")
+    got, ref = _ffn_block(8, 4096, 10240, 512, [0, 5])
+    assert np.isfinite(got).all()
+    err = np.abs(got - ref)
+    rms = float(np.sqrt(np.mean(ref ** 2)))
+    print("ffn full size: max err %.4g mean err %.4g output rms %.4g" % (err.max(), err.mean(), rms), flush=True)
+    assert err.mean() < 1.5e-2 * rms and err.max() < 0.15 * rms, (err.max(), err.mean(), rms)
+
+
+def _transformer_layer(b, d, H, dh, dff, s, lens, check, wstd):
+    """LayerNorm -> int8 Q/K/V projections -> fp16 scores (B*H, len_k, len_q) + T5 relative bias ->
+    padding mask (-inf on padded queries) -> softmax over dim 1 -> fp16 PV -> int8 output
+    projection -> residual -> LayerNorm -> int8 FFN with gelu -> residual, through the wrappers
+    only in the reference's (batch, hidden, seq) layout, and the same chain of fp32 formulations
+    on the CPU for the batch entries in `check`.  Returns (device output[check], reference, probs)."""
     g = torch.Generator().manual_seed(1005)
-    b, d, H, dh, dff, s = 2, 256, 4, 64, 640, 96
     x = torch.randn(b, d, s, generator=g).half()
-    W = {k: (torch.randn(1, o, i, generator=g) * 0.04).half()
+    W = {k: (torch.randn(1, o, i, generator=g) * wstd).half()
          for k, (o, i) in {"q": (d, d), "k": (d, d), "v": (d, d), "o": (d, d), "w1": (dff, d), "w2": (d, dff)}.items()}
-    lens = torch.tensor([s, s - 29])
     pad = (torch.arange(s)[None, :] < lens[:, None])                     # (b, s) True = real token
     ln1 = ct.LayerNorm(d, bias=True).half().cuda(); ln2 = ct.LayerNorm(d, bias=True).half().cuda()
     pe = ct.PositionEmbedding(H, 32, 128, True).half().cuda()
@@ -243,6 +259,11 @@ def test_transformer_layer_composition(gpu):
         # formulation, 0 in the kernels (NaN -> 0 in the rounding)
         aq = torch.nan_to_num(F.fake_quant_rows(act.float().transpose(1, 2)), nan=0.0).transpose(1, 2)
         return torch.matmul(F.fake_quant_rows(Wm.float()), aq)
+    got = to_np(out[check]).astype(np.float32)
+    probs_checked = probs.view(b, H, s, s)[check].cpu()
+    del q, k, v, scores, probs, ctx, y, h2, f, out, h
+    torch.cuda.empty_cache()
+    x, pad, b = x[check], pad[check], len(check)
     r = F.layernorm_dim1(x, ln1.weight.cpu(), ln1.bias.cpu(), 1e-5)
     rq, rk, rv = (qmm(W[n], r).half().view(b * H, dh, s).float() for n in "qkv")
     sc = (torch.matmul(rk.transpose(1, 2), rq).half().float() / dh ** 0.5).half().float()
@@ -257,9 +278,39 @@ def test_transformer_layer_composition(gpu):
     rf = F.gelu_tanh(qmm(W["w1"], r2).half()).float()
     ref = (qmm(W["w2"], rf).half().float() + ry.float())
 
-    got = to_np(out).astype(np.float32)
-    err = np.abs(got - ref.numpy())
+    return got, ref.numpy(), probs_checked
+
+
+def test_transformer_layer_composition(gpu):
+    """A CPM-2-shaped transformer layer at reduced size.  The tolerance is the int8 quantisation
+    noise of four chained quantised products."""
+    _name("transformer layer")
+    s = 96
+    got, ref, probs = _transformer_layer(2, 256, 4, 64, 640, s, torch.tensor([s, s - 29]), [0, 1], 0.04)
+    err = np.abs(got - ref)
     assert np.isfinite(got).all()
     assert err.max() < 6e-2 and err.mean() < 4e-3, (err.max(), err.mean())
     # padded query positions received exactly zero attention
-    assert float(probs.view(b, H, s, s)[1, :, :, s - 29:].abs().max()) == 0.0
+    assert float(probs[1, :, :, s - 29:].abs().max()) == 0.0
+
+
+def test_transformer_layer_full_size(gpu):
+    """The layer at its full size: d_model 4096, 64 heads x 64, d_ff 10240, batch 16, seq 1024,
+    lengths drawn from [512, 1024].  The device runs all 16 entries; entry 0 and the shortest
+    entry are followed on the CPU (entries are independent).  Bars relative to the output's rms."""
+    _name("transformer layer, full size")
+    g = torch.Generator().manual_seed(77)
+    lens = torch.randint(512, 1025, (16,), generator=g)
+    short = int(torch.argmin(lens))
+    check = sorted({0, short})
+    got, ref, probs = _transformer_layer(16, 4096, 64, 64, 10240, 1024, lens, check, 0.02)
+    assert np.isfinite(got).all()
+    err = np.abs(got - ref)
+    rms = float(np.sqrt(np.mean(ref ** 2)))
+    print("layer full size: max err %.4g mean err %.4g output rms %.4g" % (err.max(), err.mean(), rms), flush=True)
+    assert err.mean() < 1.5e-2 * rms and err.max() < 0.25 * rms, (err.max(), err.mean(), rms)
+    i = check.index(short)
+    assert float(probs[i, :, :, int(lens[short]):].abs().max()) == 0.0     # padded queries: exactly zero attention
+    # every real query's attention sums to one over the keys
+    sums = probs[i, :, :, :int(lens[short])].float().sum(1)
+    assert float((sums - 1).abs().max()) < 2e-3
