@@ -258,8 +258,8 @@ __device__ __forceinline__ GemmItem gemm_item(uint32_t L, const DmaArgs& da) {
 // reads).  Either way the loop body has no branches, which lets the compiler keep the
 // accumulators in place.  Returns true if the next tile's first two slabs are on their way.
 template <int WR, int WC, int TR, int TC, int BKB, int EPI>
-__device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, uint32_t lds_base, const GemmItem cur_item,
-                                              const GemmItem nxt_item, const bool have_slabs) {
+__device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, int8_t* stg, uint32_t lds_base,
+                                              const GemmItem cur_item, const GemmItem nxt_item, const bool have_slabs) {
     constexpr bool FUSED = EPI == kEpiDequant, F16 = EPI == kEpiF16;
     using acc_t = std::conditional_t<F16, float16_tv, int16_tv>;
     constexpr int KS = BKB / 32, CPR = BKB / 16;
@@ -435,35 +435,55 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, u
     if (!ahead) wait_vmcnt<0>();         // drain the clamped loads before the ring is reused
 
     const int64_t obase = (int64_t)b * a.n * a.m;
+    // Results leave through a 4 KB strip of LDS per wave: a lane holds 4-column pieces of ONE
+    // output row, so storing straight from the accumulators would touch 32 different rows
+    // with 8 or 16 bytes each per instruction.  Written to the strip as 32 rows x RB bytes
+    // and read back 16 bytes per lane, every store instruction covers whole contiguous rows
+    // of the chunk (RB = 128 bytes: eight lanes per 128-byte line).
+    constexpr int ESZ = EPI == kEpiInt32 ? 4 : 2;
+    constexpr int CT = EPI == kEpiInt32 ? 1 : TC;       // MFMA tiles side by side in one chunk
+    constexpr int NCH = EPI == kEpiInt32 ? TC : 1;      // chunks per block of 32 rows
+    constexpr int RB = CT * 32 * ESZ, PPR = RB / 16, RPW2 = 256 / RB, PASSES = PPR / 2, RPP = 64 / PPR;
+    // 16-byte piece p of strip row r sits at piece slot p ^ ((r / RPW2) % PPR): reads are conflict free
+    auto slot = [](int r, int p) __attribute__((always_inline)) { return (p ^ ((r / RPW2) & (PPR - 1))) << 4; };
 #pragma unroll
     for (int i = 0; i < TR; ++i) {
-        const int32_t row = j0 + wr * TR * 32 + i * 32 + lrow;
         float sx = 0.0f;
         if (FUSED) sx = (float)sxh[i];
 #pragma unroll
-        for (int j = 0; j < TC; ++j) {
+        for (int c = 0; c < NCH; ++c) {
+            if constexpr (EPI == kEpiInt32) {
 #pragma unroll
-            for (int g4 = 0; g4 < 4; ++g4) {
-                const int32_t col = i0 + wc * TC * 32 + j * 32 + g4 * 8 + lk * 4;
-                if (row < a.n && col < a.m) {      // m % 4 == 0: the four columns are in or out together
-                    const int64_t o = obase + (int64_t)row * a.m + col;
-                    if constexpr (F16) {
-                        half4_t h;
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) h[e] = (half_t)acc[i][j][g4 * 4 + e];
-                        *reinterpret_cast<half4_t*>(reinterpret_cast<half_t*>(a.out) + o) = h;
-                    } else if constexpr (FUSED) {
-                        const half4_t sy = syh[j][g4];
-                        half4_t h;
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) h[e] = dequant(acc[i][j][g4 * 4 + e], sx, (float)sy[e]);
-                        *reinterpret_cast<half4_t*>(reinterpret_cast<half_t*>(a.out) + o) = h;
-                    } else {
-                        const int4_t v = {(int32_t)acc[i][j][g4 * 4], (int32_t)acc[i][j][g4 * 4 + 1],
-                                          (int32_t)acc[i][j][g4 * 4 + 2], (int32_t)acc[i][j][g4 * 4 + 3]};
-                        *reinterpret_cast<int4_t*>(reinterpret_cast<int32_t*>(a.out) + o) = v;
-                    }
+                for (int g4 = 0; g4 < 4; ++g4) {
+                    const int4_t v = {(int32_t)acc[i][c][g4 * 4], (int32_t)acc[i][c][g4 * 4 + 1],
+                                      (int32_t)acc[i][c][g4 * 4 + 2], (int32_t)acc[i][c][g4 * 4 + 3]};
+                    *reinterpret_cast<int4_t*>(stg + lrow * RB + slot(lrow, g4 * 2 + lk)) = v;
                 }
+            } else {
+#pragma unroll
+                for (int j = 0; j < TC; ++j)
+#pragma unroll
+                    for (int g4 = 0; g4 < 4; ++g4) {
+                        half4_t h;
+                        if constexpr (F16) {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) h[e] = (half_t)acc[i][j][g4 * 4 + e];
+                        } else {
+                            const half4_t sy = syh[j][g4];
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) h[e] = dequant(acc[i][j][g4 * 4 + e], sx, (float)sy[e]);
+                        }
+                        *reinterpret_cast<half4_t*>(stg + lrow * RB + slot(lrow, j * 4 + g4) + lk * 8) = h;
+                    }
+            }
+#pragma unroll
+            for (int ps = 0; ps < PASSES; ++ps) {
+                const int R = ps * RPP + lane / PPR, pc = lane % PPR;
+                const int4_t v = *reinterpret_cast<const int4_t*>(stg + R * RB + slot(R, pc));
+                const int32_t row = j0 + wr * TR * 32 + i * 32 + R;
+                const int32_t col = i0 + wc * TC * 32 + c * 32 + pc * (16 / ESZ);
+                if (row < a.n && col < a.m)
+                    *reinterpret_cast<int4_t*>(reinterpret_cast<int8_t*>(a.out) + (obase + (int64_t)row * a.m + col) * ESZ) = v;
             }
         }
     }
@@ -480,6 +500,8 @@ __global__ __launch_bounds__(WR* WC * 64) void k_gemm_dma(DmaArgs da) {
     constexpr int BR = WR * TR * 32, BC = WC * TC * 32;
     extern __shared__ __attribute__((aligned(16))) int8_t smem[];
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) int8_t*)smem;
+    // behind the two-stage operand ring: one 4 KB strip per wave for the output rows on their way out
+    int8_t* stg = smem + 2 * (BR + BC) * BKB + (threadIdx.x >> 6) * 4096;
     const uint32_t G = gridDim.x;
     const uint32_t w = (G % 8 == 0) ? (blockIdx.x % 8) * (G / 8) + blockIdx.x / 8 : blockIdx.x;
     bool have_slabs = false;
@@ -488,9 +510,9 @@ __global__ __launch_bounds__(WR* WC * 64) void k_gemm_dma(DmaArgs da) {
         const GemmItem nxt = gemm_item<BR, BC>(L + G, da);
         if (HALVES && cur.half) {
             if constexpr (HALVES)
-                have_slabs = gemm_dma_tile<WR, WC, TR, TC / 2, BKB, EPI>(da.g, smem, lds_base, cur, nxt, have_slabs);
+                have_slabs = gemm_dma_tile<WR, WC, TR, TC / 2, BKB, EPI>(da.g, smem, stg, lds_base, cur, nxt, have_slabs);
         } else {
-            have_slabs = gemm_dma_tile<WR, WC, TR, TC, BKB, EPI>(da.g, smem, lds_base, cur, nxt, have_slabs);
+            have_slabs = gemm_dma_tile<WR, WC, TR, TC, BKB, EPI>(da.g, smem, stg, lds_base, cur, nxt, have_slabs);
         }
         cur = nxt;
     }
@@ -598,7 +620,7 @@ static int launch_kmajor(GemmArgs& a, int batch, hipStream_t st) {
 template <int WR, int WC, int TR, int TC, int BKB, int EPI, bool HALVES>
 static int launch_dma_kernel(const DmaArgs& da, unsigned grid, hipStream_t st) {
     constexpr int BR = WR * TR * 32, BC = WC * TC * 32;
-    constexpr int smem = 2 * (BR + BC) * BKB;
+    constexpr int smem = 2 * (BR + BC) * BKB + WR * WC * 4096;      // operand ring + output strips
     auto kern = k_gemm_dma<WR, WC, TR, TC, BKB, EPI, HALVES>;
     static bool attr_set[64] = {false};       // dynamic LDS above 64 KB must be enabled per device
     int dev = 0;
@@ -654,9 +676,11 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
     a.strideQ = batchA == 1 ? 0 : (int64_t)m * k;
     a.n = n; a.m = m; a.k = k; a.bc_row = bcr; a.bc_col = bcc;
     a.tiles_r = a.tiles_c = 0;
+    // the tile kernel stores 16-byte pieces of output rows
+    const bool wide = aligned16(out) && (!FUSED || m % 8 == 0);
     const bool p_kmajor = !bT, q_kmajor = aT != 0;
     const bool fast = p_kmajor && q_kmajor && k > 0 && (k % 16 == 0) && aligned16(A) && aligned16(B);
-    if (fast && (k % 128 == 0) && (int64_t)n * k < (1ll << 32) && (int64_t)m * k < (1ll << 32)) {
+    if (fast && wide && (k % 128 == 0) && (int64_t)n * k < (1ll << 32) && (int64_t)m * k < (1ll << 32)) {
         // 256x256 tiles when they give most compute units a tile, else 128x128
         const int64_t big = ceil_div(n, 256) * ceil_div(m, 256) * batch;
         constexpr int EPI = FUSED ? kEpiDequant : kEpiInt32;
@@ -757,8 +781,9 @@ static int gemm_f16_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, in
     a.strideQ = batchA == 1 ? 0 : (int64_t)m * k * 2;
     a.n = n; a.m = m; a.k = k * 2; a.bc_row = 0; a.bc_col = 0;
     a.tiles_r = a.tiles_c = 0;
+    const bool wide = aligned16(out) && m % 8 == 0;       // the tile kernel stores 16-byte pieces of output rows
     const bool p_kmajor = !bT, q_kmajor = aT != 0;
-    if (p_kmajor && q_kmajor && k > 0 && (k % 64 == 0) && (m % 4 == 0) && aligned16(A) && aligned16(B) &&
+    if (p_kmajor && q_kmajor && wide && k > 0 && (k % 64 == 0) && aligned16(A) && aligned16(B) &&
         (int64_t)n * k * 2 < (1ll << 32) && (int64_t)m * k * 2 < (1ll << 32)) {
         const int64_t big = ceil_div(n, 256) * ceil_div(m, 256) * batch;
         if (big * 4 >= compute_units() * 3) return launch_dma<CPMK_GEMM_BIG, kEpiF16>(a, batch, st);
