@@ -22,14 +22,12 @@ __global__ __launch_bounds__(NT) void k_col_quantize_team(int32_t n, int32_t m, 
     constexpr int LPR = 8, R = 8, COLS = 64, ROWS = NT / LPR * R;
     __shared__ float lds[(NT / 64 + 1) * COLS];
     __shared__ float tot[COLS];
-    __shared__ int failed;
     const int tid = threadIdx.x, cg = tid % LPR, rg = tid / LPR;
     const uint32_t part = blockIdx.x % parts, team = blockIdx.x / parts;
     const uint32_t b = team / tiles_per_batch, ct = team - b * tiles_per_batch;
     const int32_t col0 = ct * COLS + cg * 8;
     const int32_t row0 = part * ROWS + rg * 8;           // this lane's first row
     const int64_t boff = (int64_t)b * n * m;
-    if (tid == 0) failed = 0;
 
     half8_t v[R];
 #pragma unroll
@@ -63,7 +61,6 @@ __global__ __launch_bounds__(NT) void k_col_quantize_team(int32_t n, int32_t m, 
                 M = fmaxf(M, x);
             }
             tot[tid] = ok ? M : __builtin_nanf("");
-            if (!ok) failed = 1;
         }
         __syncthreads();
 #pragma unroll

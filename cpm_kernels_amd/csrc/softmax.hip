@@ -84,7 +84,6 @@ __global__ __launch_bounds__(NT) void k_softmax_team(int32_t n, int32_t m, int32
     static_assert(T::COLS * 2 == kXchVals, "slot layout");
     __shared__ float lds[(T::NW + 1) * T::COLS];
     __shared__ float tot[kXchVals];
-    __shared__ int failed;
     const int tid = threadIdx.x;
     const uint32_t part = blockIdx.x % parts, team = blockIdx.x / parts;
     const uint32_t b = team / tiles_per_batch, ct = team - b * tiles_per_batch;
@@ -92,7 +91,6 @@ __global__ __launch_bounds__(NT) void k_softmax_team(int32_t n, int32_t m, int32
     const int32_t own0 = part * T::ROWS;
     const int32_t own_n = min(T::ROWS, n - own0);
     const int64_t boff = (int64_t)b * n * m + (int64_t)own0 * m;
-    if (tid == 0) failed = 0;
 
     half8_t v[R];
     coltile_load<NT, LPR, R>(v, inp + boff, own_n, m, col0, (half_t)(-__builtin_inff()));
@@ -159,7 +157,6 @@ __global__ __launch_bounds__(NT) void k_softmax_team(int32_t n, int32_t m, int32
             if (q < parts) S += sp[q] * __builtin_amdgcn_exp2f(mp[q] - M);
         tot[tid] = M;
         tot[T::COLS + tid] = ok ? 1.0f / (S + 1e-10f) : __builtin_nanf("");
-        if (!ok) failed = 1;
     }
     __syncthreads();
     const int cg = tid % LPR;
