@@ -33,6 +33,10 @@ M, K, N = 4096, 4096, 10240  # north-star GEMM
 # read from inside this process): `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` over
 # `python3 bench.py --no-cpu --only <workload>`, each counter scaled by what it reads for the
 # 256 MiB device copy of `--only calib` (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000 on MI355X).
+# MFMA pipe busy cycles / kernel cycles of the fused GEMM kernel from SQ_VALU_MFMA_BUSY_CYCLES and
+# SQ_BUSY_CYCLES (same offline procedure; profiles/gemm_mfma_utilisation.txt).
+MFMA_BUSY_FRAC = 0.661
+
 TRAFFIC_BYTES = {
     "gemm_fused": 366.2e6,     # 278.6 MB fetched (operand tiles re-read across the 8 L2s) + 87.6 MB written
     "gemv": 43.9e6,
@@ -180,6 +184,7 @@ def main():
                     "ops": "int8 multiply-accumulates counted as 2 ops (TOP/s)",
                     "frac": round(tops / PEAK_INT8_TOPS, 4), "avg_kernel_us": round(ms * 1e3, 2),
                     "traffic": TRAFFIC_BYTES["gemm_fused"], "traffic_unit": "bytes per launch (HBM fetch + write counters)",
+                    "mfma_busy_frac_of_cycles": MFMA_BUSY_FRAC,
                     "algorithmic_bytes": M * K + N * K + 2 * M * N}
         out32 = torch.empty((1, M, N), dtype=torch.int32, device=dev)
 
