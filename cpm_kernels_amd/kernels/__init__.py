@@ -1,5 +1,5 @@
-"""Same export list as cpm_kernels/kernels/__init__.py:1-14 of the reference, plus the three
-fused launchers this build adds (gemm_int8_scale, gemm_quantize, gemm_quantize_cols, gemm_quantize_pair,
+"""Same export list as cpm_kernels/kernels/__init__.py:1-14 of the reference, plus the fused
+launchers this build adds (gemm_int8_scale, gemm_quantize, gemm_quantize_cols, gemm_quantize_pair,
 layernorm_affine_forward)."""
 from .embedding import embedding_forward, embedding_backward_stage1, embedding_backward_stage2, embedding_step
 from .gelu import gelu_forward, gelu_backward, gelu_inplace_forward

@@ -19,14 +19,3 @@ def _stream(stream):
     if isinstance(stream, ctypes.c_void_p):
         return stream
     return ctypes.c_void_p(stream)
-
-
-def not_on_path(name: str, where: str):
-    """Names the reference exports that are outside the int8 inference path: calling one
-    raises instead of silently doing nothing."""
-    def stub(*args, **kwargs):
-        raise NotImplementedError(
-            "%s (%s) is outside the int8 quantized-GEMM inference path implemented by "
-            "cpm_kernels_amd" % (name, where))
-    stub.__name__ = name
-    return stub

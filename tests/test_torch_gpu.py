@@ -18,7 +18,7 @@ pytestmark = pytest.mark.gpu
 
 @pytest.fixture(autouse=True)
 def _inference_only():
-    """The wrappers are forward-only; run every test without autograd bookkeeping."""
+    """Forward results only in this file (gradients: test_torch_backward_gpu.py); no autograd bookkeeping."""
     with torch.no_grad():
         yield
 
