@@ -246,18 +246,18 @@ __device__ __forceinline__ GemmItem gemm_item(uint32_t L, const DmaArgs& da) {
 }
 
 // One output tile of BR x BC = (WR*TR*32) x (WC*TC*32), K slab = BKB bytes.
-// Pipeline per K slab `it` (stage cur = it & 1):
+// NST-stage ring; pipeline per K slab `it` (stage cur = it % NST, slabs it+1 .. it+NST-1 in flight):
 //   k-steps 0 .. KS-2 : MFMAs of step s while the fragments of step s+1 are read from LDS
-//   s_waitcnt vmcnt(0); barrier     -> slab it+1 has landed in stage nxt for every wave and
+//   s_waitcnt vmcnt((NST-2)*CNT); barrier -> slab it+1 has landed in stage nxt for every wave and
 //                                      nobody reads stage cur any more
 //   k-step KS-1       : MFMAs while the step-0 fragments of slab it+1 are read and the DMA of
-//                       slab it+2 is issued into stage cur
+//                       slab it+NST is issued into stage cur
 // Past the end of K the DMA fetches slabs 0 and 1 of the NEXT tile of this workgroup (when it
 // has the same shape), so that tile starts with its operands already in LDS and the loads
 // overlap this tile's stores; otherwise the slab index is clamped (a redundant load nobody
 // reads).  Either way the loop body has no branches, which lets the compiler keep the
 // accumulators in place.  Returns true if the next tile's first two slabs are on their way.
-template <int WR, int WC, int TR, int TC, int BKB, int EPI>
+template <int WR, int WC, int TR, int TC, int BKB, int EPI, int NST>
 __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, int8_t* stg, uint32_t lds_base,
                                               const GemmItem cur_item, const GemmItem nxt_item, const bool have_slabs) {
     constexpr bool FUSED = EPI == kEpiDequant, F16 = EPI == kEpiF16;
@@ -290,12 +290,14 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
         const int r = wc * TC * 32 + j * 32 + lrow;
         offQ[j] = BR * BKB + r * BKB + ((lk ^ swz(r)) << 4);
     }
+    // without slabs on their way the waits below count only loads: let the previous tile's stores finish first
+    if (!have_slabs) wait_vmcnt<0>();
     const uint32_t b = cur_item.b;
     const int32_t j0 = cur_item.j0, i0 = cur_item.i0;
     const int8_t* Pb = a.P + (int64_t)b * a.strideP;
     const int8_t* Qb = a.Q + (int64_t)b * a.strideQ;
     // the next tile is fetched ahead only if its LDS layout is this one's and the ring parity works out
-    const bool ahead = nxt_item.valid && nxt_item.half == cur_item.half && nk >= 2 && (nk & 1) == 0;
+    const bool ahead = nxt_item.valid && nxt_item.half == cur_item.half && nk >= NST && nk % NST == 0;
     const int8_t* Pn = a.P + (int64_t)nxt_item.b * a.strideP;
     const int8_t* Qn = a.Q + (int64_t)nxt_item.b * a.strideQ;
 
@@ -389,12 +391,14 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
 
     if (!have_slabs) {
         __syncthreads();                 // every wave is done with the ring of the previous tile
-        static_for<0, CNT>([&](auto dc) __attribute__((always_inline)) { dma1(dc, 0, false, 0); });
-        wait_vmcnt<0>();
+        static_for<0, NST>([&](auto sc) __attribute__((always_inline)) {
+            constexpr int st = decltype(sc)::value;
+            static_for<0, CNT>([&](auto dc) __attribute__((always_inline)) { dma1(dc, min(st, nk - 1), false, st); });
+        });
+        wait_vmcnt<(NST - 1) * CNT>();   // slab 0 (and the scale loads issued before it) has landed
         __syncthreads();
-        static_for<0, CNT>([&](auto dc) __attribute__((always_inline)) { dma1(dc, min(1, nk - 1), false, 1); });
     } else {
-        wait_vmcnt<0>();                 // slabs 0 and 1 were requested during the previous tile
+        wait_vmcnt<0>();                 // slabs 0 .. NST-1 were requested during the previous tile; its stores drain too
         __syncthreads();
     }
     if (FUSED) {     // pin the scale loads above the K loop (the waits just above cover them)
@@ -407,8 +411,9 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
     }
     static_for<0, TR + TC>([&](auto xc) __attribute__((always_inline)) { lfrag1(xc, C0{}, 0, 0); });
 
+    int cur = 0;
     for (int it = 0; it < nk; ++it) {
-        const int cur = it & 1, nxt = cur ^ 1;
+        const int nxt = cur + 1 == NST ? 0 : cur + 1;
         static_for<0, KS - 1>([&](auto ksc) __attribute__((always_inline)) {
             constexpr int ks = decltype(ksc)::value;
             kstep(std::integral_constant<int, (ks & 1)>{},
@@ -418,11 +423,11 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
                   std::integral_constant<int, TR + TC>{});
         });
         __builtin_amdgcn_sched_barrier(0);
-        wait_vmcnt<0>();
+        wait_vmcnt<(NST - 2) * CNT>();
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
-        const bool nx = ahead && it + 2 >= nk;
-        const int kt2 = nx ? it + 2 - nk : min(it + 2, nk - 1);
+        const bool nx = ahead && it + NST >= nk;
+        const int kt2 = nx ? it + NST - nk : min(it + NST, nk - 1);
         kstep(std::integral_constant<int, ((KS - 1) & 1)>{},
               [&](auto xc) __attribute__((always_inline)) {
                   constexpr int x = decltype(xc)::value;
@@ -431,6 +436,7 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
               },
               std::integral_constant<int, TR + TC + CNT>{});
         __builtin_amdgcn_sched_barrier(0);
+        cur = nxt;
     }
     if (!ahead) wait_vmcnt<0>();         // drain the clamped loads before the ring is reused
 
@@ -495,13 +501,13 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
 // tiles and share operand slabs in that XCD's L2.  When the tile count leaves a last round
 // that at most half the workgroups could join, those tiles are issued as column halves
 // (HALVES), one per workgroup, so the round takes half as long.
-template <int WR, int WC, int TR, int TC, int BKB, int EPI, bool HALVES>
+template <int WR, int WC, int TR, int TC, int BKB, int EPI, bool HALVES, int NST>
 __global__ __launch_bounds__(WR* WC * 64) void k_gemm_dma(DmaArgs da) {
     constexpr int BR = WR * TR * 32, BC = WC * TC * 32;
     extern __shared__ __attribute__((aligned(16))) int8_t smem[];
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) int8_t*)smem;
-    // behind the two-stage operand ring: one 4 KB strip per wave for the output rows on their way out
-    int8_t* stg = smem + 2 * (BR + BC) * BKB + (threadIdx.x >> 6) * 4096;
+    // behind the operand ring: one 4 KB strip per wave for the output rows on their way out
+    int8_t* stg = smem + NST * (BR + BC) * BKB + (threadIdx.x >> 6) * 4096;
     const uint32_t G = gridDim.x;
     const uint32_t w = (G % 8 == 0) ? (blockIdx.x % 8) * (G / 8) + blockIdx.x / 8 : blockIdx.x;
     bool have_slabs = false;
@@ -510,9 +516,9 @@ __global__ __launch_bounds__(WR* WC * 64) void k_gemm_dma(DmaArgs da) {
         const GemmItem nxt = gemm_item<BR, BC>(L + G, da);
         if (HALVES && cur.half) {
             if constexpr (HALVES)
-                have_slabs = gemm_dma_tile<WR, WC, TR, TC / 2, BKB, EPI>(da.g, smem, stg, lds_base, cur, nxt, have_slabs);
+                have_slabs = gemm_dma_tile<WR, WC, TR, TC / 2, BKB, EPI, NST>(da.g, smem, stg, lds_base, cur, nxt, have_slabs);
         } else {
-            have_slabs = gemm_dma_tile<WR, WC, TR, TC, BKB, EPI>(da.g, smem, stg, lds_base, cur, nxt, have_slabs);
+            have_slabs = gemm_dma_tile<WR, WC, TR, TC, BKB, EPI, NST>(da.g, smem, stg, lds_base, cur, nxt, have_slabs);
         }
         cur = nxt;
     }
@@ -613,15 +619,19 @@ static int launch_kmajor(GemmArgs& a, int batch, hipStream_t st) {
 }
 
 // waves (rows x cols), MFMA tiles per wave (rows x cols), K bytes per slab of the large-shape kernel
+#ifndef CPMK_GEMM_NST_SMALL
+#define CPMK_GEMM_NST_SMALL 4      // ring stages of the 128x128 and 128x64 tile kernels
+#endif
 #ifndef CPMK_GEMM_BIG
 #define CPMK_GEMM_BIG 2, 4, 4, 2, 128
 #endif
 
-template <int WR, int WC, int TR, int TC, int BKB, int EPI, bool HALVES>
+template <int WR, int WC, int TR, int TC, int BKB, int EPI, bool HALVES, int NST>
 static int launch_dma_kernel(const DmaArgs& da, unsigned grid, hipStream_t st) {
     constexpr int BR = WR * TR * 32, BC = WC * TC * 32;
-    constexpr int smem = 2 * (BR + BC) * BKB + WR * WC * 4096;      // operand ring + output strips
-    auto kern = k_gemm_dma<WR, WC, TR, TC, BKB, EPI, HALVES>;
+    constexpr int smem = NST * (BR + BC) * BKB + WR * WC * 4096;      // operand ring + output strips
+    static_assert(smem <= 160 * 1024, "LDS of one compute unit");
+    auto kern = k_gemm_dma<WR, WC, TR, TC, BKB, EPI, HALVES, NST>;
     static bool attr_set[64] = {false};       // dynamic LDS above 64 KB must be enabled per device
     int dev = 0;
     (void)hipGetDevice(&dev);
@@ -635,7 +645,7 @@ static int launch_dma_kernel(const DmaArgs& da, unsigned grid, hipStream_t st) {
     return launch_status();
 }
 
-template <int WR, int WC, int TR, int TC, int BKB, int EPI>
+template <int WR, int WC, int TR, int TC, int BKB, int EPI, int NST = 2>
 static int launch_dma(GemmArgs& a, int batch, hipStream_t st) {
     constexpr int BR = WR * TR * 32, BC = WC * TC * 32;
     a.tiles_r = (int32_t)ceil_div(a.n, BR);
@@ -654,9 +664,9 @@ static int launch_dma(GemmArgs& a, int batch, hipStream_t st) {
     if (TC % 2 == 0 && r > 0 && 2 * r <= grid) {
         da.nfull = (uint32_t)(total - r);
         da.nhalf = (uint32_t)(2 * r);
-        return launch_dma_kernel<WR, WC, TR, TC, BKB, EPI, (TC % 2 == 0)>(da, (unsigned)grid, st);
+        return launch_dma_kernel<WR, WC, TR, TC, BKB, EPI, (TC % 2 == 0), NST>(da, (unsigned)grid, st);
     }
-    return launch_dma_kernel<WR, WC, TR, TC, BKB, EPI, false>(da, (unsigned)grid, st);
+    return launch_dma_kernel<WR, WC, TR, TC, BKB, EPI, false, NST>(da, (unsigned)grid, st);
 }
 
 template <bool FUSED>
@@ -687,8 +697,9 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
         if (big * 4 >= compute_units() * 3) return launch_dma<CPMK_GEMM_BIG, EPI>(a, batch, st);
         // 128x128 tiles, or 128x64 when even those leave a quarter of the compute units idle
         const int64_t mid = ceil_div(n, 128) * ceil_div(m, 128) * batch;
-        if (mid * 4 >= compute_units() * 3) return launch_dma<2, 2, 2, 2, 128, EPI>(a, batch, st);
-        return launch_dma<2, 2, 2, 1, 128, EPI>(a, batch, st);
+        // the smaller tiles finish a slab before a load from L2 returns: four ring stages keep them fed
+        if (mid * 4 >= compute_units() * 3) return launch_dma<2, 2, 2, 2, 128, EPI, CPMK_GEMM_NST_SMALL>(a, batch, st);
+        return launch_dma<2, 2, 2, 1, 128, EPI, CPMK_GEMM_NST_SMALL>(a, batch, st);
     }
     if (fast) {
         const int64_t t256 = ceil_div(n, 256) * ceil_div(m, 128) * batch;
@@ -787,7 +798,7 @@ static int gemm_f16_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, in
         (int64_t)n * k * 2 < (1ll << 32) && (int64_t)m * k * 2 < (1ll << 32)) {
         const int64_t big = ceil_div(n, 256) * ceil_div(m, 256) * batch;
         if (big * 4 >= compute_units() * 3) return launch_dma<CPMK_GEMM_BIG, kEpiF16>(a, batch, st);
-        return launch_dma<2, 2, 2, 2, 128, kEpiF16>(a, batch, st);
+        return launch_dma<2, 2, 2, 2, 128, kEpiF16, CPMK_GEMM_NST_SMALL>(a, batch, st);
     }
     dim3 grid((unsigned)ceil_div(m, 64), (unsigned)ceil_div(n, 64), (unsigned)batch);
     if (grid.y > 65535) return CPMK_ETOOBIG;
