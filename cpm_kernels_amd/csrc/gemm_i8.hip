@@ -199,10 +199,6 @@ __device__ __forceinline__ void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
-#ifndef CPMK_GEMM_MPM
-#define CPMK_GEMM_MPM 0     // >0: that many memory operations after each MFMA from the start of a k-step; 0: spread evenly
-#endif
-
 // What the tile kernel does with its accumulators.
 constexpr int kEpiInt32 = 0;     // int8 product, int32 out
 constexpr int kEpiDequant = 1;   // int8 product, fp16( (f32(acc) * s_row) * s_col ) out
@@ -377,12 +373,7 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
                                                                    __builtin_bit_cast(half8_t, fp[buf][i]), acc[i][j], 0, 0, 0);
             else
                 acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fq[buf][j], fp[buf][i], acc[i][j], 0, 0, 0);
-#if CPMK_GEMM_MPM
-            constexpr int lo = x * CPMK_GEMM_MPM < NMEM ? x * CPMK_GEMM_MPM : NMEM;
-            constexpr int hi = (x == NM - 1 || (x + 1) * CPMK_GEMM_MPM > NMEM) ? NMEM : (x + 1) * CPMK_GEMM_MPM;
-#else
             constexpr int lo = (x * NMEM) / NM, hi = ((x + 1) * NMEM) / NM;
-#endif
             static_for<lo, hi>([&](auto yc) __attribute__((always_inline)) { memop(yc); });
             __builtin_amdgcn_sched_barrier(0);
         });
