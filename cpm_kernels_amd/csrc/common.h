@@ -105,9 +105,12 @@ __device__ inline int32_t quant_i8_rcp(float x, float s, float y) {
     return min(max(n, -128), 127);
 }
 
+// Low bytes of four integers (each already within int8 range) into one dword: three byte
+// permutes.  v_perm_b32 selector bytes 0-3 pick from the second operand, 4-7 from the first, 0x0c is zero.
 __device__ inline uint32_t pack4_i8(int32_t a, int32_t b, int32_t c, int32_t d) {
-    return (uint32_t)(a & 0xff) | ((uint32_t)(b & 0xff) << 8) | ((uint32_t)(c & 0xff) << 16) |
-           ((uint32_t)d << 24);
+    const uint32_t lo = __builtin_amdgcn_perm((uint32_t)b, (uint32_t)a, 0x0c0c0400u);     // a | b << 8
+    const uint32_t hi = __builtin_amdgcn_perm((uint32_t)d, (uint32_t)c, 0x0c0c0400u);     // c | d << 8
+    return __builtin_amdgcn_perm(hi, lo, 0x05040100u);                                    // lo | hi << 16
 }
 
 // fp32 -> fp16 of a value that must first exist as a rounded fp32 number.  Without the
