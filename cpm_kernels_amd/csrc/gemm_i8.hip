@@ -498,7 +498,8 @@ __global__ __launch_bounds__(WR* WC * 64) void k_gemm_dma(DmaArgs da) {
     extern __shared__ __attribute__((aligned(16))) int8_t smem[];
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) int8_t*)smem;
     // behind the operand ring: one 4 KB strip per wave for the output rows on their way out
-    int8_t* stg = smem + NST * (BR + BC) * BKB + (threadIdx.x >> 6) * 4096;
+    constexpr int STRIP = TC * 64 * 32 > 4096 ? TC * 64 * 32 : 4096;      // 32 rows of the widest chunk (fp16: TC*64 bytes, int32: 128)
+    int8_t* stg = smem + NST * (BR + BC) * BKB + (threadIdx.x >> 6) * STRIP;
     const uint32_t G = gridDim.x;
     const uint32_t w = (G % 8 == 0) ? (blockIdx.x % 8) * (G / 8) + blockIdx.x / 8 : blockIdx.x;
     bool have_slabs = false;
@@ -620,7 +621,8 @@ static int launch_kmajor(GemmArgs& a, int batch, hipStream_t st) {
 template <int WR, int WC, int TR, int TC, int BKB, int EPI, bool HALVES, int NST>
 static int launch_dma_kernel(const DmaArgs& da, unsigned grid, hipStream_t st) {
     constexpr int BR = WR * TR * 32, BC = WC * TC * 32;
-    constexpr int smem = NST * (BR + BC) * BKB + WR * WC * 4096;      // operand ring + output strips
+    constexpr int STRIP = TC * 64 * 32 > 4096 ? TC * 64 * 32 : 4096;
+    constexpr int smem = NST * (BR + BC) * BKB + WR * WC * STRIP;      // operand ring + output strips
     static_assert(smem <= 160 * 1024, "LDS of one compute unit");
     auto kern = k_gemm_dma<WR, WC, TR, TC, BKB, EPI, HALVES, NST>;
     static bool attr_set[64] = {false};       // dynamic LDS above 64 KB must be enabled per device
