@@ -239,6 +239,28 @@ def test_gemm_int8(gpu, case):
                 _gemm_case(gpu, N, K, M, bA, bB, aT, bT, rng)
 
 
+# Tile-kernel coverage: K-major operands with k % 128 == 0 in every dispatch regime -- 256x256 tiles
+# with a last round of half tiles, 128x128 and 128x64 tiles with the four-stage ring (one tile per
+# workgroup, several with the next tile's slabs fetched ahead, slab counts that are not a multiple
+# of the ring depth), ragged edges, output widths that are not a multiple of 8 (register-staged
+# kernel instead), one to many K slabs.
+TILE_CASES = [  # (batch, kernel n = output rows, k, kernel m = output columns)
+    (1, 4096, 512, 3072), (1, 2304, 256, 4608), (1, 2048, 1024, 2048), (1, 3000, 384, 2048), (2, 1500, 640, 1100),
+    (1, 128, 128, 64), (1, 132, 128, 72), (1, 100, 256, 60), (3, 260, 384, 520), (1, 512, 128, 4096),
+    (1, 520, 1152, 1032), (1, 1024, 896, 1028), (1, 640, 2048, 644), (4, 384, 512, 392), (1, 4100, 128, 2056),
+    (1, 8, 128, 8), (1, 4, 256, 260), (2, 2816, 256, 2304),
+]
+
+
+@pytest.mark.parametrize("case", TILE_CASES)
+def test_gemm_int8_tile_kernels(gpu, case):
+    batch, n, k, m = case
+    rng = np.random.default_rng(n * 7919 + k * 31 + m)
+    for (bA, bB) in ((batch, batch),) + (((1, batch), (batch, 1)) if batch > 1 else ()):
+        _name("gemm_int8 tile kernels", case, bA, bB)
+        _gemm_case(gpu, m, k, n, bA, bB, True, False, rng)
+
+
 def test_gemm_int8_extreme_values(gpu):
     """All operands -128 / 127: largest accumulators the int8 product can produce."""
     _name("gemm_int8 extremes")
