@@ -209,10 +209,10 @@ struct DmaArgs {
     int32_t batch;
     int32_t ntiles;    // full-size tiles per batch entry (tiles_r x tiles_c)
     uint32_t nfull;    // work items [0, nfull) are whole tiles in walk order ...
-    uint32_t nhalf;    // ... items [nfull, nfull + nhalf) are column halves of the tiles that follow
+    uint32_t nhalf;    // ... items [nfull, nfull + nhalf) are row halves (top, bottom) of the tiles that follow
 };
 
-// One work item of the persistent kernel: a whole BR x BC tile, or its left/right half.
+// One work item of the persistent kernel: a whole BR x BC tile, or its top/bottom half.
 struct GemmItem {
     uint32_t b;        // batch entry
     int32_t j0, i0;    // first output row / column
@@ -236,8 +236,8 @@ __device__ __forceinline__ GemmItem gemm_item(uint32_t L, const DmaArgs& da) {
     const uint32_t g = t / group_sz;
     const uint32_t rows_in_group = min(GRP, (uint32_t)da.g.tiles_r - g * GRP);
     const uint32_t tin = t - g * group_sz;
-    it.j0 = (int32_t)((g * GRP + tin % rows_in_group) * BR);
-    it.i0 = (int32_t)((tin / rows_in_group) * BC + (h & 1) * (BC / 2));
+    it.j0 = (int32_t)((g * GRP + tin % rows_in_group) * BR + (h & 1) * (BR / 2));
+    it.i0 = (int32_t)((tin / rows_in_group) * BC);
     return it;
 }
 
@@ -490,8 +490,9 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
 // Persistent kernel: WR x WC waves, wave tile = TR x TC MFMA tiles of 32x32.  Workgroup w of G
 // takes items round*G + (w%8)*(G/8) + w/8: the workgroups of one XCD (w % 8) work on adjacent
 // tiles and share operand slabs in that XCD's L2.  When the tile count leaves a last round
-// that at most half the workgroups could join, those tiles are issued as column halves
-// (HALVES), one per workgroup, so the round takes half as long.
+// that at most half the workgroups could join, those tiles are issued as row halves (HALVES), one
+// per workgroup: a wave then owns TR/2 x TC MFMA tiles, which keeps the fragment reads per MFMA
+// lower than halving the columns would (TR/2 + TC reads for TR/2 * TC MFMAs per k-step).
 template <int WR, int WC, int TR, int TC, int BKB, int EPI, bool HALVES, int NST>
 __global__ __launch_bounds__(WR* WC * 64) void k_gemm_dma(DmaArgs da) {
     constexpr int BR = WR * TR * 32, BC = WC * TC * 32;
@@ -508,7 +509,7 @@ __global__ __launch_bounds__(WR* WC * 64) void k_gemm_dma(DmaArgs da) {
         const GemmItem nxt = gemm_item<BR, BC>(L + G, da);
         if (HALVES && cur.half) {
             if constexpr (HALVES)
-                have_slabs = gemm_dma_tile<WR, WC, TR, TC / 2, BKB, EPI, NST>(da.g, smem, stg, lds_base, cur, nxt, have_slabs);
+                have_slabs = gemm_dma_tile<WR, WC, TR / 2, TC, BKB, EPI, NST>(da.g, smem, stg, lds_base, cur, nxt, have_slabs);
         } else {
             have_slabs = gemm_dma_tile<WR, WC, TR, TC, BKB, EPI, NST>(da.g, smem, stg, lds_base, cur, nxt, have_slabs);
         }
@@ -654,10 +655,10 @@ static int launch_dma(GemmArgs& a, int batch, hipStream_t st) {
     const int64_t r = total % grid;
     da.nfull = (uint32_t)total;
     da.nhalf = 0;
-    if (TC % 2 == 0 && r > 0 && 2 * r <= grid) {
+    if (TR % 2 == 0 && r > 0 && 2 * r <= grid) {
         da.nfull = (uint32_t)(total - r);
         da.nhalf = (uint32_t)(2 * r);
-        return launch_dma_kernel<WR, WC, TR, TC, BKB, EPI, (TC % 2 == 0), NST>(da, (unsigned)grid, st);
+        return launch_dma_kernel<WR, WC, TR, TC, BKB, EPI, (TR % 2 == 0), NST>(da, (unsigned)grid, st);
     }
     return launch_dma_kernel<WR, WC, TR, TC, BKB, EPI, false, NST>(da, (unsigned)grid, st);
 }
