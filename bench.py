@@ -305,6 +305,15 @@ def main():
             "achieved": round(2.0 * 10240 * 4096 * 4096 / (ms * 1e-3) / 1e12, 1), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
             "frac": round(2.0 * 10240 * 4096 * 4096 / (ms * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4), "timing": "events, whole bmm"}
         del W1, xa
+        # fp16 product of the north-star shape on the same tile kernel (fp32 accumulation)
+        Ah = torch.randn(1, M, K, generator=gg).half().to(dev); Wh = (torch.randn(1, N, K, generator=gg) * 0.02).half().to(dev)
+        oh = torch.empty((1, M, N), dtype=torch.half, device=dev)
+        ms = event_ms(lambda: ck.gemm_fp16(N, K, M, 1, 1, True, False, Wh.data_ptr(), Ah.data_ptr(), oh.data_ptr(), st()), 20)
+        components["gemm_fp16"] = {
+            "shape": "M=%d K=%d N=%d fp16, fp32 accumulate" % (M, K, N), "bound": "mfma", "avg_us": round(ms * 1e3, 2),
+            "achieved": round(2.0 * M * K * N / (ms * 1e-3) / 1e12, 1), "peak": 2500.0, "unit": "TFLOP/s",
+            "frac": round(2.0 * M * K * N / (ms * 1e-3) / 1e12 / 2500.0, 4), "timing": "events"}
+        del Ah, Wh, oh
 
     # per-op CPU timings beside the three headline components (torch formulations, host cores)
     if not args.no_cpu and only == "":
