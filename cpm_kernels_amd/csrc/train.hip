@@ -28,25 +28,53 @@ __device__ inline half_t ew_apply(int op, half_t x, half_t a, half_t b) {
     }
 }
 
-template <int OP, int BC>
-__global__ __launch_bounds__(256) void k_ew(int64_t total, int64_t n, int64_t m, const half_t* x, const half_t* __restrict__ a,
+// The tensor is seen as rows x cols: BC 0: one row; BC 1: rows = batch, cols = n, a/b indexed by the
+// column; BC 2: rows = batch*n, cols = m, a/b indexed by row % n.  blockIdx.x = row * chunks + chunk;
+// a thread handles V adjacent elements (8 = 16-byte accesses when cols % 8 == 0 and everything is
+// 16-byte aligned, else 2: element counts are even, the reference asserts it).
+template <int OP, int BC, int V>
+__global__ __launch_bounds__(256) void k_ew(int64_t cols, uint32_t chunks, int64_t n, const half_t* x, const half_t* __restrict__ a,
                                             const half_t* __restrict__ b, half_t* out) {
-    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 2;      // element counts are even (reference asserts)
-    if (i >= total) return;
-    half2_t v = *reinterpret_cast<const half2_t*>(x + i);
-    half2_t r;
+    typedef half_t vec_t __attribute__((ext_vector_type(V)));
+    const uint32_t chunk = blockIdx.x % chunks;
+    const int64_t row = blockIdx.x / chunks;
+    const int64_t c = ((int64_t)chunk * 256 + threadIdx.x) * V;
+    if (c >= cols) return;
+    const int64_t i = row * cols + c;
+    const vec_t v = *reinterpret_cast<const vec_t*>(x + i);
+    vec_t av, bv;
+    if (BC == 2) {
+        const int64_t k = row % n;
+        const half_t a1 = a[k], b1 = b ? b[k] : (half_t)0.0f;
 #pragma unroll
-    for (int e = 0; e < 2; ++e) {
-        const int64_t idx = i + e;
-        const int64_t k = BC == 0 ? idx : (BC == 1 ? idx % n : (idx / m) % n);
-        r[e] = ew_apply(OP, v[e], a[k], b ? b[k] : (half_t)0.0f);
+        for (int e = 0; e < V; ++e) { av[e] = a1; bv[e] = b1; }
+    } else {
+        const int64_t k = BC == 0 ? i : c;
+        av = *reinterpret_cast<const vec_t*>(a + k);
+#pragma unroll
+        for (int e = 0; e < V; ++e) bv[e] = (half_t)0.0f;
+        if (b) bv = *reinterpret_cast<const vec_t*>(b + k);
     }
-    *reinterpret_cast<half2_t*>(out + i) = r;
+    vec_t r;
+#pragma unroll
+    for (int e = 0; e < V; ++e) r[e] = ew_apply(OP, v[e], av[e], bv[e]);
+    *reinterpret_cast<vec_t*>(out + i) = r;
 }
 
+template <int V>
 __global__ __launch_bounds__(256) void k_global_scale(int64_t n, const half_t* inp, float scale, half_t* out) {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i < n) out[i] = round_f16((float)inp[i] * scale);
+    typedef half_t vec_t __attribute__((ext_vector_type(V)));
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * V;
+    if (i >= n) return;
+    if (V > 1) {
+        const vec_t v = *reinterpret_cast<const vec_t*>(inp + i);
+        vec_t r;
+#pragma unroll
+        for (int e = 0; e < V; ++e) r[e] = round_f16((float)v[e] * scale);
+        *reinterpret_cast<vec_t*>(out + i) = r;
+    } else {
+        out[i] = round_f16((float)inp[i] * scale);
+    }
 }
 
 // cu_gelu_backward: grad = gelu'(x) * grad_out with the reference's constants and cut-off at |x| >= 5.
@@ -276,12 +304,21 @@ __global__ __launch_bounds__(256) void k_embedding_backward2(int32_t batch, int3
 }
 
 template <int OP, int BC>
-static int launch_ew(int64_t total, int64_t n, int64_t m, const void* x, const void* a, const void* b, void* out, void* stream) {
-    if (total < 0) return CPMK_EBADARG;
-    if (total == 0) return 0;
-    if (total % 2) return CPMK_EALIGN;
-    hipLaunchKernelGGL((k_ew<OP, BC>), dim3((unsigned)ceil_div(total / 2, 256)), dim3(256), 0, (hipStream_t)stream, total, n, m,
-                       (const half_t*)x, (const half_t*)a, (const half_t*)b, (half_t*)out);
+static int launch_ew(int64_t rows, int64_t cols, int64_t n, const void* x, const void* a, const void* b, void* out, void* stream) {
+    if (rows < 0 || cols < 0) return CPMK_EBADARG;
+    if (rows * cols == 0) return 0;
+    if (cols % 2) return CPMK_EALIGN;
+    const bool wide = cols % 8 == 0 && aligned16(x) && aligned16(out) && (BC == 2 || (aligned16(a) && (!b || aligned16(b))));
+    const int v = wide ? 8 : 2;
+    const int64_t chunks = ceil_div(cols, 256 * v);
+    if (rows * chunks > 0x7fffffffll) return CPMK_ETOOBIG;
+    const dim3 grid((unsigned)(rows * chunks));
+    if (wide)
+        hipLaunchKernelGGL((k_ew<OP, BC, 8>), grid, dim3(256), 0, (hipStream_t)stream, cols, (uint32_t)chunks, n, (const half_t*)x,
+                           (const half_t*)a, (const half_t*)b, (half_t*)out);
+    else
+        hipLaunchKernelGGL((k_ew<OP, BC, 2>), grid, dim3(256), 0, (hipStream_t)stream, cols, (uint32_t)chunks, n, (const half_t*)x,
+                           (const half_t*)a, (const half_t*)b, (half_t*)out);
     return launch_status();
 }
 
@@ -304,45 +341,52 @@ int cpmk_arith_global_scale(int64_t n, const void* inp, float scale, void* out, 
     clear_stale_error();
     if (n < 0) return CPMK_EBADARG;
     if (n == 0) return 0;
-    hipLaunchKernelGGL(k_global_scale, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, (hipStream_t)stream, n, (const half_t*)inp,
-                       scale, (half_t*)out);
+    if (n % 8 == 0 && aligned16(inp) && aligned16(out))
+        hipLaunchKernelGGL((k_global_scale<8>), dim3((unsigned)ceil_div(n, 256 * 8)), dim3(256), 0, (hipStream_t)stream, n,
+                           (const half_t*)inp, scale, (half_t*)out);
+    else
+        hipLaunchKernelGGL((k_global_scale<1>), dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, (hipStream_t)stream, n,
+                           (const half_t*)inp, scale, (half_t*)out);
     return launch_status();
 }
 int cpmk_arith_element_mul(int32_t batch, int32_t n, const void* x, const void* y, void* out, void* stream) {
     clear_stale_error();
     if (n % 2) return CPMK_EALIGN;
-    return launch_ew<kMul, 0>((int64_t)batch * n, n, 1, x, y, nullptr, out, stream);
+    return launch_ew<kMul, 0>(1, (int64_t)batch * n, 1, x, y, nullptr, out, stream);
 }
 int cpmk_arith_batch_add_forward(int32_t batch, int32_t n, const void* x, const void* y, void* out, void* stream) {
     clear_stale_error();
     if (n % 2) return CPMK_EALIGN;
-    return launch_ew<kAdd, 1>((int64_t)batch * n, n, 1, x, y, nullptr, out, stream);
+    return launch_ew<kAdd, 1>(batch, n, n, x, y, nullptr, out, stream);
 }
 int cpmk_arith_batch_mul_add(int32_t batch, int32_t n, const void* x, const void* alpha, const void* beta, void* out, void* stream) {
     clear_stale_error();
     if (n % 2) return CPMK_EALIGN;
-    return launch_ew<kFma, 1>((int64_t)batch * n, n, 1, x, alpha, beta, out, stream);
+    return launch_ew<kFma, 1>(batch, n, n, x, alpha, beta, out, stream);
 }
 int cpmk_arith_batch_mul(int32_t batch, int32_t n, const void* x, const void* alpha, void* out, void* stream) {
     clear_stale_error();
     if (n % 2) return CPMK_EALIGN;
-    return launch_ew<kMul, 1>((int64_t)batch * n, n, 1, x, alpha, nullptr, out, stream);
+    return launch_ew<kMul, 1>(batch, n, n, x, alpha, nullptr, out, stream);
 }
 int cpmk_arith_ln_add(int32_t batch, int32_t n, int32_t m, const void* inp, const void* beta, void* out, void* stream) {
     clear_stale_error();
+    if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
     if (m % 2) return CPMK_EALIGN;
-    return launch_ew<kAdd, 2>((int64_t)batch * n * m, n, m, inp, beta, nullptr, out, stream);
+    return launch_ew<kAdd, 2>((int64_t)batch * n, m, n, inp, beta, nullptr, out, stream);
 }
 int cpmk_arith_ln_div(int32_t batch, int32_t n, int32_t m, const void* inp, const void* alpha, void* out, void* stream) {
     clear_stale_error();
+    if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
     if (m % 2) return CPMK_EALIGN;
-    return launch_ew<kDiv, 2>((int64_t)batch * n * m, n, m, inp, alpha, nullptr, out, stream);
+    return launch_ew<kDiv, 2>((int64_t)batch * n, m, n, inp, alpha, nullptr, out, stream);
 }
 int cpmk_arith_ln_sub_div(int32_t batch, int32_t n, int32_t m, const void* inp, const void* alpha, const void* beta, void* out,
                           void* stream) {
     clear_stale_error();
+    if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
     if (m % 2) return CPMK_EALIGN;
-    return launch_ew<kSubDiv, 2>((int64_t)batch * n * m, n, m, inp, alpha, beta, out, stream);
+    return launch_ew<kSubDiv, 2>((int64_t)batch * n, m, n, inp, alpha, beta, out, stream);
 }
 int cpmk_arith_batch_add_backward(int32_t batch, int32_t n, const void* grad_out, void* grad, void* stream) {
     clear_stale_error();
