@@ -138,10 +138,14 @@ int cpmk_gemm_quantize_cols(int32_t batch, int32_t n, int32_t m, const void* mat
     if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
     if ((int64_t)batch * n * m == 0) return 0;
     hipStream_t st = (hipStream_t)stream;
+    // a team here only exchanges one maximum per column and gathers it in a loop over the parts, so
+    // it may be larger than the teams of the kernels that keep per-part values in registers
+    // (16384 rows; far fewer workgroups than are resident at once, which is what progress needs)
+    constexpr int64_t kColMaxParts = 32;
     const int64_t tiles = ceil_div(m, 64), parts = ceil_div(n, 512);
     const bool team_ok = (m % 8 == 0) && (!out_transposed || n % 8 == 0) && aligned16(mat) && aligned16(scale) &&
                          ((reinterpret_cast<uintptr_t>(out) & 7u) == 0) && (int64_t)n * m < (1ll << 31) &&
-                         parts <= kXchMaxParts && tiles * batch * parts <= kXchSlots;
+                         parts <= kColMaxParts && tiles * batch * parts <= kXchSlots;
     if (team_ok) {
         XchLaunch xl = {nullptr, 0};
         if (parts > 1) {

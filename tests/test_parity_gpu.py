@@ -42,7 +42,8 @@ def adversarial_rows(rng, n, m):
 
 
 QUANT_SHAPES = [(1, 512, 4096), (3, 17, 1000), (2, 5, 7), (1, 1, 8), (2, 64, 48), (1, 9, 8200), (4, 33, 16),
-                (1, 2100, 128), (1, 3, 20480), (2, 4096, 192), (1, 1032, 72), (3, 520, 8)]
+                (1, 2100, 128), (1, 3, 20480), (2, 4096, 192), (1, 1032, 72), (3, 520, 8),
+                (1, 10240, 192), (2, 16384, 64), (1, 16392, 64)]
 
 
 @pytest.mark.parametrize("shape", QUANT_SHAPES)
