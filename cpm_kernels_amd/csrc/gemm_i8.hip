@@ -688,7 +688,8 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
         // 256x256 tiles when they give most compute units a tile, else 128x128
         const int64_t big = ceil_div(n, 256) * ceil_div(m, 256) * batch;
         constexpr int EPI = FUSED ? kEpiDequant : kEpiInt32;
-        if (big * 4 >= compute_units() * 3) return launch_dma<CPMK_GEMM_BIG, EPI>(a, batch, st);
+        // (a dimension of at most 128 would leave half or more of every 256-wide tile empty)
+        if (big * 4 >= compute_units() * 3 && n > 128 && m > 128) return launch_dma<CPMK_GEMM_BIG, EPI>(a, batch, st);
         // 128x128 tiles, or 128x64 when even those leave a quarter of the compute units idle
         const int64_t mid = ceil_div(n, 128) * ceil_div(m, 128) * batch;
         // the smaller tiles finish a slab before a load from L2 returns: four ring stages keep them fed
@@ -791,7 +792,7 @@ static int gemm_f16_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, in
     if (p_kmajor && q_kmajor && wide && k > 0 && (k % 64 == 0) && aligned16(A) && aligned16(B) &&
         (int64_t)n * k * 2 < (1ll << 32) && (int64_t)m * k * 2 < (1ll << 32)) {
         const int64_t big = ceil_div(n, 256) * ceil_div(m, 256) * batch;
-        if (big * 4 >= compute_units() * 3) return launch_dma<CPMK_GEMM_BIG, kEpiF16>(a, batch, st);
+        if (big * 4 >= compute_units() * 3 && n > 128 && m > 128) return launch_dma<CPMK_GEMM_BIG, kEpiF16>(a, batch, st);
         return launch_dma<2, 2, 2, 2, 128, kEpiF16, CPMK_GEMM_NST_SMALL>(a, batch, st);
     }
     dim3 grid((unsigned)ceil_div(m, 64), (unsigned)ceil_div(n, 64), (unsigned)batch);

@@ -19,6 +19,33 @@ __global__ __launch_bounds__(256) void k_transpose(int32_t n, int32_t m, const h
         if (c0 + c < m && r0 + tx < n) out[boff + (int64_t)(c0 + c) * n + r0 + tx] = tile[tx][c];
 }
 
+// The same with 16-byte global accesses (n % 8 == 0, m % 8 == 0, 16-byte aligned pointers): a row
+// of the tile is read by eight lanes, a row of the transposed tile is written by eight lanes; the
+// transposition itself is eight 2-byte LDS reads per lane.
+__global__ __launch_bounds__(256) void k_transpose_wide(int32_t n, int32_t m, const half_t* __restrict__ in, half_t* __restrict__ out) {
+    __shared__ half_t tile[64][72];                     // pitch 144 bytes: 16-byte aligned rows, odd multiple of 16 bytes
+    const int64_t boff = (int64_t)blockIdx.z * n * m;
+    const int32_t r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+    const int pc = threadIdx.x & 7, rr = threadIdx.x >> 3;          // 8 pieces x 32 rows per pass
+#pragma unroll
+    for (int ps = 0; ps < 2; ++ps) {
+        const int r = ps * 32 + rr;
+        if (r0 + r < n && c0 + pc * 8 < m)
+            *reinterpret_cast<half8_t*>(&tile[r][pc * 8]) = *reinterpret_cast<const half8_t*>(in + boff + (int64_t)(r0 + r) * m + c0 + pc * 8);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int ps = 0; ps < 2; ++ps) {
+        const int c = ps * 32 + rr;                     // row of the transposed tile
+        if (c0 + c < m && r0 + pc * 8 < n) {
+            half8_t v;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = tile[pc * 8 + e][c];
+            *reinterpret_cast<half8_t*>(out + boff + (int64_t)(c0 + c) * n + r0 + pc * 8) = v;
+        }
+    }
+}
+
 __global__ void k_array_add(int32_t* arr, int32_t pos, int32_t val) {
     if (threadIdx.x == 0) arr[pos] += val;
 }
@@ -67,8 +94,11 @@ int cpmk_transpose(int32_t batch, int32_t n, int32_t m, const void* inp, void* o
     if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
     if ((int64_t)batch * n * m == 0) return 0;
     if (batch > 65535 || ceil_div(n, 64) > 65535) return CPMK_ETOOBIG;
-    hipLaunchKernelGGL(k_transpose, dim3((unsigned)ceil_div(m, 64), (unsigned)ceil_div(n, 64), (unsigned)batch), dim3(256), 0,
-                       (hipStream_t)stream, n, m, (const half_t*)inp, (half_t*)out);
+    const dim3 grid((unsigned)ceil_div(m, 64), (unsigned)ceil_div(n, 64), (unsigned)batch);
+    if (n % 8 == 0 && m % 8 == 0 && aligned16(inp) && aligned16(out))
+        hipLaunchKernelGGL(k_transpose_wide, grid, dim3(256), 0, (hipStream_t)stream, n, m, (const half_t*)inp, (half_t*)out);
+    else
+        hipLaunchKernelGGL(k_transpose, grid, dim3(256), 0, (hipStream_t)stream, n, m, (const half_t*)inp, (half_t*)out);
     return launch_status();
 }
 

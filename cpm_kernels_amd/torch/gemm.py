@@ -9,7 +9,7 @@ the six-launch sequence, which ``fused=False`` still runs through the kernel-lev
 import torch
 from ..kernels import gemm_calc_scale, gemm_calc_scale_transpose, gemm_round, gemm_round_transpose, \
     gemm_scale, gemm_scale_x, gemm_scale_y, gemm_int8, gemm_int8_scale, gemm_quantize, gemm_quantize_cols, \
-    gemm_quantize_pair, gemm_fp16, gemm_backward_round_scale, gemm_backward_scale_round
+    gemm_quantize_pair, gemm_fp16, gemm_backward_round_scale, gemm_backward_scale_round, transpose
 from ._common import cur_stream
 
 
@@ -171,10 +171,24 @@ class GEMMInt8(torch.autograd.Function):
         return grad_A, None, grad_B, None, None
 
 
+def _transposed_copy(x: torch.Tensor) -> torch.Tensor:
+    out = torch.empty((x.size(0), x.size(2), x.size(1)), dtype=torch.half, device=x.device)
+    transpose(x.size(0), x.size(1), x.size(2), x.data_ptr(), out.data_ptr(), cur_stream())
+    return out
+
+
 def gemm_pth_fp16(A: torch.Tensor, aT: bool, B: torch.Tensor, bT: bool) -> torch.Tensor:
     """reference: torch/gemm.py:189-203; operands are passed swapped to the kernel so that the
-    (M, N) result comes out row-major."""
+    (M, N) result comes out row-major.  The MFMA tile kernel needs both operands with K as the
+    contiguous dimension (A as (b, M, K), B as (b, N, K)); an operand given the other way round
+    is copied transposed first when the shape qualifies for that kernel (K a multiple of 64, N of
+    8), which costs one pass over it instead of the many of the general kernel."""
     M, K, N = _dims(A, B, aT, bT)
+    if K % 64 == 0 and N % 8 == 0 and M * K < 2 ** 31 and N * K < 2 ** 31:
+        if aT:
+            A, aT = _transposed_copy(A), False
+        if not bT:
+            B, bT = _transposed_copy(B), True
     out = torch.empty((max(A.size(0), B.size(0)), M, N), dtype=torch.half, device=A.device)
     gemm_fp16(N, K, M, B.size(0), A.size(0), bT, aT, B.data_ptr(), A.data_ptr(), out.data_ptr(), cur_stream())
     return out

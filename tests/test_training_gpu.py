@@ -254,7 +254,8 @@ def test_embedding_backward(gpu, shape):
     assert_close_fp16(to_np(grad), full, rtol=2e-3, atol=2e-2, what="embedding gradient")
 
 
-@pytest.mark.parametrize("shape", [(2, 64, 64), (3, 17, 100), (1, 1000, 3), (2, 5, 7), (1, 4096, 512), (4, 1, 9)])
+@pytest.mark.parametrize("shape", [(2, 64, 64), (3, 17, 100), (1, 1000, 3), (2, 5, 7), (1, 4096, 512), (4, 1, 9),
+                                   (2, 72, 40), (1, 200, 136), (3, 8, 1032)])
 def test_transpose(gpu, shape):
     _name("transpose", shape)
     b, n, m = shape
