@@ -36,8 +36,10 @@ template <int OP, int BC, int V>
 __global__ __launch_bounds__(256) void k_ew(int64_t cols, uint32_t chunks, int64_t n, const half_t* x, const half_t* __restrict__ a,
                                             const half_t* __restrict__ b, half_t* out) {
     typedef half_t vec_t __attribute__((ext_vector_type(V)));
-    const uint32_t chunk = blockIdx.x % chunks;
-    const int64_t row = blockIdx.x / chunks;
+    // BC 1: the rows of one chunk of columns run side by side, so a/b are fetched from HBM once
+    const uint32_t rows = gridDim.x / chunks;
+    const uint32_t chunk = BC == 1 ? blockIdx.x / rows : blockIdx.x % chunks;
+    const int64_t row = BC == 1 ? blockIdx.x % rows : blockIdx.x / chunks;
     const int64_t c = ((int64_t)chunk * 256 + threadIdx.x) * V;
     if (c >= cols) return;
     const int64_t i = row * cols + c;
