@@ -132,6 +132,17 @@ __global__ __launch_bounds__(NW * 64) void k_gemv_coalesced(int32_t batch, int32
     const int32_t rpb = r4 * 4;                  // rows of this workgroup
     const int32_t row0 = blockIdx.x * rpb;
     int8_t* tb = tbuf[w];
+    // the scales of the outputs this thread will write, requested first so that they arrive with
+    // the weights instead of costing a round trip to memory after the reduction
+    constexpr int NOUT = (RG * NB * 256 + NW * 64 - 1) / (NW * 64);
+    half_t osv[NOUT], osm[NOUT];
+#pragma unroll
+    for (int o = 0; o < NOUT; ++o) {
+        const int idx = tid + o * NW * 64;
+        const int rr = idx % rpb, bb = idx / rpb;
+        osv[o] = scale_vec[min(bb, batch - 1)];
+        osm[o] = scale_mat[min(row0 + rr, dim_out - 1)];
+    }
     int woff[4], roff[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -227,13 +238,17 @@ __global__ __launch_bounds__(NW * 64) void k_gemv_coalesced(int32_t batch, int32
             for (int e = 0; e < 4; ++e) atomicAdd(&part[g * NB + t][(q * 4 + e) * 16 + r], acc[g][t][e]);
     __syncthreads();
     // thread -> (vector, row) with the row fastest, so a vector's outputs are stored contiguously
-    for (int idx = tid; idx < rpb * NB * 16; idx += NW * 64) {
-        const int rr = idx % rpb, bb = idx / rpb;
-        const int g = rr >> 4, t = bb >> 4;
-        const int32_t s = part[g * NB + t][(rr & 15) * 16 + (bb & 15)];
-        const int32_t row = row0 + rr;
-        if (row < dim_out && bb < batch)
-            out[(int64_t)bb * dim_out + row] = dequant(s, (float)scale_vec[bb], (float)scale_mat[row]);
+#pragma unroll
+    for (int o = 0; o < NOUT; ++o) {
+        const int idx = tid + o * NW * 64;
+        if (idx < rpb * NB * 16) {
+            const int rr = idx % rpb, bb = idx / rpb;
+            const int g = rr >> 4, t = bb >> 4;
+            const int32_t s = part[g * NB + t][(rr & 15) * 16 + (bb & 15)];
+            const int32_t row = row0 + rr;
+            if (row < dim_out && bb < batch)
+                out[(int64_t)bb * dim_out + row] = dequant(s, (float)osv[o], (float)osm[o]);
+        }
     }
 }
 
