@@ -248,14 +248,14 @@ __device__ __forceinline__ GemmItem gemm_item(uint32_t L, const DmaArgs& da) {
 //                                      nobody reads stage cur any more
 //   k-step KS-1       : MFMAs while the step-0 fragments of slab it+1 are read and the DMA of
 //                       slab it+NST is issued into stage cur
-// Past the end of K the DMA fetches slabs 0 and 1 of the NEXT tile of this workgroup (when it
+// Past the end of K the DMA fetches the first slabs of the NEXT tile of this workgroup (when it
 // has the same shape), so that tile starts with its operands already in LDS and the loads
 // overlap this tile's stores; otherwise the slab index is clamped (a redundant load nobody
-// reads).  Either way the loop body has no branches, which lets the compiler keep the
-// accumulators in place.  Returns true if the next tile's first two slabs are on their way.
+// reads).  The ring position carries over from tile to tile (`ring`), so any slab count works.  Either way the loop body has no branches, which lets the compiler keep the
+// accumulators in place.  Returns true if the next tile's first slabs are on their way.
 template <int WR, int WC, int TR, int TC, int BKB, int EPI, int NST>
 __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, int8_t* stg, uint32_t lds_base,
-                                              const GemmItem cur_item, const GemmItem nxt_item, const bool have_slabs) {
+                                              const GemmItem cur_item, const GemmItem nxt_item, const bool have_slabs, int& ring) {
     constexpr bool FUSED = EPI == kEpiDequant, F16 = EPI == kEpiF16;
     using acc_t = std::conditional_t<F16, float16_tv, int16_tv>;
     constexpr int KS = BKB / 32, CPR = BKB / 16;
@@ -292,8 +292,14 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
     const int32_t j0 = cur_item.j0, i0 = cur_item.i0;
     const int8_t* Pb = a.P + (int64_t)b * a.strideP;
     const int8_t* Qb = a.Q + (int64_t)b * a.strideQ;
-    // the next tile is fetched ahead only if its LDS layout is this one's and the ring parity works out
-    const bool ahead = nxt_item.valid && nxt_item.half == cur_item.half && nk >= NST && nk % NST == 0;
+    // the next tile is fetched ahead only if its LDS layout is this one's
+    const bool ahead = nxt_item.valid && nxt_item.half == cur_item.half;
+    // slab s of this tile lives in stage (ring + s) % NST; the slab requested at iteration `it` is
+    // number it + LD counted from this tile's slab 0.  With fewer slabs than stages (!deep) all of a
+    // tile's slabs are requested one tile ahead and every wait is a full one.
+    const bool deep = nk >= NST;
+    const int LD = deep ? NST : nk;
+    const int ring0 = __builtin_amdgcn_readfirstlane(ring);
     const int8_t* Pn = a.P + (int64_t)nxt_item.b * a.strideP;
     const int8_t* Qn = a.Q + (int64_t)nxt_item.b * a.strideQ;
 
@@ -384,12 +390,15 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
         __syncthreads();                 // every wave is done with the ring of the previous tile
         static_for<0, NST>([&](auto sc) __attribute__((always_inline)) {
             constexpr int st = decltype(sc)::value;
-            static_for<0, CNT>([&](auto dc) __attribute__((always_inline)) { dma1(dc, min(st, nk - 1), false, st); });
+            static_for<0, CNT>([&](auto dc) __attribute__((always_inline)) {
+                dma1(dc, min(st, nk - 1), false, (ring0 + st) % NST);
+            });
         });
-        wait_vmcnt<(NST - 1) * CNT>();   // slab 0 (and the scale loads issued before it) has landed
+        if (deep) wait_vmcnt<(NST - 1) * CNT>();   // slab 0 (and the scale loads issued before it) has landed
+        else wait_vmcnt<0>();
         __syncthreads();
     } else {
-        wait_vmcnt<0>();                 // slabs 0 .. NST-1 were requested during the previous tile; its stores drain too
+        wait_vmcnt<0>();                 // the first LD slabs were requested during the previous tile; its stores drain too
         __syncthreads();
     }
     if (FUSED) {     // pin the scale loads above the K loop (the waits just above cover them)
@@ -400,9 +409,9 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
 #pragma unroll
             for (int g4 = 0; g4 < 4; ++g4) asm volatile("" : "+v"(syh[j][g4]));
     }
-    static_for<0, TR + TC>([&](auto xc) __attribute__((always_inline)) { lfrag1(xc, C0{}, 0, 0); });
+    static_for<0, TR + TC>([&](auto xc) __attribute__((always_inline)) { lfrag1(xc, C0{}, ring0, 0); });
 
-    int cur = 0;
+    int cur = ring0;
     for (int it = 0; it < nk; ++it) {
         const int nxt = cur + 1 == NST ? 0 : cur + 1;
         static_for<0, KS - 1>([&](auto ksc) __attribute__((always_inline)) {
@@ -414,22 +423,25 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
                   std::integral_constant<int, TR + TC>{});
         });
         __builtin_amdgcn_sched_barrier(0);
-        wait_vmcnt<(NST - 2) * CNT>();
+        if (NST == 2 || !deep) wait_vmcnt<0>();
+        else wait_vmcnt<(NST - 2) * CNT>();
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
-        const bool nx = ahead && it + NST >= nk;
-        const int kt2 = nx ? it + NST - nk : min(it + NST, nk - 1);
+        const bool nx = ahead && it + LD >= nk;
+        const int kt2 = nx ? it + LD - nk : min(it + LD, nk - 1);
+        const int tgt = cur + LD >= NST ? cur + LD - NST : cur + LD;       // the stage slab it + LD belongs to
         kstep(std::integral_constant<int, ((KS - 1) & 1)>{},
               [&](auto xc) __attribute__((always_inline)) {
                   constexpr int x = decltype(xc)::value;
                   if constexpr (x < TR + TC) lfrag1(xc, std::integral_constant<int, (KS & 1)>{}, nxt, 0);
-                  else dma1(std::integral_constant<int, x - (TR + TC)>{}, kt2, nx, cur);
+                  else dma1(std::integral_constant<int, x - (TR + TC)>{}, kt2, nx, tgt);
               },
               std::integral_constant<int, TR + TC + CNT>{});
         __builtin_amdgcn_sched_barrier(0);
         cur = nxt;
     }
     if (!ahead) wait_vmcnt<0>();         // drain the clamped loads before the ring is reused
+    ring = cur;                          // (ring0 + nk) % NST: where the next tile's slab 0 is, or will be put
 
     const int64_t obase = (int64_t)b * a.n * a.m;
     // Results leave through a 4 KB strip of LDS per wave: a lane holds 4-column pieces of ONE
@@ -504,14 +516,15 @@ __global__ __launch_bounds__(WR* WC * 64) void k_gemm_dma(DmaArgs da) {
     const uint32_t G = gridDim.x;
     const uint32_t w = (G % 8 == 0) ? (blockIdx.x % 8) * (G / 8) + blockIdx.x / 8 : blockIdx.x;
     bool have_slabs = false;
+    int ring = 0;
     GemmItem cur = gemm_item<BR, BC>(w, da);
     for (uint32_t L = w; cur.valid; L += G) {
         const GemmItem nxt = gemm_item<BR, BC>(L + G, da);
         if (HALVES && cur.half) {
             if constexpr (HALVES)
-                have_slabs = gemm_dma_tile<WR, WC, TR / 2, TC, BKB, EPI, NST>(da.g, smem, stg, lds_base, cur, nxt, have_slabs);
+                have_slabs = gemm_dma_tile<WR, WC, TR / 2, TC, BKB, EPI, NST>(da.g, smem, stg, lds_base, cur, nxt, have_slabs, ring);
         } else {
-            have_slabs = gemm_dma_tile<WR, WC, TR, TC, BKB, EPI, NST>(da.g, smem, stg, lds_base, cur, nxt, have_slabs);
+            have_slabs = gemm_dma_tile<WR, WC, TR, TC, BKB, EPI, NST>(da.g, smem, stg, lds_base, cur, nxt, have_slabs, ring);
         }
         cur = nxt;
     }
