@@ -253,10 +253,18 @@ __device__ __forceinline__ GemmItem gemm_item(uint32_t L, const DmaArgs& da) {
 // overlap this tile's stores; otherwise the slab index is clamped (a redundant load nobody
 // reads).  The ring position carries over from tile to tile (`ring`), so any slab count works.  Either way the loop body has no branches, which lets the compiler keep the
 // accumulators in place.  Returns true if the next tile's first slabs are on their way.
-template <int WR, int WC, int TR, int TC, int BKB, int EPI, int NST>
+//
+// LAY (fp16 only) marks operands whose rows are K instead: bit 0 = the row operand is stored
+// (K, n), bit 1 = the column operand is stored (K, m).  Such an operand's part of a stage holds
+// BKB/2 rows of K with the tile's BR (BC) halves each, DMA'd as they lie in memory; a lane then
+// collects its 8 halves of K with eight 2-byte LDS reads (32 lanes read 64 contiguous bytes: no
+// bank conflicts) instead of one 16-byte read.
+template <int WR, int WC, int TR, int TC, int BKB, int EPI, int NST, int LAY = 0>
 __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, int8_t* stg, uint32_t lds_base,
                                               const GemmItem cur_item, const GemmItem nxt_item, const bool have_slabs, int& ring) {
     constexpr bool FUSED = EPI == kEpiDequant, F16 = EPI == kEpiF16;
+    constexpr bool PT = (LAY & 1) != 0, QT = (LAY & 2) != 0;
+    static_assert(LAY == 0 || (F16 && BKB == 128), "transposed operands: fp16 with 64 halves of K per slab");
     using acc_t = std::conditional_t<F16, float16_tv, int16_tv>;
     constexpr int KS = BKB / 32, CPR = BKB / 16;
     constexpr int NW = WR * WC, BR = WR * TR * 32, BC = WC * TC * 32;
@@ -279,12 +287,12 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
 #pragma unroll
     for (int i = 0; i < TR; ++i) {
         const int r = wr * TR * 32 + i * 32 + lrow;
-        offP[i] = r * BKB + ((lk ^ swz(r)) << 4);
+        offP[i] = PT ? lk * 8 * (BR * 2) + r * 2 : r * BKB + ((lk ^ swz(r)) << 4);
     }
 #pragma unroll
     for (int j = 0; j < TC; ++j) {
         const int r = wc * TC * 32 + j * 32 + lrow;
-        offQ[j] = BR * BKB + r * BKB + ((lk ^ swz(r)) << 4);
+        offQ[j] = BR * BKB + (QT ? lk * 8 * (BC * 2) + r * 2 : r * BKB + ((lk ^ swz(r)) << 4));
     }
     // without slabs on their way the waits below count only loads: let the previous tile's stores finish first
     if (!have_slabs) wait_vmcnt<0>();
@@ -318,8 +326,20 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
         const int32_t grown = q ? min(nxt_item.i0 + (r - BR), a.m - 1) : min(nxt_item.j0 + r, a.n - 1);
         voff[d] = (uint32_t)grow * (uint32_t)K + c * 16;
         voffn[d] = (uint32_t)grown * (uint32_t)K + c * 16;
+        if ((PT && !q) || (QT && q)) {
+            // a (K, L) operand: the instruction covers 1024 / (2 * B) rows of K, a lane one 16-byte piece of a row
+            const int ppr = (q ? BC : BR) / 8;                     // pieces per row of K
+            const int dl = q ? dd - BR / RPI : dd;
+            const int kr = dl * (64 / ppr) + lane / ppr, pc = lane % ppr;
+            const int32_t L = q ? a.m : a.n;
+            const int32_t o = q ? i0 : j0, on = q ? nxt_item.i0 : nxt_item.j0;
+            voff[d] = ((uint32_t)kr * (uint32_t)L + (uint32_t)min(o + pc * 8, L - 8)) * 2u;      // L % 8 == 0
+            voffn[d] = ((uint32_t)kr * (uint32_t)L + (uint32_t)min(on + pc * 8, L - 8)) * 2u;
+        }
         ldst[d] = lds_base + dd * 1024;
     }
+    // bytes from one K slab to the next
+    const int64_t kstepP = PT ? (int64_t)BKB * a.n : BKB, kstepQ = QT ? (int64_t)BKB * a.m : BKB;
     // slab kt of this tile, or slab kt - nk of the next one (nx)
     auto dma1 = [&](auto dc, int kt, bool nx, int stage) __attribute__((always_inline)) {
         constexpr int d = decltype(dc)::value;
@@ -329,7 +349,7 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
         const bool q = isq[d];
         const int8_t* b0 = q ? qb : pb;
         const int8_t* b1 = q ? qn : pn;
-        lds_dma16(nx ? v1 : v0, (nx ? b1 : b0) + (int64_t)kt * BKB, ldst[d] + stage * STAGE);
+        lds_dma16(nx ? v1 : v0, (nx ? b1 : b0) + kt * (q ? kstepQ : kstepP), ldst[d] + stage * STAGE);
     };
 
     // the dequantisation scales of this lane's outputs, fetched now so that the epilogue does
@@ -361,10 +381,27 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
     int4_t fp[2][TR], fq[2][TC];
     auto lfrag1 = [&](auto xc, auto bufc, int stage, int ks) __attribute__((always_inline)) {
         constexpr int x = decltype(xc)::value, buf = decltype(bufc)::value;
-        if constexpr (x < TR)
-            fp[buf][x] = *reinterpret_cast<const int4_t*>(smem + stage * STAGE + (offP[x] ^ (ks << 5)));
-        else
-            fq[buf][x - TR] = *reinterpret_cast<const int4_t*>(smem + stage * STAGE + (offQ[x - TR] ^ (ks << 5)));
+        if constexpr (x < TR) {
+            if constexpr (PT) {
+                half8_t v;
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    v[e] = *reinterpret_cast<const half_t*>(smem + stage * STAGE + offP[x] + (ks * 16 + e) * (BR * 2));
+                fp[buf][x] = __builtin_bit_cast(int4_t, v);
+            } else {
+                fp[buf][x] = *reinterpret_cast<const int4_t*>(smem + stage * STAGE + (offP[x] ^ (ks << 5)));
+            }
+        } else {
+            if constexpr (QT) {
+                half8_t v;
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    v[e] = *reinterpret_cast<const half_t*>(smem + stage * STAGE + offQ[x - TR] + (ks * 16 + e) * (BC * 2));
+                fq[buf][x - TR] = __builtin_bit_cast(int4_t, v);
+            } else {
+                fq[buf][x - TR] = *reinterpret_cast<const int4_t*>(smem + stage * STAGE + (offQ[x - TR] ^ (ks << 5)));
+            }
+        }
     };
     // one k-step: NM MFMAs with NMEM memory operations spread evenly between them, order pinned
     auto kstep = [&](auto bufc, auto&& memop, auto nmem_c) __attribute__((always_inline)) {
@@ -505,8 +542,9 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
 // that at most half the workgroups could join, those tiles are issued as row halves (HALVES), one
 // per workgroup: a wave then owns TR/2 x TC MFMA tiles, which keeps the fragment reads per MFMA
 // lower than halving the columns would (TR/2 + TC reads for TR/2 * TC MFMAs per k-step).
-template <int WR, int WC, int TR, int TC, int BKB, int EPI, bool HALVES, int NST>
+template <int WR, int WC, int TR, int TC, int BKB, int EPI, bool HALVES, int NST, int LAY = 0>
 __global__ __launch_bounds__(WR* WC * 64) void k_gemm_dma(DmaArgs da) {
+    static_assert(!(HALVES && LAY != 0), "half tiles only with K-major operands");
     constexpr int BR = WR * TR * 32, BC = WC * TC * 32;
     extern __shared__ __attribute__((aligned(16))) int8_t smem[];
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) int8_t*)smem;
@@ -524,7 +562,7 @@ __global__ __launch_bounds__(WR* WC * 64) void k_gemm_dma(DmaArgs da) {
             if constexpr (HALVES)
                 have_slabs = gemm_dma_tile<WR, WC, TR / 2, TC, BKB, EPI, NST>(da.g, smem, stg, lds_base, cur, nxt, have_slabs, ring);
         } else {
-            have_slabs = gemm_dma_tile<WR, WC, TR, TC, BKB, EPI, NST>(da.g, smem, stg, lds_base, cur, nxt, have_slabs, ring);
+            have_slabs = gemm_dma_tile<WR, WC, TR, TC, BKB, EPI, NST, LAY>(da.g, smem, stg, lds_base, cur, nxt, have_slabs, ring);
         }
         cur = nxt;
     }
@@ -632,13 +670,13 @@ static int launch_kmajor(GemmArgs& a, int batch, hipStream_t st) {
 #define CPMK_GEMM_BIG 2, 4, 4, 2, 128
 #endif
 
-template <int WR, int WC, int TR, int TC, int BKB, int EPI, bool HALVES, int NST>
+template <int WR, int WC, int TR, int TC, int BKB, int EPI, bool HALVES, int NST, int LAY = 0>
 static int launch_dma_kernel(const DmaArgs& da, unsigned grid, hipStream_t st) {
     constexpr int BR = WR * TR * 32, BC = WC * TC * 32;
     constexpr int STRIP = TC * 64 * 32 > 4096 ? TC * 64 * 32 : 4096;
     constexpr int smem = NST * (BR + BC) * BKB + WR * WC * STRIP;      // operand ring + output strips
     static_assert(smem <= 160 * 1024, "LDS of one compute unit");
-    auto kern = k_gemm_dma<WR, WC, TR, TC, BKB, EPI, HALVES, NST>;
+    auto kern = k_gemm_dma<WR, WC, TR, TC, BKB, EPI, HALVES, NST, LAY>;
     static bool attr_set[64] = {false};       // dynamic LDS above 64 KB must be enabled per device
     int dev = 0;
     (void)hipGetDevice(&dev);
@@ -652,7 +690,7 @@ static int launch_dma_kernel(const DmaArgs& da, unsigned grid, hipStream_t st) {
     return launch_status();
 }
 
-template <int WR, int WC, int TR, int TC, int BKB, int EPI, int NST = 2>
+template <int WR, int WC, int TR, int TC, int BKB, int EPI, int NST = 2, int LAY = 0>
 static int launch_dma(GemmArgs& a, int batch, hipStream_t st) {
     constexpr int BR = WR * TR * 32, BC = WC * TC * 32;
     a.tiles_r = (int32_t)ceil_div(a.n, BR);
@@ -668,12 +706,14 @@ static int launch_dma(GemmArgs& a, int batch, hipStream_t st) {
     const int64_t r = total % grid;
     da.nfull = (uint32_t)total;
     da.nhalf = 0;
-    if (TR % 2 == 0 && r > 0 && 2 * r <= grid) {
-        da.nfull = (uint32_t)(total - r);
-        da.nhalf = (uint32_t)(2 * r);
-        return launch_dma_kernel<WR, WC, TR, TC, BKB, EPI, (TR % 2 == 0), NST>(da, (unsigned)grid, st);
+    if constexpr (TR % 2 == 0 && LAY == 0) {
+        if (r > 0 && 2 * r <= grid) {
+            da.nfull = (uint32_t)(total - r);
+            da.nhalf = (uint32_t)(2 * r);
+            return launch_dma_kernel<WR, WC, TR, TC, BKB, EPI, true, NST>(da, (unsigned)grid, st);
+        }
     }
-    return launch_dma_kernel<WR, WC, TR, TC, BKB, EPI, false, NST>(da, (unsigned)grid, st);
+    return launch_dma_kernel<WR, WC, TR, TC, BKB, EPI, false, NST, LAY>(da, (unsigned)grid, st);
 }
 
 template <bool FUSED>
@@ -807,6 +847,17 @@ static int gemm_f16_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, in
         const int64_t big = ceil_div(n, 256) * ceil_div(m, 256) * batch;
         if (big * 4 >= compute_units() * 3 && n > 128 && m > 128) return launch_dma<CPMK_GEMM_BIG, kEpiF16>(a, batch, st);
         return launch_dma<2, 2, 2, 2, 128, kEpiF16, CPMK_GEMM_NST_SMALL>(a, batch, st);
+    }
+    // an operand stored (K, rows): the tile kernel reads it as it lies, with 2-byte LDS reads for the fragments
+    if (!(p_kmajor && q_kmajor) && wide && k > 0 && (k % 64 == 0) && aligned16(A) && aligned16(B) && (p_kmajor || n % 8 == 0) &&
+        (int64_t)n * k * 2 < (1ll << 32) && (int64_t)m * k * 2 < (1ll << 32)) {
+        const int lay = (p_kmajor ? 0 : 1) | (q_kmajor ? 0 : 2);
+        const bool low = n <= 64;                // 64 x 256 tiles for few output rows (attention: probabilities x values)
+        switch (lay) {
+            case 1: return low ? launch_dma<1, 4, 2, 2, 128, kEpiF16, 3, 1>(a, batch, st) : launch_dma<CPMK_GEMM_BIG, kEpiF16, 2, 1>(a, batch, st);
+            case 2: return low ? launch_dma<1, 4, 2, 2, 128, kEpiF16, 3, 2>(a, batch, st) : launch_dma<CPMK_GEMM_BIG, kEpiF16, 2, 2>(a, batch, st);
+            default: return low ? launch_dma<1, 4, 2, 2, 128, kEpiF16, 3, 3>(a, batch, st) : launch_dma<CPMK_GEMM_BIG, kEpiF16, 2, 3>(a, batch, st);
+        }
     }
     dim3 grid((unsigned)ceil_div(m, 64), (unsigned)ceil_div(n, 64), (unsigned)batch);
     if (grid.y > 65535) return CPMK_ETOOBIG;

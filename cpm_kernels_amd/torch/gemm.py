@@ -179,15 +179,16 @@ def _transposed_copy(x: torch.Tensor) -> torch.Tensor:
 
 def gemm_pth_fp16(A: torch.Tensor, aT: bool, B: torch.Tensor, bT: bool) -> torch.Tensor:
     """reference: torch/gemm.py:189-203; operands are passed swapped to the kernel so that the
-    (M, N) result comes out row-major.  The MFMA tile kernel needs both operands with K as the
-    contiguous dimension (A as (b, M, K), B as (b, N, K)); an operand given the other way round
-    is copied transposed first when the shape qualifies for that kernel (K a multiple of 64, N of
-    8), which costs one pass over it instead of the many of the general kernel."""
+    (M, N) result comes out row-major.  The MFMA tile kernel is fastest with K as the contiguous
+    dimension of both operands (A as (b, M, K), B as (b, N, K)).  An operand given the other way
+    round is read as it lies (2-byte LDS reads build the MFMA fragments, 20-60 % more time in
+    the product) unless the product is so large next to the operand that one transposed copy of it
+    is cheaper: measured break-even at about 2048 rows of the other operand for B, 512 for A."""
     M, K, N = _dims(A, B, aT, bT)
     if K % 64 == 0 and N % 8 == 0 and M * K < 2 ** 31 and N * K < 2 ** 31:
-        if aT:
+        if aT and (N > 512 or M % 8 != 0):
             A, aT = _transposed_copy(A), False
-        if not bT:
+        if not bT and M > 2048:
             B, bT = _transposed_copy(B), True
     out = torch.empty((max(A.size(0), B.size(0)), M, N), dtype=torch.half, device=A.device)
     gemm_fp16(N, K, M, B.size(0), A.size(0), bT, aT, B.data_ptr(), A.data_ptr(), out.data_ptr(), cur_stream())

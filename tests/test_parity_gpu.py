@@ -646,7 +646,10 @@ def test_elementwise(gpu, shape):
 # fp16 products next to the path (fp32 accumulation; the bar is the 1e-3 of fp16 outputs)
 # ---------------------------------------------------------------------------------------------
 F16_GEMM_CASES = [  # (batch, n, k, m) in the kernel's convention: out (batch, n, m)
-    (1, 4, 4, 4), (2, 6, 10, 8), (3, 34, 64, 20), (2, 256, 128, 260), (1, 512, 1024, 384), (2, 130, 192, 70)]
+    (1, 4, 4, 4), (2, 6, 10, 8), (3, 34, 64, 20), (2, 256, 128, 260), (1, 512, 1024, 384), (2, 130, 192, 70),
+    # shapes the MFMA tile kernel takes in every layout (k % 64 == 0, m % 8 == 0; n % 8 == 0 for a (k, n) operand):
+    # few rows (64 x 256 tiles) and many, ragged edges, one and several slabs of K
+    (2, 64, 128, 264), (3, 40, 192, 1032), (2, 60, 128, 264), (2, 264, 320, 520), (1, 136, 64, 256), (2, 24, 64, 8)]
 
 
 @pytest.mark.parametrize("case", F16_GEMM_CASES)
