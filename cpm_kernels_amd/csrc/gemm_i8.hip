@@ -308,48 +308,54 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
     const bool deep = nk >= NST;
     const int LD = deep ? NST : nk;
     const int ring0 = __builtin_amdgcn_readfirstlane(ring);
-    const int8_t* Pn = a.P + (int64_t)nxt_item.b * a.strideP;
-    const int8_t* Qn = a.Q + (int64_t)nxt_item.b * a.strideQ;
+    // what the last LD iterations fetch: the next tile's first slabs, or (not ahead) this tile's last slab again
+    const uint32_t tb = ahead ? nxt_item.b : b;
+    const int32_t tj0 = ahead ? nxt_item.j0 : j0, ti0 = ahead ? nxt_item.i0 : i0;
+    const int8_t* Pn = a.P + (int64_t)tb * a.strideP;
+    const int8_t* Qn = a.Q + (int64_t)tb * a.strideQ;
 
     // this wave's DMA instructions: d -> stage rows [RPI*dd, RPI*dd + RPI), dd = wave + d*NW;
     // rows past the matrix are clamped (they only feed outputs that are never stored)
-    uint32_t voff[CNT], voffn[CNT], ldst[CNT];
+    uint32_t voff[CNT], ldst[CNT];
     bool isq[CNT];
-#pragma unroll
-    for (int d = 0; d < CNT; ++d) {
+    // byte offset of this lane's 16 bytes inside slab 0 of the tile at rows oj / columns oi
+    auto calc_voff = [&](int d, int32_t oj, int32_t oi) __attribute__((always_inline)) -> uint32_t {
         const int dd = wave + d * NW;
         const int r = dd * RPI + lane / CPR;
         const int c = (lane % CPR) ^ swz(r);
         const bool q = dd * RPI >= BR;
-        isq[d] = q;
-        const int32_t grow = q ? min(i0 + (r - BR), a.m - 1) : min(j0 + r, a.n - 1);
-        const int32_t grown = q ? min(nxt_item.i0 + (r - BR), a.m - 1) : min(nxt_item.j0 + r, a.n - 1);
-        voff[d] = (uint32_t)grow * (uint32_t)K + c * 16;
-        voffn[d] = (uint32_t)grown * (uint32_t)K + c * 16;
         if ((PT && !q) || (QT && q)) {
             // a (K, L) operand: the instruction covers 1024 / (2 * B) rows of K, a lane one 16-byte piece of a row
             const int ppr = (q ? BC : BR) / 8;                     // pieces per row of K
             const int dl = q ? dd - BR / RPI : dd;
             const int kr = dl * (64 / ppr) + lane / ppr, pc = lane % ppr;
             const int32_t L = q ? a.m : a.n;
-            const int32_t o = q ? i0 : j0, on = q ? nxt_item.i0 : nxt_item.j0;
-            voff[d] = ((uint32_t)kr * (uint32_t)L + (uint32_t)min(o + pc * 8, L - 8)) * 2u;      // L % 8 == 0
-            voffn[d] = ((uint32_t)kr * (uint32_t)L + (uint32_t)min(on + pc * 8, L - 8)) * 2u;
+            return ((uint32_t)kr * (uint32_t)L + (uint32_t)min((q ? oi : oj) + pc * 8, L - 8)) * 2u;      // L % 8 == 0
         }
+        const int32_t grow = q ? min(oi + (r - BR), a.m - 1) : min(oj + r, a.n - 1);
+        return (uint32_t)grow * (uint32_t)K + c * 16;
+    };
+#pragma unroll
+    for (int d = 0; d < CNT; ++d) {
+        const int dd = wave + d * NW;
+        isq[d] = dd * RPI >= BR;
+        voff[d] = calc_voff(d, j0, i0);
         ldst[d] = lds_base + dd * 1024;
     }
     // bytes from one K slab to the next
     const int64_t kstepP = PT ? (int64_t)BKB * a.n : BKB, kstepQ = QT ? (int64_t)BKB * a.m : BKB;
-    // slab kt of this tile, or slab kt - nk of the next one (nx)
-    auto dma1 = [&](auto dc, int kt, bool nx, int stage) __attribute__((always_inline)) {
+    // One DMA instruction of slab kt: of this tile's rows, or (TAIL) of the rows the last LD iterations
+    // fetch -- the next tile's when it is fetched ahead, else this tile's again.  Which one
+    // is a compile-time choice: a run-time select here makes the compiler branch inside the K loop,
+    // which splits its body and breaks the MFMA/memory interleave.
+    auto dma1 = [&](auto dc, int kt, auto tailc, int stage) __attribute__((always_inline)) {
         constexpr int d = decltype(dc)::value;
+        constexpr bool TAIL = decltype(tailc)::value;
         // read every candidate first and select values, never addresses of the captured variables
-        const int8_t *pb = Pb, *qb = Qb, *pn = Pn, *qn = Qn;
-        const uint32_t v0 = voff[d], v1 = voffn[d];
+        const int8_t *pb = TAIL ? Pn : Pb, *qb = TAIL ? Qn : Qb;
+        const uint32_t v = voff[d];            // (rewritten for the tail between the two loops)
         const bool q = isq[d];
-        const int8_t* b0 = q ? qb : pb;
-        const int8_t* b1 = q ? qn : pn;
-        lds_dma16(nx ? v1 : v0, (nx ? b1 : b0) + kt * (q ? kstepQ : kstepP), ldst[d] + stage * STAGE);
+        lds_dma16(v, (q ? qb : pb) + kt * (q ? kstepQ : kstepP), ldst[d] + stage * STAGE);
     };
 
     // the dequantisation scales of this lane's outputs, fetched now so that the epilogue does
@@ -428,7 +434,7 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
         static_for<0, NST>([&](auto sc) __attribute__((always_inline)) {
             constexpr int st = decltype(sc)::value;
             static_for<0, CNT>([&](auto dc) __attribute__((always_inline)) {
-                dma1(dc, min(st, nk - 1), false, (ring0 + st) % NST);
+                dma1(dc, min(st, nk - 1), std::false_type{}, (ring0 + st) % NST);
             });
         });
         if (deep) wait_vmcnt<(NST - 1) * CNT>();   // slab 0 (and the scale loads issued before it) has landed
@@ -445,11 +451,21 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
         for (int j = 0; j < TC; ++j)
 #pragma unroll
             for (int g4 = 0; g4 < 4; ++g4) asm volatile("" : "+v"(syh[j][g4]));
+        // parked in this wave's output strip, idle until the epilogue: 20 fewer registers live across the K loop
+#pragma unroll
+        for (int i = 0; i < TR; ++i) *reinterpret_cast<half_t*>(stg + (i * 64 + lane) * 2) = sxh[i];
+#pragma unroll
+        for (int j = 0; j < TC; ++j)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) *reinterpret_cast<half4_t*>(stg + 1024 + lk * 64 + (j * 4 + g4) * 8) = syh[j][g4];
     }
     static_for<0, TR + TC>([&](auto xc) __attribute__((always_inline)) { lfrag1(xc, C0{}, ring0, 0); });
 
     int cur = ring0;
-    for (int it = 0; it < nk; ++it) {
+    // tail slab index: it + LD - nk of the next tile, or nk - 1 of this one
+    const int tmul = ahead ? 1 : 0, tadd = ahead ? LD - nk : nk - 1;
+    auto slab = [&](int it, auto tailc) __attribute__((always_inline)) {
+        constexpr bool TAIL = decltype(tailc)::value;
         const int nxt = cur + 1 == NST ? 0 : cur + 1;
         static_for<0, KS - 1>([&](auto ksc) __attribute__((always_inline)) {
             constexpr int ks = decltype(ksc)::value;
@@ -460,23 +476,26 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
                   std::integral_constant<int, TR + TC>{});
         });
         __builtin_amdgcn_sched_barrier(0);
-        if (NST == 2 || !deep) wait_vmcnt<0>();
-        else wait_vmcnt<(NST - 2) * CNT>();
+        wait_vmcnt<(NST - 2) * CNT>();       // slab it + 1 has landed (with fewer slabs than stages it had before the loop)
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
-        const bool nx = ahead && it + LD >= nk;
-        const int kt2 = nx ? it + LD - nk : min(it + LD, nk - 1);
+        const int kt2 = TAIL ? it * tmul + tadd : it + LD;
         const int tgt = cur + LD >= NST ? cur + LD - NST : cur + LD;       // the stage slab it + LD belongs to
         kstep(std::integral_constant<int, ((KS - 1) & 1)>{},
               [&](auto xc) __attribute__((always_inline)) {
                   constexpr int x = decltype(xc)::value;
                   if constexpr (x < TR + TC) lfrag1(xc, std::integral_constant<int, (KS & 1)>{}, nxt, 0);
-                  else dma1(std::integral_constant<int, x - (TR + TC)>{}, kt2, nx, tgt);
+                  else dma1(std::integral_constant<int, x - (TR + TC)>{}, kt2, tailc, tgt);
               },
               std::integral_constant<int, TR + TC + CNT>{});
         __builtin_amdgcn_sched_barrier(0);
         cur = nxt;
-    }
+    };
+    int it = 0;
+    for (; it < nk - LD; ++it) slab(it, std::false_type{});       // slabs LD .. nk-1 of this tile follow
+#pragma unroll
+    for (int d = 0; d < CNT; ++d) voff[d] = calc_voff(d, tj0, ti0);
+    for (; it < nk; ++it) slab(it, std::true_type{});             // then the tail's
     if (!ahead) wait_vmcnt<0>();         // drain the clamped loads before the ring is reused
     ring = cur;                          // (ring0 + nk) % NST: where the next tile's slab 0 is, or will be put
 
@@ -492,10 +511,26 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
     constexpr int RB = CT * 32 * ESZ, PPR = RB / 16, RPW2 = 256 / RB, PASSES = PPR / 2, RPP = 64 / PPR;
     // 16-byte piece p of strip row r sits at piece slot p ^ ((r / RPW2) % PPR): reads are conflict free
     auto slot = [](int r, int p) __attribute__((always_inline)) { return (p ^ ((r / RPW2) & (PPR - 1))) << 4; };
+    half_t sxr[TR];
+    half4_t syr[TC][4];
+    if (FUSED) {      // the scales come back from the strip before the results overwrite it
+#pragma unroll
+        for (int i = 0; i < TR; ++i) sxr[i] = *reinterpret_cast<const half_t*>(stg + (i * 64 + lane) * 2);
+#pragma unroll
+        for (int j = 0; j < TC; ++j)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) syr[j][g4] = *reinterpret_cast<const half4_t*>(stg + 1024 + lk * 64 + (j * 4 + g4) * 8);
+#pragma unroll
+        for (int i = 0; i < TR; ++i) asm volatile("" : "+v"(sxr[i]));
+#pragma unroll
+        for (int j = 0; j < TC; ++j)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) asm volatile("" : "+v"(syr[j][g4]));
+    }
 #pragma unroll
     for (int i = 0; i < TR; ++i) {
         float sx = 0.0f;
-        if (FUSED) sx = (float)sxh[i];
+        if (FUSED) sx = (float)sxr[i];
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
             if constexpr (EPI == kEpiInt32) {
@@ -515,7 +550,7 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
 #pragma unroll
                             for (int e = 0; e < 4; ++e) h[e] = (half_t)acc[i][j][g4 * 4 + e];
                         } else {
-                            const half4_t sy = syh[j][g4];
+                            const half4_t sy = syr[j][g4];
 #pragma unroll
                             for (int e = 0; e < 4; ++e) h[e] = dequant(acc[i][j][g4 * 4 + e], sx, (float)sy[e]);
                         }
