@@ -248,11 +248,13 @@ __device__ __forceinline__ GemmItem gemm_item(uint32_t L, const DmaArgs& da) {
 //                                      nobody reads stage cur any more
 //   k-step KS-1       : MFMAs while the step-0 fragments of slab it+1 are read and the DMA of
 //                       slab it+NST is issued into stage cur
-// Past the end of K the DMA fetches the first slabs of the NEXT tile of this workgroup (when it
-// has the same shape), so that tile starts with its operands already in LDS and the loads
-// overlap this tile's stores; otherwise the slab index is clamped (a redundant load nobody
-// reads).  The ring position carries over from tile to tile (`ring`), so any slab count works.  Either way the loop body has no branches, which lets the compiler keep the
-// accumulators in place.  Returns true if the next tile's first slabs are on their way.
+// The last iterations (the "tail", a second copy of the loop body) fetch the first slabs of the
+// NEXT tile of this workgroup when it has the same shape, so that tile starts with its operands
+// already in LDS and the loads overlap this tile's stores; otherwise they fetch this tile's last
+// slab again (a redundant load nobody reads).  The ring position carries over from tile to tile
+// (`ring`), so any slab count works.  Each loop body is one basic block without selects, which
+// lets the compiler keep the accumulators in place and the MFMA/memory interleave as written.
+// Returns true if the next tile's first slabs are on their way.
 //
 // LAY (fp16 only) marks operands whose rows are K instead: bit 0 = the row operand is stored
 // (K, n), bit 1 = the column operand is stored (K, m).  Such an operand's part of a stage holds
