@@ -185,20 +185,6 @@ __device__ __forceinline__ void static_for(F&& f) {
     }
 }
 
-// 16 bytes per lane from global memory straight into LDS.  The LDS address is m0 + lane*16,
-// so one wave instruction fills 1 KB of contiguous LDS; the swizzle is applied by choosing
-// which global chunk each lane fetches.  Inline asm because the compiler would otherwise
-// guard every later LDS read with vmcnt(0), which serialises the prefetch.
-__device__ __forceinline__ void lds_dma16(uint32_t voff, const int8_t* sbase, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr)
-                 : "memory");
-}
-// s_waitcnt vmcnt(N) only (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14)
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
-}
-
 // What the tile kernel does with its accumulators.
 constexpr int kEpiInt32 = 0;     // int8 product, int32 out
 constexpr int kEpiDequant = 1;   // int8 product, fp16( (f32(acc) * s_row) * s_col ) out

@@ -13,25 +13,9 @@ constexpr float kLog2e = 1.4426950408889634f;
 // exp(x - M) as one fma and one v_exp_f32: exp2(x*log2e - M*log2e).
 __device__ inline float exp_shift(float x, float mlog2e) { return __builtin_amdgcn_exp2f(__builtin_fmaf(x, kLog2e, -mlog2e)); }
 
-// Register-resident column tile: HBM is read once and exp is evaluated once per element.  The
-// kernel is co-limited by HBM and by the VALU (v_exp_f32 is a quarter-rate instruction), so the
-// arithmetic is kept lean: column maxima on the packed fp16 inputs (exact), one fused
-// multiply-add and one exp2 per element, and a 16-byte piece whose 8 inputs are all -inf for
-// every lane of the wave (whole rows masked out, as in causal attention) is skipped -- its
-// exponentials are exactly 0.
+// The softmax of the columns of one register-resident tile, in place in v (rows past n hold -inf).
 template <int NT, int LPR, int R>
-__global__ __launch_bounds__(NT) void k_softmax_tile(int32_t n, int32_t m, int32_t tiles_per_batch,
-                                                     const half_t* inp, half_t* out) {
-    using T = ColTile<NT, LPR, R>;
-    __shared__ float lds[(T::NW + 1) * T::COLS];
-    const uint32_t t = xcd_remap(blockIdx.x, gridDim.x);
-    const uint32_t b = t / tiles_per_batch, ct = t - b * tiles_per_batch;
-    const int32_t col0 = ct * T::COLS + (threadIdx.x % LPR) * 8;
-    const int64_t boff = (int64_t)b * n * m;
-
-    half8_t v[R];
-    coltile_load<NT, LPR, R>(v, inp + boff, n, m, col0, (half_t)(-__builtin_inff()));
-
+__device__ __forceinline__ void softmax_cols(half8_t (&v)[R], float* lds) {
     half8_t hm = v[0];
 #pragma unroll
     for (int p = 1; p < R; ++p) hm = __builtin_elementwise_max(hm, v[p]);
@@ -68,7 +52,118 @@ __global__ __launch_bounds__(NT) void k_softmax_tile(int32_t n, int32_t m, int32
     for (int p = 0; p < R; ++p)
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[p][e] = round_f16(ex[p][e] * s[e]);
+}
+
+// Register-resident column tile: HBM is read once and exp is evaluated once per element.  The
+// kernel is co-limited by HBM and by the VALU (v_exp_f32 is a quarter-rate instruction), so the
+// arithmetic is kept lean: column maxima on the packed fp16 inputs (exact), one fused
+// multiply-add and one exp2 per element, and a 16-byte piece whose 8 inputs are all -inf for
+// every lane of the wave (whole rows masked out, as in causal attention) is skipped -- its
+// exponentials are exactly 0.
+template <int NT, int LPR, int R>
+__global__ __launch_bounds__(NT) void k_softmax_tile(int32_t n, int32_t m, int32_t tiles_per_batch,
+                                                     const half_t* inp, half_t* out) {
+    using T = ColTile<NT, LPR, R>;
+    __shared__ float lds[(T::NW + 1) * T::COLS];
+    const uint32_t t = xcd_remap(blockIdx.x, gridDim.x);
+    const uint32_t b = t / tiles_per_batch, ct = t - b * tiles_per_batch;
+    const int32_t col0 = ct * T::COLS + (threadIdx.x % LPR) * 8;
+    const int64_t boff = (int64_t)b * n * m;
+
+    half8_t v[R];
+    coltile_load<NT, LPR, R>(v, inp + boff, n, m, col0, (half_t)(-__builtin_inff()));
+
+    softmax_cols<NT, LPR, R>(v, lds);
     coltile_store<NT, LPR, R>(v, out + boff, n, m, col0);
+}
+
+// The same for many tiles per compute unit: persistent workgroups, each wave fetching its share
+// of the NEXT tile straight into LDS (global_load_lds, 1 KB per wave instruction, no registers)
+// while the current tile is reduced, exponentiated and stored.  A lane reads back exactly the 16
+// bytes it requested, so the staging needs no barrier, only the wave's own vmcnt; the wait sits
+// in front of the current tile's stores, where the loads issued a whole compute phase earlier
+// have landed, and the stores then drain under the next tile.
+//
+// Tiles are handed out dynamically: the first gridDim.x tiles by workgroup index, the rest from a
+// counter in device memory.  With a fixed share per workgroup the kernel ends with its slowest
+// compute unit, and on this chip one in eight gets 25 % less memory bandwidth than the rest.
+// The workgroup that finishes last clears the counters, so a launch (or a graph replay) always
+// finds them zero; launches that may overlap in time use different counter slots.
+constexpr int kSmSlots = 64;
+__device__ unsigned int g_sm_sched[kSmSlots][2];       // [0] tiles handed out beyond the first round, [1] finished workgroups
+
+template <int NT, int LPR, int R>
+__global__ __launch_bounds__(NT) void k_softmax_stream(int32_t n, int32_t m, int32_t tiles_per_batch, uint32_t ntiles, uint32_t slot,
+                                                       const half_t* inp, half_t* out) {
+    using T = ColTile<NT, LPR, R>;
+    constexpr int RPP = NT / LPR;
+    extern __shared__ __attribute__((aligned(16))) int8_t dyn[];        // NT*R*16 bytes of staging, the reduction scratch, one word for the next tile
+    float* lds = reinterpret_cast<float*>(dyn + NT * R * 16);
+    uint32_t* s_next = reinterpret_cast<uint32_t*>(lds + (T::NW + 1) * T::COLS);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int8_t* stage = dyn + wave * (R * 1024) + lane * 16;
+    const uint32_t stage_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) int8_t*)(dyn + wave * (R * 1024));
+    const uint32_t G = gridDim.x;
+    unsigned int* ctr = &g_sm_sched[slot][0];
+    const int rg = tid / LPR, cg = tid % LPR;
+    auto issue = [&](uint32_t t) __attribute__((always_inline)) {
+        const uint32_t b = t / tiles_per_batch, ct = t - b * tiles_per_batch;
+        const int32_t cc = min((int32_t)(ct * T::COLS + cg * 8), m - 8);          // clamped: lanes past the edge are refilled below
+        const int8_t* base = reinterpret_cast<const int8_t*>(inp + (int64_t)b * n * m);
+#pragma unroll
+        for (int p = 0; p < R; ++p) {
+            const int32_t row = min(p * RPP + rg, n - 1);
+            lds_dma16(((uint32_t)row * (uint32_t)m + (uint32_t)cc) * 2u, base, stage_addr + p * 1024);
+        }
+    };
+    uint32_t t = blockIdx.x;                       // gridDim.x <= ntiles
+    issue(t);
+    if (tid == 0) *s_next = G + atomicAdd(ctr, 1u);
+    wait_vmcnt<0>();
+    __syncthreads();
+    uint32_t tn = __builtin_amdgcn_readfirstlane(*s_next);
+    while (t < ntiles) {
+        const uint32_t b = t / tiles_per_batch, ct = t - b * tiles_per_batch;
+        const int32_t col0 = ct * T::COLS + cg * 8;
+        const int64_t boff = (int64_t)b * n * m;
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        half8_t v[R];
+#pragma unroll
+        for (int p = 0; p < R; ++p) {
+            half8_t x = *reinterpret_cast<const half8_t*>(stage + p * 1024);
+            if (!(p * RPP + rg < n && col0 < m)) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[e] = (half_t)(-__builtin_inff());
+            }
+            v[p] = x;
+        }
+#pragma unroll
+        for (int p = 0; p < R; ++p) asm volatile("" : "+v"(v[p]));      // the reads are done before the staging is refilled
+        __builtin_amdgcn_sched_barrier(0);
+        if (tn < ntiles) issue(tn);
+        uint32_t after = 0;
+        if (tid == 0) after = G + atomicAdd(ctr, 1u);                   // the tile after the next; used only after the arithmetic
+        __builtin_amdgcn_sched_barrier(0);
+        softmax_cols<NT, LPR, R>(v, lds);
+        __builtin_amdgcn_sched_barrier(0);
+        wait_vmcnt<0>();            // the next tile has landed; the previous tile's stores finished long ago
+        if (tid == 0) *s_next = after;
+        __syncthreads();
+        const uint32_t tnn = __builtin_amdgcn_readfirstlane(*s_next);
+        __builtin_amdgcn_sched_barrier(0);
+        coltile_store<NT, LPR, R>(v, out + boff, n, m, col0);
+        t = tn;
+        tn = tnn;
+    }
+    // every workgroup is past its last fetch when it signs off, so the last one to do so may clear the slot
+    if (tid == 0) {
+        if (atomicAdd(&g_sm_sched[slot][1], 1u) == G - 1) {
+            atomicExch(&g_sm_sched[slot][0], 0u);
+            atomicExch(&g_sm_sched[slot][1], 0u);
+        }
+    }
 }
 
 // Columns too tall for one workgroup's registers at 128-byte row segments: the n rows of a
@@ -222,6 +317,30 @@ static void launch_tile(int32_t batch, int32_t n, int32_t m, const half_t* inp, 
                        tiles, inp, out);
 }
 
+// persistent variant: one workgroup per compute unit, 16 bytes of LDS staging per element slot
+template <int NT, int LPR, int R>
+static int launch_stream(int32_t batch, int32_t n, int32_t m, const half_t* inp, half_t* out, hipStream_t st) {
+    using T = ColTile<NT, LPR, R>;
+    constexpr int smem = NT * R * 16 + (T::NW + 1) * T::COLS * (int)sizeof(float) + 16;
+    static_assert(smem <= 160 * 1024, "LDS of one compute unit");
+    auto kern = k_softmax_stream<NT, LPR, R>;
+    static bool attr_set[64] = {false};       // dynamic LDS above 64 KB must be enabled per device
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    if (dev >= 0 && dev < 64 && !attr_set[dev]) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+        if (e != hipSuccess) return (int)e;
+        attr_set[dev] = true;
+    }
+    const int32_t tiles = (int32_t)ceil_div(m, LPR * 8);
+    const int64_t ntiles = (int64_t)tiles * batch;
+    const int cus = compute_units();
+    static unsigned next_slot = 0;            // launches that may be in flight together get different scheduling counters
+    const unsigned slot = __atomic_fetch_add(&next_slot, 1u, __ATOMIC_RELAXED) % kSmSlots;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(ntiles < cus ? ntiles : cus)), dim3(NT), smem, st, n, m, tiles, (uint32_t)ntiles, slot, inp, out);
+    return launch_status();
+}
+
 template <int NT, int LPR>
 static bool launch_tile_r(int r, int32_t batch, int32_t n, int32_t m, const half_t* inp, half_t* out,
                           hipStream_t st) {
@@ -267,6 +386,10 @@ static int softmax_dispatch(int32_t batch, int32_t n, int32_t m, const void* inp
                 return launch_status();
             }
         }
+        // several tiles per compute unit: the persistent kernel keeps loads in flight during the arithmetic
+        if (n > 256 && n <= 1024 && m >= 64 && ceil_div(m, 64) * batch >= 2 * (int64_t)compute_units() &&
+            ceil_div(m, 64) * batch < (1ll << 31))
+            return n > 512 ? launch_stream<1024, 8, 8>(batch, n, m, x, y, st) : launch_stream<1024, 8, 4>(batch, n, m, x, y, st);
         if (n <= 64 * 8 && m >= 64) ok = launch_tile_r<512, 8>((int)ceil_div(n, 64), batch, n, m, x, y, st);
         else if (n <= 128 * 8 && m >= 64) ok = launch_tile_r<1024, 8>((int)ceil_div(n, 128), batch, n, m, x, y, st);
         else if (n <= 256 * 8 && m >= 32) ok = launch_tile_r<1024, 4>((int)ceil_div(n, 256), batch, n, m, x, y, st);
