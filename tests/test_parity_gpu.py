@@ -463,6 +463,58 @@ def test_team_kernels_in_a_replayed_graph(gpu):
         assert_close_fp16(got_sm, oracle.softmax_forward(sx), rtol=1e-3, atol=1e-7, what="replay %d softmax" % it)
 
 
+def test_scheduled_softmax_in_a_replayed_graph(gpu):
+    """The many-tile softmax hands out tiles from a counter in device memory that its last workgroup
+    clears.  Replays of a captured graph (same counter slot every time), launches back to back and
+    launches on two streams at once must each find a clean counter: every tile computed exactly once."""
+    _name("scheduled softmax, graph replay")
+    rng = np.random.default_rng(79)
+    shape = (36, 1000, 1024)                      # 576 tiles: more than two per compute unit
+    sin = torch.empty(shape, dtype=torch.half, device=gpu); sout = torch.empty_like(sin); sout2 = torch.empty_like(sin)
+
+    def launches():
+        ck.softmax_forward(*shape, sin.data_ptr(), sout.data_ptr(), stream())
+        ck.softmax_forward(*shape, sin.data_ptr(), sout2.data_ptr(), stream())
+
+    sin.normal_()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        launches()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        launches()
+    for it in range(4):
+        sx = (rng.standard_normal(shape) * 4).astype(np.float16)
+        sin.copy_(to_gpu(sx)); sout.zero_(); sout2.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        got, got2 = to_np(sout).copy(), to_np(sout2).copy()
+        assert_bits_equal(got, got2, "two launches of one replay (%d)" % it)
+        sout.zero_(); sout2.zero_()
+        for _ in range(3):
+            launches()                               # eager, back to back
+        assert_bits_equal(got, to_np(sout), "replay %d == eager" % it)
+        assert_bits_equal(got, to_np(sout2), "replay %d == eager (second output)" % it)
+        if it == 0:
+            assert_close_fp16(got, oracle.softmax_forward(sx), rtol=1e-3, atol=1e-7, max_ulp=2, what="scheduled softmax")
+    # two streams at once
+    other = torch.cuda.Stream()
+    other.wait_stream(torch.cuda.current_stream())
+    sout.zero_(); sout2.zero_()
+    torch.cuda.synchronize()
+    for _ in range(4):
+        ck.softmax_forward(*shape, sin.data_ptr(), sout.data_ptr(), stream())
+        with torch.cuda.stream(other):
+            ck.softmax_forward(*shape, sin.data_ptr(), sout2.data_ptr(), other.cuda_stream)
+    torch.cuda.synchronize()
+    assert_bits_equal(to_np(sout), got, "stream A")
+    assert_bits_equal(to_np(sout2), got, "stream B")
+
+
 @pytest.mark.parametrize("shape", [(8, 4096, 512), (3, 100, 40), (2, 777, 124), (2, 1024, 64)])
 @pytest.mark.parametrize("bias", [True, False])
 def test_layernorm_affine_fused(gpu, shape, bias):
