@@ -186,9 +186,9 @@ def gemm_pth_fp16(A: torch.Tensor, aT: bool, B: torch.Tensor, bT: bool) -> torch
     is cheaper: measured break-even at about 2048 rows of the other operand for B, 512 for A."""
     M, K, N = _dims(A, B, aT, bT)
     if K % 64 == 0 and N % 8 == 0 and M * K < 2 ** 31 and N * K < 2 ** 31:
-        if aT and (N > 512 or M % 8 != 0):
+        if aT and ((N > 512 and K > 128) or M % 8 != 0):     # (short K: the product is bound by writing its output)
             A, aT = _transposed_copy(A), False
-        if not bT and M > 2048:
+        if not bT and M > 2048 and K > 128:
             B, bT = _transposed_copy(B), True
     out = torch.empty((max(A.size(0), B.size(0)), M, N), dtype=torch.half, device=A.device)
     gemm_fp16(N, K, M, B.size(0), A.size(0), bT, aT, B.data_ptr(), A.data_ptr(), out.data_ptr(), cur_stream())
