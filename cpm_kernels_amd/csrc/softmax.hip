@@ -317,6 +317,9 @@ static void launch_tile(int32_t batch, int32_t n, int32_t m, const half_t* inp, 
                        tiles, inp, out);
 }
 
+// launches that may be in flight together get different scheduling counters (one sequence for all instantiations)
+static unsigned g_sm_next_slot = 0;
+
 // persistent variant: one workgroup per compute unit, 16 bytes of LDS staging per element slot
 template <int NT, int LPR, int R>
 static int launch_stream(int32_t batch, int32_t n, int32_t m, const half_t* inp, half_t* out, hipStream_t st) {
@@ -335,8 +338,7 @@ static int launch_stream(int32_t batch, int32_t n, int32_t m, const half_t* inp,
     const int32_t tiles = (int32_t)ceil_div(m, LPR * 8);
     const int64_t ntiles = (int64_t)tiles * batch;
     const int cus = compute_units();
-    static unsigned next_slot = 0;            // launches that may be in flight together get different scheduling counters
-    const unsigned slot = __atomic_fetch_add(&next_slot, 1u, __ATOMIC_RELAXED) % kSmSlots;
+    const unsigned slot = __atomic_fetch_add(&g_sm_next_slot, 1u, __ATOMIC_RELAXED) % kSmSlots;
     hipLaunchKernelGGL(kern, dim3((unsigned)(ntiles < cus ? ntiles : cus)), dim3(NT), smem, st, n, m, tiles, (uint32_t)ntiles, slot, inp, out);
     return launch_status();
 }

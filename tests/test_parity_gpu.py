@@ -545,7 +545,7 @@ SOFTMAX_SHAPES = [(1, 2, 32), (4, 128, 128), (4, 128, 16), (4, 123, 16), (16, 10
                   (3, 512, 64), (2, 2000, 48), (2, 4096, 16), (1, 5000, 24), (6, 333, 1), (2, 64, 200), (2, 2100, 64),
                   (1, 4096, 192), (1, 8192, 64), (1, 9000, 64),
                   # several tiles per compute unit: the persistent kernel (ragged rows, ragged last column tile)
-                  (40, 700, 1024), (64, 300, 520), (33, 1024, 1000), (600, 257, 64)]
+                  (40, 700, 1024), (64, 300, 520), (33, 1024, 1000), (600, 257, 64), (20, 1500, 1024), (70, 2048, 264)]
 
 
 @pytest.mark.parametrize("shape", SOFTMAX_SHAPES)
