@@ -22,6 +22,7 @@ __global__ __launch_bounds__(NT) void k_col_quantize_team(int32_t n, int32_t m, 
     constexpr int LPR = 8, R = 8, COLS = 64, ROWS = NT / LPR * R;
     __shared__ float lds[(NT / 64 + 1) * COLS];
     __shared__ float tot[COLS];
+    __shared__ __attribute__((aligned(16))) int8_t tbuf[COLS * ROWS];       // the transposed int8 tile on its way out
     const int tid = threadIdx.x, cg = tid % LPR, rg = tid / LPR;
     const uint32_t part = blockIdx.x % parts, team = blockIdx.x / parts;
     const uint32_t b = team / tiles_per_batch, ct = team - b * tiles_per_batch;
@@ -93,16 +94,45 @@ __global__ __launch_bounds__(NT) void k_col_quantize_team(int32_t n, int32_t m, 
                 if (row0 + p < n)
                     *reinterpret_cast<uint2_t*>(out + boff + ((uint32_t)(row0 + p) * (uint32_t)m + (uint32_t)col0)) =
                         uint2_t{q[p][0], q[p][1]};
-        } else if (row0 < n) {     // n % 8 == 0: the lane's 8 rows are in or out together
+        }
+    }
+    if (transposed) {
+        // The tile leaves through LDS as 64 columns x ROWS bytes: a lane's 8 rows of a column are 8
+        // bytes there, and 32 lanes then store one column's ROWS bytes as one contiguous run (16 bytes
+        // per lane) instead of eight lanes storing 64 bytes of it.  8-byte slot s of column c sits at
+        // slot s ^ ((c / 8) * 8): the 64 lanes of a writing wave cover every bank equally, and the
+        // 16-byte reads stay pairs of neighbouring slots.
+        static_assert(ROWS == 512, "one column of the tile is 64 slots of 8 bytes");
+        // 4x4 byte transposes with v_perm_b32 (selector bytes 0-3 pick from the second operand, 4-7 from
+        // the first): tr[h][e4][k] = rows 4k .. 4k+3 of column 4h + e4
+        uint32_t tr[2][4][2];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                uint32_t lo = 0, hi = 0;       // byte p = row p of column e
+        for (int h = 0; h < 2; ++h)
 #pragma unroll
-                for (int p = 0; p < 4; ++p) {
-                    lo |= ((q[p][e >> 2] >> ((e & 3) * 8)) & 0xffu) << (p * 8);
-                    hi |= ((q[p + 4][e >> 2] >> ((e & 3) * 8)) & 0xffu) << (p * 8);
-                }
-                *reinterpret_cast<uint2_t*>(out + boff + ((uint32_t)(col0 + e) * (uint32_t)n + (uint32_t)row0)) = uint2_t{lo, hi};
+            for (int k = 0; k < 2; ++k) {
+                const uint32_t r0 = q[4 * k][h], r1 = q[4 * k + 1][h], r2 = q[4 * k + 2][h], r3 = q[4 * k + 3][h];
+                const uint32_t a01 = __builtin_amdgcn_perm(r1, r0, 0x05010400u), b01 = __builtin_amdgcn_perm(r1, r0, 0x07030602u);
+                const uint32_t a23 = __builtin_amdgcn_perm(r3, r2, 0x05010400u), b23 = __builtin_amdgcn_perm(r3, r2, 0x07030602u);
+                tr[h][0][k] = __builtin_amdgcn_perm(a23, a01, 0x05040100u);
+                tr[h][1][k] = __builtin_amdgcn_perm(a23, a01, 0x07060302u);
+                tr[h][2][k] = __builtin_amdgcn_perm(b23, b01, 0x05040100u);
+                tr[h][3][k] = __builtin_amdgcn_perm(b23, b01, 0x07060302u);
+            }
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            *reinterpret_cast<uint2_t*>(tbuf + (cg * 8 + e) * ROWS + ((rg ^ (cg << 3)) << 3)) = uint2_t{tr[e >> 2][e & 3][0], tr[e >> 2][e & 3][1]};
+        __syncthreads();
+        const int piece = tid & 31;                                  // 16 rows of a column
+        const int32_t prow = part * ROWS + piece * 16;
+#pragma unroll
+        for (int ps = 0; ps < COLS / (NT / 32); ++ps) {
+            const int c = ps * (NT / 32) + (tid >> 5);
+            const int32_t col = ct * COLS + c;
+            const int4_t w = *reinterpret_cast<const int4_t*>(tbuf + c * ROWS + (((piece * 2) ^ ((c >> 3) << 3)) << 3));
+            int8_t* dst = out + boff + ((uint32_t)col * (uint32_t)n + (uint32_t)prow);
+            if (col < m) {             // n % 8 == 0: a piece is whole, half or not there
+                if (prow + 16 <= n) *reinterpret_cast<int4_t*>(dst) = w;
+                else if (prow + 8 <= n) *reinterpret_cast<uint2_t*>(dst) = uint2_t{(uint32_t)w.x, (uint32_t)w.y};
             }
         }
     }
