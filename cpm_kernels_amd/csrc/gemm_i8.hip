@@ -12,14 +12,16 @@
 // Three kernels, all exact (integer accumulation is order-independent, so the int32 result
 // equals the reference's bit for bit):
 //   k_gemm_dma     both operands K-major, k % 128 == 0: persistent workgroups walk the output
-//                  tiles; global memory goes straight into a two-stage, XOR-swizzled LDS ring
+//                  tiles; global memory goes straight into a ring of XOR-swizzled LDS stages
 //                  (global_load_lds_dwordx4), one barrier per 128-byte K slab, fragment double
 //                  buffering, v_mfma_i32_32x32x32_i8 with the operands swapped so that a lane
-//                  owns 4 consecutive output columns (8/16-byte stores).
+//                  owns 4 consecutive output columns; results leave through a per-wave LDS strip
+//                  as whole 128-byte lines.
 //   k_gemm_kmajor  both operands K-major, k % 16 == 0: register-staged 64-byte K slabs.
 //   k_gemm_generic any layout and size: LDS tiles + v_dot4_i32_i8.
 // The tile kernel also serves the fp16 product of kernels/gemm.py:188-256 (cpmk_gemm_fp16): the
-// same bytes of K per lane feed v_mfma_f32_32x32x16_f16, with fp32 accumulators.
+// same bytes of K per lane feed v_mfma_f32_32x32x16_f16, with fp32 accumulators; there it also
+// takes operands stored with K as the row index (template parameter LAY).
 #include "common.h"
 #include <type_traits>
 

@@ -2,7 +2,12 @@
 //   M = max(max_i x, -1e6);  S = sum_i exp(x - M) + 1e-10;  out = fp16(exp(x - M) / S)
 // (cuda/softmax.cu:6-43, :117-159).  A column that is entirely -inf therefore yields 0, not
 // NaN.  The reference reads the input three times and evaluates expf twice per element; the
-// tile kernel below reads once, evaluates exp once and keeps the results in registers.
+// tile kernels below read once, evaluate exp once and keep the results in registers:
+//   k_softmax_tile    one column tile per workgroup
+//   k_softmax_stream  many tiles per compute unit: persistent workgroups, next tile prefetched into
+//                     LDS by DMA, tiles handed out from a device-side counter
+//   k_softmax_team    columns too tall for one workgroup, shared by a team
+//   k_softmax_generic any shape;  k_softmax_rows  contiguous rows (decode step)
 #include "dim1.h"
 #include "exchange.h"
 
