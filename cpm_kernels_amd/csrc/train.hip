@@ -3,7 +3,8 @@
 // cuda/softmax.cu:86-114, cuda/position_bucket.cu:56-103, cuda/embedding.cu:38-88).  None of
 // them is on the inference hot path; they are written for coalesced 16-byte access and fp32
 // accumulation but not tuned further.
-#include "common.h"
+#include "dim1.h"
+#include "exchange.h"
 
 namespace cpmk {
 
@@ -217,6 +218,147 @@ __global__ __launch_bounds__(256) void k_col(ColArgs p) {
     }
 }
 
+// The same reductions with the tile in registers: 64 columns x 512 rows per workgroup (16-byte
+// loads, each input read once), taller columns shared by a team of up to 32 workgroups that
+// exchange their partial column statistics (exchange.h).  Used when the shape allows 16-byte
+// accesses; k_col above serves everything else.
+constexpr int kColTeamMaxParts = 32;
+
+template <int KIND>
+__global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_batch, int32_t parts, uint64_t* xch, uint32_t tag) {
+    constexpr int NT = 512, LPR = 8, R = 8;
+    using T = ColTile<NT, LPR, R>;
+    constexpr bool TWO = KIND != kLnFwdV && KIND != kLnFwdMV && KIND != kScaleRound;     // reads grad_in too
+    constexpr bool IS_MAX = KIND == kScaleRound;
+    constexpr int NV = IS_MAX ? 1 : 2;
+    __shared__ float lds[(T::NW + 1) * T::COLS * NV];
+    __shared__ float tot[T::COLS * 2];
+    const int tid = threadIdx.x, cg = tid % LPR, rg = tid / LPR;
+    const uint32_t part = blockIdx.x % parts, team = blockIdx.x / parts;
+    const uint32_t b = team / tiles_per_batch, ct = team - b * tiles_per_batch;
+    const int32_t col0 = ct * T::COLS + cg * 8;
+    const int32_t own0 = part * T::ROWS;
+    const int32_t own_n = min(T::ROWS, p.n - own0);
+    const int64_t boff = (int64_t)b * p.n * p.m + (int64_t)own0 * p.m;
+    const bool live = col0 < p.m;
+
+    half8_t va[R], vg[TWO ? R : 1];
+    coltile_load<NT, LPR, R>(va, p.a + boff, own_n, p.m, col0, (half_t)0.0f);
+    if constexpr (TWO) coltile_load<NT, LPR, R>(vg, p.g + boff, own_n, p.m, col0, (half_t)0.0f);
+    float mean[8], var[8], c3[8], sxv[R];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) mean[e] = var[e] = c3[e] = 0.0f;
+    if (live && (KIND == kLnBwdV || KIND == kLnBwdMV)) {
+        const half8_t hv = *reinterpret_cast<const half8_t*>(p.var + (int64_t)b * p.m + col0);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { var[e] = (float)hv[e]; c3[e] = -0.5f * var[e] * var[e] * var[e]; }
+    }
+    if (live && KIND == kLnBwdMV) {
+        const half8_t hm = *reinterpret_cast<const half8_t*>(p.mean + (int64_t)b * p.m + col0);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) mean[e] = (float)hm[e];
+    }
+#pragma unroll
+    for (int q = 0; q < R; ++q) {
+        sxv[q] = 0.0f;
+        if (KIND == kScaleRound) {
+            const int32_t row = own0 + q * T::RPP + rg;
+            if (row < p.n) sxv[q] = (float)p.sx[(p.bc ? 0 : (int64_t)b * p.n) + row];
+        }
+    }
+
+    float s[NV * 8];
+#pragma unroll
+    for (int e = 0; e < NV * 8; ++e) s[e] = 0.0f;
+#pragma unroll
+    for (int q = 0; q < R; ++q)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float x = (float)va[q][e];
+            const float gi = TWO ? (float)vg[TWO ? q : 0][e] : 0.0f;
+            if constexpr (KIND == kLnFwdV) s[8 + e] += x * x;
+            else if constexpr (KIND == kLnFwdMV) { s[e] += x; s[8 + e] += x * x; }
+            else if constexpr (KIND == kLnBwdV) s[e] += gi * c3[e] * x;
+            else if constexpr (KIND == kLnBwdMV) { s[e] += gi * c3[e] * (x - mean[e]); s[8 + e] += -gi * var[e]; }
+            else if constexpr (KIND == kSoftmaxBwd) s[e] += x * gi;
+            else s[e] = fmaxf(s[e], fabsf(x * sxv[q]));
+        }
+    coltile_reduce<NT, LPR, NV, IS_MAX>(s, lds);          // every lane: this part's statistics of its 8 columns
+
+    if (parts > 1) {
+        uint64_t* team_slots = xch + (size_t)team * parts * kXchVals;
+        if (tid < LPR) {
+#pragma unroll
+            for (int e = 0; e < NV * 8; ++e) xch_post(team_slots + (size_t)part * kXchVals, (e >> 3) * T::COLS + tid * 8 + (e & 7), s[e], tag);
+        }
+        if (tid < T::COLS * NV) {
+            const uint64_t deadline = wall_clock64() + kXchTimeoutTicks;
+            float acc = 0.0f;
+            bool ok = true;
+            for (int32_t q = 0; q < parts; ++q) {
+                float x;
+                ok &= xch_wait(team_slots + (size_t)q * kXchVals + tid, tag, deadline, x);
+                acc = IS_MAX ? fmaxf(acc, x) : acc + x;
+            }
+            tot[tid] = ok ? acc : __builtin_nanf("");
+        }
+        __syncthreads();
+#pragma unroll
+        for (int e = 0; e < NV * 8; ++e) s[e] = tot[(e >> 3) * T::COLS + cg * 8 + (e & 7)];
+    }
+
+    const float fn = (float)p.n;
+    float k0[8], k1[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        k0[e] = k1[e] = 0.0f;
+        if constexpr (KIND == kLnFwdV) k1[e] = rsqrtf(s[8 + e] / fn + p.eps);
+        else if constexpr (KIND == kLnFwdMV) { k0[e] = s[e] / fn; k1[e] = rsqrtf(s[8 + e] / fn - k0[e] * k0[e] + p.eps); }
+        else if constexpr (KIND == kLnBwdMV) s[8 + e] -= 2.0f * s[e] * mean[e];        // local_grad_mean -= 2 * local_grad_var * local_mean
+        else if constexpr (KIND == kScaleRound) k0[e] = (float)((double)s[e] / 127.0);     // float / double constant, as the reference writes it
+    }
+    if (live && part == 0 && rg == 0) {
+        half8_t h0, h1;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { h0[e] = (half_t)k0[e]; h1[e] = (half_t)k1[e]; }
+        if (KIND == kLnFwdV || KIND == kLnFwdMV) *reinterpret_cast<half8_t*>(p.out_var + (int64_t)b * p.m + col0) = h1;
+        if (KIND == kLnFwdMV) *reinterpret_cast<half8_t*>(p.out_mean + (int64_t)b * p.m + col0) = h0;
+        if (KIND == kScaleRound) *reinterpret_cast<half8_t*>(p.out_var + (int64_t)b * p.m + col0) = h0;
+    }
+    if constexpr (KIND == kScaleRound) {
+        if (live) {
+#pragma unroll
+            for (int q = 0; q < R; ++q) {
+                const int32_t lrow = q * T::RPP + rg;
+                if (lrow < own_n) {
+                    int32_t t[8];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) t[e] = quant_i8((float)va[q][e] * sxv[q], k0[e]);
+                    *reinterpret_cast<uint2_t*>(p.out_i8 + boff + ((uint32_t)lrow * (uint32_t)p.m + (uint32_t)col0)) =
+                        uint2_t{pack4_i8(t[0], t[1], t[2], t[3]), pack4_i8(t[4], t[5], t[6], t[7])};
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int q = 0; q < R; ++q)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float x = (float)va[q][e];
+                const float gi = TWO ? (float)vg[TWO ? q : 0][e] : 0.0f;
+                float o;
+                if constexpr (KIND == kLnFwdV) o = x * k1[e];
+                else if constexpr (KIND == kLnFwdMV) o = (x - k0[e]) * k1[e];
+                else if constexpr (KIND == kLnBwdV) o = gi * var[e] + (s[e] * x * 2.0f) / fn;
+                else if constexpr (KIND == kLnBwdMV) o = gi * var[e] + (s[8 + e] + s[e] * x * 2.0f) / fn;
+                else o = x * (gi - s[e]);
+                va[q][e] = round_f16(o);
+            }
+        coltile_store<NT, LPR, R>(va, p.out + boff, own_n, p.m, col0);
+    }
+    if (parts > 1 && tid < 64) xch_retire(xch, team, parts);
+}
+
 // cu_gemm_backward_round_scale: per-row absmax of mat * scale_y[col] -> scale_x, then rounding.
 __global__ __launch_bounds__(256) void k_round_scale_rows(int32_t n, int32_t m, const half_t* __restrict__ mat,
                                                           const half_t* __restrict__ scale_y, int8_t* __restrict__ out,
@@ -328,6 +470,23 @@ template <int KIND>
 static int launch_col(int32_t batch, const ColArgs& p, void* stream) {
     if (batch < 0 || p.n < 0 || p.m < 0) return CPMK_EBADARG;
     if ((int64_t)batch * p.n * p.m == 0) return 0;
+    // register-resident team kernel when every access can be 16 bytes wide (8 for the int8 output)
+    const int64_t tiles = ceil_div(p.m, 64), parts = ceil_div(p.n, 512);
+    const bool wide = p.m % 8 == 0 && aligned16(p.a) && (p.g == nullptr || aligned16(p.g)) && (p.out == nullptr || aligned16(p.out)) &&
+                      (p.mean == nullptr || aligned16(p.mean)) && (p.var == nullptr || aligned16(p.var)) &&
+                      (p.out_mean == nullptr || aligned16(p.out_mean)) && (p.out_var == nullptr || aligned16(p.out_var)) &&
+                      (p.out_i8 == nullptr || (reinterpret_cast<uintptr_t>(p.out_i8) & 7u) == 0) && (int64_t)p.n * p.m < (1ll << 31) &&
+                      parts <= kColTeamMaxParts && tiles * batch * parts <= kXchSlots;
+    if (wide) {
+        XchLaunch xl = {nullptr, 0};
+        if (parts > 1) {
+            const int rc = xch_begin(&xl);
+            if (rc != 0) return rc;
+        }
+        hipLaunchKernelGGL((k_col_team<KIND>), dim3((unsigned)(tiles * batch * parts)), dim3(512), 0, (hipStream_t)stream, p,
+                           (int32_t)tiles, (int32_t)parts, xl.region, xl.tag);
+        return launch_status();
+    }
     if (batch > 65535) return CPMK_ETOOBIG;
     hipLaunchKernelGGL((k_col<KIND>), dim3((unsigned)ceil_div(p.m, 64), (unsigned)batch), dim3(256), 0, (hipStream_t)stream, p);
     return launch_status();

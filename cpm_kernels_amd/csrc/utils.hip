@@ -46,6 +46,43 @@ __global__ __launch_bounds__(256) void k_transpose_wide(int32_t n, int32_t m, co
     }
 }
 
+// (batch, n, m) -> (batch, m, n) of bytes: 64x64 tile through LDS, 16-byte global accesses where
+// the shape allows (WIDE: n % 16 == 0, m % 16 == 0, aligned pointers), single bytes otherwise.
+template <bool WIDE>
+__global__ __launch_bounds__(256) void k_transpose_i8(int32_t n, int32_t m, const int8_t* __restrict__ in, int8_t* __restrict__ out) {
+    __shared__ __attribute__((aligned(16))) int8_t tile[64][68];        // pitch 68: dword-aligned rows, 17 banks apart
+    const int64_t boff = (int64_t)blockIdx.z * n * m;
+    const int32_t r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+    if (WIDE) {
+        const int pc = threadIdx.x & 3, rr = threadIdx.x >> 2;          // 4 pieces of 16 bytes x 64 rows
+        if (r0 + rr < n && c0 + pc * 16 < m) {
+            const uint4_t v = *reinterpret_cast<const uint4_t*>(in + boff + (int64_t)(r0 + rr) * m + c0 + pc * 16);
+            uint32_t* dst = reinterpret_cast<uint32_t*>(&tile[rr][pc * 16]);
+            dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
+        }
+        __syncthreads();
+        // row rr of the transposed tile = column rr of the tile; this thread's 16 bytes are its rows pc*16 .. pc*16+15
+        if (c0 + rr < m && r0 + pc * 16 < n) {
+            uint32_t w[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                uint32_t x = 0;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) x |= (uint32_t)(uint8_t)tile[pc * 16 + q * 4 + e][rr] << (8 * e);
+                w[q] = x;
+            }
+            *reinterpret_cast<uint4_t*>(out + boff + (int64_t)(c0 + rr) * n + r0 + pc * 16) = uint4_t{w[0], w[1], w[2], w[3]};
+        }
+    } else {
+        const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+        for (int r = ty; r < 64; r += 4)
+            if (r0 + r < n && c0 + tx < m) tile[r][tx] = in[boff + (int64_t)(r0 + r) * m + c0 + tx];
+        __syncthreads();
+        for (int c = ty; c < 64; c += 4)
+            if (c0 + c < m && r0 + tx < n) out[boff + (int64_t)(c0 + c) * n + r0 + tx] = tile[tx][c];
+    }
+}
+
 __global__ void k_array_add(int32_t* arr, int32_t pos, int32_t val) {
     if (threadIdx.x == 0) arr[pos] += val;
 }
@@ -99,6 +136,19 @@ int cpmk_transpose(int32_t batch, int32_t n, int32_t m, const void* inp, void* o
         hipLaunchKernelGGL(k_transpose_wide, grid, dim3(256), 0, (hipStream_t)stream, n, m, (const half_t*)inp, (half_t*)out);
     else
         hipLaunchKernelGGL(k_transpose, grid, dim3(256), 0, (hipStream_t)stream, n, m, (const half_t*)inp, (half_t*)out);
+    return launch_status();
+}
+
+int cpmk_transpose_i8(int32_t batch, int32_t n, int32_t m, const void* inp, void* out, void* stream) {
+    clear_stale_error();
+    if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
+    if ((int64_t)batch * n * m == 0) return 0;
+    if (batch > 65535 || ceil_div(n, 64) > 65535) return CPMK_ETOOBIG;
+    const dim3 grid((unsigned)ceil_div(m, 64), (unsigned)ceil_div(n, 64), (unsigned)batch);
+    if (n % 16 == 0 && m % 16 == 0 && aligned16(inp) && aligned16(out))
+        hipLaunchKernelGGL(k_transpose_i8<true>, grid, dim3(256), 0, (hipStream_t)stream, n, m, (const int8_t*)inp, (int8_t*)out);
+    else
+        hipLaunchKernelGGL(k_transpose_i8<false>, grid, dim3(256), 0, (hipStream_t)stream, n, m, (const int8_t*)inp, (int8_t*)out);
     return launch_status();
 }
 

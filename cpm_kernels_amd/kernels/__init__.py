@@ -17,6 +17,6 @@ from .layernorm import layernorm_forward, layernorm_inplace_forward, layernorm_f
 from .position_bucket import position_embedding_init, position_embedding_forward, position_embedding_backward, \
     position_embedding_step
 from .softmax import softmax_forward, softmax_backward, softmax_inplace_forward, softmax_step_inplace
-from .transpose import transpose
+from .transpose import transpose, transpose_i8
 from .utils import copy_data_to_kv, has_nan_inf
 from . import utils

@@ -9,7 +9,7 @@ the six-launch sequence, which ``fused=False`` still runs through the kernel-lev
 import torch
 from ..kernels import gemm_calc_scale, gemm_calc_scale_transpose, gemm_round, gemm_round_transpose, \
     gemm_scale, gemm_scale_x, gemm_scale_y, gemm_int8, gemm_int8_scale, gemm_quantize, gemm_quantize_cols, \
-    gemm_quantize_pair, gemm_fp16, gemm_backward_round_scale, gemm_backward_scale_round, transpose
+    gemm_quantize_pair, gemm_fp16, gemm_backward_round_scale, gemm_backward_scale_round, transpose, transpose_i8
 from ._common import cur_stream
 
 
@@ -73,11 +73,23 @@ def gemm_and_scale(quantA, scaleA, quantB, scaleB, aT, bT, fused=True) -> torch.
     M, K, N = _dims(quantA, quantB, aT, bT)
     batch = max(quantA.size(0), quantB.size(0))
     result_fp = torch.empty((batch, M, N), dtype=torch.float16, device=quantA.device)
-    if fused and scaleA is not None and scaleB is not None:
+    if fused:
+        # The MFMA tile kernel reads both operands with K contiguous; an int8 operand given the other
+        # way round (the backward products) costs one transposed copy, far less than the general kernel.
+        if aT:
+            quantA, aT = _transposed_copy_i8(quantA), False
+        if not bT:
+            quantB, bT = _transposed_copy_i8(quantB), True
+        # A missing scale is a vector of ones: (acc * s) * 1 rounds exactly as gemm_scale_x / gemm_scale_y
+        # do, and the int32 accumulators never travel through memory.
+        if scaleA is None:
+            scaleA = torch.ones((1, M), dtype=torch.half, device=quantA.device)
+        if scaleB is None:
+            scaleB = torch.ones((1, N), dtype=torch.half, device=quantA.device)
         gemm_int8_scale(N, K, M, quantB.size(0), quantA.size(0), bT, aT,
                         quantB.data_ptr(), quantA.data_ptr(),
                         scaleA.data_ptr(), scaleB.data_ptr(),
-                        quantA.size(0) == 1, quantB.size(0) == 1,
+                        scaleA.size(0) == 1, scaleB.size(0) == 1,
                         result_fp.data_ptr(), cur_stream())
         return result_fp
     result_i32 = torch.empty((batch, M, N), dtype=torch.int32, device=quantA.device)
@@ -169,6 +181,12 @@ class GEMMInt8(torch.autograd.Function):
         if ctx.layout[1] != bT:
             grad_B = grad_B.transpose(1, 2).contiguous()
         return grad_A, None, grad_B, None, None
+
+
+def _transposed_copy_i8(x: torch.Tensor) -> torch.Tensor:
+    out = torch.empty((x.size(0), x.size(2), x.size(1)), dtype=torch.int8, device=x.device)
+    transpose_i8(x.size(0), x.size(1), x.size(2), x.data_ptr(), out.data_ptr(), cur_stream())
+    return out
 
 
 def _transposed_copy(x: torch.Tensor) -> torch.Tensor:

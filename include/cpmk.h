@@ -315,6 +315,11 @@ int cpmk_embedding_backward_stage2(int32_t batch, int32_t hidden_size, const voi
 
 /* (batch, n, m) -> (batch, m, n), fp16.               kernels/transpose.py:11-29 / transpose.cu:6-24 */
 int cpmk_transpose(int32_t batch, int32_t n, int32_t m, const void* inp, void* out, void* stream);
+
+/* (batch, n, m) -> (batch, m, n), int8.  No counterpart in the reference, whose cuBLASLt call takes
+ * int8 operands in either layout (kernels/gemm.py:127-186): the backward products of
+ * torch/gemm.py:115-186 use this to bring their operands to the layout of the MFMA tile kernel. */
+int cpmk_transpose_i8(int32_t batch, int32_t n, int32_t m, const void* inp, void* out, void* stream);
 /* array[pos] += val (int32).                          kernels/utils.py:39-53 / utils.cu:31-35 */
 int cpmk_array_add(void* array, int32_t pos, int32_t val, void* stream);
 /* logits = logits / temperature - frequency_penalty*freq - presence_penalty*(freq > 0), in place.

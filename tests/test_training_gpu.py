@@ -266,6 +266,19 @@ def test_transpose(gpu, shape):
     assert_bits_equal(to_np(out), np.ascontiguousarray(x.transpose(0, 2, 1)), "transpose")
 
 
+@pytest.mark.parametrize("shape", [(2, 64, 64), (3, 17, 100), (1, 1000, 3), (2, 5, 7), (1, 4096, 512), (4, 1, 9),
+                                   (2, 80, 48), (1, 208, 144), (3, 16, 1040), (1, 10240, 4096)])
+def test_transpose_i8(gpu, shape):
+    _name("transpose_i8", shape)
+    b, n, m = shape
+    rng = np.random.default_rng(n * 37 + m)
+    x = rng.integers(-128, 128, size=(b, n, m), dtype=np.int8)
+    xd = torch.from_numpy(x).to(gpu)
+    out = torch.zeros((b, m, n), dtype=torch.int8, device=gpu)
+    ck.transpose_i8(b, n, m, xd.data_ptr(), out.data_ptr(), stream())
+    assert_bits_equal(to_np(out), np.ascontiguousarray(x.transpose(0, 2, 1)), "transpose_i8")
+
+
 def test_decode_utilities(gpu):
     _name("utils")
     rng = np.random.default_rng(11)
