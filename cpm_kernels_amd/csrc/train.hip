@@ -404,6 +404,70 @@ __global__ __launch_bounds__(256) void k_position_backward(int32_t query_len, in
     for (int i = threadIdx.x; i < num_buckets; i += 256) grad[(int64_t)h * num_buckets + i] = (half_t)hist[i];
 }
 
+// The same with the key rows of a head split over a team of workgroups (exchange.h; at most 128
+// buckets, the packets of one slot).  A thread walks down a column q of its rows: rel = q - k
+// falls by one per row, so the bucket changes rarely and the thread adds a whole run to the LDS
+// histogram at once.  Part 0 collects the partial histograms in part order and writes the result.
+__global__ __launch_bounds__(256) void k_position_backward_team(int32_t query_len, int32_t key_len, int32_t num_buckets,
+                                                                int32_t max_distance, const int32_t* __restrict__ mapping,
+                                                                const half_t* __restrict__ grad_out, half_t* __restrict__ grad,
+                                                                int bidirectional, int32_t parts, int32_t rows_per_part,
+                                                                uint64_t* xch, uint32_t tag) {
+    extern __shared__ float hist[];                       // num_buckets floats, then max_distance bucket numbers
+    int32_t* lmap = reinterpret_cast<int32_t*>(hist + num_buckets);
+    const uint32_t part = blockIdx.x % parts, h = blockIdx.x / parts;
+    const int tid = threadIdx.x;
+    for (int i = tid; i < num_buckets; i += 256) hist[i] = 0.0f;
+    for (int i = tid; i < max_distance; i += 256) lmap[i] = mapping[i];
+    __syncthreads();
+    const int32_t k0 = part * rows_per_part, k1 = min(key_len, k0 + rows_per_part);
+    const half_t* g = grad_out + (int64_t)h * key_len * query_len;
+    const int32_t half_b = num_buckets / 2;
+    for (int32_t q = tid; q < query_len; q += 256) {
+        float run = 0.0f;
+        int32_t cur = -1;
+        for (int32_t k = k0; k < k1; ++k) {
+            int32_t rel = q - k, off = 0;
+            if (rel < 0) {
+                if (bidirectional) { rel = -rel; off = half_b; }
+                else rel = 0;
+            }
+            if (rel >= max_distance) rel = max_distance - 1;
+            const int32_t bucket = lmap[rel] + off;
+            const float v = (float)g[(int64_t)k * query_len + q];
+            if (bucket != cur) {
+                if (cur >= 0) atomicAdd(&hist[cur], run);
+                cur = bucket;
+                run = 0.0f;
+            }
+            run += v;
+        }
+        if (cur >= 0) atomicAdd(&hist[cur], run);
+    }
+    __syncthreads();
+    if (parts == 1) {
+        for (int i = tid; i < num_buckets; i += 256) grad[(int64_t)h * num_buckets + i] = (half_t)hist[i];
+        return;
+    }
+    uint64_t* team_slots = xch + (size_t)h * parts * kXchVals;
+    for (int i = tid; i < num_buckets; i += 256) xch_post(team_slots + (size_t)part * kXchVals, i, hist[i], tag);
+    if (part == 0) {
+        const uint64_t deadline = wall_clock64() + kXchTimeoutTicks;
+        for (int i = tid; i < num_buckets; i += 256) {
+            float acc = 0.0f;
+            bool ok = true;
+            for (int32_t p = 0; p < parts; ++p) {
+                float x;
+                ok &= xch_wait(team_slots + (size_t)p * kXchVals + i, tag, deadline, x);
+                acc += x;
+            }
+            grad[(int64_t)h * num_buckets + i] = ok ? (half_t)acc : (half_t)__builtin_nanf("");
+        }
+        __syncthreads();
+    }
+    if (tid < 64) xch_retire(xch, h, parts);
+}
+
 // ---------------------------------------------------------------------------------------
 // Embedding gradient in two stages over ids sorted per batch entry (cuda/embedding.cu:38-88):
 // stage 1 sums runs of equal ids inside one batch entry, writes complete runs to grad and the
@@ -641,6 +705,22 @@ int cpmk_position_embedding_backward(int32_t query_len, int32_t key_len, int32_t
     if (query_len < 0 || key_len < 0 || num_buckets <= 0 || max_distance <= 0 || num_heads < 0) return CPMK_EBADARG;
     if (num_heads == 0) return 0;
     if (num_buckets > 8192) return CPMK_ETOOBIG;
+    if (num_buckets <= kXchVals && max_distance <= 8192 && key_len > 64) {
+        // key rows of a head over a team: 64 rows a part, more when that would make more than 32 parts
+        int64_t rpp = 64;
+        while (ceil_div(key_len, rpp) > kColTeamMaxParts) rpp *= 2;
+        const int64_t parts = ceil_div(key_len, rpp);
+        if ((int64_t)num_heads * parts <= kXchSlots) {
+            XchLaunch xl;
+            const int rc = xch_begin(&xl);
+            if (rc != 0) return rc;
+            hipLaunchKernelGGL(k_position_backward_team, dim3((unsigned)(num_heads * parts)), dim3(256),
+                               num_buckets * sizeof(float) + max_distance * sizeof(int32_t), (hipStream_t)stream, query_len, key_len,
+                               num_buckets, max_distance, (const int32_t*)position_mapping, (const half_t*)grad_out, (half_t*)grad,
+                               bidirectional, (int32_t)parts, (int32_t)rpp, xl.region, xl.tag);
+            return launch_status();
+        }
+    }
     hipLaunchKernelGGL(k_position_backward, dim3((unsigned)num_heads), dim3(256), num_buckets * sizeof(float), (hipStream_t)stream,
                        query_len, key_len, num_buckets, max_distance, (const int32_t*)position_mapping, (const half_t*)grad_out,
                        (half_t*)grad, bidirectional);

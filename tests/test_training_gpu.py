@@ -211,7 +211,8 @@ def test_gemm_backward_quantisers(gpu, shape, bc):
     assert_bits_equal(to_np(q), q_ref, "scale_round int8")
 
 
-@pytest.mark.parametrize("cfg", [(32, 128, True, 12, 100, 90), (32, 128, False, 4, 64, 200), (64, 512, True, 3, 17, 9)])
+@pytest.mark.parametrize("cfg", [(32, 128, True, 12, 100, 90), (32, 128, False, 4, 64, 200), (64, 512, True, 3, 17, 9),
+                                 (32, 128, True, 16, 1024, 1024), (32, 128, False, 5, 333, 2500), (256, 128, True, 2, 70, 130)])
 def test_position_embedding_backward(gpu, cfg):
     _name("position_embedding_backward", cfg)
     import oracle
