@@ -80,22 +80,40 @@ __global__ __launch_bounds__(256) void k_global_scale(int64_t n, const half_t* i
     }
 }
 
-// cu_gelu_backward: grad = gelu'(x) * grad_out with the reference's constants and cut-off at |x| >= 5.
-__global__ __launch_bounds__(256) void k_gelu_backward(int64_t total, const half_t* grad_out, const half_t* mat, half_t* grad) {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= total) return;
-    const float v = (float)grad_out[i], x = (float)mat[i];
+// cu_gelu_backward: grad = gelu'(x) * grad_out with the reference's constants and cut-off at |x| >= 5
+// (cuda/gelu.cu:18-45): gelu'(x) = 0.5 + 0.5 tanh(u) + (0.398942 x + 0.0535161 x^3) sech^2(u),
+// u = 0.797885 x + 0.0356774 x^3.  Both hyperbolic terms come from one exponential e = exp(-2|u|):
+// sech^2 = 4 e / (1 + e)^2 and 0.5 + 0.5 tanh(u) = 1 / (1 + e) for u >= 0, e / (1 + e) otherwise,
+// which has no cancellation where the derivative is small.
+__device__ inline half_t gelu_grad1(half_t gh, half_t xh) {
+    const float v = (float)gh, x = (float)xh;
     float g;
     if (-5.0f < x && x < 5.0f) {
         const float x3 = x * x * x;
         const float u = 0.797885f * x + 0.0356774f * x3;
-        float sech = 1.0f / coshf(u);
-        sech *= sech;
-        g = 0.5f + (0.398942f * x + 0.0535161f * x3) * sech + 0.5f * tanhf(u);
+        const float e = __builtin_amdgcn_exp2f(-2.8853900817779268f * fabsf(u));       // exp(-2|u|)
+        const float r = 1.0f / (1.0f + e);
+        const float hp = u < 0.0f ? e * r : r;
+        g = hp + (0.398942f * x + 0.0535161f * x3) * (4.0f * e * r * r);
     } else {
         g = x < 0.0f ? 0.0f : 1.0f;
     }
-    grad[i] = round_f16(g * v);
+    return round_f16(g * v);
+}
+
+template <int V>
+__global__ __launch_bounds__(256) void k_gelu_backward(int64_t total, const half_t* grad_out, const half_t* mat, half_t* grad) {
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * V;
+    if (i >= total) return;
+    if constexpr (V == 8) {
+        const half8_t gv = *reinterpret_cast<const half8_t*>(grad_out + i), xv = *reinterpret_cast<const half8_t*>(mat + i);
+        half8_t o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = gelu_grad1(gv[e], xv[e]);
+        *reinterpret_cast<half8_t*>(grad + i) = o;
+    } else {
+        grad[i] = gelu_grad1(grad_out[i], mat[i]);
+    }
 }
 
 // ---------------------------------------------------------------------------------------
@@ -119,14 +137,35 @@ __global__ __launch_bounds__(256) void k_batch_add_backward(int64_t batch, int64
 // grad[i] = sum_{b, j} (WITH_X ? x[b,i,j] : 1) * grad_out[b,i,j]            cu_arith_ln_mul_backward / _ln_add_backward
 template <bool WITH_X>
 __global__ __launch_bounds__(256) void k_ln_backward(int64_t batch, int64_t n, int64_t m, const half_t* __restrict__ x,
-                                                     const half_t* __restrict__ grad_out, half_t* __restrict__ grad) {
+                                                     const half_t* __restrict__ grad_out, half_t* __restrict__ grad, int vec) {
     __shared__ float red[4];
     const int64_t ch = blockIdx.x;
     float s = 0.0f;
-    for (int64_t b = 0; b < batch; ++b) {
-        const int64_t base = (b * n + ch) * m;
-        for (int64_t j = threadIdx.x; j < m; j += 256)
-            s += WITH_X ? (float)x[base + j] * (float)grad_out[base + j] : (float)grad_out[base + j];
+    if (vec) {         // m % 8 == 0, 16-byte aligned: the (b, j) pairs of this channel in pieces of 8
+        const uint32_t m8 = (uint32_t)(m >> 3), db = 256u / m8, dj = 256u % m8;      // one step of 256 pieces, as rows and remainder
+        uint32_t b = threadIdx.x / m8, j8 = threadIdx.x % m8;
+        for (; b < (uint32_t)batch; b += db, j8 += dj) {
+            if (j8 >= m8) {
+                j8 -= m8;
+                if (++b >= (uint32_t)batch) break;
+            }
+            const int64_t o = ((int64_t)b * n + ch) * m + ((int64_t)j8 << 3);
+            const half8_t gv = *reinterpret_cast<const half8_t*>(grad_out + o);
+            if (WITH_X) {
+                const half8_t xv = *reinterpret_cast<const half8_t*>(x + o);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) s += (float)xv[e] * (float)gv[e];
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) s += (float)gv[e];
+            }
+        }
+    } else {
+        for (int64_t b = 0; b < batch; ++b) {
+            const int64_t base = (b * n + ch) * m;
+            for (int64_t j = threadIdx.x; j < m; j += 256)
+                s += WITH_X ? (float)x[base + j] * (float)grad_out[base + j] : (float)grad_out[base + j];
+        }
     }
     s = block_sum<4>(s, red);
     if (threadIdx.x == 0) grad[ch] = (half_t)s;
@@ -374,6 +413,35 @@ __global__ __launch_bounds__(256) void k_round_scale_rows(int32_t n, int32_t m, 
     const float s = (float)((double)mx / 127.0);
     if (threadIdx.x == 0) scale_x[row] = (half_t)s;
     for (int32_t j = threadIdx.x; j < m; j += 256) out[row * m + j] = (int8_t)quant_i8((float)x[j] * (float)sy[j], s);
+}
+
+// The same with a wave per row and 16-byte accesses (m % 8 == 0, aligned pointers); the second pass
+// over the row finds it in the cache.
+__global__ __launch_bounds__(256) void k_round_scale_rows_wide(int64_t rows, int32_t n, int32_t m, const half_t* __restrict__ mat,
+                                                               const half_t* __restrict__ scale_y, int8_t* __restrict__ out,
+                                                               half_t* __restrict__ scale_x, int bc) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int64_t b = row / n;
+    const half_t* x = mat + row * m;
+    const half_t* sy = scale_y + (bc ? 0 : b * m);
+    float mx = 0.0f;
+    for (int32_t j = lane * 8; j < m; j += 512) {
+        const half8_t xv = *reinterpret_cast<const half8_t*>(x + j), sv = *reinterpret_cast<const half8_t*>(sy + j);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) mx = fmaxf(fabsf((float)xv[e] * (float)sv[e]), mx);
+    }
+    mx = wave_max(mx);
+    const float s = (float)((double)mx / 127.0);
+    if (lane == 0) scale_x[row] = (half_t)s;
+    for (int32_t j = lane * 8; j < m; j += 512) {
+        const half8_t xv = *reinterpret_cast<const half8_t*>(x + j), sv = *reinterpret_cast<const half8_t*>(sy + j);
+        int32_t t[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) t[e] = quant_i8((float)xv[e] * (float)sv[e], s);
+        *reinterpret_cast<uint2_t*>(out + row * m + j) = uint2_t{pack4_i8(t[0], t[1], t[2], t[3]), pack4_i8(t[4], t[5], t[6], t[7])};
+    }
 }
 
 // ---------------------------------------------------------------------------------------
@@ -626,7 +694,8 @@ int cpmk_arith_ln_mul_backward(int32_t batch, int32_t n, int32_t m, const void* 
     if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
     if (n == 0) return 0;
     hipLaunchKernelGGL((k_ln_backward<true>), dim3((unsigned)n), dim3(256), 0, (hipStream_t)stream, (int64_t)batch, (int64_t)n,
-                       (int64_t)m, (const half_t*)inp, (const half_t*)grad_out, (half_t*)grad);
+                       (int64_t)m, (const half_t*)inp, (const half_t*)grad_out, (half_t*)grad,
+                       (int)(m % 8 == 0 && aligned16(inp) && aligned16(grad_out)));
     return launch_status();
 }
 int cpmk_arith_ln_add_backward(int32_t batch, int32_t n, int32_t m, const void* grad_out, void* grad, void* stream) {
@@ -634,7 +703,8 @@ int cpmk_arith_ln_add_backward(int32_t batch, int32_t n, int32_t m, const void* 
     if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
     if (n == 0) return 0;
     hipLaunchKernelGGL((k_ln_backward<false>), dim3((unsigned)n), dim3(256), 0, (hipStream_t)stream, (int64_t)batch, (int64_t)n,
-                       (int64_t)m, (const half_t*)nullptr, (const half_t*)grad_out, (half_t*)grad);
+                       (int64_t)m, (const half_t*)nullptr, (const half_t*)grad_out, (half_t*)grad,
+                       (int)(m % 8 == 0 && aligned16(grad_out)));
     return launch_status();
 }
 
@@ -643,8 +713,12 @@ int cpmk_gelu_backward(int32_t batch, int32_t n, const void* grad_out, const voi
     if (batch < 0 || n < 0) return CPMK_EBADARG;
     const int64_t total = (int64_t)batch * n;
     if (total == 0) return 0;
-    hipLaunchKernelGGL(k_gelu_backward, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, (hipStream_t)stream, total,
-                       (const half_t*)grad_out, (const half_t*)mat, (half_t*)grad);
+    if (total % 8 == 0 && aligned16(grad_out) && aligned16(mat) && aligned16(grad))
+        hipLaunchKernelGGL((k_gelu_backward<8>), dim3((unsigned)ceil_div(total / 8, 256)), dim3(256), 0, (hipStream_t)stream, total,
+                           (const half_t*)grad_out, (const half_t*)mat, (half_t*)grad);
+    else
+        hipLaunchKernelGGL((k_gelu_backward<1>), dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, (hipStream_t)stream, total,
+                           (const half_t*)grad_out, (const half_t*)mat, (half_t*)grad);
     return launch_status();
 }
 
@@ -694,6 +768,11 @@ int cpmk_gemm_backward_round_scale(int32_t batch, int32_t n, int32_t m, const vo
     const int64_t rows = (int64_t)batch * n;
     if (rows == 0) return 0;
     if (rows > 0x7fffffff) return CPMK_ETOOBIG;
+    if (m % 8 == 0 && aligned16(mat) && aligned16(scale_y) && (reinterpret_cast<uintptr_t>(out) & 7u) == 0) {
+        hipLaunchKernelGGL(k_round_scale_rows_wide, dim3((unsigned)ceil_div(rows, 4)), dim3(256), 0, (hipStream_t)stream, rows, n, m,
+                           (const half_t*)mat, (const half_t*)scale_y, (int8_t*)out, (half_t*)scale_x, broad_cast_y);
+        return launch_status();
+    }
     hipLaunchKernelGGL(k_round_scale_rows, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, n, m, (const half_t*)mat,
                        (const half_t*)scale_y, (int8_t*)out, (half_t*)scale_x, broad_cast_y);
     return launch_status();

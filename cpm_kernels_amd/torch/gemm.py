@@ -156,6 +156,33 @@ class GEMMInt8(torch.autograd.Function):
         quant_G_a = torch.empty((batch, m, n), dtype=torch.int8, device=grad_f.device)
         gemm_backward_round_scale(batch, m, n, grad_f.data_ptr(), scale_B.data_ptr(), quant_G_a.data_ptr(),
                                   scale_G_a.data_ptr(), scale_B.size(0) == 1, st)
+        if ctx.stored == (False, True):
+            # The fused forward holds quantized_A as (bA, M, K) and quantized_B as (bB, N, K).  Each gradient is
+            # formed directly in the layout its operand came in, from operands with the contraction index
+            # contiguous: no product on the general kernel and no transposition of a result.
+            in_aT, in_bT = ctx.layout
+            qB_t = _transposed_copy_i8(quantized_B)                     # (bB, K, N)
+            if in_aT:       # grad_A (b, K, M) = qB_t x quant_G_a^T, scaled per column m
+                grad_A = gemm_and_scale(qB_t, None, quant_G_a, scale_G_a, False, True)
+            else:           # grad_A (b, M, K) = quant_G_a x qB_t^T, scaled per row m
+                grad_A = gemm_and_scale(quant_G_a, scale_G_a, qB_t, None, False, True)
+            del scale_G_a, quant_G_a, qB_t
+            scale_G_b = torch.empty((batch, n), dtype=torch.half, device=grad_f.device)
+            quant_G_b = torch.empty((batch, m, n), dtype=torch.int8, device=grad_f.device)
+            gemm_backward_scale_round(batch, m, n, grad_f.data_ptr(), scale_A.data_ptr(), quant_G_b.data_ptr(),
+                                      scale_G_b.data_ptr(), scale_A.size(0) == 1, st)
+            qG_t = _transposed_copy_i8(quant_G_b)                       # (b, N, M)
+            del quant_G_b
+            qA_t = _transposed_copy_i8(quantized_A)                     # (bA, K, M)
+            if in_bT:       # grad_B (b, N, K) = qG_t x qA_t^T, scaled per row n
+                grad_B = gemm_and_scale(qG_t, scale_G_b, qA_t, None, False, True)
+            else:           # grad_B (b, K, N) = qA_t x qG_t^T, scaled per column n
+                grad_B = gemm_and_scale(qA_t, None, qG_t, scale_G_b, False, True)
+            if scale_A.size(0) == 1 and grad_A.size(0) > 1:
+                grad_A = grad_A.sum(dim=0, keepdim=True)
+            if scale_B.size(0) == 1 and grad_B.size(0) > 1:
+                grad_B = grad_B.sum(dim=0, keepdim=True)
+            return grad_A, None, grad_B, None, None
         if aT:
             grad_A = gemm_and_scale(quantized_B, None, quant_G_a, scale_G_a, bT, True)
         else:
