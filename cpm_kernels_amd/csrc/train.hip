@@ -1,8 +1,9 @@
 // Training-side and remaining elementwise kernels of the reference, forward results and
 // gradients (cuda/arith.cu, cuda/gelu.cu:18-45, cuda/gemm.cu:100-172, cuda/layernorm.cu:142-339,
 // cuda/softmax.cu:86-114, cuda/position_bucket.cu:56-103, cuda/embedding.cu:38-88).  None of
-// them is on the inference hot path; they are written for coalesced 16-byte access and fp32
-// accumulation but not tuned further.
+// them is on the inference hot path; they use 16-byte accesses and fp32 accumulation, and the
+// reductions over dim 1 share the register-resident column tile and the team exchange of the
+// forward layernorm.
 #include "dim1.h"
 #include "exchange.h"
 
