@@ -553,14 +553,30 @@ __global__ __launch_bounds__(256) void k_embedding_backward1(int32_t n, int32_t 
     if (col >= m) return;
     const int64_t base = b * n;
     float sum = 0.0f;
-    for (int32_t i = 0; i < n; ++i) {
-        sum += (float)grad_out[(int64_t)argsort_ids[base + i] * m + col];
-        if (i + 1 == n) {
-            aux_grad[b * m + col] = (half_t)sum;
-            if (col == 0) aux_idx[b] = sorted_ids[base + i];
-        } else if (sorted_ids[base + i] != sorted_ids[base + i + 1]) {
-            grad[(int64_t)sorted_ids[base + i] * m + col] = (half_t)sum;
-            sum = 0.0f;
+    // eight gathers in flight at a time; the sums are still formed one id after the other
+    for (int32_t i0 = 0; i0 < n; i0 += 8) {
+        float v[8];
+        int32_t id[9];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int32_t i = min(i0 + u, n - 1);
+            v[u] = (float)grad_out[(int64_t)argsort_ids[base + i] * m + col];
+            id[u] = sorted_ids[base + i];
+        }
+        id[8] = sorted_ids[base + min(i0 + 8, n - 1)];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int32_t i = i0 + u;
+            if (i < n) {
+                sum += v[u];
+                if (i + 1 == n) {
+                    aux_grad[b * m + col] = (half_t)sum;
+                    if (col == 0) aux_idx[b] = id[u];
+                } else if (id[u] != id[u + 1]) {
+                    grad[(int64_t)id[u] * m + col] = (half_t)sum;
+                    sum = 0.0f;
+                }
+            }
         }
     }
 }
