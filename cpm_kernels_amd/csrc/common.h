@@ -159,6 +159,9 @@ __device__ __forceinline__ void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
+// fp16 broadcast-matrix GEMV on the MFMA kernel of gemv_i8.hip (0, a HIP error code, or -1: shape not eligible)
+int gemv_f16_coalesced(int32_t batch, int32_t dim_out, int32_t dim_in, const void* mat, const void* vec, void* out, hipStream_t st);
+
 // Compute units of the current device (cached per device ordinal; 256 if the query fails).
 inline int compute_units() {
     static int cus[64] = {0};

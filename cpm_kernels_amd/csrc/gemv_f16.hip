@@ -5,6 +5,7 @@
 //   gemv_broadcast_mat_fp16 out[b,o] = sum_k mat[o,k]   * vec[b,k]    (one matrix for all vectors)
 // All three stream the matrix from HBM once.
 #include "common.h"
+#include <type_traits>
 
 namespace cpmk {
 
@@ -50,6 +51,33 @@ __global__ __launch_bounds__(256) void k_gemv_f16_rows(int32_t batch, int32_t di
         const float s = wave_sum(acc[t]);
         if (lane == 0 && b0 + t < batch) out[(b0 + t) * dim_out + row] = (half_t)s;
     }
+}
+
+// Short rows (dim_in <= 256, the head dimension of attention scores over a key cache): LPRK lanes
+// per row, one 16-byte piece each, so a wave covers 64 / LPRK consecutive rows with one coalesced
+// load; the row sums are finished with LPRK-wide butterfly shuffles.  item = b * dim_out + row.
+template <int LPRK>
+__global__ __launch_bounds__(256) void k_gemv_f16_short(int64_t items, int32_t dim_out, int32_t dim_in,
+                                                        const half_t* __restrict__ mat, const half_t* __restrict__ vec,
+                                                        half_t* __restrict__ out) {
+    constexpr int RPW = 64 / LPRK;
+    const int lane = threadIdx.x & 63, pl = lane % LPRK;
+    const int64_t item = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * RPW + lane / LPRK;
+    const bool live = item < items;
+    const int64_t it = live ? item : items - 1;
+    const int64_t b = it / dim_out;
+    const half_t* mrow = mat + it * dim_in;
+    const half_t* v = vec + b * dim_in;
+    float acc = 0.0f;
+    for (int32_t i = pl; i < (dim_in >> 3); i += LPRK) {
+        const half8_t w = reinterpret_cast<const half8_t*>(mrow)[i];
+        const half8_t x = reinterpret_cast<const half8_t*>(v)[i];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc = __builtin_fmaf((float)w[e], (float)x[e], acc);
+    }
+#pragma unroll
+    for (int o = 1; o < LPRK; o <<= 1) acc += __shfl_xor(acc, o, kWave);
+    if (live && pl == 0) out[item] = (half_t)acc;
 }
 
 // mat (batch, dim_in, dim_out): 256 threads = 32 row groups x 8 lanes of 8 adjacent columns; the
@@ -105,6 +133,22 @@ int cpmk_gemv_fp16(int32_t batch, int32_t dim_out, int32_t dim_in, const void* m
     if ((int64_t)batch * dim_out == 0) return 0;
     const int vec8 = (dim_in % 8 == 0) && aligned16(mat) && aligned16(vec);
     const int64_t items = (int64_t)batch * dim_out;
+    if (vec8 && dim_in <= 256) {
+        const int p = dim_in >> 3;                      // 16-byte pieces per row
+        const hipStream_t st = (hipStream_t)stream;
+        auto go = [&](auto lc) {
+            constexpr int L = decltype(lc)::value;
+            hipLaunchKernelGGL((k_gemv_f16_short<L>), dim3((unsigned)ceil_div(items, 4 * (64 / L))), dim3(256), 0, st, items, dim_out,
+                               dim_in, (const half_t*)mat, (const half_t*)vec, (half_t*)out);
+        };
+        if (p <= 1) go(std::integral_constant<int, 1>{});
+        else if (p <= 2) go(std::integral_constant<int, 2>{});
+        else if (p <= 4) go(std::integral_constant<int, 4>{});
+        else if (p <= 8) go(std::integral_constant<int, 8>{});
+        else if (p <= 16) go(std::integral_constant<int, 16>{});
+        else go(std::integral_constant<int, 32>{});
+        return launch_status();
+    }
     hipLaunchKernelGGL((k_gemv_f16_rows<1>), dim3((unsigned)ceil_div(items, 4)), dim3(256), 0, (hipStream_t)stream, batch,
                        dim_out, dim_in, (int64_t)dim_out * dim_in, (const half_t*)mat, (const half_t*)vec, (half_t*)out, vec8);
     return launch_status();
@@ -128,6 +172,10 @@ int cpmk_gemv_broadcast_mat_fp16(int32_t batch, int32_t dim_out, int32_t dim_in,
     clear_stale_error();
     if (batch < 0 || dim_out < 0 || dim_in < 0) return CPMK_EBADARG;
     if ((int64_t)batch * dim_out == 0) return 0;
+    {   // matrix cores when the rows are whole 256-byte chunks
+        const int rc = gemv_f16_coalesced(batch, dim_out, dim_in, mat, vec, out, (hipStream_t)stream);
+        if (rc >= 0) return rc;
+    }
     const int vec8 = (dim_in % 8 == 0) && aligned16(mat) && aligned16(vec);
     constexpr int NB = 8;               // vectors per pass over a matrix row
     const int64_t passes = ceil_div(batch, NB);

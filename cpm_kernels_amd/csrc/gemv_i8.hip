@@ -117,7 +117,12 @@ __global__ __launch_bounds__(NW * 64) void k_gemv_mfma(int32_t batch, int32_t di
 // directions are bank-conflict free.  LDS executes one wave's operations in order, so the 4 KB
 // buffer is reused without waits.  Vectors past the end are clamped and row steps past r4 are
 // not loaded (the MFMA then sees stale LDS bytes): both only feed outputs that are never stored.
-template <int NW, int RG, int NB>
+//
+// F16: the same kernel on fp16 data (cpmk_gemv_broadcast_mat_fp16): dim_in is then the row length in
+// BYTES, a lane's 16 bytes are 8 halves of K for v_mfma_f32_16x16x32_f16 (the same lane -> byte
+// assignment as the int8 instruction), the accumulators are fp32 and leave without scales; the
+// waves add their partial sums in wave order, so the result does not depend on timing.
+template <int NW, int RG, int NB, bool F16 = false>
 __global__ __launch_bounds__(NW * 64) void k_gemv_coalesced(int32_t batch, int32_t dim_out, int32_t dim_in, int32_t r4,
                                                             const half_t* __restrict__ scale_mat,
                                                             const int8_t* __restrict__ mat,
@@ -140,8 +145,11 @@ __global__ __launch_bounds__(NW * 64) void k_gemv_coalesced(int32_t batch, int32
     for (int o = 0; o < NOUT; ++o) {
         const int idx = tid + o * NW * 64;
         const int rr = idx % rpb, bb = idx / rpb;
-        osv[o] = scale_vec[min(bb, batch - 1)];
-        osm[o] = scale_mat[min(row0 + rr, dim_out - 1)];
+        osv[o] = osm[o] = (half_t)1.0f;
+        if (!F16) {
+            osv[o] = scale_vec[min(bb, batch - 1)];
+            osm[o] = scale_mat[min(row0 + rr, dim_out - 1)];
+        }
     }
     int woff[4], roff[4];
 #pragma unroll
@@ -167,11 +175,14 @@ __global__ __launch_bounds__(NW * 64) void k_gemv_coalesced(int32_t batch, int32
 #pragma unroll
         for (int i = 0; i < 4; ++i) vo[t][i] = (uint32_t)min(t * 16 + i * 4 + y4, batch - 1) * (uint32_t)dim_in + x * 16;
 
-    int4_t acc[RG][NB];
+    using acc_t = std::conditional_t<F16, float4_t, int4_t>;
+    acc_t acc[RG][NB];
 #pragma unroll
     for (int g = 0; g < RG; ++g)
 #pragma unroll
-        for (int t = 0; t < NB; ++t) acc[g][t] = int4_t{0, 0, 0, 0};
+        for (int t = 0; t < NB; ++t)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[g][t][e] = 0;
 
     auto load_chunk = [&](int4_t (&wr)[RG][4], int4_t (&vr)[NB][4], int c) __attribute__((always_inline)) {
 #pragma unroll
@@ -206,8 +217,13 @@ __global__ __launch_bounds__(NW * 64) void k_gemv_coalesced(int32_t batch, int32
 #pragma unroll
             for (int g = 0; g < RG; ++g)
 #pragma unroll
-                for (int t = 0; t < NB; ++t)
-                    acc[g][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wr[g][j], vr[t][j], acc[g][t], 0, 0, 0);
+                for (int t = 0; t < NB; ++t) {
+                    if constexpr (F16)
+                        acc[g][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, wr[g][j]),
+                                                                           __builtin_bit_cast(half8_t, vr[t][j]), acc[g][t], 0, 0, 0);
+                    else
+                        acc[g][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wr[g][j], vr[t][j], acc[g][t], 0, 0, 0);
+                }
     };
 
     const int nchunks = dim_in >> 8;
@@ -230,13 +246,28 @@ __global__ __launch_bounds__(NW * 64) void k_gemv_coalesced(int32_t batch, int32
     for (int idx = tid; idx < RG * NB * 256; idx += NW * 64) (&part[0][0])[idx] = 0;
     __syncthreads();
     // accumulator e of lane l: matrix row (l/16)*4 + e, vector l%16 of the 16x16 tile
+    if constexpr (F16) {
+        float* fpart = reinterpret_cast<float*>(&part[0][0]);
+        for (int ww = 0; ww < NW; ++ww) {          // one wave after the other: a fixed order of summation
+            if (w == ww) {
 #pragma unroll
-    for (int g = 0; g < RG; ++g)
+                for (int g = 0; g < RG; ++g)
 #pragma unroll
-        for (int t = 0; t < NB; ++t)
+                    for (int t = 0; t < NB; ++t)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) atomicAdd(&part[g * NB + t][(q * 4 + e) * 16 + r], acc[g][t][e]);
-    __syncthreads();
+                        for (int e = 0; e < 4; ++e) fpart[(g * NB + t) * 256 + (q * 4 + e) * 16 + r] += acc[g][t][e];
+            }
+            __syncthreads();
+        }
+    } else {
+#pragma unroll
+        for (int g = 0; g < RG; ++g)
+#pragma unroll
+            for (int t = 0; t < NB; ++t)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) atomicAdd(&part[g * NB + t][(q * 4 + e) * 16 + r], (int32_t)acc[g][t][e]);
+        __syncthreads();
+    }
     // thread -> (vector, row) with the row fastest, so a vector's outputs are stored contiguously
 #pragma unroll
     for (int o = 0; o < NOUT; ++o) {
@@ -246,8 +277,10 @@ __global__ __launch_bounds__(NW * 64) void k_gemv_coalesced(int32_t batch, int32
             const int g = rr >> 4, t = bb >> 4;
             const int32_t s = part[g * NB + t][(rr & 15) * 16 + (bb & 15)];
             const int32_t row = row0 + rr;
-            if (row < dim_out && bb < batch)
-                out[(int64_t)bb * dim_out + row] = dequant(s, (float)osv[o], (float)osm[o]);
+            if (row < dim_out && bb < batch) {
+                if constexpr (F16) out[(int64_t)bb * dim_out + row] = (half_t)__builtin_bit_cast(float, s);
+                else out[(int64_t)bb * dim_out + row] = dequant(s, (float)osv[o], (float)osm[o]);
+            }
         }
     }
 }
@@ -290,7 +323,7 @@ __global__ __launch_bounds__(256) void k_gemv_dot4(int32_t batch, int32_t dim_ou
 // Rows per workgroup, in steps of 4: one workgroup per compute unit when the matrix allows it
 // (every workgroup re-reads all the vectors from L2, so fewer and larger ones are better), at
 // most 16*MAXRG rows.
-template <int NB, int MAXRG>
+template <int NB, int MAXRG, bool F16 = false>
 static void launch_coalesced(int32_t batch, int32_t dim_out, int32_t dim_in, const half_t* sm, const int8_t* mat,
                              const half_t* sv, const int8_t* vec, half_t* out, hipStream_t st) {
     int64_t r4 = ceil_div(ceil_div(dim_out, compute_units()), 4);
@@ -299,7 +332,7 @@ static void launch_coalesced(int32_t batch, int32_t dim_out, int32_t dim_in, con
     const int rg = (int)ceil_div(r4, 4);
     const dim3 grid((unsigned)ceil_div(dim_out, r4 * 4));
     auto go = [&](auto rgc) {
-        hipLaunchKernelGGL((k_gemv_coalesced<8, decltype(rgc)::value, NB>), grid, dim3(512), 0, st, batch, dim_out, dim_in,
+        hipLaunchKernelGGL((k_gemv_coalesced<8, decltype(rgc)::value, NB, F16>), grid, dim3(512), 0, st, batch, dim_out, dim_in,
                            (int32_t)r4, sm, mat, sv, vec, out);
     };
     if constexpr (MAXRG >= 4) { if (rg == 4) return go(std::integral_constant<int, 4>{}); }
@@ -325,6 +358,27 @@ static void launch_mfma(int32_t batch, int32_t dim_out, int32_t dim_in, const ha
         hipLaunchKernelGGL((k_gemv_mfma<8, 1, NB>), dim3((unsigned)ceil_div(dim_out, 16)), dim3(512), 0, st,
                            batch, dim_out, dim_in, sm, mat, sv, vec, out);
     }
+}
+
+// fp16 matrix (dim_out, dim_in) shared by `batch` fp16 vectors on the MFMA kernel above.  Returns -1 when
+// the shape does not qualify (rows of whole 256-byte chunks, 16-byte aligned, offsets within 32 bits).
+int gemv_f16_coalesced(int32_t batch, int32_t dim_out, int32_t dim_in, const void* mat, const void* vec, void* out, hipStream_t st) {
+    const int64_t row_bytes = (int64_t)dim_in * 2;
+    if (dim_in <= 0 || row_bytes % 256 != 0 || !aligned16(mat) || !aligned16(vec) || (int64_t)dim_out * row_bytes >= (1ll << 32))
+        return -1;
+    const int8_t* M = (const int8_t*)mat;
+    for (int32_t b0 = 0; b0 < batch; b0 += 128) {
+        const int32_t nb = batch - b0 < 128 ? batch - b0 : 128;
+        if ((int64_t)nb * row_bytes >= (1ll << 32)) return -1;
+        const int8_t* v = (const int8_t*)vec + (int64_t)b0 * row_bytes;
+        half_t* o = (half_t*)out + (int64_t)b0 * dim_out;
+        if (nb <= 16) launch_coalesced<1, 4, true>(nb, dim_out, (int32_t)row_bytes, nullptr, M, nullptr, v, o, st);
+        else if (nb <= 32) launch_coalesced<2, 4, true>(nb, dim_out, (int32_t)row_bytes, nullptr, M, nullptr, v, o, st);
+        else if (nb <= 64) launch_coalesced<4, 2, true>(nb, dim_out, (int32_t)row_bytes, nullptr, M, nullptr, v, o, st);
+        else launch_coalesced<8, 1, true>(nb, dim_out, (int32_t)row_bytes, nullptr, M, nullptr, v, o, st);
+        if (int e = launch_status()) return e;
+    }
+    return 0;
 }
 
 }  // namespace cpmk

@@ -726,7 +726,9 @@ def test_gemm_fp16(gpu, case, aT, bT):
         assert_close_fp16(to_np(out), ref.astype(np.float16), rtol=1e-3, atol=1e-3, what="gemm_fp16 %s" % (case,))
 
 
-@pytest.mark.parametrize("shape", [(4, 64, 256), (3, 33, 100), (2, 1000, 4096), (1, 7, 6)])
+@pytest.mark.parametrize("shape", [(4, 64, 256), (3, 33, 100), (2, 1000, 4096), (1, 7, 6),
+                                   # short rows (lanes share a wave's rows) and rows of whole 256-byte chunks (matrix cores)
+                                   (5, 70, 64), (2, 1000, 128), (3, 9, 8), (40, 300, 512), (33, 1100, 1024), (130, 48, 384)])
 def test_gemv_fp16_family(gpu, shape):
     _name("gemv fp16", shape)
     batch, dim_out, dim_in = shape
