@@ -296,6 +296,21 @@ def main():
         ms, how = graph_ms([(lambda o_=o_: ck.position_embedding_forward(1024, 1024, 32, 128, 64, tbl.data_ptr(), pw.data_ptr(), o_.data_ptr(), True, st())) for o_ in pos], max(3, reps // 12))
         hbm("position_embedding_forward", 2 * 64 * 1024 * 1024 + 2 * 64 * 32 + 4 * 128, ms, how, "64 heads x 1024 x 1024 fp16 written", None)
         del pos
+        # fp16 decode-step products: one weight matrix for 32 vectors, and attention over a key / value cache
+        # of 32 sequences x 64 heads x 1024 positions x 64 (2 x 268 MB rotate)
+        wf = rot((10240, 4096), 4)
+        vf = torch.randn(32, 4096, generator=gg).half().to(dev); of = torch.empty((32, 10240), dtype=torch.half, device=dev)
+        ms, how = graph_ms([(lambda w_=w_: ck.gemv_broadcast_mat_fp16(32, 10240, 4096, w_.data_ptr(), vf.data_ptr(), of.data_ptr(), st())) for w_ in wf], max(3, reps // 8))
+        hbm("gemv_broadcast_mat_fp16", 2 * 10240 * 4096 + 2 * 32 * 4096 + 2 * 32 * 10240, ms, how, "W fp16 [10240,4096] x 32 vectors", None)
+        del wf
+        kc = rot((2048, 1024, 64), 2)
+        qf = torch.randn(2048, 64, generator=gg).half().to(dev); sc = torch.empty((2048, 1024), dtype=torch.half, device=dev)
+        ms, how = graph_ms([(lambda k_=k_: ck.gemv_fp16(2048, 1024, 64, k_.data_ptr(), qf.data_ptr(), sc.data_ptr(), st())) for k_ in kc], max(3, reps // 8))
+        hbm("gemv_fp16 (attention scores over a key cache)", 2 * 2048 * 1024 * 64 + 2 * 2048 * 64 + 2 * 2048 * 1024, ms, how, "2048 x [1024,64] fp16", None)
+        ov = torch.empty((2048, 64), dtype=torch.half, device=dev)
+        ms, how = graph_ms([(lambda k_=k_: ck.gemv_fp16_transpose(2048, 64, 1024, k_.data_ptr(), sc.data_ptr(), ov.data_ptr(), st())) for k_ in kc], max(3, reps // 8))
+        hbm("gemv_fp16_transpose (probabilities x value cache)", 2 * 2048 * 1024 * 64 + 2 * 2048 * 1024 + 2 * 2048 * 64, ms, how, "2048 x [1024,64] fp16", None)
+        del kc
         # config 4 up-projection in the reference's native layout: bmm(W1[1,10240,4096], x[8,4096,512], int8)
         W1 = (torch.randn(1, 10240, 4096, generator=gg) * 0.02).half().to(dev)
         xa = torch.randn(8, 4096, 512, generator=gg).half().to(dev)
