@@ -229,6 +229,29 @@ __device__ __forceinline__ GemmItem gemm_item(uint32_t L, const DmaArgs& da) {
     return it;
 }
 
+// The 16 bytes of K one lane feeds to an MFMA, collected from a stage part that holds rows of K
+// with B elements each (an operand stored with K as the row index): eight 2-byte reads for fp16,
+// sixteen 1-byte reads for int8.  `p` points at the lane's element of the k-step's first row.
+template <bool F16, int B>
+__device__ __forceinline__ int4_t gather_k(const int8_t* p, int ks) {
+    if constexpr (F16) {
+        half8_t v;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = *reinterpret_cast<const half_t*>(p + (ks * 16 + e) * (B * 2));
+        return __builtin_bit_cast(int4_t, v);
+    } else {
+        uint32_t w[4];
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            uint32_t x = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) x |= (uint32_t)(uint8_t)p[(ks * 32 + d * 4 + e) * B] << (8 * e);
+            w[d] = x;
+        }
+        return int4_t{(int32_t)w[0], (int32_t)w[1], (int32_t)w[2], (int32_t)w[3]};
+    }
+}
+
 // One output tile of BR x BC = (WR*TR*32) x (WC*TC*32), K slab = BKB bytes.
 // NST-stage ring; pipeline per K slab `it` (stage cur = it % NST, slabs it+1 .. it+NST-1 in flight):
 //   k-steps 0 .. KS-2 : MFMAs of step s while the fragments of step s+1 are read from LDS
@@ -244,17 +267,19 @@ __device__ __forceinline__ GemmItem gemm_item(uint32_t L, const DmaArgs& da) {
 // lets the compiler keep the accumulators in place and the MFMA/memory interleave as written.
 // Returns true if the next tile's first slabs are on their way.
 //
-// LAY (fp16 only) marks operands whose rows are K instead: bit 0 = the row operand is stored
-// (K, n), bit 1 = the column operand is stored (K, m).  Such an operand's part of a stage holds
-// BKB/2 rows of K with the tile's BR (BC) halves each, DMA'd as they lie in memory; a lane then
-// collects its 8 halves of K with eight 2-byte LDS reads (32 lanes read 64 contiguous bytes: no
-// bank conflicts) instead of one 16-byte read.
+// LAY marks operands whose rows are K instead: bit 0 = the row operand is stored (K, n), bit 1 =
+// the column operand is stored (K, m).  Such an operand's part of a stage holds the slab's rows
+// of K (64 for fp16, 128 for int8) with the tile's BR (BC) elements each, DMA'd as they lie in
+// memory; a lane then collects its 16 bytes of K element by element (gather_k: 32 lanes read
+// contiguous bytes of one row, no bank conflicts) instead of with one 16-byte read.
 template <int WR, int WC, int TR, int TC, int BKB, int EPI, int NST, int LAY = 0>
 __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, int8_t* stg, uint32_t lds_base,
                                               const GemmItem cur_item, const GemmItem nxt_item, const bool have_slabs, int& ring) {
     constexpr bool FUSED = EPI == kEpiDequant, F16 = EPI == kEpiF16;
     constexpr bool PT = (LAY & 1) != 0, QT = (LAY & 2) != 0;
-    static_assert(LAY == 0 || (F16 && BKB == 128), "transposed operands: fp16 with 64 halves of K per slab");
+    static_assert(LAY == 0 || BKB == 128, "transposed operands: 128 bytes of K per slab");
+    constexpr int ESZ_IN = F16 ? 2 : 1;            // bytes per operand element
+    constexpr int EPP = 16 / ESZ_IN;               // elements per 16-byte piece
     using acc_t = std::conditional_t<F16, float16_tv, int16_tv>;
     constexpr int KS = BKB / 32, CPR = BKB / 16;
     constexpr int NW = WR * WC, BR = WR * TR * 32, BC = WC * TC * 32;
@@ -277,12 +302,12 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
 #pragma unroll
     for (int i = 0; i < TR; ++i) {
         const int r = wr * TR * 32 + i * 32 + lrow;
-        offP[i] = PT ? lk * 8 * (BR * 2) + r * 2 : r * BKB + ((lk ^ swz(r)) << 4);
+        offP[i] = PT ? lk * EPP * (BR * ESZ_IN) + r * ESZ_IN : r * BKB + ((lk ^ swz(r)) << 4);
     }
 #pragma unroll
     for (int j = 0; j < TC; ++j) {
         const int r = wc * TC * 32 + j * 32 + lrow;
-        offQ[j] = BR * BKB + (QT ? lk * 8 * (BC * 2) + r * 2 : r * BKB + ((lk ^ swz(r)) << 4));
+        offQ[j] = BR * BKB + (QT ? lk * EPP * (BC * ESZ_IN) + r * ESZ_IN : r * BKB + ((lk ^ swz(r)) << 4));
     }
     // without slabs on their way the waits below count only loads: let the previous tile's stores finish first
     if (!have_slabs) wait_vmcnt<0>();
@@ -316,11 +341,11 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
         const bool q = dd * RPI >= BR;
         if ((PT && !q) || (QT && q)) {
             // a (K, L) operand: the instruction covers 1024 / (2 * B) rows of K, a lane one 16-byte piece of a row
-            const int ppr = (q ? BC : BR) / 8;                     // pieces per row of K
+            const int ppr = (q ? BC : BR) / EPP;                   // pieces per row of K
             const int dl = q ? dd - BR / RPI : dd;
             const int kr = dl * (64 / ppr) + lane / ppr, pc = lane % ppr;
             const int32_t L = q ? a.m : a.n;
-            return ((uint32_t)kr * (uint32_t)L + (uint32_t)min((q ? oi : oj) + pc * 8, L - 8)) * 2u;      // L % 8 == 0
+            return ((uint32_t)kr * (uint32_t)L + (uint32_t)min((q ? oi : oj) + pc * EPP, L - EPP)) * (uint32_t)ESZ_IN;      // L % EPP == 0
         }
         const int32_t grow = q ? min(oi + (r - BR), a.m - 1) : min(oj + r, a.n - 1);
         return (uint32_t)grow * (uint32_t)K + c * 16;
@@ -379,21 +404,13 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
         constexpr int x = decltype(xc)::value, buf = decltype(bufc)::value;
         if constexpr (x < TR) {
             if constexpr (PT) {
-                half8_t v;
-#pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    v[e] = *reinterpret_cast<const half_t*>(smem + stage * STAGE + offP[x] + (ks * 16 + e) * (BR * 2));
-                fp[buf][x] = __builtin_bit_cast(int4_t, v);
+                fp[buf][x] = gather_k<F16, BR>(smem + stage * STAGE + offP[x], ks);
             } else {
                 fp[buf][x] = *reinterpret_cast<const int4_t*>(smem + stage * STAGE + (offP[x] ^ (ks << 5)));
             }
         } else {
             if constexpr (QT) {
-                half8_t v;
-#pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    v[e] = *reinterpret_cast<const half_t*>(smem + stage * STAGE + offQ[x - TR] + (ks * 16 + e) * (BC * 2));
-                fq[buf][x - TR] = __builtin_bit_cast(int4_t, v);
+                fq[buf][x - TR] = gather_k<F16, BC>(smem + stage * STAGE + offQ[x - TR], ks);
             } else {
                 fq[buf][x - TR] = *reinterpret_cast<const int4_t*>(smem + stage * STAGE + (offQ[x - TR] ^ (ks << 5)));
             }
@@ -773,6 +790,16 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
         // the smaller tiles finish a slab before a load from L2 returns: four ring stages keep them fed
         if (mid * 4 >= compute_units() * 3) return launch_dma<2, 2, 2, 2, 128, EPI, CPMK_GEMM_NST_SMALL>(a, batch, st);
         return launch_dma<2, 2, 2, 1, 128, EPI, CPMK_GEMM_NST_SMALL>(a, batch, st);
+    }
+    // an operand stored (K, rows): the tile kernel reads it as it lies and gathers the fragments byte by byte in LDS
+    if (!(p_kmajor && q_kmajor) && wide && k > 0 && (k % 128 == 0) && aligned16(A) && aligned16(B) && (p_kmajor || n % 16 == 0) &&
+        (q_kmajor || m % 16 == 0) && (int64_t)n * k < (1ll << 32) && (int64_t)m * k < (1ll << 32)) {
+        constexpr int EPI = FUSED ? kEpiDequant : kEpiInt32;
+        switch ((p_kmajor ? 0 : 1) | (q_kmajor ? 0 : 2)) {
+            case 1: return launch_dma<CPMK_GEMM_BIG, EPI, 2, 1>(a, batch, st);
+            case 2: return launch_dma<CPMK_GEMM_BIG, EPI, 2, 2>(a, batch, st);
+            default: return launch_dma<CPMK_GEMM_BIG, EPI, 2, 3>(a, batch, st);
+        }
     }
     if (fast) {
         const int64_t t256 = ceil_div(n, 256) * ceil_div(m, 128) * batch;

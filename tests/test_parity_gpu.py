@@ -262,6 +262,21 @@ def test_gemm_int8_tile_kernels(gpu, case):
         _gemm_case(gpu, m, k, n, bA, bB, True, False, rng)
 
 
+# int8 operands with the contraction index as the row (the other three aT/bT combinations) on the tile kernel:
+# k % 128 == 0 and row lengths that are multiples of 16; ragged tiles, one to several slabs, batch broadcast.
+LAYOUT_CASES = [(1, 512, 256, 768), (2, 272, 128, 528), (1, 48, 384, 1040), (3, 1040, 640, 16), (1, 2304, 1024, 2064)]
+
+
+@pytest.mark.parametrize("case", LAYOUT_CASES)
+def test_gemm_int8_tile_kernel_layouts(gpu, case):
+    batch, n, k, m = case
+    rng = np.random.default_rng(n * 7919 + k * 31 + m + 5)
+    for aT, bT in ((True, True), (False, False), (False, True)):
+        for (bA, bB) in ((batch, batch),) + (((1, batch), (batch, 1)) if batch > 1 else ()):
+            _name("gemm_int8 tile kernel layouts", case, aT, bT, bA, bB)
+            _gemm_case(gpu, m, k, n, bA, bB, aT, bT, rng)
+
+
 def test_gemm_int8_extreme_values(gpu):
     """All operands -128 / 127: largest accumulators the int8 product can produce."""
     _name("gemm_int8 extremes")
