@@ -17,11 +17,12 @@
 //                  buffering, v_mfma_i32_32x32x32_i8 with the operands swapped so that a lane
 //                  owns 4 consecutive output columns; results leave through a per-wave LDS strip
 //                  as whole 128-byte lines.
+//                  With template parameter LAY it also takes operands stored with K as the row index
+//                  (rows of whole 16-byte pieces), gathering the MFMA fragments element by element.
 //   k_gemm_kmajor  both operands K-major, k % 16 == 0: register-staged 64-byte K slabs.
 //   k_gemm_generic any layout and size: LDS tiles + v_dot4_i32_i8.
 // The tile kernel also serves the fp16 product of kernels/gemm.py:188-256 (cpmk_gemm_fp16): the
-// same bytes of K per lane feed v_mfma_f32_32x32x16_f16, with fp32 accumulators; there it also
-// takes operands stored with K as the row index (template parameter LAY).
+// same bytes of K per lane feed v_mfma_f32_32x32x16_f16, with fp32 accumulators.
 #include "common.h"
 #include <type_traits>
 
