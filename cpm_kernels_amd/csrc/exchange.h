@@ -53,7 +53,7 @@ __device__ inline bool xch_wait(const uint64_t* p, uint32_t tag, uint64_t deadli
             v = __builtin_bit_cast(float, (uint32_t)pkt);
             return true;
         }
-        if (wall_clock64() > deadline) {
+        if ((uint64_t)wall_clock64() > deadline) {
             v = 0.0f;
             return false;
         }
