@@ -625,16 +625,33 @@ static int launch_col(int32_t batch, const ColArgs& p, void* stream) {
                       (p.mean == nullptr || aligned16(p.mean)) && (p.var == nullptr || aligned16(p.var)) &&
                       (p.out_mean == nullptr || aligned16(p.out_mean)) && (p.out_var == nullptr || aligned16(p.out_var)) &&
                       (p.out_i8 == nullptr || (reinterpret_cast<uintptr_t>(p.out_i8) & 7u) == 0) && (int64_t)p.n * p.m < (1ll << 31) &&
-                      parts <= kColTeamMaxParts && tiles * batch * parts <= kXchSlots;
+                      parts <= kColTeamMaxParts && tiles * parts <= kXchSlots;
     if (wide) {
-        XchLaunch xl = {nullptr, 0};
-        if (parts > 1) {
-            const int rc = xch_begin(&xl);
-            if (rc != 0) return rc;
+        // teams use one packet slot per (team, part): batches beyond the pool go out in several launches
+        const int64_t per_launch = parts > 1 ? kXchSlots / (tiles * parts) : ((1ll << 31) - 1) / (tiles * parts);
+        for (int64_t b0 = 0; b0 < batch; b0 += per_launch) {
+            const int64_t nb = batch - b0 < per_launch ? batch - b0 : per_launch;
+            ColArgs q = p;
+            const int64_t e0 = b0 * p.n * p.m, c0 = b0 * p.m;
+            q.a = p.a + e0;
+            if (p.g) q.g = p.g + e0;
+            if (p.out) q.out = p.out + e0;
+            if (p.out_i8) q.out_i8 = p.out_i8 + e0;
+            if (p.mean) q.mean = p.mean + c0;
+            if (p.var) q.var = p.var + c0;
+            if (p.out_mean) q.out_mean = p.out_mean + c0;
+            if (p.out_var) q.out_var = p.out_var + c0;
+            if (p.sx && !p.bc) q.sx = p.sx + b0 * p.n;
+            XchLaunch xl = {nullptr, 0};
+            if (parts > 1) {
+                const int rc = xch_begin(&xl);
+                if (rc != 0) return rc;
+            }
+            hipLaunchKernelGGL((k_col_team<KIND>), dim3((unsigned)(tiles * nb * parts)), dim3(512), 0, (hipStream_t)stream, q,
+                               (int32_t)tiles, (int32_t)parts, xl.region, xl.tag);
+            if (int e = launch_status()) return e;
         }
-        hipLaunchKernelGGL((k_col_team<KIND>), dim3((unsigned)(tiles * batch * parts)), dim3(512), 0, (hipStream_t)stream, p,
-                           (int32_t)tiles, (int32_t)parts, xl.region, xl.tag);
-        return launch_status();
+        return 0;
     }
     if (batch > 65535) return CPMK_ETOOBIG;
     hipLaunchKernelGGL((k_col<KIND>), dim3((unsigned)ceil_div(p.m, 64), (unsigned)batch), dim3(256), 0, (hipStream_t)stream, p);

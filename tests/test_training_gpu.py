@@ -154,6 +154,26 @@ def test_softmax_backward(gpu, shape):
     assert_close_fp16(to_np(grad), ot.softmax_backward(out, g), rtol=2e-3, atol=1e-5, what="softmax_backward")
 
 
+def test_softmax_backward_more_teams_than_packet_slots(gpu):
+    """4200 x 2 team parts exceed the 8192 packet slots of one launch: the batch then goes out in several
+    launches.  The whole result must equal the result of the two halves run on their own, and the first
+    and last batch entries must match the oracle."""
+    _name("softmax_backward, batch split over launches")
+    b, n, m = 4200, 600, 64
+    gen = torch.Generator(device="cpu").manual_seed(5)
+    out = torch.softmax(torch.randn(b, n, m, generator=gen) * 2, dim=1).half().to(gpu)
+    g = torch.randn(b, n, m, generator=gen).half().to(gpu)
+    grad = torch.zeros_like(out)
+    ck.softmax_backward(b, n, m, out.data_ptr(), g.data_ptr(), grad.data_ptr(), stream())
+    halves = torch.zeros_like(out)
+    h = b // 2
+    ck.softmax_backward(h, n, m, out.data_ptr(), g.data_ptr(), halves.data_ptr(), stream())
+    ck.softmax_backward(b - h, n, m, out[h:].data_ptr(), g[h:].data_ptr(), halves[h:].data_ptr(), stream())
+    assert_bits_equal(to_np(grad), to_np(halves), "one call == two half calls")
+    for sl in (slice(0, 3), slice(b - 3, b), slice(4094, 4098)):
+        assert_close_fp16(to_np(grad[sl]), ot.softmax_backward(to_np(out[sl]), to_np(g[sl])), rtol=2e-3, atol=1e-5, what="softmax_backward %s" % (sl,))
+
+
 @pytest.mark.parametrize("shape", COL_SHAPES)
 def test_layernorm_training_kernels(gpu, shape):
     _name("layernorm forward_v/mv backward_v/mv", shape)
