@@ -175,17 +175,23 @@ int cpmk_gemm_quantize_cols(int32_t batch, int32_t n, int32_t m, const void* mat
     const int64_t tiles = ceil_div(m, 64), parts = ceil_div(n, 512);
     const bool team_ok = (m % 8 == 0) && (!out_transposed || n % 8 == 0) && aligned16(mat) && aligned16(scale) &&
                          ((reinterpret_cast<uintptr_t>(out) & 7u) == 0) && (int64_t)n * m < (1ll << 31) &&
-                         parts <= kColMaxParts && tiles * batch * parts <= kXchSlots;
+                         parts <= kColMaxParts && tiles * parts <= kXchSlots;
     if (team_ok) {
-        XchLaunch xl = {nullptr, 0};
-        if (parts > 1) {
-            const int rc = xch_begin(&xl);
-            if (rc != 0) return rc;
+        // teams use one packet slot per (team, part): batches beyond the pool go out in several launches
+        const int64_t per_launch = parts > 1 ? kXchSlots / (tiles * parts) : ((1ll << 31) - 1) / (tiles * parts);
+        for (int64_t b0 = 0; b0 < batch; b0 += per_launch) {
+            const int64_t nb = batch - b0 < per_launch ? batch - b0 : per_launch;
+            XchLaunch xl = {nullptr, 0};
+            if (parts > 1) {
+                const int rc = xch_begin(&xl);
+                if (rc != 0) return rc;
+            }
+            hipLaunchKernelGGL((k_col_quantize_team<512>), dim3((unsigned)(tiles * nb * parts)), dim3(512), 0, st, n, m,
+                               (int32_t)tiles, (int32_t)parts, (const half_t*)mat + b0 * n * m, (half_t*)scale + b0 * m,
+                               (int8_t*)out + b0 * n * m, out_transposed, xl.region, xl.tag);
+            if (int e = launch_status()) return e;
         }
-        hipLaunchKernelGGL((k_col_quantize_team<512>), dim3((unsigned)(tiles * batch * parts)), dim3(512), 0, st, n, m,
-                           (int32_t)tiles, (int32_t)parts, (const half_t*)mat, (half_t*)scale, (int8_t*)out,
-                           out_transposed, xl.region, xl.tag);
-        return launch_status();
+        return 0;
     }
     if (int e = cpmk_gemm_calc_scale_transpose(batch, n, m, mat, scale, stream)) return e;
     if (!out_transposed) return cpmk_gemm_round_transpose(batch, n, m, mat, scale, out, stream);

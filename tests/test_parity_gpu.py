@@ -106,6 +106,30 @@ def test_calc_scale_and_round_transpose(gpu, shape):
         assert_bits_equal(to_np(q3), np.ascontiguousarray(want), "gemm_quantize_cols int8 (transposed=%s)" % tr)
 
 
+def test_quantize_cols_more_teams_than_packet_slots(gpu):
+    """4200 columns tiles x 2 parts exceed the 8192 packet slots of one launch: the batch goes out in several
+    launches and must equal two half calls bit for bit; first and last entries against the oracle."""
+    _name("quantize_cols, batch split over launches")
+    b, n, m = 4200, 1000, 64
+    gen = torch.Generator(device="cpu").manual_seed(6)
+    x = (torch.randn(b, n, m, generator=gen) * 3).half().to(gpu)
+    for tr in (False, True):
+        sc = torch.zeros((b, m), dtype=torch.half, device=gpu); q = torch.zeros((b, m, n) if tr else (b, n, m), dtype=torch.int8, device=gpu)
+        ck.gemm_quantize_cols(b, n, m, x.data_ptr(), sc.data_ptr(), q.data_ptr(), tr, stream())
+        sc2 = torch.zeros_like(sc); q2 = torch.zeros_like(q)
+        h = b // 2
+        ck.gemm_quantize_cols(h, n, m, x.data_ptr(), sc2.data_ptr(), q2.data_ptr(), tr, stream())
+        ck.gemm_quantize_cols(b - h, n, m, x[h:].data_ptr(), sc2[h:].data_ptr(), q2[h:].data_ptr(), tr, stream())
+        assert_bits_equal(to_np(sc), to_np(sc2), "scales: one call == two half calls")
+        assert_bits_equal(to_np(q), to_np(q2), "int8: one call == two half calls")
+        for sl in (slice(0, 2), slice(b - 2, b), slice(4095, 4097)):
+            xs = to_np(x[sl])
+            s_ref = oracle.gemm_calc_scale_transpose(xs)
+            q_ref = oracle.gemm_round_transpose(xs, s_ref)
+            assert_bits_equal(to_np(sc[sl]), s_ref, "scales %s" % (sl,))
+            assert_bits_equal(to_np(q[sl]), np.ascontiguousarray(q_ref.transpose(0, 2, 1)) if tr else q_ref, "int8 %s" % (sl,))
+
+
 @pytest.mark.parametrize("rows0,rows1,m", [(512, 4096, 4096), (3, 0, 1000), (0, 7, 24), (5, 9, 30), (33, 17, 8200)])
 def test_quantize_pair(gpu, rows0, rows1, m):
     """Two tensors with rows of one length quantised by one launch == each by itself."""
