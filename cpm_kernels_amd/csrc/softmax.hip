@@ -379,18 +379,26 @@ static int softmax_dispatch(int32_t batch, int32_t n, int32_t m, const void* inp
             const int64_t tiles = ceil_div(m, 64);
             const bool big = n >= 2048;                       // 1024 rows a part, else 512
             const int64_t parts = ceil_div(n, big ? 1024 : 512);
-            if (parts <= kXchMaxParts && tiles * batch * parts <= kXchSlots) {
-                XchLaunch xl;
-                const int rc = xch_begin(&xl);
-                if (rc != 0) return rc;
-                const dim3 grid((unsigned)(tiles * batch * parts));
-                if (big)
-                    hipLaunchKernelGGL((k_softmax_team<1024, 8>), grid, dim3(1024), 0, st, n, m, (int32_t)tiles,
-                                       (int32_t)parts, x, y, xl.region, xl.tag);
-                else
-                    hipLaunchKernelGGL((k_softmax_team<512, 8>), grid, dim3(512), 0, st, n, m, (int32_t)tiles,
-                                       (int32_t)parts, x, y, xl.region, xl.tag);
-                return launch_status();
+            if (parts <= kXchMaxParts && tiles * parts <= kXchSlots) {
+                // one packet slot per (team, part): batches beyond the pool go out in several launches
+                const int64_t per_launch = kXchSlots / (tiles * parts);
+                for (int64_t b0 = 0; b0 < batch; b0 += per_launch) {
+                    const int64_t nb = batch - b0 < per_launch ? batch - b0 : per_launch;
+                    XchLaunch xl;
+                    const int rc = xch_begin(&xl);
+                    if (rc != 0) return rc;
+                    const dim3 grid((unsigned)(tiles * nb * parts));
+                    const half_t* xb = x + b0 * n * m;
+                    half_t* yb = y + b0 * n * m;
+                    if (big)
+                        hipLaunchKernelGGL((k_softmax_team<1024, 8>), grid, dim3(1024), 0, st, n, m, (int32_t)tiles,
+                                           (int32_t)parts, xb, yb, xl.region, xl.tag);
+                    else
+                        hipLaunchKernelGGL((k_softmax_team<512, 8>), grid, dim3(512), 0, st, n, m, (int32_t)tiles,
+                                           (int32_t)parts, xb, yb, xl.region, xl.tag);
+                    if (int e = launch_status()) return e;
+                }
+                return 0;
             }
         }
         // several tiles per compute unit: the persistent kernel keeps loads in flight during the arithmetic

@@ -502,6 +502,37 @@ def test_team_kernels_in_a_replayed_graph(gpu):
         assert_close_fp16(got_sm, oracle.softmax_forward(sx), rtol=1e-3, atol=1e-7, what="replay %d softmax" % it)
 
 
+def test_team_kernels_more_teams_than_packet_slots(gpu):
+    """3000 column tiles x 3 parts exceed the 8192 packet slots of one launch: layernorm and softmax then send
+    the batch out in several launches.  One call must equal two half calls bit for bit, and the first, last and
+    boundary batch entries must match the oracle."""
+    _name("team kernels, batch split over launches")
+    b, m = 3000, 64
+    gen = torch.Generator(device=gpu).manual_seed(8)
+    for name, n in (("layernorm", 1100), ("softmax", 2100)):
+        x = torch.randn(b, n, m, generator=gen, device=gpu, dtype=torch.float32).mul_(3).half()
+        y = torch.zeros_like(x); y2 = torch.zeros_like(x)
+        h = b // 2
+
+        def run(cnt, xin, out):
+            if name == "layernorm":
+                ck.layernorm_forward(cnt, n, m, xin.data_ptr(), out.data_ptr(), 1e-5, True, stream())
+            else:
+                ck.softmax_forward(cnt, n, m, xin.data_ptr(), out.data_ptr(), stream())
+        run(b, x, y)
+        run(h, x, y2)
+        run(b - h, x[h:], y2[h:])
+        assert_bits_equal(to_np(y), to_np(y2), name + ": one call == two half calls")
+        per_launch = 8192 // 3
+        for sl in (slice(0, 2), slice(b - 2, b), slice(per_launch - 1, per_launch + 1)):
+            xs = to_np(x[sl])
+            if name == "layernorm":
+                assert_close_fp16(to_np(y[sl]), oracle.layernorm_forward(xs, 1e-5, True), rtol=1e-3, atol=2e-4, what="layernorm %s" % (sl,))
+            else:
+                assert_close_fp16(to_np(y[sl]), oracle.softmax_forward(xs), rtol=1e-3, atol=1e-7, max_ulp=2, what="softmax %s" % (sl,))
+        del x, y, y2
+
+
 def test_scheduled_softmax_in_a_replayed_graph(gpu):
     """The many-tile softmax hands out tiles from a counter in device memory that its last workgroup
     clears.  Replays of a captured graph (same counter slot every time), launches back to back and
