@@ -105,6 +105,15 @@ __global__ __launch_bounds__(256) void k_copy_extend(int32_t old_size, int32_t n
     if (col < old_size) nw_buf[(int64_t)blockIdx.y * nw_size + col] = old_buf[(int64_t)blockIdx.y * old_size + col];
 }
 
+// the same, 8 halves per thread (both row lengths multiples of 8, 16-byte aligned buffers)
+__global__ __launch_bounds__(256) void k_copy_extend_wide(int32_t old_size, int32_t nw_size, const half_t* __restrict__ old_buf,
+                                                          half_t* __restrict__ nw_buf) {
+    const int32_t col = (blockIdx.x * 256 + threadIdx.x) * 8;
+    if (col < old_size)
+        *reinterpret_cast<half8_t*>(nw_buf + (int64_t)blockIdx.y * nw_size + col) =
+            *reinterpret_cast<const half8_t*>(old_buf + (int64_t)blockIdx.y * old_size + col);
+}
+
 // out[0] = 1 when any element is +-inf or NaN; out is left untouched otherwise (the caller clears it).
 __global__ __launch_bounds__(256) void k_has_nan_inf(int64_t n, const uint16_t* __restrict__ inp, int8_t* out) {
     bool bad = false;
@@ -175,8 +184,12 @@ int cpmk_copy_extend_buffer(int32_t batch, int32_t old_size, int32_t nw_size, co
     if (batch < 0 || old_size < 0 || nw_size < old_size) return CPMK_EBADARG;
     if ((int64_t)batch * old_size == 0) return 0;
     if (batch > 65535) return CPMK_ETOOBIG;
-    hipLaunchKernelGGL(k_copy_extend, dim3((unsigned)ceil_div(old_size, 256), (unsigned)batch), dim3(256), 0, (hipStream_t)stream,
-                       old_size, nw_size, (const half_t*)old_buffer, (half_t*)new_buffer);
+    if (old_size % 8 == 0 && nw_size % 8 == 0 && aligned16(old_buffer) && aligned16(new_buffer))
+        hipLaunchKernelGGL(k_copy_extend_wide, dim3((unsigned)ceil_div(old_size, 2048), (unsigned)batch), dim3(256), 0,
+                           (hipStream_t)stream, old_size, nw_size, (const half_t*)old_buffer, (half_t*)new_buffer);
+    else
+        hipLaunchKernelGGL(k_copy_extend, dim3((unsigned)ceil_div(old_size, 256), (unsigned)batch), dim3(256), 0, (hipStream_t)stream,
+                           old_size, nw_size, (const half_t*)old_buffer, (half_t*)new_buffer);
     return launch_status();
 }
 

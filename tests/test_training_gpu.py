@@ -316,7 +316,7 @@ def test_decode_utilities(gpu):
         ck.utils.adjustify_logits(b, n, ld.data_ptr(), 0.7, 0.25, 0.5, dev(freq).data_ptr(), stream())
         assert_bits_equal(to_np(ld), ot.adjustify_logits(logits, 0.7, 0.25, 0.5, freq), "adjustify_logits")
 
-    for b, old, new in ((3, 100, 250), (2, 1025, 1025), (1, 1, 5)):
+    for b, old, new in ((3, 100, 250), (2, 1025, 1025), (1, 1, 5), (5, 4096, 4160), (2, 2056, 2056), (3, 8, 24)):
         src = rand_half(rng, (b, old))
         dst0 = rand_half(rng, (b, new))
         dd = to_gpu(dst0)
