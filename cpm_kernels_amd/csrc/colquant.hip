@@ -56,10 +56,11 @@ __global__ __launch_bounds__(NT) void k_col_quantize_team(int32_t n, int32_t m, 
             const uint64_t deadline = wall_clock64() + kXchTimeoutTicks;
             float M = 0.0f;
             bool ok = true;
-            for (int32_t q = 0; q < parts; ++q) {
-                float x;
-                ok &= xch_wait(team_slots + (size_t)q * kXchVals + tid, tag, deadline, x);
-                M = fmaxf(M, x);
+            for (int32_t q0 = 0; q0 < parts; q0 += 8) {
+                float x[8];
+                ok &= xch_gather<8>(team_slots, parts, q0, tid, tag, deadline, x);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) M = fmaxf(M, x[j]);       // maxima are >= 0: absent parts (zeros) do not matter
             }
             tot[tid] = ok ? M : __builtin_nanf("");
         }

@@ -61,6 +61,36 @@ __device__ inline bool xch_wait(const uint64_t* p, uint32_t tag, uint64_t deadli
     }
 }
 
+// Packet `idx` of up to W consecutive parts q0 .. q0+W-1 (< parts) of a team, polled together so
+// that their round trips to the L2 overlap instead of following one another.  v[j] receives the value
+// of part q0 + j (0 where there is no such part, or none arrived in time); false on a time-out.
+template <int W>
+__device__ inline bool xch_gather(const uint64_t* team_slots, int parts, int q0, int idx, uint32_t tag, uint64_t deadline,
+                                  float (&v)[W]) {
+    uint32_t missing = 0;
+#pragma unroll
+    for (int j = 0; j < W; ++j) {
+        v[j] = 0.0f;
+        if (q0 + j < parts) missing |= 1u << j;
+    }
+    for (;;) {
+        uint64_t pk[W];
+#pragma unroll
+        for (int j = 0; j < W; ++j)
+            if (missing >> j & 1u)
+                pk[j] = __hip_atomic_load(team_slots + (size_t)(q0 + j) * kXchVals + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+        for (int j = 0; j < W; ++j)
+            if ((missing >> j & 1u) && (uint32_t)(pk[j] >> 32) == tag) {
+                v[j] = __builtin_bit_cast(float, (uint32_t)pk[j]);
+                missing &= ~(1u << j);
+            }
+        if (missing == 0) return true;
+        if ((uint64_t)wall_clock64() > deadline) return false;
+        __builtin_amdgcn_s_sleep(2);
+    }
+}
+
 // To be called by the first wave of a workgroup once the whole workgroup has collected its
 // packets (i.e. after the barrier that follows the xch_wait calls): counts the team members that
 // are done and lets the last one clear the team's `parts` slots and the counter.

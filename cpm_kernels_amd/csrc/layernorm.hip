@@ -134,10 +134,11 @@ __global__ __launch_bounds__(NT) void k_layernorm_team(int32_t n, int32_t m, int
         const uint64_t deadline = wall_clock64() + kXchTimeoutTicks;
         float acc = 0.0f;
         bool ok = true;
-        for (int32_t q = 0; q < parts; ++q) {
-            float x;
-            ok &= xch_wait(team_slots + (size_t)q * kXchVals + tid, tag, deadline, x);
-            acc += x;
+        for (int32_t q0 = 0; q0 < parts; q0 += 4) {        // four at a time: the registers of this kernel are full
+            float x[4];
+            ok &= xch_gather<4>(team_slots, parts, q0, tid, tag, deadline, x);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc += x[j];       // in part order; absent parts are zeros
         }
         tot[tid] = acc;
         if (!ok) failed = 1;

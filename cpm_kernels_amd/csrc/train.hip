@@ -335,10 +335,11 @@ __global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_b
             const uint64_t deadline = wall_clock64() + kXchTimeoutTicks;
             float acc = 0.0f;
             bool ok = true;
-            for (int32_t q = 0; q < parts; ++q) {
-                float x;
-                ok &= xch_wait(team_slots + (size_t)q * kXchVals + tid, tag, deadline, x);
-                acc = IS_MAX ? fmaxf(acc, x) : acc + x;
+            for (int32_t q0 = 0; q0 < parts; q0 += 8) {
+                float x[8];
+                ok &= xch_gather<8>(team_slots, parts, q0, tid, tag, deadline, x);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc = IS_MAX ? fmaxf(acc, x[j]) : acc + x[j];     // part order; absent parts are zeros
             }
             tot[tid] = ok ? acc : __builtin_nanf("");
         }
@@ -525,10 +526,11 @@ __global__ __launch_bounds__(256) void k_position_backward_team(int32_t query_le
         for (int i = tid; i < num_buckets; i += 256) {
             float acc = 0.0f;
             bool ok = true;
-            for (int32_t p = 0; p < parts; ++p) {
-                float x;
-                ok &= xch_wait(team_slots + (size_t)p * kXchVals + i, tag, deadline, x);
-                acc += x;
+            for (int32_t p0 = 0; p0 < parts; p0 += 8) {
+                float x[8];
+                ok &= xch_gather<8>(team_slots, parts, p0, i, tag, deadline, x);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc += x[j];
             }
             grad[(int64_t)h * num_buckets + i] = ok ? (half_t)acc : (half_t)__builtin_nanf("");
         }
