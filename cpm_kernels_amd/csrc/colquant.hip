@@ -44,14 +44,12 @@ __global__ __launch_bounds__(NT) void k_col_quantize_team(int32_t n, int32_t m, 
     float mx[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) mx[e] = (float)hm[e];
-    coltile_reduce<NT, LPR, 1, true>(mx, lds);           // every lane: this part's maxima of its 8 columns
-
-    if (parts > 1) {
+    if (parts == 1) {
+        coltile_reduce<NT, LPR, 1, true>(mx, lds);       // every lane: the maxima of its 8 columns
+    } else {
         uint64_t* team_slots = xch + (size_t)team * parts * kXchVals;
-        if (tid < LPR) {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) xch_post(team_slots + (size_t)part * kXchVals, tid * 8 + e, mx[e], tag);
-        }
+        // this part's maxima go straight from the reduction to its slot
+        coltile_reduce_to<NT, LPR, 1, true>(mx, lds, [&](int i, float r) { xch_post(team_slots + (size_t)part * kXchVals, i, r, tag); });
         if (tid < COLS) {
             const uint64_t deadline = wall_clock64() + kXchTimeoutTicks;
             float M = 0.0f;

@@ -105,4 +105,35 @@ __device__ inline void coltile_reduce(float (&v)[NV * 8], float* lds) {
     __syncthreads();
 }
 
+// The same reduction for kernels that only hand the totals on (to their team): thread i < COLS*NV
+// calls sink(i, total of packet i) -- packet g*COLS + c is statistic g of tile column c -- and
+// nothing is read back, which saves two barriers.  Needs more than one wave.
+template <int NT, int LPR, int NV, bool IS_MAX, class F>
+__device__ inline void coltile_reduce_to(float (&v)[NV * 8], float* lds, F&& sink) {
+    constexpr int NW = NT / 64, COLS = LPR * 8, W = COLS * NV;
+    static_assert(NW > 1, "one wave has nothing to combine");
+#pragma unroll
+    for (int o = LPR; o < 64; o <<= 1) {
+#pragma unroll
+        for (int e = 0; e < NV * 8; ++e) {
+            const float t = __shfl_xor(v[e], o, kWave);
+            v[e] = IS_MAX ? fmaxf(v[e], t) : v[e] + t;
+        }
+    }
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    if (lane < LPR) {
+#pragma unroll
+        for (int g = 0; g < NV; ++g)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) lds[w * W + g * COLS + lane * 8 + e] = v[g * 8 + e];
+    }
+    __syncthreads();
+    if (tid < W) {
+        float r = lds[tid];
+#pragma unroll
+        for (int i = 1; i < NW; ++i) r = IS_MAX ? fmaxf(r, lds[i * W + tid]) : r + lds[i * W + tid];
+        sink(tid, r);
+    }
+}
+
 }  // namespace cpmk

@@ -121,15 +121,10 @@ __global__ __launch_bounds__(NT) void k_layernorm_team(int32_t n, int32_t m, int
             s[e] += x;
             s[8 + e] += x * x;
         }
-    coltile_reduce<NT, LPR, 2, false>(s, lds);      // every lane: this part's sums of its 8 columns
-
-    // packet g*64 + c of a slot: statistic g (0 sum, 1 sum of squares) of tile column c
+    // packet g*64 + c of a slot: statistic g (0 sum, 1 sum of squares) of tile column c; the part's own
+    // totals go straight from the reduction to its slot
     uint64_t* team_slots = xch + (size_t)team * parts * kXchVals;
-    if (tid < LPR) {
-        uint64_t* slot = team_slots + (size_t)part * kXchVals;
-#pragma unroll
-        for (int k = 0; k < 16; ++k) xch_post(slot, (k >> 3) * T::COLS + tid * 8 + (k & 7), s[k], tag);
-    }
+    coltile_reduce_to<NT, LPR, 2, false>(s, lds, [&](int i, float r) { xch_post(team_slots + (size_t)part * kXchVals, i, r, tag); });
     if (tid < kXchVals) {
         const uint64_t deadline = wall_clock64() + kXchTimeoutTicks;
         float acc = 0.0f;

@@ -323,14 +323,12 @@ __global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_b
             else if constexpr (KIND == kSoftmaxBwd) s[e] += x * gi;
             else s[e] = fmaxf(s[e], fabsf(x * sxv[q]));
         }
-    coltile_reduce<NT, LPR, NV, IS_MAX>(s, lds);          // every lane: this part's statistics of its 8 columns
-
-    if (parts > 1) {
+    if (parts == 1) {
+        coltile_reduce<NT, LPR, NV, IS_MAX>(s, lds);      // every lane: the statistics of its 8 columns
+    } else {
         uint64_t* team_slots = xch + (size_t)team * parts * kXchVals;
-        if (tid < LPR) {
-#pragma unroll
-            for (int e = 0; e < NV * 8; ++e) xch_post(team_slots + (size_t)part * kXchVals, (e >> 3) * T::COLS + tid * 8 + (e & 7), s[e], tag);
-        }
+        // this part's statistics go straight from the reduction to its slot
+        coltile_reduce_to<NT, LPR, NV, IS_MAX>(s, lds, [&](int i, float r) { xch_post(team_slots + (size_t)part * kXchVals, i, r, tag); });
         if (tid < T::COLS * NV) {
             const uint64_t deadline = wall_clock64() + kXchTimeoutTicks;
             float acc = 0.0f;
