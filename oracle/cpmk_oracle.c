@@ -28,7 +28,7 @@
  *                             every (num_buckets, max_distance, bidirectional) of the
  *                             reference's tests (tests/test_position_embedding.py:6-13)
  *   arith / mask ............ exact float64 closed forms
- * Parity unpinned (undefined behaviour in the reference, documented in DESIGN.md): float->int8
+ * Parity unpinned (undefined behaviour in the reference): float->int8
  * conversion of quotients outside [-128,127] and of NaN (cuda/gemm.cu:16); saturation and
  * NaN->0 are this build's choice.
  */
@@ -315,8 +315,13 @@ void o_position_embedding_step(int32_t query_pos, int32_t key_len, int32_t num_b
     }
 }
 
-/* cuda/arith.cu:97-112 -- __hfma2: one rounding.  x*a+b is exact in double for fp16 inputs
- * whenever the result is finite in fp16, so d2h rounds once. */
+/* cuda/arith.cu:97-112 -- __hfma2: one rounding.  The product x*a of two fp16 values has at most
+ * 22 significant bits and is exact in double.  Adding b is exact in double as well whenever the
+ * product matters to the result (a finite result keeps the product below 2^17 and b's last bit
+ * is at least 2^-24: a span of 41 bits); where the product lies further below b than a double
+ * holds, the double sum is b or a double next to it, and b, itself an fp16 value, is far from
+ * any fp16 rounding boundary.  Either way d2h of the double sum equals the single rounding of
+ * the fused operation (tests/test_oracle.py checks it against exact rational arithmetic). */
 void o_arith_ln_mul_add(int32_t batch, int32_t n, int32_t m, const uint16_t* x, const uint16_t* alpha,
                         const uint16_t* beta, uint16_t* out) {
     for (int32_t b = 0; b < batch; ++b)

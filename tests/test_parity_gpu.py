@@ -314,7 +314,7 @@ def test_gemm_int8_extreme_values(gpu):
 
 
 def test_gemm_int8_config1_full(gpu):
-    """BASELINE config 1 at full size (A [1,512,4096], W [1,4096,4096]) through the whole
+    """The reference's own CPU-runnable case at full size (A [1,512,4096], W [1,4096,4096]) through the whole
     kernel-level pipeline, every stage bit-exact against the oracle."""
     _name("config1 full pipeline")
     g = torch.Generator().manual_seed(1001)
