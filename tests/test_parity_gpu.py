@@ -773,7 +773,9 @@ F16_GEMM_CASES = [  # (batch, n, k, m) in the kernel's convention: out (batch, n
     (1, 4, 4, 4), (2, 6, 10, 8), (3, 34, 64, 20), (2, 256, 128, 260), (1, 512, 1024, 384), (2, 130, 192, 70),
     # shapes the MFMA tile kernel takes in every layout (k % 64 == 0, m % 8 == 0; n % 8 == 0 for a (k, n) operand):
     # few rows (64 x 256 tiles) and many, ragged edges, one and several slabs of K
-    (2, 64, 128, 264), (3, 40, 192, 1032), (2, 60, 128, 264), (2, 264, 320, 520), (1, 136, 64, 256), (2, 24, 64, 8)]
+    (2, 64, 128, 264), (3, 40, 192, 1032), (2, 60, 128, 264), (2, 264, 320, 520), (1, 136, 64, 256), (2, 24, 64, 8),
+    # one slab of K and several 256 x 256 tiles per workgroup (attention scores): whole tiles only, and ragged edges
+    (32, 512, 64, 768), (24, 520, 64, 776)]
 
 
 @pytest.mark.parametrize("case", F16_GEMM_CASES)
