@@ -8,6 +8,7 @@ import numpy as np
 import pytest
 
 import test_parity_gpu as tp
+import test_training_gpu as tt
 
 pytestmark = pytest.mark.gpu
 
@@ -147,3 +148,32 @@ def _gemv_f16_shapes(seed, count):
 @pytest.mark.parametrize("shape", _gemv_f16_shapes(20245, 32))
 def test_random_gemv_fp16(gpu, shape):
     tp.test_gemv_fp16_family(gpu, shape)
+
+
+def _col_shapes(seed, count):
+    """(batch, n, m) for the dim-1 reductions of the training kernels: column heights around the
+    register-resident limit and the team sizes, widths with and without 16-byte accesses."""
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(count):
+        b = int(rng.choice([1, 2, 3, 9]))
+        n = _near(rng, [2, 64, 512, 1024, 2048, 4096, 6000], 24, lo=1)
+        m = _near(rng, [2, 8, 64, 128, 200, 520], 10, lo=2, step=int(rng.choice([2, 8])))
+        if b * n * m > 4_000_000:
+            b = 1
+        out.append((b, n, m))
+    return out
+
+
+@pytest.mark.parametrize("shape", _col_shapes(20246, 40))
+def test_random_training_reductions(gpu, shape):
+    tt.test_softmax_backward(gpu, shape)
+    tt.test_layernorm_training_kernels(gpu, shape)
+    tt.test_gemm_backward_quantisers(gpu, shape, bool(sum(shape) % 2))
+
+
+@pytest.mark.parametrize("shape", [(int(b), int(n), int(m)) for b, n, m in
+                                   np.random.default_rng(20247).integers(1, 300, (24, 3))])
+def test_random_transposes(gpu, shape):
+    tt.test_transpose(gpu, shape)
+    tt.test_transpose_i8(gpu, shape)
