@@ -177,3 +177,27 @@ def test_random_training_reductions(gpu, shape):
 def test_random_transposes(gpu, shape):
     tt.test_transpose(gpu, shape)
     tt.test_transpose_i8(gpu, shape)
+
+
+def _bmm_shapes(seed, count):
+    """(batch, M, K, N) of the torch-level bmm: multiples of 4, around the tile kernels' K % 128 and
+    16-byte conditions (the column quantisers and int8 transposes switch kernels on the same sizes)."""
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(count):
+        K = int(rng.choice([4 * int(rng.integers(1, 40)), 16 * int(rng.integers(1, 30)), 128 * int(rng.integers(1, 6))]))
+        M = _near(rng, [8, 64, 136, 264, 520], 20, lo=4, step=int(rng.choice([4, 16])))
+        N = _near(rng, [8, 64, 136, 264, 520], 20, lo=4, step=int(rng.choice([4, 16])))
+        out.append((int(rng.choice([1, 2, 3])), M, K, N))
+    return out
+
+
+@pytest.mark.parametrize("case", _bmm_shapes(20248, 24))
+def test_random_bmm_forward_backward(gpu, case):
+    import test_torch_gpu as tg
+    import test_torch_backward_gpu as tb
+    rng = np.random.default_rng(sum(case))
+    aT, bT = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+    tg.test_bmm_int8(gpu, case, aT, bT)
+    tb.test_bmm_backward(gpu, case, aT, bT, "int8")
+    tb.test_bmm_backward(gpu, case, not aT, bT, "fp16")
