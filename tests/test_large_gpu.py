@@ -1,0 +1,163 @@
+"""Tensors with more than 2^31 elements (and int8 operands beyond 2 GB): the element and byte
+offsets inside every kernel must be 64-bit, or unsigned 32-bit where the launcher bounds them.
+Inputs are drawn on the GPU; the oracle checks slices at the start, on either side of element
+2^31 and at the end, where a wrapped index would read or write the wrong place.  The outputs are
+pre-filled with a sentinel so that an element nobody wrote is seen as well.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import cpm_kernels_amd.kernels as ck
+from util import stream, to_np, assert_bits_equal, assert_close_fp16
+
+pytestmark = pytest.mark.gpu
+
+TWO31 = 2 ** 31
+
+
+def _name(*a):
+    print("case", *a, flush=True)
+
+
+def _randn_half(shape, seed, gpu, scale=1.0):
+    g = torch.Generator(device=gpu).manual_seed(seed)
+    x = torch.empty(shape, dtype=torch.half, device=gpu)
+    flat = x.view(-1)
+    step = 1 << 28                      # draw in pieces: no fp32 copy of the whole tensor
+    for i in range(0, flat.numel(), step):
+        n = min(step, flat.numel() - i)
+        flat[i:i + n] = (torch.randn(n, generator=g, device=gpu) * scale).half()
+    return x
+
+
+def _spans(total, width):
+    """Flat element ranges worth checking: start, around 2^31, end."""
+    out = [(0, width)]
+    if total > TWO31 + width:
+        out.append((TWO31 - width, TWO31 + width))
+    out.append((total - width, total))
+    return out
+
+
+def test_elementwise_beyond_2_31_elements(gpu):
+    batch, n = 2, 2 ** 30 + 2048
+    total = batch * n
+    _name("elementwise", batch, n)
+    x = _randn_half((batch, n), 11, gpu, 2.0)
+    y = _randn_half((batch, n), 12, gpu, 2.0)
+    out = torch.full((batch, n), 77.0, dtype=torch.half, device=gpu)
+    ck.arith_element_add(batch, n, x.data_ptr(), y.data_ptr(), out.data_ptr(), stream())
+    xf, yf, of = x.view(-1), y.view(-1), out.view(-1)
+    for a, b in _spans(total, 4096):
+        assert_bits_equal(to_np(of[a:b]), oracle.arith_element_add(to_np(xf[a:b])[None], to_np(yf[a:b])[None])[0], "element_add [%d,%d)" % (a, b))
+    out.fill_(77.0)
+    ck.gelu_forward(batch, n, x.data_ptr(), out.data_ptr(), stream())
+    for a, b in _spans(total, 4096):
+        # tanh-GELU, 1e-3 relative; atol covers the fp16 subnormal tail for very negative inputs
+        assert_close_fp16(to_np(of[a:b]), oracle.gelu_forward(to_np(xf[a:b])[None])[0], rtol=1e-3, atol=1e-6, what="gelu [%d,%d)" % (a, b))
+    assert int((of == 77.0).sum()) == 0, "gelu left elements unwritten"
+
+
+def test_softmax_layernorm_beyond_2_31_elements(gpu):
+    b, n, m = 2064, 1024, 1024         # batch 2048 starts at element 2^31
+    _name("softmax / layernorm, many tiles", (b, n, m))
+    x = _randn_half((b, n, m), 13, gpu, 3.0)
+    out = torch.full((b, n, m), 77.0, dtype=torch.half, device=gpu)
+    ck.softmax_forward(b, n, m, x.data_ptr(), out.data_ptr(), stream())
+    for i in (0, 2047, 2048, b - 1):
+        assert_close_fp16(to_np(out[i:i + 1]), oracle.softmax_forward(to_np(x[i:i + 1])), rtol=1e-3, atol=1e-7, max_ulp=2, what="softmax batch %d" % i)
+    out.fill_(77.0)
+    ck.layernorm_forward(b, n, m, x.data_ptr(), out.data_ptr(), 1e-5, True, stream())
+    for i in (0, 2047, 2048, b - 1):
+        assert_close_fp16(to_np(out[i:i + 1]), oracle.layernorm_forward(to_np(x[i:i + 1]), 1e-5, True), rtol=1e-3, atol=2e-4, what="layernorm batch %d" % i)
+    del out
+    # tall columns: teams of workgroups, batch 128 starts at element 2^31 (the same 129 * 2^24 values)
+    b, n, m = 129, 8192, 2048
+    _name("softmax / layernorm, teams", (b, n, m))
+    x = x.view(b, n, m)
+    out = torch.full((b, n, m), 77.0, dtype=torch.half, device=gpu)
+    ck.layernorm_forward(b, n, m, x.data_ptr(), out.data_ptr(), 1e-5, True, stream())
+    for i in (0, 127, 128):
+        assert_close_fp16(to_np(out[i:i + 1]), oracle.layernorm_forward(to_np(x[i:i + 1]), 1e-5, True), rtol=1e-3, atol=2e-4, what="tall layernorm batch %d" % i)
+    out.fill_(77.0)
+    ck.softmax_forward(b, n, m, x.data_ptr(), out.data_ptr(), stream())
+    for i in (0, 127, 128):
+        assert_close_fp16(to_np(out[i:i + 1]), oracle.softmax_forward(to_np(x[i:i + 1])), rtol=1e-3, atol=1e-7, max_ulp=2, what="tall softmax batch %d" % i)
+
+
+def test_quantisers_beyond_2_31_elements(gpu):
+    b, n, m = 1, 2 ** 20 + 16, 2048    # row 2^20 starts at element 2^31
+    _name("row quantiser", (b, n, m))
+    x = _randn_half((b, n, m), 14, gpu, 1.5)
+    sc = torch.full((b, n), 77.0, dtype=torch.half, device=gpu)
+    q = torch.full((b, n, m), 99, dtype=torch.int8, device=gpu)
+    ck.gemm_quantize(b, n, m, x.data_ptr(), sc.data_ptr(), q.data_ptr(), False, stream())
+    for r0 in (0, 2 ** 20 - 8, n - 16):
+        xs = to_np(x[:, r0:r0 + 16])
+        s_ref = oracle.gemm_calc_scale(xs)
+        assert_bits_equal(to_np(sc[:, r0:r0 + 16]), s_ref, "row scales at %d" % r0)
+        assert_bits_equal(to_np(q[:, r0:r0 + 16]), oracle.gemm_round(xs, s_ref), "row int8 at %d" % r0)
+    del q, sc
+    # per column, written transposed: batch 128 of 129 x (8192, 2048) starts at element 2^31
+    del x
+    b, n, m = 129, 8192, 2048
+    _name("column quantiser", (b, n, m))
+    x = _randn_half((b, n, m), 16, gpu, 1.5)
+    for tr in (False, True):
+        sc = torch.full((b, m), 77.0, dtype=torch.half, device=gpu)
+        q = torch.full((b, m, n) if tr else (b, n, m), 99, dtype=torch.int8, device=gpu)
+        ck.gemm_quantize_cols(b, n, m, x.data_ptr(), sc.data_ptr(), q.data_ptr(), tr, stream())
+        for i in (0, 127, 128):
+            xs = to_np(x[i:i + 1])
+            s_ref = oracle.gemm_calc_scale_transpose(xs)
+            q_ref = oracle.gemm_round_transpose(xs, s_ref)
+            assert_bits_equal(to_np(sc[i:i + 1]), s_ref, "column scales, batch %d" % i)
+            want = np.ascontiguousarray(q_ref.transpose(0, 2, 1)) if tr else q_ref
+            assert_bits_equal(to_np(q[i:i + 1]), want, "column int8 (transposed=%s), batch %d" % (tr, i))
+        del q, sc
+
+
+def _rows_ref(P, Q, rows):
+    """Exact int32 rows of P @ Q^T (K-major operands) for the given row indices."""
+    return (P[rows].astype(np.float64) @ Q.astype(np.float64).T).astype(np.int32)
+
+
+def test_gemm_int8_operand_beyond_2_gib_and_output_beyond_2_31(gpu):
+    # a row operand of 2.6 GB: byte offsets of its last rows exceed 2^31
+    n, k, m = 40000, 65536, 256
+    _name("gemm_int8, operand of %.1f GB" % (n * k / 2 ** 30), (n, k, m))
+    g = torch.Generator(device=gpu).manual_seed(15)
+    P = torch.randint(-127, 128, (1, n, k), generator=g, dtype=torch.int8, device=gpu)     # kernel "B": (n, k)
+    Q = torch.randint(-127, 128, (1, m, k), generator=g, dtype=torch.int8, device=gpu)     # kernel "A" with aT: (m, k)
+    out = torch.full((1, n, m), 12345, dtype=torch.int32, device=gpu)
+    ck.gemm_int8(m, k, n, 1, 1, True, False, Q.data_ptr(), P.data_ptr(), out.data_ptr(), stream())
+    Qn = to_np(Q[0])
+    for r0 in (0, 32768 - 8, n - 16):      # row 32768 starts at byte 2^31
+        rows = slice(r0, r0 + 16)
+        assert_bits_equal(to_np(out[0, rows]), _rows_ref(to_np(P[0, rows]), Qn, slice(None)), "rows %d.." % r0)
+    del P, Q, out
+    # an int32 product of 2.7e9 elements: the output index crosses 2^31 inside row 52428
+    n, k, m = 65536, 128, 40960
+    _name("gemm_int8, output of %.1f G elements" % (n * m / 1e9), (n, k, m))
+    P = torch.randint(-127, 128, (1, n, k), generator=g, dtype=torch.int8, device=gpu)
+    Q = torch.randint(-127, 128, (1, m, k), generator=g, dtype=torch.int8, device=gpu)
+    out = torch.full((1, n, m), 12345, dtype=torch.int32, device=gpu)
+    ck.gemm_int8(m, k, n, 1, 1, True, False, Q.data_ptr(), P.data_ptr(), out.data_ptr(), stream())
+    Qn = to_np(Q[0])
+    for r0 in (0, TWO31 // m - 8, n - 16):
+        rows = slice(r0, r0 + 16)
+        assert_bits_equal(to_np(out[0, rows]), _rows_ref(to_np(P[0, rows]), Qn, slice(None)), "rows %d.." % r0)
+    # the fused epilogue writes fp16 at the same indices
+    srow = (torch.rand(n, generator=g, device=gpu) * 0.05 + 1e-4).half()
+    scol = (torch.rand(m, generator=g, device=gpu) * 0.01 + 1e-5).half()
+    del out
+    o16 = torch.full((1, n, m), 77.0, dtype=torch.half, device=gpu)
+    ck.gemm_int8_scale(m, k, n, 1, 1, True, False, Q.data_ptr(), P.data_ptr(), srow.data_ptr(), scol.data_ptr(),
+                       True, True, o16.data_ptr(), stream())
+    for r0 in (0, TWO31 // m - 8, n - 16):
+        rows = slice(r0, r0 + 16)
+        acc = _rows_ref(to_np(P[0, rows]), Qn, slice(None))[None]
+        ref = oracle.gemm_scale(acc, to_np(srow[rows]), to_np(scol), True, True)
+        assert_bits_equal(to_np(o16[:, rows]), ref, "fused rows %d.." % r0)
