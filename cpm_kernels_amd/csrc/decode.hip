@@ -66,12 +66,16 @@ int cpmk_embedding_forward(int32_t batch, int32_t hidden_size, int32_t seq_len, 
     clear_stale_error();
     if (batch < 0 || hidden_size < 0 || seq_len < 0) return CPMK_EBADARG;
     if ((int64_t)batch * hidden_size * seq_len == 0) return 0;
-    if (batch > 65535 || ceil_div(hidden_size, 64) > 65535) return CPMK_ETOOBIG;
+    if (ceil_div(hidden_size, 64) > 65535) return CPMK_ETOOBIG;
     const int vec = (hidden_size % 8 == 0) && aligned16(weights);
-    dim3 grid((unsigned)ceil_div(seq_len, 64), (unsigned)ceil_div(hidden_size, 64), (unsigned)batch);
-    hipLaunchKernelGGL(k_embedding_forward, grid, dim3(256), 0, (hipStream_t)stream, hidden_size, seq_len,
-                       (const int32_t*)ids, (const half_t*)weights, (half_t*)out, vec);
-    return launch_status();
+    for (int64_t b0 = 0; b0 < batch; b0 += 65535) {       // (grid z: at most 65535 batch entries per launch)
+        const int64_t nb = batch - b0 < 65535 ? batch - b0 : 65535;
+        dim3 grid((unsigned)ceil_div(seq_len, 64), (unsigned)ceil_div(hidden_size, 64), (unsigned)nb);
+        hipLaunchKernelGGL(k_embedding_forward, grid, dim3(256), 0, (hipStream_t)stream, hidden_size, seq_len,
+                           (const int32_t*)ids + b0 * seq_len, (const half_t*)weights, (half_t*)out + b0 * hidden_size * seq_len, vec);
+        if (int e = launch_status()) return e;
+    }
+    return 0;
 }
 
 int cpmk_embedding_step(int32_t batch, int32_t embedding_size, const void* ids, const void* weights, void* out,

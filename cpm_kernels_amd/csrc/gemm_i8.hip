@@ -768,7 +768,19 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
     if (!(batchA == batchB || batchA == 1 || batchB == 1)) return CPMK_EBADARG;   // :140
     const int batch = batchA > batchB ? batchA : batchB;
     if (m == 0 || n == 0) return 0;
-    if (batch > 65535) return CPMK_ETOOBIG;
+    if (batch > 65535) {      // some kernels index the batch with the grid's z dimension: at most 65535 entries per call
+        constexpr int64_t ESZ_OUT = FUSED ? 2 : 4;
+        for (int64_t b0 = 0; b0 < batch; b0 += 65535) {
+            const int32_t nb = (int32_t)(batch - b0 < 65535 ? batch - b0 : 65535);
+            const int rc = gemm_dispatch<FUSED>(
+                m, k, n, batchA == 1 ? 1 : nb, batchB == 1 ? 1 : nb, aT, bT,
+                (const int8_t*)A + (batchA == 1 ? 0 : b0 * m * k), (const int8_t*)B + (batchB == 1 ? 0 : b0 * n * k),
+                srow ? (const half_t*)srow + (bcr ? 0 : b0 * n) : nullptr, scol ? (const half_t*)scol + (bcc ? 0 : b0 * m) : nullptr,
+                bcr, bcc, (int8_t*)out + b0 * n * m * ESZ_OUT, st);
+            if (rc != 0) return rc;
+        }
+        return 0;
+    }
     GemmArgs a;
     a.P = (const int8_t*)B; a.Q = (const int8_t*)A; a.out = out;
     a.srow = (const half_t*)srow; a.scol = (const half_t*)scol;
@@ -885,7 +897,17 @@ static int gemm_f16_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, in
     if (!(batchA == batchB || batchA == 1 || batchB == 1)) return CPMK_EBADARG;   // :201
     const int batch = batchA > batchB ? batchA : batchB;
     if (m == 0 || n == 0) return 0;
-    if (batch > 65535 || k > (1 << 30)) return CPMK_ETOOBIG;
+    if (k > (1 << 30)) return CPMK_ETOOBIG;
+    if (batch > 65535) {      // (grid z: at most 65535 batch entries per call)
+        for (int64_t b0 = 0; b0 < batch; b0 += 65535) {
+            const int32_t nb = (int32_t)(batch - b0 < 65535 ? batch - b0 : 65535);
+            const int rc = gemm_f16_dispatch(m, k, n, batchA == 1 ? 1 : nb, batchB == 1 ? 1 : nb, aT, bT,
+                                             (const half_t*)A + (batchA == 1 ? 0 : b0 * m * k), (const half_t*)B + (batchB == 1 ? 0 : b0 * n * k),
+                                             (half_t*)out + b0 * n * m, st);
+            if (rc != 0) return rc;
+        }
+        return 0;
+    }
     GemmArgs a;
     a.P = (const int8_t*)B; a.Q = (const int8_t*)A; a.out = out;
     a.srow = nullptr; a.scol = nullptr;

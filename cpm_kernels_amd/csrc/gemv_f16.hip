@@ -159,12 +159,15 @@ int cpmk_gemv_fp16_transpose(int32_t batch, int32_t dim_out, int32_t dim_in, con
     clear_stale_error();
     if (batch < 0 || dim_out < 0 || dim_in < 0) return CPMK_EBADARG;
     if ((int64_t)batch * dim_out == 0) return 0;
-    if (batch > 65535) return CPMK_ETOOBIG;
     const int vec8 = (dim_out % 8 == 0) && aligned16(mat);
-    dim3 grid((unsigned)ceil_div(dim_out, 64), (unsigned)batch);
-    hipLaunchKernelGGL(k_gemv_f16_transpose, grid, dim3(256), 0, (hipStream_t)stream, dim_out, dim_in, (const half_t*)mat,
-                       (const half_t*)vec, (half_t*)out, vec8);
-    return launch_status();
+    for (int64_t b0 = 0; b0 < batch; b0 += 65535) {       // (grid y: at most 65535 batch entries per launch)
+        const int64_t nb = batch - b0 < 65535 ? batch - b0 : 65535;
+        dim3 grid((unsigned)ceil_div(dim_out, 64), (unsigned)nb);
+        hipLaunchKernelGGL(k_gemv_f16_transpose, grid, dim3(256), 0, (hipStream_t)stream, dim_out, dim_in,
+                           (const half_t*)mat + b0 * dim_in * dim_out, (const half_t*)vec + b0 * dim_in, (half_t*)out + b0 * dim_out, vec8);
+        if (int e = launch_status()) return e;
+    }
+    return 0;
 }
 
 int cpmk_gemv_broadcast_mat_fp16(int32_t batch, int32_t dim_out, int32_t dim_in, const void* mat, const void* vec,

@@ -387,10 +387,16 @@ int cpmk_gemm_calc_scale_transpose(int32_t batch, int32_t n, int32_t m, const vo
     if (int e = check3(batch, n, m)) return e;
     if (batch == 0 || m == 0) return 0;
     const bool vec = (m % 8 == 0) && aligned16(mat);
-    dim3 grid((unsigned)ceil_div(m, 64), (unsigned)batch);
-    if (vec) hipLaunchKernelGGL((k_col_absmax<true>), grid, dim3(256), 0, (hipStream_t)stream, n, m, (const half_t*)mat, (half_t*)out);
-    else hipLaunchKernelGGL((k_col_absmax<false>), grid, dim3(256), 0, (hipStream_t)stream, n, m, (const half_t*)mat, (half_t*)out);
-    return launch_status();
+    for (int64_t b0 = 0; b0 < batch; b0 += 65535) {       // (grid y: at most 65535 batch entries per launch)
+        const int64_t nb = batch - b0 < 65535 ? batch - b0 : 65535;
+        dim3 grid((unsigned)ceil_div(m, 64), (unsigned)nb);
+        const half_t* src = (const half_t*)mat + b0 * n * m;
+        half_t* dst = (half_t*)out + b0 * m;
+        if (vec) hipLaunchKernelGGL((k_col_absmax<true>), grid, dim3(256), 0, (hipStream_t)stream, n, m, src, dst);
+        else hipLaunchKernelGGL((k_col_absmax<false>), grid, dim3(256), 0, (hipStream_t)stream, n, m, src, dst);
+        if (int e = launch_status()) return e;
+    }
+    return 0;
 }
 
 int cpmk_gemm_round(int32_t batch, int32_t n, int32_t m, const void* mat, const void* scale, void* out,

@@ -411,10 +411,14 @@ static int softmax_dispatch(int32_t batch, int32_t n, int32_t m, const void* inp
         else if (n <= 512 * 8) ok = launch_tile_r<1024, 2>((int)ceil_div(n, 512), batch, n, m, x, y, st);
         if (ok) return launch_status();
     }
-    if (batch > 65535) return CPMK_ETOOBIG;
-    dim3 grid((unsigned)ceil_div(m, 64), (unsigned)batch);
-    hipLaunchKernelGGL(k_softmax_generic, grid, dim3(256), 0, st, n, m, x, y);
-    return launch_status();
+    // the batch is the grid's y dimension (at most 65535): larger batches go out in several launches
+    for (int64_t b0 = 0; b0 < batch; b0 += 65535) {
+        const int64_t nb = batch - b0 < 65535 ? batch - b0 : 65535;
+        hipLaunchKernelGGL(k_softmax_generic, dim3((unsigned)ceil_div(m, 64), (unsigned)nb), dim3(256), 0, st, n, m,
+                           x + b0 * n * m, y + b0 * n * m);
+        if (int e = launch_status()) return e;
+    }
+    return 0;
 }
 
 }  // namespace cpmk

@@ -615,6 +615,22 @@ static int launch_ew(int64_t rows, int64_t cols, int64_t n, const void* x, const
     return launch_status();
 }
 
+// the arguments of batch entries b0 onwards
+static ColArgs col_args_from(const ColArgs& p, int64_t b0) {
+    ColArgs q = p;
+    const int64_t e0 = b0 * p.n * p.m, c0 = b0 * p.m;
+    q.a = p.a + e0;
+    if (p.g) q.g = p.g + e0;
+    if (p.out) q.out = p.out + e0;
+    if (p.out_i8) q.out_i8 = p.out_i8 + e0;
+    if (p.mean) q.mean = p.mean + c0;
+    if (p.var) q.var = p.var + c0;
+    if (p.out_mean) q.out_mean = p.out_mean + c0;
+    if (p.out_var) q.out_var = p.out_var + c0;
+    if (p.sx && !p.bc) q.sx = p.sx + b0 * p.n;
+    return q;
+}
+
 template <int KIND>
 static int launch_col(int32_t batch, const ColArgs& p, void* stream) {
     if (batch < 0 || p.n < 0 || p.m < 0) return CPMK_EBADARG;
@@ -631,17 +647,7 @@ static int launch_col(int32_t batch, const ColArgs& p, void* stream) {
         const int64_t per_launch = parts > 1 ? kXchSlots / (tiles * parts) : ((1ll << 31) - 1) / (tiles * parts);
         for (int64_t b0 = 0; b0 < batch; b0 += per_launch) {
             const int64_t nb = batch - b0 < per_launch ? batch - b0 : per_launch;
-            ColArgs q = p;
-            const int64_t e0 = b0 * p.n * p.m, c0 = b0 * p.m;
-            q.a = p.a + e0;
-            if (p.g) q.g = p.g + e0;
-            if (p.out) q.out = p.out + e0;
-            if (p.out_i8) q.out_i8 = p.out_i8 + e0;
-            if (p.mean) q.mean = p.mean + c0;
-            if (p.var) q.var = p.var + c0;
-            if (p.out_mean) q.out_mean = p.out_mean + c0;
-            if (p.out_var) q.out_var = p.out_var + c0;
-            if (p.sx && !p.bc) q.sx = p.sx + b0 * p.n;
+            const ColArgs q = col_args_from(p, b0);
             XchLaunch xl = {nullptr, 0};
             if (parts > 1) {
                 const int rc = xch_begin(&xl);
@@ -653,9 +659,14 @@ static int launch_col(int32_t batch, const ColArgs& p, void* stream) {
         }
         return 0;
     }
-    if (batch > 65535) return CPMK_ETOOBIG;
-    hipLaunchKernelGGL((k_col<KIND>), dim3((unsigned)ceil_div(p.m, 64), (unsigned)batch), dim3(256), 0, (hipStream_t)stream, p);
-    return launch_status();
+    // the batch is the grid's y dimension (at most 65535): larger batches go out in several launches
+    for (int64_t b0 = 0; b0 < batch; b0 += 65535) {
+        const int64_t nb = batch - b0 < 65535 ? batch - b0 : 65535;
+        hipLaunchKernelGGL((k_col<KIND>), dim3((unsigned)ceil_div(p.m, 64), (unsigned)nb), dim3(256), 0, (hipStream_t)stream,
+                           col_args_from(p, b0));
+        if (int e = launch_status()) return e;
+    }
+    return 0;
 }
 
 }  // namespace cpmk

@@ -139,26 +139,37 @@ int cpmk_transpose(int32_t batch, int32_t n, int32_t m, const void* inp, void* o
     clear_stale_error();
     if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
     if ((int64_t)batch * n * m == 0) return 0;
-    if (batch > 65535 || ceil_div(n, 64) > 65535) return CPMK_ETOOBIG;
-    const dim3 grid((unsigned)ceil_div(m, 64), (unsigned)ceil_div(n, 64), (unsigned)batch);
-    if (n % 8 == 0 && m % 8 == 0 && aligned16(inp) && aligned16(out))
-        hipLaunchKernelGGL(k_transpose_wide, grid, dim3(256), 0, (hipStream_t)stream, n, m, (const half_t*)inp, (half_t*)out);
-    else
-        hipLaunchKernelGGL(k_transpose, grid, dim3(256), 0, (hipStream_t)stream, n, m, (const half_t*)inp, (half_t*)out);
-    return launch_status();
+    if (ceil_div(n, 64) > 65535) return CPMK_ETOOBIG;
+    const bool wide = n % 8 == 0 && m % 8 == 0 && aligned16(inp) && aligned16(out);
+    // the batch is the grid's z dimension (at most 65535): larger batches go out in several launches
+    for (int64_t b0 = 0; b0 < batch; b0 += 65535) {
+        const int64_t nb = batch - b0 < 65535 ? batch - b0 : 65535;
+        const dim3 grid((unsigned)ceil_div(m, 64), (unsigned)ceil_div(n, 64), (unsigned)nb);
+        const half_t* src = (const half_t*)inp + b0 * n * m;
+        half_t* dst = (half_t*)out + b0 * n * m;
+        if (wide) hipLaunchKernelGGL(k_transpose_wide, grid, dim3(256), 0, (hipStream_t)stream, n, m, src, dst);
+        else hipLaunchKernelGGL(k_transpose, grid, dim3(256), 0, (hipStream_t)stream, n, m, src, dst);
+        if (int e = launch_status()) return e;
+    }
+    return 0;
 }
 
 int cpmk_transpose_i8(int32_t batch, int32_t n, int32_t m, const void* inp, void* out, void* stream) {
     clear_stale_error();
     if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
     if ((int64_t)batch * n * m == 0) return 0;
-    if (batch > 65535 || ceil_div(n, 64) > 65535) return CPMK_ETOOBIG;
-    const dim3 grid((unsigned)ceil_div(m, 64), (unsigned)ceil_div(n, 64), (unsigned)batch);
-    if (n % 16 == 0 && m % 16 == 0 && aligned16(inp) && aligned16(out))
-        hipLaunchKernelGGL(k_transpose_i8<true>, grid, dim3(256), 0, (hipStream_t)stream, n, m, (const int8_t*)inp, (int8_t*)out);
-    else
-        hipLaunchKernelGGL(k_transpose_i8<false>, grid, dim3(256), 0, (hipStream_t)stream, n, m, (const int8_t*)inp, (int8_t*)out);
-    return launch_status();
+    if (ceil_div(n, 64) > 65535) return CPMK_ETOOBIG;
+    const bool wide = n % 16 == 0 && m % 16 == 0 && aligned16(inp) && aligned16(out);
+    for (int64_t b0 = 0; b0 < batch; b0 += 65535) {       // (grid z: at most 65535 batch entries per launch)
+        const int64_t nb = batch - b0 < 65535 ? batch - b0 : 65535;
+        const dim3 grid((unsigned)ceil_div(m, 64), (unsigned)ceil_div(n, 64), (unsigned)nb);
+        const int8_t* src = (const int8_t*)inp + b0 * n * m;
+        int8_t* dst = (int8_t*)out + b0 * n * m;
+        if (wide) hipLaunchKernelGGL(k_transpose_i8<true>, grid, dim3(256), 0, (hipStream_t)stream, n, m, src, dst);
+        else hipLaunchKernelGGL(k_transpose_i8<false>, grid, dim3(256), 0, (hipStream_t)stream, n, m, src, dst);
+        if (int e = launch_status()) return e;
+    }
+    return 0;
 }
 
 int cpmk_array_add(void* array, int32_t pos, int32_t val, void* stream) {
@@ -183,14 +194,20 @@ int cpmk_copy_extend_buffer(int32_t batch, int32_t old_size, int32_t nw_size, co
     clear_stale_error();
     if (batch < 0 || old_size < 0 || nw_size < old_size) return CPMK_EBADARG;
     if ((int64_t)batch * old_size == 0) return 0;
-    if (batch > 65535) return CPMK_ETOOBIG;
-    if (old_size % 8 == 0 && nw_size % 8 == 0 && aligned16(old_buffer) && aligned16(new_buffer))
-        hipLaunchKernelGGL(k_copy_extend_wide, dim3((unsigned)ceil_div(old_size, 2048), (unsigned)batch), dim3(256), 0,
-                           (hipStream_t)stream, old_size, nw_size, (const half_t*)old_buffer, (half_t*)new_buffer);
-    else
-        hipLaunchKernelGGL(k_copy_extend, dim3((unsigned)ceil_div(old_size, 256), (unsigned)batch), dim3(256), 0, (hipStream_t)stream,
-                           old_size, nw_size, (const half_t*)old_buffer, (half_t*)new_buffer);
-    return launch_status();
+    const bool wide = old_size % 8 == 0 && nw_size % 8 == 0 && aligned16(old_buffer) && aligned16(new_buffer);
+    for (int64_t b0 = 0; b0 < batch; b0 += 65535) {       // (grid y: at most 65535 batch entries per launch)
+        const int64_t nb = batch - b0 < 65535 ? batch - b0 : 65535;
+        const half_t* src = (const half_t*)old_buffer + b0 * old_size;
+        half_t* dst = (half_t*)new_buffer + b0 * nw_size;
+        if (wide)
+            hipLaunchKernelGGL(k_copy_extend_wide, dim3((unsigned)ceil_div(old_size, 2048), (unsigned)nb), dim3(256), 0,
+                               (hipStream_t)stream, old_size, nw_size, src, dst);
+        else
+            hipLaunchKernelGGL(k_copy_extend, dim3((unsigned)ceil_div(old_size, 256), (unsigned)nb), dim3(256), 0, (hipStream_t)stream,
+                               old_size, nw_size, src, dst);
+        if (int e = launch_status()) return e;
+    }
+    return 0;
 }
 
 int cpmk_has_nan_inf(int64_t n, const void* inp, void* out, void* stream) {
@@ -207,10 +224,14 @@ int cpmk_copy_pos_hidden(int32_t batch, int32_t hidden_size, int32_t seq_len, in
     clear_stale_error();
     if (batch < 0 || hidden_size < 0 || seq_len < 0 || pos < 0 || (seq_len > 0 && pos >= seq_len)) return CPMK_EBADARG;
     if ((int64_t)batch * hidden_size * seq_len == 0) return 0;
-    if (batch > 65535) return CPMK_ETOOBIG;
-    hipLaunchKernelGGL(k_copy_pos_hidden, dim3((unsigned)ceil_div(hidden_size, 256), (unsigned)batch), dim3(256), 0,
-                       (hipStream_t)stream, hidden_size, seq_len, pos, (const half_t*)inp, (half_t*)out);
-    return launch_status();
+    for (int64_t b0 = 0; b0 < batch; b0 += 65535) {       // (grid y: at most 65535 batch entries per launch)
+        const int64_t nb = batch - b0 < 65535 ? batch - b0 : 65535;
+        hipLaunchKernelGGL(k_copy_pos_hidden, dim3((unsigned)ceil_div(hidden_size, 256), (unsigned)nb), dim3(256), 0,
+                           (hipStream_t)stream, hidden_size, seq_len, pos, (const half_t*)inp + b0 * hidden_size * seq_len,
+                           (half_t*)out + b0 * hidden_size);
+        if (int e = launch_status()) return e;
+    }
+    return 0;
 }
 
 }  // extern "C"

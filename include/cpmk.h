@@ -12,6 +12,14 @@
  *   - Launch geometry is private to the library (the reference computes grid/block in
  *     its Python wrappers; here the Python wrappers only forward arguments).
  *   - fp16 is IEEE binary16; "b,n,m" tensors are row-major with m contiguous.
+ *   - Sizes: element counts and byte offsets are 64-bit throughout (tensors beyond 2^31
+ *     elements work), and batches of any int32 size are split over launches where a kernel
+ *     indexes the batch with a grid dimension.  CPMK_ETOOBIG remains for: a matrix dimension
+ *     beyond 4 194 240 (65535 tiles of 64) in the transposes, the embedding kernels and the
+ *     general GEMM kernels; k above 2^30 in the fp16 GEMM; more than 524 280 vectors in the
+ *     general fp16 broadcast GEMV; more than 2^31-1 rows in the elementwise and row-quantising
+ *     training kernels; position bias with more than 65535 heads, a query_len above 32752
+ *     (forward) or more than 8192 buckets (backward).
  *
  * Each declaration cites the reference interface it replaces as
  * <python wrapper file:line> / <CUDA kernel file:line> relative to the reference tree.

@@ -161,3 +161,44 @@ def test_gemm_int8_operand_beyond_2_gib_and_output_beyond_2_31(gpu):
         acc = _rows_ref(to_np(P[0, rows]), Qn, slice(None))[None]
         ref = oracle.gemm_scale(acc, to_np(srow[rows]), to_np(scol), True, True)
         assert_bits_equal(to_np(o16[:, rows]), ref, "fused rows %d.." % r0)
+
+
+def test_batches_beyond_the_grid_limit(gpu):
+    """70000 batch entries: more than a grid's y or z dimension holds (65535).  The reference indexes
+    the batch with the grid's x dimension and has no such limit (kernels/softmax.py:20,
+    kernels/transpose.py:17), so the launchers here split such batches over several launches; entry
+    65535 onwards must come out like the rest.  Small odd shapes, which take the general kernels."""
+    import test_parity_gpu as tp
+    import test_training_gpu as tt
+    B = 70000
+    _name("batch of", B)
+    tp.test_softmax_forward(gpu, (B, 5, 3))
+    tp.test_layernorm_forward(gpu, (B, 5, 3), True)
+    tp.test_calc_scale_and_round_transpose(gpu, (B, 5, 6))
+    tp.test_embedding_and_kv_copy(gpu, (B, 4, 3))
+    tt.test_softmax_backward(gpu, (B, 6, 2))
+    tt.test_layernorm_training_kernels(gpu, (B, 6, 2))
+    tt.test_gemm_backward_quantisers(gpu, (B, 6, 2), False)
+    tt.test_transpose(gpu, (B, 3, 5))
+    tt.test_transpose_i8(gpu, (B, 3, 5))
+    rng = np.random.default_rng(17)
+    for aT in (False, True):
+        for bT in (False, True):
+            tp._gemm_case(gpu, 4, 8, 4, B, B, aT, bT, rng)
+    tp._gemm_case(gpu, 4, 8, 4, 1, B, True, False, rng)
+    tp._gemm_case(gpu, 4, 8, 4, B, 1, True, False, rng)
+    # fp16 product and the per-batch transposed GEMV
+    A = rng.standard_normal((B, 2, 4)).astype(np.float16)          # (batch, k, m), aT = False
+    Bm = rng.standard_normal((B, 6, 2)).astype(np.float16)         # (batch, n, k), bT = False
+    Ad, Bd = torch.from_numpy(A).to(gpu), torch.from_numpy(Bm).to(gpu)
+    out = torch.full((B, 6, 4), 77.0, dtype=torch.half, device=gpu)
+    ck.gemm_fp16(4, 2, 6, B, B, False, False, Ad.data_ptr(), Bd.data_ptr(), out.data_ptr(), stream())
+    ref = np.einsum("bnk,bkm->bnm", Bm.astype(np.float64), A.astype(np.float64)).astype(np.float16)
+    assert_close_fp16(to_np(out), ref, rtol=1e-3, atol=1e-3, what="gemm_fp16, batch %d" % B)
+    mat = rng.standard_normal((B, 6, 8)).astype(np.float16)        # (batch, dim_in, dim_out)
+    vec = rng.standard_normal((B, 6)).astype(np.float16)
+    md, vd = torch.from_numpy(mat).to(gpu), torch.from_numpy(vec).to(gpu)
+    o2 = torch.full((B, 8), 77.0, dtype=torch.half, device=gpu)
+    ck.gemv_fp16_transpose(B, 8, 6, md.data_ptr(), vd.data_ptr(), o2.data_ptr(), stream())
+    ref = np.einsum("bko,bk->bo", mat.astype(np.float64), vec.astype(np.float64)).astype(np.float16)
+    assert_close_fp16(to_np(o2), ref, rtol=1e-3, atol=1e-3, what="gemv_fp16_transpose, batch %d" % B)
