@@ -1,0 +1,104 @@
+"""Pointers that are only 4-byte aligned: torch hands out 256-byte aligned tensors, but a caller's
+view into a larger buffer need not be, and the reference asks for nothing beyond the alignment of
+its half2 / char4 accesses.  Every 16-byte fast path must step aside for such pointers: each
+function is run on aligned tensors and again with every operand moved 4 bytes off, and the two
+results must agree (to the bit for the exact kernels)."""
+import numpy as np
+import pytest
+import torch
+
+import cpm_kernels_amd.kernels as ck
+from util import stream, to_np, assert_bits_equal, assert_close_fp16
+
+pytestmark = pytest.mark.gpu
+
+
+def _name(*a):
+    print("case", *a, flush=True)
+
+
+def shifted(t):
+    """The same values at an address 4 bytes past a 256-byte boundary."""
+    e = 4 // t.element_size()
+    buf = torch.empty(t.numel() + 64, dtype=t.dtype, device=t.device)
+    v = buf[e:e + t.numel()].view(t.shape)
+    v.copy_(t)
+    assert v.data_ptr() % 16 == 4
+    return v
+
+
+def both(fn, inputs, out_shape, out_dtype, gpu, exact=True, what=""):
+    """fn(*pointers of inputs, pointer of out) on aligned and on shifted operands."""
+    out_a = torch.zeros(out_shape, dtype=out_dtype, device=gpu)
+    fn(*[t.data_ptr() for t in inputs], out_a.data_ptr())
+    sh = [shifted(t) for t in inputs]
+    out_s = shifted(torch.zeros(out_shape, dtype=out_dtype, device=gpu))
+    fn(*[t.data_ptr() for t in sh], out_s.data_ptr())
+    if exact:
+        assert_bits_equal(to_np(out_s), to_np(out_a), what + ": shifted == aligned")
+    else:
+        assert_close_fp16(to_np(out_s), to_np(out_a).astype(np.float64), rtol=1e-3, atol=2e-4, what=what + ": shifted vs aligned")
+    return out_a
+
+
+def test_quantised_gemm_path_unaligned(gpu):
+    _name("quantise / gemm / dequant, 4-byte aligned pointers")
+    g = torch.Generator().manual_seed(31)
+    n, k, m = 136, 256, 264
+    X = torch.randn(1, n, k, generator=g).half().to(gpu)
+    W = (torch.randn(1, m, k, generator=g) * 0.05).half().to(gpu)
+    s = stream()
+    sx = both(lambda x, o: ck.gemm_calc_scale(1, n, k, x, o, s), [X], (1, n), torch.half, gpu, what="calc_scale")
+    sw = both(lambda x, o: ck.gemm_calc_scale(1, m, k, x, o, s), [W], (1, m), torch.half, gpu, what="calc_scale W")
+    qx = both(lambda x, sc, o: ck.gemm_round(1, n, k, x, sc, o, s), [X, sx], (1, n, k), torch.int8, gpu, what="round")
+    qw = both(lambda x, sc, o: ck.gemm_round(1, m, k, x, sc, o, s), [W, sw], (1, m, k), torch.int8, gpu, what="round W")
+    both(lambda x, o: ck.gemm_calc_scale_transpose(1, n, k, x, o, s), [X], (1, k), torch.half, gpu, what="calc_scale_transpose")
+    for aT, bT, A, B in ((True, False, qw, qx), (False, False, qw.transpose(1, 2).contiguous(), qx),
+                         (True, True, qw, qx.transpose(1, 2).contiguous())):
+        acc = both(lambda a, b, o: ck.gemm_int8(m, k, n, 1, 1, aT, bT, a, b, o, s), [A, B], (1, n, m), torch.int32, gpu,
+                   what="gemm_int8 aT=%d bT=%d" % (aT, bT))
+        both(lambda a, b, r, c, o: ck.gemm_int8_scale(m, k, n, 1, 1, aT, bT, a, b, r, c, True, True, o, s), [A, B, sx[0], sw[0]],
+             (1, n, m), torch.half, gpu, what="gemm_int8_scale aT=%d bT=%d" % (aT, bT))
+    both(lambda a, r, c, o: ck.gemm_scale(1, n, m, a, r, c, o, True, True, s), [acc, sx[0], sw[0]], (1, n, m), torch.half, gpu, what="gemm_scale")
+    Xh = X[0, :, :64].contiguous().view(1, n, 64)
+    Wh = W[0, :, :64].contiguous().view(1, m, 64)
+    both(lambda a, b, o: ck.gemm_fp16(m, 64, n, 1, 1, True, False, a, b, o, s), [Wh, Xh], (1, n, m), torch.half, gpu, exact=False, what="gemm_fp16")
+    # GEMV: 32 vectors against the quantised weights
+    vq, vs = qx[0, :32].contiguous(), sx[0, :32].contiguous()
+    both(lambda sm, mt, sv, v, o: ck.gemv_broadcast_mat_int8(32, m, k, sm, mt, sv, v, o, s), [sw[0], qw[0], vs, vq], (32, m), torch.half, gpu,
+         what="gemv_broadcast_mat_int8")
+    both(lambda mt, v, o: ck.gemv_broadcast_mat_fp16(32, m, k, mt, v, o, s), [W[0], X[0, :32].contiguous()], (32, m), torch.half, gpu,
+         exact=False, what="gemv_broadcast_mat_fp16")
+
+
+@pytest.mark.parametrize("shape", [(3, 512, 128), (2, 2048, 64), (4, 100, 72)])
+def test_dim1_and_elementwise_unaligned(gpu, shape):
+    _name("layernorm / softmax / elementwise, 4-byte aligned pointers", shape)
+    b, n, m = shape
+    g = torch.Generator().manual_seed(32 + n)
+    x = (torch.randn(b, n, m, generator=g) * 2).half().to(gpu)
+    y = torch.randn(b, n, m, generator=g).half().to(gpu)
+    al = (1 + 0.1 * torch.randn(n, generator=g)).half().to(gpu)
+    be = (0.1 * torch.randn(n, generator=g)).half().to(gpu)
+    mk = (torch.rand(b, m, generator=g) > 0.3).to(torch.int8).to(gpu)
+    s = stream()
+    both(lambda i, o: ck.layernorm_forward(b, n, m, i, o, 1e-5, True, s), [x], shape, torch.half, gpu, exact=False, what="layernorm")
+    both(lambda i, o: ck.softmax_forward(b, n, m, i, o, s), [x], shape, torch.half, gpu, exact=False, what="softmax")
+    # (the 8-wide and the element-wise code of gelu may round the last bit differently: a 1e-3 kernel)
+    both(lambda i, o: ck.gelu_forward(b, n * m, i, o, s), [x], shape, torch.half, gpu, exact=False, what="gelu")
+    both(lambda i, j, o: ck.arith_element_add(b, n * m, i, j, o, s), [x, y], shape, torch.half, gpu, what="element_add")
+    both(lambda i, a, c, o: ck.arith_ln_mul_add(b, n, m, i, a, c, o, s), [x, al, be], shape, torch.half, gpu, what="ln_mul_add")
+    both(lambda i, k_, o: ck.mask(b, n, m, i, k_, float("-inf"), o, s), [x, mk], shape, torch.half, gpu, what="mask")
+    both(lambda i, o: ck.transpose(b, n, m, i, o, s), [x], (b, m, n), torch.half, gpu, what="transpose")
+    p = torch.softmax(x.float(), dim=1).half()
+    both(lambda o_, g_, o: ck.softmax_backward(b, n, m, o_, g_, o, s), [p, y], shape, torch.half, gpu, exact=False, what="softmax_backward")
+    # one-pass quantisers: scale and int8 through one call each
+    sc = both(lambda i, o: ck.gemm_calc_scale_transpose(b, n, m, i, o, s), [x], (b, m), torch.half, gpu, what="calc_scale_transpose")
+    both(lambda i, c, o: ck.gemm_round_transpose(b, n, m, i, c, o, s), [x, sc], shape, torch.int8, gpu, what="round_transpose")
+    for tr in (False, True):
+        q_a = torch.zeros((b, m, n) if tr else shape, dtype=torch.int8, device=gpu); s_a = torch.zeros((b, m), dtype=torch.half, device=gpu)
+        ck.gemm_quantize_cols(b, n, m, x.data_ptr(), s_a.data_ptr(), q_a.data_ptr(), tr, s)
+        xs, q_s, s_s = shifted(x), shifted(torch.zeros_like(q_a)), shifted(torch.zeros_like(s_a))
+        ck.gemm_quantize_cols(b, n, m, xs.data_ptr(), s_s.data_ptr(), q_s.data_ptr(), tr, s)
+        assert_bits_equal(to_np(s_s), to_np(s_a), "quantize_cols scales (transposed=%s)" % tr)
+        assert_bits_equal(to_np(q_s), to_np(q_a), "quantize_cols int8 (transposed=%s)" % tr)
