@@ -1,4 +1,5 @@
-"""Pointers that are only 4-byte aligned: torch hands out 256-byte aligned tensors, but a caller's
+"""Two properties beside parity.  Repeatability: results must not depend on timing (last test).
+Pointers that are only 4-byte aligned: torch hands out 256-byte aligned tensors, but a caller's
 view into a larger buffer need not be, and the reference asks for nothing beyond the alignment of
 its half2 / char4 accesses.  Every 16-byte fast path must step aside for such pointers: each
 function is run on aligned tensors and again with every operand moved 4 bytes off, and the two
@@ -102,3 +103,48 @@ def test_dim1_and_elementwise_unaligned(gpu, shape):
         ck.gemm_quantize_cols(b, n, m, xs.data_ptr(), s_s.data_ptr(), q_s.data_ptr(), tr, s)
         assert_bits_equal(to_np(s_s), to_np(s_a), "quantize_cols scales (transposed=%s)" % tr)
         assert_bits_equal(to_np(q_s), to_np(q_a), "quantize_cols int8 (transposed=%s)" % tr)
+
+
+def test_results_do_not_depend_on_timing(gpu):
+    """The team kernels add their partial sums in part order and the many-tile softmax hands tiles
+    out dynamically: neither may show in the results.  Each kernel runs five times on the same
+    input, with other work queued in between, and every run must reproduce the first bit for bit."""
+    _name("repeatability")
+    g = torch.Generator().manual_seed(41)
+    s = stream()
+    x = (torch.randn(8, 4096, 512, generator=g) * 2).half().to(gpu)            # teams of 4 (layernorm), 8 (column quantiser)
+    sm = (torch.randn(64, 1024, 1024, generator=g) * 3).half().to(gpu)         # 1024 tiles on 256 persistent workgroups
+    W = torch.randint(-127, 128, (10240, 4096), generator=g, dtype=torch.int8).to(gpu)
+    v = torch.randint(-127, 128, (32, 4096), generator=g, dtype=torch.int8).to(gpu)
+    sW = (torch.rand(10240, generator=g) * 0.01 + 1e-3).half().to(gpu); sv = (torch.rand(32, generator=g) * 0.05 + 1e-3).half().to(gpu)
+    Wh = torch.randn(2048, 4096, generator=g).half().to(gpu); vh = torch.randn(32, 4096, generator=g).half().to(gpu)
+    noise = torch.empty(64 << 20, dtype=torch.half, device=gpu)
+
+    def runs(fn, outs):
+        first = None
+        for i in range(5):
+            for o in outs:
+                o.fill_(0)
+            if i % 2:
+                noise.normal_()          # other kernels ahead of it in the queue
+            fn()
+            got = [to_np(o).copy() for o in outs]
+            if first is None:
+                first = got
+            else:
+                for a, b in zip(got, first):
+                    assert_bits_equal(a, b, "run %d differs from run 0" % i)
+
+    y = torch.empty_like(x)
+    runs(lambda: ck.layernorm_forward(8, 4096, 512, x.data_ptr(), y.data_ptr(), 1e-5, True, s), [y])
+    sc = torch.empty((8, 512), dtype=torch.half, device=gpu); q = torch.empty((8, 512, 4096), dtype=torch.int8, device=gpu)
+    runs(lambda: ck.gemm_quantize_cols(8, 4096, 512, x.data_ptr(), sc.data_ptr(), q.data_ptr(), True, s), [sc, q])
+    so = torch.empty_like(sm)
+    runs(lambda: ck.softmax_forward(64, 1024, 1024, sm.data_ptr(), so.data_ptr(), s), [so])
+    tall = sm.view(8, 8192, 1024); to = torch.empty_like(tall)
+    runs(lambda: ck.softmax_forward(8, 8192, 1024, tall.data_ptr(), to.data_ptr(), s), [to])
+    runs(lambda: ck.softmax_backward(8, 8192, 1024, tall.data_ptr(), tall.data_ptr(), to.data_ptr(), s), [to])
+    o = torch.empty((32, 10240), dtype=torch.half, device=gpu)
+    runs(lambda: ck.gemv_broadcast_mat_int8(32, 10240, 4096, sW.data_ptr(), W.data_ptr(), sv.data_ptr(), v.data_ptr(), o.data_ptr(), s), [o])
+    o2 = torch.empty((32, 2048), dtype=torch.half, device=gpu)
+    runs(lambda: ck.gemv_broadcast_mat_fp16(32, 2048, 4096, Wh.data_ptr(), vh.data_ptr(), o2.data_ptr(), s), [o2])
