@@ -24,6 +24,7 @@ __global__ __launch_bounds__(NT) void k_layernorm_tile(int32_t n, int32_t m, int
                                                        int rd_mean) {
     using T = ColTile<NT, LPR, R>;
     __shared__ float lds[(T::NW + 1) * T::COLS * 2];
+    __shared__ half_t coef[2][T::ROWS];   // alpha and beta of the tile's rows
     const uint32_t t = xcd_remap(blockIdx.x, gridDim.x);
     const uint32_t b = t / tiles_per_batch, ct = t - b * tiles_per_batch;
     const int32_t col0 = ct * T::COLS + (threadIdx.x % LPR) * 8;
@@ -31,6 +32,15 @@ __global__ __launch_bounds__(NT) void k_layernorm_tile(int32_t n, int32_t m, int
 
     half8_t v[R];
     coltile_load<NT, LPR, R>(v, mat + boff, n, m, col0, (half_t)0.0f);
+    // the affine coefficients of the tile's rows, contiguous loads requested with the tile and
+    // parked in LDS until the output pass (the barriers of the reduction order write and reads)
+    if (alpha != nullptr) {
+        for (int32_t r = threadIdx.x; r < T::ROWS; r += NT) {
+            const int32_t row = min(r, n - 1);
+            coef[0][r] = alpha[row];
+            coef[1][r] = beta != nullptr ? beta[row] : (half_t)0.0f;
+        }
+    }
 
     float s[16];
 #pragma unroll
@@ -63,10 +73,7 @@ __global__ __launch_bounds__(NT) void k_layernorm_tile(int32_t n, int32_t m, int
         half8_t y;
 #pragma unroll
         for (int e = 0; e < 8; ++e) y[e] = round_f16(((float)v[p][e] - mean[e]) * rstd[e]);
-        if (alpha != nullptr) {
-            const int32_t row = p * T::RPP + rg;
-            if (row < n) y = affine8(y, alpha[row], beta ? beta[row] : (half_t)0.0f, beta != nullptr);
-        }
+        if (alpha != nullptr) y = affine8(y, coef[0][p * T::RPP + rg], coef[1][p * T::RPP + rg], beta != nullptr);
         v[p] = y;
     }
     coltile_store<NT, LPR, R>(v, out + boff, n, m, col0);
@@ -89,7 +96,9 @@ __global__ __launch_bounds__(NT) void k_layernorm_team(int32_t n, int32_t m, int
     static_assert(T::COLS * 2 == kXchVals, "slot layout");
     __shared__ float lds[(T::NW + 1) * T::COLS * 2];
     __shared__ float tot[kXchVals];
+    __shared__ half_t coef[2][NT];        // alpha and beta of this workgroup's rows (T::ROWS == NT)
     __shared__ int failed;
+    static_assert(T::ROWS == NT, "one affine coefficient pair per thread");
     const int tid = threadIdx.x;
     const uint32_t part = blockIdx.x % parts, team = blockIdx.x / parts;
     const uint32_t b = team / tiles_per_batch, ct = team - b * tiles_per_batch;
@@ -101,14 +110,14 @@ __global__ __launch_bounds__(NT) void k_layernorm_team(int32_t n, int32_t m, int
 
     half8_t v[R];
     coltile_load<NT, LPR, R>(v, mat + boff, own_n, m, col0, (half_t)0.0f);
-    // the affine coefficients of this lane's rows, requested now so that they arrive during the exchange
+    // The affine coefficients of the workgroup's rows: one pair per thread, contiguous, parked in
+    // LDS until the output pass (a thread's own rows are RPP apart; fetching them lane by lane
+    // took 2 x R two-byte loads per thread, as many load instructions again as the tile itself).
     const int rg = tid / LPR;
-    half_t al[R], be[R];
-#pragma unroll
-    for (int p = 0; p < R; ++p) {
-        const int32_t row = min(own0 + p * T::RPP + rg, n - 1);
-        al[p] = alpha != nullptr ? alpha[row] : (half_t)1.0f;
-        be[p] = beta != nullptr ? beta[row] : (half_t)0.0f;
+    if (alpha != nullptr) {
+        const int32_t row = min(own0 + tid, n - 1);
+        coef[0][tid] = alpha[row];
+        coef[1][tid] = beta != nullptr ? beta[row] : (half_t)0.0f;
     }
     float s[16];
 #pragma unroll
@@ -161,7 +170,7 @@ __global__ __launch_bounds__(NT) void k_layernorm_team(int32_t n, int32_t m, int
         half8_t y;
 #pragma unroll
         for (int e = 0; e < 8; ++e) y[e] = round_f16(((float)v[p][e] - mean[e]) * rstd[e]);
-        if (alpha != nullptr) y = affine8(y, al[p], be[p], beta != nullptr);
+        if (alpha != nullptr) y = affine8(y, coef[0][p * T::RPP + rg], coef[1][p * T::RPP + rg], beta != nullptr);
         v[p] = y;
     }
     coltile_store<NT, LPR, R>(v, out + boff, own_n, m, col0);
