@@ -35,7 +35,7 @@ M, K, N = 4096, 4096, 10240  # north-star GEMM
 # 256 MiB device copy of `--only calib` (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000 on MI355X).
 # MFMA pipe busy cycles / kernel cycles of the fused GEMM kernel from SQ_VALU_MFMA_BUSY_CYCLES and
 # SQ_BUSY_CYCLES (same offline procedure; profiles/gemm_mfma_utilisation.txt).
-MFMA_BUSY_FRAC = 0.670
+MFMA_BUSY_FRAC = 0.669
 
 TRAFFIC_BYTES = {
     "gemm_fused": 353.6e6,     # 269.8 MB fetched (operand tiles re-read across the 8 L2s) + 83.9 MB written
