@@ -202,3 +202,56 @@ def test_batches_beyond_the_grid_limit(gpu):
     ck.gemv_fp16_transpose(B, 8, 6, md.data_ptr(), vd.data_ptr(), o2.data_ptr(), stream())
     ref = np.einsum("bko,bk->bo", mat.astype(np.float64), vec.astype(np.float64)).astype(np.float16)
     assert_close_fp16(to_np(o2), ref, rtol=1e-3, atol=1e-3, what="gemv_fp16_transpose, batch %d" % B)
+
+
+def test_training_and_helper_kernels_beyond_2_31_elements(gpu):
+    """The remaining kernels with a per-batch layout, on 129 x (8192, 2048): batch 128 starts at
+    element 2^31.  Batches 0, 127 and 128 against the CPU restatements."""
+    import oracle.training as ot
+    b, n, m = 129, 8192, 2048
+    _name("training / helper kernels", (b, n, m))
+    s = stream()
+    x = _randn_half((b, n, m), 21, gpu, 1.5)
+    gsrc = _randn_half((b, n, m), 22, gpu, 1.0)
+    out = torch.full((b, n, m), 77.0, dtype=torch.half, device=gpu)
+    picks = (0, 127, 128)
+    # mask and the layernorm affine
+    g = torch.Generator(device=gpu).manual_seed(23)
+    mk = (torch.rand((b, m), generator=g, device=gpu) > 0.3).to(torch.int8)
+    ck.mask(b, n, m, x.data_ptr(), mk.data_ptr(), float("-inf"), out.data_ptr(), s)
+    for i in picks:
+        assert_bits_equal(to_np(out[i:i + 1]), oracle.mask(to_np(x[i:i + 1]), to_np(mk[i:i + 1]), float("-inf")), "mask batch %d" % i)
+    al = (1 + 0.1 * torch.randn(n, generator=g, device=gpu)).half(); be = (0.1 * torch.randn(n, generator=g, device=gpu)).half()
+    out.fill_(77.0)
+    ck.arith_ln_mul_add(b, n, m, x.data_ptr(), al.data_ptr(), be.data_ptr(), out.data_ptr(), s)
+    for i in picks:
+        assert_bits_equal(to_np(out[i:i + 1]), oracle.arith_ln_mul_add(to_np(x[i:i + 1]), to_np(al), to_np(be)), "ln_mul_add batch %d" % i)
+    # transposes
+    outT = torch.full((b, m, n), 77.0, dtype=torch.half, device=gpu)
+    ck.transpose(b, n, m, x.data_ptr(), outT.data_ptr(), s)
+    for i in picks:
+        assert_bits_equal(to_np(outT[i]), np.ascontiguousarray(to_np(x[i]).T), "transpose batch %d" % i)
+    del outT
+    q = (x.view(torch.int16) & 0xff).to(torch.int8)          # some bytes
+    qT = torch.full((b, m, n), 99, dtype=torch.int8, device=gpu)
+    ck.transpose_i8(b, n, m, q.data_ptr(), qT.data_ptr(), s)
+    for i in picks:
+        assert_bits_equal(to_np(qT[i]), np.ascontiguousarray(to_np(q[i]).T), "transpose_i8 batch %d" % i)
+    del q, qT
+    # dim-1 reductions of the backward pass (teams of 16 workgroups per 64 columns)
+    out.fill_(77.0)
+    ck.softmax_forward(b, n, m, x.data_ptr(), out.data_ptr(), s)
+    grad = torch.full((b, n, m), 77.0, dtype=torch.half, device=gpu)
+    ck.softmax_backward(b, n, m, out.data_ptr(), gsrc.data_ptr(), grad.data_ptr(), s)
+    for i in picks:
+        assert_close_fp16(to_np(grad[i:i + 1]), ot.softmax_backward(to_np(out[i:i + 1]), to_np(gsrc[i:i + 1])), rtol=2e-3, atol=1e-5, what="softmax_backward batch %d" % i)
+    mean = torch.empty((b, m), dtype=torch.half, device=gpu); var = torch.empty((b, m), dtype=torch.half, device=gpu)
+    ck.layernorm_forward_mv(b, n, m, x.data_ptr(), out.data_ptr(), mean.data_ptr(), var.data_ptr(), 1e-5, s)
+    grad.fill_(77.0)
+    ck.layernorm_backward_mv(b, n, m, x.data_ptr(), gsrc.data_ptr(), mean.data_ptr(), var.data_ptr(), grad.data_ptr(), s)
+    for i in picks:
+        o_ref, m_ref, v_ref = ot.layernorm_forward_mv(to_np(x[i:i + 1]), 1e-5)
+        assert_close_fp16(to_np(out[i:i + 1]), o_ref, rtol=1e-3, atol=1e-3, what="forward_mv batch %d" % i)
+        assert_close_fp16(to_np(mean[i:i + 1]), m_ref, rtol=1e-3, atol=1e-4, what="forward_mv mean, batch %d" % i)
+        assert_close_fp16(to_np(grad[i:i + 1]), ot.layernorm_backward_mv(to_np(x[i:i + 1]), to_np(gsrc[i:i + 1]), to_np(mean[i:i + 1]), to_np(var[i:i + 1])),
+                          rtol=2e-3, atol=1e-3, what="backward_mv batch %d" % i)
