@@ -99,7 +99,23 @@ def test_quantisers_beyond_2_31_elements(gpu):
         s_ref = oracle.gemm_calc_scale(xs)
         assert_bits_equal(to_np(sc[:, r0:r0 + 16]), s_ref, "row scales at %d" % r0)
         assert_bits_equal(to_np(q[:, r0:r0 + 16]), oracle.gemm_round(xs, s_ref), "row int8 at %d" % r0)
-    del q, sc
+    # the two-launch form of the same quantisation, whole tensors compared on the device
+    sc2 = torch.full((b, n), 77.0, dtype=torch.half, device=gpu)
+    q2 = torch.full((b, n, m), 99, dtype=torch.int8, device=gpu)
+    ck.gemm_calc_scale(b, n, m, x.data_ptr(), sc2.data_ptr(), stream())
+    ck.gemm_round(b, n, m, x.data_ptr(), sc2.data_ptr(), q2.data_ptr(), stream())
+    assert torch.equal(sc2, sc) and torch.equal(q2, q), "calc_scale + round == quantize"
+    del q, sc, q2
+    # dequantisation of an int32 tensor of the same shape
+    g = torch.Generator(device=gpu).manual_seed(18)
+    acc = torch.randint(-3000000, 3000000, (b, n, m), generator=g, dtype=torch.int32, device=gpu)
+    sy = (torch.rand(m, generator=g, device=gpu) * 0.001 + 1e-5).half()
+    o16 = torch.full((b, n, m), 77.0, dtype=torch.half, device=gpu)
+    ck.gemm_scale(b, n, m, acc.data_ptr(), sc2.data_ptr(), sy.data_ptr(), o16.data_ptr(), True, True, stream())
+    for r0 in (0, 2 ** 20 - 8, n - 16):
+        ref = oracle.gemm_scale(to_np(acc[:, r0:r0 + 16]), to_np(sc2[0, r0:r0 + 16]), to_np(sy), True, True)
+        assert_bits_equal(to_np(o16[:, r0:r0 + 16]), ref, "gemm_scale rows %d.." % r0)
+    del acc, o16, sc2
     # per column, written transposed: batch 128 of 129 x (8192, 2048) starts at element 2^31
     del x
     b, n, m = 129, 8192, 2048
