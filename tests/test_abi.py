@@ -173,3 +173,21 @@ def test_single_hip_runtime_whichever_is_imported_first():
     out = subprocess.run([sys.executable, "-c", code], env=dict(os.environ, PYTHONPATH=ROOT), stdout=subprocess.PIPE,
                          stderr=subprocess.STDOUT, text=True)
     assert "HIPLIBS 1 " in out.stdout, out.stdout
+
+
+def test_torch_surface_through_the_alias_package():
+    """`import cpm_kernels.torch as ct` must give every operator name of the reference's
+    torch/__init__.py:1-14 -- including gelu, mask, softmax and transpose, which are also the
+    names of submodules (a star import that listed the modules instead would hide the functions)."""
+    import types
+    import cpm_kernels.torch as ct
+    names = """OpEmbedding Embedding EmbeddingTH gelu geluTH gelu_inplace bmm mask mask_inplace maskTH
+        ln_div ln_div_inplace ln_divTH ln_mul_add ln_mul_add_inplace ln_mul_addTH ln_mul ln_mul_inplace ln_mulTH
+        ln_sub_div ln_sub_divTH ln_sub_div_inplace element_add element_add_inplace element_addTH
+        batched_add batched_add_inplace batched_addTH element_mul element_mul_inplace element_mulTH
+        ln_add ln_add_inplace ln_addTH global_scale global_scale_inplace global_scaleTH
+        LayerNorm LayerNormTH normalize_inplace normalizeTH PositionEmbedding PositionEmbeddingTH
+        softmax softmaxTH softmax_inplace transpose transposeTH has_nan_inf""".split()
+    for n in names:
+        obj = getattr(ct, n, None)
+        assert obj is not None and not isinstance(obj, types.ModuleType) and callable(obj), n
