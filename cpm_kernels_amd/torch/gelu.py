@@ -33,6 +33,9 @@ def geluTH(x: torch.Tensor) -> torch.Tensor:
     return 0.5 * x * (1.0 + torch.tanh(0.7978845608028654 * x * (1.0 + 0.044715 * x * x)))
 
 
+gelu_impl = geluTH      # the reference's name for the same formulation (torch/gelu.py:42-45)
+
+
 def gelu_inplace(x: torch.Tensor) -> None:
     check_half(x)
     gelu_inplace_forward(x.size(0), x.stride(0), x.data_ptr(), cur_stream())

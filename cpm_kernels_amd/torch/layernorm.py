@@ -65,6 +65,33 @@ class OpLayerNorm(torch.autograd.Function):
         return grad, None, grad_weight, grad_bias, None
 
 
+class OpLayerNormMean(OpLayerNorm):
+    """The reference's name and argument list (x, eps, weight, bias) for the mean-subtracting
+    norm (torch/layernorm.py:7-86)."""
+
+    @staticmethod
+    def forward(ctx, x: torch.Tensor, eps: float, weight: torch.Tensor, bias: torch.Tensor):
+        assert bias is not None
+        return OpLayerNorm.forward(ctx, x, eps, weight, bias)
+
+    @staticmethod
+    def backward(ctx, grad_output: torch.Tensor):
+        return OpLayerNorm.backward(ctx, grad_output)[:4]
+
+
+class OpLayerNormNoMean(OpLayerNorm):
+    """The reference's name and argument list (x, eps, weight) for the RMS norm
+    (torch/layernorm.py:88-156)."""
+
+    @staticmethod
+    def forward(ctx, x: torch.Tensor, eps: float, weight: torch.Tensor):
+        return OpLayerNorm.forward(ctx, x, eps, weight, None)
+
+    @staticmethod
+    def backward(ctx, grad_output: torch.Tensor):
+        return OpLayerNorm.backward(ctx, grad_output)[:3]
+
+
 class LayerNorm(torch.nn.Module):
     """reference: torch/layernorm.py:158-172"""
 

@@ -191,3 +191,38 @@ def test_torch_surface_through_the_alias_package():
     for n in names:
         obj = getattr(ct, n, None)
         assert obj is not None and not isinstance(obj, types.ModuleType) and callable(obj), n
+
+
+def test_torch_submodules_through_the_alias_package():
+    """Every submodule of the reference's torch package imports under the drop-in name and is the
+    implementation's module object (not the function of the same name), and the classes a user
+    imports from them are there (torch/*.py of the reference)."""
+    import importlib
+    import types
+    wanted = {
+        "arith": ["OpGlobalScale", "OpElementAdd", "OpElementMul", "OpBatchedAdd", "OpLnMulAdd", "OpLnMul", "OpLnAdd",
+                  "ln_sub_div", "ln_div"],
+        "embedding": ["OpEmbedding", "Embedding", "EmbeddingTH"],
+        "gelu": ["OpGeLU", "gelu", "gelu_impl", "geluTH", "gelu_inplace"],
+        "gemm": ["calc_scale", "round_i8", "gemm_and_scale", "GEMMInt8", "gemm_pth_fp16", "GEMMFloat", "bmm"],
+        "layernorm": ["OpLayerNormMean", "OpLayerNormNoMean", "LayerNorm", "LayerNormTH", "normalize_inplace", "normalizeTH"],
+        "mask": ["OpMask", "mask", "mask_inplace", "maskTH"],
+        "position_embedding": ["OpPositionEmbedding", "PositionEmbedding", "PositionEmbeddingTH"],
+        "softmax": ["OpSoftmax", "softmax", "softmax_inplace", "softmaxTH"],
+        "transpose": ["OpTranspose", "transpose", "transposeTH"],
+        "utils": ["has_nan_inf"],
+    }
+    import cpm_kernels.torch as ct
+    for sub, names in wanted.items():
+        mod = importlib.import_module("cpm_kernels.torch." + sub)
+        assert isinstance(mod, types.ModuleType), sub
+        assert mod is importlib.import_module("cpm_kernels_amd.torch." + sub), sub
+        assert sys.modules["cpm_kernels.torch." + sub] is mod
+        for n in names:
+            assert callable(getattr(mod, n, None)), "%s.%s" % (sub, n)
+    from cpm_kernels.torch.softmax import OpSoftmax      # noqa: F401
+    import cpm_kernels.torch.embedding, cpm_kernels.torch.transpose, cpm_kernels.torch.utils      # noqa: F401,E401
+    # in the package namespace the function wins where both exist, as in the reference
+    for n in ("gelu", "mask", "softmax", "transpose"):
+        assert not isinstance(getattr(ct, n), types.ModuleType), n
+    assert isinstance(ct.utils, types.ModuleType) and isinstance(ct.gemm, types.ModuleType)
