@@ -17,9 +17,10 @@ namespace cpmk {
 template <int NT>
 __global__ __launch_bounds__(NT) void k_col_quantize_team(int32_t n, int32_t m, int32_t tiles_per_batch, int32_t parts,
                                                           const half_t* __restrict__ mat, half_t* __restrict__ scale,
-                                                          int8_t* __restrict__ out, int transposed, uint64_t* xch,
-                                                          uint32_t tag) {
+                                                          int8_t* __restrict__ out, int transposed, XchLaunch xl) {
     constexpr int LPR = 8, R = 8, COLS = 64, ROWS = NT / LPR * R;
+    uint64_t* const xch = xl.region;
+    const uint32_t tag = xl.tag;
     __shared__ float lds[(NT / 64 + 1) * COLS];
     __shared__ float tot[COLS];
     __shared__ __attribute__((aligned(16))) int8_t tbuf[COLS * ROWS];       // the transposed int8 tile on its way out
@@ -61,6 +62,7 @@ __global__ __launch_bounds__(NT) void k_col_quantize_team(int32_t n, int32_t m, 
                 for (int j = 0; j < 8; ++j) M = fmaxf(M, x[j]);       // maxima are >= 0: absent parts (zeros) do not matter
             }
             tot[tid] = ok ? M : __builtin_nanf("");
+            if (!ok) xch_flag(xl.status, kXchStatusTimeout);
         }
         __syncthreads();
 #pragma unroll
@@ -135,7 +137,7 @@ __global__ __launch_bounds__(NT) void k_col_quantize_team(int32_t n, int32_t m, 
             }
         }
     }
-    if (parts > 1 && tid < 64) xch_retire(xch, team, parts);
+    if (parts > 1 && tid < 64) xch_retire(xl, team, parts);
 }
 
 // Any shape: rounding with per-column scales into the transposed layout, one element per thread.
@@ -180,15 +182,17 @@ int cpmk_gemm_quantize_cols(int32_t batch, int32_t n, int32_t m, const void* mat
         const int64_t per_launch = parts > 1 ? kXchSlots / (tiles * parts) : ((1ll << 31) - 1) / (tiles * parts);
         for (int64_t b0 = 0; b0 < batch; b0 += per_launch) {
             const int64_t nb = batch - b0 < per_launch ? batch - b0 : per_launch;
-            XchLaunch xl = {nullptr, 0};
+            XchLaunch xl = {nullptr, nullptr, nullptr, 0, -1};
             if (parts > 1) {
-                const int rc = xch_begin(&xl);
+                const int rc = xch_begin(&xl, tiles * nb * parts, st);
                 if (rc != 0) return rc;
             }
             hipLaunchKernelGGL((k_col_quantize_team<512>), dim3((unsigned)(tiles * nb * parts)), dim3(512), 0, st, n, m,
                                (int32_t)tiles, (int32_t)parts, (const half_t*)mat + b0 * n * m, (half_t*)scale + b0 * m,
-                               (int8_t*)out + b0 * n * m, out_transposed, xl.region, xl.tag);
-            if (int e = launch_status()) return e;
+                               (int8_t*)out + b0 * n * m, out_transposed, xl);
+            const int e = launch_status();
+            const int rc2 = xch_end(xl, st);
+            if (e != 0 || rc2 != 0) return e ? e : rc2;
         }
         return 0;
     }

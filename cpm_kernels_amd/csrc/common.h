@@ -3,6 +3,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <atomic>
 #include "../../include/cpmk.h"
 
 namespace cpmk {
@@ -162,17 +163,32 @@ __device__ __forceinline__ void wait_vmcnt() {
 // fp16 broadcast-matrix GEMV on the MFMA kernel of gemv_i8.hip (0, a HIP error code, or -1: shape not eligible)
 int gemv_f16_coalesced(int32_t batch, int32_t dim_out, int32_t dim_in, const void* mat, const void* vec, void* out, hipStream_t st);
 
-// Compute units of the current device (cached per device ordinal; 256 if the query fails).
+// Compute units of the current device (cached per device ordinal; 256 if the query fails).  The cache
+// is atomic: host threads that make their first call together each ask the runtime and store the
+// same value.
 inline int compute_units() {
-    static int cus[64] = {0};
+    static std::atomic<int> cus[64];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-    if (cus[dev] == 0) {
-        int n = 0;
+    int n = cus[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
         if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-        cus[dev] = n;
+        cus[dev].store(n, std::memory_order_relaxed);
     }
-    return cus[dev];
+    return n;
+}
+
+// Dynamic LDS above the default limit must be enabled per kernel and device.  `done` is the
+// kernel's array of 64 per-device flags (static storage, so zero at start); the attribute call is
+// idempotent, so host threads racing through their first launch at worst all make it.
+inline int enable_dynamic_lds(const void* kern, int bytes, std::atomic<bool>* done) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    if (done[dev].load(std::memory_order_acquire)) return 0;
+    const hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess) return (int)e;
+    done[dev].store(true, std::memory_order_release);
+    return 0;
 }
 
 }  // namespace cpmk

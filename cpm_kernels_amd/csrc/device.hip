@@ -13,6 +13,7 @@ const char* cpmk_error_string(int code) {
         case CPMK_EBADARG: return "cpmk: invalid argument (negative size, bad batch combination or null pointer)";
         case CPMK_EALIGN: return "cpmk: size violates a divisibility precondition of the reference kernel";
         case CPMK_ETOOBIG: return "cpmk: problem exceeds a size limit of this library";
+        case CPMK_ETIMEOUT: return "cpmk: a kernel gave up waiting for another workgroup of its launch; its output holds NaN (0 in int8 tensors)";
         default: return hipGetErrorString((hipError_t)code);
     }
 }

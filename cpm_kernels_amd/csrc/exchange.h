@@ -11,34 +11,57 @@
 // replayed with the same arguments (a captured graph) starts from a clean slate as well.
 //
 // The packets live in a fixed pool in device memory owned by the library (nothing is allocated
-// per call).  Consecutive launches rotate over kXchRegions regions of the pool, so launches that
-// overlap in time on different streams do not share packets unless more than kXchRegions of
-// them are in flight at once.  A launch may use at most kXchSlots (team, part) pairs.
+// per call): kXchPoolSlots slots of kXchVals packets, handed out as a ring.  A launch takes as
+// many slots as it has (team, part) pairs (at most kXchSlots), so the pool holds the slots of
+// many launches at once (128 tall layernorms of 8 x 4096 x 512); before a launch reuses slots that
+// an earlier launch was given, its stream waits for that launch's completion event
+// (xch_begin / xch_end), so launches on any number of streams never share live packets.  The
+// exception is a launch recorded during stream capture: a graph's replays cannot be tracked by
+// events, so a captured launch keeps the slots it was recorded with and the host only avoids
+// them until the ring comes round again.
 //
 // Progress: a workgroup only ever waits for workgroups of its own team, whose indices differ by
-// less than P <= kXchMaxParts; workgroups start in index order, so all members of the oldest
+// less than the team size; the dispatcher starts the workgroups of a launch in index order (an
+// observed property of the hardware queue, not a documented one), so all members of the oldest
 // unfinished team are resident and that team completes.  Should a packet nevertheless not arrive
-// within about a second the wait gives up and the caller writes NaN: a visible failure instead
-// of a hung GPU.
+// within about a second the wait gives up, the caller writes NaN (0 in an int8 output) and sets
+// the device's sticky status word, which cpmk_async_status() reports and clears: a visible
+// failure instead of a hung GPU.
 #pragma once
 #include "common.h"
 
 namespace cpmk {
 
-constexpr int kXchRegions = 4;
-constexpr int kXchSlots = 8192;      // (team, part) pairs per launch
-constexpr int kXchVals = 128;        // packets per slot: 64 columns x 2 statistics
+constexpr int kXchPoolSlots = 32768;  // slots in the pool (1 KB each)
+constexpr int kXchSlots = 8192;       // (team, part) pairs per launch
+constexpr int kXchVals = 128;         // packets per slot: 64 columns x 2 statistics
 constexpr int kXchMaxParts = 8;
+constexpr int kXchGranule = 64;       // slots are handed out in multiples of this
 
-constexpr size_t kXchRegionWords = (size_t)kXchSlots * kXchVals + kXchSlots;   // packets, then one counter per team
+constexpr uint32_t kXchStatusTimeout = 1u;   // bit of the status word: a packet did not arrive in time
 
+// What a team kernel needs of the pool; passed to the kernel by value.
 struct XchLaunch {
-    uint64_t* region;   // kXchRegionWords 8-byte words in device memory
-    uint32_t tag;       // never 0, differs from the tags of the launches that used this region before
+    uint64_t* region;     // this launch's slots: slot i at region + i * kXchVals
+    uint64_t* counters;   // one retire counter per team: counters[team]
+    uint32_t* status;     // the device's sticky status word
+    uint32_t tag;         // never 0, differs from the tags of the launches that used these slots before
+    int32_t first;        // host bookkeeping: first pool slot of the launch, -1 if it holds none
 };
 
-// Host: region and tag for the next launch on the current device.  Returns 0 or a HIP error code.
-int xch_begin(XchLaunch* out);
+// Host, before the launch: `slots` slots (and as many team counters) for a launch on stream `st` of the
+// current device; makes `st` wait for the launches that last held those slots.  0 or an error code.
+int xch_begin(XchLaunch* out, int64_t slots, hipStream_t st);
+// Host, after the launch: records the launch's completion on `st` so that a later holder of its slots
+// can wait for it.  0 or an error code.
+int xch_end(const XchLaunch& xl, hipStream_t st);
+// Host: reads and clears the current device's status word (0, kXchStatus* bits, or -1 - hipError on failure to read).
+int xch_take_status(uint32_t* bits);
+
+// A wait gave up: leave a mark that the host can see (cpmk_async_status).
+__device__ inline void xch_flag(uint32_t* status, uint32_t bit) {
+    __hip_atomic_fetch_or(status, bit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 __device__ inline void xch_post(uint64_t* slot, int idx, float v, uint32_t tag) {
     const uint64_t pkt = ((uint64_t)tag << 32) | (uint64_t)__builtin_bit_cast(uint32_t, v);
@@ -94,9 +117,9 @@ __device__ inline bool xch_gather(const uint64_t* team_slots, int parts, int q0,
 // To be called by the first wave of a workgroup once the whole workgroup has collected its
 // packets (i.e. after the barrier that follows the xch_wait calls): counts the team members that
 // are done and lets the last one clear the team's `parts` slots and the counter.
-__device__ inline void xch_retire(uint64_t* region, uint32_t team, int parts) {
-    uint64_t* counter = region + (size_t)kXchSlots * kXchVals + team;
-    uint64_t* team_slots = region + (size_t)team * parts * kXchVals;
+__device__ inline void xch_retire(const XchLaunch& xl, uint32_t team, int parts) {
+    uint64_t* counter = xl.counters + team;
+    uint64_t* team_slots = xl.region + (size_t)team * parts * kXchVals;
     const int lane = threadIdx.x & 63;
     uint64_t old = 0;
     if (lane == 0) old = __hip_atomic_fetch_add(counter, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

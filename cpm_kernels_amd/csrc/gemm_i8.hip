@@ -691,15 +691,9 @@ static int launch_kmajor(GemmArgs& a, int batch, hipStream_t st) {
     a.tiles_r = (int32_t)ceil_div(a.n, BR);
     a.tiles_c = (int32_t)ceil_div(a.m, BC);
     auto kern = k_gemm_kmajor<WAVES_R, WAVES_C, TR, TC, FUSED>;
-    static bool attr_set[64] = {false};   // per device; raising the dynamic LDS limit is idempotent
-    int dev = 0;
-    (void)hipGetDevice(&dev);
-    if (smem > 48 * 1024 && dev >= 0 && dev < 64 && !attr_set[dev]) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-        if (e != hipSuccess) return (int)e;
-        attr_set[dev] = true;
-    }
+    static std::atomic<bool> lds_enabled[64];
+    if (smem > 48 * 1024)
+        if (int e = enable_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_enabled)) return e;
     dim3 grid((unsigned)(a.tiles_r * a.tiles_c), 1, (unsigned)batch);
     hipLaunchKernelGGL(kern, grid, dim3(WAVES_R * WAVES_C * 64), smem, st, a);
     return launch_status();
@@ -720,15 +714,8 @@ static int launch_dma_kernel(const DmaArgs& da, unsigned grid, hipStream_t st) {
     constexpr int smem = NST * (BR + BC) * BKB + WR * WC * STRIP;      // operand ring + output strips
     static_assert(smem <= 160 * 1024, "LDS of one compute unit");
     auto kern = k_gemm_dma<WR, WC, TR, TC, BKB, EPI, HALVES, NST, LAY>;
-    static bool attr_set[64] = {false};       // dynamic LDS above 64 KB must be enabled per device
-    int dev = 0;
-    (void)hipGetDevice(&dev);
-    if (dev >= 0 && dev < 64 && !attr_set[dev]) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-        if (e != hipSuccess) return (int)e;
-        attr_set[dev] = true;
-    }
+    static std::atomic<bool> lds_enabled[64];
+    if (int e = enable_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_enabled)) return e;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(WR * WC * 64), smem, st, da);
     return launch_status();
 }

@@ -90,10 +90,12 @@ __global__ __launch_bounds__(NT) void k_layernorm_team(int32_t n, int32_t m, int
                                                        const half_t* mat, half_t* out,
                                                        const half_t* __restrict__ alpha,
                                                        const half_t* __restrict__ beta, float eps, int rd_mean,
-                                                       uint64_t* xch, uint32_t tag) {
+                                                       XchLaunch xl) {
     constexpr int LPR = 8;
     using T = ColTile<NT, LPR, R>;
     static_assert(T::COLS * 2 == kXchVals, "slot layout");
+    uint64_t* const xch = xl.region;
+    const uint32_t tag = xl.tag;
     __shared__ float lds[(T::NW + 1) * T::COLS * 2];
     __shared__ float tot[kXchVals];
     __shared__ half_t coef[2][NT];        // alpha and beta of this workgroup's rows (T::ROWS == NT)
@@ -145,7 +147,10 @@ __global__ __launch_bounds__(NT) void k_layernorm_team(int32_t n, int32_t m, int
             for (int j = 0; j < 4; ++j) acc += x[j];       // in part order; absent parts are zeros
         }
         tot[tid] = acc;
-        if (!ok) failed = 1;
+        if (!ok) {
+            failed = 1;
+            xch_flag(xl.status, kXchStatusTimeout);
+        }
     }
     __syncthreads();
     const int cg = tid % LPR;
@@ -174,7 +179,7 @@ __global__ __launch_bounds__(NT) void k_layernorm_team(int32_t n, int32_t m, int
         v[p] = y;
     }
     coltile_store<NT, LPR, R>(v, out + boff, own_n, m, col0);
-    if (tid < 64) xch_retire(xch, team, parts);     // after the barrier above: this workgroup holds all it needs
+    if (tid < 64) xch_retire(xl, team, parts);     // after the barrier above: this workgroup holds all it needs
 }
 
 // Generic fallback (any n, m, alignment): 64 columns x 4 row groups per workgroup, two
@@ -288,18 +293,20 @@ static int layernorm_dispatch(int32_t batch, int32_t n, int32_t m, const void* m
                 for (int64_t b0 = 0; b0 < batch; b0 += per_launch) {
                     const int64_t nb = batch - b0 < per_launch ? batch - b0 : per_launch;
                     XchLaunch xl;
-                    const int rc = xch_begin(&xl);
+                    const int rc = xch_begin(&xl, tiles * nb * parts, st);
                     if (rc != 0) return rc;
                     const dim3 grid((unsigned)(tiles * nb * parts));
                     const half_t* xb = x + b0 * n * m;
                     half_t* yb = y + b0 * n * m;
                     if (big)
                         hipLaunchKernelGGL((k_layernorm_team<1024, 8>), grid, dim3(1024), 0, st, n, m, (int32_t)tiles,
-                                           (int32_t)parts, xb, yb, al, be, eps, rd_mean, xl.region, xl.tag);
+                                           (int32_t)parts, xb, yb, al, be, eps, rd_mean, xl);
                     else
                         hipLaunchKernelGGL((k_layernorm_team<512, 8>), grid, dim3(512), 0, st, n, m, (int32_t)tiles,
-                                           (int32_t)parts, xb, yb, al, be, eps, rd_mean, xl.region, xl.tag);
-                    if (int e = launch_status()) return e;
+                                           (int32_t)parts, xb, yb, al, be, eps, rd_mean, xl);
+                    const int e = launch_status();
+                    const int rc2 = xch_end(xl, st);
+                    if (e != 0 || rc2 != 0) return e ? e : rc2;
                 }
                 return 0;
             }

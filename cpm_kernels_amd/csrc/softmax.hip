@@ -178,10 +178,12 @@ __global__ __launch_bounds__(NT) void k_softmax_stream(int32_t n, int32_t m, int
 // which is the single-workgroup result up to two extra fp32 roundings.
 template <int NT, int R>
 __global__ __launch_bounds__(NT) void k_softmax_team(int32_t n, int32_t m, int32_t tiles_per_batch, int32_t parts,
-                                                     const half_t* inp, half_t* out, uint64_t* xch, uint32_t tag) {
+                                                     const half_t* inp, half_t* out, XchLaunch xl) {
     constexpr int LPR = 8;
     using T = ColTile<NT, LPR, R>;
     static_assert(T::COLS * 2 == kXchVals, "slot layout");
+    uint64_t* const xch = xl.region;
+    const uint32_t tag = xl.tag;
     __shared__ float lds[(T::NW + 1) * T::COLS];
     __shared__ float tot[kXchVals];
     const int tid = threadIdx.x;
@@ -257,6 +259,7 @@ __global__ __launch_bounds__(NT) void k_softmax_team(int32_t n, int32_t m, int32
             if (q < parts) S += sp[q] * __builtin_amdgcn_exp2f(mp[q] - M);
         tot[tid] = M;
         tot[T::COLS + tid] = ok ? 1.0f / (S + 1e-10f) : __builtin_nanf("");
+        if (!ok) xch_flag(xl.status, kXchStatusTimeout);
     }
     __syncthreads();
     const int cg = tid % LPR;
@@ -269,7 +272,7 @@ __global__ __launch_bounds__(NT) void k_softmax_team(int32_t n, int32_t m, int32
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[p][e] = round_f16(ex[p][e] * f[e]);
     coltile_store<NT, LPR, R>(v, out + boff, own_n, m, col0);
-    if (tid < 64) xch_retire(xch, team, parts);     // after the barrier above: this workgroup holds all it needs
+    if (tid < 64) xch_retire(xl, team, parts);     // after the barrier above: this workgroup holds all it needs
 }
 
 // Generic fallback: 64 columns x 4 row groups, three passes (max, sum, write).  All reads of
@@ -332,14 +335,8 @@ static int launch_stream(int32_t batch, int32_t n, int32_t m, const half_t* inp,
     constexpr int smem = NT * R * 16 + (T::NW + 1) * T::COLS * (int)sizeof(float) + 16;
     static_assert(smem <= 160 * 1024, "LDS of one compute unit");
     auto kern = k_softmax_stream<NT, LPR, R>;
-    static bool attr_set[64] = {false};       // dynamic LDS above 64 KB must be enabled per device
-    int dev = 0;
-    (void)hipGetDevice(&dev);
-    if (dev >= 0 && dev < 64 && !attr_set[dev]) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-        if (e != hipSuccess) return (int)e;
-        attr_set[dev] = true;
-    }
+    static std::atomic<bool> lds_enabled[64];
+    if (int e = enable_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_enabled)) return e;
     const int32_t tiles = (int32_t)ceil_div(m, LPR * 8);
     const int64_t ntiles = (int64_t)tiles * batch;
     const int cus = compute_units();
@@ -385,18 +382,20 @@ static int softmax_dispatch(int32_t batch, int32_t n, int32_t m, const void* inp
                 for (int64_t b0 = 0; b0 < batch; b0 += per_launch) {
                     const int64_t nb = batch - b0 < per_launch ? batch - b0 : per_launch;
                     XchLaunch xl;
-                    const int rc = xch_begin(&xl);
+                    const int rc = xch_begin(&xl, tiles * nb * parts, st);
                     if (rc != 0) return rc;
                     const dim3 grid((unsigned)(tiles * nb * parts));
                     const half_t* xb = x + b0 * n * m;
                     half_t* yb = y + b0 * n * m;
                     if (big)
                         hipLaunchKernelGGL((k_softmax_team<1024, 8>), grid, dim3(1024), 0, st, n, m, (int32_t)tiles,
-                                           (int32_t)parts, xb, yb, xl.region, xl.tag);
+                                           (int32_t)parts, xb, yb, xl);
                     else
                         hipLaunchKernelGGL((k_softmax_team<512, 8>), grid, dim3(512), 0, st, n, m, (int32_t)tiles,
-                                           (int32_t)parts, xb, yb, xl.region, xl.tag);
-                    if (int e = launch_status()) return e;
+                                           (int32_t)parts, xb, yb, xl);
+                    const int e = launch_status();
+                    const int rc2 = xch_end(xl, st);
+                    if (e != 0 || rc2 != 0) return e ? e : rc2;
                 }
                 return 0;
             }

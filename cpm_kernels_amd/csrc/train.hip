@@ -265,7 +265,9 @@ __global__ __launch_bounds__(256) void k_col(ColArgs p) {
 constexpr int kColTeamMaxParts = 32;
 
 template <int KIND>
-__global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_batch, int32_t parts, uint64_t* xch, uint32_t tag) {
+__global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_batch, int32_t parts, XchLaunch xl) {
+    uint64_t* const xch = xl.region;
+    const uint32_t tag = xl.tag;
     constexpr int NT = 512, LPR = 8, R = 8;
     using T = ColTile<NT, LPR, R>;
     constexpr bool TWO = KIND != kLnFwdV && KIND != kLnFwdMV && KIND != kScaleRound;     // reads grad_in too
@@ -340,6 +342,7 @@ __global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_b
                 for (int j = 0; j < 8; ++j) acc = IS_MAX ? fmaxf(acc, x[j]) : acc + x[j];     // part order; absent parts are zeros
             }
             tot[tid] = ok ? acc : __builtin_nanf("");
+            if (!ok) xch_flag(xl.status, kXchStatusTimeout);
         }
         __syncthreads();
 #pragma unroll
@@ -395,7 +398,7 @@ __global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_b
             }
         coltile_store<NT, LPR, R>(va, p.out + boff, own_n, p.m, col0);
     }
-    if (parts > 1 && tid < 64) xch_retire(xch, team, parts);
+    if (parts > 1 && tid < 64) xch_retire(xl, team, parts);
 }
 
 // cu_gemm_backward_round_scale: per-row absmax of mat * scale_y[col] -> scale_x, then rounding.
@@ -480,7 +483,9 @@ __global__ __launch_bounds__(256) void k_position_backward_team(int32_t query_le
                                                                 int32_t max_distance, const int32_t* __restrict__ mapping,
                                                                 const half_t* __restrict__ grad_out, half_t* __restrict__ grad,
                                                                 int bidirectional, int32_t parts, int32_t rows_per_part,
-                                                                uint64_t* xch, uint32_t tag) {
+                                                                XchLaunch xl) {
+    uint64_t* const xch = xl.region;
+    const uint32_t tag = xl.tag;
     extern __shared__ float hist[];                       // num_buckets floats, then max_distance bucket numbers
     int32_t* lmap = reinterpret_cast<int32_t*>(hist + num_buckets);
     const uint32_t part = blockIdx.x % parts, h = blockIdx.x / parts;
@@ -531,10 +536,11 @@ __global__ __launch_bounds__(256) void k_position_backward_team(int32_t query_le
                 for (int j = 0; j < 8; ++j) acc += x[j];
             }
             grad[(int64_t)h * num_buckets + i] = ok ? (half_t)acc : (half_t)__builtin_nanf("");
+            if (!ok) xch_flag(xl.status, kXchStatusTimeout);
         }
         __syncthreads();
     }
-    if (tid < 64) xch_retire(xch, h, parts);
+    if (tid < 64) xch_retire(xl, h, parts);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -648,14 +654,16 @@ static int launch_col(int32_t batch, const ColArgs& p, void* stream) {
         for (int64_t b0 = 0; b0 < batch; b0 += per_launch) {
             const int64_t nb = batch - b0 < per_launch ? batch - b0 : per_launch;
             const ColArgs q = col_args_from(p, b0);
-            XchLaunch xl = {nullptr, 0};
+            XchLaunch xl = {nullptr, nullptr, nullptr, 0, -1};
             if (parts > 1) {
-                const int rc = xch_begin(&xl);
+                const int rc = xch_begin(&xl, tiles * nb * parts, (hipStream_t)stream);
                 if (rc != 0) return rc;
             }
             hipLaunchKernelGGL((k_col_team<KIND>), dim3((unsigned)(tiles * nb * parts)), dim3(512), 0, (hipStream_t)stream, q,
-                               (int32_t)tiles, (int32_t)parts, xl.region, xl.tag);
-            if (int e = launch_status()) return e;
+                               (int32_t)tiles, (int32_t)parts, xl);
+            const int e = launch_status();
+            const int rc2 = xch_end(xl, (hipStream_t)stream);
+            if (e != 0 || rc2 != 0) return e ? e : rc2;
         }
         return 0;
     }
@@ -836,13 +844,15 @@ int cpmk_position_embedding_backward(int32_t query_len, int32_t key_len, int32_t
         const int64_t parts = ceil_div(key_len, rpp);
         if ((int64_t)num_heads * parts <= kXchSlots) {
             XchLaunch xl;
-            const int rc = xch_begin(&xl);
+            const int rc = xch_begin(&xl, (int64_t)num_heads * parts, (hipStream_t)stream);
             if (rc != 0) return rc;
             hipLaunchKernelGGL(k_position_backward_team, dim3((unsigned)(num_heads * parts)), dim3(256),
                                num_buckets * sizeof(float) + max_distance * sizeof(int32_t), (hipStream_t)stream, query_len, key_len,
                                num_buckets, max_distance, (const int32_t*)position_mapping, (const half_t*)grad_out, (half_t*)grad,
-                               bidirectional, (int32_t)parts, (int32_t)rpp, xl.region, xl.tag);
-            return launch_status();
+                               bidirectional, (int32_t)parts, (int32_t)rpp, xl);
+            const int e = launch_status();
+            const int rc2 = xch_end(xl, (hipStream_t)stream);
+            return e ? e : rc2;
         }
     }
     hipLaunchKernelGGL(k_position_backward, dim3((unsigned)num_heads), dim3(256), num_buckets * sizeof(float), (hipStream_t)stream,

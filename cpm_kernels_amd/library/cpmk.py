@@ -76,6 +76,8 @@ _LAUNCHERS = {
     "cpmk_copy_extend_buffer": [ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p],
     "cpmk_has_nan_inf": [ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p],
     "cpmk_copy_pos_hidden": [ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p],
+    "cpmk_async_status": [],
+    "cpmk_selftest_exchange_timeout": [ctypes.c_int32, ctypes.c_void_p],
 }
 
 EXPORTED_SYMBOLS = sorted(list(_LAUNCHERS) + [

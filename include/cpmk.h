@@ -36,6 +36,7 @@ extern "C" {
 #define CPMK_EBADARG   10001  /* negative size, null pointer with non-empty work, ...   */
 #define CPMK_EALIGN    10002  /* divisibility precondition of the reference violated    */
 #define CPMK_ETOOBIG   10003  /* problem exceeds a documented limit of this library     */
+#define CPMK_ETIMEOUT  10004  /* cpmk_async_status: a kernel's bounded wait ran out      */
 
 /* ---- library / device queries (replace cpm_kernels/library/cudart.py and
  *      cpm_kernels/device/__init__.py:106-158) ------------------------------------ */
@@ -53,6 +54,19 @@ int         cpmk_device_props(int device, char* name, int name_len, int* compute
                               int* lds_bytes, int* wavefront, int* clock_khz,
                               int* mem_clock_khz, int* mem_bus_bits, int* l2_bytes,
                               uint64_t* global_mem_bytes);
+
+/* Failures that a kernel can only discover while it runs.  The kernels that split a column over
+ * several workgroups (tall layernorm / softmax, the column quantiser, the dim-1 reductions of the
+ * training side) wait for each other's partial results with a bound of about one second; a wait
+ * that runs out fills the affected outputs with NaN (0 in int8 tensors) and sets a sticky word on
+ * the device.  This call copies that word to the host and clears it: 0, CPMK_ETIMEOUT, or a HIP
+ * error code.  It blocks like a hipMemcpy, so synchronise the streams in question first.  The
+ * reference reports every failure of a launch or a synchronisation as an exception
+ * (library/cudart.py:325-327, cudaGetLastError); the Python binding raises on a non-zero value. */
+int         cpmk_async_status(void);
+/* Launches one workgroup that waits `microseconds` for a result nobody produces and then reports
+ * the time-out as above: exercises the failure path with a kernel that ends normally (tests). */
+int         cpmk_selftest_exchange_timeout(int32_t microseconds, void* stream);
 
 /* ---- row / column quantisation (kernels/gemm.py, cuda/gemm.cu) ------------------- */
 /* out[b,i] = fp16( max_j |mat[b,i,j]| / 127 )            gemm.py:91-107 / gemm.cu:60-76 */

@@ -364,6 +364,49 @@ def test_gemm_int8_north_star_checksums(gpu):
     assert np.array_equal(o[jj, ii], (a64[jj] * w64[ii]).sum(axis=1))
 
 
+def test_north_star_fused_pipeline_bits(gpu):
+    """The benchmarked call itself at full size -- quantise A [4096,4096] and W [10240,4096] (seed 1000, the
+    bench's data), then the fused int8 GEMM + dequantisation -- checked to the bit on 64 output rows
+    (four in every row tile, in both row halves of a tile) and all 10240 columns against the oracle's
+    quantise -> exact integer product -> gemm_scale chain, and `ct.bmm` against the kernel-level calls
+    on the whole output."""
+    _name("north-star fused bits")
+    import cpm_kernels_amd.torch as ct
+    M, K, N = 4096, 4096, 10240
+    g = torch.Generator().manual_seed(1000)
+    A = torch.randn(1, M, K, generator=g).half()
+    W = (torch.randn(1, N, K, generator=g) * 0.02).half()
+    Ad, Wd = A.cuda(), W.cuda()
+    sA = torch.empty((1, M), dtype=torch.half, device=gpu); qA = torch.empty((1, M, K), dtype=torch.int8, device=gpu)
+    sW = torch.empty((1, N), dtype=torch.half, device=gpu); qW = torch.empty((1, N, K), dtype=torch.int8, device=gpu)
+    ck.gemm_quantize(1, M, K, Ad.data_ptr(), sA.data_ptr(), qA.data_ptr(), False, stream())
+    ck.gemm_quantize(1, N, K, Wd.data_ptr(), sW.data_ptr(), qW.data_ptr(), False, stream())
+    out = torch.empty((1, M, N), dtype=torch.half, device=gpu)
+    ck.gemm_int8_scale(N, K, M, 1, 1, True, False, qW.data_ptr(), qA.data_ptr(), sA.data_ptr(), sW.data_ptr(),
+                       True, True, out.data_ptr(), stream())
+    rows = np.array([t * 256 + off for t in range(16) for off in (3, 130, 200, 255)])
+    An, Wn = A.numpy(), W.numpy()
+    sWr = oracle.gemm_calc_scale(Wn); qWr = oracle.gemm_round(Wn, sWr)
+    assert_bits_equal(to_np(sW), sWr, "W scales"); assert_bits_equal(to_np(qW), qWr, "W int8")
+    Ar = np.ascontiguousarray(An[:, rows])
+    sAr = oracle.gemm_calc_scale(Ar); qAr = oracle.gemm_round(Ar, sAr)
+    assert_bits_equal(to_np(sA)[:, rows], sAr, "A scales (sampled rows)")
+    assert_bits_equal(to_np(qA)[:, rows], qAr, "A int8 (sampled rows)")
+    acc = oracle.gemm_int8_blas(N, K, len(rows), True, False, qWr, qAr)
+    ref = oracle.gemm_scale(acc, sAr, sWr, True, True)
+    assert_bits_equal(to_np(out)[:, rows], ref, "fused GEMM, sampled rows x all columns")
+    # the int32 variant on the same operands, and the separate dequantisation of it
+    acc_d = torch.empty((1, M, N), dtype=torch.int32, device=gpu)
+    ck.gemm_int8(N, K, M, 1, 1, True, False, qW.data_ptr(), qA.data_ptr(), acc_d.data_ptr(), stream())
+    assert_bits_equal(to_np(acc_d)[:, rows], acc, "int32 GEMM, sampled rows")
+    two = torch.empty_like(out)
+    ck.gemm_scale(1, M, N, acc_d.data_ptr(), sA.data_ptr(), sW.data_ptr(), two.data_ptr(), True, True, stream())
+    assert torch.equal(two.view(torch.int16), out.view(torch.int16)), "fused != gemm_int8 + gemm_scale"
+    del acc_d, two
+    y = ct.bmm(Ad, False, Wd, True, int8=True)
+    assert y.shape == (1, M, N) and torch.equal(y.view(torch.int16), out.view(torch.int16)), "ct.bmm != kernel-level calls"
+
+
 # ---------------------------------------------------------------------------------------------
 # decode GEMV
 # ---------------------------------------------------------------------------------------------
@@ -663,6 +706,76 @@ def test_softmax_causal_full_size_properties(gpu):
     assert torch.allclose(o.sum(dim=1), torch.ones(b, m, device=gpu), atol=2e-3)
     ref = oracle.softmax_forward(s[:2].numpy())
     assert_close_fp16(to_np(out[:2]), ref, rtol=1e-3, atol=1e-7, max_ulp=2, what="softmax causal sample")
+
+
+STEP_SHAPES = [(32, 4096), (32, 10240), (3, 4099), (128, 768), (1, 2), (7, 1024)]
+
+
+@pytest.mark.parametrize("shape", STEP_SHAPES)
+@pytest.mark.parametrize("rd_mean", [True, False])
+def test_layernorm_step_decode_sizes(gpu, shape, rd_mean):
+    """layernorm_step and layernorm_step_inplace at decode sizes: equal to forward(m=1) as the
+    reference pins it (tests/test_layernorm.py:115-152, isclose 1e-5 there, bits here) and within
+    1e-3 of the oracle."""
+    _name("layernorm_step", shape, rd_mean)
+    b, n = shape
+    rng = np.random.default_rng(2003 + n)
+    x = (rng.standard_normal(shape) * 1.7 + (0.4 if rd_mean else 0.0)).astype(np.float16)
+    for eps in (1e-5, 1e-3):
+        ref = oracle.layernorm_forward(x[:, :, None], eps, rd_mean)[:, :, 0]
+        xd = to_gpu(x)
+        fwd = torch.empty_like(xd); out = torch.empty_like(xd)
+        ck.layernorm_forward(b, n, 1, xd.data_ptr(), fwd.data_ptr(), eps, rd_mean, stream())
+        ck.layernorm_step(b, n, xd.data_ptr(), out.data_ptr(), eps, rd_mean, stream())
+        assert_close_fp16(to_np(out), ref, rtol=1e-3, atol=2e-4, what="layernorm_step vs oracle")
+        assert_bits_equal(to_np(out), to_np(fwd), "layernorm_step == forward(m=1)")
+        ck.layernorm_step_inplace(b, n, xd.data_ptr(), eps, rd_mean, stream())
+        assert_bits_equal(to_np(xd), to_np(out), "layernorm_step_inplace == layernorm_step")
+
+
+@pytest.mark.parametrize("shape", STEP_SHAPES + [(3, 12321), (123, 321)])
+def test_softmax_step_decode_sizes(gpu, shape):
+    """softmax_step_inplace at decode sizes against forward(m=1) (tests/test_softmax.py:51-76 of the
+    reference) and the oracle, with masked (-inf) entries and one fully masked row."""
+    _name("softmax_step", shape)
+    b, n = shape
+    rng = np.random.default_rng(2004 + n)
+    x = rand_half(rng, shape, 4.0)
+    x[0, n // 2:] = -np.inf
+    if b > 1:
+        x[1, :] = -np.inf
+    ref = oracle.softmax_forward(x[:, :, None])[:, :, 0]
+    xd = to_gpu(x); fwd = torch.empty_like(xd)
+    ck.softmax_forward(b, n, 1, xd.data_ptr(), fwd.data_ptr(), stream())
+    ck.softmax_step_inplace(b, n, xd.data_ptr(), stream())
+    assert_close_fp16(to_np(xd), ref, rtol=1e-3, atol=1e-7, max_ulp=2, what="softmax_step_inplace vs oracle")
+    assert_bits_equal(to_np(xd), to_np(fwd), "softmax_step_inplace == forward(m=1)")
+    assert (to_np(xd)[0, n // 2:] == 0).all()
+
+
+def test_softmax_config3_full_size_properties(gpu):
+    """The exact config-3 workload, [512,1024,1024] causal (the bench's tensor): masked entries exactly
+    0, every column sums to 1, the first and last batch entries match the oracle, and the eight
+    repeats of the 64 distinct score matrices give identical results."""
+    _name("softmax config 3 full size")
+    g = torch.Generator().manual_seed(1003)
+    s = (torch.randn(64, 1024, 1024, generator=g) * 4).half()
+    kk = torch.arange(1024)[:, None]; qq = torch.arange(1024)[None, :]
+    s.masked_fill_((kk > qq)[None], float("-inf"))
+    xd = s.cuda().repeat(8, 1, 1).contiguous()
+    out = torch.empty_like(xd)
+    ck.softmax_forward(512, 1024, 1024, xd.data_ptr(), out.data_ptr(), stream())
+    torch.cuda.synchronize()
+    masked = (kk > qq).cuda()
+    for c in range(0, 512, 64):
+        o = out[c:c + 64]
+        assert torch.all(o.masked_select(masked[None]) == 0)
+        assert torch.allclose(o.float().sum(dim=1), torch.ones(64, 1024, device=gpu), atol=2e-3)
+        assert torch.equal(o.view(torch.int16), out[:64].view(torch.int16)), "repeat %d differs" % (c // 64)
+    ref = oracle.softmax_forward(s[[0, 63]].numpy())
+    assert_close_fp16(to_np(out[[448, 511]]), ref, rtol=1e-3, atol=1e-7, max_ulp=2, what="softmax config 3 sample")
+    ck.softmax_inplace_forward(512, 1024, 1024, xd.data_ptr(), stream())
+    assert torch.equal(xd.view(torch.int16), out.view(torch.int16)), "in place != out of place"
 
 
 def test_gelu_all_fp16_inputs(gpu):

@@ -148,3 +148,93 @@ def test_results_do_not_depend_on_timing(gpu):
     runs(lambda: ck.gemv_broadcast_mat_int8(32, 10240, 4096, sW.data_ptr(), W.data_ptr(), sv.data_ptr(), v.data_ptr(), o.data_ptr(), s), [o])
     o2 = torch.empty((32, 2048), dtype=torch.half, device=gpu)
     runs(lambda: ck.gemv_broadcast_mat_fp16(32, 2048, 4096, Wh.data_ptr(), vh.data_ptr(), o2.data_ptr(), s), [o2])
+
+
+def test_team_launches_overlapping_on_eight_streams(gpu):
+    """Team kernels of different kinds queued on eight streams at once, three rounds of them: each
+    launch gets packet slots of its own, so every result equals the single-stream result bit for
+    bit and no wait runs out.  The reference's kernels keep no state between launches
+    (cuda/layernorm.cu:6-71, cuda/softmax.cu:6-43), so callers may overlap them freely."""
+    _name("eight streams of team kernels")
+    from cpm_kernels_amd.library import cpmk
+    g = torch.Generator().manual_seed(43)
+    s0 = stream()
+    xs = [(torch.randn(8, 4096, 512, generator=g) * (1 + i)).half().to(gpu) for i in range(8)]
+    tall = [(torch.randn(2, 8192, 256, generator=g) * 3).half().to(gpu) for i in range(8)]
+    cpmk.async_status()                                         # nothing pending from earlier tests
+
+    def one(i, x, t, s):
+        y = torch.empty_like(x); so = torch.empty_like(t)
+        sc = torch.empty((8, 512), dtype=torch.half, device=gpu); q = torch.empty((8, 512, 4096), dtype=torch.int8, device=gpu)
+        if i % 3 == 0:
+            ck.layernorm_forward(8, 4096, 512, x.data_ptr(), y.data_ptr(), 1e-5, True, s)
+            ck.softmax_forward(2, 8192, 256, t.data_ptr(), so.data_ptr(), s)
+            ck.gemm_quantize_cols(8, 4096, 512, x.data_ptr(), sc.data_ptr(), q.data_ptr(), True, s)
+        elif i % 3 == 1:
+            ck.softmax_forward(2, 8192, 256, t.data_ptr(), so.data_ptr(), s)
+            ck.gemm_quantize_cols(8, 4096, 512, x.data_ptr(), sc.data_ptr(), q.data_ptr(), True, s)
+            ck.layernorm_forward(8, 4096, 512, x.data_ptr(), y.data_ptr(), 1e-5, True, s)
+        else:
+            ck.gemm_quantize_cols(8, 4096, 512, x.data_ptr(), sc.data_ptr(), q.data_ptr(), True, s)
+            ck.layernorm_forward(8, 4096, 512, x.data_ptr(), y.data_ptr(), 1e-5, True, s)
+            ck.softmax_forward(2, 8192, 256, t.data_ptr(), so.data_ptr(), s)
+        return y, so, sc, q
+
+    ref = [one(0, xs[i], tall[i], s0) for i in range(8)]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream() for _ in range(8)]
+    for rnd in range(3):
+        got = []
+        for i, st in enumerate(streams):
+            with torch.cuda.stream(st):
+                got.append(one(i + rnd, xs[i], tall[i], st.cuda_stream))
+        torch.cuda.synchronize()
+        cpmk.async_status()                                     # raises if any wait ran out
+        for i in range(8):
+            for a, b, what in zip(got[i], ref[i], ("layernorm", "softmax", "column scales", "column int8")):
+                assert_bits_equal(to_np(a), to_np(b), "round %d stream %d %s" % (rnd, i, what))
+
+
+def test_more_launches_than_the_pool_holds(gpu):
+    """300 tall layernorms back to back on two streams take more packet slots than the pool has, so
+    slots are reused while earlier launches may still run: the later launch must wait for the
+    earlier one's completion, and all results stay equal."""
+    _name("packet pool wraps around")
+    from cpm_kernels_amd.library import cpmk
+    g = torch.Generator().manual_seed(44)
+    x = torch.randn(8, 4096, 512, generator=g).half().to(gpu)
+    ref = torch.empty_like(x)
+    ck.layernorm_forward(8, 4096, 512, x.data_ptr(), ref.data_ptr(), 1e-5, True, stream())
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream() for _ in range(2)]
+    outs = [torch.zeros_like(x) for _ in range(6)]
+    for i in range(300):
+        st = streams[i % 2]
+        with torch.cuda.stream(st):
+            ck.layernorm_forward(8, 4096, 512, x.data_ptr(), outs[i % 6].data_ptr(), 1e-5, True, st.cuda_stream)
+    torch.cuda.synchronize()
+    cpmk.async_status()
+    for o in outs:
+        assert torch.equal(o.view(torch.int16), ref.view(torch.int16))
+
+
+def test_a_wait_that_runs_out_is_reported(gpu):
+    """A workgroup that gives up waiting sets the device's status word; cpmk_async_status turns it into
+    the RuntimeError the reference raises for any failed launch or synchronisation
+    (library/cudart.py:325-327), once, and clears it.  The self-test kernel waits 2 ms for a packet
+    nobody posts and then ends normally."""
+    _name("time-out status")
+    from cpm_kernels_amd.library import cpmk
+    torch.cuda.synchronize()
+    cpmk.async_status()
+    cpmk.selftest_exchange_timeout(2000, stream())
+    torch.cuda.synchronize()
+    with pytest.raises(RuntimeError, match="gave up waiting"):
+        cpmk.async_status()
+    cpmk.async_status()                                         # cleared by the read
+    # the pool still works afterwards
+    x = torch.randn(2, 4096, 64).half().to(gpu); y = torch.empty_like(x); z = torch.empty_like(x)
+    ck.layernorm_forward(2, 4096, 64, x.data_ptr(), y.data_ptr(), 1e-5, True, stream())
+    ck.layernorm_forward(2, 4096, 64, x.data_ptr(), z.data_ptr(), 1e-5, True, stream())
+    assert torch.equal(y.view(torch.int16), z.view(torch.int16)) and bool(torch.isfinite(y).all())
+    cpmk.async_status()
