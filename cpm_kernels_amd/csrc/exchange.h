@@ -55,6 +55,10 @@ int xch_begin(XchLaunch* out, int64_t slots, hipStream_t st);
 // Host, after the launch: records the launch's completion on `st` so that a later holder of its slots
 // can wait for it.  0 or an error code.
 int xch_end(const XchLaunch& xl, hipStream_t st);
+// Host: a tag for a team launch that brings its own packet slots (never 0, from the same sequence as xch_begin's).
+uint32_t xch_next_tag();
+// Host: the address of the current device's status word, for such a launch.  0 or an error code.
+int xch_status_word(uint32_t** out);
 // Host: reads and clears the current device's status word (0, kXchStatus* bits, or -1 - hipError on failure to read).
 int xch_take_status(uint32_t* bits);
 

@@ -59,6 +59,20 @@ bool capturing(hipStream_t st) {
 
 }  // namespace
 
+uint32_t xch_next_tag() {
+    uint32_t s = g_seq.fetch_add(1, std::memory_order_relaxed) + 1;
+    if (s == 0) s = g_seq.fetch_add(1, std::memory_order_relaxed) + 1;   // tag 0 is what a fresh pool holds
+    return s;
+}
+
+int xch_status_word(uint32_t** out) {
+    std::lock_guard<std::mutex> lock(g_mu);
+    DevicePool* d = nullptr;
+    if (int rc = device_pool(&d)) return rc;
+    *out = d->status;
+    return 0;
+}
+
 int xch_begin(XchLaunch* out, int64_t slots, hipStream_t st) {
     if (slots < 1 || slots > kXchSlots) return CPMK_ETOOBIG;
     const int32_t need = (int32_t)(ceil_div(slots, kXchGranule) * kXchGranule);
@@ -86,8 +100,7 @@ int xch_begin(XchLaunch* out, int64_t slots, hipStream_t st) {
             ++i;
         }
     }
-    uint32_t s = g_seq.fetch_add(1, std::memory_order_relaxed) + 1;
-    if (s == 0) s = g_seq.fetch_add(1, std::memory_order_relaxed) + 1;   // tag 0 is what a fresh pool holds
+    const uint32_t s = xch_next_tag();
     out->region = d->base + (size_t)first * kXchVals;
     out->counters = d->base + (size_t)kXchPoolSlots * kXchVals + first;
     out->status = d->status;

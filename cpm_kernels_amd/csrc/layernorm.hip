@@ -5,6 +5,7 @@
 // cu_arith_ln_mul (cuda/arith.cu:97-127): fp16 fma(y, alpha[i], beta[i]) or y * alpha[i].
 #include "dim1.h"
 #include "exchange.h"
+#include <mutex>
 
 namespace cpmk {
 
@@ -267,8 +268,12 @@ static bool launch_tile_r(int r, int32_t batch, int32_t n, int32_t m, const half
     return true;
 }
 
+// `fixed` == nullptr: team launches take their packet slots from the library's pool (exchange.hip).
+// Otherwise the one team launch a call may need uses the slots, counters and status word `fixed`
+// names (fixed_slots of them) and a shape that needs more is refused with CPMK_ETOOBIG.
 static int layernorm_dispatch(int32_t batch, int32_t n, int32_t m, const void* mat, void* out, const void* alpha,
-                              const void* beta, float eps, int rd_mean, hipStream_t st) {
+                              const void* beta, float eps, int rd_mean, hipStream_t st, const XchLaunch* fixed = nullptr,
+                              int64_t fixed_slots = 0) {
     if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
     if ((int64_t)batch * n * m == 0) return 0;
     const half_t* x = (const half_t*)mat;
@@ -287,14 +292,19 @@ static int layernorm_dispatch(int32_t batch, int32_t n, int32_t m, const void* m
             const int64_t tiles = ceil_div(m, 64);
             const bool big = n >= 2048;                       // 1024 rows a part, else 512
             const int64_t parts = ceil_div(n, big ? 1024 : 512);
+            if (fixed != nullptr && parts <= kXchMaxParts && tiles * parts * batch > fixed_slots) return CPMK_ETOOBIG;
             if (parts <= kXchMaxParts && tiles * parts <= kXchSlots) {
                 // one packet slot per (team, part): batches beyond the pool go out in several launches
-                const int64_t per_launch = kXchSlots / (tiles * parts);
+                const int64_t per_launch = fixed != nullptr ? batch : kXchSlots / (tiles * parts);
                 for (int64_t b0 = 0; b0 < batch; b0 += per_launch) {
                     const int64_t nb = batch - b0 < per_launch ? batch - b0 : per_launch;
                     XchLaunch xl;
-                    const int rc = xch_begin(&xl, tiles * nb * parts, st);
-                    if (rc != 0) return rc;
+                    if (fixed != nullptr) {
+                        xl = *fixed;
+                    } else {
+                        const int rc = xch_begin(&xl, tiles * nb * parts, st);
+                        if (rc != 0) return rc;
+                    }
                     const dim3 grid((unsigned)(tiles * nb * parts));
                     const half_t* xb = x + b0 * n * m;
                     half_t* yb = y + b0 * n * m;
@@ -305,7 +315,7 @@ static int layernorm_dispatch(int32_t batch, int32_t n, int32_t m, const void* m
                         hipLaunchKernelGGL((k_layernorm_team<512, 8>), grid, dim3(512), 0, st, n, m, (int32_t)tiles,
                                            (int32_t)parts, xb, yb, al, be, eps, rd_mean, xl);
                     const int e = launch_status();
-                    const int rc2 = xch_end(xl, st);
+                    const int rc2 = fixed != nullptr ? 0 : xch_end(xl, st);
                     if (e != 0 || rc2 != 0) return e ? e : rc2;
                 }
                 return 0;
@@ -326,6 +336,35 @@ static int layernorm_dispatch(int32_t batch, int32_t n, int32_t m, const void* m
     return 0;
 }
 
+// ---------------------------------------------------------------------------------------
+// Packet slots of cpmk_layernorm_forward_noalloc: kNoAllocSlots slots of kXchVals packets, then
+// one retire counter per slot.  Static storage, so every GPU the library runs on holds its own
+// copy (2.1 MB) at its own address until the process ends.  All zero at load; a team launch
+// leaves it all zero again (the last member of each team clears the team's slots and counter).
+constexpr int kNoAllocSlots = 2048;
+static __device__ __align__(256) uint64_t scratch[(size_t)kNoAllocSlots * kXchVals + kNoAllocSlots];
+
+// The array's address on the current device, looked up once per device (`scratch` itself is only a
+// host-side handle for the symbol, not a device address).
+static int noalloc_scratch(uint64_t** out) {
+    static std::mutex mu;
+    static uint64_t* ptr[64] = {nullptr};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= 64) return CPMK_EBADARG;
+    std::lock_guard<std::mutex> lock(mu);
+    if (ptr[dev] == nullptr) {
+        uint64_t* p = nullptr;
+        e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (p == nullptr) return CPMK_EBADARG;
+        ptr[dev] = p;
+    }
+    *out = ptr[dev];
+    return 0;
+}
+
 }  // namespace cpmk
 
 using namespace cpmk;
@@ -336,6 +375,20 @@ int cpmk_layernorm_forward(int32_t batch, int32_t n, int32_t m, const void* mat,
                            int rd_mean, void* stream) {
     clear_stale_error();
     return layernorm_dispatch(batch, n, m, mat, out, nullptr, nullptr, eps, rd_mean, (hipStream_t)stream);
+}
+
+int cpmk_layernorm_forward_noalloc(int32_t batch, int32_t n, int32_t m, const void* mat, void* out, float eps,
+                                   int rd_mean, void* stream) {
+    clear_stale_error();
+    uint64_t* base = nullptr;
+    if (int rc = noalloc_scratch(&base)) return rc;
+    XchLaunch xl;
+    xl.region = base;
+    xl.counters = base + (size_t)kNoAllocSlots * kXchVals;
+    xl.tag = xch_next_tag();
+    xl.first = -1;
+    if (int rc = xch_status_word(&xl.status)) return rc;
+    return layernorm_dispatch(batch, n, m, mat, out, nullptr, nullptr, eps, rd_mean, (hipStream_t)stream, &xl, kNoAllocSlots);
 }
 
 int cpmk_layernorm_affine_forward(int32_t batch, int32_t n, int32_t m, const void* mat, const void* alpha,

@@ -204,6 +204,18 @@ int cpmk_layernorm_forward(int32_t batch, int32_t n, int32_t m, const void* mat,
  *                         layernorm.py:152-190 / layernorm.cu:343-421 */
 int cpmk_layernorm_step(int32_t batch, int32_t n, const void* mat, void* out, float eps,
                         int rd_mean, void* stream);
+/* cpmk_layernorm_forward for callers that cannot let the library allocate or track anything: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc and event creation.
+ * It has no counterpart in the reference.  Same arguments, same results to the bit.  Columns taller
+ * than 1024 rows are normalised by teams of workgroups that exchange partial sums through a fixed
+ * 2.1 MB array inside the library (2048 packet slots, one per (64-column tile, row part) pair; held
+ * by every GPU the library runs on) instead of the shared pool with its completion events: a call
+ * that needs more slots -- batch * ceil(m/64) * ceil(n / (n >= 2048 ? 1024 : 512)) > 2048 -- returns
+ * CPMK_ETOOBIG.  Makes no hipMalloc/hipFree/event call.  Every call on a GPU uses that GPU's one
+ * array: calls that overlap in time on one GPU (two streams, two host threads, a replay of a
+ * captured call concurrent with another) race; calls in stream order are safe. */
+int cpmk_layernorm_forward_noalloc(int32_t batch, int32_t n, int32_t m, const void* mat, void* out,
+                                   float eps, int rd_mean, void* stream);
 /* Normalisation followed by the affine of arith_ln_mul_add / arith_ln_mul applied to the
  * fp16-rounded result (beta == NULL -> multiply only), as
  * cpm_kernels/torch/layernorm.py:9-29,88-111 do in two launches.  Bit-identical to them. */
