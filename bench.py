@@ -1,7 +1,8 @@
 #!/usr/bin/env python3
 """Benchmark of the int8 quantized-GEMM inference path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only gemm|gemv|ln|softmax|other|pipeline|calib]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
+                    [--only gemm|gemv|ln|softmax|other|pipeline|c1|chains|ceilings|calib]
 
 One "step" is one pass of the path over the north-star workload: activations A fp16
 [1,4096,4096] ~N(0,1) and weights W fp16 [1,10240,4096] ~N(0,0.02) (seed 1000, generated on
@@ -13,7 +14,10 @@ Prints ONE JSON line.  `value` is 2*M*N*K / step time in TOP/s for that whole st
 `roofline` object is the GEMM kernel alone against the dense int8 MFMA peak; `components`
 carries the decode GEMV, layernorm and softmax kernels (and, after them, every other kernel of
 the path) against the HBM peak; `cpu_baseline`
-is the torch formulation of the same step timed on the host cores (a reported baseline).
+is the torch formulation of the same step timed on the host cores (a reported baseline);
+`ceilings` holds what yardstick kernels that do nothing else reach on the same chip in the same
+run (matrix pipe on zero / random operands, plain and tiled copies, a cold 42 MB read) and the
+vendor library's int8 product on the same shapes (calibration only; the library does not use it).
 """
 import argparse
 import json
@@ -29,12 +33,14 @@ PEAK_INT8_TOPS = 5000.0      # MI355X dense int8 MFMA, published
 PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, published
 M, K, N = 4096, 4096, 10240  # north-star GEMM
 
-# HBM bytes per launch of each kernel, measured offline with hardware counters (they cannot be
-# read from inside this process): `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` over
-# `python3 bench.py --no-cpu --only <workload>`, each counter scaled by what it reads for the
-# 256 MiB device copy of `--only calib` (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000 on MI355X).
-# MFMA pipe busy cycles / kernel cycles of the fused GEMM kernel from SQ_VALU_MFMA_BUSY_CYCLES and
-# SQ_BUSY_CYCLES (same offline procedure; profiles/gemm_mfma_utilisation.txt).
+# Hardware-counter figures cannot be read from inside this process.  They are taken offline --
+# `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` over `python3 bench.py --no-cpu --only <workload>`,
+# each counter scaled by what it reads for the 256 MiB device copy of `--only calib` (FETCH_SIZE x 2.000,
+# WRITE_SIZE x 1.000 on MI355X); MFMA pipe busy cycles / kernel cycles from SQ_VALU_MFMA_BUSY_CYCLES and
+# SQ_BUSY_CYCLES -- and are emitted with their source file so that they are not mistaken for
+# measurements of this run.
+OFFLINE_SOURCE = {"traffic": "profiles/hbm_traffic_counters.txt (offline rocprofv3 --pmc run of this bench, not measured by this process)",
+                  "mfma": "profiles/gemm_mfma_utilisation.txt (offline rocprofv3 --pmc run of this bench, not measured by this process)"}
 MFMA_BUSY_FRAC = 0.669
 
 TRAFFIC_BYTES = {
@@ -51,26 +57,32 @@ def parse():
     p.add_argument("--steps", type=int, default=50)
     p.add_argument("--warmup", type=int, default=10)
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    p.add_argument("--only", default="", help="run only one kernel loop (for profiling): gemm|gemv|ln|softmax|other|pipeline|calib "
+    p.add_argument("--only", default="", help="run only one leg (for profiling): gemm|gemv|ln|softmax|other|pipeline|c1|chains|ceilings|calib "
                         "(calib = a plain 256 MiB device copy, the known-size kernel that scales the HBM counters)")
     p.add_argument("--reps", type=int, default=200, help="launches per timed batch in the per-kernel loops")
     return p.parse_args()
 
 
-def event_ms(fn, reps, warmup=3):
-    """Average milliseconds per call of fn over `reps` back-to-back calls, from HIP events on
-    torch's current stream (the stream every launcher is given)."""
+def event_ms(fn, reps, warmup=3, batches=5):
+    """Milliseconds per call of fn from HIP events on torch's current stream (the stream every
+    launcher is given): `reps` back-to-back calls split into `batches` timed batches, median batch.
+    (One long batch is at the mercy of a single stall -- a monitoring tool sampling the device
+    takes tens of milliseconds now and then -- which the median discards.)"""
     import torch
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(reps):
-        fn()
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) / reps
+    per = max(1, reps // batches)
+    times = []
+    for _ in range(batches):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(per):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        times.append(e0.elapsed_time(e1) / per)
+    return sorted(times)[len(times) // 2]
 
 
 def graph_ms(launches, reps):
@@ -92,13 +104,17 @@ def graph_ms(launches, reps):
                 f()
         g.replay()
         torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(reps):
-            g.replay()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / (reps * len(launches)), "hipgraph"
+        per = max(1, reps // 3)
+        times = []
+        for _ in range(3):                   # three timed batches of replays, median batch
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(per):
+                g.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            times.append(e0.elapsed_time(e1) / (per * len(launches)))
+        return sorted(times)[1], "hipgraph"
     except Exception as ex:   # pragma: no cover
         sys.stderr.write("graph capture failed (%s); eager timing\n" % ex)
         i = [0]
@@ -129,6 +145,17 @@ def main():
     st = lambda: torch.cuda.current_stream().cuda_stream   # noqa: E731
     only = args.only
     result = {}
+
+    # peaks: the published ones every `frac` divides by, and the ones this device's own clocks give
+    props = cpmk.device_props(0)
+    peak_int8_clock = props["compute_units"] * props["clock_khz"] * 1e3 * 8192 / 1e12          # CUs x clock x 8192 int8 ops/clk/CU
+    peak_hbm_clock = props["mem_clock_khz"] * 1e3 * 2 * props["mem_bus_bits"] / 8 / 1e9        # memory clock x 2 (double data rate) x bus width
+    result["peaks"] = {
+        "int8_tops_published": PEAK_INT8_TOPS, "hbm_gbs_published": PEAK_HBM_GBS,
+        "int8_tops_clock_derived": round(peak_int8_clock, 1), "hbm_gbs_clock_derived": round(peak_hbm_clock, 1),
+        "formula": "int8: compute_units x clock_khz x 8192 ops/clk/CU; hbm: mem_clock_khz x 2 x mem_bus_bits / 8",
+        "compute_units": props["compute_units"], "clock_khz": props["clock_khz"], "mem_clock_khz": props["mem_clock_khz"],
+        "mem_bus_bits": props["mem_bus_bits"], "l2_bytes": props["l2_bytes"], "arch": props["name"]}
 
     if only == "calib":
         # a copy of known size: FETCH_SIZE / WRITE_SIZE read for it give the counters' scale
@@ -180,11 +207,14 @@ def main():
         ms = event_ms(gemm, max(20, args.steps), warmup=max(3, args.warmup))
         tops = ops / (ms * 1e-3) / 1e12
         roofline = {"kernel": "k_gemm_dma<2,4,4,2,128,1,true,2,0> (int8 MFMA GEMM + fused fp16 dequant), M=%d K=%d N=%d" % (M, K, N),
-                    "bound": "mfma", "achieved": round(tops, 2), "peak": PEAK_INT8_TOPS, "unit": "TFLOP/s",
-                    "ops": "int8 multiply-accumulates counted as 2 ops (TOP/s)",
+                    "bound": "mfma", "achieved": round(tops, 2), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
+                    "ops": "int8 multiply-accumulates counted as 2 ops",
                     "frac": round(tops / PEAK_INT8_TOPS, 4), "avg_kernel_us": round(ms * 1e3, 2),
+                    "peak_clock_derived": round(peak_int8_clock, 1), "frac_of_clock_derived": round(tops / peak_int8_clock, 4),
+                    "operands": "MALL-resident (one 58.7 MB operand pair and one 83.9 MB output reused by every launch)",
                     "traffic": TRAFFIC_BYTES["gemm_fused"], "traffic_unit": "bytes per launch (HBM fetch + write counters)",
-                    "mfma_busy_frac_of_cycles": MFMA_BUSY_FRAC,
+                    "traffic_source": OFFLINE_SOURCE["traffic"],
+                    "mfma_busy_frac_of_cycles": MFMA_BUSY_FRAC, "mfma_busy_source": OFFLINE_SOURCE["mfma"],
                     "algorithmic_bytes": M * K + N * K + 2 * M * N}
         out32 = torch.empty((1, M, N), dtype=torch.int32, device=dev)
 
@@ -194,15 +224,107 @@ def main():
         roofline["int32_out_tops"] = round(ops / (ms32 * 1e-3) / 1e12, 2)
         del out32
 
-    # ---- HBM-bound components ---------------------------------------------------------------
     components = {}
     reps = args.reps
+
+    # ---- config 1: the reference's own test shape, A [1,512,4096] x W [1,4096,4096] ----------------
+    if only in ("", "c1"):
+        gg = torch.Generator().manual_seed(1001)
+        A1 = torch.randn(1, 512, 4096, generator=gg).half().to(dev)
+        W1c = (torch.randn(1, 4096, 4096, generator=gg) * 0.02).half().to(dev)
+        ops1 = 2.0 * 512 * 4096 * 4096
+        sA1 = torch.empty((1, 512), dtype=torch.half, device=dev); qA1 = torch.empty((1, 512, 4096), dtype=torch.int8, device=dev)
+        sW1 = torch.empty((1, 4096), dtype=torch.half, device=dev); qW1 = torch.empty((1, 4096, 4096), dtype=torch.int8, device=dev)
+        acc1 = torch.empty((1, 512, 4096), dtype=torch.int32, device=dev); o1 = torch.empty((1, 512, 4096), dtype=torch.half, device=dev)
+
+        def c1_kernel_by_kernel():      # the six launches of the reference's pipeline (tests/test_gemm.py, torch/gemm.py:40-66)
+            ck.gemm_calc_scale(1, 512, 4096, A1.data_ptr(), sA1.data_ptr(), st())
+            ck.gemm_calc_scale(1, 4096, 4096, W1c.data_ptr(), sW1.data_ptr(), st())
+            ck.gemm_round(1, 512, 4096, A1.data_ptr(), sA1.data_ptr(), qA1.data_ptr(), st())
+            ck.gemm_round(1, 4096, 4096, W1c.data_ptr(), sW1.data_ptr(), qW1.data_ptr(), st())
+            ck.gemm_int8(4096, 4096, 512, 1, 1, True, False, qW1.data_ptr(), qA1.data_ptr(), acc1.data_ptr(), st())
+            ck.gemm_scale(1, 512, 4096, acc1.data_ptr(), sA1.data_ptr(), sW1.data_ptr(), o1.data_ptr(), True, True, st())
+        # ten launches per captured graph, so that the replay overhead is shared like in the other legs
+        ms_six, how = graph_ms([c1_kernel_by_kernel] * 10, max(5, reps // 10))
+        ms_g32, _ = graph_ms([lambda: ck.gemm_int8(4096, 4096, 512, 1, 1, True, False, qW1.data_ptr(), qA1.data_ptr(), acc1.data_ptr(), st())] * 10, max(5, reps // 10))
+        ms_g16, _ = graph_ms([lambda: ck.gemm_int8_scale(4096, 4096, 512, 1, 1, True, False, qW1.data_ptr(), qA1.data_ptr(), sA1.data_ptr(),
+                                                         sW1.data_ptr(), True, True, o1.data_ptr(), st())] * 10, max(5, reps // 10))
+        ms_pair, _ = graph_ms([lambda: ck.gemm_quantize_pair(512, A1.data_ptr(), sA1.data_ptr(), qA1.data_ptr(), 4096, W1c.data_ptr(), sW1.data_ptr(),
+                                                            qW1.data_ptr(), 4096, st())] * 10, max(5, reps // 10))
+        ms_bmm = event_ms(lambda: ct.bmm(A1, False, W1c, True, int8=True), max(20, reps // 2), warmup=10)
+        components["config 1 pipeline (A [1,512,4096] x W [1,4096,4096])"] = {
+            "bound": "mfma", "ops": ops1, "seed": 1001, "operands": "MALL-resident",
+            "gemm_int8_us": round(ms_g32 * 1e3, 2), "gemm_int8_tops": round(ops1 / (ms_g32 * 1e-3) / 1e12, 1),
+            "gemm_int8_scale_fused_us": round(ms_g16 * 1e3, 2), "gemm_int8_scale_fused_tops": round(ops1 / (ms_g16 * 1e-3) / 1e12, 1),
+            "frac": round(ops1 / (ms_g16 * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
+            "six_kernel_pipeline_us": round(ms_six * 1e3, 2), "quantize_pair_us": round(ms_pair * 1e3, 2), "bmm_int8_us": round(ms_bmm * 1e3, 2),
+            "bmm_int8_tops": round(ops1 / (ms_bmm * 1e-3) / 1e12, 1), "timing": how + " (kernels), events (bmm)"}
+        del A1, W1c, qA1, qW1, acc1, o1
+
+    # ---- configs 4 and 5 as whole chains through the torch wrappers, native (batch, hidden, seq) layout ----
+    if only in ("", "chains"):
+        with torch.no_grad():
+            d, dff = 4096, 10240
+            gg = torch.Generator().manual_seed(1004)
+            b4, s4 = 8, 512
+            x4 = torch.randn(b4, d, s4, generator=gg).half().to(dev)
+            W1f = (torch.randn(1, dff, d, generator=gg) * 0.02).half().to(dev); W2f = (torch.randn(1, d, dff, generator=gg) * 0.02).half().to(dev)
+            ln4 = ct.LayerNorm(d, bias=True).half().to(dev)
+            ln4.weight.copy_((1 + 0.1 * torch.randn(d, generator=gg)).half()); ln4.bias.copy_((0.1 * torch.randn(d, generator=gg)).half())
+
+            def ffn(x, ln, Wa, Wb):
+                h = ct.bmm(Wa, False, ln(x), False, int8=True)
+                h = ct.bmm(Wb, False, ct.gelu(h), False, int8=True)
+                return ct.element_add(h, x)
+            ms4 = event_ms(lambda: ffn(x4, ln4, W1f, W2f), 20)
+            ops4 = 2.0 * 2 * b4 * s4 * d * dff
+            components["config 4 FFN block (tokens 8 x 512)"] = {
+                "chain": "LayerNorm -> int8 bmm 4096->10240 -> gelu -> int8 bmm 10240->4096 -> residual add (weights and activations quantised in every call)",
+                "seed": 1004, "avg_us": round(ms4 * 1e3, 1), "tops_over_the_two_products": round(ops4 / (ms4 * 1e-3) / 1e12, 1),
+                "tokens_per_s": round(b4 * s4 / (ms4 * 1e-3), 0), "timing": "events, whole chain"}
+            del x4
+
+            gg = torch.Generator().manual_seed(1005)
+            b5, H, dh, s5 = 16, 64, 64, 1024
+            x5 = torch.randn(b5, d, s5, generator=gg).half().to(dev)
+            Wp = {n_: (torch.randn(1, d, d, generator=gg) * 0.02).half().to(dev) for n_ in "qkvo"}
+            ln1 = ct.LayerNorm(d, bias=True).half().to(dev); ln2 = ct.LayerNorm(d, bias=True).half().to(dev)
+            pe = ct.PositionEmbedding(H, 32, 128, True).half().to(dev)
+            pe.weight.copy_((torch.randn(H, 32, generator=gg) * 0.02).half())
+            lens = torch.randint(512, 1025, (b5,), generator=gg)
+            pad = (torch.arange(s5)[None, :] < lens[:, None]).to(dev)
+
+            def layer(x):
+                h = ln1(x)
+                q, k, v = (ct.bmm(Wp[n_], False, h, False, int8=True).view(b5 * H, dh, s5) for n_ in "qkv")
+                scores = ct.bmm(k, True, q, False, int8=False)                       # (b*H, len_k, len_q)
+                ct.global_scale_inplace(scores, 1.0 / dh ** 0.5)
+                bias = pe(s5, s5)
+                scores = ct.batched_add(scores.view(b5, H * s5 * s5), bias.view(-1)).view(b5, H * s5, s5)
+                ct.mask_inplace(scores, pad, float("-inf"))
+                scores = scores.view(b5 * H, s5, s5)
+                ct.softmax_inplace(scores)
+                ctx = ct.bmm(v, False, scores, False, int8=False).view(b5, d, s5)
+                y = ct.element_add(ct.bmm(Wp["o"], False, ctx, False, int8=True), x)
+                return ffn(y, ln2, W1f, W2f)
+            ms5 = event_ms(lambda: layer(x5), 5, warmup=2)
+            ops5 = 2.0 * b5 * s5 * (4 * d * d + 2 * d * dff) + 2.0 * 2 * b5 * H * s5 * s5 * dh
+            components["config 5 transformer layer (batch 16, seq 1024)"] = {
+                "chain": "LayerNorm -> int8 q,k,v -> fp16 scores -> scale, T5 bias, padding mask, softmax (one launch each) -> fp16 PV -> int8 out-proj + residual -> LayerNorm -> int8 FFN with gelu + residual",
+                "seed": 1005, "avg_ms": round(ms5, 3), "tops_overall": round(ops5 / (ms5 * 1e-3) / 1e12, 1),
+                "tokens_per_s": round(b5 * s5 / (ms5 * 1e-3), 0), "timing": "events, whole chain"}
+            del x5, Wp, W1f, W2f
+            torch.cuda.empty_cache()
+
+    # ---- HBM-bound components ---------------------------------------------------------------
 
     def hbm(name, nbytes, ms, how, shape, traffic):
         gbs = nbytes / (ms * 1e-3) / 1e9
         components[name] = {"shape": shape, "bound": "hbm", "algorithmic_bytes": int(nbytes), "avg_us": round(ms * 1e3, 3),
                             "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                             "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": traffic, "timing": how}
+        if traffic is not None:
+            components[name]["traffic_source"] = OFFLINE_SOURCE["traffic"]
 
     if only in ("", "gemv"):
         # config 2: W int8 [10240,4096], 32 vectors; 8 weight copies (336 MB) rotate so every
@@ -330,29 +452,122 @@ def main():
             "frac": round(2.0 * M * K * N / (ms * 1e-3) / 1e12 / 2500.0, 4), "timing": "events"}
         del Ah, Wh, oh
 
-    # per-op CPU timings beside the three headline components (torch formulations, host cores)
+
+    # ---- what the chip sustains: yardstick kernels and the vendor library on the same shapes ----------
+    if only in ("", "ceilings"):
+        import ctypes
+        from cpm_kernels_amd.build import bench_library_path, build_bench_library
+        if not os.path.exists(bench_library_path()):
+            build_bench_library(verbose=False)
+        cl = ctypes.CDLL(bench_library_path())
+        VP, I32, I64 = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64
+        cl.ceil_mfma_i8.argtypes = [VP, I32, I32, VP, VP]
+        cl.ceil_read.argtypes = [VP, I64, VP, VP]
+        cl.ceil_write.argtypes = [VP, I64, VP]
+        cl.ceil_copy.argtypes = [VP, VP, I64, VP]
+        cl.ceil_copy_segments.argtypes = [VP, VP, I64, I32, I32, VP]
+
+        def ok(rc):
+            assert rc == 0, "yardstick launch failed: %d" % rc
+        ceil = {"note": "kernels of cpm_kernels_amd/bench/ceilings.hip (not part of the library) and, for calibration only, "
+                        "the vendor library through torch; same process, same device, HIP events on the launch stream"}
+        gg = torch.Generator().manual_seed(11)
+        sink = torch.zeros(64, dtype=torch.int32, device=dev)
+        cus = props["compute_units"]
+        iters = 2048
+        mfma_ops = float(cus) * 8 * iters * 16 * 2 * 32 ** 3
+        for label, opnd in (("zero", torch.zeros(12 * 512 * 16, dtype=torch.int8)),
+                            ("random", torch.randint(-127, 128, (12 * 512 * 16,), generator=gg, dtype=torch.int8))):
+            od = opnd.to(dev)
+            ms = event_ms(lambda: ok(cl.ceil_mfma_i8(od.data_ptr(), cus, iters, sink.data_ptr(), st())), 10, warmup=3)
+            ceil["mfma_i8_only_%s_operands" % label] = {"tops": round(mfma_ops / (ms * 1e-3) / 1e12, 1), "us": round(ms * 1e3, 1),
+                                                         "frac_of_published_peak": round(mfma_ops / (ms * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4)}
+        big = torch.randint(-128, 128, (1 << 30,), generator=None, dtype=torch.int8, device=dev)
+        big2 = torch.empty_like(big)
+        nb = big.numel()
+
+        def gbs(nbytes, ms):
+            return {"us": round(ms * 1e3, 2), "gbs": round(nbytes / (ms * 1e-3) / 1e9, 1), "frac_of_published_peak": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
+        ceil["read_1GiB"] = gbs(nb, event_ms(lambda: ok(cl.ceil_read(big.data_ptr(), nb, sink.data_ptr(), st())), 10))
+        ceil["write_1GiB"] = gbs(nb, event_ms(lambda: ok(cl.ceil_write(big2.data_ptr(), nb, st())), 10))
+        ceil["copy_1GiB"] = gbs(2 * nb, event_ms(lambda: ok(cl.ceil_copy(big.data_ptr(), big2.data_ptr(), nb, st())), 10))
+        # the GEMV's traffic: a cold 42 MB read, eight different 42 MB pieces of the buffer in turn (336 MB > Infinity Cache)
+        piece = 10240 * 4096
+        ms, how = graph_ms([(lambda i=i: ok(cl.ceil_read(big.data_ptr() + i * (128 << 20), piece, sink.data_ptr(), st()))) for i in range(8)], 10)
+        ceil["cold_read_42MB (gemv traffic)"] = dict(gbs(piece, ms), timing=how)
+        # the layernorm's traffic and pattern: [8*4096 rows, 1024 bytes] in 128-byte (and wider) column segments, ten buffers in turn
+        for seg in (128, 256, 512, 1024):
+            ms, how = graph_ms([(lambda i=i: ok(cl.ceil_copy_segments(big.data_ptr() + i * (64 << 20), big2.data_ptr(), 8 * 4096, 1024, seg, st())))
+                                for i in range(10)], 10)
+            ceil["tiled_copy_33.5MB_rows_of_1KB_seg%d (layernorm traffic)" % seg] = dict(gbs(2 * 8 * 4096 * 1024, ms), timing=how)
+        # the softmax's: [512*1024 rows, 2048 bytes], tiles of 1024 x 128 bytes as the kernel holds them, and wider segments
+        for seg in (128, 256, 1024):
+            ms = event_ms(lambda: ok(cl.ceil_copy_segments(big.data_ptr(), big2.data_ptr(), 512 * 1024, 2048, seg, st())), 5)
+            ceil["tiled_copy_1GiB_rows_of_2KB_seg%d (softmax traffic)" % seg] = gbs(2 * nb, ms)
+        del big, big2
+        # vendor library, calibration only: torch._int_mm (hipBLASLt) on the north-star and config-1 operands, int32 out
+        try:
+            qa = torch.randint(-127, 128, (M, K), generator=gg, dtype=torch.int8).to(dev)
+            qw = torch.randint(-127, 128, (N, K), generator=gg, dtype=torch.int8).to(dev)
+            ms = event_ms(lambda: torch._int_mm(qa, qw.t()), 20, warmup=5)
+            ceil["vendor_int_mm_north_star_int32_out"] = {"us": round(ms * 1e3, 1), "tops": round(ops / (ms * 1e-3) / 1e12, 1)}
+            o32 = torch.empty((1, M, N), dtype=torch.int32, device=dev)
+            ms = event_ms(lambda: ck.gemm_int8(N, K, M, 1, 1, True, False, qw.data_ptr(), qa.data_ptr(), o32.data_ptr(), st()), 20, warmup=5)
+            ceil["this_library_gemm_int8_same_operands"] = {"us": round(ms * 1e3, 1), "tops": round(ops / (ms * 1e-3) / 1e12, 1)}
+            qa1, qw1 = qa[:512].contiguous(), qw[:4096].contiguous()
+            ms = event_ms(lambda: torch._int_mm(qa1, qw1.t()), 50, warmup=5)
+            ceil["vendor_int_mm_config_1_int32_out"] = {"us": round(ms * 1e3, 2), "tops": round(2.0 * 512 * 4096 * 4096 / (ms * 1e-3) / 1e12, 1)}
+            del qa, qw, o32
+        except Exception as ex:     # pragma: no cover  (calibration only)
+            ceil["vendor_int_mm"] = "unavailable: %s" % ex
+        result["ceilings"] = ceil
+
+    # per-op CPU timings beside the components: the torch formulations the reference's tests compare
+    # with (oracle/formulations.py), on all host cores, full shapes (fewer repetitions for the big ones)
     if not args.no_cpu and only == "":
         from oracle import formulations as F
         torch.set_num_threads(os.cpu_count() or 1)
 
-        def cpu_us(fn, n=3):
-            fn()
+        def cpu_us(fn, n=5, warm=True):
+            if warm:
+                fn()
             ts = []
             for _ in range(n):
                 t0 = time.perf_counter(); fn(); ts.append(time.perf_counter() - t0)
             return round(sorted(ts)[len(ts) // 2] * 1e6, 1)
-        gg = torch.Generator().manual_seed(7)
-        Wq = torch.randint(-127, 128, (10240, 4096), generator=gg).float(); vq = torch.randint(-127, 128, (32, 4096), generator=gg).float()
-        if "gemv_broadcast_mat_int8" in components:
-            components["gemv_broadcast_mat_int8"]["cpu_us"] = cpu_us(lambda: torch.matmul(vq, Wq.t()))
-        xl = torch.randn(8, 4096, 512, generator=gg).half(); wl = torch.ones(4096); bl = torch.zeros(4096)
-        if "layernorm_forward" in components:
-            components["layernorm_forward"]["cpu_us"] = cpu_us(lambda: F.layernorm_dim1(xl, wl, bl, 1e-5))
-        xsm = (torch.randn(16, 1024, 1024, generator=gg) * 4).half()
+
+        def put(name, us, sample):
+            if name in components:
+                components[name]["cpu_us"] = us
+                components[name]["cpu_sample"] = sample
+                components[name]["cpu_cores"] = torch.get_num_threads()
+        gg = torch.Generator().manual_seed(1002)
+        Wq = torch.randint(-127, 128, (10240, 4096), generator=gg, dtype=torch.int8)
+        sm_ = (torch.rand(10240, generator=gg) * 0.009 + 0.001).half()
+        vv = torch.randn(32, 4096, generator=gg).half()
+        Wdeq = (Wq.float() * sm_.float()[:, None]).half()[None]          # the dequantised weight the formulation starts from
+        put("gemv_broadcast_mat_int8", cpu_us(lambda: F.quant_bmm_rowwise(vv[None], Wdeq)),
+            "fp32 fake-quant of 32 vectors and of the dequantised [10240,4096] weight + fp32 matmul, median of 5")
+        del Wq, Wdeq
+        gg = torch.Generator().manual_seed(1003)
+        xl = torch.randn(8, 4096, 512, generator=gg).half()
+        wl = (1 + 0.1 * torch.randn(4096, generator=gg)).half(); bl = (0.1 * torch.randn(4096, generator=gg)).half()
+        put("layernorm_forward", cpu_us(lambda: F.layernorm_dim1(xl, wl, bl, 1e-5)), "full [8,4096,512], fp32 formulation with gamma/beta, median of 5")
+        del xl
         if "softmax_forward" in components:
-            components["softmax_forward"]["cpu_us"] = round(cpu_us(lambda: F.softmax_dim1(xsm)) * 32, 1)
-            components["softmax_forward"]["cpu_sample"] = "1/32 of the tensor timed, scaled"
-        del Wq, vq, xl, xsm
+            xsm = (torch.randn(64, 1024, 1024, generator=gg) * 4).half()
+            kk = torch.arange(1024)[:, None]; qq = torch.arange(1024)[None, :]
+            xsm.masked_fill_((kk > qq)[None], float("-inf"))
+            xsm = xsm.repeat(8, 1, 1)
+            put("softmax_forward", cpu_us(lambda: F.softmax_dim1(xsm), n=1, warm=False), "full [512,1024,1024] causal, torch.softmax on an fp32 copy, one run")
+            del xsm
+        gg = torch.Generator().manual_seed(1004)
+        xg = torch.randn(8, 10240 * 512, generator=gg).half()
+        put("gelu_forward", cpu_us(lambda: F.gelu_tanh(xg), n=3), "full [8, 10240*512], tanh form in fp32, median of 3")
+        del xg
+        pw_ = (torch.randn(64, 32, generator=gg) * 0.02).half()
+        put("position_embedding_forward", cpu_us(lambda: F.position_bias(pw_, 1024, 1024, True, 32, 128), n=3),
+            "64 heads x 1024 x 1024: T5 bucket formula + gather, median of 3")
 
     # ---- CPU baseline: torch formulation of the same step on the host cores ------------------
     cpu = None

@@ -1,0 +1,150 @@
+// What the chip sustains, measured with kernels that do nothing else: the yardsticks bench.py's
+// `--only ceilings` leg reports beside the library's own kernels.  Built into its own shared
+// library (libcpmk_ceilings.so); nothing here is linked into or called by libcpmk_hip.so.
+//
+//   ceil_mfma_i8        v_mfma_i32_32x32x32_i8 back to back from registers, no memory traffic in the
+//                       loop: 8 waves per workgroup, 8 accumulator tiles per wave and two sets of
+//                       operand fragments used in turn -- the register shape of the library's
+//                       256x256 GEMM tile -- so the result is the matrix pipe's rate on the given
+//                       operand bytes (all zero: the clock stays high; random: it drops)
+//   ceil_read / ceil_write / ceil_copy      contiguous 16-byte accesses
+//   ceil_copy_segments  a (rows, row_bytes) matrix copied in tiles of `seg` bytes x many rows, one
+//                       tile per 1024-thread workgroup, all loads of a tile before its stores: the
+//                       access pattern of the dim-1 kernels (layernorm, softmax) without arithmetic
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef int int4_t __attribute__((ext_vector_type(4)));
+typedef int int16_tv __attribute__((ext_vector_type(16)));
+
+namespace {
+
+__global__ __launch_bounds__(512) void k_mfma_i8(const int4_t* __restrict__ operands, int32_t iters, int32_t* sink) {
+    // 12 fragments per lane: two sets of 4 row-operand and 2 column-operand fragments
+    int4_t fp[2][4], fq[2][2];
+    const int t = threadIdx.x;
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) fp[s][i] = operands[(size_t)(s * 6 + i) * 512 + t];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) fq[s][j] = operands[(size_t)(s * 6 + 4 + j) * 512 + t];
+    }
+    int16_tv acc[4][2];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+    for (int32_t it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fq[s][j], fp[s][i], acc[i][j], 0, 0, 0);
+    }
+    int32_t x = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) x ^= acc[i][j][e];
+    if (x == 0x5a5a5a5a) sink[0] = x;       // keeps the loop alive; practically never true
+}
+
+__global__ __launch_bounds__(256) void k_read(const int4_t* __restrict__ p, int64_t n16, int4_t* sink) {
+    int64_t i = (int64_t)blockIdx.x * 1024 + threadIdx.x;
+    int4_t a = {0, 0, 0, 0};
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+        if (i + u * 256 < n16) a += p[i + u * 256];
+    if (a.x == 0x12345678 && a.y == 1) sink[0] = a;
+}
+
+__global__ __launch_bounds__(256) void k_write(int4_t* p, int64_t n16) {
+    int64_t i = (int64_t)blockIdx.x * 1024 + threadIdx.x;
+    const int4_t v = {1, 2, 3, (int)threadIdx.x};
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+        if (i + u * 256 < n16) p[i + u * 256] = v;
+}
+
+__global__ __launch_bounds__(256) void k_copy(const int4_t* __restrict__ p, int4_t* __restrict__ q, int64_t n16) {
+    int64_t i = (int64_t)blockIdx.x * 1024 + threadIdx.x;
+    int4_t v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+        if (i + u * 256 < n16) v[u] = p[i + u * 256];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+        if (i + u * 256 < n16) q[i + u * 256] = v[u];
+}
+
+// Tile = TROWS rows x seg bytes; a workgroup of 1024 threads holds it in 8 x 16 bytes per thread.
+__global__ __launch_bounds__(1024) void k_copy_segments(const char* __restrict__ src, char* __restrict__ dst, int32_t row_bytes,
+                                                        int32_t seg, int32_t tiles_per_row, int32_t tile_rows) {
+    const int ppr = seg / 16;                    // 16-byte pieces per row segment
+    const int rpp = 1024 / ppr;                  // rows per pass of the workgroup
+    const int64_t tr = blockIdx.x / tiles_per_row, tc = blockIdx.x % tiles_per_row;
+    const int64_t base = tr * (int64_t)tile_rows * row_bytes + tc * seg + (threadIdx.x % ppr) * 16;
+    const int r0 = threadIdx.x / ppr;
+    int4_t v[8];
+#pragma unroll
+    for (int p = 0; p < 8; ++p) v[p] = *reinterpret_cast<const int4_t*>(src + base + (int64_t)(r0 + p * rpp) * row_bytes);
+#pragma unroll
+    for (int p = 0; p < 8; ++p) *reinterpret_cast<int4_t*>(dst + base + (int64_t)(r0 + p * rpp) * row_bytes) = v[p];
+}
+
+int status() { return (int)hipGetLastError(); }
+
+}  // namespace
+
+extern "C" {
+
+// operands: 12 * 512 * 16 = 98304 bytes.  One workgroup per compute unit is the caller's choice of `workgroups`.
+// int8 operations done: workgroups * 8 waves * iters * 16 MFMAs * 2 * 32^3.
+int ceil_mfma_i8(const void* operands, int32_t workgroups, int32_t iters, void* sink, void* stream) {
+    if (workgroups < 1 || iters < 0) return 1;
+    hipLaunchKernelGGL(k_mfma_i8, dim3((unsigned)workgroups), dim3(512), 0, (hipStream_t)stream, (const int4_t*)operands, iters,
+                       (int32_t*)sink);
+    return status();
+}
+
+int ceil_read(const void* src, int64_t bytes, void* sink, void* stream) {
+    const int64_t n16 = bytes / 16;
+    hipLaunchKernelGGL(k_read, dim3((unsigned)((n16 + 1023) / 1024)), dim3(256), 0, (hipStream_t)stream, (const int4_t*)src, n16,
+                       (int4_t*)sink);
+    return status();
+}
+
+int ceil_write(void* dst, int64_t bytes, void* stream) {
+    const int64_t n16 = bytes / 16;
+    hipLaunchKernelGGL(k_write, dim3((unsigned)((n16 + 1023) / 1024)), dim3(256), 0, (hipStream_t)stream, (int4_t*)dst, n16);
+    return status();
+}
+
+int ceil_copy(const void* src, void* dst, int64_t bytes, void* stream) {
+    const int64_t n16 = bytes / 16;
+    hipLaunchKernelGGL(k_copy, dim3((unsigned)((n16 + 1023) / 1024)), dim3(256), 0, (hipStream_t)stream, (const int4_t*)src,
+                       (int4_t*)dst, n16);
+    return status();
+}
+
+// rows x row_bytes matrix; seg in {32, 64, 128, 256, 512, 1024} must divide row_bytes; a tile is
+// 131072 / seg rows, which must divide rows.
+int ceil_copy_segments(const void* src, void* dst, int64_t rows, int32_t row_bytes, int32_t seg, void* stream) {
+    if (seg < 32 || seg > 1024 || (seg & (seg - 1)) || row_bytes % seg) return 1;
+    const int32_t tile_rows = 131072 / seg;
+    if (rows % tile_rows) return 1;
+    const int64_t tiles = rows / tile_rows * (row_bytes / seg);
+    if (tiles > 0x7fffffff) return 1;
+    hipLaunchKernelGGL(k_copy_segments, dim3((unsigned)tiles), dim3(1024), 0, (hipStream_t)stream, (const char*)src, (char*)dst,
+                       row_bytes, seg, row_bytes / seg, tile_rows);
+    return status();
+}
+
+}  // extern "C"

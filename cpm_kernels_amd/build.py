@@ -13,8 +13,10 @@ from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
+BENCH_SRC = os.path.join(HERE, "bench")       # yardstick kernels for bench.py; a library of their own
 LIBDIR = os.path.join(HERE, "lib")
 LIBNAME = "libcpmk_hip.so"
+BENCH_LIBNAME = "libcpmk_ceilings.so"
 ARCH = "gfx950"
 
 # No fast-math: correctly rounded fp32 divide is part of the rounding contract.
@@ -39,6 +41,10 @@ def sources():
 
 def library_path():
     return os.path.join(LIBDIR, LIBNAME)
+
+
+def bench_library_path():
+    return os.path.join(LIBDIR, BENCH_LIBNAME)
 
 
 def _run(cmd):
@@ -72,7 +78,21 @@ def build_library(verbose=True, jobs=None):
     os.replace(tmp, library_path())
     if verbose:
         print("[cpmk build] linked %s" % library_path(), flush=True)
+    build_bench_library(verbose)
     return library_path()
+
+
+def build_bench_library(verbose=True):
+    """The yardstick kernels bench.py measures beside the library's own (not part of the product)."""
+    hipcc = find_hipcc()
+    os.makedirs(LIBDIR, exist_ok=True)
+    srcs = sorted(os.path.join(BENCH_SRC, f) for f in os.listdir(BENCH_SRC) if f.endswith(".hip"))
+    tmp = bench_library_path() + ".tmp"
+    _run([hipcc] + HIPCC_FLAGS + ["-shared", "-o", tmp] + srcs)
+    os.replace(tmp, bench_library_path())
+    if verbose:
+        print("[cpmk build] linked %s" % bench_library_path(), flush=True)
+    return bench_library_path()
 
 
 if __name__ == "__main__":
