@@ -706,6 +706,9 @@ static int launch_kmajor(GemmArgs& a, int batch, hipStream_t st) {
 #ifndef CPMK_GEMM_BIG
 #define CPMK_GEMM_BIG 2, 4, 4, 2, 128
 #endif
+#ifndef CPMK_GEMM_BIG_NST
+#define CPMK_GEMM_BIG_NST 2        // ring stages of the 256x256 tile kernel (K-major operands)
+#endif
 
 template <int WR, int WC, int TR, int TC, int BKB, int EPI, bool HALVES, int NST, int LAY = 0>
 static int launch_dma_kernel(const DmaArgs& da, unsigned grid, hipStream_t st) {
@@ -784,7 +787,7 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
         const int64_t big = ceil_div(n, 256) * ceil_div(m, 256) * batch;
         constexpr int EPI = FUSED ? kEpiDequant : kEpiInt32;
         // (a dimension of at most 128 would leave half or more of every 256-wide tile empty)
-        if (big * 4 >= compute_units() * 3 && n > 128 && m > 128) return launch_dma<CPMK_GEMM_BIG, EPI>(a, batch, st);
+        if (big * 4 >= compute_units() * 3 && n > 128 && m > 128) return launch_dma<CPMK_GEMM_BIG, EPI, CPMK_GEMM_BIG_NST>(a, batch, st);
         // 128x128 tiles, or 128x64 when even those leave a quarter of the compute units idle
         const int64_t mid = ceil_div(n, 128) * ceil_div(m, 128) * batch;
         // the smaller tiles finish a slab before a load from L2 returns: four ring stages keep them fed
@@ -796,9 +799,9 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
         (q_kmajor || m % 16 == 0) && (int64_t)n * k < (1ll << 32) && (int64_t)m * k < (1ll << 32)) {
         constexpr int EPI = FUSED ? kEpiDequant : kEpiInt32;
         switch ((p_kmajor ? 0 : 1) | (q_kmajor ? 0 : 2)) {
-            case 1: return launch_dma<CPMK_GEMM_BIG, EPI, 2, 1>(a, batch, st);
-            case 2: return launch_dma<CPMK_GEMM_BIG, EPI, 2, 2>(a, batch, st);
-            default: return launch_dma<CPMK_GEMM_BIG, EPI, 2, 3>(a, batch, st);
+            case 1: return launch_dma<2, 4, 4, 2, 128, EPI, 2, 1>(a, batch, st);
+            case 2: return launch_dma<2, 4, 4, 2, 128, EPI, 2, 2>(a, batch, st);
+            default: return launch_dma<2, 4, 4, 2, 128, EPI, 2, 3>(a, batch, st);
         }
     }
     if (fast) {
@@ -907,7 +910,7 @@ static int gemm_f16_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, in
     if (p_kmajor && q_kmajor && wide && k > 0 && (k % 64 == 0) && aligned16(A) && aligned16(B) &&
         (int64_t)n * k * 2 < (1ll << 32) && (int64_t)m * k * 2 < (1ll << 32)) {
         const int64_t big = ceil_div(n, 256) * ceil_div(m, 256) * batch;
-        if (big * 4 >= compute_units() * 3 && n > 128 && m > 128) return launch_dma<CPMK_GEMM_BIG, kEpiF16>(a, batch, st);
+        if (big * 4 >= compute_units() * 3 && n > 128 && m > 128) return launch_dma<2, 4, 4, 2, 128, kEpiF16>(a, batch, st);
         return launch_dma<2, 2, 2, 2, 128, kEpiF16, CPMK_GEMM_NST_SMALL>(a, batch, st);
     }
     // an operand stored (K, rows): the tile kernel reads it as it lies, with 2-byte LDS reads for the fragments
@@ -916,9 +919,9 @@ static int gemm_f16_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, in
         const int lay = (p_kmajor ? 0 : 1) | (q_kmajor ? 0 : 2);
         const bool low = n <= 64;                // 64 x 256 tiles for few output rows (attention: probabilities x values)
         switch (lay) {
-            case 1: return low ? launch_dma<1, 4, 2, 2, 128, kEpiF16, 3, 1>(a, batch, st) : launch_dma<CPMK_GEMM_BIG, kEpiF16, 2, 1>(a, batch, st);
-            case 2: return low ? launch_dma<1, 4, 2, 2, 128, kEpiF16, 3, 2>(a, batch, st) : launch_dma<CPMK_GEMM_BIG, kEpiF16, 2, 2>(a, batch, st);
-            default: return low ? launch_dma<1, 4, 2, 2, 128, kEpiF16, 3, 3>(a, batch, st) : launch_dma<CPMK_GEMM_BIG, kEpiF16, 2, 3>(a, batch, st);
+            case 1: return low ? launch_dma<1, 4, 2, 2, 128, kEpiF16, 3, 1>(a, batch, st) : launch_dma<2, 4, 4, 2, 128, kEpiF16, 2, 1>(a, batch, st);
+            case 2: return low ? launch_dma<1, 4, 2, 2, 128, kEpiF16, 3, 2>(a, batch, st) : launch_dma<2, 4, 4, 2, 128, kEpiF16, 2, 2>(a, batch, st);
+            default: return low ? launch_dma<1, 4, 2, 2, 128, kEpiF16, 3, 3>(a, batch, st) : launch_dma<2, 4, 4, 2, 128, kEpiF16, 2, 3>(a, batch, st);
         }
     }
     dim3 grid((unsigned)ceil_div(m, 64), (unsigned)ceil_div(n, 64), (unsigned)batch);

@@ -210,7 +210,9 @@ int cpmk_layernorm_step(int32_t batch, int32_t n, const void* mat, void* out, fl
  * than 1024 rows are normalised by teams of workgroups that exchange partial sums through a fixed
  * 2.1 MB array inside the library (2048 packet slots, one per (64-column tile, row part) pair; held
  * by every GPU the library runs on) instead of the shared pool with its completion events: a call
- * that needs more slots -- batch * ceil(m/64) * ceil(n / (n >= 2048 ? 1024 : 512)) > 2048 -- returns
+ * that needs more slots -- batch * ceil(m/64) * ceil(n / R) > 2048, where R is the rows per part that
+ * cpmk_layernorm_forward uses for the shape: 1024 for n > 4096, and for n >= 2048 when
+ * batch * ceil(m/64) * ceil(n/1024) does not exceed the number of compute units, else 512 -- returns
  * CPMK_ETOOBIG.  Makes no hipMalloc/hipFree/event call.  Every call on a GPU uses that GPU's one
  * array: calls that overlap in time on one GPU (two streams, two host threads, a replay of a
  * captured call concurrent with another) race; calls in stream order are safe. */

@@ -49,13 +49,14 @@ def test_shapes_that_need_no_scratch(gpu, shape):
 
 
 def test_sizes_beyond_the_scratch_are_refused(gpu):
-    x = torch.zeros(9, 4096, 4096, dtype=torch.half, device=gpu)       # 9 * 64 * 4 = 2304 slots > 2048
+    x = torch.zeros(17, 4096, 1024, dtype=torch.half, device=gpu)      # 17 * 16 tiles * 8 parts of 512 rows = 2176 slots > 2048
     y = torch.full_like(x, 3.0)
     with pytest.raises(RuntimeError, match="exceeds a size limit"):
-        cpmk.layernorm_forward_noalloc(9, 4096, 4096, x.data_ptr(), y.data_ptr(), 1e-5, 1, stream())
+        cpmk.layernorm_forward_noalloc(17, 4096, 1024, x.data_ptr(), y.data_ptr(), 1e-5, 1, stream())
     torch.cuda.synchronize()
     assert bool((y == 3.0).all()), "a refused call must not write"
-    _pair(gpu, (8, 4096, 4096), 80)                                    # exactly 2048 slots
+    _pair(gpu, (16, 4096, 1024), 80)                                   # exactly 2048 slots
+    _pair(gpu, (1, 16384 - 8192, 2048 * 8), 81)                        # 256 tiles * 8 parts of 1024 rows = 2048 slots
 
 
 def test_graph_capture_and_replay(gpu):
