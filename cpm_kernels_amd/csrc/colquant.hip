@@ -14,8 +14,9 @@ namespace cpmk {
 // exchanges the per-column maxima.  Lane (cg = tid % 8, rg = tid / 8) holds 8 columns of the 8
 // consecutive rows rg*8 .. rg*8+7, so that its int8 results are 8 contiguous bytes in either
 // output layout.
+// (two 512-thread workgroups share a compute unit: at most 128 registers per lane)
 template <int NT>
-__global__ __launch_bounds__(NT) void k_col_quantize_team(int32_t n, int32_t m, int32_t tiles_per_batch, int32_t parts,
+__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void k_col_quantize_team(int32_t n, int32_t m, int32_t tiles_per_batch, int32_t parts,
                                                           const half_t* __restrict__ mat, half_t* __restrict__ scale,
                                                           int8_t* __restrict__ out, int transposed, XchLaunch xl) {
     constexpr int LPR = 8, R = 8, COLS = 64, ROWS = NT / LPR * R;
@@ -80,13 +81,31 @@ __global__ __launch_bounds__(NT) void k_col_quantize_team(int32_t n, int32_t m, 
     if (part == 0 && rg == 0 && col0 < m) *reinterpret_cast<half8_t*>(scale + (int64_t)b * m + col0) = sh;
 
     uint32_t q[R][2];       // [row p][columns 0-3 | 4-7], one byte each
+    bool normal = true;
 #pragma unroll
-    for (int p = 0; p < R; ++p) {
-        int32_t t[8];
+    for (int e = 0; e < 8; ++e) normal = normal && scale_is_normal(sh[e]);
+    if (__builtin_amdgcn_ballot_w64(!normal) == 0) {    // every scale of the wave's columns is a normal number: the short rounding sequence
 #pragma unroll
-        for (int e = 0; e < 8; ++e) t[e] = quant_i8_rcp((float)v[p][e], s[e], y[e]);
-        q[p][0] = pack4_i8(t[0], t[1], t[2], t[3]);
-        q[p][1] = pack4_i8(t[4], t[5], t[6], t[7]);
+        for (int p = 0; p < R; ++p) {
+            uint32_t t[8];
+            int4_t vp = __builtin_bit_cast(int4_t, v[p]);
+            asm volatile("" : "+v"(vp));             // keeps the fp32 conversions of the two paths apart (hoisted above the branch they hold 64 registers)
+            const half8_t vh = __builtin_bit_cast(half8_t, vp);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) t[e] = quant_i8_own_scale_bits((float)vh[e], s[e], y[e]);
+            q[p][0] = pack4_i8((int32_t)t[0], (int32_t)t[1], (int32_t)t[2], (int32_t)t[3]);
+            q[p][1] = pack4_i8((int32_t)t[4], (int32_t)t[5], (int32_t)t[6], (int32_t)t[7]);
+            __builtin_amdgcn_sched_barrier(0);      // one row at a time: interleaving all 64 elements costs registers
+        }
+    } else {
+#pragma unroll
+        for (int p = 0; p < R; ++p) {
+            int32_t t[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) t[e] = quant_i8_rcp((float)v[p][e], s[e], y[e]);
+            q[p][0] = pack4_i8(t[0], t[1], t[2], t[3]);
+            q[p][1] = pack4_i8(t[4], t[5], t[6], t[7]);
+        }
     }
     if (col0 < m) {
         if (!transposed) {

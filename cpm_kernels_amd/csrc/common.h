@@ -106,6 +106,27 @@ __device__ inline int32_t quant_i8_rcp(float x, float s, float y) {
     return min(max(n, -128), 127);
 }
 
+// The short form for a scale that comes from the data it divides and is a normal fp16 number:
+//     s = fp16(absmax / 127),  |x| <= absmax   =>   |x / s| <= 127 * (1 + 2^-11),
+// so nothing saturates and the residual is always finite.  q + 1.5 * 2^23 lands in [2^23, 2^24),
+// where the fp32 grid is the integers: the one round-to-nearest-even of that addition is rint(q), and
+// the low byte of the sum's bit pattern is the two's-complement int8.  A NaN element (which the
+// absmax ignores) propagates as a quiet NaN whose low byte is 0, the value the long form gives it.
+// Equality with quant_i8 for every such (absmax, x) pair is proven by enumeration in
+// tests/native/fused_round_check.c.  Returns the fp32 bit pattern; its low byte is the result.
+__device__ inline bool scale_is_normal(half_t sh) {
+    const uint16_t b = __builtin_bit_cast(uint16_t, sh);
+    return b >= 0x0400u && b <= 0x7bffu;
+}
+__device__ inline uint32_t quant_i8_own_scale_bits(float x, float s, float y) {
+    const float q0 = x * y;
+    const float r = __builtin_fmaf(-s, q0, x);
+    const float q1 = __builtin_fmaf(r, y, q0);
+    float t = q1 + 12582912.0f;
+    asm("" : "+v"(t));          // the sum must exist as a rounded fp32 number
+    return __builtin_bit_cast(uint32_t, t);
+}
+
 // Low bytes of four integers (each already within int8 range) into one dword: three byte
 // permutes.  v_perm_b32 selector bytes 0-3 pick from the second operand, 4-7 from the first, 0x0c is zero.
 __device__ inline uint32_t pack4_i8(int32_t a, int32_t b, int32_t c, int32_t d) {

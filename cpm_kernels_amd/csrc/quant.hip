@@ -245,17 +245,34 @@ __global__ __launch_bounds__(256) void k_rows(RowsArgs a) {
         if (QUANT) {
             const float s = (float)sh, y = 1.0f / s;
             uint2_t* o8 = reinterpret_cast<uint2_t*>((second ? a.out1 : a.out0) + lrow * m);
+            if (scale_is_normal(sh)) {       // (the same for the whole wave) the short rounding sequence
 #pragma unroll
-            for (int i = 0; i < NV; ++i) {
-                const int j = lane + i * 64;
-                if (j < m8) {
-                    int32_t q[8];
+                for (int i = 0; i < NV; ++i) {
+                    const int j = lane + i * 64;
+                    uint32_t q[8];
+                    int4_t ci = __builtin_bit_cast(int4_t, cur[i]);
+                    asm volatile("" : "+v"(ci));     // keeps the fp32 conversions of the two paths apart (hoisted above the branch they hold NV * 8 registers)
+                    const half8_t ch = __builtin_bit_cast(half8_t, ci);
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) q[e] = quant_i8_rcp((float)cur[i][e], s, y);
+                    for (int e = 0; e < 8; ++e) q[e] = quant_i8_own_scale_bits((float)ch[e], s, y);
                     uint2_t w;
-                    w.x = pack4_i8(q[0], q[1], q[2], q[3]);
-                    w.y = pack4_i8(q[4], q[5], q[6], q[7]);
-                    o8[j] = w;
+                    w.x = pack4_i8((int32_t)q[0], (int32_t)q[1], (int32_t)q[2], (int32_t)q[3]);
+                    w.y = pack4_i8((int32_t)q[4], (int32_t)q[5], (int32_t)q[6], (int32_t)q[7]);
+                    if (j < m8) o8[j] = w;
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < NV; ++i) {
+                    const int j = lane + i * 64;
+                    if (j < m8) {
+                        int32_t q[8];
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) q[e] = quant_i8_rcp((float)cur[i][e], s, y);
+                        uint2_t w;
+                        w.x = pack4_i8(q[0], q[1], q[2], q[3]);
+                        w.y = pack4_i8(q[4], q[5], q[6], q[7]);
+                        o8[j] = w;
+                    }
                 }
             }
         }

@@ -383,3 +383,19 @@ def test_reciprocal_rounding_equals_divide_rounding_exhaustively(tmp_path):
     r = subprocess.run([exe], capture_output=True, text=True)       # the whole grid: seconds on a few cores
     assert r.returncode == 0, r.stdout + r.stderr
     assert r.stdout.startswith("4294967296 pairs, 0 mismatches"), r.stdout
+
+
+def test_short_rounding_of_the_fused_quantisers_exhaustively(tmp_path):
+    """The fused quantisers round a row (column) whose scale is a normal fp16 number through
+    y = 1/s, one residual step and the low byte of q + 1.5 * 2^23; tests/native/fused_round_check.c
+    enumerates every (absmax, x) pair such a row can hold -- about 10^9 -- against the
+    divide-then-round of cuda/gemm.cu:16 with the same IEEE operations on the host."""
+    import os, shutil, subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    src = os.path.join(os.path.dirname(os.path.abspath(__file__)), "native", "fused_round_check.c")
+    exe = str(tmp_path / "fused_round_check")
+    subprocess.run(["gcc", "-O2", "-ffp-contract=off", "-mfma", "-msse4.1", "-fopenmp", src, "-o", exe, "-lm"], check=True)
+    r = subprocess.run([exe], capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert r.stdout.startswith("23568 rows, 989078256 pairs, 0 mismatches"), r.stdout
