@@ -73,6 +73,29 @@ __device__ inline float block_sum(float v, float* red) {
     return r;
 }
 
+// ---- |x| maxima on packed halves ---------------------------------------------------------
+// Magnitudes of fp16 numbers that are not NaN order like their bit patterns with the sign cleared,
+// so a running maximum needs one AND and one packed 16-bit integer maximum per two elements.  A NaN
+// element has the largest patterns of all (above 0x7c00, infinity): a result above 0x7c00 says that
+// the data held one, and the caller repeats the maximum in floating point, which skips NaN elements
+// like the reference's fmaxf (cuda/gemm.cu:68-72).
+typedef uint16_t ushort8_t __attribute__((ext_vector_type(8)));
+__device__ inline ushort8_t absbits_max(ushort8_t m, half8_t x) {
+    const uint4_t b = __builtin_bit_cast(uint4_t, x) & 0x7fff7fffu;
+    return __builtin_elementwise_max(m, __builtin_bit_cast(ushort8_t, b));
+}
+__device__ inline uint32_t absbits_max_of(ushort8_t m) {
+    uint32_t r = 0;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r = max(r, (uint32_t)m[e]);
+    return r;
+}
+__device__ inline uint32_t wave_max_u32(uint32_t v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = max(v, (uint32_t)__shfl_xor((int)v, o, kWave));
+    return v;
+}
+
 // ---- quantisation arithmetic ---------------------------------------------------------
 // absmax/127 rounded to fp16.  The reference divides in double and converts
 // double->float->half (cuda/gemm.cu:74); for every fp16 magnitude that equals the
@@ -119,7 +142,7 @@ __device__ inline bool scale_is_normal(half_t sh) {
     return b >= 0x0400u && b <= 0x7bffu;
 }
 __device__ inline uint32_t quant_i8_own_scale_bits(float x, float s, float y) {
-    const float q0 = x * y;
+    const float q0 = __builtin_fmaf(x, y, 0.0f);     // x * y (the sign of a zero does not matter below); as an fma the fp16 -> fp32 conversion of x folds into the instruction
     const float r = __builtin_fmaf(-s, q0, x);
     const float q1 = __builtin_fmaf(r, y, q0);
     float t = q1 + 12582912.0f;

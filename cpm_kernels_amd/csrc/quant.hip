@@ -204,8 +204,9 @@ struct RowsArgs {
     int32_t m;
 };
 
+// (the launcher counts on 8 resident workgroups per compute unit up to NV = 8, 4 beyond)
 template <int NV, bool QUANT>
-__global__ __launch_bounds__(256) void k_rows(RowsArgs a) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NV <= 8 ? 8 : 4))) void k_rows(RowsArgs a) {
     const int lane = threadIdx.x & 63;
     const int64_t nw = (int64_t)gridDim.x * 4;
     const int64_t rows = a.rows0 + a.rows1;
@@ -228,16 +229,27 @@ __global__ __launch_bounds__(256) void k_rows(RowsArgs a) {
     load(cur, row);
     while (true) {
         const int64_t next = row + nw;
-        // |x| maxima on the packed halves (exact), then across the wave
-        half8_t hm;
+        // |x| maxima on the packed halves as integers, then across the wave
+        ushort8_t um = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-        for (int e = 0; e < 8; ++e) hm[e] = (half_t)0.0f;
+        for (int i = 0; i < NV; ++i) um = absbits_max(um, cur[i]);
+        const uint32_t ub = wave_max_u32(absbits_max_of(um));
+        float mx = (float)__builtin_bit_cast(half_t, (uint16_t)ub);
+        if (ub > 0x7c00u) {      // (the same for the whole wave) a NaN in the row: the maximum that skips NaN elements
+            half8_t hm;
 #pragma unroll
-        for (int i = 0; i < NV; ++i) hm = __builtin_elementwise_max(hm, __builtin_elementwise_abs(cur[i]));
-        float mx = 0.0f;
+            for (int e = 0; e < 8; ++e) hm[e] = (half_t)0.0f;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) mx = fmaxf((float)hm[e], mx);
-        mx = wave_max(mx);
+            for (int i = 0; i < NV; ++i) {
+                int4_t ci = __builtin_bit_cast(int4_t, cur[i]);
+                asm volatile("" : "+v"(ci));         // nothing of this rare path is to be computed ahead of the branch
+                hm = __builtin_elementwise_max(hm, __builtin_elementwise_abs(__builtin_bit_cast(half8_t, ci)));
+            }
+            mx = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) mx = fmaxf((float)hm[e], mx);
+            mx = wave_max(mx);
+        }
         const half_t sh = scale_from_absmax(mx);
         const bool second = row >= a.rows0;
         const int64_t lrow = second ? row - a.rows0 : row;

@@ -103,10 +103,15 @@ static int8_t quant(float x, float s) {
  * half).  Restated literally. */
 static uint16_t scale_of(float mx) { return f2h((float)((double)mx / 127.0)); }
 
+/* The device's fmaxf returns the other operand for ANY NaN operand (cuda/gemm.cu:68-72 relies on
+ * it: a NaN element takes no part in the maximum).  The host's fmaxf does so for quiet NaNs only
+ * and hands a signalling one on as NaN, so the NaN test is spelled out here. */
+static float max_skip_nan(float v, float mx) { return (v != v) ? mx : fmaxf(v, mx); }
+
 void o_gemm_calc_scale(int32_t batch, int32_t n, int32_t m, const uint16_t* mat, uint16_t* out) {
     for (int64_t r = 0; r < (int64_t)batch * n; ++r) {
         float mx = 0.0f;
-        for (int32_t j = 0; j < m; ++j) mx = fmaxf(fabsf(h2f(mat[r * m + j])), mx);
+        for (int32_t j = 0; j < m; ++j) mx = max_skip_nan(fabsf(h2f(mat[r * m + j])), mx);
         out[r] = scale_of(mx);
     }
 }
@@ -116,7 +121,7 @@ void o_gemm_calc_scale_transpose(int32_t batch, int32_t n, int32_t m, const uint
     for (int32_t b = 0; b < batch; ++b)
         for (int32_t j = 0; j < m; ++j) {
             float mx = 0.0f;
-            for (int32_t i = 0; i < n; ++i) mx = fmaxf(fabsf(h2f(mat[((int64_t)b * n + i) * m + j])), mx);
+            for (int32_t i = 0; i < n; ++i) mx = max_skip_nan(fabsf(h2f(mat[((int64_t)b * n + i) * m + j])), mx);
             out[(int64_t)b * m + j] = scale_of(mx);
         }
 }

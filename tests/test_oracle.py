@@ -399,3 +399,20 @@ def test_short_rounding_of_the_fused_quantisers_exhaustively(tmp_path):
     r = subprocess.run([exe], capture_output=True, text=True)
     assert r.returncode == 0, r.stdout + r.stderr
     assert r.stdout.startswith("23568 rows, 989078256 pairs, 0 mismatches"), r.stdout
+
+
+def test_calc_scale_skips_nan_elements_of_either_kind():
+    """cuda/gemm.cu:68-72 takes the maximum with the device's fmaxf, which drops any NaN operand:
+    the scale is that of the row with its NaN elements, quiet or signalling, replaced by zeros."""
+    rng = np.random.default_rng(3)
+    x = (rng.standard_normal((2, 6, 40)) * 3).astype(np.float16)
+    b = x.view(np.uint16)
+    for (i, j, k, pat) in ((0, 0, 0, 0x7e00), (0, 1, 5, 0x7c01), (1, 2, 39, 0xfdff), (1, 5, 7, 0xffff)):
+        b[i, j, k] = pat
+    a = np.abs(x.astype(np.float32))
+    want = (np.where(np.isnan(a), np.float32(0), a).max(axis=-1) / np.float32(127)).astype(np.float16)
+    assert_bits_equal(oracle.gemm_calc_scale(x), want, "row scales with NaN elements")
+    xt = np.ascontiguousarray(x.transpose(0, 2, 1))
+    assert_bits_equal(oracle.gemm_calc_scale_transpose(xt), want, "column scales with NaN elements")
+    q = oracle.gemm_round(x, want)
+    assert q[0, 0, 0] == 0 and q[0, 1, 5] == 0 and q[1, 2, 39] == 0 and q[1, 5, 7] == 0

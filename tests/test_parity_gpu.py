@@ -148,6 +148,39 @@ def test_quantize_pair(gpu, rows0, rows1, m):
             assert_bits_equal(to_np(q[i]), oracle.gemm_round(xs[i][None], s_ref)[0], "pair int8 %d" % i)
 
 
+def test_quantisers_skip_nan_elements(gpu):
+    """A NaN element (quiet or signalling) takes no part in a row's or a column's absmax -- the
+    reference's fmaxf drops it (cuda/gemm.cu:68-72) -- and rounds to 0; the other elements of the
+    row are quantised as if it were not there.  Rows with normal and with subnormal scales."""
+    _name("quantisers with NaN elements")
+    rng = np.random.default_rng(77)
+    n, m = 40, 4096
+    x = rand_half(rng, (1, n, m), 2.0)
+    x[0, 5] *= np.float16(1e-4)                                   # subnormal scale
+    bits_ = x.view(np.uint16)
+    for r, c, pat in ((0, 0, 0x7e00), (3, 100, 0x7c01), (5, 7, 0xfe00), (9, 4095, 0xfdff), (9, 1, 0x7fff), (20, 2048, 0x7d55)):
+        bits_[0, r, c] = pat
+    xd = to_gpu(x)
+    s_ref = oracle.gemm_calc_scale(x); q_ref = oracle.gemm_round(x, s_ref)
+    assert np.isfinite(s_ref.astype(np.float32)).all()
+    sd = torch.empty((1, n), dtype=torch.half, device=gpu); qd = torch.empty((1, n, m), dtype=torch.int8, device=gpu)
+    ck.gemm_calc_scale(1, n, m, xd.data_ptr(), sd.data_ptr(), stream())
+    assert_bits_equal(to_np(sd), s_ref, "calc_scale with NaN elements")
+    sd.zero_()
+    ck.gemm_quantize(1, n, m, xd.data_ptr(), sd.data_ptr(), qd.data_ptr(), False, stream())
+    assert_bits_equal(to_np(sd), s_ref, "gemm_quantize scale with NaN elements")
+    assert_bits_equal(to_np(qd), q_ref, "gemm_quantize int8 with NaN elements")
+    assert to_np(qd)[0, 3, 100] == 0 and to_np(qd)[0, 9, 4095] == 0
+    # columns: the same tensor transposed
+    xt = np.ascontiguousarray(x.transpose(0, 2, 1)); xtd = to_gpu(xt)
+    for tr in (False, True):
+        sc = torch.zeros((1, n), dtype=torch.half, device=gpu)
+        qc = torch.zeros((1, n, m) if tr else (1, m, n), dtype=torch.int8, device=gpu)
+        ck.gemm_quantize_cols(1, m, n, xtd.data_ptr(), sc.data_ptr(), qc.data_ptr(), tr, stream())
+        assert_bits_equal(to_np(sc), s_ref, "quantize_cols scale with NaN elements")
+        assert_bits_equal(to_np(qc), q_ref if tr else np.ascontiguousarray(q_ref.transpose(0, 2, 1)), "quantize_cols int8 with NaN elements (transposed=%s)" % tr)
+
+
 def test_round_unaligned_views(gpu):
     """Pointers that are only 2-byte aligned take the scalar kernels."""
     _name("round unaligned")
