@@ -40,9 +40,17 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         if (row0 + p < n && col0 < m)
             v[p] = *reinterpret_cast<const half8_t*>(mat + boff + ((uint32_t)(row0 + p) * (uint32_t)m + (uint32_t)col0));
     }
-    half8_t hm = __builtin_elementwise_abs(v[0]);
+    // |x| maxima of the lane's 8 columns as integers; a NaN among them (rare) repeats the maximum in
+    // floating point, which skips NaN elements
+    ushort8_t um = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-    for (int p = 1; p < R; ++p) hm = __builtin_elementwise_max(hm, __builtin_elementwise_abs(v[p]));
+    for (int p = 0; p < R; ++p) um = absbits_max(um, v[p]);
+    half8_t hm = __builtin_bit_cast(half8_t, um);
+    if (absbits_max_of(um) > 0x7c00u) {
+        hm = __builtin_elementwise_abs(v[0]);
+#pragma unroll
+        for (int p = 1; p < R; ++p) hm = __builtin_elementwise_max(hm, __builtin_elementwise_abs(v[p]));
+    }
     float mx[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) mx[e] = (float)hm[e];
