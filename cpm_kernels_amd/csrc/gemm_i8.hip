@@ -616,14 +616,14 @@ __global__ __launch_bounds__(WR* WC * 64) void k_gemm_dma(DmaArgs da) {
 // 4x4 block with v_dot4_i32_i8.  Element-wise guarded loads handle every layout and size.
 // ---------------------------------------------------------------------------------------
 template <bool FUSED>
-__global__ __launch_bounds__(256) void k_gemm_generic(GemmArgs a, int p_kmajor, int q_kmajor) {
+__global__ __launch_bounds__(256) void k_gemm_generic(GemmArgs a, int p_kmajor, int q_kmajor, int32_t row_base) {
     constexpr int T = 64, GK = 32, LD = GK + 4;
     __shared__ __attribute__((aligned(4))) int8_t sP[T * LD];
     __shared__ __attribute__((aligned(4))) int8_t sQ[T * LD];
     const int b = blockIdx.z;
     const int8_t* P = a.P + (int64_t)b * a.strideP;
     const int8_t* Q = a.Q + (int64_t)b * a.strideQ;
-    const int32_t j0 = blockIdx.y * T, i0 = blockIdx.x * T;
+    const int32_t j0 = row_base + blockIdx.y * T, i0 = blockIdx.x * T;
     const int tid = threadIdx.x, ty = tid >> 4, tx = tid & 15;
     int32_t acc[4][4];
 #pragma unroll
@@ -809,10 +809,14 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
         if (t256 >= 256) return launch_kmajor<2, 2, 4, 2, FUSED>(a, batch, st);
         return launch_kmajor<2, 2, 2, 2, FUSED>(a, batch, st);
     }
-    dim3 grid((unsigned)ceil_div(m, 64), (unsigned)ceil_div(n, 64), (unsigned)batch);
-    if (grid.y > 65535) return CPMK_ETOOBIG;
-    hipLaunchKernelGGL((k_gemm_generic<FUSED>), grid, dim3(256), 0, st, a, (int)p_kmajor, (int)q_kmajor);
-    return launch_status();
+    // output rows are the grid's y dimension (65535 tiles of 64 rows): taller products go out in several launches
+    for (int64_t r0 = 0; r0 < n; r0 += 65535ll * 64) {
+        const int64_t nr = n - r0 < 65535ll * 64 ? n - r0 : 65535ll * 64;
+        dim3 grid((unsigned)ceil_div(m, 64), (unsigned)ceil_div(nr, 64), (unsigned)batch);
+        hipLaunchKernelGGL((k_gemm_generic<FUSED>), grid, dim3(256), 0, st, a, (int)p_kmajor, (int)q_kmajor, (int32_t)r0);
+        if (int e = launch_status()) return e;
+    }
+    return 0;
 }
 
 // ---------------------------------------------------------------------------------------
@@ -820,7 +824,7 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
 // stage, 256 threads each computing a 4x4 block.  The K-major, k % 64 == 0 case runs on the
 // tile kernel above with the fp16 MFMA instead.
 // ---------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void k_gemm_f16_generic(GemmArgs a, int p_kmajor, int q_kmajor) {
+__global__ __launch_bounds__(256) void k_gemm_f16_generic(GemmArgs a, int p_kmajor, int q_kmajor, int32_t row_base) {
     constexpr int T = 64, GK = 16, LD = GK + 2;
     __shared__ half_t sP[T * LD];
     __shared__ half_t sQ[T * LD];
@@ -828,7 +832,7 @@ __global__ __launch_bounds__(256) void k_gemm_f16_generic(GemmArgs a, int p_kmaj
     const int32_t k = a.k >> 1;                        // a.k is the row length in bytes
     const half_t* P = reinterpret_cast<const half_t*>(a.P + (int64_t)b * a.strideP);
     const half_t* Q = reinterpret_cast<const half_t*>(a.Q + (int64_t)b * a.strideQ);
-    const int32_t j0 = blockIdx.y * T, i0 = blockIdx.x * T;
+    const int32_t j0 = row_base + blockIdx.y * T, i0 = blockIdx.x * T;
     const int tid = threadIdx.x, ty = tid >> 4, tx = tid & 15;
     float acc[4][4];
 #pragma unroll
@@ -924,10 +928,13 @@ static int gemm_f16_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, in
             default: return low ? launch_dma<1, 4, 2, 2, 128, kEpiF16, 3, 3>(a, batch, st) : launch_dma<2, 4, 4, 2, 128, kEpiF16, 2, 3>(a, batch, st);
         }
     }
-    dim3 grid((unsigned)ceil_div(m, 64), (unsigned)ceil_div(n, 64), (unsigned)batch);
-    if (grid.y > 65535) return CPMK_ETOOBIG;
-    hipLaunchKernelGGL(k_gemm_f16_generic, grid, dim3(256), 0, st, a, (int)p_kmajor, (int)q_kmajor);
-    return launch_status();
+    for (int64_t r0 = 0; r0 < n; r0 += 65535ll * 64) {        // (rows beyond the grid's y dimension: several launches)
+        const int64_t nr = n - r0 < 65535ll * 64 ? n - r0 : 65535ll * 64;
+        dim3 grid((unsigned)ceil_div(m, 64), (unsigned)ceil_div(nr, 64), (unsigned)batch);
+        hipLaunchKernelGGL(k_gemm_f16_generic, grid, dim3(256), 0, st, a, (int)p_kmajor, (int)q_kmajor, (int32_t)r0);
+        if (int e = launch_status()) return e;
+    }
+    return 0;
 }
 
 }  // namespace cpmk

@@ -32,27 +32,31 @@ __device__ inline int32_t bucket_of(int32_t rel, int32_t num_buckets, int32_t ma
 // out[h, k, q] = weight[h, bucket(q - k)].  The bias is Toeplitz: for one head it depends on
 // q - k only.  A workgroup builds that head's diagonal vector d[r], r = q - k + (key_len-1),
 // for the q - k range of its KR key rows in LDS and then streams the rows out.
-// grid = (ceil(key_len / KR), num_heads)
+// Long rows are cut into pieces of at most QC queries, each with a diagonal of its own.
+// grid = (ceil(key_len / KR), num_heads, ceil(query_len / QC))
 constexpr int KR = 16;
+constexpr int QC = 16384;
 __global__ __launch_bounds__(256) void k_position_forward(int32_t query_len, int32_t key_len, int32_t num_buckets,
                                                           int32_t max_distance, const int32_t* __restrict__ table,
                                                           const half_t* __restrict__ weight, half_t* out,
                                                           int bidirectional) {
-    extern __shared__ half_t diag[];          // query_len + KR - 1 entries
+    extern __shared__ half_t diag[];          // min(query_len, QC) + KR - 1 entries
     const int32_t k0 = blockIdx.x * KR;
     const int32_t h = blockIdx.y;
+    const int32_t q0 = blockIdx.z * QC;
+    const int32_t nq = min(QC, query_len - q0);
     const int32_t kend = min(k0 + KR, key_len);
-    // diag[t] holds rel = t - (kend - 1 - k0) + ... : rel ranges over [-(kend-1), query_len-1-k0]
-    const int32_t rel_min = -(kend - 1);
-    const int32_t nd = query_len + (kend - k0) - 1;
+    // diag[t] holds the weight of rel = rel_min + t; rel = q - k ranges over [q0 - (kend-1), q0 + nq - 1 - k0]
+    const int32_t rel_min = q0 - (kend - 1);
+    const int32_t nd = nq + (kend - k0) - 1;
     const half_t* wh = weight + (int64_t)h * num_buckets;
     for (int32_t t = threadIdx.x; t < nd; t += 256)
         diag[t] = wh[bucket_of(rel_min + t, num_buckets, max_distance, table, bidirectional)];
     __syncthreads();
     for (int32_t k = k0; k < kend; ++k) {
-        half_t* orow = out + ((int64_t)h * key_len + k) * query_len;
-        const int32_t shift = -k - rel_min;    // q - k - rel_min = q + shift
-        for (int32_t q = threadIdx.x; q < query_len; q += 256) orow[q] = diag[q + shift];
+        half_t* orow = out + ((int64_t)h * key_len + k) * query_len + q0;
+        const int32_t shift = q0 - k - rel_min;    // q - k - rel_min = (q - q0) + shift
+        for (int32_t q = threadIdx.x; q < nq; q += 256) orow[q] = diag[q + shift];
     }
 }
 
@@ -90,14 +94,17 @@ int cpmk_position_embedding_forward(int32_t query_len, int32_t key_len, int32_t 
     clear_stale_error();
     if (query_len < 0 || key_len < 0 || num_heads < 0 || num_buckets <= 0 || max_distance <= 0) return CPMK_EBADARG;
     if ((int64_t)query_len * key_len * num_heads == 0) return 0;
-    if (num_heads > 65535) return CPMK_ETOOBIG;
-    const size_t smem = (size_t)(query_len + KR - 1) * sizeof(half_t);
-    if (smem > 64 * 1024) return CPMK_ETOOBIG;     // query_len up to 32752
-    dim3 grid((unsigned)ceil_div(key_len, KR), (unsigned)num_heads);
-    hipLaunchKernelGGL(k_position_forward, grid, dim3(256), smem, (hipStream_t)stream, query_len, key_len,
-                       num_buckets, max_distance, (const int32_t*)position_mapping, (const half_t*)weight,
-                       (half_t*)out, bidirectional);
-    return launch_status();
+    const size_t smem = (size_t)((query_len < QC ? query_len : QC) + KR - 1) * sizeof(half_t);
+    // heads are the grid's y dimension (at most 65535): more go out in several launches
+    for (int64_t h0 = 0; h0 < num_heads; h0 += 65535) {
+        const int64_t nh = num_heads - h0 < 65535 ? num_heads - h0 : 65535;
+        dim3 grid((unsigned)ceil_div(key_len, KR), (unsigned)nh, (unsigned)ceil_div(query_len, QC));
+        hipLaunchKernelGGL(k_position_forward, grid, dim3(256), smem, (hipStream_t)stream, query_len, key_len,
+                           num_buckets, max_distance, (const int32_t*)position_mapping,
+                           (const half_t*)weight + h0 * num_buckets, (half_t*)out + h0 * key_len * query_len, bidirectional);
+        if (int e = launch_status()) return e;
+    }
+    return 0;
 }
 
 int cpmk_position_embedding_step(int32_t query_pos, int32_t key_len, int32_t num_buckets, int32_t max_distance,

@@ -15,11 +15,10 @@
  *   - Sizes: element counts and byte offsets are 64-bit throughout (tensors beyond 2^31
  *     elements work), and batches of any int32 size are split over launches where a kernel
  *     indexes the batch with a grid dimension.  CPMK_ETOOBIG remains for: a matrix dimension
- *     beyond 4 194 240 (65535 tiles of 64) in the transposes, the embedding kernels and the
- *     general GEMM kernels; k above 2^30 in the fp16 GEMM; more than 524 280 vectors in the
- *     general fp16 broadcast GEMV; more than 2^31-1 rows in the elementwise and row-quantising
- *     training kernels; position bias with more than 65535 heads, a query_len above 32752
- *     (forward) or more than 8192 buckets (backward).
+ *     beyond 4 194 240 (65535 tiles of 64) in the transposes and the embedding kernels; k above
+ *     2^30 in the fp16 GEMM; more than 524 280 vectors in the general fp16 broadcast GEMV; more
+ *     than 2^31-1 rows in the elementwise and row-quantising training kernels; more than 8192
+ *     buckets in the position-bias gradient.
  *
  * Each declaration cites the reference interface it replaces as
  * <python wrapper file:line> / <CUDA kernel file:line> relative to the reference tree.

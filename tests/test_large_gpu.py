@@ -271,3 +271,39 @@ def test_training_and_helper_kernels_beyond_2_31_elements(gpu):
         assert_close_fp16(to_np(mean[i:i + 1]), m_ref, rtol=1e-3, atol=1e-4, what="forward_mv mean, batch %d" % i)
         assert_close_fp16(to_np(grad[i:i + 1]), ot.layernorm_backward_mv(to_np(x[i:i + 1]), to_np(gsrc[i:i + 1]), to_np(mean[i:i + 1]), to_np(var[i:i + 1])),
                           rtol=2e-3, atol=1e-3, what="backward_mv batch %d" % i)
+
+
+def test_position_bias_rows_longer_than_one_diagonal(gpu):
+    """query_len beyond what one LDS diagonal holds (16384 queries): rows are written in pieces, each
+    with its own diagonal.  The reference has no such limit (cuda/position_bucket.cu:25-54)."""
+    print("case position bias, query_len 40000", flush=True)
+    rng = np.random.default_rng(9)
+    for (ql, kl, bidi) in ((40000, 19, True), (16385, 33, False), (32768, 5, True)):
+        table = oracle.position_embedding_init(32, 128, bidi)
+        w = (rng.standard_normal((3, 32)) * 0.02).astype(np.float16)
+        td = torch.from_numpy(table).cuda(); wd = torch.from_numpy(w).cuda()
+        out = torch.full((3, kl, ql), 7.0, dtype=torch.half, device=gpu)
+        ck.position_embedding_forward(ql, kl, 32, 128, 3, td.data_ptr(), wd.data_ptr(), out.data_ptr(), bidi, stream())
+        ref = oracle.position_embedding_forward(ql, kl, 32, 128, table, w, bidi)
+        assert_bits_equal(to_np(out), ref, "position bias query_len %d" % ql)
+
+
+def test_general_gemm_with_more_rows_than_a_grid_dimension(gpu):
+    """The general (any-shape) product kernels index 64-row tiles with the grid's y dimension: more than
+    65535 x 64 output rows go out in several launches.  K = 4 (int8) and 2 (fp16) keep the tensors small;
+    rows on either side of the boundary and at the end are compared with exact products."""
+    print("case general gemm, 4194340 output rows", flush=True)
+    n, m = 65535 * 64 + 100, 4
+    g = torch.Generator().manual_seed(12)
+    B = torch.randint(-127, 128, (1, n, 4), generator=g, dtype=torch.int8).to(gpu)        # row operand (n, k)
+    A = torch.randint(-127, 128, (1, m, 4), generator=g, dtype=torch.int8).to(gpu)        # column operand (m, k)
+    out = torch.full((1, n, m), -1, dtype=torch.int32, device=gpu)
+    ck.gemm_int8(m, 4, n, 1, 1, True, False, A.data_ptr(), B.data_ptr(), out.data_ptr(), stream())
+    ref = (B[0].double() @ A[0].double().t()).to(torch.int32)
+    assert torch.equal(out[0], ref)
+    Bh = torch.randn(1, n, 2, generator=g).half().to(gpu); Ah = torch.randn(1, m, 2, generator=g).half().to(gpu)
+    oh = torch.full((1, n, m), 9.0, dtype=torch.half, device=gpu)
+    ck.gemm_fp16(m, 2, n, 1, 1, True, False, Ah.data_ptr(), Bh.data_ptr(), oh.data_ptr(), stream())
+    refh = (Bh[0].double() @ Ah[0].double().t())
+    for sl in (slice(0, 200), slice(65535 * 64 - 100, 65535 * 64 + 100), slice(n - 50, n)):
+        assert_close_fp16(to_np(oh[0, sl]), refh[sl].cpu().numpy(), rtol=1e-3, atol=1e-3, what="general fp16 gemm rows %s" % (sl,))
