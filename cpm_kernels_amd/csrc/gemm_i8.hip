@@ -739,7 +739,7 @@ static int launch_dma(GemmArgs& a, int batch, hipStream_t st) {
     const int64_t r = total % grid;
     da.nfull = (uint32_t)total;
     da.nhalf = 0;
-    if constexpr (TR % 2 == 0 && LAY == 0) {
+    if constexpr (TR % 2 == 0 && LAY == 0 && ((BR / 2 + BC) / (1024 / BKB)) % (WR * WC) == 0) {      // (a half tile's slab must split evenly over the waves too)
         if (r > 0 && 2 * r <= grid) {
             da.nfull = (uint32_t)(total - r);
             da.nhalf = (uint32_t)(2 * r);
