@@ -13,11 +13,16 @@
 
 namespace cpmk {
 
+// One row's coefficients applied to the lane's 8 columns with packed fp16 operations (a singly rounded
+// fma, or a product): two elements per instruction, and `has_beta`, which is the same for the whole
+// launch, decides between two instruction streams instead of between two results per element.
 __device__ inline half8_t affine8(half8_t y, half_t a, half_t b, bool has_beta) {
-    half8_t o;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) o[e] = has_beta ? __builtin_fmaf16(y[e], a, b) : (half_t)(y[e] * a);
-    return o;
+    const half8_t a8 = {a, a, a, a, a, a, a, a};
+    if (has_beta) {
+        const half8_t b8 = {b, b, b, b, b, b, b, b};
+        return __builtin_elementwise_fma(y, a8, b8);
+    }
+    return y * a8;
 }
 
 // Single pass: the whole (n x LPR*8) column tile lives in registers.
