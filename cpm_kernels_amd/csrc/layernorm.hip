@@ -109,7 +109,6 @@ __global__ __launch_bounds__(NT) void k_layernorm_team(int32_t n, int32_t m, int
     __shared__ float lds[(T::NW + 1) * T::COLS * 2];
     __shared__ float tot[kXchVals];
     __shared__ half_t coef[2][NT];        // alpha and beta of this workgroup's rows (T::ROWS == NT)
-    __shared__ int failed;
     static_assert(T::ROWS == NT, "one affine coefficient pair per thread");
     const int tid = threadIdx.x;
     const uint32_t part = blockIdx.x % parts, team = blockIdx.x / parts;
@@ -118,7 +117,6 @@ __global__ __launch_bounds__(NT) void k_layernorm_team(int32_t n, int32_t m, int
     const int32_t own0 = part * T::ROWS;                 // first row this workgroup normalises
     const int32_t own_n = min(T::ROWS, n - own0);        // > 0 by construction
     const int64_t boff = (int64_t)b * n * m + (int64_t)own0 * m;
-    if (tid == 0) failed = 0;
 
     half8_t v[R];
     coltile_load<NT, LPR, R>(v, mat + boff, own_n, m, col0, (half_t)0.0f);
@@ -146,39 +144,40 @@ __global__ __launch_bounds__(NT) void k_layernorm_team(int32_t n, int32_t m, int
     // totals go straight from the reduction to its slot
     uint64_t* team_slots = xch + (size_t)team * parts * kXchVals;
     coltile_reduce_to<NT, LPR, 2, false>(s, lds, [&](int i, float r) { xch_post(team_slots + (size_t)part * kXchVals, i, r, tag); });
-    if (tid < kXchVals) {
+    // One thread per column collects the team's sums of that column, both statistics, and turns them into
+    // the column's mean and reciprocal deviation once; the 128 lanes that hold rows of the column then read
+    // the two numbers instead of each repeating the two divisions and the square root.
+    if (tid < T::COLS) {
         const uint64_t deadline = wall_clock64() + kXchTimeoutTicks;
-        float acc = 0.0f;
+        float sum = 0.0f, sq = 0.0f;
         bool ok = true;
-        for (int32_t q0 = 0; q0 < parts; q0 += 4) {        // four at a time: the registers of this kernel are full
-            float x[4];
+        for (int32_t q0 = 0; q0 < parts; q0 += 4) {
+            float x[4], y[4];
             ok &= xch_gather<4>(team_slots, parts, q0, tid, tag, deadline, x);
+            ok &= xch_gather<4>(team_slots, parts, q0, T::COLS + tid, tag, deadline, y);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc += x[j];       // in part order; absent parts are zeros
+            for (int j = 0; j < 4; ++j) {                  // in part order; absent parts are zeros
+                sum += x[j];
+                sq += y[j];
+            }
         }
-        tot[tid] = acc;
-        if (!ok) {
-            failed = 1;
-            xch_flag(xl.status, kXchStatusTimeout);
+        const float fn = (float)n;
+        float var = sq / fn, mu = 0.0f;
+        if (rd_mean) {
+            mu = sum / fn;
+            var -= mu * mu;
         }
+        tot[tid] = mu;
+        tot[T::COLS + tid] = ok ? rsqrtf(var + eps) : __builtin_nanf("");
+        if (!ok) xch_flag(xl.status, kXchStatusTimeout);
     }
     __syncthreads();
     const int cg = tid % LPR;
-#pragma unroll
-    for (int k = 0; k < 16; ++k) s[k] = tot[(k >> 3) * T::COLS + cg * 8 + (k & 7)];
-    const bool bad = failed != 0;
-
     float mean[8], rstd[8];
-    const float fn = (float)n;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-        float var = s[8 + e] / fn;
-        mean[e] = 0.0f;
-        if (rd_mean) {
-            mean[e] = s[e] / fn;
-            var -= mean[e] * mean[e];
-        }
-        rstd[e] = bad ? __builtin_nanf("") : rsqrtf(var + eps);
+        mean[e] = tot[cg * 8 + e];
+        rstd[e] = tot[T::COLS + cg * 8 + e];
     }
 #pragma unroll
     for (int p = 0; p < R; ++p) {
