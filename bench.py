@@ -462,7 +462,7 @@ def main():
             build_bench_library(verbose=False)
         cl = ctypes.CDLL(bench_library_path())
         VP, I32, I64 = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64
-        cl.ceil_mfma_i8.argtypes = [VP, I32, I32, VP, VP]
+        cl.ceil_mfma_i8.argtypes = [VP, I32, I32, I32, VP, VP]
         cl.ceil_read.argtypes = [VP, I64, VP, VP]
         cl.ceil_write.argtypes = [VP, I64, VP]
         cl.ceil_copy.argtypes = [VP, VP, I64, VP]
@@ -476,13 +476,14 @@ def main():
         sink = torch.zeros(64, dtype=torch.int32, device=dev)
         cus = props["compute_units"]
         iters = 2048
-        mfma_ops = float(cus) * 8 * iters * 16 * 2 * 32 ** 3
         for label, opnd in (("zero", torch.zeros(12 * 512 * 16, dtype=torch.int8)),
                             ("random", torch.randint(-127, 128, (12 * 512 * 16,), generator=gg, dtype=torch.int8))):
             od = opnd.to(dev)
-            ms = event_ms(lambda: ok(cl.ceil_mfma_i8(od.data_ptr(), cus, iters, sink.data_ptr(), st())), 10, warmup=3)
-            ceil["mfma_i8_only_%s_operands" % label] = {"tops": round(mfma_ops / (ms * 1e-3) / 1e12, 1), "us": round(ms * 1e3, 1),
-                                                         "frac_of_published_peak": round(mfma_ops / (ms * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4)}
+            for waves, key in ((8, "mfma_i8_only_%s_operands" % label), (4, "mfma_i8_only_%s_operands_one_wave_per_simd" % label)):
+                mfma_ops = float(cus) * waves * iters * 16 * 2 * 32 ** 3
+                ms = event_ms(lambda: ok(cl.ceil_mfma_i8(od.data_ptr(), cus, waves, iters, sink.data_ptr(), st())), 10, warmup=3)
+                ceil[key] = {"tops": round(mfma_ops / (ms * 1e-3) / 1e12, 1), "us": round(ms * 1e3, 1),
+                             "frac_of_published_peak": round(mfma_ops / (ms * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4)}
         big = torch.randint(-128, 128, (1 << 30,), generator=None, dtype=torch.int8, device=dev)
         big2 = torch.empty_like(big)
         nb = big.numel()

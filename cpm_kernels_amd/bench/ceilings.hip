@@ -105,12 +105,13 @@ int status() { return (int)hipGetLastError(); }
 
 extern "C" {
 
-// operands: 12 * 512 * 16 = 98304 bytes.  One workgroup per compute unit is the caller's choice of `workgroups`.
-// int8 operations done: workgroups * 8 waves * iters * 16 MFMAs * 2 * 32^3.
-int ceil_mfma_i8(const void* operands, int32_t workgroups, int32_t iters, void* sink, void* stream) {
-    if (workgroups < 1 || iters < 0) return 1;
-    hipLaunchKernelGGL(k_mfma_i8, dim3((unsigned)workgroups), dim3(512), 0, (hipStream_t)stream, (const int4_t*)operands, iters,
-                       (int32_t*)sink);
+// operands: 12 * 512 * 16 = 98304 bytes.  One workgroup per compute unit is the caller's choice of `workgroups`;
+// `waves` per workgroup: 8 = two per SIMD (the GEMM's occupancy), 4 = one per SIMD.
+// int8 operations done: workgroups * waves * iters * 16 MFMAs * 2 * 32^3.
+int ceil_mfma_i8(const void* operands, int32_t workgroups, int32_t waves, int32_t iters, void* sink, void* stream) {
+    if (workgroups < 1 || iters < 0 || waves < 1 || waves > 8) return 1;
+    hipLaunchKernelGGL(k_mfma_i8, dim3((unsigned)workgroups), dim3((unsigned)waves * 64), 0, (hipStream_t)stream,
+                       (const int4_t*)operands, iters, (int32_t*)sink);
     return status();
 }
 
