@@ -226,3 +226,24 @@ def test_torch_submodules_through_the_alias_package():
     for n in ("gelu", "mask", "softmax", "transpose"):
         assert not isinstance(getattr(ct, n), types.ModuleType), n
     assert isinstance(ct.utils, types.ModuleType) and isinstance(ct.gemm, types.ModuleType)
+
+
+def test_yardstick_library_is_separate_from_the_product():
+    """bench.py's yardstick kernels live in a library of their own: it builds, exports the entry points
+    the bench binds, rejects bad arguments without a GPU, and the product library neither exports nor
+    needs any of them."""
+    from cpm_kernels_amd.build import bench_library_path, build_bench_library, library_path
+    if not os.path.exists(bench_library_path()):
+        build_bench_library(verbose=False)
+    lib = ctypes.CDLL(bench_library_path())
+    for s in ("ceil_mfma_i8", "ceil_read", "ceil_write", "ceil_copy", "ceil_copy_segments"):
+        assert hasattr(lib, s), s
+    lib.ceil_copy_segments.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p]
+    assert lib.ceil_copy_segments(None, None, 1024, 1024, 48, None) == 1        # segment width not a power of two
+    assert lib.ceil_copy_segments(None, None, 1000, 1024, 128, None) == 1       # rows not whole tiles
+    prod = ctypes.CDLL(library_path())
+    assert not hasattr(prod, "ceil_mfma_i8")
+    out = subprocess.run(["nm", "-D", "--undefined-only", library_path()], capture_output=True, text=True).stdout
+    assert "ceil_" not in out
+    # the async status and the allocation-free entry point are part of the product ABI
+    assert "gave up waiting" in __import__("cpm_kernels_amd.library.cpmk", fromlist=["x"]).error_string(10004)
