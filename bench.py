@@ -484,6 +484,27 @@ def main():
                 ms = event_ms(lambda: ok(cl.ceil_mfma_i8(od.data_ptr(), cus, waves, iters, sink.data_ptr(), st())), 10, warmup=3)
                 ceil[key] = {"tops": round(mfma_ops / (ms * 1e-3) / 1e12, 1), "us": round(ms * 1e3, 1),
                              "frac_of_published_peak": round(mfma_ops / (ms * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4)}
+        # the library's K loop against that loop: one round of 256x256 tiles (4096 x 4096 outputs) at two depths of
+        # K; the difference is 64 slabs of 128 bytes per compute unit and nothing else (no launch, prologue or epilogue)
+        sweep = {"shape": "M=N=4096 int32 out, K=8192 and K=16384: (t2 - t1) / 64 = time of one 128-byte slab of a 256x256 tile per compute unit"}
+        o32 = torch.empty((1, 4096, 4096), dtype=torch.int32, device=dev)
+        for label in ("zero", "random"):
+            ts = []
+            for kk in (8192, 16384):
+                if label == "zero":
+                    qa = torch.zeros((1, 4096, kk), dtype=torch.int8, device=dev); qw = torch.zeros((1, 4096, kk), dtype=torch.int8, device=dev)
+                else:
+                    qa = torch.randint(-127, 128, (1, 4096, kk), generator=gg, dtype=torch.int8).to(dev)
+                    qw = torch.randint(-127, 128, (1, 4096, kk), generator=gg, dtype=torch.int8).to(dev)
+                ts.append(event_ms(lambda: ck.gemm_int8(4096, kk, 4096, 1, 1, True, False, qw.data_ptr(), qa.data_ptr(), o32.data_ptr(), st()), 20, warmup=5))
+                del qa, qw
+            slab_us = (ts[1] - ts[0]) * 1e3 / 64
+            mfma_only_us = 256 * 256 * 128 * 2.0 * cus / (ceil["mfma_i8_only_%s_operands" % label]["tops"] * 1e12) * 1e6
+            sweep["%s_operands" % label] = {"k8192_us": round(ts[0] * 1e3, 2), "k16384_us": round(ts[1] * 1e3, 2), "slab_us": round(slab_us, 4),
+                                            "mfma_only_slab_us": round(mfma_only_us, 4), "k_loop_frac_of_mfma_only": round(mfma_only_us / slab_us, 4),
+                                            "k16384_tops": round(2.0 * 4096 * 4096 * 16384 / (ts[1] * 1e-3) / 1e12, 1)}
+        del o32
+        ceil["gemm_k_loop (library kernel, K sweep)"] = sweep
         big = torch.randint(-128, 128, (1 << 30,), generator=None, dtype=torch.int8, device=dev)
         big2 = torch.empty_like(big)
         nb = big.numel()
