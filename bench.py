@@ -206,7 +206,7 @@ def main():
                                True, True, out16.data_ptr(), st())
         ms = event_ms(gemm, max(20, args.steps), warmup=max(3, args.warmup))
         tops = ops / (ms * 1e-3) / 1e12
-        roofline = {"kernel": "k_gemm_dma<2,4,4,2,128,1,true,2,0> (int8 MFMA GEMM + fused fp16 dequant), M=%d K=%d N=%d" % (M, K, N),
+        roofline = {"kernel": "k_gemm_dma<2,4,4,2,128,1,true,2,0,16> (int8 MFMA GEMM + fused fp16 dequant), M=%d K=%d N=%d" % (M, K, N),
                     "bound": "mfma", "achieved": round(tops, 2), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                     "ops": "int8 multiply-accumulates counted as 2 ops",
                     "frac": round(tops / PEAK_INT8_TOPS, 4), "avg_kernel_us": round(ms * 1e3, 2),

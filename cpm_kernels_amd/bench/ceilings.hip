@@ -7,6 +7,7 @@
 //                       operand fragments used in turn -- the register shape of the library's
 //                       256x256 GEMM tile -- so the result is the matrix pipe's rate on the given
 //                       operand bytes (all zero: the clock stays high; random: it drops)
+//   ceil_mfma_i8_16x16x64   the same wave tile with v_mfma_i32_16x16x64_i8
 //   ceil_read / ceil_write / ceil_copy      contiguous 16-byte accesses
 //   ceil_copy_segments  a (rows, row_bytes) matrix copied in tiles of `seg` bytes x many rows, one
 //                       tile per 1024-thread workgroup, all loads of a tile before its stores: the
@@ -54,6 +55,34 @@ __global__ __launch_bounds__(512) void k_mfma_i8(const int4_t* __restrict__ oper
 #pragma unroll
             for (int e = 0; e < 16; ++e) x ^= acc[i][j][e];
     if (x == 0x5a5a5a5a) sink[0] = x;       // keeps the loop alive; practically never true
+}
+
+// The same amount of work per wave with v_mfma_i32_16x16x64_i8: a 128x64 wave tile is 8 x 4 tiles of
+// 16x16 (128 accumulator registers, as above), a k-step of 64 bytes takes 8 + 4 operand fragments.
+__global__ __launch_bounds__(512) void k_mfma_i8_16(const int4_t* __restrict__ operands, int32_t iters, int32_t* sink) {
+    int4_t fp[8], fq[4];
+    const int t = threadIdx.x;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) fp[i] = operands[(size_t)i * 512 + t];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) fq[j] = operands[(size_t)(8 + j) * 512 + t];
+    int4_t acc[8][4];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = int4_t{0, 0, 0, 0};
+    for (int32_t it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fq[j], fp[i], acc[i][j], 0, 0, 0);
+    }
+    int32_t x = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) x ^= acc[i][j].x ^ acc[i][j].y ^ acc[i][j].z ^ acc[i][j].w;
+    if (x == 0x5a5a5a5a) sink[0] = x;
 }
 
 __global__ __launch_bounds__(256) void k_read(const int4_t* __restrict__ p, int64_t n16, int4_t* sink) {
@@ -111,6 +140,14 @@ extern "C" {
 int ceil_mfma_i8(const void* operands, int32_t workgroups, int32_t waves, int32_t iters, void* sink, void* stream) {
     if (workgroups < 1 || iters < 0 || waves < 1 || waves > 8) return 1;
     hipLaunchKernelGGL(k_mfma_i8, dim3((unsigned)workgroups), dim3((unsigned)waves * 64), 0, (hipStream_t)stream,
+                       (const int4_t*)operands, iters, (int32_t*)sink);
+    return status();
+}
+
+// The 16x16x64 form of the same instruction: int8 operations done = workgroups * waves * iters * 32 MFMAs * 2 * 16*16*64.
+int ceil_mfma_i8_16x16x64(const void* operands, int32_t workgroups, int32_t waves, int32_t iters, void* sink, void* stream) {
+    if (workgroups < 1 || iters < 0 || waves < 1 || waves > 8) return 1;
+    hipLaunchKernelGGL(k_mfma_i8_16, dim3((unsigned)workgroups), dim3((unsigned)waves * 64), 0, (hipStream_t)stream,
                        (const int4_t*)operands, iters, (int32_t*)sink);
     return status();
 }

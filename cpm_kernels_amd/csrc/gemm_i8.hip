@@ -13,8 +13,9 @@
 // equals the reference's bit for bit):
 //   k_gemm_dma     both operands K-major, k % 128 == 0: persistent workgroups walk the output
 //                  tiles; global memory goes straight into a ring of XOR-swizzled LDS stages
-//                  (global_load_lds_dwordx4), one barrier per 128-byte K slab, fragment double
-//                  buffering, v_mfma_i32_32x32x32_i8 with the operands swapped so that a lane
+//                  (global_load_lds_dwordx4), one barrier per 128-byte K slab, fragments read
+//                  ahead of their MFMAs, v_mfma_i32_16x16x64_i8 (256x256 tiles) or
+//                  v_mfma_i32_32x32x32_i8 (smaller tiles) with the operands swapped so that a lane
 //                  owns 4 consecutive output columns; results leave through a per-wave LDS strip
 //                  as whole 128-byte lines.
 //                  With template parameter LAY it also takes operands stored with K as the row index
@@ -22,7 +23,7 @@
 //   k_gemm_kmajor  both operands K-major, k % 16 == 0: register-staged 64-byte K slabs.
 //   k_gemm_generic any layout and size: LDS tiles + v_dot4_i32_i8.
 // The tile kernel also serves the fp16 product of kernels/gemm.py:188-256 (cpmk_gemm_fp16): the
-// same bytes of K per lane feed v_mfma_f32_32x32x16_f16, with fp32 accumulators.
+// same bytes of K per lane feed v_mfma_f32_16x16x32_f16 / v_mfma_f32_32x32x16_f16, with fp32 accumulators.
 #include "common.h"
 #include <type_traits>
 
@@ -232,9 +233,357 @@ __device__ __forceinline__ GemmItem gemm_item(uint32_t L, const DmaArgs& da) {
 
 // The 16 bytes of K one lane feeds to an MFMA, collected from a stage part that holds rows of K
 // with B elements each (an operand stored with K as the row index): eight 2-byte reads for fp16,
-// sixteen 1-byte reads for int8.  `p` points at the lane's element of the k-step's first row.
+// sixteen 1-byte reads for int8.  `p` points at the lane's element of the k-step's first row of K;
+// a k-step is 64 bytes of K (32 halves, 64 int8).
 template <bool F16, int B>
 __device__ __forceinline__ int4_t gather_k(const int8_t* p, int ks) {
+    if constexpr (F16) {
+        half8_t v;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = *reinterpret_cast<const half_t*>(p + (ks * 32 + e) * (B * 2));
+        return __builtin_bit_cast(int4_t, v);
+    } else {
+        uint32_t w[4];
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            uint32_t x = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) x |= (uint32_t)(uint8_t)p[(ks * 64 + d * 4 + e) * B] << (8 * e);
+            w[d] = x;
+        }
+        return int4_t{(int32_t)w[0], (int32_t)w[1], (int32_t)w[2], (int32_t)w[3]};
+    }
+}
+
+// One output tile of BR x BC = (WR*TR*32) x (WC*TC*32), K slab = BKB bytes.
+// The MFMA is the 16x16 one with 64 bytes of K (v_mfma_i32_16x16x64_i8, v_mfma_f32_16x16x32_f16):
+// per operation it moves half the accumulator registers of the 32x32 form, and on random operands,
+// where the chip's power limit sets the clock, the same product finishes about a tenth sooner.
+// A wave owns AR x AC = 2TR x 2TC such tiles; lane (r = l % 16, q = l / 16) feeds 16 bytes of K
+// (chunk q of the k-step) of row r of each operand block and receives output row r, columns
+// 4q .. 4q+3 of each 16x16 tile (the operands are passed swapped).
+// NST-stage ring; pipeline per K slab `it` (stage cur = it % NST, slabs it+1 .. it+NST-1 in flight):
+// A k-step is two passes over the wave's rows, one per half of its columns.
+//   k-steps 0 .. KS-2, and the first pass of k-step KS-1 : MFMAs while the fragments that come
+//                       next are read from stage cur
+//   s_waitcnt vmcnt((NST-2)*CNT); barrier -> slab it+1 has landed in stage nxt for every wave and
+//                                      nobody reads stage cur any more
+//   second pass of k-step KS-1 : MFMAs while the step-0 fragments of slab it+1 are read and
+//                       the DMA of slab it+NST is issued into stage cur
+// The last iterations (the "tail", a second copy of the loop body) fetch the first slabs of the
+// NEXT tile of this workgroup when it has the same shape, so that tile starts with its operands
+// already in LDS and the loads overlap this tile's stores; otherwise they fetch this tile's last
+// slab again (a redundant load nobody reads).  The ring position carries over from tile to tile
+// (`ring`), so any slab count works.  Each loop body is one basic block without selects, which
+// lets the compiler keep the accumulators in place and the MFMA/memory interleave as written.
+// Returns true if the next tile's first slabs are on their way.
+//
+// LAY marks operands whose rows are K instead: bit 0 = the row operand is stored (K, n), bit 1 =
+// the column operand is stored (K, m).  Such an operand's part of a stage holds the slab's rows
+// of K (64 for fp16, 128 for int8) with the tile's BR (BC) elements each, DMA'd as they lie in
+// memory; a lane then collects its 16 bytes of K element by element (gather_k: 16 lanes read
+// contiguous bytes of one row, no bank conflicts) instead of with one 16-byte read.
+template <int WR, int WC, int TR, int TC, int BKB, int EPI, int NST, int LAY = 0>
+__device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, int8_t* stg, uint32_t lds_base,
+                                              const GemmItem cur_item, const GemmItem nxt_item, const bool have_slabs, int& ring) {
+    constexpr bool FUSED = EPI == kEpiDequant, F16 = EPI == kEpiF16;
+    constexpr bool PT = (LAY & 1) != 0, QT = (LAY & 2) != 0;
+    static_assert(LAY == 0 || BKB == 128, "transposed operands: 128 bytes of K per slab");
+    constexpr int ESZ_IN = F16 ? 2 : 1;            // bytes per operand element
+    constexpr int EPP = 16 / ESZ_IN;               // elements per 16-byte piece
+    using acc_t = std::conditional_t<F16, float4_t, int4_t>;
+    constexpr int KS = BKB / 64, CPR = BKB / 16;
+    static_assert(KS >= 1, "k-steps of 64 bytes");
+    constexpr int AR = TR * 2, AC = TC * 2;        // 16x16 MFMA tiles of a wave
+    constexpr int NW = WR * WC, BR = WR * TR * 32, BC = WC * TC * 32;
+    constexpr int STAGE = (BR + BC) * BKB;
+    constexpr int RPI = 1024 / BKB;                // rows per DMA instruction
+    constexpr int NDMA = (BR + BC) / RPI;
+    static_assert(NDMA % NW == 0, "stage must split evenly over the waves");
+    constexpr int CNT = NDMA / NW;
+    constexpr int NM = AR * AC;
+    constexpr int RPW = 256 / BKB;                 // rows per 256-byte bank wrap
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wr = wave / WC, wc = wave % WC;
+    const int r16 = lane & 15, q = lane >> 4;
+    const int32_t K = a.k;
+    const int nk = K / BKB;
+    auto swz = [](int r) __attribute__((always_inline)) { return (r / RPW) & (CPR - 1); };
+    // fragment offsets of the wave's first block of 16 rows, k-step 0.  Step s reads logical chunk
+    // 4s + q: xor (4s << 4) commutes with the swizzle; block i lies 16 rows further on, where the swizzle repeats.
+    static_assert((16 / RPW) % CPR == 0, "the swizzle must repeat every 16 rows");
+    constexpr int BLKP = PT ? 16 * ESZ_IN : 16 * BKB, BLKQ = QT ? 16 * ESZ_IN : 16 * BKB;
+    const int rp0 = wr * TR * 32 + r16, rq0 = wc * TC * 32 + r16;
+    const int offP0 = PT ? q * EPP * (BR * ESZ_IN) + rp0 * ESZ_IN : rp0 * BKB + ((q ^ swz(rp0)) << 4);
+    const int offQ0 = BR * BKB + (QT ? q * EPP * (BC * ESZ_IN) + rq0 * ESZ_IN : rq0 * BKB + ((q ^ swz(rq0)) << 4));
+    // without slabs on their way the waits below count only loads: let the previous tile's stores finish first
+    if (!have_slabs) wait_vmcnt<0>();
+    const uint32_t b = cur_item.b;
+    const int32_t j0 = cur_item.j0, i0 = cur_item.i0;
+    const int8_t* Pb = a.P + (int64_t)b * a.strideP;
+    const int8_t* Qb = a.Q + (int64_t)b * a.strideQ;
+    // the next tile is fetched ahead only if its LDS layout is this one's
+    const bool ahead = nxt_item.valid && nxt_item.half == cur_item.half;
+    // slab s of this tile lives in stage (ring + s) % NST; the slab requested at iteration `it` is
+    // number it + LD counted from this tile's slab 0.  With fewer slabs than stages (!deep) all of a
+    // tile's slabs are requested one tile ahead and every wait is a full one.
+    const bool deep = nk >= NST;
+    const int LD = deep ? NST : nk;
+    const int ring0 = __builtin_amdgcn_readfirstlane(ring);
+    // what the last LD iterations fetch: the next tile's first slabs, or (not ahead) this tile's last slab again
+    const uint32_t tb = ahead ? nxt_item.b : b;
+    const int32_t tj0 = ahead ? nxt_item.j0 : j0, ti0 = ahead ? nxt_item.i0 : i0;
+    const int8_t* Pn = a.P + (int64_t)tb * a.strideP;
+    const int8_t* Qn = a.Q + (int64_t)tb * a.strideQ;
+
+    // this wave's DMA instructions: d -> stage rows [RPI*dd, RPI*dd + RPI), dd = wave + d*NW;
+    // rows past the matrix are clamped (they only feed outputs that are never stored)
+    uint32_t voff[CNT], ldst[CNT];
+    bool isq[CNT];
+    // byte offset of this lane's 16 bytes inside slab 0 of the tile at rows oj / columns oi
+    auto calc_voff = [&](int d, int32_t oj, int32_t oi) __attribute__((always_inline)) -> uint32_t {
+        const int dd = wave + d * NW;
+        const int r = dd * RPI + lane / CPR;
+        const int c = (lane % CPR) ^ swz(r);
+        const bool q = dd * RPI >= BR;
+        if ((PT && !q) || (QT && q)) {
+            // a (K, L) operand: the instruction covers 1024 / (2 * B) rows of K, a lane one 16-byte piece of a row
+            const int ppr = (q ? BC : BR) / EPP;                   // pieces per row of K
+            const int dl = q ? dd - BR / RPI : dd;
+            const int kr = dl * (64 / ppr) + lane / ppr, pc = lane % ppr;
+            const int32_t L = q ? a.m : a.n;
+            return ((uint32_t)kr * (uint32_t)L + (uint32_t)min((q ? oi : oj) + pc * EPP, L - EPP)) * (uint32_t)ESZ_IN;      // L % EPP == 0
+        }
+        const int32_t grow = q ? min(oi + (r - BR), a.m - 1) : min(oj + r, a.n - 1);
+        return (uint32_t)grow * (uint32_t)K + c * 16;
+    };
+#pragma unroll
+    for (int d = 0; d < CNT; ++d) {
+        const int dd = wave + d * NW;
+        isq[d] = dd * RPI >= BR;
+        voff[d] = calc_voff(d, j0, i0);
+        ldst[d] = lds_base + dd * 1024;
+    }
+    // bytes from one K slab to the next
+    const int64_t kstepP = PT ? (int64_t)BKB * a.n : BKB, kstepQ = QT ? (int64_t)BKB * a.m : BKB;
+    // One DMA instruction of slab kt: of this tile's rows, or (TAIL) of the rows the last LD iterations
+    // fetch -- the next tile's when it is fetched ahead, else this tile's again.  Which one
+    // is a compile-time choice: a run-time select here makes the compiler branch inside the K loop,
+    // which splits its body and breaks the MFMA/memory interleave.
+    auto dma1 = [&](auto dc, int kt, auto tailc, int stage) __attribute__((always_inline)) {
+        constexpr int d = decltype(dc)::value;
+        constexpr bool TAIL = decltype(tailc)::value;
+        // read every candidate first and select values, never addresses of the captured variables
+        const int8_t *pb = TAIL ? Pn : Pb, *qb = TAIL ? Qn : Qb;
+        const uint32_t v = voff[d];            // (rewritten for the tail between the two loops)
+        const bool q = isq[d];
+        lds_dma16(v, (q ? qb : pb) + kt * (q ? kstepQ : kstepP), ldst[d] + stage * STAGE);
+    };
+
+    // the dequantisation scales of this lane's outputs, fetched now so that the epilogue does
+    // not wait on memory between its stores
+    half_t sxh[AR];
+    half4_t syh[AC];
+    if (FUSED) {
+#pragma unroll
+        for (int i = 0; i < AR; ++i) {
+            const int32_t row = min(j0 + wr * TR * 32 + i * 16 + r16, a.n - 1);
+            sxh[i] = a.srow[a.bc_row ? row : (int64_t)b * a.n + row];
+        }
+#pragma unroll
+        for (int j = 0; j < AC; ++j) {
+            const int32_t col = min(i0 + wc * TC * 32 + j * 16 + q * 4, a.m - 4);   // m % 4 == 0
+            syh[j] = *reinterpret_cast<const half4_t*>(a.scol + (a.bc_col ? 0 : (int64_t)b * a.m) + col);
+        }
+    }
+
+    acc_t acc[AR][AC];
+#pragma unroll
+    for (int i = 0; i < AR; ++i)
+#pragma unroll
+        for (int j = 0; j < AC; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[i][j][e] = 0;
+    // Fragments: all AR of the row operand, and the column operand's in two sets of AC/2 -- a k-step is two
+    // passes over the wave's rows, one per half of its columns, and while one set is multiplied the
+    // other is read.  A row fragment's register is refilled with the next k-step's right after
+    // its last MFMA of the second pass.
+    constexpr int HC = AC / 2;
+    int4_t fp[AR], fq[2][HC];
+    auto lfragP = [&](auto ic, int stage, int ks) __attribute__((always_inline)) {
+        constexpr int i = decltype(ic)::value;
+        if constexpr (PT) fp[i] = gather_k<F16, BR>(smem + stage * STAGE + offP0 + i * BLKP, ks);
+        else fp[i] = *reinterpret_cast<const int4_t*>(smem + stage * STAGE + (offP0 ^ (ks << 6)) + i * BLKP);
+    };
+    auto lfragQ = [&](auto setc, auto jjc, int stage, int ks) __attribute__((always_inline)) {       // fragment jj of column half `set`
+        constexpr int set = decltype(setc)::value, jj = decltype(jjc)::value;
+        constexpr int j = set * HC + jj;
+        if constexpr (QT) fq[set][jj] = gather_k<F16, BC>(smem + stage * STAGE + offQ0 + j * BLKQ, ks);
+        else fq[set][jj] = *reinterpret_cast<const int4_t*>(smem + stage * STAGE + (offQ0 ^ (ks << 6)) + j * BLKQ);
+    };
+    // One pass: the AR x HC MFMAs of column half `jh`, order pinned.  Between them the other set of column
+    // fragments is read from k-step `qks` of stage `qs`; with REFILL the row fragments are refilled from
+    // k-step `nks` of stage `ns`; and ND further memory operations (`memop`) are spread over the pass.
+    constexpr int NMP = AR * HC;
+    auto pass = [&](auto jhc, int qs, int qks, auto refillc, int ns, int nks, auto&& memop, auto nd_c) __attribute__((always_inline)) {
+        constexpr int jh = decltype(jhc)::value, ND = decltype(nd_c)::value;
+        constexpr bool REFILL = decltype(refillc)::value;
+        static_for<0, NMP>([&](auto xc) __attribute__((always_inline)) {
+            constexpr int x = decltype(xc)::value;
+            constexpr int i = x / HC, jj = x % HC;
+            // MFMA "A" = column-operand rows, "B" = row-operand rows: lane l, register e of the
+            // result is output row l%16, column (l/16)*4 + e of the 16x16 tile
+            if constexpr (F16)      // 64 bytes of K are 32 halves: same lane -> byte assignment as the int8 MFMA
+                acc[i][jh * HC + jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, fq[jh][jj]),
+                                                                              __builtin_bit_cast(half8_t, fp[i]), acc[i][jh * HC + jj], 0, 0, 0);
+            else
+                acc[i][jh * HC + jj] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fq[jh][jj], fp[i], acc[i][jh * HC + jj], 0, 0, 0);
+            if constexpr (REFILL && jj == HC - 1) lfragP(std::integral_constant<int, i>{}, ns, nks);
+            if constexpr (x % AR == 0 && x / AR < HC)
+                lfragQ(std::integral_constant<int, 1 - jh>{}, std::integral_constant<int, x / AR>{}, qs, qks);
+            constexpr int lo = (x * ND) / NMP, hi = ((x + 1) * ND) / NMP;
+            static_for<lo, hi>([&](auto yc) __attribute__((always_inline)) { memop(yc); });
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    auto no_memop = [](auto) __attribute__((always_inline)) {};
+
+    if (!have_slabs) {
+        __syncthreads();                 // every wave is done with the ring of the previous tile
+        static_for<0, NST>([&](auto sc) __attribute__((always_inline)) {
+            constexpr int st = decltype(sc)::value;
+            static_for<0, CNT>([&](auto dc) __attribute__((always_inline)) {
+                dma1(dc, min(st, nk - 1), std::false_type{}, (ring0 + st) % NST);
+            });
+        });
+        if (deep) wait_vmcnt<(NST - 1) * CNT>();   // slab 0 (and the scale loads issued before it) has landed
+        else wait_vmcnt<0>();
+        __syncthreads();
+    } else {
+        wait_vmcnt<0>();                 // the first LD slabs were requested during the previous tile; its stores drain too
+        __syncthreads();
+    }
+    if (FUSED) {     // pin the scale loads above the K loop (the waits just above cover them)
+#pragma unroll
+        for (int i = 0; i < AR; ++i) asm volatile("" : "+v"(sxh[i]));
+#pragma unroll
+        for (int j = 0; j < AC; ++j) asm volatile("" : "+v"(syh[j]));
+        // parked in this wave's output strip, idle until the epilogue: fewer registers live across the K loop
+#pragma unroll
+        for (int i = 0; i < AR; ++i) *reinterpret_cast<half_t*>(stg + (i * 64 + lane) * 2) = sxh[i];
+#pragma unroll
+        for (int j = 0; j < AC; ++j) *reinterpret_cast<half4_t*>(stg + 1024 + (j * 64 + lane) * 8) = syh[j];
+    }
+    static_for<0, AR>([&](auto xc) __attribute__((always_inline)) { lfragP(xc, ring0, 0); });
+    static_for<0, HC>([&](auto xc) __attribute__((always_inline)) { lfragQ(I0{}, xc, ring0, 0); });
+
+    int cur = ring0;
+    // tail slab index: it + LD - nk of the next tile, or nk - 1 of this one
+    const int tmul = ahead ? 1 : 0, tadd = ahead ? LD - nk : nk - 1;
+    auto slab = [&](int it, auto tailc) __attribute__((always_inline)) {
+        constexpr bool TAIL = decltype(tailc)::value;
+        const int nxt = cur + 1 == NST ? 0 : cur + 1;
+        static_for<0, KS - 1>([&](auto ksc) __attribute__((always_inline)) {
+            constexpr int ks = decltype(ksc)::value;
+            pass(I0{}, cur, ks, std::false_type{}, 0, 0, no_memop, I0{});
+            pass(I1{}, cur, ks + 1, std::true_type{}, cur, ks + 1, no_memop, I0{});
+        });
+        pass(I0{}, cur, KS - 1, std::false_type{}, 0, 0, no_memop, I0{});       // the last reads of stage cur
+        __builtin_amdgcn_sched_barrier(0);
+        wait_vmcnt<(NST - 2) * CNT>();       // slab it + 1 has landed (with fewer slabs than stages it had before the loop)
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        const int kt2 = TAIL ? it * tmul + tadd : it + LD;
+        const int tgt = cur + LD >= NST ? cur + LD - NST : cur + LD;       // the stage slab it + LD belongs to
+        pass(I1{}, nxt, 0, std::true_type{}, nxt, 0,
+             [&](auto dc) __attribute__((always_inline)) { dma1(dc, kt2, tailc, tgt); },
+             std::integral_constant<int, CNT>{});
+        __builtin_amdgcn_sched_barrier(0);
+        cur = nxt;
+    };
+    int it = 0;
+    for (; it < nk - LD; ++it) slab(it, std::false_type{});       // slabs LD .. nk-1 of this tile follow
+#pragma unroll
+    for (int d = 0; d < CNT; ++d) voff[d] = calc_voff(d, tj0, ti0);
+    for (; it < nk; ++it) slab(it, std::true_type{});             // then the tail's
+    if (!ahead) wait_vmcnt<0>();         // drain the clamped loads before the ring is reused
+    ring = cur;                          // (ring0 + nk) % NST: where the next tile's slab 0 is, or will be put
+
+    const int64_t obase = (int64_t)b * a.n * a.m;
+    // Results leave through a 4 KB strip of LDS per wave: a lane holds 4-column pieces of ONE
+    // output row, so storing straight from the accumulators would touch 32 different rows
+    // with 8 or 16 bytes each per instruction.  Written to the strip as 32 rows x RB bytes
+    // and read back 16 bytes per lane, every store instruction covers whole contiguous rows
+    // of the chunk (RB = 128 bytes: eight lanes per 128-byte line).
+    constexpr int ESZ = EPI == kEpiInt32 ? 4 : 2;
+    constexpr int CT = EPI == kEpiInt32 ? 1 : TC;       // MFMA tiles side by side in one chunk
+    constexpr int NCH = EPI == kEpiInt32 ? TC : 1;      // chunks per block of 32 rows
+    constexpr int RB = CT * 32 * ESZ, PPR = RB / 16, RPW2 = 256 / RB, PASSES = PPR / 2, RPP = 64 / PPR;
+    // 16-byte piece p of strip row r sits at piece slot p ^ ((r / RPW2) % PPR): reads are conflict free
+    auto slot = [](int r, int p) __attribute__((always_inline)) { return (p ^ ((r / RPW2) & (PPR - 1))) << 4; };
+    half_t sxr[AR];
+    half4_t syr[AC];
+    if (FUSED) {      // the scales come back from the strip before the results overwrite it
+#pragma unroll
+        for (int i = 0; i < AR; ++i) sxr[i] = *reinterpret_cast<const half_t*>(stg + (i * 64 + lane) * 2);
+#pragma unroll
+        for (int j = 0; j < AC; ++j) syr[j] = *reinterpret_cast<const half4_t*>(stg + 1024 + (j * 64 + lane) * 8);
+#pragma unroll
+        for (int i = 0; i < AR; ++i) asm volatile("" : "+v"(sxr[i]));
+#pragma unroll
+        for (int j = 0; j < AC; ++j) asm volatile("" : "+v"(syr[j]));
+    }
+#pragma unroll
+    for (int i = 0; i < TR; ++i) {        // blocks of 32 output rows: two rows of MFMA tiles
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int srow = h * 16 + r16;      // row of the strip
+                if constexpr (EPI == kEpiInt32) {
+#pragma unroll
+                    for (int jj = 0; jj < 2; ++jj)
+                        *reinterpret_cast<int4_t*>(stg + srow * RB + slot(srow, jj * 4 + q)) = acc[2 * i + h][2 * c + jj];
+                } else {
+                    float sx = 0.0f;
+                    if (FUSED) sx = (float)sxr[2 * i + h];
+#pragma unroll
+                    for (int j = 0; j < AC; ++j) {
+                        half4_t hv;
+                        if constexpr (F16) {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) hv[e] = (half_t)acc[2 * i + h][j][e];
+                        } else {
+                            const half4_t sy = syr[j];
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) hv[e] = dequant(acc[2 * i + h][j][e], sx, (float)sy[e]);
+                        }
+                        *reinterpret_cast<half4_t*>(stg + srow * RB + slot(srow, j * 2 + (q >> 1)) + (q & 1) * 8) = hv;
+                    }
+                }
+            }
+#pragma unroll
+            for (int ps = 0; ps < PASSES; ++ps) {
+                const int R = ps * RPP + lane / PPR, pc = lane % PPR;
+                const int4_t v = *reinterpret_cast<const int4_t*>(stg + R * RB + slot(R, pc));
+                const int32_t row = j0 + wr * TR * 32 + i * 32 + R;
+                const int32_t col = i0 + wc * TC * 32 + c * 32 + pc * (16 / ESZ);
+                if (row < a.n && col < a.m)
+                    *reinterpret_cast<int4_t*>(reinterpret_cast<int8_t*>(a.out) + (obase + (int64_t)row * a.m + col) * ESZ) = v;
+            }
+        }
+    }
+    return ahead;
+}
+
+// The same for k-steps of 32 bytes (the 32x32 MFMAs): the 16 bytes of K one lane feeds to an MFMA, collected from a stage part that holds rows of K
+// with B elements each (an operand stored with K as the row index): eight 2-byte reads for fp16,
+// sixteen 1-byte reads for int8.  `p` points at the lane's element of the k-step's first row.
+template <bool F16, int B>
+__device__ __forceinline__ int4_t gather_k32(const int8_t* p, int ks) {
     if constexpr (F16) {
         half8_t v;
 #pragma unroll
@@ -253,28 +602,14 @@ __device__ __forceinline__ int4_t gather_k(const int8_t* p, int ks) {
     }
 }
 
-// One output tile of BR x BC = (WR*TR*32) x (WC*TC*32), K slab = BKB bytes.
-// NST-stage ring; pipeline per K slab `it` (stage cur = it % NST, slabs it+1 .. it+NST-1 in flight):
-//   k-steps 0 .. KS-2 : MFMAs of step s while the fragments of step s+1 are read from LDS
-//   s_waitcnt vmcnt((NST-2)*CNT); barrier -> slab it+1 has landed in stage nxt for every wave and
-//                                      nobody reads stage cur any more
-//   k-step KS-1       : MFMAs while the step-0 fragments of slab it+1 are read and the DMA of
-//                       slab it+NST is issued into stage cur
-// The last iterations (the "tail", a second copy of the loop body) fetch the first slabs of the
-// NEXT tile of this workgroup when it has the same shape, so that tile starts with its operands
-// already in LDS and the loads overlap this tile's stores; otherwise they fetch this tile's last
-// slab again (a redundant load nobody reads).  The ring position carries over from tile to tile
-// (`ring`), so any slab count works.  Each loop body is one basic block without selects, which
-// lets the compiler keep the accumulators in place and the MFMA/memory interleave as written.
-// Returns true if the next tile's first slabs are on their way.
-//
-// LAY marks operands whose rows are K instead: bit 0 = the row operand is stored (K, n), bit 1 =
-// the column operand is stored (K, m).  Such an operand's part of a stage holds the slab's rows
-// of K (64 for fp16, 128 for int8) with the tile's BR (BC) elements each, DMA'd as they lie in
-// memory; a lane then collects its 16 bytes of K element by element (gather_k: 32 lanes read
-// contiguous bytes of one row, no bank conflicts) instead of with one 16-byte read.
+// The same tile with v_mfma_i32_32x32x32_i8 / v_mfma_f32_32x32x16_f16 (k-steps of 32 bytes, a wave owns
+// TR x TC tiles of 32x32, lane l holds output row l%32; both operands' fragments double buffered,
+// the barrier before the last k-step).  Used where a wave's share of a k-step is too small for the
+// row fragments' refill-after-last-use above to hide the LDS latency (the 128x128 and smaller
+// workgroup tiles, one wave per SIMD) and for products of a single slab.  DMA, ring and tail are
+// the ones described above.
 template <int WR, int WC, int TR, int TC, int BKB, int EPI, int NST, int LAY = 0>
-__device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, int8_t* stg, uint32_t lds_base,
+__device__ __forceinline__ bool gemm_dma_tile32(const GemmArgs& a, int8_t* smem, int8_t* stg, uint32_t lds_base,
                                               const GemmItem cur_item, const GemmItem nxt_item, const bool have_slabs, int& ring) {
     constexpr bool FUSED = EPI == kEpiDequant, F16 = EPI == kEpiF16;
     constexpr bool PT = (LAY & 1) != 0, QT = (LAY & 2) != 0;
@@ -405,13 +740,13 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
         constexpr int x = decltype(xc)::value, buf = decltype(bufc)::value;
         if constexpr (x < TR) {
             if constexpr (PT) {
-                fp[buf][x] = gather_k<F16, BR>(smem + stage * STAGE + offP[x], ks);
+                fp[buf][x] = gather_k32<F16, BR>(smem + stage * STAGE + offP[x], ks);
             } else {
                 fp[buf][x] = *reinterpret_cast<const int4_t*>(smem + stage * STAGE + (offP[x] ^ (ks << 5)));
             }
         } else {
             if constexpr (QT) {
-                fq[buf][x - TR] = gather_k<F16, BC>(smem + stage * STAGE + offQ[x - TR], ks);
+                fq[buf][x - TR] = gather_k32<F16, BC>(smem + stage * STAGE + offQ[x - TR], ks);
             } else {
                 fq[buf][x - TR] = *reinterpret_cast<const int4_t*>(smem + stage * STAGE + (offQ[x - TR] ^ (ks << 5)));
             }
@@ -579,15 +914,17 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
     return ahead;
 }
 
-// Persistent kernel: WR x WC waves, wave tile = TR x TC MFMA tiles of 32x32.  Workgroup w of G
+// Persistent kernel: WR x WC waves, wave tile = TR x TC blocks of 32x32 outputs, computed with the
+// 16x16 MFMAs (MF = 16) or the 32x32 ones (MF = 32).  Workgroup w of G
 // takes items round*G + (w%8)*(G/8) + w/8: the workgroups of one XCD (w % 8) work on adjacent
 // tiles and share operand slabs in that XCD's L2.  When the tile count leaves a last round
 // that at most half the workgroups could join, those tiles are issued as row halves (HALVES), one
-// per workgroup: a wave then owns TR/2 x TC MFMA tiles, which keeps the fragment reads per MFMA
-// lower than halving the columns would (TR/2 + TC reads for TR/2 * TC MFMAs per k-step).
-template <int WR, int WC, int TR, int TC, int BKB, int EPI, bool HALVES, int NST, int LAY = 0>
+// per workgroup: a wave then owns TR/2 x TC blocks, which keeps the fragment reads per MFMA
+// lower than halving the columns would.
+template <int WR, int WC, int TR, int TC, int BKB, int EPI, bool HALVES, int NST, int LAY, int MF>
 __global__ __launch_bounds__(WR* WC * 64) void k_gemm_dma(DmaArgs da) {
     static_assert(!(HALVES && LAY != 0), "half tiles only with K-major operands");
+    static_assert(MF == 16 || MF == 32, "MFMA tile");
     constexpr int BR = WR * TR * 32, BC = WC * TC * 32;
     extern __shared__ __attribute__((aligned(16))) int8_t smem[];
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) int8_t*)smem;
@@ -602,10 +939,13 @@ __global__ __launch_bounds__(WR* WC * 64) void k_gemm_dma(DmaArgs da) {
     for (uint32_t L = w; cur.valid; L += G) {
         const GemmItem nxt = gemm_item<BR, BC>(L + G, da);
         if (HALVES && cur.half) {
-            if constexpr (HALVES)
-                have_slabs = gemm_dma_tile<WR, WC, TR / 2, TC, BKB, EPI, NST>(da.g, smem, stg, lds_base, cur, nxt, have_slabs, ring);
+            if constexpr (HALVES) {
+                if constexpr (MF == 16) have_slabs = gemm_dma_tile<WR, WC, TR / 2, TC, BKB, EPI, NST>(da.g, smem, stg, lds_base, cur, nxt, have_slabs, ring);
+                else have_slabs = gemm_dma_tile32<WR, WC, TR / 2, TC, BKB, EPI, NST>(da.g, smem, stg, lds_base, cur, nxt, have_slabs, ring);
+            }
         } else {
-            have_slabs = gemm_dma_tile<WR, WC, TR, TC, BKB, EPI, NST, LAY>(da.g, smem, stg, lds_base, cur, nxt, have_slabs, ring);
+            if constexpr (MF == 16) have_slabs = gemm_dma_tile<WR, WC, TR, TC, BKB, EPI, NST, LAY>(da.g, smem, stg, lds_base, cur, nxt, have_slabs, ring);
+            else have_slabs = gemm_dma_tile32<WR, WC, TR, TC, BKB, EPI, NST, LAY>(da.g, smem, stg, lds_base, cur, nxt, have_slabs, ring);
         }
         cur = nxt;
     }
@@ -710,20 +1050,21 @@ static int launch_kmajor(GemmArgs& a, int batch, hipStream_t st) {
 #define CPMK_GEMM_BIG_NST 2        // ring stages of the 256x256 tile kernel (K-major operands)
 #endif
 
-template <int WR, int WC, int TR, int TC, int BKB, int EPI, bool HALVES, int NST, int LAY = 0>
+template <int WR, int WC, int TR, int TC, int BKB, int EPI, bool HALVES, int NST, int LAY, int MF>
 static int launch_dma_kernel(const DmaArgs& da, unsigned grid, hipStream_t st) {
     constexpr int BR = WR * TR * 32, BC = WC * TC * 32;
     constexpr int STRIP = TC * 64 * 32 > 4096 ? TC * 64 * 32 : 4096;
     constexpr int smem = NST * (BR + BC) * BKB + WR * WC * STRIP;      // operand ring + output strips
     static_assert(smem <= 160 * 1024, "LDS of one compute unit");
-    auto kern = k_gemm_dma<WR, WC, TR, TC, BKB, EPI, HALVES, NST, LAY>;
+    auto kern = k_gemm_dma<WR, WC, TR, TC, BKB, EPI, HALVES, NST, LAY, MF>;
     static std::atomic<bool> lds_enabled[64];
     if (int e = enable_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_enabled)) return e;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(WR * WC * 64), smem, st, da);
     return launch_status();
 }
 
-template <int WR, int WC, int TR, int TC, int BKB, int EPI, int NST = 2, int LAY = 0>
+// MF: 16 = the 16x16 MFMAs (the large tile on products of several slabs), 32 = the 32x32 ones
+template <int WR, int WC, int TR, int TC, int BKB, int EPI, int NST, int LAY, int MF>
 static int launch_dma(GemmArgs& a, int batch, hipStream_t st) {
     constexpr int BR = WR * TR * 32, BC = WC * TC * 32;
     a.tiles_r = (int32_t)ceil_div(a.n, BR);
@@ -743,10 +1084,10 @@ static int launch_dma(GemmArgs& a, int batch, hipStream_t st) {
         if (r > 0 && 2 * r <= grid) {
             da.nfull = (uint32_t)(total - r);
             da.nhalf = (uint32_t)(2 * r);
-            return launch_dma_kernel<WR, WC, TR, TC, BKB, EPI, true, NST>(da, (unsigned)grid, st);
+            return launch_dma_kernel<WR, WC, TR, TC, BKB, EPI, true, NST, 0, MF>(da, (unsigned)grid, st);
         }
     }
-    return launch_dma_kernel<WR, WC, TR, TC, BKB, EPI, false, NST, LAY>(da, (unsigned)grid, st);
+    return launch_dma_kernel<WR, WC, TR, TC, BKB, EPI, false, NST, LAY, MF>(da, (unsigned)grid, st);
 }
 
 template <bool FUSED>
@@ -787,21 +1128,21 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
         const int64_t big = ceil_div(n, 256) * ceil_div(m, 256) * batch;
         constexpr int EPI = FUSED ? kEpiDequant : kEpiInt32;
         // (a dimension of at most 128 would leave half or more of every 256-wide tile empty)
-        if (big * 4 >= compute_units() * 3 && n > 128 && m > 128) return launch_dma<CPMK_GEMM_BIG, EPI, CPMK_GEMM_BIG_NST>(a, batch, st);
+        if (big * 4 >= compute_units() * 3 && n > 128 && m > 128) return launch_dma<CPMK_GEMM_BIG, EPI, CPMK_GEMM_BIG_NST, 0, 16>(a, batch, st);
         // 128x128 tiles, or 128x64 when even those leave a quarter of the compute units idle
         const int64_t mid = ceil_div(n, 128) * ceil_div(m, 128) * batch;
         // the smaller tiles finish a slab before a load from L2 returns: four ring stages keep them fed
-        if (mid * 4 >= compute_units() * 3) return launch_dma<2, 2, 2, 2, 128, EPI, CPMK_GEMM_NST_SMALL>(a, batch, st);
-        return launch_dma<2, 2, 2, 1, 128, EPI, CPMK_GEMM_NST_SMALL>(a, batch, st);
+        if (mid * 4 >= compute_units() * 3) return launch_dma<2, 2, 2, 2, 128, EPI, CPMK_GEMM_NST_SMALL, 0, 32>(a, batch, st);
+        return launch_dma<2, 2, 2, 1, 128, EPI, CPMK_GEMM_NST_SMALL, 0, 32>(a, batch, st);
     }
     // an operand stored (K, rows): the tile kernel reads it as it lies and gathers the fragments byte by byte in LDS
     if (!(p_kmajor && q_kmajor) && wide && k > 0 && (k % 128 == 0) && aligned16(A) && aligned16(B) && (p_kmajor || n % 16 == 0) &&
         (q_kmajor || m % 16 == 0) && (int64_t)n * k < (1ll << 32) && (int64_t)m * k < (1ll << 32)) {
         constexpr int EPI = FUSED ? kEpiDequant : kEpiInt32;
         switch ((p_kmajor ? 0 : 1) | (q_kmajor ? 0 : 2)) {
-            case 1: return launch_dma<2, 4, 4, 2, 128, EPI, 2, 1>(a, batch, st);
-            case 2: return launch_dma<2, 4, 4, 2, 128, EPI, 2, 2>(a, batch, st);
-            default: return launch_dma<2, 4, 4, 2, 128, EPI, 2, 3>(a, batch, st);
+            case 1: return launch_dma<2, 4, 4, 2, 128, EPI, 2, 1, 16>(a, batch, st);
+            case 2: return launch_dma<2, 4, 4, 2, 128, EPI, 2, 2, 16>(a, batch, st);
+            default: return launch_dma<2, 4, 4, 2, 128, EPI, 2, 3, 16>(a, batch, st);
         }
     }
     if (fast) {
@@ -914,8 +1255,12 @@ static int gemm_f16_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, in
     if (p_kmajor && q_kmajor && wide && k > 0 && (k % 64 == 0) && aligned16(A) && aligned16(B) &&
         (int64_t)n * k * 2 < (1ll << 32) && (int64_t)m * k * 2 < (1ll << 32)) {
         const int64_t big = ceil_div(n, 256) * ceil_div(m, 256) * batch;
-        if (big * 4 >= compute_units() * 3 && n > 128 && m > 128) return launch_dma<2, 4, 4, 2, 128, kEpiF16>(a, batch, st);
-        return launch_dma<2, 2, 2, 2, 128, kEpiF16, CPMK_GEMM_NST_SMALL>(a, batch, st);
+        if (big * 4 >= compute_units() * 3 && n > 128 && m > 128) {
+            // (products of a few slabs -- attention scores, K = 64 -- are all prologue and epilogue: the 32x32 form is quicker there)
+            if (k >= 256) return launch_dma<2, 4, 4, 2, 128, kEpiF16, 2, 0, 16>(a, batch, st);
+            return launch_dma<2, 4, 4, 2, 128, kEpiF16, 2, 0, 32>(a, batch, st);
+        }
+        return launch_dma<2, 2, 2, 2, 128, kEpiF16, CPMK_GEMM_NST_SMALL, 0, 32>(a, batch, st);
     }
     // an operand stored (K, rows): the tile kernel reads it as it lies, with 2-byte LDS reads for the fragments
     if (!(p_kmajor && q_kmajor) && wide && k > 0 && (k % 64 == 0) && aligned16(A) && aligned16(B) && (p_kmajor || n % 8 == 0) &&
@@ -923,9 +1268,9 @@ static int gemm_f16_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, in
         const int lay = (p_kmajor ? 0 : 1) | (q_kmajor ? 0 : 2);
         const bool low = n <= 64;                // 64 x 256 tiles for few output rows (attention: probabilities x values)
         switch (lay) {
-            case 1: return low ? launch_dma<1, 4, 2, 2, 128, kEpiF16, 3, 1>(a, batch, st) : launch_dma<2, 4, 4, 2, 128, kEpiF16, 2, 1>(a, batch, st);
-            case 2: return low ? launch_dma<1, 4, 2, 2, 128, kEpiF16, 3, 2>(a, batch, st) : launch_dma<2, 4, 4, 2, 128, kEpiF16, 2, 2>(a, batch, st);
-            default: return low ? launch_dma<1, 4, 2, 2, 128, kEpiF16, 3, 3>(a, batch, st) : launch_dma<2, 4, 4, 2, 128, kEpiF16, 2, 3>(a, batch, st);
+            case 1: return low ? launch_dma<1, 4, 2, 2, 128, kEpiF16, 3, 1, 32>(a, batch, st) : launch_dma<2, 4, 4, 2, 128, kEpiF16, 2, 1, 16>(a, batch, st);
+            case 2: return low ? launch_dma<1, 4, 2, 2, 128, kEpiF16, 3, 2, 32>(a, batch, st) : launch_dma<2, 4, 4, 2, 128, kEpiF16, 2, 2, 16>(a, batch, st);
+            default: return low ? launch_dma<1, 4, 2, 2, 128, kEpiF16, 3, 3, 32>(a, batch, st) : launch_dma<2, 4, 4, 2, 128, kEpiF16, 2, 3, 16>(a, batch, st);
         }
     }
     for (int64_t r0 = 0; r0 < n; r0 += 65535ll * 64) {        // (rows beyond the grid's y dimension: several launches)
