@@ -41,7 +41,7 @@ M, K, N = 4096, 4096, 10240  # north-star GEMM
 # measurements of this run.
 OFFLINE_SOURCE = {"traffic": "profiles/hbm_traffic_counters.txt (offline rocprofv3 --pmc run of this bench, not measured by this process)",
                   "mfma": "profiles/gemm_mfma_utilisation.txt (offline rocprofv3 --pmc run of this bench, not measured by this process)"}
-MFMA_BUSY_FRAC = 0.667
+MFMA_BUSY_FRAC = 0.658
 
 TRAFFIC_BYTES = {
     "gemm_fused": 353.6e6,     # 269.8 MB fetched (operand tiles re-read across the 8 L2s) + 83.9 MB written
@@ -463,6 +463,7 @@ def main():
         cl = ctypes.CDLL(bench_library_path())
         VP, I32, I64 = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64
         cl.ceil_mfma_i8.argtypes = [VP, I32, I32, I32, VP, VP]
+        cl.ceil_mfma_i8_16x16x64.argtypes = [VP, I32, I32, I32, VP, VP]
         cl.ceil_read.argtypes = [VP, I64, VP, VP]
         cl.ceil_write.argtypes = [VP, I64, VP]
         cl.ceil_copy.argtypes = [VP, VP, I64, VP]
@@ -484,6 +485,11 @@ def main():
                 ms = event_ms(lambda: ok(cl.ceil_mfma_i8(od.data_ptr(), cus, waves, iters, sink.data_ptr(), st())), 10, warmup=3)
                 ceil[key] = {"tops": round(mfma_ops / (ms * 1e-3) / 1e12, 1), "us": round(ms * 1e3, 1),
                              "frac_of_published_peak": round(mfma_ops / (ms * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4)}
+            # the same work per wave with the 16x16x64 form of the instruction (the one the 256x256 tile kernel uses)
+            mfma_ops = float(cus) * 8 * iters * 32 * 2 * 16 * 16 * 64
+            ms = event_ms(lambda: ok(cl.ceil_mfma_i8_16x16x64(od.data_ptr(), cus, 8, iters, sink.data_ptr(), st())), 10, warmup=3)
+            ceil["mfma_i8_16x16x64_only_%s_operands" % label] = {"tops": round(mfma_ops / (ms * 1e-3) / 1e12, 1), "us": round(ms * 1e3, 1),
+                                                                "frac_of_published_peak": round(mfma_ops / (ms * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4)}
         # the library's K loop against that loop: one round of 256x256 tiles (4096 x 4096 outputs) at two depths of
         # K; the difference is 64 slabs of 128 bytes per compute unit and nothing else (no launch, prologue or epilogue)
         sweep = {"shape": "M=N=4096 int32 out, K=8192 and K=16384: (t2 - t1) / 64 = time of one 128-byte slab of a 256x256 tile per compute unit"}
@@ -499,7 +505,7 @@ def main():
                 ts.append(event_ms(lambda: ck.gemm_int8(4096, kk, 4096, 1, 1, True, False, qw.data_ptr(), qa.data_ptr(), o32.data_ptr(), st()), 20, warmup=5))
                 del qa, qw
             slab_us = (ts[1] - ts[0]) * 1e3 / 64
-            mfma_only_us = 256 * 256 * 128 * 2.0 * cus / (ceil["mfma_i8_only_%s_operands" % label]["tops"] * 1e12) * 1e6
+            mfma_only_us = 256 * 256 * 128 * 2.0 * cus / (ceil["mfma_i8_16x16x64_only_%s_operands" % label]["tops"] * 1e12) * 1e6
             sweep["%s_operands" % label] = {"k8192_us": round(ts[0] * 1e3, 2), "k16384_us": round(ts[1] * 1e3, 2), "slab_us": round(slab_us, 4),
                                             "mfma_only_slab_us": round(mfma_only_us, 4), "k_loop_frac_of_mfma_only": round(mfma_only_us / slab_us, 4),
                                             "k16384_tops": round(2.0 * 4096 * 4096 * 16384 / (ts[1] * 1e-3) / 1e12, 1)}
