@@ -444,7 +444,10 @@ def test_north_star_fused_pipeline_bits(gpu):
 # decode GEMV
 # ---------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("batch,dim_out,dim_in", [(32, 10240, 4096), (16, 4444, 8888), (1, 48, 256), (33, 100, 4096),
-                                                  (130, 64, 512), (5, 17, 12), (128, 1000, 1040), (8, 40, 16)])
+                                                  (130, 64, 512), (5, 17, 12), (128, 1000, 1040), (8, 40, 16),
+                                                  # dim_in 4096: the one-round kernel at 40, 36, 25 (odd), 20, 2 and 1 rows per workgroup, ragged ends
+                                                  (32, 10239, 4096), (17, 9000, 4096), (3, 6145, 4096), (16, 5000, 4096),
+                                                  (7, 257, 4096), (1, 256, 4096), (31, 4096, 4096), (32, 10241, 4096)])
 def test_gemv_broadcast_mat_int8(gpu, batch, dim_out, dim_in):
     _name("gemv", batch, dim_out, dim_in)
     rng = np.random.default_rng(1002 + dim_out)
