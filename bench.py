@@ -41,7 +41,7 @@ M, K, N = 4096, 4096, 10240  # north-star GEMM
 # measurements of this run.
 OFFLINE_SOURCE = {"traffic": "profiles/hbm_traffic_counters.txt (offline rocprofv3 --pmc run of this bench, not measured by this process)",
                   "mfma": "profiles/gemm_mfma_utilisation.txt (offline rocprofv3 --pmc run of this bench, not measured by this process)"}
-MFMA_BUSY_FRAC = 0.658
+MFMA_BUSY_FRAC = 0.653
 
 TRAFFIC_BYTES = {
     "gemm_fused": 353.6e6,     # 269.8 MB fetched (operand tiles re-read across the 8 L2s) + 83.9 MB written
