@@ -262,8 +262,10 @@ __device__ __forceinline__ int4_t gather_k(const int8_t* p, int ks) {
 // A wave owns AR x AC = 2TR x 2TC such tiles; lane (r = l % 16, q = l / 16) feeds 16 bytes of K
 // (chunk q of the k-step) of row r of each operand block and receives output row r, columns
 // 4q .. 4q+3 of each 16x16 tile (the operands are passed swapped).
+// A k-step is two passes over the wave's rows, one per half of its columns: the column fragments
+// come in two sets, one multiplied while the other is read, and a row fragment's register is
+// refilled with the next k-step's right after its last MFMA of the second pass.
 // NST-stage ring; pipeline per K slab `it` (stage cur = it % NST, slabs it+1 .. it+NST-1 in flight):
-// A k-step is two passes over the wave's rows, one per half of its columns.
 //   k-steps 0 .. KS-2, and the first pass of k-step KS-1 : MFMAs while the fragments that come
 //                       next are read from stage cur
 //   s_waitcnt vmcnt((NST-2)*CNT); barrier -> slab it+1 has landed in stage nxt for every wave and
