@@ -174,8 +174,8 @@ def main():
     A, W = A_cpu.to(dev), W_cpu.to(dev)
     ops = 2.0 * M * N * K
 
-    step_ms = None
-    if only in ("", "pipeline"):
+    def leg_pipeline():
+        """W untimed warm-up steps, then exactly K timed steps between synchronisations: (ms per step from HIP events, from the host clock)."""
         def step():
             return ct.bmm(A, False, W, True, int8=True)
         for _ in range(args.warmup):
@@ -188,13 +188,11 @@ def main():
             step()
         e1.record()
         torch.cuda.synchronize()
-        wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
-        step_ms = max(e0.elapsed_time(e1) / args.steps, 0.0)
-        result["wall_ms_per_step"] = round(wall_ms, 4)
+        wall = (time.perf_counter() - t0) * 1e3 / args.steps
+        return max(e0.elapsed_time(e1) / args.steps, 0.0), wall
 
-    # ---- GEMM kernel alone (roofline) ------------------------------------------------------
-    roofline = None
-    if only in ("", "gemm"):
+    def leg_gemm():
+        """The GEMM kernel alone (roofline)."""
         sA = torch.empty((1, M), dtype=torch.half, device=dev); qA = torch.empty((1, M, K), dtype=torch.int8, device=dev)
         sW = torch.empty((1, N), dtype=torch.half, device=dev); qW = torch.empty((1, N, K), dtype=torch.int8, device=dev)
         ck.gemm_quantize(1, M, K, A.data_ptr(), sA.data_ptr(), qA.data_ptr(), False, st())
@@ -223,7 +221,22 @@ def main():
         ms32 = event_ms(gemm32, max(20, args.steps), warmup=3)
         roofline["int32_out_tops"] = round(ops / (ms32 * 1e-3) / 1e12, 2)
         roofline["timing"] = "HIP events around back-to-back eager launches, median of 5 batches (replayed from a graph without launch gaps the kernel runs 3-4 % slower: the clock follows the sustained load)"
-        del out32
+        return roofline
+
+    # The device raises its clock over the first ~30 ms of load (the same step takes 212, 190, 178, 172, 168 us
+    # in consecutive batches of 25 right after start or half a second of idling).  The W + K steps are
+    # therefore run twice: first thing in the process ("from_idle", reported beside the result) and, for
+    # `value`, after the per-kernel legs below have kept the device busy for seconds -- the state a
+    # serving loop is in.  With --only pipeline there is only the first.
+    step_ms = None
+    roofline = None
+    if only in ("", "pipeline"):
+        step_ms, wall_ms = leg_pipeline()
+        result["wall_ms_per_step"] = round(wall_ms, 4)
+        result["from_idle"] = {"ms_per_step": round(step_ms, 4), "value": round(ops / (step_ms * 1e-3) / 1e12, 2),
+                               "note": "the same W warm-up + K timed steps as `value`, run first thing in the process: the device's clock is still rising"}
+    if only == "gemm":
+        roofline = leg_gemm()
 
     components = {}
     reps = args.reps
@@ -550,6 +563,12 @@ def main():
         except Exception as ex:     # pragma: no cover  (calibration only)
             ceil["vendor_int_mm"] = "unavailable: %s" % ex
         result["ceilings"] = ceil
+
+    # ---- the north-star step and its GEMM kernel on the busy device (see the note at leg_pipeline's first call) ----
+    if only == "":
+        step_ms, wall_ms = leg_pipeline()
+        result["wall_ms_per_step"] = round(wall_ms, 4)
+        roofline = leg_gemm()
 
     # per-op CPU timings beside the components: the torch formulations the reference's tests compare
     # with (oracle/formulations.py), on all host cores, full shapes (fewer repetitions for the big ones)
