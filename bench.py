@@ -10,7 +10,9 @@ the CPU and resident in HBM before timing) through ``bmm(A, False, W, True, int8
 row-absmax scales and int8 rounding of both operands, int8 MFMA GEMM with int32 accumulation,
 fp16 dequantisation -- exactly what the reference's GEMMInt8.forward does per call.
 
-Prints ONE JSON line.  `value` is 2*M*N*K / step time in TOP/s for that whole step; the
+Prints ONE JSON line.  `value` is 2*M*N*K / step time in TOP/s for that whole step (W warm-up and K
+timed steps on the device kept busy by the per-kernel legs; `from_idle` is the same W + K run first
+thing in the process, while the device's clock is still rising); the
 `roofline` object is the GEMM kernel alone against the dense int8 MFMA peak; `components`
 carries the decode GEMV, layernorm and softmax kernels (and, after them, every other kernel of
 the path) against the HBM peak; `cpu_baseline`
