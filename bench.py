@@ -65,6 +65,20 @@ def parse():
     return p.parse_args()
 
 
+SETTLE_S = 0.05     # the device raises its clock over the first ~30 ms of load; per-kernel loops are timed after this much of it
+
+
+def settle(fn, seconds=SETTLE_S):
+    """Keep the device busy with fn for `seconds` (host clock), so that what follows is timed at the clock a
+    sustained load runs at.  Not used for the W + K steps of `value`, whose warm-up is W steps by definition."""
+    import torch
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(8):
+            fn()
+        torch.cuda.synchronize()
+
+
 def event_ms(fn, reps, warmup=3, batches=5):
     """Milliseconds per call of fn from HIP events on torch's current stream (the stream every
     launcher is given): `reps` back-to-back calls split into `batches` timed batches, median batch.
@@ -74,6 +88,7 @@ def event_ms(fn, reps, warmup=3, batches=5):
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
+    settle(fn)
     per = max(1, reps // batches)
     times = []
     for _ in range(batches):
@@ -106,6 +121,7 @@ def graph_ms(launches, reps):
                 f()
         g.replay()
         torch.cuda.synchronize()
+        settle(g.replay)
         per = max(1, reps // 3)
         times = []
         for _ in range(3):                   # three timed batches of replays, median batch
@@ -226,10 +242,11 @@ def main():
         return roofline
 
     # The device raises its clock over the first ~30 ms of load (the same step takes 212, 190, 178, 172, 168 us
-    # in consecutive batches of 25 right after start or half a second of idling).  The W + K steps are
-    # therefore run twice: first thing in the process ("from_idle", reported beside the result) and, for
-    # `value`, after the per-kernel legs below have kept the device busy for seconds -- the state a
-    # serving loop is in.  With --only pipeline there is only the first.
+    # in consecutive batches of 25 right after start or half a second of idling; the GEMM alone 160 ... 135 us).
+    # The W + K steps are therefore run twice: first thing in the process ("from_idle", reported beside the
+    # result) and, for `value`, at the end of the per-kernel legs, right after the roofline loop of the GEMM
+    # kernel has kept the device busy -- the state a serving loop is in.  With --only pipeline there is only
+    # the first.
     step_ms = None
     roofline = None
     if only in ("", "pipeline"):
@@ -568,9 +585,9 @@ def main():
 
     # ---- the north-star step and its GEMM kernel on the busy device (see the note at leg_pipeline's first call) ----
     if only == "":
+        roofline = leg_gemm()
         step_ms, wall_ms = leg_pipeline()
         result["wall_ms_per_step"] = round(wall_ms, 4)
-        roofline = leg_gemm()
 
     # per-op CPU timings beside the components: the torch formulations the reference's tests compare
     # with (oracle/formulations.py), on all host cores, full shapes (fewer repetitions for the big ones)
