@@ -588,6 +588,9 @@ def main():
         roofline = leg_gemm()
         step_ms, wall_ms = leg_pipeline()
         result["wall_ms_per_step"] = round(wall_ms, 4)
+        result["value_protocol"] = ("W warm-up steps, then exactly K timed steps between synchronisations, run right after the roofline loop of "
+                                    "this process, i.e. with the device at the clock a sustained load runs at; `from_idle` is the same W + K run "
+                                    "first thing in the process, while the clock is still rising (it takes ~30 ms of load)")
 
     # per-op CPU timings beside the components: the torch formulations the reference's tests compare
     # with (oracle/formulations.py), on all host cores, full shapes (fewer repetitions for the big ones)
