@@ -100,7 +100,7 @@ __global__ __launch_bounds__(NT) void k_layernorm_team(int32_t n, int32_t m, int
                                                        const half_t* mat, half_t* out,
                                                        const half_t* __restrict__ alpha,
                                                        const half_t* __restrict__ beta, float eps, int rd_mean,
-                                                       XchLaunch xl) {
+                                                       int xcd_local, XchLaunch xl) {
     constexpr int LPR = 8;
     using T = ColTile<NT, LPR, R>;
     static_assert(T::COLS * 2 == kXchVals, "slot layout");
@@ -111,7 +111,12 @@ __global__ __launch_bounds__(NT) void k_layernorm_team(int32_t n, int32_t m, int
     __shared__ half_t coef[2][NT];        // alpha and beta of this workgroup's rows (T::ROWS == NT)
     static_assert(T::ROWS == NT, "one affine coefficient pair per thread");
     const int tid = threadIdx.x;
-    const uint32_t part = blockIdx.x % parts, team = blockIdx.x / parts;
+    // xcd_local (a launch of one round whose eighths hold whole teams): workgroup i runs on XCD i % 8, so
+    // renumbering puts the members of a team on one XCD and their packets stay in that XCD's L2 (1.4 % at
+    // 8 x 4096 x 512; with more rounds than one the same renumbering loses 3 %)
+    const uint32_t G = gridDim.x;
+    const uint32_t wid = xcd_local ? (blockIdx.x % 8) * (G / 8) + blockIdx.x / 8 : blockIdx.x;
+    const uint32_t part = wid % parts, team = wid / parts;
     const uint32_t b = team / tiles_per_batch, ct = team - b * tiles_per_batch;
     const int32_t col0 = ct * T::COLS + (tid % LPR) * 8;
     const int32_t own0 = part * T::ROWS;                 // first row this workgroup normalises
@@ -320,12 +325,15 @@ static int layernorm_dispatch(int32_t batch, int32_t n, int32_t m, const void* m
                     const dim3 grid((unsigned)(tiles * nb * parts));
                     const half_t* xb = x + b0 * n * m;
                     half_t* yb = y + b0 * n * m;
+                    // (one round: every workgroup is resident at once, whatever order they start in)
+                    const int64_t G = tiles * nb * parts;
+                    const int xcd_local = G % 8 == 0 && (G / 8) % parts == 0 && G <= compute_units() * (big ? 1 : 2);
                     if (big)
                         hipLaunchKernelGGL((k_layernorm_team<1024, 8>), grid, dim3(1024), 0, st, n, m, (int32_t)tiles,
-                                           (int32_t)parts, xb, yb, al, be, eps, rd_mean, xl);
+                                           (int32_t)parts, xb, yb, al, be, eps, rd_mean, xcd_local, xl);
                     else
                         hipLaunchKernelGGL((k_layernorm_team<512, 8>), grid, dim3(512), 0, st, n, m, (int32_t)tiles,
-                                           (int32_t)parts, xb, yb, al, be, eps, rd_mean, xl);
+                                           (int32_t)parts, xb, yb, al, be, eps, rd_mean, xcd_local, xl);
                     const int e = launch_status();
                     const int rc2 = fixed != nullptr ? 0 : xch_end(xl, st);
                     if (e != 0 || rc2 != 0) return e ? e : rc2;
