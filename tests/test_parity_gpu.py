@@ -397,6 +397,38 @@ def test_gemm_int8_north_star_checksums(gpu):
     assert np.array_equal(o[jj, ii], (a64[jj] * w64[ii]).sum(axis=1))
 
 
+@pytest.mark.parametrize("M,K,N", [(2048, 512, 6144),      # 192 tiles of 256x256, one round, no half tiles
+                                   (4096, 384, 4352),      # 272 tiles: 256 whole + 32 half tiles, three slabs (the ring position carries over)
+                                   (2304, 128, 5888),      # 207 tiles of a single slab each
+                                   (4100, 640, 4104)])     # ragged edges in both directions
+def test_gemm_int8_large_tiles_exact(gpu, M, K, N):
+    """Shapes that give every compute unit a 256x256 tile (the 16x16x64 MFMA form of the tile kernel): the int32
+    product checked exactly through row and column sums and 4000 sampled entries, the fused variant against
+    gemm_scale of that product on the whole output."""
+    _name("gemm large tiles", M, K, N)
+    rng = np.random.default_rng(M + K + N)
+    qA = rng.integers(-127, 128, (1, M, K), dtype=np.int8)
+    qW = rng.integers(-127, 128, (1, N, K), dtype=np.int8)
+    sA = (rng.random((1, M)) * 0.01 + 1e-3).astype(np.float16); sW = (rng.random((1, N)) * 0.01 + 1e-3).astype(np.float16)
+    out = torch.empty((1, M, N), dtype=torch.int32, device=gpu)
+    qWd, qAd, sAd, sWd = to_gpu(qW), to_gpu(qA), to_gpu(sA), to_gpu(sW)
+    ck.gemm_int8(N, K, M, 1, 1, True, False, qWd.data_ptr(), qAd.data_ptr(), out.data_ptr(), stream())
+    o = to_np(out)[0].astype(np.int64)
+    a64, w64 = qA[0].astype(np.int64), qW[0].astype(np.int64)
+    assert np.array_equal(o.sum(axis=1), a64 @ w64.sum(axis=0))
+    assert np.array_equal(o.sum(axis=0), w64 @ a64.sum(axis=0))
+    jj = rng.integers(0, M, 4000); ii = rng.integers(0, N, 4000)
+    assert np.array_equal(o[jj, ii], (a64[jj] * w64[ii]).sum(axis=1))
+    fused = torch.empty((1, M, N), dtype=torch.half, device=gpu)
+    ck.gemm_int8_scale(N, K, M, 1, 1, True, False, qWd.data_ptr(), qAd.data_ptr(), sAd.data_ptr(), sWd.data_ptr(),
+                       True, True, fused.data_ptr(), stream())
+    two = torch.empty_like(fused)
+    ck.gemm_scale(1, M, N, out.data_ptr(), sAd.data_ptr(), sWd.data_ptr(), two.data_ptr(), True, True, stream())
+    assert torch.equal(two.view(torch.int16), fused.view(torch.int16)), "fused != gemm_int8 + gemm_scale"
+    ref = oracle.gemm_scale(to_np(out)[:, :64], sA[:, :64], sW, True, True)
+    assert_bits_equal(to_np(two)[:, :64], ref, "gemm_scale of the first 64 rows")
+
+
 def test_north_star_fused_pipeline_bits(gpu):
     """The benchmarked call itself at full size -- quantise A [4096,4096] and W [10240,4096] (seed 1000, the
     bench's data), then the fused int8 GEMM + dequantisation -- checked to the bit on 64 output rows
