@@ -1066,8 +1066,9 @@ static int launch_dma_kernel(const DmaArgs& da, unsigned grid, hipStream_t st) {
 }
 
 // MF: 16 = the 16x16 MFMAs (the large tile on products of several slabs), 32 = the 32x32 ones
+// per_cu: workgroups a compute unit holds at once (their LDS and registers must allow it)
 template <int WR, int WC, int TR, int TC, int BKB, int EPI, int NST, int LAY, int MF>
-static int launch_dma(GemmArgs& a, int batch, hipStream_t st) {
+static int launch_dma(GemmArgs& a, int batch, hipStream_t st, int per_cu = 1) {
     constexpr int BR = WR * TR * 32, BC = WC * TC * 32;
     a.tiles_r = (int32_t)ceil_div(a.n, BR);
     a.tiles_c = (int32_t)ceil_div(a.m, BC);
@@ -1076,7 +1077,7 @@ static int launch_dma(GemmArgs& a, int batch, hipStream_t st) {
     da.batch = batch;
     da.ntiles = a.tiles_r * a.tiles_c;
     const int64_t total = (int64_t)da.ntiles * batch;
-    const int cus = compute_units();
+    const int cus = compute_units() * per_cu;
     const int64_t grid = total < cus ? total : cus;
     // a last round of r <= grid/2 tiles is issued as 2r half tiles
     const int64_t r = total % grid;
@@ -1133,8 +1134,17 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
         if (big * 4 >= compute_units() * 3 && n > 128 && m > 128) return launch_dma<CPMK_GEMM_BIG, EPI, CPMK_GEMM_BIG_NST, 0, 16>(a, batch, st);
         // 128x128 tiles, or 128x64 when even those leave a quarter of the compute units idle
         const int64_t mid = ceil_div(n, 128) * ceil_div(m, 128) * batch;
-        // the smaller tiles finish a slab before a load from L2 returns: four ring stages keep them fed
-        if (mid * 4 >= compute_units() * 3) return launch_dma<2, 2, 2, 2, 128, EPI, CPMK_GEMM_NST_SMALL, 0, 32>(a, batch, st);
+        // the smaller tiles finish a slab before a load from L2 returns: four ring stages keep them fed.  More
+        // tiles than compute units but at most two each: a ring of two stages instead, which lets two
+        // workgroups share a compute unit (2 x 80 KB of LDS) and all tiles run in one round, each
+        // workgroup's waits covered by the other's MFMAs (6-11 % over 1.25-2 rounds of single workgroups)
+        const int64_t cus = compute_units();
+        if (mid * 4 >= cus * 3) {
+            if (mid > cus && mid <= 2 * cus) return launch_dma<2, 2, 2, 2, 128, EPI, 2, 0, 32>(a, batch, st, 2);
+            return launch_dma<2, 2, 2, 2, 128, EPI, CPMK_GEMM_NST_SMALL, 0, 32>(a, batch, st);
+        }
+        const int64_t small = ceil_div(n, 128) * ceil_div(m, 64) * batch;
+        if (small > cus && small <= 2 * cus) return launch_dma<2, 2, 2, 1, 128, EPI, 2, 0, 32>(a, batch, st, 2);
         return launch_dma<2, 2, 2, 1, 128, EPI, CPMK_GEMM_NST_SMALL, 0, 32>(a, batch, st);
     }
     // an operand stored (K, rows): the tile kernel reads it as it lies and gathers the fragments byte by byte in LDS

@@ -400,11 +400,14 @@ def test_gemm_int8_north_star_checksums(gpu):
 @pytest.mark.parametrize("M,K,N", [(2048, 512, 6144),      # 192 tiles of 256x256, one round, no half tiles
                                    (4096, 384, 4352),      # 272 tiles: 256 whole + 32 half tiles, three slabs (the ring position carries over)
                                    (2304, 128, 5888),      # 207 tiles of a single slab each
-                                   (4100, 640, 4104)])     # ragged edges in both directions
+                                   (4100, 640, 4104),      # ragged edges in both directions
+                                   # more 128x128 (128x64) tiles than compute units, at most two each: two workgroups share a
+                                   # compute unit on a two-stage ring -- two slabs, one slab (fewer than stages), three
+                                   (1536, 256, 4096), (1280, 128, 4096), (256, 384, 10240), (2048, 4096, 4096)])
 def test_gemm_int8_large_tiles_exact(gpu, M, K, N):
-    """Shapes that give every compute unit a 256x256 tile (the 16x16x64 MFMA form of the tile kernel): the int32
-    product checked exactly through row and column sums and 4000 sampled entries, the fused variant against
-    gemm_scale of that product on the whole output."""
+    """Shapes that give every compute unit a 256x256 tile (the 16x16x64 MFMA form of the tile kernel) or two smaller
+    ones at once: the int32 product checked exactly through row and column sums and 4000 sampled entries, the
+    fused variant against gemm_scale of that product on the whole output."""
     _name("gemm large tiles", M, K, N)
     rng = np.random.default_rng(M + K + N)
     qA = rng.integers(-127, 128, (1, M, K), dtype=np.int8)
