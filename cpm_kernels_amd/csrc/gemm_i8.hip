@@ -1272,6 +1272,9 @@ static int gemm_f16_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, in
             if (k >= 256) return launch_dma<2, 4, 4, 2, 128, kEpiF16, 2, 0, 16>(a, batch, st);
             return launch_dma<2, 4, 4, 2, 128, kEpiF16, 2, 0, 32>(a, batch, st);
         }
+        // (as for int8: more 128x128 tiles than compute units but at most two each -> two workgroups per compute unit)
+        const int64_t mid = ceil_div(n, 128) * ceil_div(m, 128) * batch, cus = compute_units();
+        if (mid > cus && mid <= 2 * cus) return launch_dma<2, 2, 2, 2, 128, kEpiF16, 2, 0, 32>(a, batch, st, 2);
         return launch_dma<2, 2, 2, 2, 128, kEpiF16, CPMK_GEMM_NST_SMALL, 0, 32>(a, batch, st);
     }
     // an operand stored (K, rows): the tile kernel reads it as it lies, with 2-byte LDS reads for the fragments

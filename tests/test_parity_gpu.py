@@ -961,7 +961,9 @@ F16_GEMM_CASES = [  # (batch, n, k, m) in the kernel's convention: out (batch, n
     # one slab of K and several 256 x 256 tiles per workgroup (attention scores): whole tiles only, and ragged edges
     (32, 512, 64, 768), (24, 520, 64, 776),
     # several slabs of K and enough 256 x 256 tiles for every compute unit (the 16x16 MFMA form of the tile kernel)
-    (48, 512, 256, 512), (50, 520, 320, 264)]
+    (48, 512, 256, 512), (50, 520, 320, 264),
+    # more 128 x 128 tiles than compute units, at most two each (two workgroups per compute unit, two-stage ring)
+    (24, 512, 128, 512)]
 
 
 @pytest.mark.parametrize("case", F16_GEMM_CASES)
