@@ -35,22 +35,51 @@ PEAK_INT8_TOPS = 5000.0      # MI355X dense int8 MFMA, published
 PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, published
 M, K, N = 4096, 4096, 10240  # north-star GEMM
 
-# Hardware-counter figures cannot be read from inside this process.  They are taken offline --
+# Hardware-counter figures cannot be taken from inside this process.  They come from offline runs --
 # `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` over `python3 bench.py --no-cpu --only <workload>`,
-# each counter scaled by what it reads for the 256 MiB device copy of `--only calib` (FETCH_SIZE x 2.000,
-# WRITE_SIZE x 1.000 on MI355X); MFMA pipe busy cycles / kernel cycles from SQ_VALU_MFMA_BUSY_CYCLES and
-# SQ_BUSY_CYCLES -- and are emitted with their source file so that they are not mistaken for
-# measurements of this run.
-OFFLINE_SOURCE = {"traffic": "profiles/hbm_traffic_counters.txt (offline rocprofv3 --pmc run of this bench, not measured by this process)",
-                  "mfma": "profiles/gemm_mfma_utilisation.txt (offline rocprofv3 --pmc run of this bench, not measured by this process)"}
-MFMA_BUSY_FRAC = 0.651
+# each counter scaled by what it reads for the 256 MiB device copy of `--only calib`; MFMA pipe busy
+# cycles / kernel cycles from SQ_VALU_MFMA_BUSY_CYCLES and SQ_BUSY_CYCLES -- whose summaries are the
+# text files under profiles/.  The figures are read from those files at run time (never typed in here)
+# and emitted with their source, so that they are not mistaken for measurements of this run.
+PROFILES = os.path.join(ROOT, "profiles")
+OFFLINE_SOURCE = {"traffic": "profiles/hbm_traffic_counters.txt (offline rocprofv3 --pmc run of this bench, read at run time, not measured by this process)",
+                  "mfma": "profiles/gemm_mfma_utilisation.txt (offline rocprofv3 --pmc run of this bench, read at run time, not measured by this process)"}
+# which row of profiles/hbm_traffic_counters.txt belongs to which workload (a substring of the kernel's name)
+TRAFFIC_KERNELS = {"gemm_fused": "k_gemm_dma<2, 4, 4, 2, 128, 1,", "gemv": "k_gemv", "layernorm": "k_layernorm", "softmax": "k_softmax"}
 
-TRAFFIC_BYTES = {
-    "gemm_fused": 354.3e6,     # 270.4 MB fetched (operand tiles re-read across the 8 L2s) + 83.9 MB written
-    "gemv": 43.9e6,
-    "layernorm": 68.3e6,
-    "softmax": 2147.8e6,
-}
+
+def offline_counters():
+    """({workload: HBM bytes per launch}, MFMA busy fraction of the fused GEMM kernel's cycles) from the
+    summaries under profiles/; a missing or unreadable figure is None."""
+    traffic = {k: None for k in TRAFFIC_KERNELS}
+    try:
+        for ln in open(os.path.join(PROFILES, "hbm_traffic_counters.txt")):
+            f = ln.split()
+            if len(f) < 8:
+                continue
+            try:
+                total_mb, calls = float(f[-1]), int(f[-6])
+            except ValueError:
+                continue
+            for k, sub in TRAFFIC_KERNELS.items():
+                if sub in ln and calls > 1 and traffic[k] is None:      # (single-call rows are the set-up launches)
+                    traffic[k] = round(total_mb * 1e6)
+    except OSError:
+        pass
+    busy = None
+    try:
+        fused = False
+        for ln in open(os.path.join(PROFILES, "gemm_mfma_utilisation.txt")):
+            if ln.startswith("k_gemm_dma"):
+                fused = TRAFFIC_KERNELS["gemm_fused"] in ln
+            elif fused and "MFMA utilisation" in ln and busy is None:
+                busy = float(ln.split()[3])
+    except (OSError, ValueError, IndexError):
+        pass
+    return traffic, busy
+
+
+TRAFFIC_BYTES, MFMA_BUSY_FRAC = offline_counters()
 
 
 def parse():
@@ -657,6 +686,24 @@ def main():
                "kind": "port", "seconds_per_step": round(best, 3),
                "sample": "full north-star step (fp32 fake-quant of A and W + fp32 matmul), median of %d runs" % len(times)}
 
+    # The HBM half of the metric inside `roofline`, so that the one object carries all four headline kernels:
+    # kernel, average launch time, algorithmic bytes, achieved rate, fraction of the published HBM peak, and
+    # the HBM bytes the counters saw per launch (profiles/hbm_traffic_counters.txt).
+    hbm_block = {}
+    for name, kernel in (("gemv_broadcast_mat_int8", "k_gemv_direct<2,3>"), ("layernorm_forward", "k_layernorm_team<1024,8>"),
+                         ("softmax_forward", "k_softmax_stream<1024,8,8>")):
+        c = components.get(name)
+        if c is not None:
+            hbm_block[name] = {"kernel": kernel, "shape": c["shape"], "avg_us": c["avg_us"], "algorithmic_bytes": c["algorithmic_bytes"],
+                               "achieved": c["achieved"], "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": c["frac"], "traffic": c["traffic"],
+                               "timing": c["timing"]}
+    if hbm_block:
+        if roofline is None:
+            roofline = {}
+        roofline["hbm"] = hbm_block
+        roofline["hbm_note"] = ("the metric's HBM-bound kernels: frac = algorithmic_bytes / avg_us / 8 TB/s; inputs rotate through buffers larger "
+                                "than the 256 MB Infinity Cache; traffic = HBM bytes per launch from " + OFFLINE_SOURCE["traffic"])
+
     value = ops / (step_ms * 1e-3) / 1e12 if step_ms else None
     line = {
         "metric": "int8 quant-GEMM TOPS + GEMV/LN/softmax HBM GB/s (frac of peak) at 1 GPU",
@@ -668,6 +715,7 @@ def main():
         "config": {"workload": "north-star int8 quant-GEMM M=4096 K=4096 N=10240: bmm(A[1,4096,4096] fp16, "
                                "W[1,10240,4096] fp16, int8=True) = quantise A and W, int8 MFMA GEMM, fp16 dequant",
                    "seed": 1000},
+        "value_cold": result.get("from_idle", {}).get("value"), "ms_per_step_cold": result.get("from_idle", {}).get("ms_per_step"),
         "roofline": roofline, "cpu_baseline": cpu, "components": components,
         "device": torch.cuda.get_device_name(0),
     }

@@ -7,3 +7,4 @@ on demand; it needs PyTorch) holds the wrappers of ``cpm_kernels.torch`` for thi
 """
 from . import library
 from .kernels import *  # noqa: F401,F403
+from .library.cpmk import check  # noqa: F401  (raise a pending asynchronous kernel failure)

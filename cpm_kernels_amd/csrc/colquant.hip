@@ -71,7 +71,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
                 for (int j = 0; j < 8; ++j) M = fmaxf(M, x[j]);       // maxima are >= 0: absent parts (zeros) do not matter
             }
             tot[tid] = ok ? M : __builtin_nanf("");
-            if (!ok) xch_flag(xl.status, kXchStatusTimeout);
+            if (!ok) xch_flag(xl, kXchStatusTimeout);
         }
         __syncthreads();
 #pragma unroll
@@ -207,21 +207,26 @@ int cpmk_gemm_quantize_cols(int32_t batch, int32_t n, int32_t m, const void* mat
     if (team_ok) {
         // teams use one packet slot per (team, part): batches beyond the pool go out in several launches
         const int64_t per_launch = parts > 1 ? kXchSlots / (tiles * parts) : ((1ll << 31) - 1) / (tiles * parts);
+        bool no_slots = false;
         for (int64_t b0 = 0; b0 < batch; b0 += per_launch) {
             const int64_t nb = batch - b0 < per_launch ? batch - b0 : per_launch;
-            XchLaunch xl = {nullptr, nullptr, nullptr, 0, -1};
+            XchScope xs;
             if (parts > 1) {
-                const int rc = xch_begin(&xl, tiles * nb * parts, st);
-                if (rc != 0) return rc;
+                const int rc = xs.begin(tiles * nb * parts, st);
+                if (rc == kXchFull && b0 == 0) {
+                    no_slots = true;       // recorded into a graph and the capture reserve is used up: the separate kernels below
+                    break;
+                }
+                if (rc != 0) return rc == kXchFull ? CPMK_ETOOBIG : rc;
             }
             hipLaunchKernelGGL((k_col_quantize_team<512>), dim3((unsigned)(tiles * nb * parts)), dim3(512), 0, st, n, m,
                                (int32_t)tiles, (int32_t)parts, (const half_t*)mat + b0 * n * m, (half_t*)scale + b0 * m,
-                               (int8_t*)out + b0 * n * m, out_transposed, xl);
+                               (int8_t*)out + b0 * n * m, out_transposed, xs.xl);
             const int e = launch_status();
-            const int rc2 = xch_end(xl, st);
+            const int rc2 = xs.end();
             if (e != 0 || rc2 != 0) return e ? e : rc2;
         }
-        return 0;
+        if (!no_slots) return 0;
     }
     if (int e = cpmk_gemm_calc_scale_transpose(batch, n, m, mat, scale, stream)) return e;
     if (!out_transposed) return cpmk_gemm_round_transpose(batch, n, m, mat, scale, out, stream);

@@ -177,7 +177,17 @@ __device__ inline half_t dequant(int32_t acc, float sx, float sy) {
 // call (for instance a failed device probe of another library) would otherwise be reported
 // by the first launcher that asks.  Every launcher therefore clears it on entry.
 inline void clear_stale_error() { (void)hipGetLastError(); }
-inline int launch_status() { return (int)hipGetLastError(); }
+// CPMK_ETIMEOUT if a kernel of an earlier launch on the current device gave up a bounded wait for another
+// workgroup (it left NaN, or 0 in an int8 output, behind) and cpmk_async_status() has not taken the report
+// yet, else 0: one load from pinned host memory that the kernel writes to (exchange.hip).
+int async_failure();
+// What every launcher returns after its launch: the runtime's error if the launch failed, else the pending
+// asynchronous failure of an earlier kernel -- reported by the next call, like the runtime's own
+// asynchronous errors (the reference raises them from its status checks, library/cudart.py:325-327).
+inline int launch_status() {
+    const int e = (int)hipGetLastError();
+    return e != 0 ? e : async_failure();
+}
 
 // Map a linear workgroup index so that consecutive logical tiles land on the same XCD.
 // Workgroups are dealt round-robin to the 8 XCDs of an MI355X (workgroup i -> XCD i % 8),

@@ -11,28 +11,36 @@
 // replayed with the same arguments (a captured graph) starts from a clean slate as well.
 //
 // The packets live in a fixed pool in device memory owned by the library (nothing is allocated
-// per call): kXchPoolSlots slots of kXchVals packets, handed out as a ring.  A launch takes as
-// many slots as it has (team, part) pairs (at most kXchSlots), so the pool holds the slots of
-// many launches at once (128 tall layernorms of 8 x 4096 x 512); before a launch reuses slots that
-// an earlier launch was given, its stream waits for that launch's completion event
-// (xch_begin / xch_end), so launches on any number of streams never share live packets.  The
-// exception is a launch recorded during stream capture: a graph's replays cannot be tracked by
-// events, so a captured launch keeps the slots it was recorded with and the host only avoids
-// them until the ring comes round again.
+// per call).  Its first kXchRingSlots slots of kXchVals packets are handed out as a ring.  A launch
+// takes as many slots as it has (team, part) pairs (at most kXchSlots), so the ring holds the
+// slots of many launches at once (128 tall layernorms of 8 x 4096 x 512); before a launch reuses
+// slots that an earlier launch was given, its stream waits for that launch's completion event,
+// so launches on any number of streams never share live packets.  The pool's lock is held from
+// the moment a launch is given its slots until its completion event is recorded (XchScope), so
+// no other host thread ever sees slots whose holder cannot be waited for.
+// A launch recorded during stream capture cannot be tracked by events (a graph is replayed any
+// number of times, at any time): it gets slots from a reserve of kXchCaptureSlots further slots
+// that the ring never hands out and that are never given to anyone else, so its replays cannot
+// meet the packets of any other launch, eager or captured.  When the reserve is used up XchScope::
+// begin says so (kXchFull) and the caller records its kernel that needs no packets instead.
 //
 // Progress: a workgroup only ever waits for workgroups of its own team, whose indices differ by
 // less than the team size; the dispatcher starts the workgroups of a launch in index order (an
 // observed property of the hardware queue, not a documented one), so all members of the oldest
 // unfinished team are resident and that team completes.  Should a packet nevertheless not arrive
 // within about a second the wait gives up, the caller writes NaN (0 in an int8 output) and sets
-// the device's sticky status word, which cpmk_async_status() reports and clears: a visible
-// failure instead of a hung GPU.
+// the device's sticky status word and its mirror in pinned host memory.  Every launcher of the
+// library looks at the mirror before it returns (launch_status() in common.h), so the failure is
+// reported by the next call, whichever it is, like an asynchronous error of the runtime itself;
+// cpmk_async_status() reports and clears it: a visible failure instead of a hung GPU.
 #pragma once
 #include "common.h"
 
 namespace cpmk {
 
-constexpr int kXchPoolSlots = 32768;  // slots in the pool (1 KB each)
+constexpr int kXchRingSlots = 32768;     // slots handed out as a ring to eager launches (1 KB each)
+constexpr int kXchCaptureSlots = 32768;  // slots beyond the ring, given once and for all to launches recorded during stream capture
+constexpr int kXchPoolSlots = kXchRingSlots + kXchCaptureSlots;
 constexpr int kXchSlots = 8192;       // (team, part) pairs per launch
 constexpr int kXchVals = 128;         // packets per slot: 64 columns x 2 statistics
 constexpr int kXchMaxParts = 8;
@@ -40,31 +48,53 @@ constexpr int kXchGranule = 64;       // slots are handed out in multiples of th
 
 constexpr uint32_t kXchStatusTimeout = 1u;   // bit of the status word: a packet did not arrive in time
 
+constexpr int kXchFull = -2;          // XchScope::begin: the capture reserve is used up (not an error: record the kernel without packets)
+
 // What a team kernel needs of the pool; passed to the kernel by value.
 struct XchLaunch {
     uint64_t* region;     // this launch's slots: slot i at region + i * kXchVals
     uint64_t* counters;   // one retire counter per team: counters[team]
     uint32_t* status;     // the device's sticky status word
+    uint32_t* host_status;  // its mirror in pinned host memory (nullptr if there is none)
     uint32_t tag;         // never 0, differs from the tags of the launches that used these slots before
     int32_t first;        // host bookkeeping: first pool slot of the launch, -1 if it holds none
 };
+constexpr XchLaunch kXchNone = {nullptr, nullptr, nullptr, nullptr, 0, -1};     // a launch without packets
 
-// Host, before the launch: `slots` slots (and as many team counters) for a launch on stream `st` of the
-// current device; makes `st` wait for the launches that last held those slots.  0 or an error code.
-int xch_begin(XchLaunch* out, int64_t slots, hipStream_t st);
-// Host, after the launch: records the launch's completion on `st` so that a later holder of its slots
-// can wait for it.  0 or an error code.
-int xch_end(const XchLaunch& xl, hipStream_t st);
-// Host: a tag for a team launch that brings its own packet slots (never 0, from the same sequence as xch_begin's).
+// Host: the slots of one team launch.  begin() gives `slots` slots (and as many team counters) to a launch on
+// stream `st` of the current device and makes `st` wait for the launches that last held them; end(), after the
+// kernel launch, records the launch's completion on `st` so that a later holder of its slots can wait for it.
+// The pool stays locked in between (and is unlocked by the destructor on every path), so the launch itself
+// must follow begin() directly.  begin(): 0, kXchFull (recorded during stream capture and the capture reserve
+// is used up; nothing is held), or an error code.  end(): 0 or an error code.
+class XchScope {
+public:
+    XchScope() = default;
+    XchScope(const XchScope&) = delete;
+    XchScope& operator=(const XchScope&) = delete;
+    ~XchScope();
+    int begin(int64_t slots, hipStream_t st);
+    int end();
+    XchLaunch xl = kXchNone;
+private:
+    hipStream_t st_ = nullptr;
+    int32_t last_ = 0;                 // end of the slot range [xl.first, last_)
+    bool locked_ = false, captured_ = false;
+};
+// Host: a tag for a team launch that brings its own packet slots (never 0, from the same sequence as XchScope's).
 uint32_t xch_next_tag();
-// Host: the address of the current device's status word, for such a launch.  0 or an error code.
-int xch_status_word(uint32_t** out);
-// Host: reads and clears the current device's status word (0, kXchStatus* bits, or -1 - hipError on failure to read).
+// Host: the addresses of the current device's status word and of its host mirror (nullptr if none), for such a
+// launch.  0 or an error code.
+int xch_status_words(uint32_t** device_word, uint32_t** host_word);
+// Host: slots left in the current device's capture reserve.  0 or an error code.
+int xch_capture_slots_left(int32_t* slots);
+// Host: reads and clears the current device's status word and its mirror (0, kXchStatus* bits; an error code on failure to read).
 int xch_take_status(uint32_t* bits);
 
-// A wait gave up: leave a mark that the host can see (cpmk_async_status).
-__device__ inline void xch_flag(uint32_t* status, uint32_t bit) {
-    __hip_atomic_fetch_or(status, bit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+// A wait gave up: leave a mark that the host can see (launch_status, cpmk_async_status).
+__device__ inline void xch_flag(const XchLaunch& xl, uint32_t bit) {
+    __hip_atomic_fetch_or(xl.status, bit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (xl.host_status != nullptr) __hip_atomic_fetch_or(xl.host_status, bit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
 __device__ inline void xch_post(uint64_t* slot, int idx, float v, uint32_t tag) {

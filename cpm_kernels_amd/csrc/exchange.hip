@@ -9,18 +9,25 @@ namespace cpmk {
 // packets, then one counter per slot (a team uses the counter of its index within the launch's range)
 static __device__ __align__(256) uint64_t g_xch_pool[(size_t)kXchPoolSlots * kXchVals + kXchPoolSlots];
 static __device__ uint32_t g_xch_status;
+static __device__ uint32_t g_xch_taken;       // where k_xch_take_status leaves what it took
+
+// The host mirrors of the status words, one per device (nullptr until the device's pool is set up, or if
+// pinned memory could not be had).  Read without the lock by async_failure().
+static std::atomic<uint32_t*> g_host_status[64];
 
 namespace {
 
-struct Held {             // a range of slots given to a launch that may still be running
+struct Held {             // a range of ring slots given to a launch that may still be running
     int32_t first, last;  // [first, last)
-    hipEvent_t done;      // recorded after the launch; nullptr for a launch recorded during stream capture
+    hipEvent_t done;      // recorded after the launch
 };
 
 struct DevicePool {
     uint64_t* base = nullptr;       // the pool's address on this device
     uint32_t* status = nullptr;
+    uint32_t* taken = nullptr;
     int32_t head = 0;               // next free slot of the ring
+    int32_t capture_head = kXchRingSlots;   // next slot of the capture reserve; they are never taken back
     std::vector<Held> held;
     std::vector<hipEvent_t> spare;  // events ready for reuse
 };
@@ -28,25 +35,6 @@ struct DevicePool {
 std::mutex g_mu;
 DevicePool g_dev[64];
 std::atomic<uint32_t> g_seq{0};
-
-int device_pool(DevicePool** out) {      // g_mu held
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return (int)e;
-    if (dev < 0 || dev >= 64) return CPMK_EBADARG;
-    DevicePool& d = g_dev[dev];
-    if (d.base == nullptr) {
-        void *pool = nullptr, *stat = nullptr;
-        e = hipGetSymbolAddress(&pool, HIP_SYMBOL(g_xch_pool));
-        if (e != hipSuccess) return (int)e;
-        e = hipGetSymbolAddress(&stat, HIP_SYMBOL(g_xch_status));
-        if (e != hipSuccess) return (int)e;
-        d.status = (uint32_t*)stat;
-        d.base = (uint64_t*)pool;
-    }
-    *out = &d;
-    return 0;
-}
 
 bool capturing(hipStream_t st) {
     hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
@@ -57,7 +45,53 @@ bool capturing(hipStream_t st) {
     return cs != hipStreamCaptureStatusNone;
 }
 
+// `may_allocate`: the caller is not recording into a graph, so the one-time allocation of the status word's
+// host mirror (4 bytes of pinned memory per device) may be made now; otherwise it is left for a later call.
+int device_pool(DevicePool** out, int* device, bool may_allocate) {      // g_mu held
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= 64) return CPMK_EBADARG;
+    DevicePool& d = g_dev[dev];
+    if (d.base == nullptr) {
+        void *pool = nullptr, *stat = nullptr, *taken = nullptr;
+        e = hipGetSymbolAddress(&pool, HIP_SYMBOL(g_xch_pool));
+        if (e != hipSuccess) return (int)e;
+        e = hipGetSymbolAddress(&stat, HIP_SYMBOL(g_xch_status));
+        if (e != hipSuccess) return (int)e;
+        e = hipGetSymbolAddress(&taken, HIP_SYMBOL(g_xch_taken));
+        if (e != hipSuccess) return (int)e;
+        d.status = (uint32_t*)stat;
+        d.taken = (uint32_t*)taken;
+        d.base = (uint64_t*)pool;
+    }
+    if (may_allocate && g_host_status[dev].load(std::memory_order_acquire) == nullptr) {
+        void* h = nullptr;
+        if (hipHostMalloc(&h, 64, hipHostMallocDefault) == hipSuccess && h != nullptr) {
+            *(volatile uint32_t*)h = 0;
+            g_host_status[dev].store((uint32_t*)h, std::memory_order_release);
+        } else {
+            (void)hipGetLastError();      // no mirror: time-outs are then only seen by cpmk_async_status()
+        }
+    }
+    *out = &d;
+    if (device != nullptr) *device = dev;
+    return 0;
+}
+
+__global__ void k_xch_take_status(uint32_t* status, uint32_t* taken) {
+    *taken = __hip_atomic_exchange(status, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 }  // namespace
+
+int async_failure() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    const uint32_t* h = g_host_status[dev].load(std::memory_order_acquire);
+    if (h == nullptr) return 0;
+    return (__atomic_load_n(h, __ATOMIC_RELAXED) & kXchStatusTimeout) ? CPMK_ETIMEOUT : 0;
+}
 
 uint32_t xch_next_tag() {
     uint32_t s = g_seq.fetch_add(1, std::memory_order_relaxed) + 1;
@@ -65,95 +99,128 @@ uint32_t xch_next_tag() {
     return s;
 }
 
-int xch_status_word(uint32_t** out) {
+int xch_status_words(uint32_t** device_word, uint32_t** host_word) {
     std::lock_guard<std::mutex> lock(g_mu);
     DevicePool* d = nullptr;
-    if (int rc = device_pool(&d)) return rc;
-    *out = d->status;
+    int dev = 0;
+    if (int rc = device_pool(&d, &dev, false)) return rc;      // (callers of this one may not allocate)
+    *device_word = d->status;
+    *host_word = g_host_status[dev].load(std::memory_order_acquire);
     return 0;
 }
 
-int xch_begin(XchLaunch* out, int64_t slots, hipStream_t st) {
+XchScope::~XchScope() {
+    if (locked_) g_mu.unlock();
+}
+
+int XchScope::begin(int64_t slots, hipStream_t st) {
+    if (locked_) return CPMK_EBADARG;
     if (slots < 1 || slots > kXchSlots) return CPMK_ETOOBIG;
     const int32_t need = (int32_t)(ceil_div(slots, kXchGranule) * kXchGranule);
     const bool cap = capturing(st);
-    std::lock_guard<std::mutex> lock(g_mu);
+    g_mu.lock();
+    locked_ = true;
     DevicePool* d = nullptr;
-    if (int rc = device_pool(&d)) return rc;
-    if (d->head + need > kXchPoolSlots) d->head = 0;
-    const int32_t first = d->head, last = first + need;
-    d->head = last;
-    // whoever last held any of these slots must have finished before this launch starts
-    for (size_t i = 0; i < d->held.size();) {
-        Held& h = d->held[i];
-        if (h.first < last && first < h.last) {
-            if (h.done != nullptr) {
-                if (!cap) {
-                    const hipError_t e = hipStreamWaitEvent(st, h.done, 0);
-                    if (e != hipSuccess) return (int)e;
-                }
+    int dev = 0;
+    if (int rc = device_pool(&d, &dev, !cap)) return rc;
+    int32_t first;
+    if (cap) {
+        // a graph may be replayed at any time: its slots are its own for good
+        if (d->capture_head + need > kXchPoolSlots) {
+            g_mu.unlock();
+            locked_ = false;
+            return kXchFull;
+        }
+        first = d->capture_head;
+        d->capture_head += need;
+    } else {
+        if (d->head + need > kXchRingSlots) d->head = 0;
+        first = d->head;
+        const int32_t last = first + need;
+        d->head = last;
+        // whoever last held any of these slots must have finished before this launch starts
+        for (size_t i = 0; i < d->held.size();) {
+            Held& h = d->held[i];
+            if (h.first < last && first < h.last) {
+                const hipError_t e = hipStreamWaitEvent(st, h.done, 0);
+                if (e != hipSuccess) return (int)e;      // (the entry stays: its slots are still its holder's)
                 d->spare.push_back(h.done);
+                d->held[i] = d->held.back();
+                d->held.pop_back();
+            } else {
+                ++i;
             }
-            d->held[i] = d->held.back();
-            d->held.pop_back();
-        } else {
-            ++i;
         }
     }
-    const uint32_t s = xch_next_tag();
-    out->region = d->base + (size_t)first * kXchVals;
-    out->counters = d->base + (size_t)kXchPoolSlots * kXchVals + first;
-    out->status = d->status;
-    out->tag = s;
-    out->first = first;
-    // the slots are taken from now on, whether or not the launch succeeds
-    d->held.push_back(Held{first, last, nullptr});
+    xl.region = d->base + (size_t)first * kXchVals;
+    xl.counters = d->base + (size_t)kXchPoolSlots * kXchVals + first;
+    xl.status = d->status;
+    xl.host_status = g_host_status[dev].load(std::memory_order_acquire);
+    xl.tag = xch_next_tag();
+    xl.first = first;
+    last_ = first + need;
+    st_ = st;
+    captured_ = cap;
     return 0;
 }
 
-int xch_end(const XchLaunch& xl, hipStream_t st) {
-    if (xl.first < 0) return 0;
-    if (capturing(st)) return 0;         // a graph's replays are not tracked
+int XchScope::end() {
+    if (!locked_) return 0;               // nothing was begun (a launch without packets)
+    int rc = 0;
+    if (!captured_ && xl.first >= 0) {
+        // The slots are taken from now on, whether or not the launch succeeded: the next holder waits for
+        // everything queued on this stream up to here.
+        DevicePool* d = nullptr;
+        rc = device_pool(&d, nullptr, false);
+        if (rc == 0) {
+            hipEvent_t ev = nullptr;
+            if (!d->spare.empty()) {
+                ev = d->spare.back();
+                d->spare.pop_back();
+            } else {
+                const hipError_t e = hipEventCreateWithFlags(&ev, hipEventDisableTiming);
+                if (e != hipSuccess) rc = (int)e;
+            }
+            if (rc == 0) {
+                const hipError_t e = hipEventRecord(ev, st_);
+                if (e != hipSuccess) {
+                    d->spare.push_back(ev);
+                    rc = (int)e;
+                } else {
+                    d->held.push_back(Held{xl.first, last_, ev});
+                }
+            }
+        }
+    }
+    g_mu.unlock();
+    locked_ = false;
+    return rc;
+}
+
+int xch_capture_slots_left(int32_t* slots) {
     std::lock_guard<std::mutex> lock(g_mu);
     DevicePool* d = nullptr;
-    if (int rc = device_pool(&d)) return rc;
-    for (Held& h : d->held) {
-        if (h.first != xl.first || h.done != nullptr) continue;
-        hipEvent_t ev = nullptr;
-        if (!d->spare.empty()) {
-            ev = d->spare.back();
-            d->spare.pop_back();
-        } else {
-            const hipError_t e = hipEventCreateWithFlags(&ev, hipEventDisableTiming);
-            if (e != hipSuccess) return (int)e;
-        }
-        const hipError_t e = hipEventRecord(ev, st);
-        if (e != hipSuccess) {
-            d->spare.push_back(ev);
-            return (int)e;
-        }
-        h.done = ev;
-        break;
-    }
+    if (int rc = device_pool(&d, nullptr, false)) return rc;
+    *slots = kXchPoolSlots - d->capture_head;
     return 0;
 }
 
 int xch_take_status(uint32_t* bits) {
     *bits = 0;
-    uint32_t* status = nullptr;
-    {
-        std::lock_guard<std::mutex> lock(g_mu);
-        DevicePool* d = nullptr;
-        if (int rc = device_pool(&d)) return rc;
-        status = d->status;
-    }
-    uint32_t v = 0;
-    hipError_t e = hipMemcpy(&v, status, sizeof(v), hipMemcpyDeviceToHost);
+    std::lock_guard<std::mutex> lock(g_mu);
+    DevicePool* d = nullptr;
+    int dev = 0;
+    if (int rc = device_pool(&d, &dev, false)) return rc;
+    // read and clear in one step on the device (a flag raised in between is kept for the next call) ...
+    hipLaunchKernelGGL(k_xch_take_status, dim3(1), dim3(1), 0, nullptr, d->status, d->taken);
+    hipError_t e = hipGetLastError();
     if (e != hipSuccess) return (int)e;
-    if (v != 0) {
-        e = hipMemset(status, 0, sizeof(v));
-        if (e != hipSuccess) return (int)e;
-    }
+    uint32_t v = 0;
+    e = hipMemcpy(&v, d->taken, sizeof(v), hipMemcpyDeviceToHost);       // (waits for the kernel: both use the null stream)
+    if (e != hipSuccess) return (int)e;
+    // ... and the mirror on the host
+    uint32_t* h = g_host_status[dev].load(std::memory_order_acquire);
+    if (h != nullptr) v |= __atomic_exchange_n(h, 0u, __ATOMIC_RELAXED);
     *bits = v;
     return 0;
 }
@@ -163,7 +230,7 @@ int xch_take_status(uint32_t* bits) {
 // kernel that still ends normally.
 __global__ void k_xch_selftest(XchLaunch xl, uint64_t ticks) {
     float v;
-    if (threadIdx.x == 0 && !xch_wait(xl.region, xl.tag, wall_clock64() + ticks, v)) xch_flag(xl.status, kXchStatusTimeout);
+    if (threadIdx.x == 0 && !xch_wait(xl.region, xl.tag, wall_clock64() + ticks, v)) xch_flag(xl, kXchStatusTimeout);
 }
 
 }  // namespace cpmk
@@ -178,16 +245,21 @@ int cpmk_async_status(void) {
     return (bits & kXchStatusTimeout) ? CPMK_ETIMEOUT : 0;
 }
 
+int cpmk_exchange_capture_slots_left(int32_t* slots) {
+    if (slots == nullptr) return CPMK_EBADARG;
+    return xch_capture_slots_left(slots);
+}
+
 int cpmk_selftest_exchange_timeout(int32_t microseconds, void* stream) {
     clear_stale_error();
     if (microseconds < 0 || microseconds > 100000) return CPMK_EBADARG;
     hipStream_t st = (hipStream_t)stream;
-    XchLaunch xl;
-    if (int rc = xch_begin(&xl, 1, st)) return rc;
-    hipLaunchKernelGGL(k_xch_selftest, dim3(1), dim3(64), 0, st, xl, (uint64_t)microseconds * 100ull);
-    const int e = launch_status();
-    if (int rc = xch_end(xl, st)) return e ? e : rc;
-    return e;
+    XchScope xs;
+    if (int rc = xs.begin(1, st)) return rc == kXchFull ? CPMK_ETOOBIG : rc;
+    hipLaunchKernelGGL(k_xch_selftest, dim3(1), dim3(64), 0, st, xs.xl, (uint64_t)microseconds * 100ull);
+    const int e = (int)hipGetLastError();
+    const int rc = xs.end();
+    return e ? e : rc;
 }
 
 }  // extern "C"

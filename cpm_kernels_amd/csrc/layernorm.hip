@@ -174,7 +174,7 @@ __global__ __launch_bounds__(NT) void k_layernorm_team(int32_t n, int32_t m, int
         }
         tot[tid] = mu;
         tot[T::COLS + tid] = ok ? rsqrtf(var + eps) : __builtin_nanf("");
-        if (!ok) xch_flag(xl.status, kXchStatusTimeout);
+        if (!ok) xch_flag(xl, kXchStatusTimeout);
     }
     __syncthreads();
     const int cg = tid % LPR;
@@ -313,21 +313,30 @@ static int layernorm_dispatch(int32_t batch, int32_t n, int32_t m, const void* m
             if (parts <= kXchMaxParts && tiles * parts <= kXchSlots) {
                 // one packet slot per (team, part): batches beyond the pool go out in several launches
                 const int64_t per_launch = fixed != nullptr ? batch : kXchSlots / (tiles * parts);
-                for (int64_t b0 = 0; b0 < batch; b0 += per_launch) {
+                bool no_slots = false;
+                for (int64_t b0 = 0; b0 < batch && !no_slots; b0 += per_launch) {
                     const int64_t nb = batch - b0 < per_launch ? batch - b0 : per_launch;
-                    XchLaunch xl;
+                    XchScope xs;
                     if (fixed != nullptr) {
-                        xl = *fixed;
+                        xs.xl = *fixed;
                     } else {
-                        const int rc = xch_begin(&xl, tiles * nb * parts, st);
-                        if (rc != 0) return rc;
+                        const int rc = xs.begin(tiles * nb * parts, st);
+                        if (rc == kXchFull && b0 == 0) {
+                            no_slots = true;       // recorded into a graph and the capture reserve is used up: the kernel without packets below
+                            break;
+                        }
+                        if (rc != 0) return rc == kXchFull ? CPMK_ETOOBIG : rc;
                     }
+                    const XchLaunch& xl = xs.xl;
                     const dim3 grid((unsigned)(tiles * nb * parts));
                     const half_t* xb = x + b0 * n * m;
                     half_t* yb = y + b0 * n * m;
-                    // (one round: every workgroup is resident at once, whatever order they start in)
+                    // Members of a team on one XCD when the launch is one round whose eighths hold whole teams.  With
+                    // the renumbering a team's members are 8 workgroup indices apart, so up to 8 * (parts - 1)
+                    // workgroups of a launch can be waiting for members that have not started when other launches
+                    // share the chip; kept to teams of at most four so that this stays a small part of the chip.
                     const int64_t G = tiles * nb * parts;
-                    const int xcd_local = G % 8 == 0 && (G / 8) % parts == 0 && G <= compute_units() * (big ? 1 : 2);
+                    const int xcd_local = parts <= 4 && G % 8 == 0 && (G / 8) % parts == 0 && G <= compute_units() * (big ? 1 : 2);
                     if (big)
                         hipLaunchKernelGGL((k_layernorm_team<1024, 8>), grid, dim3(1024), 0, st, n, m, (int32_t)tiles,
                                            (int32_t)parts, xb, yb, al, be, eps, rd_mean, xcd_local, xl);
@@ -335,10 +344,10 @@ static int layernorm_dispatch(int32_t batch, int32_t n, int32_t m, const void* m
                         hipLaunchKernelGGL((k_layernorm_team<512, 8>), grid, dim3(512), 0, st, n, m, (int32_t)tiles,
                                            (int32_t)parts, xb, yb, al, be, eps, rd_mean, xcd_local, xl);
                     const int e = launch_status();
-                    const int rc2 = fixed != nullptr ? 0 : xch_end(xl, st);
+                    const int rc2 = xs.end();
                     if (e != 0 || rc2 != 0) return e ? e : rc2;
                 }
-                return 0;
+                if (!no_slots) return 0;
             }
         }
         if (n <= 128 * 8 && m >= 64) ok = launch_tile_r<8>((int)ceil_div(n, 128), batch, n, m, x, y, al, be, eps, rd_mean, st);
@@ -407,7 +416,7 @@ int cpmk_layernorm_forward_noalloc(int32_t batch, int32_t n, int32_t m, const vo
     xl.counters = base + (size_t)kNoAllocSlots * kXchVals;
     xl.tag = xch_next_tag();
     xl.first = -1;
-    if (int rc = xch_status_word(&xl.status)) return rc;
+    if (int rc = xch_status_words(&xl.status, &xl.host_status)) return rc;
     return layernorm_dispatch(batch, n, m, mat, out, nullptr, nullptr, eps, rd_mean, (hipStream_t)stream, &xl, kNoAllocSlots);
 }
 

@@ -259,7 +259,7 @@ __global__ __launch_bounds__(NT) void k_softmax_team(int32_t n, int32_t m, int32
             if (q < parts) S += sp[q] * __builtin_amdgcn_exp2f(mp[q] - M);
         tot[tid] = M;
         tot[T::COLS + tid] = ok ? 1.0f / (S + 1e-10f) : __builtin_nanf("");
-        if (!ok) xch_flag(xl.status, kXchStatusTimeout);
+        if (!ok) xch_flag(xl, kXchStatusTimeout);
     }
     __syncthreads();
     const int cg = tid % LPR;
@@ -357,9 +357,7 @@ static bool launch_tile_r(int r, int32_t batch, int32_t n, int32_t m, const half
 }
 
 // columns taller than this go to the team kernel (single workgroups hold up to 2048 rows at 64-byte row segments)
-#ifndef CPMK_SOFTMAX_TEAM_MIN
-#define CPMK_SOFTMAX_TEAM_MIN 2048
-#endif
+constexpr int32_t kSoftmaxTeamMin = 2048;
 
 static int softmax_dispatch(int32_t batch, int32_t n, int32_t m, const void* inp, void* out, hipStream_t st) {
     if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
@@ -372,32 +370,32 @@ static int softmax_dispatch(int32_t batch, int32_t n, int32_t m, const void* inp
     }
     if (m % 8 == 0 && aligned16(inp) && aligned16(out) && (int64_t)n * m < (1ll << 31)) {
         bool ok = false;
-        if (n > CPMK_SOFTMAX_TEAM_MIN && m >= 64) {
+        if (n > kSoftmaxTeamMin && m >= 64) {
             const int64_t tiles = ceil_div(m, 64);
-            const bool big = n >= 2048;                       // 1024 rows a part, else 512
-            const int64_t parts = ceil_div(n, big ? 1024 : 512);
+            const int64_t parts = ceil_div(n, 1024);          // 1024 rows a part
             if (parts <= kXchMaxParts && tiles * parts <= kXchSlots) {
                 // one packet slot per (team, part): batches beyond the pool go out in several launches
                 const int64_t per_launch = kXchSlots / (tiles * parts);
+                bool no_slots = false;
                 for (int64_t b0 = 0; b0 < batch; b0 += per_launch) {
                     const int64_t nb = batch - b0 < per_launch ? batch - b0 : per_launch;
-                    XchLaunch xl;
-                    const int rc = xch_begin(&xl, tiles * nb * parts, st);
-                    if (rc != 0) return rc;
+                    XchScope xs;
+                    const int rc = xs.begin(tiles * nb * parts, st);
+                    if (rc == kXchFull && b0 == 0) {
+                        no_slots = true;       // recorded into a graph and the capture reserve is used up: a kernel without packets below
+                        break;
+                    }
+                    if (rc != 0) return rc == kXchFull ? CPMK_ETOOBIG : rc;
                     const dim3 grid((unsigned)(tiles * nb * parts));
                     const half_t* xb = x + b0 * n * m;
                     half_t* yb = y + b0 * n * m;
-                    if (big)
-                        hipLaunchKernelGGL((k_softmax_team<1024, 8>), grid, dim3(1024), 0, st, n, m, (int32_t)tiles,
-                                           (int32_t)parts, xb, yb, xl);
-                    else
-                        hipLaunchKernelGGL((k_softmax_team<512, 8>), grid, dim3(512), 0, st, n, m, (int32_t)tiles,
-                                           (int32_t)parts, xb, yb, xl);
+                    hipLaunchKernelGGL((k_softmax_team<1024, 8>), grid, dim3(1024), 0, st, n, m, (int32_t)tiles,
+                                       (int32_t)parts, xb, yb, xs.xl);
                     const int e = launch_status();
-                    const int rc2 = xch_end(xl, st);
+                    const int rc2 = xs.end();
                     if (e != 0 || rc2 != 0) return e ? e : rc2;
                 }
-                return 0;
+                if (!no_slots) return 0;
             }
         }
         // several tiles per compute unit: the persistent kernel keeps loads in flight during the arithmetic

@@ -342,7 +342,7 @@ __global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_b
                 for (int j = 0; j < 8; ++j) acc = IS_MAX ? fmaxf(acc, x[j]) : acc + x[j];     // part order; absent parts are zeros
             }
             tot[tid] = ok ? acc : __builtin_nanf("");
-            if (!ok) xch_flag(xl.status, kXchStatusTimeout);
+            if (!ok) xch_flag(xl, kXchStatusTimeout);
         }
         __syncthreads();
 #pragma unroll
@@ -536,7 +536,7 @@ __global__ __launch_bounds__(256) void k_position_backward_team(int32_t query_le
                 for (int j = 0; j < 8; ++j) acc += x[j];
             }
             grad[(int64_t)h * num_buckets + i] = ok ? (half_t)acc : (half_t)__builtin_nanf("");
-            if (!ok) xch_flag(xl.status, kXchStatusTimeout);
+            if (!ok) xch_flag(xl, kXchStatusTimeout);
         }
         __syncthreads();
     }
@@ -651,21 +651,26 @@ static int launch_col(int32_t batch, const ColArgs& p, void* stream) {
     if (wide) {
         // teams use one packet slot per (team, part): batches beyond the pool go out in several launches
         const int64_t per_launch = parts > 1 ? kXchSlots / (tiles * parts) : ((1ll << 31) - 1) / (tiles * parts);
+        bool no_slots = false;
         for (int64_t b0 = 0; b0 < batch; b0 += per_launch) {
             const int64_t nb = batch - b0 < per_launch ? batch - b0 : per_launch;
             const ColArgs q = col_args_from(p, b0);
-            XchLaunch xl = {nullptr, nullptr, nullptr, 0, -1};
+            XchScope xs;
             if (parts > 1) {
-                const int rc = xch_begin(&xl, tiles * nb * parts, (hipStream_t)stream);
-                if (rc != 0) return rc;
+                const int rc = xs.begin(tiles * nb * parts, (hipStream_t)stream);
+                if (rc == kXchFull && b0 == 0) {
+                    no_slots = true;       // recorded into a graph and the capture reserve is used up: the kernel without packets below
+                    break;
+                }
+                if (rc != 0) return rc == kXchFull ? CPMK_ETOOBIG : rc;
             }
             hipLaunchKernelGGL((k_col_team<KIND>), dim3((unsigned)(tiles * nb * parts)), dim3(512), 0, (hipStream_t)stream, q,
-                               (int32_t)tiles, (int32_t)parts, xl);
+                               (int32_t)tiles, (int32_t)parts, xs.xl);
             const int e = launch_status();
-            const int rc2 = xch_end(xl, (hipStream_t)stream);
+            const int rc2 = xs.end();
             if (e != 0 || rc2 != 0) return e ? e : rc2;
         }
-        return 0;
+        if (!no_slots) return 0;
     }
     // the batch is the grid's y dimension (at most 65535): larger batches go out in several launches
     for (int64_t b0 = 0; b0 < batch; b0 += 65535) {
@@ -843,16 +848,18 @@ int cpmk_position_embedding_backward(int32_t query_len, int32_t key_len, int32_t
         while (ceil_div(key_len, rpp) > kColTeamMaxParts) rpp *= 2;
         const int64_t parts = ceil_div(key_len, rpp);
         if ((int64_t)num_heads * parts <= kXchSlots) {
-            XchLaunch xl;
-            const int rc = xch_begin(&xl, (int64_t)num_heads * parts, (hipStream_t)stream);
-            if (rc != 0) return rc;
-            hipLaunchKernelGGL(k_position_backward_team, dim3((unsigned)(num_heads * parts)), dim3(256),
-                               num_buckets * sizeof(float) + max_distance * sizeof(int32_t), (hipStream_t)stream, query_len, key_len,
-                               num_buckets, max_distance, (const int32_t*)position_mapping, (const half_t*)grad_out, (half_t*)grad,
-                               bidirectional, (int32_t)parts, (int32_t)rpp, xl);
-            const int e = launch_status();
-            const int rc2 = xch_end(xl, (hipStream_t)stream);
-            return e ? e : rc2;
+            XchScope xs;
+            const int rc = xs.begin((int64_t)num_heads * parts, (hipStream_t)stream);
+            if (rc != 0 && rc != kXchFull) return rc;
+            if (rc == 0) {      // (kXchFull: recorded into a graph and the capture reserve is used up: the kernel without packets below)
+                hipLaunchKernelGGL(k_position_backward_team, dim3((unsigned)(num_heads * parts)), dim3(256),
+                                   num_buckets * sizeof(float) + max_distance * sizeof(int32_t), (hipStream_t)stream, query_len, key_len,
+                                   num_buckets, max_distance, (const int32_t*)position_mapping, (const half_t*)grad_out, (half_t*)grad,
+                                   bidirectional, (int32_t)parts, (int32_t)rpp, xs.xl);
+                const int e = launch_status();
+                const int rc2 = xs.end();
+                return e ? e : rc2;
+            }
         }
     }
     hipLaunchKernelGGL(k_position_backward, dim3((unsigned)num_heads), dim3(256), num_buckets * sizeof(float), (hipStream_t)stream,

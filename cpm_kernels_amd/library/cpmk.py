@@ -83,7 +83,7 @@ _LAUNCHERS = {
 
 EXPORTED_SYMBOLS = sorted(list(_LAUNCHERS) + [
     "cpmk_version", "cpmk_error_string", "cpmk_device_count", "cpmk_get_device",
-    "cpmk_set_device", "cpmk_device_props",
+    "cpmk_set_device", "cpmk_device_props", "cpmk_exchange_capture_slots_left",
 ])
 
 
@@ -113,6 +113,23 @@ def _make(name, argtypes):
 
 for _name, _argtypes in _LAUNCHERS.items():
     globals()[_name[len("cpmk_"):]] = _make(_name, _argtypes)
+
+
+def check() -> None:
+    """Raise ``RuntimeError`` if a kernel launched on the current device has failed while it ran (a
+    team of workgroups whose partial results did not arrive in time: the outputs then hold NaN, or 0
+    in int8 tensors), and clear the condition.  Blocks like a device-to-host copy, so it sees all work
+    queued before it on the blocking streams; synchronise non-blocking streams first.  Until it is
+    called, every other call into the library raises the same error (the reference raises pending
+    failures from the status check of whichever call comes next, library/cudart.py:325-327)."""
+    globals()["async_status"]()
+
+
+@lib.bind("cpmk_exchange_capture_slots_left", [ctypes.POINTER(ctypes.c_int32)], ctypes.c_int)
+def exchange_capture_slots_left() -> int:
+    n = ctypes.c_int32(0)
+    checkStatus(lib.cpmk_exchange_capture_slots_left(ctypes.byref(n)))
+    return n.value
 
 
 @lib.bind("cpmk_device_count", [ctypes.POINTER(ctypes.c_int)], ctypes.c_int)

@@ -7,8 +7,9 @@
  *     all buffers (inputs, outputs); nothing is allocated per call.
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).
  *   - Every launcher is asynchronous and returns 0 on success, a hipError_t value if the
- *     HIP runtime reported an error at launch, or a CPMK_E* code (>= 10000) for an
- *     argument the kernels cannot handle.  cpmk_error_string() explains any of them.
+ *     HIP runtime reported an error at launch, a CPMK_E* code (>= 10000) for an
+ *     argument the kernels cannot handle, or CPMK_ETIMEOUT while a failure of an earlier
+ *     kernel is pending (cpmk_async_status).  cpmk_error_string() explains any of them.
  *   - Launch geometry is private to the library (the reference computes grid/block in
  *     its Python wrappers; here the Python wrappers only forward arguments).
  *   - fp16 is IEEE binary16; "b,n,m" tensors are row-major with m contiguous.
@@ -35,7 +36,7 @@ extern "C" {
 #define CPMK_EBADARG   10001  /* negative size, null pointer with non-empty work, ...   */
 #define CPMK_EALIGN    10002  /* divisibility precondition of the reference violated    */
 #define CPMK_ETOOBIG   10003  /* problem exceeds a documented limit of this library     */
-#define CPMK_ETIMEOUT  10004  /* cpmk_async_status: a kernel's bounded wait ran out      */
+#define CPMK_ETIMEOUT  10004  /* a kernel's bounded wait ran out (sticky, see cpmk_async_status) */
 
 /* ---- library / device queries (replace cpm_kernels/library/cudart.py and
  *      cpm_kernels/device/__init__.py:106-158) ------------------------------------ */
@@ -58,14 +59,25 @@ int         cpmk_device_props(int device, char* name, int name_len, int* compute
  * several workgroups (tall layernorm / softmax, the column quantiser, the dim-1 reductions of the
  * training side) wait for each other's partial results with a bound of about one second; a wait
  * that runs out fills the affected outputs with NaN (0 in int8 tensors) and sets a sticky word on
- * the device.  This call copies that word to the host and clears it: 0, CPMK_ETIMEOUT, or a HIP
- * error code.  It blocks like a hipMemcpy, so synchronise the streams in question first.  The
- * reference reports every failure of a launch or a synchronisation as an exception
- * (library/cudart.py:325-327, cudaGetLastError); the Python binding raises on a non-zero value. */
+ * the device and its mirror in pinned host memory.  From then on EVERY launcher of this library
+ * returns CPMK_ETIMEOUT instead of 0 (its own launch is still made), so the failure is reported by
+ * the next call on that device, whichever it is, as the reference reports every failure of a launch
+ * or a synchronisation from its status checks (library/cudart.py:325-327, cudaGetLastError); the
+ * Python binding raises RuntimeError on any non-zero status.  cpmk_async_status() returns the
+ * condition (0, CPMK_ETIMEOUT, or a HIP error code) and clears it; it runs a one-thread kernel on
+ * the null stream and blocks like a hipMemcpy, so it also catches a time-out of work that has only
+ * just finished: synchronise the streams in question first, then call it (a serving loop: once per
+ * step, where it synchronises anyway). */
 int         cpmk_async_status(void);
 /* Launches one workgroup that waits `microseconds` for a result nobody produces and then reports
  * the time-out as above: exercises the failure path with a kernel that ends normally (tests). */
 int         cpmk_selftest_exchange_timeout(int32_t microseconds, void* stream);
+/* A team launch recorded during stream capture is given packet slots that stay its own for good (its
+ * graph may be replayed at any time), out of a reserve of 32768 per device; a tall layernorm of
+ * 8 x 4096 x 512 takes 256.  Writes how many are left on the current device.  When a recorded call
+ * needs more than are left, the library records kernels that need no packets instead (same results
+ * for the exact kernels, the same tolerances for layernorm and softmax, more time). */
+int         cpmk_exchange_capture_slots_left(int32_t* slots);
 
 /* ---- row / column quantisation (kernels/gemm.py, cuda/gemm.cu) ------------------- */
 /* out[b,i] = fp16( max_j |mat[b,i,j]| / 127 )            gemm.py:91-107 / gemm.cu:60-76 */

@@ -219,22 +219,70 @@ def test_more_launches_than_the_pool_holds(gpu):
 
 
 def test_a_wait_that_runs_out_is_reported(gpu):
-    """A workgroup that gives up waiting sets the device's status word; cpmk_async_status turns it into
-    the RuntimeError the reference raises for any failed launch or synchronisation
-    (library/cudart.py:325-327), once, and clears it.  The self-test kernel waits 2 ms for a packet
-    nobody posts and then ends normally."""
+    """A workgroup that gives up waiting sets the device's status word and its mirror in pinned host
+    memory.  From then on every call into the library raises the RuntimeError the reference raises
+    for any failed launch or synchronisation (library/cudart.py:325-327) -- no caller has to ask --
+    until cpmk_async_status has reported the condition once, which clears it.  The self-test kernel
+    waits 2 ms for a packet nobody posts and then ends normally."""
     _name("time-out status")
     from cpm_kernels_amd.library import cpmk
+    import cpm_kernels_amd
     torch.cuda.synchronize()
     cpmk.async_status()
+    x = torch.randn(2, 4096, 64).half().to(gpu); y = torch.empty_like(x); z = torch.empty_like(x)
+    ck.layernorm_forward(2, 4096, 64, x.data_ptr(), y.data_ptr(), 1e-5, True, stream())      # (sets the pool up: the mirror exists from here on)
+    torch.cuda.synchronize()
     cpmk.selftest_exchange_timeout(2000, stream())
     torch.cuda.synchronize()
+    # the next call, whichever it is, reports the failure (its own launch is still made) ...
     with pytest.raises(RuntimeError, match="gave up waiting"):
-        cpmk.async_status()
+        ck.gelu_forward(1, 64, x.data_ptr(), z.data_ptr(), stream())
+    with pytest.raises(RuntimeError, match="gave up waiting"):
+        ck.layernorm_forward(2, 4096, 64, x.data_ptr(), z.data_ptr(), 1e-5, True, stream())
+    # ... until the status call has taken it
+    with pytest.raises(RuntimeError, match="gave up waiting"):
+        cpm_kernels_amd.check()
     cpmk.async_status()                                         # cleared by the read
     # the pool still works afterwards
-    x = torch.randn(2, 4096, 64).half().to(gpu); y = torch.empty_like(x); z = torch.empty_like(x)
-    ck.layernorm_forward(2, 4096, 64, x.data_ptr(), y.data_ptr(), 1e-5, True, stream())
     ck.layernorm_forward(2, 4096, 64, x.data_ptr(), z.data_ptr(), 1e-5, True, stream())
     assert torch.equal(y.view(torch.int16), z.view(torch.int16)) and bool(torch.isfinite(y).all())
     cpmk.async_status()
+
+
+def test_captured_team_launch_between_eager_launches_on_another_stream(gpu):
+    """A tall layernorm recorded into a HIP graph keeps packet slots that no other launch is ever given,
+    so its replays may run while eager team launches on a second stream go round the ring of slots
+    (200 launches of 256 slots wrap the 32768-slot ring): every replay and every eager result equals
+    the single-stream result bit for bit, and no wait runs out."""
+    _name("captured layernorm replayed beside 200 eager team launches on a second stream")
+    from cpm_kernels_amd.library import cpmk
+    g = torch.Generator().manual_seed(45)
+    xa = torch.randn(8, 4096, 512, generator=g).half().to(gpu)
+    xb = (torch.randn(8, 4096, 512, generator=g) * 2 + 0.5).half().to(gpu)
+    ref_a, ref_b = torch.empty_like(xa), torch.empty_like(xb)
+    ck.layernorm_forward(8, 4096, 512, xa.data_ptr(), ref_a.data_ptr(), 1e-5, True, stream())
+    ck.layernorm_forward(8, 4096, 512, xb.data_ptr(), ref_b.data_ptr(), 1e-5, True, stream())
+    torch.cuda.synchronize()
+    cpmk.async_status()
+    left = cpmk.exchange_capture_slots_left()
+    ya = torch.zeros_like(xa)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ck.layernorm_forward(8, 4096, 512, xa.data_ptr(), ya.data_ptr(), 1e-5, True, stream())
+    assert cpmk.exchange_capture_slots_left() == left - 256, "a recorded team launch takes its slots from the capture reserve"
+    sa, sb = torch.cuda.Stream(), torch.cuda.Stream()
+    outs = [torch.zeros_like(xb) for _ in range(4)]
+    for rnd in range(4):
+        ya.fill_(0)
+        torch.cuda.synchronize()
+        for i in range(50):
+            with torch.cuda.stream(sb):
+                ck.layernorm_forward(8, 4096, 512, xb.data_ptr(), outs[i % 4].data_ptr(), 1e-5, True, sb.cuda_stream)
+            if i % 10 == 5:
+                with torch.cuda.stream(sa):
+                    graph.replay()
+        torch.cuda.synchronize()
+        cpmk.async_status()
+        assert_bits_equal(to_np(ya), to_np(ref_a), "replays of round %d" % rnd)
+        for o in outs:
+            assert_bits_equal(to_np(o), to_np(ref_b), "eager launches of round %d" % rnd)

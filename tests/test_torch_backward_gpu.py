@@ -11,6 +11,7 @@ import torch
 import oracle
 from oracle import training as ot
 import cpm_kernels.torch as ct
+import cpm_kernels_amd.torch.layernorm as ctl
 from util import to_np, assert_bits_equal
 
 pytestmark = pytest.mark.gpu
@@ -148,6 +149,50 @@ def test_layernorm_backward(gpu, bias, shape):
     close(l1.weight.grad, l2.weight.grad, 1e-2, 1e-2 * (b * m) ** 0.5, "grad weight")   # reference: 1e-1, 5e-1
     if bias:
         close(l1.bias.grad, l2.bias.grad, 1e-2, 1e-2 * (b * m) ** 0.5, "grad bias")
+
+
+@pytest.mark.parametrize("shape", [(2, 256, 64), (1, 1536, 72)])
+def test_layernorm_ops_with_the_reference_argument_lists(gpu, shape):
+    """OpLayerNormMean(x, eps, weight, bias) and OpLayerNormNoMean(x, eps, weight), the reference's two
+    autograd functions (torch/layernorm.py:7-156): outputs and every gradient equal to OpLayerNorm's bit
+    for bit (they run the same kernels), the right number of gradients for their argument lists, and the
+    output against the oracle's layernorm followed by the fp16 affine."""
+    _name("OpLayerNormMean / OpLayerNormNoMean", shape)
+    b, n, m = shape
+    torch.manual_seed(n * 3 + m)
+    x = torch.randn(shape, device="cuda").half()
+    w = (torch.randn(n, device="cuda") * 0.1 + 1).half()
+    bb = (torch.randn(n, device="cuda") * 0.1).half()
+    rd = torch.randn(shape, device="cuda").half()
+    for mean in (True, False):
+        x1, w1, x2, w2 = leaf(x), leaf(w), leaf(x), leaf(w)
+        if mean:
+            b1, b2 = leaf(bb), leaf(bb)
+            y1 = ctl.OpLayerNormMean.apply(x1, 1e-5, w1, b1)
+            y2 = ctl.OpLayerNorm.apply(x2, 1e-5, w2, b2, True)
+        else:
+            y1 = ctl.OpLayerNormNoMean.apply(x1, 1e-5, w1)
+            y2 = ctl.OpLayerNorm.apply(x2, 1e-5, w2, None, True)
+        assert_bits_equal(to_np(y1), to_np(y2), "forward, mean=%s" % mean)
+        norm = oracle.layernorm_forward(to_np(x), 1e-5, mean).astype(np.float32)
+        wf = to_np(w).astype(np.float32)[None, :, None]
+        exp = norm * wf + (to_np(bb).astype(np.float32)[None, :, None] if mean else 0.0)
+        got = to_np(y1).astype(np.float32)
+        assert np.all(np.abs(got - exp) <= 2e-3 * np.abs(exp) + 2e-3), "forward against the oracle, mean=%s" % mean
+        y1.backward(gradient=rd); y2.backward(gradient=rd)
+        assert_bits_equal(to_np(x1.grad), to_np(x2.grad), "grad x, mean=%s" % mean)
+        assert_bits_equal(to_np(w1.grad), to_np(w2.grad), "grad weight, mean=%s" % mean)
+        if mean:
+            assert_bits_equal(to_np(b1.grad), to_np(b2.grad), "grad bias")
+        # against the TH formulation in fp32, at test_layernorm_backward's bars
+        l2 = ct.LayerNormTH(n, 1e-5, bias=mean).cuda()
+        l2.weight.data = w.float().clone()
+        if mean:
+            l2.bias.data = bb.float().clone()
+        x3 = leaf(x.float())
+        l2(x3).backward(gradient=rd.float())
+        close(x1.grad, x3.grad, 1e-2, 1e-2, "grad x vs TH, mean=%s" % mean)
+        close(w1.grad, l2.weight.grad, 1e-2, 1e-2 * (b * m) ** 0.5, "grad weight vs TH, mean=%s" % mean)
 
 
 @pytest.mark.parametrize("shape", [(2, 128, 64), (3, 1000, 17), (1, 4096, 40)])

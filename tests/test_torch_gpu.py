@@ -65,6 +65,51 @@ def test_bmm_int8(gpu, case, aT, bT):
         assert err < 0.5 and err <= 2e-2 * max(1.0, np.abs(loose).max()), err
 
 
+# The reference's large TEST_CASES at full size (tests/test_gemm.py:55-59), with its generate_matrix
+# (:62-85): batch 8, one side possibly broadcast, each operand possibly stored transposed, values
+# randn / k^(1/4) -- drawn from a seed here instead of `random`.  N = 7996 is not a multiple of 8.
+BMM_FULL_CASES = [(8, 512, 4096, 2048), (8, 500, 4096, 7996), (8, 512, 10240, 4096), (8, 1024, 512, 4096)]
+
+
+@pytest.mark.parametrize("case", BMM_FULL_CASES)
+def test_bmm_reference_cases_full_size(gpu, case):
+    batch, M, K, N = case
+    rng = np.random.default_rng(M + 3 * K + 7 * N)
+    g = torch.Generator().manual_seed(M * 13 + K * 5 + N)
+    for draw in range(2):
+        tp = int(rng.integers(0, 3))
+        bA, bB = (batch, batch) if tp == 0 else ((1, batch) if tp == 1 else (batch, 1))
+        aT, bT = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        _name("bmm full size", case, "draw", draw, "bA", bA, "bB", bB, "aT", aT, "bT", bT)
+        skk = K ** 0.25
+        a = (torch.randn(bA, M, K, generator=g) / skk).half()              # (bA, M, K)
+        b = (torch.randn(bB, N, K, generator=g) / skk).half()              # (bB, N, K): the reference draws (k, n) and transposes; the values are i.i.d. either way
+        A = a.transpose(1, 2).contiguous() if aT else a
+        B = b if bT else b.transpose(1, 2).contiguous()
+        Ad, Bd = A.cuda(), B.cuda()
+        out = ct.bmm(Ad, aT, Bd, bT, int8=True)
+        assert out.shape == (batch, M, N) and out.dtype == torch.half
+        # the oracle's sequence (calc_scale, round, integer product, gemm_scale) on 32 sampled rows of every batch entry
+        a_np, b_np = a.numpy(), b.numpy()
+        sa, sb = oracle.gemm_calc_scale(a_np), oracle.gemm_calc_scale(b_np)
+        qa, qb = oracle.gemm_round(a_np, sa), oracle.gemm_round(b_np, sb)
+        rows = np.sort(rng.choice(M, size=32, replace=False))
+        got = to_np(out[:, torch.from_numpy(rows).cuda(), :])
+        for bi in range(batch):
+            ia, ib = (0 if bA == 1 else bi), (0 if bB == 1 else bi)
+            acc = (qa[ia, rows].astype(np.float64) @ qb[ib].astype(np.float64).T).astype(np.int32)      # exact: |sum| < 2^53
+            ref = oracle.gemm_scale(acc[None], sa[ia:ia + 1, rows].copy(), sb[ib:ib + 1].copy(), False, False)[0]
+            assert_bits_equal(got[bi], ref, "bmm int8 full size, batch entry %d" % bi)
+        # and the fp16 product of the same operands (int8=False) against float64 on the same rows
+        out16 = ct.bmm(Ad, aT, Bd, bT, int8=False)
+        got16 = to_np(out16[:, torch.from_numpy(rows).cuda(), :])
+        for bi in range(0, batch, 3):
+            ia, ib = (0 if bA == 1 else bi), (0 if bB == 1 else bi)
+            ref16 = a_np[ia, rows].astype(np.float64) @ b_np[ib].astype(np.float64).T
+            assert_close_fp16(got16[bi], ref16, rtol=1e-3, atol=1e-3 * float(np.abs(ref16).max()), what="bmm fp16 full size, batch entry %d" % bi)
+        del Ad, Bd, out, out16
+
+
 @pytest.mark.parametrize("aT", [False, True])
 @pytest.mark.parametrize("bT", [False, True])
 def test_bmm_fp16(gpu, aT, bT):
