@@ -37,8 +37,10 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     for (int p = 0; p < R; ++p) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[p][e] = (half_t)0.0f;
-        if (row0 + p < n && col0 < m)
-            v[p] = *reinterpret_cast<const half8_t*>(mat + boff + ((uint32_t)(row0 + p) * (uint32_t)m + (uint32_t)col0));
+        if (row0 + p < n && col0 < m) {
+            const half8_t* src = reinterpret_cast<const half8_t*>(mat + boff + ((uint32_t)(row0 + p) * (uint32_t)m + (uint32_t)col0));
+            v[p] = __builtin_nontemporal_load(src);        // read once; the int8 output below is what the next kernel wants in cache
+        }
     }
     // |x| maxima of the lane's 8 columns as integers; a NaN among them (rare) repeats the maximum in
     // floating point, which skips NaN elements

@@ -208,6 +208,11 @@ __device__ __forceinline__ void lds_dma16(uint32_t voff, const int8_t* sbase, ui
     asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_addr)
                  : "memory");
 }
+// The same with the non-temporal hint: for data that is read once.
+__device__ __forceinline__ void lds_dma16_nt(uint32_t voff, const int8_t* sbase, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1 nt" ::"v"(voff), "s"(sbase), "s"(lds_addr)
+                 : "memory");
+}
 // s_waitcnt vmcnt(N) only (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14)
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {

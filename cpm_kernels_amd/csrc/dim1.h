@@ -11,12 +11,6 @@
 #pragma once
 #include "common.h"
 
-// Column tiles touch row segments shorter than a cache line that neighbouring workgroups
-// complete, so their loads and stores must allocate in L2 (no non-temporal hint).
-#ifndef CPMK_COLTILE_NT
-#define CPMK_COLTILE_NT 0
-#endif
-
 namespace cpmk {
 
 template <int NT, int LPR, int R>
@@ -32,7 +26,11 @@ struct ColTile {
 // (wave-uniform) start of this batch entry; element offsets inside it are 32-bit, which lets
 // the compiler address with a scalar base plus one VGPR offset instead of holding R 64-bit
 // pointers across the reduction phases (callers guarantee n*m < 2^31).
-template <int NT, int LPR, int R>
+//
+// NTL / NTS: non-temporal loads / stores.  Only for tiles whose row segments are whole 128-byte cache
+// lines (LPR == 8) and for data that is not read again soon: a segment shorter than a line is completed
+// by a neighbouring workgroup, so it has to allocate in L2.
+template <int NT, int LPR, int R, bool NTL = false>
 __device__ inline void coltile_load(half8_t (&v)[R], const half_t* base, int32_t n, int32_t m, int32_t col0,
                                     half_t fill) {
     constexpr int RPP = NT / LPR;
@@ -46,13 +44,13 @@ __device__ inline void coltile_load(half8_t (&v)[R], const half_t* base, int32_t
         for (int e = 0; e < 8; ++e) x[e] = fill;
         if (row < n && col0 < m) {
             const half8_t* src = reinterpret_cast<const half8_t*>(base + (off0 + p * stride));
-            x = CPMK_COLTILE_NT ? __builtin_nontemporal_load(src) : *src;
+            x = NTL ? __builtin_nontemporal_load(src) : *src;
         }
         v[p] = x;
     }
 }
 
-template <int NT, int LPR, int R>
+template <int NT, int LPR, int R, bool NTS = false>
 __device__ inline void coltile_store(const half8_t (&v)[R], half_t* base, int32_t n, int32_t m, int32_t col0) {
     constexpr int RPP = NT / LPR;
     const int rg = threadIdx.x / LPR;
@@ -62,7 +60,7 @@ __device__ inline void coltile_store(const half8_t (&v)[R], half_t* base, int32_
         const int32_t row = p * RPP + rg;
         if (row < n && col0 < m) {
             half8_t* dst = reinterpret_cast<half8_t*>(base + (off0 + p * stride));
-            if (CPMK_COLTILE_NT) __builtin_nontemporal_store(v[p], dst);
+            if (NTS) __builtin_nontemporal_store(v[p], dst);
             else *dst = v[p];
         }
     }

@@ -300,13 +300,14 @@ def test_gemm_int8(gpu, case):
 # Tile-kernel coverage: K-major operands with k % 128 == 0 in every dispatch regime -- 256x256 tiles
 # with a last round of half tiles, 128x128 and 128x64 tiles with the four-stage ring (one tile per
 # workgroup, several with the next tile's slabs fetched ahead, slab counts that are not a multiple
-# of the ring depth), ragged edges, output widths that are not a multiple of 8 (register-staged
-# kernel instead), one to many K slabs.
+# of the ring depth), ragged edges, output widths of 8j + 4 columns (fp16 rows that end in half a
+# 16-byte piece and start on 8-byte boundaries: 8-byte stores; N = 7996 of the reference's
+# tests/test_gemm.py:57 is such a width), one to many K slabs.
 TILE_CASES = [  # (batch, kernel n = output rows, k, kernel m = output columns)
     (1, 4096, 512, 3072), (1, 2304, 256, 4608), (1, 2048, 1024, 2048), (1, 3000, 384, 2048), (2, 1500, 640, 1100),
     (1, 128, 128, 64), (1, 132, 128, 72), (1, 100, 256, 60), (3, 260, 384, 520), (1, 512, 128, 4096),
     (1, 520, 1152, 1032), (1, 1024, 896, 1028), (1, 640, 2048, 644), (4, 384, 512, 392), (1, 4100, 128, 2056),
-    (1, 8, 128, 8), (1, 4, 256, 260), (2, 2816, 256, 2304),
+    (1, 8, 128, 8), (1, 4, 256, 260), (2, 2816, 256, 2304), (1, 4096, 256, 3076), (2, 500, 1024, 1996), (1, 2052, 128, 4100),
 ]
 
 
@@ -321,7 +322,7 @@ def test_gemm_int8_tile_kernels(gpu, case):
 
 # int8 operands with the contraction index as the row (the other three aT/bT combinations) on the tile kernel:
 # k % 128 == 0 and row lengths that are multiples of 16; ragged tiles, one to several slabs, batch broadcast.
-LAYOUT_CASES = [(1, 512, 256, 768), (2, 272, 128, 528), (1, 48, 384, 1040), (3, 1040, 640, 16), (1, 2304, 1024, 2064)]
+LAYOUT_CASES = [(1, 512, 256, 768), (2, 272, 128, 528), (1, 48, 384, 1040), (3, 1040, 640, 16), (1, 2304, 1024, 2064), (2, 2048, 256, 2560)]
 
 
 @pytest.mark.parametrize("case", LAYOUT_CASES)
@@ -963,7 +964,9 @@ F16_GEMM_CASES = [  # (batch, n, k, m) in the kernel's convention: out (batch, n
     # several slabs of K and enough 256 x 256 tiles for every compute unit (the 16x16 MFMA form of the tile kernel)
     (48, 512, 256, 512), (50, 520, 320, 264),
     # more 128 x 128 tiles than compute units, at most two each (two workgroups per compute unit, two-stage ring)
-    (24, 512, 128, 512)]
+    (24, 512, 128, 512),
+    # output rows of 8j + 4 halves on the tile kernels (8-byte stores): 128 x 128 tiles, and 256 x 256 on every compute unit
+    (2, 520, 256, 1028), (40, 512, 256, 524)]
 
 
 @pytest.mark.parametrize("case", F16_GEMM_CASES)
