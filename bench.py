@@ -390,22 +390,27 @@ def main():
 
     if only in ("", "gemv"):
         # config 2: W int8 [10240,4096], 32 vectors; 8 weight copies (336 MB) rotate so every
-        # launch streams its matrix from HBM, not from the 256 MB Infinity Cache
+        # launch streams its matrix from HBM, not from the 256 MB Infinity Cache.  Then the decode shapes of
+        # configs 4 and 5 (the FFN's two projections) at 1, 8 and 32 vectors.
         gg = torch.Generator().manual_seed(1002)
         nrot = 8
-        mats = [torch.randint(-127, 128, (10240, 4096), generator=gg, dtype=torch.int8).to(dev) for _ in range(nrot)]
-        smat = (torch.rand(10240, generator=gg) * 0.009 + 0.001).half().to(dev)
-        v = torch.randn(32, 4096, generator=gg).half().to(dev)
-        sv = torch.empty((32,), dtype=torch.half, device=dev); qv = torch.empty((32, 4096), dtype=torch.int8, device=dev)
-        ck.gemv_calc_scale(32, 4096, v.data_ptr(), sv.data_ptr(), st())
-        ck.gemv_round(32, 4096, v.data_ptr(), sv.data_ptr(), qv.data_ptr(), st())
-        o = torch.empty((32, 10240), dtype=torch.half, device=dev)
-        launches = [(lambda m_=m_: ck.gemv_broadcast_mat_int8(32, 10240, 4096, smat.data_ptr(), m_.data_ptr(), sv.data_ptr(),
-                                                               qv.data_ptr(), o.data_ptr(), st())) for m_ in mats]
-        ms, how = graph_ms(launches, max(5, reps // nrot))
-        hbm("gemv_broadcast_mat_int8", 10240 * 4096 + 32 * 4096 + 2 * 32 * 10240 + 2 * 10240 + 2 * 32, ms, how,
-            "W int8 [10240,4096] x 32 vectors", TRAFFIC_BYTES["gemv"])
-        del mats
+        for dim_out, dim_in in ((10240, 4096), (4096, 10240)):
+            mats = [torch.randint(-127, 128, (dim_out, dim_in), generator=gg, dtype=torch.int8).to(dev) for _ in range(nrot)]
+            smat = (torch.rand(dim_out, generator=gg) * 0.009 + 0.001).half().to(dev)
+            for nv in (32, 8, 1):
+                v = torch.randn(nv, dim_in, generator=gg).half().to(dev)
+                sv = torch.empty((nv,), dtype=torch.half, device=dev); qv = torch.empty((nv, dim_in), dtype=torch.int8, device=dev)
+                ck.gemv_calc_scale(nv, dim_in, v.data_ptr(), sv.data_ptr(), st())
+                ck.gemv_round(nv, dim_in, v.data_ptr(), sv.data_ptr(), qv.data_ptr(), st())
+                o = torch.empty((nv, dim_out), dtype=torch.half, device=dev)
+                launches = [(lambda m_=m_: ck.gemv_broadcast_mat_int8(nv, dim_out, dim_in, smat.data_ptr(), m_.data_ptr(), sv.data_ptr(),
+                                                                       qv.data_ptr(), o.data_ptr(), st())) for m_ in mats]
+                ms, how = graph_ms(launches, max(5, reps // nrot))
+                headline = (dim_out, dim_in, nv) == (10240, 4096, 32)
+                hbm("gemv_broadcast_mat_int8" if headline else "gemv_broadcast_mat_int8 [%d,%d] x %d" % (dim_out, dim_in, nv),
+                    dim_out * dim_in + nv * dim_in + 2 * nv * dim_out + 2 * dim_out + 2 * nv, ms, how,
+                    "W int8 [%d,%d] x %d vectors" % (dim_out, dim_in, nv), TRAFFIC_BYTES["gemv"] if headline else None)
+            del mats
 
     if only in ("", "ln"):
         gg = torch.Generator().manual_seed(1003)

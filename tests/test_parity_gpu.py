@@ -483,7 +483,14 @@ def test_north_star_fused_pipeline_bits(gpu):
                                                   (130, 64, 512), (5, 17, 12), (128, 1000, 1040), (8, 40, 16),
                                                   # dim_in 4096: the one-round kernel at 40, 36, 25 (odd), 20, 2 and 1 rows per workgroup, ragged ends
                                                   (32, 10239, 4096), (17, 9000, 4096), (3, 6145, 4096), (16, 5000, 4096),
-                                                  (7, 257, 4096), (1, 256, 4096), (31, 4096, 4096), (32, 10241, 4096)])
+                                                  (7, 257, 4096), (1, 256, 4096), (31, 4096, 4096), (32, 10241, 4096),
+                                                  # other row lengths of whole 256-byte chunks (the chunked kernel): the decode shapes of a 4096 / 10240 FFN
+                                                  # and rows of 2048 and 8192 bytes, at one workgroup per compute unit with 16, 40 and ragged row counts
+                                                  (32, 4096, 10240), (8, 4096, 10240), (1, 4096, 10240), (17, 4001, 10240), (32, 300, 10240),
+                                                  (32, 4096, 8192), (5, 3333, 8192), (16, 100, 8192),
+                                                  (32, 10240, 2048), (20, 7000, 2048), (3, 513, 2048), (32, 4096, 2048),
+                                                  # and with more rows than one workgroup per compute unit holds
+                                                  (32, 5000, 10240), (32, 12500, 2048)])
 def test_gemv_broadcast_mat_int8(gpu, batch, dim_out, dim_in):
     _name("gemv", batch, dim_out, dim_in)
     rng = np.random.default_rng(1002 + dim_out)
