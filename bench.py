@@ -131,11 +131,18 @@ def event_ms(fn, reps, warmup=3, batches=5):
     return sorted(times)[len(times) // 2]
 
 
+GRAPH_NODES = 64    # kernel launches per captured graph
+
+
 def graph_ms(launches, reps):
-    """Capture the list of launch closures once into a HIP graph (no host launch overhead
-    between kernels) and time `reps` replays; returns ms per launch.  Falls back to eager
-    timing if capture is unavailable."""
+    """Capture the launch closures into a HIP graph (no host launch overhead between kernels) and time replays;
+    returns ms per launch.  The list is repeated until the graph holds GRAPH_NODES launches: between two graph
+    launches the device idles for several microseconds, which a short graph charges to its few kernels (an empty
+    kernel costs 2.55 us per launch in a graph of 8 and 1.67 us in a graph of 64).  `reps` = launches of each
+    closure per timed batch.  Falls back to eager timing if capture is unavailable."""
     import torch
+    n = len(launches)
+    copies = max(1, GRAPH_NODES // n) if n < GRAPH_NODES else 1
     try:
         s = torch.cuda.Stream()
         s.wait_stream(torch.cuda.current_stream())
@@ -146,12 +153,13 @@ def graph_ms(launches, reps):
         torch.cuda.synchronize()
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
-            for f in launches:
-                f()
+            for _ in range(copies):
+                for f in launches:
+                    f()
         g.replay()
         torch.cuda.synchronize()
         settle(g.replay)
-        per = max(1, reps // 3)
+        per = max(2, (reps // 3 + copies - 1) // copies)
         times = []
         for _ in range(3):                   # three timed batches of replays, median batch
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -160,8 +168,8 @@ def graph_ms(launches, reps):
                 g.replay()
             e1.record()
             torch.cuda.synchronize()
-            times.append(e0.elapsed_time(e1) / (per * len(launches)))
-        return sorted(times)[1], "hipgraph"
+            times.append(e0.elapsed_time(e1) / (per * n * copies))
+        return sorted(times)[1], "hipgraph of %d launches" % (n * copies)
     except Exception as ex:   # pragma: no cover
         sys.stderr.write("graph capture failed (%s); eager timing\n" % ex)
         i = [0]
@@ -530,10 +538,12 @@ def main():
         VP, I32, I64 = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64
         cl.ceil_mfma_i8.argtypes = [VP, I32, I32, I32, VP, VP]
         cl.ceil_mfma_i8_16x16x64.argtypes = [VP, I32, I32, I32, VP, VP]
-        cl.ceil_read.argtypes = [VP, I64, VP, VP]
+        cl.ceil_read.argtypes = [VP, I64, VP, ctypes.c_int, VP]
+        cl.ceil_read_span.argtypes = [VP, I32, VP, VP, VP]
+        cl.ceil_empty.argtypes = [I32, I32, VP, VP]
         cl.ceil_write.argtypes = [VP, I64, VP]
-        cl.ceil_copy.argtypes = [VP, VP, I64, VP]
-        cl.ceil_copy_segments.argtypes = [VP, VP, I64, I32, I32, VP]
+        cl.ceil_copy.argtypes = [VP, VP, I64, ctypes.c_int, VP]
+        cl.ceil_copy_segments.argtypes = [VP, VP, I64, I32, I32, ctypes.c_int, VP]
 
         def ok(rc):
             assert rc == 0, "yardstick launch failed: %d" % rc
@@ -583,22 +593,41 @@ def main():
 
         def gbs(nbytes, ms):
             return {"us": round(ms * 1e3, 2), "gbs": round(nbytes / (ms * 1e-3) / 1e9, 1), "frac_of_published_peak": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
-        ceil["read_1GiB"] = gbs(nb, event_ms(lambda: ok(cl.ceil_read(big.data_ptr(), nb, sink.data_ptr(), st())), 10))
+        ceil["read_1GiB"] = gbs(nb, event_ms(lambda: ok(cl.ceil_read(big.data_ptr(), nb, sink.data_ptr(), 0, st())), 10))
         ceil["write_1GiB"] = gbs(nb, event_ms(lambda: ok(cl.ceil_write(big2.data_ptr(), nb, st())), 10))
-        ceil["copy_1GiB"] = gbs(2 * nb, event_ms(lambda: ok(cl.ceil_copy(big.data_ptr(), big2.data_ptr(), nb, st())), 10))
+        ceil["copy_1GiB"] = gbs(2 * nb, event_ms(lambda: ok(cl.ceil_copy(big.data_ptr(), big2.data_ptr(), nb, 0, st())), 10))
+        ceil["copy_1GiB_nontemporal"] = gbs(2 * nb, event_ms(lambda: ok(cl.ceil_copy(big.data_ptr(), big2.data_ptr(), nb, 1, st())), 10))
+        # what one kernel launch costs between two others: a kernel that does nothing, in a graph like the per-kernel legs'
+        ms, how = graph_ms([lambda: ok(cl.ceil_empty(256, 512, sink.data_ptr(), st()))], 640)
+        ceil["empty_kernel (what a launch costs in the per-kernel legs)"] = {"us": round(ms * 1e3, 2), "timing": how}
         # the GEMV's traffic: a cold 42 MB read, eight different 42 MB pieces of the buffer in turn (336 MB > Infinity Cache)
         piece = 10240 * 4096
-        ms, how = graph_ms([(lambda i=i: ok(cl.ceil_read(big.data_ptr() + i * (128 << 20), piece, sink.data_ptr(), st()))) for i in range(8)], 10)
-        ceil["cold_read_42MB (gemv traffic)"] = dict(gbs(piece, ms), timing=how)
+        for nt_ in (0, 1):
+            ms, how = graph_ms([(lambda i=i: ok(cl.ceil_read(big.data_ptr() + i * (128 << 20), piece, sink.data_ptr(), nt_, st()))) for i in range(8)], 80)
+            ceil["cold_read_42MB%s (gemv traffic)" % ("_nontemporal" if nt_ else "")] = dict(gbs(piece, ms), timing=how)
+        # the same bytes as one contiguous share per compute unit, every load requested at once (the one-round kernels' shape),
+        # timed inside the kernel: last workgroup's end - first workgroup's start, on the device's 100 MHz wall clock
+        stamps = torch.zeros(8, 512, dtype=torch.int64, device=dev)
+        for _ in range(3):
+            for i in range(8):
+                ok(cl.ceil_read_span(big.data_ptr() + i * (128 << 20), 256, sink.data_ptr(), stamps[i].data_ptr(), st()))
+        torch.cuda.synchronize()
+        sp = stamps.cpu().view(8, 256, 2)
+        span_us = float(((sp[:, :, 1].max(dim=1).values - sp[:, :, 0].min(dim=1).values).double().mean()) * 0.01)
+        ms, how = graph_ms([(lambda i=i: ok(cl.ceil_read_span(big.data_ptr() + i * (128 << 20), 256, sink.data_ptr(), stamps[i].data_ptr(), st()))) for i in range(8)], 80)
+        ceil["cold_read_42MB_one_share_per_compute_unit"] = dict(gbs(piece, ms), timing=how, in_kernel_span_us=round(span_us, 2),
+                                                               in_kernel_span_frac_of_published_peak=round(piece / (span_us * 1e-6) / 1e9 / PEAK_HBM_GBS, 4),
+                                                               note="span = last workgroup's end - first workgroup's start (wall clock stamps inside the kernel); the rest of "
+                                                                    "the per-launch time is what a launch costs (see empty_kernel)")
         # the layernorm's traffic and pattern: [8*4096 rows, 1024 bytes] in 128-byte (and wider) column segments, ten buffers in turn
-        for seg in (128, 256, 512, 1024):
-            ms, how = graph_ms([(lambda i=i: ok(cl.ceil_copy_segments(big.data_ptr() + i * (64 << 20), big2.data_ptr(), 8 * 4096, 1024, seg, st())))
-                                for i in range(10)], 10)
-            ceil["tiled_copy_33.5MB_rows_of_1KB_seg%d (layernorm traffic)" % seg] = dict(gbs(2 * 8 * 4096 * 1024, ms), timing=how)
+        for seg, nt_ in ((128, 0), (128, 1), (256, 1), (1024, 1)):
+            ms, how = graph_ms([(lambda i=i: ok(cl.ceil_copy_segments(big.data_ptr() + i * (64 << 20), big2.data_ptr(), 8 * 4096, 1024, seg, nt_, st())))
+                                for i in range(10)], 60)
+            ceil["tiled_copy_33.5MB_rows_of_1KB_seg%d%s (layernorm traffic)" % (seg, "_nontemporal" if nt_ else "")] = dict(gbs(2 * 8 * 4096 * 1024, ms), timing=how)
         # the softmax's: [512*1024 rows, 2048 bytes], tiles of 1024 x 128 bytes as the kernel holds them, and wider segments
-        for seg in (128, 256, 1024):
-            ms = event_ms(lambda: ok(cl.ceil_copy_segments(big.data_ptr(), big2.data_ptr(), 512 * 1024, 2048, seg, st())), 5)
-            ceil["tiled_copy_1GiB_rows_of_2KB_seg%d (softmax traffic)" % seg] = gbs(2 * nb, ms)
+        for seg, nt_ in ((128, 0), (128, 1), (256, 1), (1024, 1)):
+            ms = event_ms(lambda: ok(cl.ceil_copy_segments(big.data_ptr(), big2.data_ptr(), 512 * 1024, 2048, seg, nt_, st())), 5)
+            ceil["tiled_copy_1GiB_rows_of_2KB_seg%d%s (softmax traffic)" % (seg, "_nontemporal" if nt_ else "")] = gbs(2 * nb, ms)
         del big, big2
         # vendor library, calibration only: torch._int_mm (hipBLASLt) on the north-star and config-1 operands, int32 out
         try:

@@ -8,7 +8,12 @@
 //                       256x256 GEMM tile -- so the result is the matrix pipe's rate on the given
 //                       operand bytes (all zero: the clock stays high; random: it drops)
 //   ceil_mfma_i8_16x16x64   the same wave tile with v_mfma_i32_16x16x64_i8
-//   ceil_read / ceil_write / ceil_copy      contiguous 16-byte accesses
+//   ceil_read / ceil_write / ceil_copy      contiguous 16-byte accesses; `nontemporal` != 0 gives the loads and
+//                       stores the non-temporal hint (data touched once), which a 1 GiB copy rewards with 10 %
+//   ceil_read_span      256 workgroups read one contiguous share each, every load requested at once, and stamp
+//                       their start and end with the 100 MHz wall clock: last end - first start is the time the
+//                       memory system needs for those bytes, without what a kernel launch costs around it
+//   ceil_empty          a kernel that does nothing: what one launch costs between two others
 //   ceil_copy_segments  a (rows, row_bytes) matrix copied in tiles of `seg` bytes x many rows, one
 //                       tile per 1024-thread workgroup, all loads of a tile before its stores: the
 //                       access pattern of the dim-1 kernels (layernorm, softmax) without arithmetic
@@ -85,13 +90,37 @@ __global__ __launch_bounds__(512) void k_mfma_i8_16(const int4_t* __restrict__ o
     if (x == 0x5a5a5a5a) sink[0] = x;
 }
 
+template <bool NTEMP>
 __global__ __launch_bounds__(256) void k_read(const int4_t* __restrict__ p, int64_t n16, int4_t* sink) {
     int64_t i = (int64_t)blockIdx.x * 1024 + threadIdx.x;
     int4_t a = {0, 0, 0, 0};
 #pragma unroll
     for (int u = 0; u < 4; ++u)
-        if (i + u * 256 < n16) a += p[i + u * 256];
+        if (i + u * 256 < n16) a += NTEMP ? __builtin_nontemporal_load(p + i + u * 256) : p[i + u * 256];
     if (a.x == 0x12345678 && a.y == 1) sink[0] = a;
+}
+
+__global__ void k_empty(int4_t* sink) {
+    if (threadIdx.x == 0x7fffffff) sink[0] = int4_t{1, 2, 3, 4};      // never
+}
+
+// 512 threads, NLD pieces of 16 bytes per thread: a share of NLD * 8 KB per workgroup; stamps[2b], [2b+1] = start, end of workgroup b
+template <int NLD>
+__global__ __launch_bounds__(512) void k_read_span(const char* __restrict__ src, int4_t* sink, unsigned long long* stamps) {
+    const unsigned long long t0 = wall_clock64();
+    const char* base = src + (int64_t)blockIdx.x * (NLD * 8192) + threadIdx.x * 16;
+    int4_t v[NLD];
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) v[i] = __builtin_nontemporal_load(reinterpret_cast<const int4_t*>(base + i * 8192));
+    int4_t a = {0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) a += v[i];
+    if (a.x == 0x12345678 && a.y == 1) sink[0] = a;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        stamps[2 * blockIdx.x] = t0;
+        stamps[2 * blockIdx.x + 1] = wall_clock64();
+    }
 }
 
 __global__ __launch_bounds__(256) void k_write(int4_t* p, int64_t n16) {
@@ -102,18 +131,23 @@ __global__ __launch_bounds__(256) void k_write(int4_t* p, int64_t n16) {
         if (i + u * 256 < n16) p[i + u * 256] = v;
 }
 
+template <bool NTEMP>
 __global__ __launch_bounds__(256) void k_copy(const int4_t* __restrict__ p, int4_t* __restrict__ q, int64_t n16) {
     int64_t i = (int64_t)blockIdx.x * 1024 + threadIdx.x;
     int4_t v[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u)
-        if (i + u * 256 < n16) v[u] = p[i + u * 256];
+        if (i + u * 256 < n16) v[u] = NTEMP ? __builtin_nontemporal_load(p + i + u * 256) : p[i + u * 256];
 #pragma unroll
     for (int u = 0; u < 4; ++u)
-        if (i + u * 256 < n16) q[i + u * 256] = v[u];
+        if (i + u * 256 < n16) {
+            if (NTEMP) __builtin_nontemporal_store(v[u], q + i + u * 256);
+            else q[i + u * 256] = v[u];
+        }
 }
 
 // Tile = TROWS rows x seg bytes; a workgroup of 1024 threads holds it in 8 x 16 bytes per thread.
+template <bool NTEMP>
 __global__ __launch_bounds__(1024) void k_copy_segments(const char* __restrict__ src, char* __restrict__ dst, int32_t row_bytes,
                                                         int32_t seg, int32_t tiles_per_row, int32_t tile_rows) {
     const int ppr = seg / 16;                    // 16-byte pieces per row segment
@@ -123,9 +157,16 @@ __global__ __launch_bounds__(1024) void k_copy_segments(const char* __restrict__
     const int r0 = threadIdx.x / ppr;
     int4_t v[8];
 #pragma unroll
-    for (int p = 0; p < 8; ++p) v[p] = *reinterpret_cast<const int4_t*>(src + base + (int64_t)(r0 + p * rpp) * row_bytes);
+    for (int p = 0; p < 8; ++p) {
+        const int4_t* s = reinterpret_cast<const int4_t*>(src + base + (int64_t)(r0 + p * rpp) * row_bytes);
+        v[p] = NTEMP ? __builtin_nontemporal_load(s) : *s;
+    }
 #pragma unroll
-    for (int p = 0; p < 8; ++p) *reinterpret_cast<int4_t*>(dst + base + (int64_t)(r0 + p * rpp) * row_bytes) = v[p];
+    for (int p = 0; p < 8; ++p) {
+        int4_t* d = reinterpret_cast<int4_t*>(dst + base + (int64_t)(r0 + p * rpp) * row_bytes);
+        if (NTEMP) __builtin_nontemporal_store(v[p], d);
+        else *d = v[p];
+    }
 }
 
 int status() { return (int)hipGetLastError(); }
@@ -152,10 +193,25 @@ int ceil_mfma_i8_16x16x64(const void* operands, int32_t workgroups, int32_t wave
     return status();
 }
 
-int ceil_read(const void* src, int64_t bytes, void* sink, void* stream) {
+int ceil_read(const void* src, int64_t bytes, void* sink, int nontemporal, void* stream) {
     const int64_t n16 = bytes / 16;
-    hipLaunchKernelGGL(k_read, dim3((unsigned)((n16 + 1023) / 1024)), dim3(256), 0, (hipStream_t)stream, (const int4_t*)src, n16,
-                       (int4_t*)sink);
+    const dim3 grid((unsigned)((n16 + 1023) / 1024));
+    if (nontemporal) hipLaunchKernelGGL(k_read<true>, grid, dim3(256), 0, (hipStream_t)stream, (const int4_t*)src, n16, (int4_t*)sink);
+    else hipLaunchKernelGGL(k_read<false>, grid, dim3(256), 0, (hipStream_t)stream, (const int4_t*)src, n16, (int4_t*)sink);
+    return status();
+}
+
+// `workgroups` x 20 x 8192 bytes from src, one contiguous share per workgroup; stamps: 2 x workgroups 64-bit words (100 MHz ticks)
+int ceil_read_span(const void* src, int32_t workgroups, void* sink, void* stamps, void* stream) {
+    if (workgroups < 1) return 1;
+    hipLaunchKernelGGL(k_read_span<20>, dim3((unsigned)workgroups), dim3(512), 0, (hipStream_t)stream, (const char*)src, (int4_t*)sink,
+                       (unsigned long long*)stamps);
+    return status();
+}
+
+int ceil_empty(int32_t workgroups, int32_t threads, void* sink, void* stream) {
+    if (workgroups < 1 || threads < 1 || threads > 1024) return 1;
+    hipLaunchKernelGGL(k_empty, dim3((unsigned)workgroups), dim3((unsigned)threads), 0, (hipStream_t)stream, (int4_t*)sink);
     return status();
 }
 
@@ -165,23 +221,28 @@ int ceil_write(void* dst, int64_t bytes, void* stream) {
     return status();
 }
 
-int ceil_copy(const void* src, void* dst, int64_t bytes, void* stream) {
+int ceil_copy(const void* src, void* dst, int64_t bytes, int nontemporal, void* stream) {
     const int64_t n16 = bytes / 16;
-    hipLaunchKernelGGL(k_copy, dim3((unsigned)((n16 + 1023) / 1024)), dim3(256), 0, (hipStream_t)stream, (const int4_t*)src,
-                       (int4_t*)dst, n16);
+    const dim3 grid((unsigned)((n16 + 1023) / 1024));
+    if (nontemporal) hipLaunchKernelGGL(k_copy<true>, grid, dim3(256), 0, (hipStream_t)stream, (const int4_t*)src, (int4_t*)dst, n16);
+    else hipLaunchKernelGGL(k_copy<false>, grid, dim3(256), 0, (hipStream_t)stream, (const int4_t*)src, (int4_t*)dst, n16);
     return status();
 }
 
 // rows x row_bytes matrix; seg in {32, 64, 128, 256, 512, 1024} must divide row_bytes; a tile is
 // 131072 / seg rows, which must divide rows.
-int ceil_copy_segments(const void* src, void* dst, int64_t rows, int32_t row_bytes, int32_t seg, void* stream) {
+int ceil_copy_segments(const void* src, void* dst, int64_t rows, int32_t row_bytes, int32_t seg, int nontemporal, void* stream) {
     if (seg < 32 || seg > 1024 || (seg & (seg - 1)) || row_bytes % seg) return 1;
     const int32_t tile_rows = 131072 / seg;
     if (rows % tile_rows) return 1;
     const int64_t tiles = rows / tile_rows * (row_bytes / seg);
     if (tiles > 0x7fffffff) return 1;
-    hipLaunchKernelGGL(k_copy_segments, dim3((unsigned)tiles), dim3(1024), 0, (hipStream_t)stream, (const char*)src, (char*)dst,
-                       row_bytes, seg, row_bytes / seg, tile_rows);
+    if (nontemporal)
+        hipLaunchKernelGGL(k_copy_segments<true>, dim3((unsigned)tiles), dim3(1024), 0, (hipStream_t)stream, (const char*)src, (char*)dst,
+                           row_bytes, seg, row_bytes / seg, tile_rows);
+    else
+        hipLaunchKernelGGL(k_copy_segments<false>, dim3((unsigned)tiles), dim3(1024), 0, (hipStream_t)stream, (const char*)src, (char*)dst,
+                           row_bytes, seg, row_bytes / seg, tile_rows);
     return status();
 }
 

@@ -20,9 +20,11 @@
 // no other host thread ever sees slots whose holder cannot be waited for.
 // A launch recorded during stream capture cannot be tracked by events (a graph is replayed any
 // number of times, at any time): it gets slots from a reserve of kXchCaptureSlots further slots
-// that the ring never hands out and that are never given to anyone else, so its replays cannot
-// meet the packets of any other launch, eager or captured.  When the reserve is used up XchScope::
-// begin says so (kXchFull) and the caller records its kernel that needs no packets instead.
+// that the ring never hands out.  A range of the reserve belongs to one (capture, stream) pair
+// for good: the launches recorded on one stream during one capture form a chain of graph nodes
+// that run one after the other, so they share a range, and no launch outside that chain, eager
+// or captured, is ever given it.  When the reserve is used up XchScope::begin says so (kXchFull)
+// and the caller records its kernel that needs no packets instead.
 //
 // Progress: a workgroup only ever waits for workgroups of its own team, whose indices differ by
 // less than the team size; the dispatcher starts the workgroups of a launch in index order (an

@@ -22,6 +22,15 @@ struct Held {             // a range of ring slots given to a launch that may st
     hipEvent_t done;      // recorded after the launch
 };
 
+// Slots of the capture reserve belong to one (recording, stream) pair for good.  Launches recorded on one stream
+// during one capture become a chain of graph nodes that run one after the other, and every team launch leaves its
+// slots clean, so they share one range (a graph of many tall layernorms takes the slots of one).
+struct CaptureRange {
+    unsigned long long id;
+    hipStream_t stream;
+    int32_t first, size;
+};
+
 struct DevicePool {
     uint64_t* base = nullptr;       // the pool's address on this device
     uint32_t* status = nullptr;
@@ -30,15 +39,18 @@ struct DevicePool {
     int32_t capture_head = kXchRingSlots;   // next slot of the capture reserve; they are never taken back
     std::vector<Held> held;
     std::vector<hipEvent_t> spare;  // events ready for reuse
+    std::vector<CaptureRange> captured;
 };
 
 std::mutex g_mu;
 DevicePool g_dev[64];
 std::atomic<uint32_t> g_seq{0};
 
-bool capturing(hipStream_t st) {
+// Is `st` recording into a graph?  `id` then identifies the recording (unique per capture).
+bool capturing(hipStream_t st, unsigned long long* id) {
     hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(st, &cs) != hipSuccess) {
+    *id = 0;
+    if (hipStreamGetCaptureInfo(st, &cs, id) != hipSuccess) {
         (void)hipGetLastError();
         return false;
     }
@@ -117,7 +129,8 @@ int XchScope::begin(int64_t slots, hipStream_t st) {
     if (locked_) return CPMK_EBADARG;
     if (slots < 1 || slots > kXchSlots) return CPMK_ETOOBIG;
     const int32_t need = (int32_t)(ceil_div(slots, kXchGranule) * kXchGranule);
-    const bool cap = capturing(st);
+    unsigned long long cap_id = 0;
+    const bool cap = capturing(st, &cap_id);
     g_mu.lock();
     locked_ = true;
     DevicePool* d = nullptr;
@@ -126,13 +139,19 @@ int XchScope::begin(int64_t slots, hipStream_t st) {
     int32_t first;
     if (cap) {
         // a graph may be replayed at any time: its slots are its own for good
-        if (d->capture_head + need > kXchPoolSlots) {
-            g_mu.unlock();
-            locked_ = false;
-            return kXchFull;
+        first = -1;
+        for (const CaptureRange& c : d->captured)
+            if (c.id == cap_id && c.stream == st && c.size >= need) first = c.first;
+        if (first < 0) {
+            if (d->capture_head + need > kXchPoolSlots) {
+                g_mu.unlock();
+                locked_ = false;
+                return kXchFull;
+            }
+            first = d->capture_head;
+            d->capture_head += need;
+            d->captured.push_back(CaptureRange{cap_id, st, first, need});
         }
-        first = d->capture_head;
-        d->capture_head += need;
     } else {
         if (d->head + need > kXchRingSlots) d->head = 0;
         first = d->head;

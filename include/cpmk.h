@@ -72,11 +72,13 @@ int         cpmk_async_status(void);
 /* Launches one workgroup that waits `microseconds` for a result nobody produces and then reports
  * the time-out as above: exercises the failure path with a kernel that ends normally (tests). */
 int         cpmk_selftest_exchange_timeout(int32_t microseconds, void* stream);
-/* A team launch recorded during stream capture is given packet slots that stay its own for good (its
- * graph may be replayed at any time), out of a reserve of 32768 per device; a tall layernorm of
- * 8 x 4096 x 512 takes 256.  Writes how many are left on the current device.  When a recorded call
- * needs more than are left, the library records kernels that need no packets instead (same results
- * for the exact kernels, the same tolerances for layernorm and softmax, more time). */
+/* A team launch recorded during stream capture is given packet slots that stay with its graph for good
+ * (it may be replayed at any time), out of a reserve of 32768 per device; a tall layernorm of
+ * 8 x 4096 x 512 takes 256, and the launches recorded on one stream during one capture, which run one
+ * after the other, share the slots of the largest of them.  Writes how many are left on the current
+ * device.  When a recorded call needs more than are left, the library records kernels that need no
+ * packets instead (same results for the exact kernels, the same tolerances for layernorm and
+ * softmax, more time). */
 int         cpmk_exchange_capture_slots_left(int32_t* slots);
 
 /* ---- row / column quantisation (kernels/gemm.py, cuda/gemm.cu) ------------------- */

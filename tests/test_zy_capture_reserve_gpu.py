@@ -29,28 +29,46 @@ def test_recorded_launches_beyond_the_reserve_run_without_packets(gpu):
     assert cpmk.exchange_capture_slots_left() <= 140 * 256
     ys = [torch.zeros_like(x) for _ in range(4)]
     sm_team = torch.zeros_like(xt); sm = torch.zeros_like(xt); sc = torch.zeros_like(ref_sc); q = torch.zeros_like(ref_q)
-    n_team = 0
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
-        while cpmk.exchange_capture_slots_left() >= 256:           # a tall layernorm of this size takes 256 slots
-            ck.layernorm_forward(8, 4096, 512, x.data_ptr(), ys[n_team % 3].data_ptr(), 1e-5, True, stream())
-            n_team += 1
-        while cpmk.exchange_capture_slots_left() >= 64:            # slots are given out in multiples of 64
-            ck.softmax_forward(2, 4096, 128, xt.data_ptr(), sm_team.data_ptr(), stream())
-        # the reserve is empty: these are recorded as kernels that need no packets
+
+    def record(fn):
+        g_ = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g_):
+            fn()
+        return g_
+
+    # The launches recorded on one stream during one capture share a range of slots (they run one after the other):
+    # three tall layernorms in one graph take the 256 slots of one ...
+    left = cpmk.exchange_capture_slots_left()
+    chain = record(lambda: [ck.layernorm_forward(8, 4096, 512, x.data_ptr(), ys[i].data_ptr(), 1e-5, True, stream()) for i in range(3)])
+    assert cpmk.exchange_capture_slots_left() == left - 256
+    # ... and every capture takes a range of its own: record one launch per graph until the reserve is used up
+    graphs = []
+    while cpmk.exchange_capture_slots_left() >= 256:           # a tall layernorm of this size takes 256 slots
+        graphs.append(record(lambda: ck.layernorm_forward(8, 4096, 512, x.data_ptr(), ys[len(graphs) % 3].data_ptr(), 1e-5, True, stream())))
+    sm_graphs = []
+    while cpmk.exchange_capture_slots_left() >= 64:            # slots are given out in multiples of 64
+        sm_graphs.append(record(lambda: ck.softmax_forward(2, 4096, 128, xt.data_ptr(), sm_team.data_ptr(), stream())))
+    assert cpmk.exchange_capture_slots_left() < 64 and len(graphs) >= 3
+
+    def without_packets():
         ck.layernorm_forward(8, 4096, 512, x.data_ptr(), ys[3].data_ptr(), 1e-5, True, stream())
         ck.softmax_forward(2, 4096, 128, xt.data_ptr(), sm.data_ptr(), stream())
         ck.gemm_quantize_cols(2, 4096, 128, xt.data_ptr(), sc.data_ptr(), q.data_ptr(), True, stream())
-    assert cpmk.exchange_capture_slots_left() < 64 and n_team >= 3
+    last = record(without_packets)                             # the reserve is empty: recorded as kernels that need no packets
     for rep in range(2):
         for y in ys:
             y.fill_(0)
         torch.cuda.synchronize()
-        graph.replay()
+        chain.replay()
+        for g_ in graphs[:4] + graphs[-2:] + sm_graphs:
+            g_.replay()
+        last.replay()
         torch.cuda.synchronize()
         cpmk.async_status()
         for y in ys[:3]:
             assert_bits_equal(to_np(y), to_np(ref), "replay %d: launches with slots" % rep)
+        if sm_graphs:
+            assert_bits_equal(to_np(sm_team), to_np(ref_sm), "replay %d: softmax with slots" % rep)
         # without packets the sums are added in another order: the 1e-3 bar of the path's fp16 outputs, against the oracle
         exp = oracle.layernorm_forward(to_np(x), 1e-5, True)
         assert_close_fp16(to_np(ys[3]), exp.astype(np.float64), rtol=1e-3, atol=2e-4, what="replay %d: launches without slots" % rep)
