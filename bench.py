@@ -399,11 +399,11 @@ def main():
     if only in ("", "gemv"):
         # config 2: W int8 [10240,4096], 32 vectors; 8 weight copies (336 MB) rotate so every
         # launch streams its matrix from HBM, not from the 256 MB Infinity Cache.  Then the decode shapes of
-        # configs 4 and 5 (the FFN's two projections) at 1, 8 and 32 vectors.
+        # configs 4 and 5 (the FFN's two projections and the attention projections) at 1, 8 and 32 vectors.
         gg = torch.Generator().manual_seed(1002)
         nrot = 8
-        for dim_out, dim_in in ((10240, 4096), (4096, 10240)):
-            mats = [torch.randint(-127, 128, (dim_out, dim_in), generator=gg, dtype=torch.int8).to(dev) for _ in range(nrot)]
+        for dim_out, dim_in in ((10240, 4096), (4096, 10240), (4096, 4096)):
+            mats = [torch.randint(-127, 128, (dim_out, dim_in), generator=gg, dtype=torch.int8).to(dev) for _ in range(nrot * (2 if dim_out * dim_in < (32 << 20) else 1))]
             smat = (torch.rand(dim_out, generator=gg) * 0.009 + 0.001).half().to(dev)
             for nv in (32, 8, 1):
                 v = torch.randn(nv, dim_in, generator=gg).half().to(dev)

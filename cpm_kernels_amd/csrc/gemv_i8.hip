@@ -448,14 +448,19 @@ static void launch_coalesced(int32_t batch, int32_t dim_out, int32_t dim_in, con
     go(std::integral_constant<int, 1>{});
 }
 
-// The one-round kernel: dim_in == 4096, at most 32 vectors, and at most 48 rows per compute unit, one
-// workgroup each.  Returns false when the shape does not qualify.
+// The one-round kernel: dim_in == 4096, at most 32 vectors, and 17 to 48 rows per compute unit, one workgroup
+// each.  Returns false when the shape does not qualify.  With at most 16 rows per compute unit the vectors outweigh
+// a workgroup's share of the matrix and the chunked kernel is quicker (32 x [4096, 4096]: 6.3 against 7.1 us; one
+// vector: 5.1 against 5.8).  The same kernel built for rows of 2048, 8192 and 10240 bytes (sixteen waves for the
+// long rows, the vectors straight into registers where the LDS cannot hold them) measured equal (2048) or slower
+// (32 x [4096, 8192]: 15.7 against 10.4 us; 32 x [4096, 10240]: 19.7 against 13.4) than the chunked kernel,
+// which therefore keeps every other row length.
 template <int NB>
 static bool launch_gemv_direct(int32_t batch, int32_t dim_out, int32_t dim_in, const half_t* sm, const int8_t* mat,
                                const half_t* sv, const int8_t* vec, half_t* out, hipStream_t st, int* err) {
     if (dim_in != 4096) return false;
     const int64_t rpb = ceil_div(dim_out, compute_units());
-    if (rpb > 48 || (int64_t)dim_out * dim_in >= (1ll << 32)) return false;
+    if (rpb <= 16 || rpb > 48 || (int64_t)dim_out * dim_in >= (1ll << 32)) return false;
     const int rg = (int)ceil_div(rpb, 16);
     const dim3 grid((unsigned)ceil_div(dim_out, rpb));
     auto go = [&](auto rgc) {
@@ -467,8 +472,7 @@ static bool launch_gemv_direct(int32_t batch, int32_t dim_out, int32_t dim_in, c
         hipLaunchKernelGGL(kern, grid, dim3(512), smem, st, batch, dim_out, (int32_t)rpb, sm, mat, sv, vec, out);
     };
     if (rg == 3) go(std::integral_constant<int, 3>{});
-    else if (rg == 2) go(std::integral_constant<int, 2>{});
-    else go(std::integral_constant<int, 1>{});
+    else go(std::integral_constant<int, 2>{});
     return true;
 }
 
