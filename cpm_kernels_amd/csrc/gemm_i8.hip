@@ -269,6 +269,127 @@ __device__ __forceinline__ void store_piece(int8_t* dst, int4_t v, int32_t left)
     }
 }
 
+// What the two forms of the tile function below share: the rows a wave's DMA instructions fetch, a slab's place in
+// the ring, what the last iterations of a tile fetch (the "tail"), and the priming of the ring at a tile's start.
+// BR x BC outputs per workgroup of NW waves, BKB bytes of K per slab, NST ring stages; LAY / F16 as in the tile functions.
+template <int BR, int BC, int BKB, int NW, int NST, int LAY, bool F16>
+struct SlabDma {
+    static constexpr bool PT = (LAY & 1) != 0, QT = (LAY & 2) != 0;
+    static constexpr int ESZ_IN = F16 ? 2 : 1;            // bytes per operand element
+    static constexpr int EPP = 16 / ESZ_IN;               // elements per 16-byte piece
+    static constexpr int CPR = BKB / 16;                  // 16-byte chunks per row of a slab
+    static constexpr int RPW = 256 / BKB;                 // rows per 256-byte bank wrap
+    static constexpr int STAGE = (BR + BC) * BKB;
+    static constexpr int RPI = 1024 / BKB;                // rows per DMA instruction
+    static constexpr int NDMA = (BR + BC) / RPI;
+    static_assert(NDMA % NW == 0, "stage must split evenly over the waves");
+    static constexpr int CNT = NDMA / NW;                 // DMA instructions per wave and slab
+
+    const GemmArgs& a;
+    const int wave, lane;
+    int nk;                     // slabs per tile
+    bool ahead;                 // the next tile is fetched ahead (only if its LDS layout is this one's)
+    bool deep;                  // at least as many slabs as stages
+    int LD;                     // slabs in flight: the slab requested at iteration `it` is number it + LD of this tile
+    int ring0;                  // stage of this tile's slab 0
+    int32_t tj0, ti0;           // rows / columns the tail fetches
+    const int8_t *Pb, *Qb, *Pn, *Qn;
+    uint32_t voff[CNT], ldst[CNT];
+    bool isq[CNT];
+    int64_t kstepP, kstepQ;     // bytes from one K slab to the next
+
+    __device__ __forceinline__ static int swz(int r) { return (r / RPW) & (CPR - 1); }
+
+    // byte offset of this lane's 16 bytes inside slab 0 of the tile at rows oj / columns oi, for the wave's DMA
+    // instruction d -> stage rows [RPI*dd, RPI*dd + RPI), dd = wave + d*NW; rows past the matrix are clamped (they only
+    // feed outputs that are never stored)
+    __device__ __forceinline__ uint32_t calc_voff(int d, int32_t oj, int32_t oi) const {
+        const int dd = wave + d * NW;
+        const int r = dd * RPI + lane / CPR;
+        const int c = (lane % CPR) ^ swz(r);
+        const bool q = dd * RPI >= BR;
+        if ((PT && !q) || (QT && q)) {
+            // a (K, L) operand: the instruction covers 1024 / (2 * B) rows of K, a lane one 16-byte piece of a row
+            const int ppr = (q ? BC : BR) / EPP;                   // pieces per row of K
+            const int dl = q ? dd - BR / RPI : dd;
+            const int kr = dl * (64 / ppr) + lane / ppr, pc = lane % ppr;
+            const int32_t L = q ? a.m : a.n;
+            return ((uint32_t)kr * (uint32_t)L + (uint32_t)min((q ? oi : oj) + pc * EPP, L - EPP)) * (uint32_t)ESZ_IN;      // L % EPP == 0
+        }
+        const int32_t grow = q ? min(oi + (r - BR), a.m - 1) : min(oj + r, a.n - 1);
+        return (uint32_t)grow * (uint32_t)a.k + c * 16;
+    }
+
+    __device__ __forceinline__ SlabDma(const GemmArgs& a_, uint32_t lds_base, const GemmItem& cur_item, const GemmItem& nxt_item,
+                                       int wave_, int lane_, int ring)
+        : a(a_), wave(wave_), lane(lane_) {
+        nk = a.k / BKB;
+        const uint32_t b = cur_item.b;
+        Pb = a.P + (int64_t)b * a.strideP;
+        Qb = a.Q + (int64_t)b * a.strideQ;
+        ahead = nxt_item.valid && nxt_item.half == cur_item.half;
+        // slab s of this tile lives in stage (ring + s) % NST.  With fewer slabs than stages (!deep) all of a
+        // tile's slabs are requested one tile ahead and every wait is a full one.
+        deep = nk >= NST;
+        LD = deep ? NST : nk;
+        ring0 = __builtin_amdgcn_readfirstlane(ring);
+        // what the last LD iterations fetch: the next tile's first slabs, or (not ahead) this tile's last slab again
+        const uint32_t tb = ahead ? nxt_item.b : b;
+        tj0 = ahead ? nxt_item.j0 : cur_item.j0;
+        ti0 = ahead ? nxt_item.i0 : cur_item.i0;
+        Pn = a.P + (int64_t)tb * a.strideP;
+        Qn = a.Q + (int64_t)tb * a.strideQ;
+#pragma unroll
+        for (int d = 0; d < CNT; ++d) {
+            const int dd = wave + d * NW;
+            isq[d] = dd * RPI >= BR;
+            voff[d] = calc_voff(d, cur_item.j0, cur_item.i0);
+            ldst[d] = lds_base + dd * 1024;
+        }
+        kstepP = PT ? (int64_t)BKB * a.n : BKB;
+        kstepQ = QT ? (int64_t)BKB * a.m : BKB;
+    }
+
+    // One DMA instruction of slab kt into ring stage `stage`: of this tile's rows, or (TAIL) of the rows the last LD
+    // iterations fetch -- the next tile's when it is fetched ahead, else this tile's again.  Which one is a
+    // compile-time choice: a run-time select here makes the compiler branch inside the K loop, which splits its
+    // body and breaks the MFMA/memory interleave.
+    template <int d, bool TAIL>
+    __device__ __forceinline__ void issue(int kt, int stage) const {
+        // read every candidate first and select values, never addresses of the members
+        const int8_t *pb = TAIL ? Pn : Pb, *qb = TAIL ? Qn : Qb;
+        const uint32_t v = voff[d];            // (rewritten for the tail between the two loops: retarget)
+        const bool q = isq[d];
+        lds_dma16(v, (q ? qb : pb) + kt * (q ? kstepQ : kstepP), ldst[d] + stage * STAGE);
+    }
+
+    // between a tile's main iterations and its tail: the offsets of the rows the tail fetches
+    __device__ __forceinline__ void retarget() {
+#pragma unroll
+        for (int d = 0; d < CNT; ++d) voff[d] = calc_voff(d, tj0, ti0);
+    }
+
+    // A tile's start.  Without slabs on their way: request the first NST, wait for slab 0.  Otherwise the first LD
+    // slabs were requested during the previous tile; its stores drain too.
+    __device__ __forceinline__ void prime(bool have_slabs) const {
+        if (!have_slabs) {
+            __syncthreads();                 // every wave is done with the ring of the previous tile
+            static_for<0, NST>([&](auto sc) __attribute__((always_inline)) {
+                constexpr int st = decltype(sc)::value;
+                static_for<0, CNT>([&](auto dc) __attribute__((always_inline)) {
+                    issue<decltype(dc)::value, false>(min(st, nk - 1), (ring0 + st) % NST);
+                });
+            });
+            if (deep) wait_vmcnt<(NST - 1) * CNT>();   // slab 0 (and the scale loads issued before it) has landed
+            else wait_vmcnt<0>();
+            __syncthreads();
+        } else {
+            wait_vmcnt<0>();
+            __syncthreads();
+        }
+    }
+};
+
 // One output tile of BR x BC = (WR*TR*32) x (WC*TC*32), K slab = BKB bytes.
 // The MFMA is the 16x16 one with 64 bytes of K (v_mfma_i32_16x16x64_i8, v_mfma_f32_16x16x32_f16):
 // per operation it moves half the accumulator registers of the 32x32 form, and on random operands,
@@ -312,12 +433,8 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
     static_assert(KS >= 1, "k-steps of 64 bytes");
     constexpr int AR = TR * 2, AC = TC * 2;        // 16x16 MFMA tiles of a wave
     constexpr int NW = WR * WC, BR = WR * TR * 32, BC = WC * TC * 32;
-    constexpr int STAGE = (BR + BC) * BKB;
-    constexpr int RPI = 1024 / BKB;                // rows per DMA instruction
-    constexpr int NDMA = (BR + BC) / RPI;
-    static_assert(NDMA % NW == 0, "stage must split evenly over the waves");
-    constexpr int CNT = NDMA / NW;
-    constexpr int NM = AR * AC;
+    using Dma = SlabDma<BR, BC, BKB, NW, NST, LAY, F16>;
+    constexpr int STAGE = Dma::STAGE, CNT = Dma::CNT;      // bytes per ring stage; DMA instructions per wave and slab
     constexpr int RPW = 256 / BKB;                 // rows per 256-byte bank wrap
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -335,66 +452,13 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
     const int offQ0 = BR * BKB + (QT ? q * EPP * (BC * ESZ_IN) + rq0 * ESZ_IN : rq0 * BKB + ((q ^ swz(rq0)) << 4));
     // without slabs on their way the waits below count only loads: let the previous tile's stores finish first
     if (!have_slabs) wait_vmcnt<0>();
+    Dma dma(a, lds_base, cur_item, nxt_item, wave, lane, ring);
     const uint32_t b = cur_item.b;
     const int32_t j0 = cur_item.j0, i0 = cur_item.i0;
-    const int8_t* Pb = a.P + (int64_t)b * a.strideP;
-    const int8_t* Qb = a.Q + (int64_t)b * a.strideQ;
-    // the next tile is fetched ahead only if its LDS layout is this one's
-    const bool ahead = nxt_item.valid && nxt_item.half == cur_item.half;
-    // slab s of this tile lives in stage (ring + s) % NST; the slab requested at iteration `it` is
-    // number it + LD counted from this tile's slab 0.  With fewer slabs than stages (!deep) all of a
-    // tile's slabs are requested one tile ahead and every wait is a full one.
-    const bool deep = nk >= NST;
-    const int LD = deep ? NST : nk;
-    const int ring0 = __builtin_amdgcn_readfirstlane(ring);
-    // what the last LD iterations fetch: the next tile's first slabs, or (not ahead) this tile's last slab again
-    const uint32_t tb = ahead ? nxt_item.b : b;
-    const int32_t tj0 = ahead ? nxt_item.j0 : j0, ti0 = ahead ? nxt_item.i0 : i0;
-    const int8_t* Pn = a.P + (int64_t)tb * a.strideP;
-    const int8_t* Qn = a.Q + (int64_t)tb * a.strideQ;
-
-    // this wave's DMA instructions: d -> stage rows [RPI*dd, RPI*dd + RPI), dd = wave + d*NW;
-    // rows past the matrix are clamped (they only feed outputs that are never stored)
-    uint32_t voff[CNT], ldst[CNT];
-    bool isq[CNT];
-    // byte offset of this lane's 16 bytes inside slab 0 of the tile at rows oj / columns oi
-    auto calc_voff = [&](int d, int32_t oj, int32_t oi) __attribute__((always_inline)) -> uint32_t {
-        const int dd = wave + d * NW;
-        const int r = dd * RPI + lane / CPR;
-        const int c = (lane % CPR) ^ swz(r);
-        const bool q = dd * RPI >= BR;
-        if ((PT && !q) || (QT && q)) {
-            // a (K, L) operand: the instruction covers 1024 / (2 * B) rows of K, a lane one 16-byte piece of a row
-            const int ppr = (q ? BC : BR) / EPP;                   // pieces per row of K
-            const int dl = q ? dd - BR / RPI : dd;
-            const int kr = dl * (64 / ppr) + lane / ppr, pc = lane % ppr;
-            const int32_t L = q ? a.m : a.n;
-            return ((uint32_t)kr * (uint32_t)L + (uint32_t)min((q ? oi : oj) + pc * EPP, L - EPP)) * (uint32_t)ESZ_IN;      // L % EPP == 0
-        }
-        const int32_t grow = q ? min(oi + (r - BR), a.m - 1) : min(oj + r, a.n - 1);
-        return (uint32_t)grow * (uint32_t)K + c * 16;
-    };
-#pragma unroll
-    for (int d = 0; d < CNT; ++d) {
-        const int dd = wave + d * NW;
-        isq[d] = dd * RPI >= BR;
-        voff[d] = calc_voff(d, j0, i0);
-        ldst[d] = lds_base + dd * 1024;
-    }
-    // bytes from one K slab to the next
-    const int64_t kstepP = PT ? (int64_t)BKB * a.n : BKB, kstepQ = QT ? (int64_t)BKB * a.m : BKB;
-    // One DMA instruction of slab kt: of this tile's rows, or (TAIL) of the rows the last LD iterations
-    // fetch -- the next tile's when it is fetched ahead, else this tile's again.  Which one
-    // is a compile-time choice: a run-time select here makes the compiler branch inside the K loop,
-    // which splits its body and breaks the MFMA/memory interleave.
+    const bool ahead = dma.ahead;
+    const int LD = dma.LD, ring0 = dma.ring0;
     auto dma1 = [&](auto dc, int kt, auto tailc, int stage) __attribute__((always_inline)) {
-        constexpr int d = decltype(dc)::value;
-        constexpr bool TAIL = decltype(tailc)::value;
-        // read every candidate first and select values, never addresses of the captured variables
-        const int8_t *pb = TAIL ? Pn : Pb, *qb = TAIL ? Qn : Qb;
-        const uint32_t v = voff[d];            // (rewritten for the tail between the two loops)
-        const bool q = isq[d];
-        lds_dma16(v, (q ? qb : pb) + kt * (q ? kstepQ : kstepP), ldst[d] + stage * STAGE);
+        dma.template issue<decltype(dc)::value, decltype(tailc)::value>(kt, stage);
     };
 
     // the dequantisation scales of this lane's outputs, fetched now so that the epilogue does
@@ -467,21 +531,7 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
     using I1 = std::integral_constant<int, 1>;
     auto no_memop = [](auto) __attribute__((always_inline)) {};
 
-    if (!have_slabs) {
-        __syncthreads();                 // every wave is done with the ring of the previous tile
-        static_for<0, NST>([&](auto sc) __attribute__((always_inline)) {
-            constexpr int st = decltype(sc)::value;
-            static_for<0, CNT>([&](auto dc) __attribute__((always_inline)) {
-                dma1(dc, min(st, nk - 1), std::false_type{}, (ring0 + st) % NST);
-            });
-        });
-        if (deep) wait_vmcnt<(NST - 1) * CNT>();   // slab 0 (and the scale loads issued before it) has landed
-        else wait_vmcnt<0>();
-        __syncthreads();
-    } else {
-        wait_vmcnt<0>();                 // the first LD slabs were requested during the previous tile; its stores drain too
-        __syncthreads();
-    }
+    dma.prime(have_slabs);
     if (FUSED) {     // pin the scale loads above the K loop (the waits just above cover them)
 #pragma unroll
         for (int i = 0; i < AR; ++i) asm volatile("" : "+v"(sxh[i]));
@@ -522,8 +572,7 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
     };
     int it = 0;
     for (; it < nk - LD; ++it) slab(it, std::false_type{});       // slabs LD .. nk-1 of this tile follow
-#pragma unroll
-    for (int d = 0; d < CNT; ++d) voff[d] = calc_voff(d, tj0, ti0);
+    dma.retarget();
     for (; it < nk; ++it) slab(it, std::true_type{});             // then the tail's
     if (!ahead) wait_vmcnt<0>();         // drain the clamped loads before the ring is reused
     ring = cur;                          // (ring0 + nk) % NST: where the next tile's slab 0 is, or will be put
@@ -635,11 +684,8 @@ __device__ __forceinline__ bool gemm_dma_tile32(const GemmArgs& a, int8_t* smem,
     using acc_t = std::conditional_t<F16, float16_tv, int16_tv>;
     constexpr int KS = BKB / 32, CPR = BKB / 16;
     constexpr int NW = WR * WC, BR = WR * TR * 32, BC = WC * TC * 32;
-    constexpr int STAGE = (BR + BC) * BKB;
-    constexpr int RPI = 1024 / BKB;                // rows per DMA instruction
-    constexpr int NDMA = (BR + BC) / RPI;
-    static_assert(NDMA % NW == 0, "stage must split evenly over the waves");
-    constexpr int CNT = NDMA / NW;
+    using Dma = SlabDma<BR, BC, BKB, NW, NST, LAY, F16>;
+    constexpr int STAGE = Dma::STAGE, CNT = Dma::CNT;      // bytes per ring stage; DMA instructions per wave and slab
     constexpr int NM = TR * TC;
     constexpr int RPW = 256 / BKB;                 // rows per 256-byte bank wrap
     const int tid = threadIdx.x, lane = tid & 63;
@@ -663,66 +709,13 @@ __device__ __forceinline__ bool gemm_dma_tile32(const GemmArgs& a, int8_t* smem,
     }
     // without slabs on their way the waits below count only loads: let the previous tile's stores finish first
     if (!have_slabs) wait_vmcnt<0>();
+    Dma dma(a, lds_base, cur_item, nxt_item, wave, lane, ring);
     const uint32_t b = cur_item.b;
     const int32_t j0 = cur_item.j0, i0 = cur_item.i0;
-    const int8_t* Pb = a.P + (int64_t)b * a.strideP;
-    const int8_t* Qb = a.Q + (int64_t)b * a.strideQ;
-    // the next tile is fetched ahead only if its LDS layout is this one's
-    const bool ahead = nxt_item.valid && nxt_item.half == cur_item.half;
-    // slab s of this tile lives in stage (ring + s) % NST; the slab requested at iteration `it` is
-    // number it + LD counted from this tile's slab 0.  With fewer slabs than stages (!deep) all of a
-    // tile's slabs are requested one tile ahead and every wait is a full one.
-    const bool deep = nk >= NST;
-    const int LD = deep ? NST : nk;
-    const int ring0 = __builtin_amdgcn_readfirstlane(ring);
-    // what the last LD iterations fetch: the next tile's first slabs, or (not ahead) this tile's last slab again
-    const uint32_t tb = ahead ? nxt_item.b : b;
-    const int32_t tj0 = ahead ? nxt_item.j0 : j0, ti0 = ahead ? nxt_item.i0 : i0;
-    const int8_t* Pn = a.P + (int64_t)tb * a.strideP;
-    const int8_t* Qn = a.Q + (int64_t)tb * a.strideQ;
-
-    // this wave's DMA instructions: d -> stage rows [RPI*dd, RPI*dd + RPI), dd = wave + d*NW;
-    // rows past the matrix are clamped (they only feed outputs that are never stored)
-    uint32_t voff[CNT], ldst[CNT];
-    bool isq[CNT];
-    // byte offset of this lane's 16 bytes inside slab 0 of the tile at rows oj / columns oi
-    auto calc_voff = [&](int d, int32_t oj, int32_t oi) __attribute__((always_inline)) -> uint32_t {
-        const int dd = wave + d * NW;
-        const int r = dd * RPI + lane / CPR;
-        const int c = (lane % CPR) ^ swz(r);
-        const bool q = dd * RPI >= BR;
-        if ((PT && !q) || (QT && q)) {
-            // a (K, L) operand: the instruction covers 1024 / (2 * B) rows of K, a lane one 16-byte piece of a row
-            const int ppr = (q ? BC : BR) / EPP;                   // pieces per row of K
-            const int dl = q ? dd - BR / RPI : dd;
-            const int kr = dl * (64 / ppr) + lane / ppr, pc = lane % ppr;
-            const int32_t L = q ? a.m : a.n;
-            return ((uint32_t)kr * (uint32_t)L + (uint32_t)min((q ? oi : oj) + pc * EPP, L - EPP)) * (uint32_t)ESZ_IN;      // L % EPP == 0
-        }
-        const int32_t grow = q ? min(oi + (r - BR), a.m - 1) : min(oj + r, a.n - 1);
-        return (uint32_t)grow * (uint32_t)K + c * 16;
-    };
-#pragma unroll
-    for (int d = 0; d < CNT; ++d) {
-        const int dd = wave + d * NW;
-        isq[d] = dd * RPI >= BR;
-        voff[d] = calc_voff(d, j0, i0);
-        ldst[d] = lds_base + dd * 1024;
-    }
-    // bytes from one K slab to the next
-    const int64_t kstepP = PT ? (int64_t)BKB * a.n : BKB, kstepQ = QT ? (int64_t)BKB * a.m : BKB;
-    // One DMA instruction of slab kt: of this tile's rows, or (TAIL) of the rows the last LD iterations
-    // fetch -- the next tile's when it is fetched ahead, else this tile's again.  Which one
-    // is a compile-time choice: a run-time select here makes the compiler branch inside the K loop,
-    // which splits its body and breaks the MFMA/memory interleave.
+    const bool ahead = dma.ahead;
+    const int LD = dma.LD, ring0 = dma.ring0;
     auto dma1 = [&](auto dc, int kt, auto tailc, int stage) __attribute__((always_inline)) {
-        constexpr int d = decltype(dc)::value;
-        constexpr bool TAIL = decltype(tailc)::value;
-        // read every candidate first and select values, never addresses of the captured variables
-        const int8_t *pb = TAIL ? Pn : Pb, *qb = TAIL ? Qn : Qb;
-        const uint32_t v = voff[d];            // (rewritten for the tail between the two loops)
-        const bool q = isq[d];
-        lds_dma16(v, (q ? qb : pb) + kt * (q ? kstepQ : kstepP), ldst[d] + stage * STAGE);
+        dma.template issue<decltype(dc)::value, decltype(tailc)::value>(kt, stage);
     };
 
     // the dequantisation scales of this lane's outputs, fetched now so that the epilogue does
@@ -788,21 +781,7 @@ __device__ __forceinline__ bool gemm_dma_tile32(const GemmArgs& a, int8_t* smem,
     };
     using C0 = std::integral_constant<int, 0>;
 
-    if (!have_slabs) {
-        __syncthreads();                 // every wave is done with the ring of the previous tile
-        static_for<0, NST>([&](auto sc) __attribute__((always_inline)) {
-            constexpr int st = decltype(sc)::value;
-            static_for<0, CNT>([&](auto dc) __attribute__((always_inline)) {
-                dma1(dc, min(st, nk - 1), std::false_type{}, (ring0 + st) % NST);
-            });
-        });
-        if (deep) wait_vmcnt<(NST - 1) * CNT>();   // slab 0 (and the scale loads issued before it) has landed
-        else wait_vmcnt<0>();
-        __syncthreads();
-    } else {
-        wait_vmcnt<0>();                 // the first LD slabs were requested during the previous tile; its stores drain too
-        __syncthreads();
-    }
+    dma.prime(have_slabs);
     if (FUSED) {     // pin the scale loads above the K loop (the waits just above cover them)
 #pragma unroll
         for (int i = 0; i < TR; ++i) asm volatile("" : "+v"(sxh[i]));
@@ -852,8 +831,7 @@ __device__ __forceinline__ bool gemm_dma_tile32(const GemmArgs& a, int8_t* smem,
     };
     int it = 0;
     for (; it < nk - LD; ++it) slab(it, std::false_type{});       // slabs LD .. nk-1 of this tile follow
-#pragma unroll
-    for (int d = 0; d < CNT; ++d) voff[d] = calc_voff(d, tj0, ti0);
+    dma.retarget();
     for (; it < nk; ++it) slab(it, std::true_type{});             // then the tail's
     if (!ahead) wait_vmcnt<0>();         // drain the clamped loads before the ring is reused
     ring = cur;                          // (ring0 + nk) % NST: where the next tile's slab 0 is, or will be put
@@ -1055,16 +1033,10 @@ static int launch_kmajor(GemmArgs& a, int batch, hipStream_t st) {
     return launch_status();
 }
 
-// waves (rows x cols), MFMA tiles per wave (rows x cols), K bytes per slab of the large-shape kernel
-#ifndef CPMK_GEMM_NST_SMALL
-#define CPMK_GEMM_NST_SMALL 4      // ring stages of the 128x128 and 128x64 tile kernels
-#endif
-#ifndef CPMK_GEMM_BIG
-#define CPMK_GEMM_BIG 2, 4, 4, 2, 128
-#endif
-#ifndef CPMK_GEMM_BIG_NST
-#define CPMK_GEMM_BIG_NST 2        // ring stages of the 256x256 tile kernel (K-major operands)
-#endif
+// Ring stages: four for the 128x128 and 128x64 tile kernels, which finish a slab before a load from L2 returns (two, three,
+// six and eight stages, and slabs of 64 or 256 bytes, all measured 1-3 us slower at 512 x 4096 x 4096); two for the
+// 256x256 tile, whose ring then fills the LDS beside the output strips.
+constexpr int kRingSmall = 4, kRingBig = 2;
 
 template <int WR, int WC, int TR, int TC, int BKB, int EPI, bool HALVES, int NST, int LAY, int MF>
 static int launch_dma_kernel(const DmaArgs& da, unsigned grid, hipStream_t st) {
@@ -1145,7 +1117,7 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
         const int64_t big = ceil_div(n, 256) * ceil_div(m, 256) * batch;
         constexpr int EPI = FUSED ? kEpiDequant : kEpiInt32;
         // (a dimension of at most 128 would leave half or more of every 256-wide tile empty)
-        if (big * 4 >= compute_units() * 3 && n > 128 && m > 128) return launch_dma<CPMK_GEMM_BIG, EPI, CPMK_GEMM_BIG_NST, 0, 16>(a, batch, st);
+        if (big * 4 >= compute_units() * 3 && n > 128 && m > 128) return launch_dma<2, 4, 4, 2, 128, EPI, kRingBig, 0, 16>(a, batch, st);
         // 128x128 tiles, or 128x64 when even those leave a quarter of the compute units idle
         const int64_t mid = ceil_div(n, 128) * ceil_div(m, 128) * batch;
         // the smaller tiles finish a slab before a load from L2 returns: four ring stages keep them fed.  More
@@ -1155,11 +1127,11 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
         const int64_t cus = compute_units();
         if (mid * 4 >= cus * 3) {
             if (mid > cus && mid <= 2 * cus) return launch_dma<2, 2, 2, 2, 128, EPI, 2, 0, 32>(a, batch, st, 2);
-            return launch_dma<2, 2, 2, 2, 128, EPI, CPMK_GEMM_NST_SMALL, 0, 32>(a, batch, st);
+            return launch_dma<2, 2, 2, 2, 128, EPI, kRingSmall, 0, 32>(a, batch, st);
         }
         const int64_t small = ceil_div(n, 128) * ceil_div(m, 64) * batch;
         if (small > cus && small <= 2 * cus) return launch_dma<2, 2, 2, 1, 128, EPI, 2, 0, 32>(a, batch, st, 2);
-        return launch_dma<2, 2, 2, 1, 128, EPI, CPMK_GEMM_NST_SMALL, 0, 32>(a, batch, st);
+        return launch_dma<2, 2, 2, 1, 128, EPI, kRingSmall, 0, 32>(a, batch, st);
     }
     // an operand stored (K, rows): the tile kernel reads it as it lies and gathers the fragments byte by byte in LDS
     if (!(p_kmajor && q_kmajor) && wide && k > 0 && (k % 128 == 0) && aligned16(A) && aligned16(B) && (p_kmajor || n % 16 == 0) &&
@@ -1289,7 +1261,7 @@ static int gemm_f16_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, in
         // (as for int8: more 128x128 tiles than compute units but at most two each -> two workgroups per compute unit)
         const int64_t mid = ceil_div(n, 128) * ceil_div(m, 128) * batch, cus = compute_units();
         if (mid > cus && mid <= 2 * cus) return launch_dma<2, 2, 2, 2, 128, kEpiF16, 2, 0, 32>(a, batch, st, 2);
-        return launch_dma<2, 2, 2, 2, 128, kEpiF16, CPMK_GEMM_NST_SMALL, 0, 32>(a, batch, st);
+        return launch_dma<2, 2, 2, 2, 128, kEpiF16, kRingSmall, 0, 32>(a, batch, st);
     }
     // an operand stored (K, rows): the tile kernel reads it as it lies, with 2-byte LDS reads for the fragments
     if (!(p_kmajor && q_kmajor) && wide && k > 0 && (k % 64 == 0) && aligned16(A) && aligned16(B) && (p_kmajor || n % 8 == 0) &&
