@@ -45,7 +45,7 @@ PROFILES = os.path.join(ROOT, "profiles")
 OFFLINE_SOURCE = {"traffic": "profiles/hbm_traffic_counters.txt (offline rocprofv3 --pmc run of this bench, read at run time, not measured by this process)",
                   "mfma": "profiles/gemm_mfma_utilisation.txt (offline rocprofv3 --pmc run of this bench, read at run time, not measured by this process)"}
 # which row of profiles/hbm_traffic_counters.txt belongs to which workload (a substring of the kernel's name)
-TRAFFIC_KERNELS = {"gemm_fused": "k_gemm_dma<2, 4, 4, 2, 128, 1,", "gemv": "k_gemv", "layernorm": "k_layernorm", "softmax": "k_softmax"}
+TRAFFIC_KERNELS = {"gemm_fused": "k_gemm_dma<2, 4, 4, 2, 128, 1,", "gemv": "k_gemv_directILi2ELi3", "layernorm": "k_layernorm_team", "softmax": "k_softmax_stream"}
 
 
 def offline_counters():
