@@ -544,6 +544,7 @@ def main():
         cl.ceil_write.argtypes = [VP, I64, VP]
         cl.ceil_copy.argtypes = [VP, VP, I64, ctypes.c_int, VP]
         cl.ceil_copy_segments.argtypes = [VP, VP, I64, I32, I32, ctypes.c_int, VP]
+        cl.ceil_copy_segments_persistent.argtypes = [VP, VP, I64, I32, I32, I32, VP, VP]
 
         def ok(rc):
             assert rc == 0, "yardstick launch failed: %d" % rc
@@ -628,6 +629,11 @@ def main():
         for seg, nt_ in ((128, 0), (128, 1), (256, 1), (1024, 1)):
             ms = event_ms(lambda: ok(cl.ceil_copy_segments(big.data_ptr(), big2.data_ptr(), 512 * 1024, 2048, seg, nt_, st())), 5)
             ceil["tiled_copy_1GiB_rows_of_2KB_seg%d%s (softmax traffic)" % (seg, "_nontemporal" if nt_ else "")] = gbs(2 * nb, ms)
+        # the same tiles through persistent workgroups with the next tile in flight and tiles from a counter (the softmax kernel's structure)
+        sched = torch.zeros(2, dtype=torch.int32, device=dev)
+        for seg in (128, 256, 512):
+            ms = event_ms(lambda: ok(cl.ceil_copy_segments_persistent(big.data_ptr(), big2.data_ptr(), 512 * 1024, 2048, seg, cus, sched.data_ptr(), st())), 5)
+            ceil["persistent_tiled_copy_1GiB_rows_of_2KB_seg%d_nontemporal (softmax traffic and structure)" % seg] = gbs(2 * nb, ms)
         del big, big2
         # vendor library, calibration only: torch._int_mm (hipBLASLt) on the north-star and config-1 operands, int32 out
         try:

@@ -10,6 +10,9 @@
 //   ceil_mfma_i8_16x16x64   the same wave tile with v_mfma_i32_16x16x64_i8
 //   ceil_read / ceil_write / ceil_copy      contiguous 16-byte accesses; `nontemporal` != 0 gives the loads and
 //                       stores the non-temporal hint (data touched once), which a 1 GiB copy rewards with 10 %
+//   ceil_copy_segments_persistent   the same tiles through one persistent workgroup per compute unit that loads the next
+//                       tile while it stores the current one and takes its tiles from a counter: what the many-tile
+//                       softmax's structure reaches without its arithmetic
 //   ceil_read_span      256 workgroups read one contiguous share each, every load requested at once, and stamp
 //                       their start and end with the 100 MHz wall clock: last end - first start is the time the
 //                       memory system needs for those bytes, without what a kernel launch costs around it
@@ -169,6 +172,49 @@ __global__ __launch_bounds__(1024) void k_copy_segments(const char* __restrict__
     }
 }
 
+// The same tiles copied by persistent workgroups (one per compute unit) that load the next tile while they store the
+// current one and take their tiles from a counter in device memory: the shape of the library's many-tile softmax.
+// sched[0] = tiles handed out beyond the first round, sched[1] = workgroups done (the last one clears both).
+template <int LPR>
+__global__ __launch_bounds__(1024) void k_copy_segments_persistent(const char* __restrict__ src, char* __restrict__ dst, int32_t row_bytes,
+                                                                   uint32_t ntiles, unsigned int* sched) {
+    constexpr int SEG = LPR * 16, RPP = 1024 / LPR, ROWS = RPP * 8;
+    __shared__ uint32_t s_next;
+    const int tid = threadIdx.x, cg = tid % LPR, rg = tid / LPR;
+    const uint32_t tpr = (uint32_t)row_bytes / SEG;
+    auto addr = [&](uint32_t t, int p) -> int64_t {
+        const int64_t tr = t / tpr, tc = t % tpr;
+        return (tr * ROWS + p * RPP + rg) * row_bytes + tc * SEG + cg * 16;
+    };
+    uint32_t t = blockIdx.x;
+    int4_t v[8], w[8];
+#pragma unroll
+    for (int p = 0; p < 8; ++p) v[p] = __builtin_nontemporal_load(reinterpret_cast<const int4_t*>(src + addr(t, p)));
+    if (tid == 0) s_next = gridDim.x + atomicAdd(&sched[0], 1u);
+    __syncthreads();
+    uint32_t tn = s_next;
+    while (t < ntiles) {
+        if (tn < ntiles) {
+#pragma unroll
+            for (int p = 0; p < 8; ++p) w[p] = __builtin_nontemporal_load(reinterpret_cast<const int4_t*>(src + addr(tn, p)));
+        }
+        __syncthreads();
+        if (tid == 0) s_next = gridDim.x + atomicAdd(&sched[0], 1u);
+        __syncthreads();
+        const uint32_t tnn = s_next;
+#pragma unroll
+        for (int p = 0; p < 8; ++p) __builtin_nontemporal_store(v[p], reinterpret_cast<int4_t*>(dst + addr(t, p)));
+#pragma unroll
+        for (int p = 0; p < 8; ++p) v[p] = w[p];
+        t = tn;
+        tn = tnn;
+    }
+    if (tid == 0 && atomicAdd(&sched[1], 1u) == gridDim.x - 1) {
+        atomicExch(&sched[0], 0u);
+        atomicExch(&sched[1], 0u);
+    }
+}
+
 int status() { return (int)hipGetLastError(); }
 
 }  // namespace
@@ -243,6 +289,28 @@ int ceil_copy_segments(const void* src, void* dst, int64_t rows, int32_t row_byt
     else
         hipLaunchKernelGGL(k_copy_segments<false>, dim3((unsigned)tiles), dim3(1024), 0, (hipStream_t)stream, (const char*)src, (char*)dst,
                            row_bytes, seg, row_bytes / seg, tile_rows);
+    return status();
+}
+
+// The persistent form: `workgroups` workgroups (at most the number of tiles); seg in {128, 256, 512}; sched: two zeroed 32-bit words
+// that the kernel leaves zeroed.  rows must be a multiple of the tile's 131072 / seg rows.
+int ceil_copy_segments_persistent(const void* src, void* dst, int64_t rows, int32_t row_bytes, int32_t seg, int32_t workgroups, void* sched,
+                                  void* stream) {
+    if ((seg != 128 && seg != 256 && seg != 512) || row_bytes % seg) return 1;
+    const int32_t tile_rows = 131072 / seg;
+    if (rows % tile_rows) return 1;
+    const int64_t tiles = rows / tile_rows * (row_bytes / seg);
+    if (tiles > 0x7fffffff || workgroups < 1 || workgroups > tiles) return 1;
+    const dim3 grid((unsigned)workgroups);
+    if (seg == 128)
+        hipLaunchKernelGGL(k_copy_segments_persistent<8>, grid, dim3(1024), 0, (hipStream_t)stream, (const char*)src, (char*)dst, row_bytes,
+                           (uint32_t)tiles, (unsigned int*)sched);
+    else if (seg == 256)
+        hipLaunchKernelGGL(k_copy_segments_persistent<16>, grid, dim3(1024), 0, (hipStream_t)stream, (const char*)src, (char*)dst, row_bytes,
+                           (uint32_t)tiles, (unsigned int*)sched);
+    else
+        hipLaunchKernelGGL(k_copy_segments_persistent<32>, grid, dim3(1024), 0, (hipStream_t)stream, (const char*)src, (char*)dst, row_bytes,
+                           (uint32_t)tiles, (unsigned int*)sched);
     return status();
 }
 
