@@ -131,6 +131,38 @@ def event_ms(fn, reps, warmup=3, batches=5):
     return sorted(times)[len(times) // 2]
 
 
+def sclk_under_load(fn, seconds):
+    """Median shader clock in MHz that `rocm-smi --showclocks` reports while fn is launched back to back for `seconds`
+    (None if the tool is missing or prints nothing usable)."""
+    import re
+    import subprocess
+    import threading
+    import torch
+    samples, stop = [], [False]
+
+    def sampler():
+        while not stop[0]:
+            try:
+                out = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=5).stdout
+            except Exception:
+                return
+            m = re.search(r"sclk clock level:?\s*\d+:?\s*\((\d+)Mhz\)", out)
+            if m:
+                samples.append(int(m.group(1)))
+            time.sleep(0.1)
+    th = threading.Thread(target=sampler)
+    th.start()
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(50):
+            fn()
+        torch.cuda.synchronize()
+    stop[0] = True
+    th.join()
+    samples = sorted(samples[1:] or samples)      # (the first sample may predate the load)
+    return samples[len(samples) // 2] if samples else None
+
+
 GRAPH_NODES = 64    # kernel launches per captured graph
 
 
@@ -269,6 +301,22 @@ def main():
                     "traffic_source": OFFLINE_SOURCE["traffic"],
                     "mfma_busy_frac_of_cycles": MFMA_BUSY_FRAC, "mfma_busy_source": OFFLINE_SOURCE["mfma"],
                     "algorithmic_bytes": M * K + N * K + 2 * M * N}
+        # The shader clock under this kernel, as the driver's monitoring tool reports it while the kernel runs back to back for a
+        # second (not inside a timed loop: a sample stalls the device for a moment), on the step's operands and on all-zero
+        # ones: the kernel needs the same number of cycles for both, the chip clocks lower on the operands that toggle.
+        qz_a, qz_w = torch.zeros_like(qA), torch.zeros_like(qW)
+
+        def gemm_zero():
+            ck.gemm_int8_scale(N, K, M, 1, 1, True, False, qz_w.data_ptr(), qz_a.data_ptr(), sA.data_ptr(), sW.data_ptr(),
+                               True, True, out16.data_ptr(), st())
+        clocks = {}
+        for label, fn in (("step_operands", gemm), ("zero_operands", gemm_zero)):
+            mhz = sclk_under_load(fn, 1.2)
+            ms_l = event_ms(fn, 20, warmup=3)
+            clocks[label] = {"sclk_mhz": mhz, "kernel_us": round(ms_l * 1e3, 2),
+                             "kilocycles": round(ms_l * 1e3 * mhz / 1e3, 1) if mhz else None}
+        roofline["clock_under_load"] = dict(clocks, source="rocm-smi --showclocks sampled while the kernel runs back to back; kilocycles = kernel_us x sclk")
+        del qz_a, qz_w
         out32 = torch.empty((1, M, N), dtype=torch.int32, device=dev)
 
         def gemm32():

@@ -1,6 +1,6 @@
 // Library and device queries of the C ABI (the part of cpm_kernels/library/cudart.py and
 // cpm_kernels/device/__init__.py the path needs), plus error strings.
-#include "common.h"
+#include "exchange.h"
 #include <string.h>
 
 extern "C" {
@@ -20,7 +20,11 @@ const char* cpmk_error_string(int code) {
 
 int cpmk_device_count(int* count) { return (int)hipGetDeviceCount(count); }
 int cpmk_get_device(int* device) { return (int)hipGetDevice(device); }
-int cpmk_set_device(int device) { return (int)hipSetDevice(device); }
+int cpmk_set_device(int device) {
+    const hipError_t e = hipSetDevice(device);
+    if (e == hipSuccess) cpmk::xch_prepare();      // (the packet pool's one host allocation, outside any stream capture)
+    return (int)e;
+}
 
 int cpmk_device_props(int device, char* name, int name_len, int* compute_units, int* lds_bytes, int* wavefront,
                       int* clock_khz, int* mem_clock_khz, int* mem_bus_bits, int* l2_bytes,

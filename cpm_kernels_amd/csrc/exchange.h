@@ -88,6 +88,9 @@ uint32_t xch_next_tag();
 // Host: the addresses of the current device's status word and of its host mirror (nullptr if none), for such a
 // launch.  0 or an error code.
 int xch_status_words(uint32_t** device_word, uint32_t** host_word);
+// Host: sets the current device's pool up (symbol addresses, the status word's host mirror) ahead of the first team launch, so
+// that a process whose first team launch is recorded during stream capture has the mirror too.  Failures are left to that launch.
+void xch_prepare();
 // Host: slots left in the current device's capture reserve.  0 or an error code.
 int xch_capture_slots_left(int32_t* slots);
 // Host: reads and clears the current device's status word and its mirror (0, kXchStatus* bits; an error code on failure to read).

@@ -153,16 +153,18 @@ int XchScope::begin(int64_t slots, hipStream_t st) {
             d->captured.push_back(CaptureRange{cap_id, st, first, need});
         }
     } else {
-        if (d->head + need > kXchRingSlots) d->head = 0;
-        first = d->head;
+        first = d->head + need > kXchRingSlots ? 0 : d->head;
         const int32_t last = first + need;
-        d->head = last;
-        // whoever last held any of these slots must have finished before this launch starts
+        // whoever last held any of these slots must have finished before this launch starts; nothing of the
+        // bookkeeping changes until every wait is queued, so a failure here leaves the ring as it was
+        for (const Held& h : d->held)
+            if (h.first < last && first < h.last) {
+                const hipError_t e = hipStreamWaitEvent(st, h.done, 0);
+                if (e != hipSuccess) return (int)e;
+            }
         for (size_t i = 0; i < d->held.size();) {
             Held& h = d->held[i];
             if (h.first < last && first < h.last) {
-                const hipError_t e = hipStreamWaitEvent(st, h.done, 0);
-                if (e != hipSuccess) return (int)e;      // (the entry stays: its slots are still its holder's)
                 d->spare.push_back(h.done);
                 d->held[i] = d->held.back();
                 d->held.pop_back();
@@ -170,6 +172,7 @@ int XchScope::begin(int64_t slots, hipStream_t st) {
                 ++i;
             }
         }
+        d->head = last;
     }
     xl.region = d->base + (size_t)first * kXchVals;
     xl.counters = d->base + (size_t)kXchPoolSlots * kXchVals + first;
@@ -214,6 +217,12 @@ int XchScope::end() {
     g_mu.unlock();
     locked_ = false;
     return rc;
+}
+
+void xch_prepare() {
+    std::lock_guard<std::mutex> lock(g_mu);
+    DevicePool* d = nullptr;
+    (void)device_pool(&d, nullptr, true);
 }
 
 int xch_capture_slots_left(int32_t* slots) {
