@@ -132,24 +132,34 @@ def event_ms(fn, reps, warmup=3, batches=5):
 
 
 def sclk_under_load(fn, seconds):
-    """Median shader clock in MHz that `rocm-smi --showclocks` reports while fn is launched back to back for `seconds`
-    (None if the tool is missing or prints nothing usable)."""
+    """Median shader clock in MHz that the driver reports (the current level of pp_dpm_sclk in sysfs, the file the
+    monitoring tools read) while fn is launched back to back for `seconds`; None if no such file can be read.
+    The file is read in this process: nothing is spawned."""
+    import glob
     import re
-    import subprocess
     import threading
     import torch
+    paths = sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"))
     samples, stop = [], [False]
+
+    def current_mhz():
+        for p in paths:
+            try:
+                with open(p) as f:
+                    m = re.search(r"(\d+)Mhz\s*\*", f.read())
+            except OSError:
+                continue
+            if m:
+                return int(m.group(1))
+        return None
 
     def sampler():
         while not stop[0]:
-            try:
-                out = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=5).stdout
-            except Exception:
+            v = current_mhz()
+            if v is None:
                 return
-            m = re.search(r"sclk clock level:?\s*\d+:?\s*\((\d+)Mhz\)", out)
-            if m:
-                samples.append(int(m.group(1)))
-            time.sleep(0.1)
+            samples.append(v)
+            time.sleep(0.05)
     th = threading.Thread(target=sampler)
     th.start()
     t0 = time.perf_counter()
@@ -159,7 +169,7 @@ def sclk_under_load(fn, seconds):
         torch.cuda.synchronize()
     stop[0] = True
     th.join()
-    samples = sorted(samples[1:] or samples)      # (the first sample may predate the load)
+    samples = sorted(samples[2:] or samples)      # (the first samples may predate the load)
     return samples[len(samples) // 2] if samples else None
 
 
@@ -289,20 +299,8 @@ def main():
         def gemm():
             ck.gemm_int8_scale(N, K, M, 1, 1, True, False, qW.data_ptr(), qA.data_ptr(), sA.data_ptr(), sW.data_ptr(),
                                True, True, out16.data_ptr(), st())
-        ms = event_ms(gemm, max(20, args.steps), warmup=max(3, args.warmup))
-        tops = ops / (ms * 1e-3) / 1e12
-        roofline = {"kernel": "k_gemm_dma<2,4,4,2,128,1,true,2,0,16> (int8 MFMA GEMM + fused fp16 dequant), M=%d K=%d N=%d" % (M, K, N),
-                    "bound": "mfma", "achieved": round(tops, 2), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
-                    "ops": "int8 multiply-accumulates counted as 2 ops",
-                    "frac": round(tops / PEAK_INT8_TOPS, 4), "avg_kernel_us": round(ms * 1e3, 2),
-                    "peak_clock_derived": round(peak_int8_clock, 1), "frac_of_clock_derived": round(tops / peak_int8_clock, 4),
-                    "operands": "MALL-resident (one 58.7 MB operand pair and one 83.9 MB output reused by every launch)",
-                    "traffic": TRAFFIC_BYTES["gemm_fused"], "traffic_unit": "bytes per launch (HBM fetch + write counters)",
-                    "traffic_source": OFFLINE_SOURCE["traffic"],
-                    "mfma_busy_frac_of_cycles": MFMA_BUSY_FRAC, "mfma_busy_source": OFFLINE_SOURCE["mfma"],
-                    "algorithmic_bytes": M * K + N * K + 2 * M * N}
-        # The shader clock under this kernel, as the driver's monitoring tool reports it while the kernel runs back to back for a
-        # second (not inside a timed loop: a sample stalls the device for a moment), on the step's operands and on all-zero
+        # The shader clock under this kernel, as the driver reports it while the kernel runs back to back for a
+        # second (not inside a timed loop: a sample may stall the device for a moment), on the step's operands and on all-zero
         # ones: the kernel needs the same number of cycles for both, the chip clocks lower on the operands that toggle.
         qz_a, qz_w = torch.zeros_like(qA), torch.zeros_like(qW)
 
@@ -315,8 +313,20 @@ def main():
             ms_l = event_ms(fn, 20, warmup=3)
             clocks[label] = {"sclk_mhz": mhz, "kernel_us": round(ms_l * 1e3, 2),
                              "kilocycles": round(ms_l * 1e3 * mhz / 1e3, 1) if mhz else None}
-        roofline["clock_under_load"] = dict(clocks, source="rocm-smi --showclocks sampled while the kernel runs back to back; kilocycles = kernel_us x sclk")
+        clock_under_load = dict(clocks, source="current level of /sys/class/drm/card*/device/pp_dpm_sclk sampled while the kernel runs back to back; kilocycles = kernel_us x sclk")
         del qz_a, qz_w
+        ms = event_ms(gemm, max(20, args.steps), warmup=max(3, args.warmup))
+        tops = ops / (ms * 1e-3) / 1e12
+        roofline = {"kernel": "k_gemm_dma<2,4,4,2,128,1,true,2,0,16> (int8 MFMA GEMM + fused fp16 dequant), M=%d K=%d N=%d" % (M, K, N),
+                    "bound": "mfma", "achieved": round(tops, 2), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
+                    "ops": "int8 multiply-accumulates counted as 2 ops",
+                    "frac": round(tops / PEAK_INT8_TOPS, 4), "avg_kernel_us": round(ms * 1e3, 2),
+                    "peak_clock_derived": round(peak_int8_clock, 1), "frac_of_clock_derived": round(tops / peak_int8_clock, 4),
+                    "operands": "MALL-resident (one 58.7 MB operand pair and one 83.9 MB output reused by every launch)",
+                    "traffic": TRAFFIC_BYTES["gemm_fused"], "traffic_unit": "bytes per launch (HBM fetch + write counters)",
+                    "traffic_source": OFFLINE_SOURCE["traffic"],
+                    "mfma_busy_frac_of_cycles": MFMA_BUSY_FRAC, "mfma_busy_source": OFFLINE_SOURCE["mfma"],
+                    "algorithmic_bytes": M * K + N * K + 2 * M * N, "clock_under_load": clock_under_load}
         out32 = torch.empty((1, M, N), dtype=torch.int32, device=dev)
 
         def gemm32():
