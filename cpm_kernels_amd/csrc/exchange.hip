@@ -58,7 +58,7 @@ bool capturing(hipStream_t st, unsigned long long* id) {
 }
 
 // `may_allocate`: the caller is not recording into a graph, so the one-time allocation of the status word's
-// host mirror (4 bytes of pinned memory per device) may be made now; otherwise it is left for a later call.
+// host mirror (64 bytes of pinned memory per device) may be made now; otherwise it is left for a later call.
 int device_pool(DevicePool** out, int* device, bool may_allocate) {      // g_mu held
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
@@ -122,7 +122,7 @@ int xch_status_words(uint32_t** device_word, uint32_t** host_word) {
 }
 
 XchScope::~XchScope() {
-    if (locked_) g_mu.unlock();
+    if (locked_) (void)end();      // a caller that left early: whatever it launched is still waited for by the next holder
 }
 
 int XchScope::begin(int64_t slots, hipStream_t st) {
