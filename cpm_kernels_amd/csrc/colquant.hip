@@ -196,7 +196,9 @@ int cpmk_gemm_quantize_cols(int32_t batch, int32_t n, int32_t m, const void* mat
                             int out_transposed, void* stream) {
     clear_stale_error();
     if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
-    if ((int64_t)batch * n * m == 0) return 0;
+    if ((int64_t)batch * m == 0) return 0;
+    if (n == 0) return cpmk_gemm_calc_scale_transpose(batch, n, m, mat, scale, stream);       // (columns of no elements: scale 0, nothing to round)
+    if (any_null(mat, scale, out)) return CPMK_EBADARG;
     hipStream_t st = (hipStream_t)stream;
     // a team here only exchanges one maximum per column and gathers it in a loop over the parts, so
     // it may be larger than the teams of the kernels that keep per-part values in registers

@@ -26,6 +26,14 @@ __host__ __device__ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + 
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// A null buffer with work to do would be a memory fault on the device, which ends the process: the
+// launchers refuse it on the host (CPMK_EBADARG) once they know that the call is not empty.
+template <class... P>
+inline bool any_null(const P*... p) { return (... || (p == nullptr)); }
+
+// Workgroups along a grid's x dimension: the runtime takes at most 2^31 - 1.
+inline bool grid_fits(int64_t blocks) { return blocks <= 0x7fffffffll; }
+
 // ---- wave64 reductions (butterfly over all 6 lane bits) -----------------------------
 __device__ inline float wave_max(float v) {
 #pragma unroll

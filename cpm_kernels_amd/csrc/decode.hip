@@ -66,6 +66,7 @@ int cpmk_embedding_forward(int32_t batch, int32_t hidden_size, int32_t seq_len, 
     clear_stale_error();
     if (batch < 0 || hidden_size < 0 || seq_len < 0) return CPMK_EBADARG;
     if ((int64_t)batch * hidden_size * seq_len == 0) return 0;
+    if (any_null(ids, weights, out)) return CPMK_EBADARG;
     if (ceil_div(hidden_size, 64) > 65535) return CPMK_ETOOBIG;
     const int vec = (hidden_size % 8 == 0) && aligned16(weights);
     for (int64_t b0 = 0; b0 < batch; b0 += 65535) {       // (grid z: at most 65535 batch entries per launch)
@@ -83,6 +84,7 @@ int cpmk_embedding_step(int32_t batch, int32_t embedding_size, const void* ids, 
     clear_stale_error();
     if (batch < 0 || embedding_size < 0) return CPMK_EBADARG;
     if ((int64_t)batch * embedding_size == 0) return 0;
+    if (any_null(ids, weights, out)) return CPMK_EBADARG;
     const int vec = (embedding_size % 8 == 0) && aligned16(weights) && aligned16(out);
     hipLaunchKernelGGL(k_row_copy, dim3((unsigned)batch), dim3(256), 0, (hipStream_t)stream, embedding_size,
                        (const int32_t*)ids, (const half_t*)weights, (half_t*)out, (int64_t)embedding_size, (int64_t)0, vec);
@@ -95,6 +97,7 @@ int cpmk_copy_data_to_kv(int32_t batch, int32_t buffer_len, int32_t n, const voi
     if (batch < 0 || buffer_len < 0 || n < 0 || pos < 0 || pos >= buffer_len) return CPMK_EBADARG;
     if (n % 2) return CPMK_EALIGN;      // kernels/utils.py:25
     if ((int64_t)batch * n == 0) return 0;
+    if (any_null(inp, out)) return CPMK_EBADARG;
     const int vec = (n % 8 == 0) && aligned16(inp) && aligned16(out);
     hipLaunchKernelGGL(k_row_copy, dim3((unsigned)batch), dim3(256), 0, (hipStream_t)stream, n, (const int32_t*)nullptr,
                        (const half_t*)inp, (half_t*)out, (int64_t)buffer_len * n, (int64_t)pos * n, vec);

@@ -109,6 +109,7 @@ int cpmk_gelu_forward(int32_t batch, int32_t n, const void* mat, void* out, void
     if (batch < 0 || n < 0) return CPMK_EBADARG;
     const int64_t total = (int64_t)batch * n;
     if (total == 0) return 0;
+    if (any_null(mat, out)) return CPMK_EBADARG;
     const int vec = aligned16(mat) && aligned16(out);
     const int64_t g = ceil_div(vec ? ceil_div(total, 8) : total, 256);
     hipLaunchKernelGGL(k_gelu, dim3((unsigned)g), dim3(256), 0, (hipStream_t)stream, total, (const half_t*)mat,
@@ -122,6 +123,7 @@ static int ln_affine(int32_t batch, int32_t n, int32_t m, const void* inp, const
     if (m % 2) return CPMK_EALIGN;   // kernels/arith.py:146,200
     const int64_t total = (int64_t)batch * n * m;
     if (total == 0) return 0;
+    if (any_null(inp, alpha, out)) return CPMK_EBADARG;
     const int vec = (m % 8 == 0) && aligned16(inp) && aligned16(out);
     const int64_t g = ceil_div(total / (vec ? 8 : 2), 256);
     if (beta)
@@ -152,6 +154,7 @@ int cpmk_arith_element_add(int32_t batch, int32_t n, const void* x, const void* 
     if (n % 2) return CPMK_EALIGN;   // kernels/arith.py:53
     const int64_t total = (int64_t)batch * n;
     if (total == 0) return 0;
+    if (any_null(x, y, out)) return CPMK_EBADARG;
     const int vec = aligned16(x) && aligned16(y) && aligned16(out);
     const int64_t g = ceil_div(vec ? ceil_div(total, 8) : total, 256);
     hipLaunchKernelGGL(k_add, dim3((unsigned)g), dim3(256), 0, (hipStream_t)stream, total, (const half_t*)x,
@@ -165,6 +168,7 @@ int cpmk_mask(int32_t batch, int32_t n, int32_t m, const void* inp, const void* 
     if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
     const int64_t total = (int64_t)batch * n * m;
     if (total == 0) return 0;
+    if (any_null(inp, mask, out)) return CPMK_EBADARG;
     const int vec = (m % 8 == 0) && aligned16(inp) && aligned16(out) && ((reinterpret_cast<uintptr_t>(mask) & 7u) == 0);
     const int64_t g = ceil_div(vec ? total / 8 : total, 256);
     hipLaunchKernelGGL(k_mask, dim3((unsigned)g), dim3(256), 0, (hipStream_t)stream, total, n, m, (const half_t*)inp,

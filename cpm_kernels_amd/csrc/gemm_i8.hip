@@ -1088,6 +1088,7 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
     if (!(batchA == batchB || batchA == 1 || batchB == 1)) return CPMK_EBADARG;   // :140
     const int batch = batchA > batchB ? batchA : batchB;
     if (m == 0 || n == 0) return 0;
+    if (out == nullptr || (k > 0 && any_null(A, B)) || (FUSED && any_null(srow, scol))) return CPMK_EBADARG;
     if (batch > 65535) {      // some kernels index the batch with the grid's z dimension: at most 65535 entries per call
         constexpr int64_t ESZ_OUT = FUSED ? 2 : 4;
         for (int64_t b0 = 0; b0 < batch; b0 += 65535) {
@@ -1230,6 +1231,7 @@ static int gemm_f16_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, in
     if (!(batchA == batchB || batchA == 1 || batchB == 1)) return CPMK_EBADARG;   // :201
     const int batch = batchA > batchB ? batchA : batchB;
     if (m == 0 || n == 0) return 0;
+    if (out == nullptr || (k > 0 && any_null(A, B))) return CPMK_EBADARG;
     if (k > (1 << 30)) return CPMK_ETOOBIG;
     if (batch > 65535) {      // (grid z: at most 65535 batch entries per call)
         for (int64_t b0 = 0; b0 < batch; b0 += 65535) {

@@ -131,8 +131,10 @@ int cpmk_gemv_fp16(int32_t batch, int32_t dim_out, int32_t dim_in, const void* m
     clear_stale_error();
     if (batch < 0 || dim_out < 0 || dim_in < 0) return CPMK_EBADARG;
     if ((int64_t)batch * dim_out == 0) return 0;
+    if (out == nullptr || (dim_in > 0 && any_null(mat, vec))) return CPMK_EBADARG;
     const int vec8 = (dim_in % 8 == 0) && aligned16(mat) && aligned16(vec);
     const int64_t items = (int64_t)batch * dim_out;
+    if (!grid_fits(ceil_div(items, 4))) return CPMK_ETOOBIG;
     if (vec8 && dim_in <= 256) {
         const int p = dim_in >> 3;                      // 16-byte pieces per row
         const hipStream_t st = (hipStream_t)stream;
@@ -159,6 +161,7 @@ int cpmk_gemv_fp16_transpose(int32_t batch, int32_t dim_out, int32_t dim_in, con
     clear_stale_error();
     if (batch < 0 || dim_out < 0 || dim_in < 0) return CPMK_EBADARG;
     if ((int64_t)batch * dim_out == 0) return 0;
+    if (out == nullptr || (dim_in > 0 && any_null(mat, vec))) return CPMK_EBADARG;
     const int vec8 = (dim_out % 8 == 0) && aligned16(mat);
     for (int64_t b0 = 0; b0 < batch; b0 += 65535) {       // (grid y: at most 65535 batch entries per launch)
         const int64_t nb = batch - b0 < 65535 ? batch - b0 : 65535;
@@ -175,6 +178,7 @@ int cpmk_gemv_broadcast_mat_fp16(int32_t batch, int32_t dim_out, int32_t dim_in,
     clear_stale_error();
     if (batch < 0 || dim_out < 0 || dim_in < 0) return CPMK_EBADARG;
     if ((int64_t)batch * dim_out == 0) return 0;
+    if (out == nullptr || (dim_in > 0 && any_null(mat, vec))) return CPMK_EBADARG;
     {   // matrix cores when the rows are whole 256-byte chunks
         const int rc = gemv_f16_coalesced(batch, dim_out, dim_in, mat, vec, out, (hipStream_t)stream);
         if (rc >= 0) return rc;

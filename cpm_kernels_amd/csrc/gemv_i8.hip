@@ -522,6 +522,7 @@ extern "C" int cpmk_gemv_broadcast_mat_int8(int32_t batch, int32_t dim_out, int3
     if (batch < 0 || dim_out < 0 || dim_in < 0) return CPMK_EBADARG;
     if (dim_in % 4) return CPMK_EALIGN;   // kernels/gemv.py:65
     if (batch == 0 || dim_out == 0) return 0;
+    if (any_null(scale_mat, scale_vec, out) || (dim_in > 0 && any_null(mat, vec))) return CPMK_EBADARG;
     hipStream_t st = (hipStream_t)stream;
     const half_t* sm = (const half_t*)scale_mat;
     const half_t* sv = (const half_t*)scale_vec;

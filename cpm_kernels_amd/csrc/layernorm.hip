@@ -288,6 +288,7 @@ static int layernorm_dispatch(int32_t batch, int32_t n, int32_t m, const void* m
                               int64_t fixed_slots = 0) {
     if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
     if ((int64_t)batch * n * m == 0) return 0;
+    if (any_null(mat, out)) return CPMK_EBADARG;
     const half_t* x = (const half_t*)mat;
     half_t* y = (half_t*)out;
     const half_t* al = (const half_t*)alpha;
@@ -431,6 +432,7 @@ int cpmk_layernorm_step(int32_t batch, int32_t n, const void* mat, void* out, fl
     clear_stale_error();
     if (batch < 0 || n < 0) return CPMK_EBADARG;
     if ((int64_t)batch * n == 0) return 0;
+    if (any_null(mat, out)) return CPMK_EBADARG;
     hipLaunchKernelGGL(k_layernorm_rows, dim3((unsigned)batch), dim3(256), 0, (hipStream_t)stream, n,
                        (const half_t*)mat, (half_t*)out, eps, rd_mean);
     return launch_status();

@@ -83,6 +83,7 @@ int cpmk_position_embedding_init(int32_t num_buckets, int32_t max_distance, void
     clear_stale_error();
     if (num_buckets < (bidirectional ? 4 : 2) || max_distance < 0) return CPMK_EBADARG;
     if (max_distance == 0) return 0;
+    if (out == nullptr) return CPMK_EBADARG;
     hipLaunchKernelGGL(k_position_init, dim3((unsigned)ceil_div(max_distance, 256)), dim3(256), 0,
                        (hipStream_t)stream, num_buckets, max_distance, (int32_t*)out, bidirectional);
     return launch_status();
@@ -94,6 +95,7 @@ int cpmk_position_embedding_forward(int32_t query_len, int32_t key_len, int32_t 
     clear_stale_error();
     if (query_len < 0 || key_len < 0 || num_heads < 0 || num_buckets <= 0 || max_distance <= 0) return CPMK_EBADARG;
     if ((int64_t)query_len * key_len * num_heads == 0) return 0;
+    if (any_null(position_mapping, weight, out)) return CPMK_EBADARG;
     const size_t smem = (size_t)((query_len < QC ? query_len : QC) + KR - 1) * sizeof(half_t);
     // heads are the grid's y dimension (at most 65535): more go out in several launches
     for (int64_t h0 = 0; h0 < num_heads; h0 += 65535) {
@@ -113,6 +115,7 @@ int cpmk_position_embedding_step(int32_t query_pos, int32_t key_len, int32_t num
     clear_stale_error();
     if (key_len < 0 || num_heads < 0 || num_buckets <= 0 || max_distance <= 0) return CPMK_EBADARG;
     if ((int64_t)key_len * num_heads == 0) return 0;
+    if (any_null(position_mapping, weight, out)) return CPMK_EBADARG;
     hipLaunchKernelGGL(k_position_step, dim3((unsigned)ceil_div(key_len, 256)), dim3(256), 0, (hipStream_t)stream,
                        query_pos, key_len, num_buckets, max_distance, num_heads, (const int32_t*)position_mapping,
                        (const half_t*)weight, (half_t*)out, bidirectional);

@@ -331,6 +331,7 @@ static int check3(int32_t batch, int32_t n, int32_t m) {
 
 static int row_absmax(int64_t rows, int32_t m, const void* mat, void* out, hipStream_t st) {
     if (rows == 0) return 0;
+    if (out == nullptr || (m > 0 && mat == nullptr)) return CPMK_EBADARG;       // (rows of no elements have no buffer)
     const bool vec = (m % 8 == 0) && aligned16(mat);
     const half_t* p = (const half_t*)mat;
     half_t* o = (half_t*)out;
@@ -346,6 +347,7 @@ static int row_absmax(int64_t rows, int32_t m, const void* mat, void* out, hipSt
             launch_rows<false>(ra, nv, st);
             return launch_status();
         }
+        if (!grid_fits(ceil_div(rows, 4))) return CPMK_ETOOBIG;
         const unsigned g = (unsigned)ceil_div(rows, 4);
         if (vec) hipLaunchKernelGGL((k_row_absmax<64, true>), dim3(g), dim3(256), 0, st, rows, m, p, o);
         else hipLaunchKernelGGL((k_row_absmax<64, false>), dim3(g), dim3(256), 0, st, rows, m, p, o);
@@ -358,6 +360,7 @@ static int round_launch(int32_t batch, int32_t n, int32_t m, const void* mat, co
                         void* out, hipStream_t st) {
     const int64_t total = (int64_t)batch * n * m;
     if (total == 0) return 0;
+    if (any_null(mat, scale, out)) return CPMK_EBADARG;
     const bool vec = (m % 16 == 0) && aligned16(mat) && aligned16(out) && (MODE == 0 || aligned16(scale));
     const half_t* p = (const half_t*)mat;
     const half_t* s = (const half_t*)scale;
@@ -377,6 +380,7 @@ static int dequant_launch(int32_t batch, int32_t n, int32_t m, const void* mat, 
                           const void* sy, void* out, int bcx, int bcy, hipStream_t st) {
     const int64_t total = (int64_t)batch * n * m;
     if (total == 0) return 0;
+    if (any_null(mat, out) || (MODE != 2 && sx == nullptr) || (MODE != 1 && sy == nullptr)) return CPMK_EBADARG;
     const bool vec = (m % 8 == 0) && aligned16(mat) && aligned16(out) && (MODE == 1 || aligned16(sy));
     if (vec) {
         const int64_t g = ceil_div(total / 8, 256);
@@ -415,6 +419,7 @@ int cpmk_gemm_calc_scale_transpose(int32_t batch, int32_t n, int32_t m, const vo
     clear_stale_error();
     if (int e = check3(batch, n, m)) return e;
     if (batch == 0 || m == 0) return 0;
+    if (any_null(out) || (n > 0 && mat == nullptr)) return CPMK_EBADARG;
     const bool vec = (m % 8 == 0) && aligned16(mat);
     for (int64_t b0 = 0; b0 < batch; b0 += 65535) {       // (grid y: at most 65535 batch entries per launch)
         const int64_t nb = batch - b0 < 65535 ? batch - b0 : 65535;
@@ -477,6 +482,7 @@ int cpmk_gemm_quantize(int32_t batch, int32_t n, int32_t m, const void* mat, voi
     if (!transpose) {
         const int64_t rows = (int64_t)batch * n;
         if (rows == 0) return 0;
+        if (any_null(scale) || (m > 0 && any_null(mat, out))) return CPMK_EBADARG;
         const bool vec = (m % 8 == 0) && aligned16(mat) && ((reinterpret_cast<uintptr_t>(out) & 7u) == 0);
         if (vec && m <= 64 * 8 * 16) {
             const RowsArgs ra = {(const half_t*)mat, (half_t*)scale, (int8_t*)out, rows, nullptr, nullptr, nullptr, 0, m};
@@ -494,6 +500,7 @@ int cpmk_gemm_quantize_pair(int64_t rows0, const void* mat0, void* scale0, void*
     clear_stale_error();
     if (rows0 < 0 || rows1 < 0 || m < 0 || rows0 > 0x7fffffff || rows1 > 0x7fffffff) return CPMK_EBADARG;
     if (m == 0 || rows0 + rows1 == 0) return 0;
+    if ((rows0 > 0 && any_null(mat0, scale0, out0)) || (rows1 > 0 && any_null(mat1, scale1, out1))) return CPMK_EBADARG;
     const bool vec = (m % 8 == 0) && m <= 64 * 8 * 16 && (rows0 == 0 || (aligned16(mat0) && (reinterpret_cast<uintptr_t>(out0) & 7u) == 0)) &&
                      (rows1 == 0 || (aligned16(mat1) && (reinterpret_cast<uintptr_t>(out1) & 7u) == 0));
     if (vec) {

@@ -363,6 +363,7 @@ constexpr int32_t kSoftmaxTeamMin = 2048;
 static int softmax_dispatch(int32_t batch, int32_t n, int32_t m, const void* inp, void* out, hipStream_t st) {
     if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
     if ((int64_t)batch * n * m == 0) return 0;
+    if (any_null(inp, out)) return CPMK_EBADARG;
     const half_t* x = (const half_t*)inp;
     half_t* y = (half_t*)out;
     if (m == 1) {
@@ -434,6 +435,7 @@ int cpmk_softmax_step_inplace(int32_t batch, int32_t n, void* x, void* stream) {
     clear_stale_error();
     if (batch < 0 || n < 0) return CPMK_EBADARG;
     if ((int64_t)batch * n == 0) return 0;
+    if (x == nullptr) return CPMK_EBADARG;
     hipLaunchKernelGGL(k_softmax_rows, dim3((unsigned)batch), dim3(256), 0, (hipStream_t)stream, n,
                        (const half_t*)x, (half_t*)x);
     return launch_status();

@@ -607,6 +607,7 @@ static int launch_ew(int64_t rows, int64_t cols, int64_t n, const void* x, const
     if (rows < 0 || cols < 0) return CPMK_EBADARG;
     if (rows * cols == 0) return 0;
     if (cols % 2) return CPMK_EALIGN;
+    if (any_null(x, a, out) || ((OP == kFma || OP == kSubDiv) && b == nullptr)) return CPMK_EBADARG;
     const bool wide = cols % 8 == 0 && aligned16(x) && aligned16(out) && (BC == 2 || (aligned16(a) && (!b || aligned16(b))));
     const int v = wide ? 8 : 2;
     const int64_t chunks = ceil_div(cols, 256 * v);
@@ -638,9 +639,10 @@ static ColArgs col_args_from(const ColArgs& p, int64_t b0) {
 }
 
 template <int KIND>
-static int launch_col(int32_t batch, const ColArgs& p, void* stream) {
+static int launch_col(int32_t batch, const ColArgs& p, void* stream, bool missing) {
     if (batch < 0 || p.n < 0 || p.m < 0) return CPMK_EBADARG;
     if ((int64_t)batch * p.n * p.m == 0) return 0;
+    if (missing) return CPMK_EBADARG;       // (a null buffer, found by the caller, in a call that has work to do)
     // register-resident team kernel when every access can be 16 bytes wide (8 for the int8 output)
     const int64_t tiles = ceil_div(p.m, 64), parts = ceil_div(p.n, 512);
     const bool wide = p.m % 8 == 0 && aligned16(p.a) && (p.g == nullptr || aligned16(p.g)) && (p.out == nullptr || aligned16(p.out)) &&
@@ -692,6 +694,7 @@ int cpmk_arith_global_scale(int64_t n, const void* inp, float scale, void* out, 
     clear_stale_error();
     if (n < 0) return CPMK_EBADARG;
     if (n == 0) return 0;
+    if (any_null(inp, out)) return CPMK_EBADARG;
     if (n % 8 == 0 && aligned16(inp) && aligned16(out))
         hipLaunchKernelGGL((k_global_scale<8>), dim3((unsigned)ceil_div(n, 256 * 8)), dim3(256), 0, (hipStream_t)stream, n,
                            (const half_t*)inp, scale, (half_t*)out);
@@ -743,6 +746,7 @@ int cpmk_arith_batch_add_backward(int32_t batch, int32_t n, const void* grad_out
     clear_stale_error();
     if (batch < 0 || n < 0) return CPMK_EBADARG;
     if (n == 0) return 0;
+    if (grad == nullptr || (batch > 0 && grad_out == nullptr)) return CPMK_EBADARG;
     hipLaunchKernelGGL(k_batch_add_backward, dim3((unsigned)ceil_div(n, 64)), dim3(256), 0, (hipStream_t)stream, (int64_t)batch,
                        (int64_t)n, (const half_t*)grad_out, (half_t*)grad);
     return launch_status();
@@ -751,6 +755,7 @@ int cpmk_arith_ln_mul_backward(int32_t batch, int32_t n, int32_t m, const void* 
     clear_stale_error();
     if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
     if (n == 0) return 0;
+    if (grad == nullptr || ((int64_t)batch * m > 0 && any_null(inp, grad_out))) return CPMK_EBADARG;
     hipLaunchKernelGGL((k_ln_backward<true>), dim3((unsigned)n), dim3(256), 0, (hipStream_t)stream, (int64_t)batch, (int64_t)n,
                        (int64_t)m, (const half_t*)inp, (const half_t*)grad_out, (half_t*)grad,
                        (int)(m % 8 == 0 && aligned16(inp) && aligned16(grad_out)));
@@ -760,6 +765,7 @@ int cpmk_arith_ln_add_backward(int32_t batch, int32_t n, int32_t m, const void* 
     clear_stale_error();
     if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
     if (n == 0) return 0;
+    if (grad == nullptr || ((int64_t)batch * m > 0 && grad_out == nullptr)) return CPMK_EBADARG;
     hipLaunchKernelGGL((k_ln_backward<false>), dim3((unsigned)n), dim3(256), 0, (hipStream_t)stream, (int64_t)batch, (int64_t)n,
                        (int64_t)m, (const half_t*)nullptr, (const half_t*)grad_out, (half_t*)grad,
                        (int)(m % 8 == 0 && aligned16(grad_out)));
@@ -771,6 +777,7 @@ int cpmk_gelu_backward(int32_t batch, int32_t n, const void* grad_out, const voi
     if (batch < 0 || n < 0) return CPMK_EBADARG;
     const int64_t total = (int64_t)batch * n;
     if (total == 0) return 0;
+    if (any_null(grad_out, mat, grad)) return CPMK_EBADARG;
     if (total % 8 == 0 && aligned16(grad_out) && aligned16(mat) && aligned16(grad))
         hipLaunchKernelGGL((k_gelu_backward<8>), dim3((unsigned)ceil_div(total / 8, 256)), dim3(256), 0, (hipStream_t)stream, total,
                            (const half_t*)grad_out, (const half_t*)mat, (half_t*)grad);
@@ -783,41 +790,41 @@ int cpmk_gelu_backward(int32_t batch, int32_t n, const void* grad_out, const voi
 int cpmk_layernorm_forward_v(int32_t batch, int32_t n, int32_t m, const void* mat, void* out, void* out_var, float eps, void* stream) {
     clear_stale_error();
     ColArgs p = {n, m, (const half_t*)mat, nullptr, nullptr, nullptr, nullptr, (half_t*)out, nullptr, nullptr, (half_t*)out_var, eps, 0};
-    return launch_col<kLnFwdV>(batch, p, stream);
+    return launch_col<kLnFwdV>(batch, p, stream, any_null(mat, out, out_var));
 }
 int cpmk_layernorm_forward_mv(int32_t batch, int32_t n, int32_t m, const void* mat, void* out, void* out_mean, void* out_var,
                               float eps, void* stream) {
     clear_stale_error();
     ColArgs p = {n, m, (const half_t*)mat, nullptr, nullptr, nullptr, nullptr, (half_t*)out, nullptr, (half_t*)out_mean,
                  (half_t*)out_var, eps, 0};
-    return launch_col<kLnFwdMV>(batch, p, stream);
+    return launch_col<kLnFwdMV>(batch, p, stream, any_null(mat, out, out_mean, out_var));
 }
 int cpmk_layernorm_backward_v(int32_t batch, int32_t n, int32_t m, const void* mat, const void* grad_out, const void* var, void* grad,
                               void* stream) {
     clear_stale_error();
     ColArgs p = {n, m, (const half_t*)mat, (const half_t*)grad_out, nullptr, (const half_t*)var, nullptr, (half_t*)grad, nullptr,
                  nullptr, nullptr, 0.0f, 0};
-    return launch_col<kLnBwdV>(batch, p, stream);
+    return launch_col<kLnBwdV>(batch, p, stream, any_null(mat, grad_out, var, grad));
 }
 int cpmk_layernorm_backward_mv(int32_t batch, int32_t n, int32_t m, const void* mat, const void* grad_out, const void* mean,
                                const void* var, void* grad, void* stream) {
     clear_stale_error();
     ColArgs p = {n, m, (const half_t*)mat, (const half_t*)grad_out, (const half_t*)mean, (const half_t*)var, nullptr, (half_t*)grad,
                  nullptr, nullptr, nullptr, 0.0f, 0};
-    return launch_col<kLnBwdMV>(batch, p, stream);
+    return launch_col<kLnBwdMV>(batch, p, stream, any_null(mat, grad_out, mean, var, grad));
 }
 int cpmk_softmax_backward(int32_t batch, int32_t n, int32_t m, const void* out, const void* grad_out, void* grad, void* stream) {
     clear_stale_error();
     ColArgs p = {n, m, (const half_t*)out, (const half_t*)grad_out, nullptr, nullptr, nullptr, (half_t*)grad, nullptr, nullptr, nullptr,
                  0.0f, 0};
-    return launch_col<kSoftmaxBwd>(batch, p, stream);
+    return launch_col<kSoftmaxBwd>(batch, p, stream, any_null(out, grad_out, grad));
 }
 int cpmk_gemm_backward_scale_round(int32_t batch, int32_t n, int32_t m, const void* mat, const void* scale_x, void* out, void* scale_y,
                                    int broad_cast_x, void* stream) {
     clear_stale_error();
     ColArgs p = {n, m, (const half_t*)mat, nullptr, nullptr, nullptr, (const half_t*)scale_x, nullptr, (int8_t*)out, nullptr,
                  (half_t*)scale_y, 0.0f, broad_cast_x};
-    return launch_col<kScaleRound>(batch, p, stream);
+    return launch_col<kScaleRound>(batch, p, stream, any_null(mat, scale_x, out, scale_y));
 }
 int cpmk_gemm_backward_round_scale(int32_t batch, int32_t n, int32_t m, const void* mat, const void* scale_y, void* out, void* scale_x,
                                    int broad_cast_y, void* stream) {
@@ -826,6 +833,7 @@ int cpmk_gemm_backward_round_scale(int32_t batch, int32_t n, int32_t m, const vo
     const int64_t rows = (int64_t)batch * n;
     if (rows == 0) return 0;
     if (rows > 0x7fffffff) return CPMK_ETOOBIG;
+    if (scale_x == nullptr || (m > 0 && any_null(mat, scale_y, out))) return CPMK_EBADARG;
     if (m % 8 == 0 && aligned16(mat) && aligned16(scale_y) && (reinterpret_cast<uintptr_t>(out) & 7u) == 0) {
         hipLaunchKernelGGL(k_round_scale_rows_wide, dim3((unsigned)ceil_div(rows, 4)), dim3(256), 0, (hipStream_t)stream, rows, n, m,
                            (const half_t*)mat, (const half_t*)scale_y, (int8_t*)out, (half_t*)scale_x, broad_cast_y);
@@ -842,6 +850,7 @@ int cpmk_position_embedding_backward(int32_t query_len, int32_t key_len, int32_t
     if (query_len < 0 || key_len < 0 || num_buckets <= 0 || max_distance <= 0 || num_heads < 0) return CPMK_EBADARG;
     if (num_heads == 0) return 0;
     if (num_buckets > 8192) return CPMK_ETOOBIG;
+    if (grad == nullptr || ((int64_t)query_len * key_len > 0 && any_null(position_mapping, grad_out))) return CPMK_EBADARG;
     if (num_buckets <= kXchVals && max_distance <= 8192 && key_len > 64) {
         // key rows of a head over a team: 64 rows a part, more when that would make more than 32 parts
         int64_t rpp = 64;
@@ -874,6 +883,7 @@ int cpmk_embedding_backward_stage1(int32_t batch, int32_t seq_len, int32_t hidde
     if (batch < 0 || seq_len < 0 || hidden_size < 0) return CPMK_EBADARG;
     if ((int64_t)batch * seq_len * hidden_size == 0) return 0;
     if (ceil_div(hidden_size, 256) > 65535) return CPMK_ETOOBIG;
+    if (any_null(grad_out, argsort_ids, sorted_ids, grad, aux_grad, aux_grad_idx)) return CPMK_EBADARG;
     hipLaunchKernelGGL(k_embedding_backward1, dim3((unsigned)batch, (unsigned)ceil_div(hidden_size, 256)), dim3(256), 0,
                        (hipStream_t)stream, seq_len, hidden_size, (const half_t*)grad_out, (const int32_t*)argsort_ids,
                        (const int32_t*)sorted_ids, (half_t*)grad, (half_t*)aux_grad, (int32_t*)aux_grad_idx);
@@ -884,6 +894,7 @@ int cpmk_embedding_backward_stage2(int32_t batch, int32_t hidden_size, const voi
     clear_stale_error();
     if (batch < 0 || hidden_size < 0) return CPMK_EBADARG;
     if ((int64_t)batch * hidden_size == 0) return 0;
+    if (any_null(aux_grad, aux_grad_idx, grad)) return CPMK_EBADARG;
     hipLaunchKernelGGL(k_embedding_backward2, dim3((unsigned)ceil_div(hidden_size, 256)), dim3(256), 0, (hipStream_t)stream, batch,
                        hidden_size, (const half_t*)aux_grad, (const int32_t*)aux_grad_idx, (half_t*)grad);
     return launch_status();

@@ -139,6 +139,7 @@ int cpmk_transpose(int32_t batch, int32_t n, int32_t m, const void* inp, void* o
     clear_stale_error();
     if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
     if ((int64_t)batch * n * m == 0) return 0;
+    if (any_null(inp, out)) return CPMK_EBADARG;
     if (ceil_div(n, 64) > 65535) return CPMK_ETOOBIG;
     const bool wide = n % 8 == 0 && m % 8 == 0 && aligned16(inp) && aligned16(out);
     // the batch is the grid's z dimension (at most 65535): larger batches go out in several launches
@@ -158,6 +159,7 @@ int cpmk_transpose_i8(int32_t batch, int32_t n, int32_t m, const void* inp, void
     clear_stale_error();
     if (batch < 0 || n < 0 || m < 0) return CPMK_EBADARG;
     if ((int64_t)batch * n * m == 0) return 0;
+    if (any_null(inp, out)) return CPMK_EBADARG;
     if (ceil_div(n, 64) > 65535) return CPMK_ETOOBIG;
     const bool wide = n % 16 == 0 && m % 16 == 0 && aligned16(inp) && aligned16(out);
     for (int64_t b0 = 0; b0 < batch; b0 += 65535) {       // (grid z: at most 65535 batch entries per launch)
@@ -185,6 +187,7 @@ int cpmk_adjustify_logits(int32_t batch, int32_t n, void* logits, float temperat
     if (batch < 0 || n < 0) return CPMK_EBADARG;
     const int64_t total = (int64_t)batch * n;
     if (total == 0) return 0;
+    if (any_null(logits, frequency)) return CPMK_EBADARG;
     hipLaunchKernelGGL(k_adjustify_logits, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, (hipStream_t)stream, total,
                        (half_t*)logits, temperature, frequency_penalty, presence_penalty, (const int32_t*)frequency);
     return launch_status();
@@ -194,6 +197,7 @@ int cpmk_copy_extend_buffer(int32_t batch, int32_t old_size, int32_t nw_size, co
     clear_stale_error();
     if (batch < 0 || old_size < 0 || nw_size < old_size) return CPMK_EBADARG;
     if ((int64_t)batch * old_size == 0) return 0;
+    if (any_null(old_buffer, new_buffer)) return CPMK_EBADARG;
     const bool wide = old_size % 8 == 0 && nw_size % 8 == 0 && aligned16(old_buffer) && aligned16(new_buffer);
     for (int64_t b0 = 0; b0 < batch; b0 += 65535) {       // (grid y: at most 65535 batch entries per launch)
         const int64_t nb = batch - b0 < 65535 ? batch - b0 : 65535;
@@ -214,6 +218,7 @@ int cpmk_has_nan_inf(int64_t n, const void* inp, void* out, void* stream) {
     clear_stale_error();
     if (n < 0) return CPMK_EBADARG;
     if (n == 0) return 0;
+    if (any_null(inp, out)) return CPMK_EBADARG;
     const int64_t blocks = ceil_div(n, 256 * 16);
     hipLaunchKernelGGL(k_has_nan_inf, dim3((unsigned)(blocks > 2048 ? 2048 : blocks)), dim3(256), 0, (hipStream_t)stream, n,
                        (const uint16_t*)inp, (int8_t*)out);
@@ -224,6 +229,7 @@ int cpmk_copy_pos_hidden(int32_t batch, int32_t hidden_size, int32_t seq_len, in
     clear_stale_error();
     if (batch < 0 || hidden_size < 0 || seq_len < 0 || pos < 0 || (seq_len > 0 && pos >= seq_len)) return CPMK_EBADARG;
     if ((int64_t)batch * hidden_size * seq_len == 0) return 0;
+    if (any_null(inp, out)) return CPMK_EBADARG;
     for (int64_t b0 = 0; b0 < batch; b0 += 65535) {       // (grid y: at most 65535 batch entries per launch)
         const int64_t nb = batch - b0 < 65535 ? batch - b0 : 65535;
         hipLaunchKernelGGL(k_copy_pos_hidden, dim3((unsigned)ceil_div(hidden_size, 256), (unsigned)nb), dim3(256), 0,

@@ -119,6 +119,67 @@ def test_argument_errors_from_the_c_abi_without_a_gpu():
     cpmk.position_embedding_forward(0, 4, 32, 128, 2, None, None, None, 1, None)
 
 
+def test_null_buffers_are_refused_before_any_launch():
+    """A null buffer in a call that has work to do would be a memory fault on the device; every launcher
+    answers it with CPMK_EBADARG on the host instead (so this runs on a GPU-less host too)."""
+    from cpm_kernels_amd.library import cpmk
+    N = None
+    calls = [
+        lambda: cpmk.gemm_calc_scale(1, 4, 8, N, N, N),
+        lambda: cpmk.gemm_calc_scale_transpose(1, 4, 8, N, N, N),
+        lambda: cpmk.gemm_round(1, 4, 16, N, N, N, N),
+        lambda: cpmk.gemm_round_transpose(1, 4, 16, N, N, N, N),
+        lambda: cpmk.gemm_scale(1, 4, 8, N, N, N, N, 0, 0, N),
+        lambda: cpmk.gemm_scale_x(1, 4, 8, N, N, N, N),
+        lambda: cpmk.gemm_scale_y(1, 4, 8, N, N, N, N),
+        lambda: cpmk.gemm_int8(4, 4, 4, 1, 1, 0, 0, N, N, N, N),
+        lambda: cpmk.gemm_int8_scale(4, 4, 4, 1, 1, 0, 0, N, N, N, N, 0, 0, N, N),
+        lambda: cpmk.gemm_fp16(4, 4, 4, 1, 1, 0, 0, N, N, N, N),
+        lambda: cpmk.gemm_quantize(1, 4, 8, N, N, N, 0, N),
+        lambda: cpmk.gemm_quantize(1, 4, 8, N, N, N, 1, N),
+        lambda: cpmk.gemm_quantize_pair(4, N, N, N, 4, N, N, N, 8, N),
+        lambda: cpmk.gemm_quantize_cols(1, 4, 8, N, N, N, 0, N),
+        lambda: cpmk.gemv_calc_scale(2, 8, N, N, N),
+        lambda: cpmk.gemv_round(2, 8, N, N, N, N),
+        lambda: cpmk.gemv_broadcast_mat_int8(1, 4, 8, N, N, N, N, N, N),
+        lambda: cpmk.gemv_fp16(1, 4, 8, N, N, N, N),
+        lambda: cpmk.gemv_fp16_transpose(1, 4, 8, N, N, N, N),
+        lambda: cpmk.gemv_broadcast_mat_fp16(1, 4, 8, N, N, N, N),
+        lambda: cpmk.layernorm_forward(1, 4, 8, N, N, 1e-5, 1, N),
+        lambda: cpmk.layernorm_step(1, 8, N, N, 1e-5, 1, N),
+        lambda: cpmk.softmax_forward(1, 4, 8, N, N, N),
+        lambda: cpmk.softmax_step_inplace(1, 8, N, N),
+        lambda: cpmk.gelu_forward(1, 8, N, N, N),
+        lambda: cpmk.arith_ln_mul(1, 4, 8, N, N, N, N),
+        lambda: cpmk.arith_element_add(1, 8, N, N, N, N),
+        lambda: cpmk.mask(1, 4, 8, N, N, 0.0, N, N),
+        lambda: cpmk.position_embedding_init(32, 128, N, 1, N),
+        lambda: cpmk.position_embedding_forward(4, 4, 32, 128, 2, N, N, N, 1, N),
+        lambda: cpmk.position_embedding_step(1, 4, 32, 128, 2, N, N, N, 1, N),
+        lambda: cpmk.embedding_forward(1, 8, 4, N, N, N, N),
+        lambda: cpmk.embedding_step(1, 8, N, N, N, N),
+        lambda: cpmk.copy_data_to_kv(1, 4, 8, N, N, 0, N),
+        lambda: cpmk.transpose(1, 4, 8, N, N, N),
+        lambda: cpmk.has_nan_inf(8, N, N, N),
+        lambda: cpmk.arith_global_scale(8, N, 1.0, N, N),
+        lambda: cpmk.arith_element_mul(1, 8, N, N, N, N),
+        lambda: cpmk.arith_batch_add_backward(2, 8, N, N, N),
+        lambda: cpmk.arith_ln_mul_backward(1, 4, 8, N, N, N, N),
+        lambda: cpmk.gelu_backward(1, 8, N, N, N, N),
+        lambda: cpmk.softmax_backward(1, 4, 8, N, N, N, N),
+        lambda: cpmk.layernorm_forward_mv(1, 4, 8, N, N, N, N, 1e-5, N),
+        lambda: cpmk.layernorm_backward_v(1, 4, 8, N, N, N, N, N),
+        lambda: cpmk.gemm_backward_round_scale(1, 4, 8, N, N, N, N, 0, N),
+        lambda: cpmk.gemm_backward_scale_round(1, 4, 8, N, N, N, N, 0, N),
+        lambda: cpmk.position_embedding_backward(4, 4, 32, 128, 2, N, N, N, 1, N),
+        lambda: cpmk.embedding_backward_stage2(2, 8, N, N, N, N),
+    ]
+    for i, call in enumerate(calls):
+        with pytest.raises(RuntimeError, match="invalid argument"):
+            call()
+            pytest.fail(f"call {i} accepted a null buffer")
+
+
 def test_missing_library_gives_stubs_not_import_errors():
     """cpm_kernels/library/base.py:67-74 of the reference: an absent library leaves the package
     importable and every bound call raises RuntimeError('Library ... is not initialized')."""
