@@ -656,6 +656,15 @@ def main():
         ceil["write_1GiB"] = gbs(nb, event_ms(lambda: ok(cl.ceil_write(big2.data_ptr(), nb, st())), 10))
         ceil["copy_1GiB"] = gbs(2 * nb, event_ms(lambda: ok(cl.ceil_copy(big.data_ptr(), big2.data_ptr(), nb, 0, st())), 10))
         ceil["copy_1GiB_nontemporal"] = gbs(2 * nb, event_ms(lambda: ok(cl.ceil_copy(big.data_ptr(), big2.data_ptr(), nb, 1, st())), 10))
+        # calibration only, not this build's code: the runtime's own device-to-device copy (torch's copy_ of a contiguous
+        # tensor is hipMemcpyAsync), 1 GiB and the layernorm's 33.5 MB from ten buffers in turn
+        ceil["runtime_memcpy_d2d_1GiB"] = gbs(2 * nb, event_ms(lambda: big2.copy_(big), 10))
+        ln_bytes = 8 * 4096 * 1024
+        srcs = [big[i * (64 << 20): i * (64 << 20) + ln_bytes] for i in range(10)]
+        dst_ln = big2[:ln_bytes]
+        ms, how = graph_ms([(lambda i=i: dst_ln.copy_(srcs[i])) for i in range(10)], 60)
+        ceil["runtime_memcpy_d2d_33.5MB"] = dict(gbs(2 * ln_bytes, ms), timing=how)
+        del srcs, dst_ln
         # what one kernel launch costs between two others: a kernel that does nothing, in a graph like the per-kernel legs'
         ms, how = graph_ms([lambda: ok(cl.ceil_empty(256, 512, sink.data_ptr(), st()))], 640)
         ceil["empty_kernel (what a launch costs in the per-kernel legs)"] = {"us": round(ms * 1e3, 2), "timing": how}
