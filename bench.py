@@ -715,8 +715,28 @@ def main():
             ms = event_ms(lambda: torch._int_mm(qa1, qw1.t()), 50, warmup=5)
             ceil["vendor_int_mm_config_1_int32_out"] = {"us": round(ms * 1e3, 2), "tops": round(2.0 * 512 * 4096 * 4096 / (ms * 1e-3) / 1e12, 1)}
             del qa, qw, o32
+            # the GEMV's shape through the vendor's GEMM: 32 vectors x [10240, 4096], eight weight copies in turn (cold), eager launches
+            ws = [torch.randint(-127, 128, (10240, 4096), generator=gg, dtype=torch.int8).to(dev) for _ in range(8)]
+            v32 = torch.randint(-127, 128, (32, 4096), generator=gg, dtype=torch.int8).to(dev)
+            turn = [0]
+
+            def vendor_gemv():
+                turn[0] = (turn[0] + 1) % 8
+                torch._int_mm(v32, ws[turn[0]].t())
+            ms = event_ms(vendor_gemv, 400, warmup=16)
+            ceil["vendor_int_mm_gemv_shape_int32_out"] = dict(gbs(10240 * 4096 + 32 * 4096 + 4 * 32 * 10240, ms), timing="events, eager launches")
+            del ws, v32
         except Exception as ex:     # pragma: no cover  (calibration only)
             ceil["vendor_int_mm"] = "unavailable: %s" % ex
+        # torch's own softmax over dim 1 on config 3's tensor (the same operation, without the -1e6 floor and the 1e-10)
+        try:
+            xs = torch.randn((512, 1024, 1024), generator=gg, dtype=torch.float16).to(dev)
+            ys = torch.empty_like(xs)
+            ms = event_ms(lambda: torch.softmax(xs, dim=1, out=ys), 10, warmup=3)
+            ceil["torch_softmax_dim1_config_3"] = gbs(2 * xs.numel() * 2, ms)
+            del xs, ys
+        except Exception as ex:     # pragma: no cover  (calibration only)
+            ceil["torch_softmax_dim1_config_3"] = "unavailable: %s" % ex
         result["ceilings"] = ceil
 
     # ---- the north-star step and its GEMM kernel on the busy device (see the note at leg_pipeline's first call) ----
