@@ -212,6 +212,8 @@ int XchScope::end() {
                     d->held.push_back(Held{xl.first, last_, ev});
                 }
             }
+            // no event to wait for later: the slots must be idle before anyone else can be given them
+            if (rc != 0) (void)hipStreamSynchronize(st_);
         }
     }
     g_mu.unlock();
