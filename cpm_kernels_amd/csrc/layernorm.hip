@@ -25,7 +25,7 @@ __device__ inline half8_t affine8(half8_t y, half_t a, half_t b, bool has_beta) 
 // Single pass: the whole (n x LPR*8) column tile lives in registers.  Tiles of whole cache lines (LPR == 8) are
 // read and written with the non-temporal hint: every byte is touched once (8 x 4096 x 512 through the team
 // kernel: 17.2 -> 15.2 us).
-template <int NT, int LPR, int R>
+template <int NT, int LPR, int R, bool AFF>
 __global__ __launch_bounds__(NT) void k_layernorm_tile(int32_t n, int32_t m, int32_t tiles_per_batch,
                                                        const half_t* mat, half_t* out,
                                                        const half_t* __restrict__ alpha,
@@ -39,15 +39,29 @@ __global__ __launch_bounds__(NT) void k_layernorm_tile(int32_t n, int32_t m, int
     const int32_t col0 = ct * T::COLS + (threadIdx.x % LPR) * 8;
     const int64_t boff = (int64_t)b * n * m;
 
+    // the affine coefficients of the tile's rows, contiguous loads requested ahead of the tile (loads
+    // return in order: behind the tile they would hold the sums below back until its last piece had
+    // arrived) and parked in LDS until the output pass (the barriers of the reduction order write and reads)
+    constexpr int CPT = (T::ROWS + NT - 1) / NT;       // coefficient pairs per thread
+    half_t ca[CPT], cb[CPT];
+    if constexpr (AFF) {
+#pragma unroll
+        for (int i = 0; i < CPT; ++i) {
+            const int32_t row = min((int32_t)(threadIdx.x + i * NT), n - 1);
+            ca[i] = alpha[row];
+            cb[i] = beta != nullptr ? beta[row] : (half_t)0.0f;
+        }
+    }
     half8_t v[R];
     coltile_load<NT, LPR, R, LPR == 8>(v, mat + boff, n, m, col0, (half_t)0.0f);
-    // the affine coefficients of the tile's rows, contiguous loads requested with the tile and
-    // parked in LDS until the output pass (the barriers of the reduction order write and reads)
-    if (alpha != nullptr) {
-        for (int32_t r = threadIdx.x; r < T::ROWS; r += NT) {
-            const int32_t row = min(r, n - 1);
-            coef[0][r] = alpha[row];
-            coef[1][r] = beta != nullptr ? beta[row] : (half_t)0.0f;
+    if constexpr (AFF) {
+#pragma unroll
+        for (int i = 0; i < CPT; ++i) {
+            const int r = threadIdx.x + i * NT;
+            if (r < T::ROWS) {
+                coef[0][r] = ca[i];
+                coef[1][r] = cb[i];
+            }
         }
     }
 
@@ -82,7 +96,7 @@ __global__ __launch_bounds__(NT) void k_layernorm_tile(int32_t n, int32_t m, int
         half8_t y;
 #pragma unroll
         for (int e = 0; e < 8; ++e) y[e] = round_f16(((float)v[p][e] - mean[e]) * rstd[e]);
-        if (alpha != nullptr) y = affine8(y, coef[0][p * T::RPP + rg], coef[1][p * T::RPP + rg], beta != nullptr);
+        if constexpr (AFF) y = affine8(y, coef[0][p * T::RPP + rg], coef[1][p * T::RPP + rg], beta != nullptr);
         v[p] = y;
     }
     coltile_store<NT, LPR, R, LPR == 8>(v, out + boff, n, m, col0);
@@ -94,7 +108,7 @@ __global__ __launch_bounds__(NT) void k_layernorm_tile(int32_t n, int32_t m, int
 // each keeps its own rows in registers, posts its partial column sums, adds up the team's
 // partials in part order (so the result does not depend on timing) and normalises its rows.
 // A workgroup reads and writes only its own rows: out may alias mat.
-template <int NT, int R>
+template <int NT, int R, bool AFF>
 __global__ __launch_bounds__(NT) void k_layernorm_team(int32_t n, int32_t m, int32_t tiles_per_batch, int32_t parts,
                                                        const half_t* mat, half_t* out,
                                                        const half_t* __restrict__ alpha,
@@ -122,16 +136,23 @@ __global__ __launch_bounds__(NT) void k_layernorm_team(int32_t n, int32_t m, int
     const int32_t own_n = min(T::ROWS, n - own0);        // > 0 by construction
     const int64_t boff = (int64_t)b * n * m + (int64_t)own0 * m;
 
-    half8_t v[R];
-    coltile_load<NT, LPR, R, true>(v, mat + boff, own_n, m, col0, (half_t)0.0f);
     // The affine coefficients of the workgroup's rows: one pair per thread, contiguous, parked in
     // LDS until the output pass (a thread's own rows are RPP apart; fetching them lane by lane
     // took 2 x R two-byte loads per thread, as many load instructions again as the tile itself).
+    // Requested ahead of the tile: loads return in order, so behind the tile they would hold the
+    // sums below back until the last piece of the tile had arrived.
     const int rg = tid / LPR;
-    if (alpha != nullptr) {
+    half_t ca = (half_t)0.0f, cb = (half_t)0.0f;
+    if constexpr (AFF) {
         const int32_t row = min(own0 + tid, n - 1);
-        coef[0][tid] = alpha[row];
-        coef[1][tid] = beta != nullptr ? beta[row] : (half_t)0.0f;
+        ca = alpha[row];
+        if (beta != nullptr) cb = beta[row];
+    }
+    half8_t v[R];
+    coltile_load<NT, LPR, R, true>(v, mat + boff, own_n, m, col0, (half_t)0.0f);
+    if constexpr (AFF) {
+        coef[0][tid] = ca;
+        coef[1][tid] = cb;
     }
     float s[16];
 #pragma unroll
@@ -188,7 +209,7 @@ __global__ __launch_bounds__(NT) void k_layernorm_team(int32_t n, int32_t m, int
         half8_t y;
 #pragma unroll
         for (int e = 0; e < 8; ++e) y[e] = round_f16(((float)v[p][e] - mean[e]) * rstd[e]);
-        if (alpha != nullptr) y = affine8(y, coef[0][p * T::RPP + rg], coef[1][p * T::RPP + rg], beta != nullptr);
+        if constexpr (AFF) y = affine8(y, coef[0][p * T::RPP + rg], coef[1][p * T::RPP + rg], beta != nullptr);
         v[p] = y;
     }
     coltile_store<NT, LPR, R, true>(v, out + boff, own_n, m, col0);
@@ -265,8 +286,12 @@ static void launch_tile(int32_t batch, int32_t n, int32_t m, const half_t* mat, 
                         const half_t* beta, float eps, int rd_mean, hipStream_t st) {
     constexpr int NT = 1024;
     const int32_t tiles = (int32_t)ceil_div(m, LPR * 8);
-    hipLaunchKernelGGL((k_layernorm_tile<NT, LPR, R>), dim3((unsigned)((int64_t)tiles * batch)), dim3(NT), 0, st, n,
-                       m, tiles, mat, out, alpha, beta, eps, rd_mean);
+    if (alpha != nullptr)
+        hipLaunchKernelGGL((k_layernorm_tile<NT, LPR, R, true>), dim3((unsigned)((int64_t)tiles * batch)), dim3(NT), 0, st, n,
+                           m, tiles, mat, out, alpha, beta, eps, rd_mean);
+    else
+        hipLaunchKernelGGL((k_layernorm_tile<NT, LPR, R, false>), dim3((unsigned)((int64_t)tiles * batch)), dim3(NT), 0, st, n,
+                           m, tiles, mat, out, alpha, beta, eps, rd_mean);
 }
 
 template <int LPR>
@@ -337,12 +362,17 @@ static int layernorm_dispatch(int32_t batch, int32_t n, int32_t m, const void* m
                     // share the chip; kept to teams of at most four so that this stays a small part of the chip.
                     const int64_t G = tiles * nb * parts;
                     const int xcd_local = parts <= 4 && G % 8 == 0 && (G / 8) % parts == 0 && G <= compute_units() * (big ? 1 : 2);
-                    if (big)
-                        hipLaunchKernelGGL((k_layernorm_team<1024, 8>), grid, dim3(1024), 0, st, n, m, (int32_t)tiles,
-                                           (int32_t)parts, xb, yb, al, be, eps, rd_mean, xcd_local, xl);
-                    else
-                        hipLaunchKernelGGL((k_layernorm_team<512, 8>), grid, dim3(512), 0, st, n, m, (int32_t)tiles,
-                                           (int32_t)parts, xb, yb, al, be, eps, rd_mean, xcd_local, xl);
+                    auto go = [&](auto kern, int threads) {
+                        hipLaunchKernelGGL(kern, grid, dim3(threads), 0, st, n, m, (int32_t)tiles, (int32_t)parts, xb, yb, al, be, eps,
+                                           rd_mean, xcd_local, xl);
+                    };
+                    if (big) {
+                        if (al != nullptr) go(k_layernorm_team<1024, 8, true>, 1024);
+                        else go(k_layernorm_team<1024, 8, false>, 1024);
+                    } else {
+                        if (al != nullptr) go(k_layernorm_team<512, 8, true>, 512);
+                        else go(k_layernorm_team<512, 8, false>, 512);
+                    }
                     const int e = launch_status();
                     const int rc2 = xs.end();
                     if (e != 0 || rc2 != 0) return e ? e : rc2;

@@ -284,30 +284,32 @@ __global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_b
     const int64_t boff = (int64_t)b * p.n * p.m + (int64_t)own0 * p.m;
     const bool live = col0 < p.m;
 
+    // The per-column and per-row operands of the sums are requested ahead of the tiles: loads return in
+    // order, and behind the tiles they would hold the sums back until the last piece had arrived.
+    half8_t hv = {0, 0, 0, 0, 0, 0, 0, 0}, hm = {0, 0, 0, 0, 0, 0, 0, 0};
+    half_t sxh[R];
+    if (live && (KIND == kLnBwdV || KIND == kLnBwdMV)) hv = *reinterpret_cast<const half8_t*>(p.var + (int64_t)b * p.m + col0);
+    if (live && KIND == kLnBwdMV) hm = *reinterpret_cast<const half8_t*>(p.mean + (int64_t)b * p.m + col0);
+#pragma unroll
+    for (int q = 0; q < R; ++q) {
+        sxh[q] = (half_t)0.0f;
+        if (KIND == kScaleRound) {
+            const int32_t row = own0 + q * T::RPP + rg;
+            if (row < p.n) sxh[q] = p.sx[(p.bc ? 0 : (int64_t)b * p.n) + row];
+        }
+    }
     half8_t va[R], vg[TWO ? R : 1];
     coltile_load<NT, LPR, R>(va, p.a + boff, own_n, p.m, col0, (half_t)0.0f);
     if constexpr (TWO) coltile_load<NT, LPR, R>(vg, p.g + boff, own_n, p.m, col0, (half_t)0.0f);
     float mean[8], var[8], c3[8], sxv[R];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) mean[e] = var[e] = c3[e] = 0.0f;
-    if (live && (KIND == kLnBwdV || KIND == kLnBwdMV)) {
-        const half8_t hv = *reinterpret_cast<const half8_t*>(p.var + (int64_t)b * p.m + col0);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) { var[e] = (float)hv[e]; c3[e] = -0.5f * var[e] * var[e] * var[e]; }
-    }
-    if (live && KIND == kLnBwdMV) {
-        const half8_t hm = *reinterpret_cast<const half8_t*>(p.mean + (int64_t)b * p.m + col0);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) mean[e] = (float)hm[e];
+    for (int e = 0; e < 8; ++e) {
+        var[e] = (float)hv[e];
+        c3[e] = -0.5f * var[e] * var[e] * var[e];
+        mean[e] = (float)hm[e];
     }
 #pragma unroll
-    for (int q = 0; q < R; ++q) {
-        sxv[q] = 0.0f;
-        if (KIND == kScaleRound) {
-            const int32_t row = own0 + q * T::RPP + rg;
-            if (row < p.n) sxv[q] = (float)p.sx[(p.bc ? 0 : (int64_t)b * p.n) + row];
-        }
-    }
+    for (int q = 0; q < R; ++q) sxv[q] = (float)sxh[q];
 
     float s[NV * 8];
 #pragma unroll
