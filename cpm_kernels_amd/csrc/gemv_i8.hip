@@ -308,16 +308,7 @@ __global__ __launch_bounds__(512) void k_gemv_direct(int32_t batch, int32_t dim_
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, q = lane >> 4;
     const int32_t row0 = blockIdx.x * rpb;
-    // the scales of the outputs this thread will write, requested first
-    constexpr int NOUT = (RG * NB * 256 + 511) / 512;
-    half_t osv[NOUT], osm[NOUT];
-#pragma unroll
-    for (int o = 0; o < NOUT; ++o) {
-        const int idx = tid + o * 512;
-        const int rr = idx % rpb, bb = idx / rpb;
-        osv[o] = scale_vec[min(bb, batch - 1)];
-        osm[o] = scale_mat[min(row0 + rr, dim_out - 1)];
-    }
+    constexpr int NOUT = (RG * NB * 256 + 511) / 512;     // outputs per thread
     // The first 16 rows of the matrix, then the vectors, then the other rows: the requests to memory are
     // under way while the address unit works off the 128 KB of vectors, which come from L2.
     int4_t wf[RG][KB];
@@ -346,9 +337,24 @@ __global__ __launch_bounds__(512) void k_gemv_direct(int32_t batch, int32_t dim_
     if constexpr (RG > 1) load_rows(std::integral_constant<int, 1>{});
     if constexpr (RG > 2) load_rows(std::integral_constant<int, 2>{});
     __builtin_amdgcn_sched_barrier(0);
+    // The outputs this thread will write (vector bb, row rr of the workgroup's share; the row runs fastest, so a
+    // vector's outputs are stored contiguously) and their scales.  Worked out and requested here, behind the
+    // last matrix load: the two divisions per output then run while the memory works, and the scales, needed
+    // last, are also the last loads to return.
+    int orr[NOUT], obb[NOUT];
+    half_t osv[NOUT], osm[NOUT];
+#pragma unroll
+    for (int o = 0; o < NOUT; ++o) {
+        const int idx = tid + o * 512;
+        obb[o] = idx / rpb;
+        orr[o] = idx - obb[o] * rpb;
+        osv[o] = scale_vec[min(obb[o], batch - 1)];
+        osm[o] = scale_mat[min(row0 + orr[o], dim_out - 1)];
+    }
+    __builtin_amdgcn_sched_barrier(0);
     for (int idx = tid; idx < RG * NB * 256; idx += 512) part[idx] = 0;
-    // the vectors (and the rows requested before them) have landed when only the later matrix loads are still under way
-    wait_vmcnt<(RG - 1) * KB>();
+    // the vectors (and the rows requested before them) have landed when only the later matrix loads and the scales are still under way
+    wait_vmcnt<(RG - 1) * KB + 2 * NOUT>();
     __builtin_amdgcn_sched_barrier(0);
     int4_t vf[NB][KB];
 #pragma unroll
@@ -358,32 +364,30 @@ __global__ __launch_bounds__(512) void k_gemv_direct(int32_t batch, int32_t dim_
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb) vf[t][kb] = *reinterpret_cast<const int4_t*>(vp + (((kb * 4 + q) ^ (v & 15)) << 4));
     }
-    int4_t acc[RG][NB];
+    __syncthreads();       // (part is zero)
+    // A row group's products are added to the workgroup's sums as soon as they exist, so that behind the last
+    // data only the last group's remain.  Accumulator e of lane l: matrix row (l/16)*4 + e, vector l%16 of the 16x16 tile.
 #pragma unroll
-    for (int g = 0; g < RG; ++g)
+    for (int g = 0; g < RG; ++g) {
+        int4_t acc[NB];
 #pragma unroll
-        for (int t = 0; t < NB; ++t) acc[g][t] = int4_t{0, 0, 0, 0};
-#pragma unroll
-    for (int g = 0; g < RG; ++g)
+        for (int t = 0; t < NB; ++t) acc[t] = int4_t{0, 0, 0, 0};
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
-            for (int t = 0; t < NB; ++t) acc[g][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[g][kb], vf[t][kb], acc[g][t], 0, 0, 0);
-    __syncthreads();       // (part is zero)
-    // accumulator e of lane l: matrix row (l/16)*4 + e, vector l%16 of the 16x16 tile
-#pragma unroll
-    for (int g = 0; g < RG; ++g)
+            for (int t = 0; t < NB; ++t) acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[g][kb], vf[t][kb], acc[t], 0, 0, 0);
 #pragma unroll
         for (int t = 0; t < NB; ++t)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) atomicAdd(&part[(g * NB + t) * 256 + (q * 4 + e) * 16 + r], (int32_t)acc[g][t][e]);
+            for (int e = 0; e < 4; ++e) atomicAdd(&part[(g * NB + t) * 256 + (q * 4 + e) * 16 + r], (int32_t)acc[t][e]);
+        __builtin_amdgcn_sched_barrier(0);
+    }
     __syncthreads();
-    // thread -> (vector, row) with the row fastest, so a vector's outputs are stored contiguously
 #pragma unroll
     for (int o = 0; o < NOUT; ++o) {
         const int idx = tid + o * 512;
         if (idx < rpb * NB * 16) {
-            const int rr = idx % rpb, bb = idx / rpb;
+            const int rr = orr[o], bb = obb[o];
             const int g = rr >> 4, t = bb >> 4;
             const int32_t s = part[(g * NB + t) * 256 + (rr & 15) * 16 + (bb & 15)];
             const int32_t row = row0 + rr;
