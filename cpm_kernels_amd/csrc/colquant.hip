@@ -15,16 +15,16 @@ namespace cpmk {
 // consecutive rows rg*8 .. rg*8+7, so that its int8 results are 8 contiguous bytes in either
 // output layout.
 // (two 512-thread workgroups share a compute unit: at most 128 registers per lane)
-template <int NT>
+template <int NT, bool TRANSPOSED>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void k_col_quantize_team(int32_t n, int32_t m, int32_t tiles_per_batch, int32_t parts,
                                                           const half_t* __restrict__ mat, half_t* __restrict__ scale,
-                                                          int8_t* __restrict__ out, int transposed, XchLaunch xl) {
+                                                          int8_t* __restrict__ out, XchLaunch xl) {
     constexpr int LPR = 8, R = 8, COLS = 64, ROWS = NT / LPR * R;
     uint64_t* const xch = xl.region;
     const uint32_t tag = xl.tag;
     __shared__ float lds[(NT / 64 + 1) * COLS];
     __shared__ float tot[COLS];
-    __shared__ __attribute__((aligned(16))) int8_t tbuf[COLS * ROWS];       // the transposed int8 tile on its way out
+    __shared__ __attribute__((aligned(16))) int8_t tbuf[TRANSPOSED ? COLS * ROWS : 16];       // the transposed int8 tile on its way out
     const int tid = threadIdx.x, cg = tid % LPR, rg = tid / LPR;
     const uint32_t part = blockIdx.x % parts, team = blockIdx.x / parts;
     const uint32_t b = team / tiles_per_batch, ct = team - b * tiles_per_batch;
@@ -118,7 +118,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         }
     }
     if (col0 < m) {
-        if (!transposed) {
+        if constexpr (!TRANSPOSED) {
 #pragma unroll
             for (int p = 0; p < R; ++p)
                 if (row0 + p < n)
@@ -126,7 +126,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
                         uint2_t{q[p][0], q[p][1]};
         }
     }
-    if (transposed) {
+    if constexpr (TRANSPOSED) {
         // The tile leaves through LDS as 64 columns x ROWS bytes: a lane's 8 rows of a column are 8
         // bytes there, and 32 lanes then store one column's ROWS bytes as one contiguous run (16 bytes
         // per lane) instead of eight lanes storing 64 bytes of it.  8-byte slot s of column c sits at
@@ -223,9 +223,14 @@ int cpmk_gemm_quantize_cols(int32_t batch, int32_t n, int32_t m, const void* mat
                 }
                 if (rc != 0) return rc == kXchFull ? CPMK_ETOOBIG : rc;
             }
-            hipLaunchKernelGGL((k_col_quantize_team<512>), dim3((unsigned)(tiles * nb * parts)), dim3(512), 0, st, n, m,
-                               (int32_t)tiles, (int32_t)parts, (const half_t*)mat + b0 * n * m, (half_t*)scale + b0 * m,
-                               (int8_t*)out + b0 * n * m, out_transposed, xs.xl);
+            if (out_transposed)
+                hipLaunchKernelGGL((k_col_quantize_team<512, true>), dim3((unsigned)(tiles * nb * parts)), dim3(512), 0, st, n, m,
+                                   (int32_t)tiles, (int32_t)parts, (const half_t*)mat + b0 * n * m, (half_t*)scale + b0 * m,
+                                   (int8_t*)out + b0 * n * m, xs.xl);
+            else
+                hipLaunchKernelGGL((k_col_quantize_team<512, false>), dim3((unsigned)(tiles * nb * parts)), dim3(512), 0, st, n, m,
+                                   (int32_t)tiles, (int32_t)parts, (const half_t*)mat + b0 * n * m, (half_t*)scale + b0 * m,
+                                   (int8_t*)out + b0 * n * m, xs.xl);
             const int e = launch_status();
             const int rc2 = xs.end();
             if (e != 0 || rc2 != 0) return e ? e : rc2;
