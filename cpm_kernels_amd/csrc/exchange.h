@@ -153,6 +153,38 @@ __device__ inline bool xch_gather(const uint64_t* team_slots, int parts, int q0,
     }
 }
 
+// The same for two packets of every part, `ia` and `ib`, all polled together: one round trip to the L2 where
+// two calls of xch_gather would make two, one after the other.
+template <int W>
+__device__ inline bool xch_gather2(const uint64_t* team_slots, int parts, int q0, int ia, int ib, uint32_t tag, uint64_t deadline,
+                                   float (&va)[W], float (&vb)[W]) {
+    uint32_t missing = 0;           // bit j: packet ia of part q0 + j, bit W + j: packet ib
+#pragma unroll
+    for (int j = 0; j < W; ++j) {
+        va[j] = vb[j] = 0.0f;
+        if (q0 + j < parts) missing |= (1u << j) | (1u << (W + j));
+    }
+    for (;;) {
+        uint64_t pk[2 * W];
+#pragma unroll
+        for (int j = 0; j < 2 * W; ++j)
+            if (missing >> j & 1u)
+                pk[j] = __hip_atomic_load(team_slots + (size_t)(q0 + j % W) * kXchVals + (j < W ? ia : ib), __ATOMIC_RELAXED,
+                                          __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+        for (int j = 0; j < 2 * W; ++j)
+            if ((missing >> j & 1u) && (uint32_t)(pk[j] >> 32) == tag) {
+                const float x = __builtin_bit_cast(float, (uint32_t)pk[j]);
+                if (j < W) va[j] = x;
+                else vb[j - W] = x;
+                missing &= ~(1u << j);
+            }
+        if (missing == 0) return true;
+        if ((uint64_t)wall_clock64() > deadline) return false;
+        __builtin_amdgcn_s_sleep(2);
+    }
+}
+
 // To be called by the first wave of a workgroup once the whole workgroup has collected its
 // packets (i.e. after the barrier that follows the xch_wait calls): counts the team members that
 // are done and lets the last one clear the team's `parts` slots and the counter.

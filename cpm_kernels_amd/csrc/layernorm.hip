@@ -178,8 +178,7 @@ __global__ __launch_bounds__(NT) void k_layernorm_team(int32_t n, int32_t m, int
         bool ok = true;
         for (int32_t q0 = 0; q0 < parts; q0 += 4) {
             float x[4], y[4];
-            ok &= xch_gather<4>(team_slots, parts, q0, tid, tag, deadline, x);
-            ok &= xch_gather<4>(team_slots, parts, q0, T::COLS + tid, tag, deadline, y);
+            ok &= xch_gather2<4>(team_slots, parts, q0, tid, T::COLS + tid, tag, deadline, x, y);      // both statistics of four parts in one round trip
 #pragma unroll
             for (int j = 0; j < 4; ++j) {                  // in part order; absent parts are zeros
                 sum += x[j];

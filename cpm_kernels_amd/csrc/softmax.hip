@@ -241,19 +241,23 @@ __global__ __launch_bounds__(NT) void k_softmax_team(int32_t n, int32_t m, int32
     }
     if (tid < T::COLS) {
         const uint64_t deadline = wall_clock64() + kXchTimeoutTicks;
+        static_assert(kXchMaxParts == 8, "two rounds of gathers cover a team");
         float mp[kXchMaxParts], sp[kXchMaxParts];
         bool ok = true;
-        float M = -__builtin_inff();
 #pragma unroll
-        for (int q = 0; q < kXchMaxParts; ++q) {
-            mp[q] = -__builtin_inff();
-            sp[q] = 0.0f;
-            if (q < parts) {
-                ok &= xch_wait(team_slots + (size_t)q * kXchVals + tid, tag, deadline, mp[q]);
-                ok &= xch_wait(team_slots + (size_t)q * kXchVals + T::COLS + tid, tag, deadline, sp[q]);
-                M = fmaxf(M, mp[q]);
+        for (int q0 = 0; q0 < kXchMaxParts; q0 += 4) {          // four parts' m_p, then their s_p, per round trip (all eight at once, or both statistics at once, spill registers)
+            float a[4], c[4];
+            ok &= xch_gather<4>(team_slots, parts, q0, tid, tag, deadline, a);
+            ok &= xch_gather<4>(team_slots, parts, q0, T::COLS + tid, tag, deadline, c);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                mp[q0 + j] = q0 + j < parts ? a[j] : -__builtin_inff();        // (absent parts: s_p is 0 already)
+                sp[q0 + j] = c[j];
             }
         }
+        float M = -__builtin_inff();
+#pragma unroll
+        for (int q = 0; q < kXchMaxParts; ++q) M = fmaxf(M, mp[q]);
         float S = 0.0f;
 #pragma unroll
         for (int q = 0; q < kXchMaxParts; ++q)
