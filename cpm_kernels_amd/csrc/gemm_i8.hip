@@ -390,6 +390,33 @@ struct SlabDma {
     }
 };
 
+// The way out of a tile, shared by the two forms of the tile function.  Results leave through a 4 KB strip of
+// LDS per wave: a lane holds 4-column pieces of ONE output row, so storing straight from the accumulators
+// would touch 32 different rows with 8 or 16 bytes each per instruction.  Written to the strip as 32 rows x RB
+// bytes and read back 16 bytes per lane, every store instruction covers whole contiguous rows of the chunk
+// (RB = 128 bytes: eight lanes per 128-byte line).
+template <int EPI, int TC>
+struct StripOut {
+    static constexpr int ESZ = EPI == kEpiInt32 ? 4 : 2;
+    static constexpr int CT = EPI == kEpiInt32 ? 1 : TC;       // MFMA tile columns (of 32) side by side in one chunk
+    static constexpr int NCH = EPI == kEpiInt32 ? TC : 1;      // chunks per block of 32 rows
+    static constexpr int RB = CT * 32 * ESZ, PPR = RB / 16, RPW2 = 256 / RB, PASSES = PPR / 2, RPP = 64 / PPR;
+    // 16-byte piece p of strip row r sits at piece slot p ^ ((r / RPW2) % PPR): reads are conflict free
+    static __device__ __forceinline__ int slot(int r, int p) { return (p ^ ((r / RPW2) & (PPR - 1))) << 4; }
+    // the strip's 32 rows go out: output rows row0 .. row0 + 31, columns from col0 on
+    static __device__ __forceinline__ void store_rows(const GemmArgs& a, const int8_t* stg, int64_t obase, int32_t row0, int32_t col0, int lane) {
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ++ps) {
+            const int R = ps * RPP + lane / PPR, pc = lane % PPR;
+            const int4_t v = *reinterpret_cast<const int4_t*>(stg + R * RB + slot(R, pc));
+            const int32_t row = row0 + R;
+            const int32_t col = col0 + pc * (16 / ESZ);
+            if (row < a.n && col < a.m)
+                store_piece<ESZ>(reinterpret_cast<int8_t*>(a.out) + (obase + (int64_t)row * a.m + col) * ESZ, v, a.m - col);
+        }
+    }
+};
+
 // One output tile of BR x BC = (WR*TR*32) x (WC*TC*32), K slab = BKB bytes.
 // The MFMA is the 16x16 one with 64 bytes of K (v_mfma_i32_16x16x64_i8, v_mfma_f32_16x16x32_f16):
 // per operation it moves half the accumulator registers of the 32x32 form, and on random operands,
@@ -578,17 +605,9 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
     ring = cur;                          // (ring0 + nk) % NST: where the next tile's slab 0 is, or will be put
 
     const int64_t obase = (int64_t)b * a.n * a.m;
-    // Results leave through a 4 KB strip of LDS per wave: a lane holds 4-column pieces of ONE
-    // output row, so storing straight from the accumulators would touch 32 different rows
-    // with 8 or 16 bytes each per instruction.  Written to the strip as 32 rows x RB bytes
-    // and read back 16 bytes per lane, every store instruction covers whole contiguous rows
-    // of the chunk (RB = 128 bytes: eight lanes per 128-byte line).
-    constexpr int ESZ = EPI == kEpiInt32 ? 4 : 2;
-    constexpr int CT = EPI == kEpiInt32 ? 1 : TC;       // MFMA tiles side by side in one chunk
-    constexpr int NCH = EPI == kEpiInt32 ? TC : 1;      // chunks per block of 32 rows
-    constexpr int RB = CT * 32 * ESZ, PPR = RB / 16, RPW2 = 256 / RB, PASSES = PPR / 2, RPP = 64 / PPR;
-    // 16-byte piece p of strip row r sits at piece slot p ^ ((r / RPW2) % PPR): reads are conflict free
-    auto slot = [](int r, int p) __attribute__((always_inline)) { return (p ^ ((r / RPW2) & (PPR - 1))) << 4; };
+    using Out = StripOut<EPI, TC>;       // the results leave through this wave's strip of LDS
+    constexpr int NCH = Out::NCH, RB = Out::RB;
+    auto slot = [](int r, int p) __attribute__((always_inline)) { return Out::slot(r, p); };
     half_t sxr[AR];
     half4_t syr[AC];
     if (FUSED) {      // the scales come back from the strip before the results overwrite it
@@ -630,15 +649,7 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
                     }
                 }
             }
-#pragma unroll
-            for (int ps = 0; ps < PASSES; ++ps) {
-                const int R = ps * RPP + lane / PPR, pc = lane % PPR;
-                const int4_t v = *reinterpret_cast<const int4_t*>(stg + R * RB + slot(R, pc));
-                const int32_t row = j0 + wr * TR * 32 + i * 32 + R;
-                const int32_t col = i0 + wc * TC * 32 + c * 32 + pc * (16 / ESZ);
-                if (row < a.n && col < a.m)
-                    store_piece<ESZ>(reinterpret_cast<int8_t*>(a.out) + (obase + (int64_t)row * a.m + col) * ESZ, v, a.m - col);
-            }
+            Out::store_rows(a, stg, obase, j0 + wr * TR * 32 + i * 32, i0 + wc * TC * 32 + c * 32, lane);
         }
     }
     return ahead;
@@ -837,17 +848,9 @@ __device__ __forceinline__ bool gemm_dma_tile32(const GemmArgs& a, int8_t* smem,
     ring = cur;                          // (ring0 + nk) % NST: where the next tile's slab 0 is, or will be put
 
     const int64_t obase = (int64_t)b * a.n * a.m;
-    // Results leave through a 4 KB strip of LDS per wave: a lane holds 4-column pieces of ONE
-    // output row, so storing straight from the accumulators would touch 32 different rows
-    // with 8 or 16 bytes each per instruction.  Written to the strip as 32 rows x RB bytes
-    // and read back 16 bytes per lane, every store instruction covers whole contiguous rows
-    // of the chunk (RB = 128 bytes: eight lanes per 128-byte line).
-    constexpr int ESZ = EPI == kEpiInt32 ? 4 : 2;
-    constexpr int CT = EPI == kEpiInt32 ? 1 : TC;       // MFMA tiles side by side in one chunk
-    constexpr int NCH = EPI == kEpiInt32 ? TC : 1;      // chunks per block of 32 rows
-    constexpr int RB = CT * 32 * ESZ, PPR = RB / 16, RPW2 = 256 / RB, PASSES = PPR / 2, RPP = 64 / PPR;
-    // 16-byte piece p of strip row r sits at piece slot p ^ ((r / RPW2) % PPR): reads are conflict free
-    auto slot = [](int r, int p) __attribute__((always_inline)) { return (p ^ ((r / RPW2) & (PPR - 1))) << 4; };
+    using Out = StripOut<EPI, TC>;       // the results leave through this wave's strip of LDS
+    constexpr int NCH = Out::NCH, RB = Out::RB;
+    auto slot = [](int r, int p) __attribute__((always_inline)) { return Out::slot(r, p); };
     half_t sxr[TR];
     half4_t syr[TC][4];
     if (FUSED) {      // the scales come back from the strip before the results overwrite it
@@ -894,15 +897,7 @@ __device__ __forceinline__ bool gemm_dma_tile32(const GemmArgs& a, int8_t* smem,
                         *reinterpret_cast<half4_t*>(stg + lrow * RB + slot(lrow, j * 4 + g4) + lk * 8) = h;
                     }
             }
-#pragma unroll
-            for (int ps = 0; ps < PASSES; ++ps) {
-                const int R = ps * RPP + lane / PPR, pc = lane % PPR;
-                const int4_t v = *reinterpret_cast<const int4_t*>(stg + R * RB + slot(R, pc));
-                const int32_t row = j0 + wr * TR * 32 + i * 32 + R;
-                const int32_t col = i0 + wc * TC * 32 + c * 32 + pc * (16 / ESZ);
-                if (row < a.n && col < a.m)
-                    store_piece<ESZ>(reinterpret_cast<int8_t*>(a.out) + (obase + (int64_t)row * a.m + col) * ESZ, v, a.m - col);
-            }
+            Out::store_rows(a, stg, obase, j0 + wr * TR * 32 + i * 32, i0 + wc * TC * 32 + c * 32, lane);
         }
     }
     return ahead;
