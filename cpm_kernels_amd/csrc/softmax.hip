@@ -93,13 +93,13 @@ __global__ __launch_bounds__(NT) void k_softmax_tile(int32_t n, int32_t m, int32
 // Tiles are handed out dynamically: the first gridDim.x tiles by workgroup index, the rest from a
 // counter in device memory.  With a fixed share per workgroup the kernel ends with its slowest
 // compute unit, and on this chip one in eight gets 25 % less memory bandwidth than the rest.
-// The workgroup that finishes last clears the counters, so a launch (or a graph replay) always
-// finds them zero; launches that may overlap in time use different counter slots.
-constexpr int kSmSlots = 64;
-__device__ unsigned int g_sm_sched[kSmSlots][2];       // [0] tiles handed out beyond the first round, [1] finished workgroups
+// The two counters (sched[0]: tiles handed out beyond the first round, sched[1]: finished workgroups) are the
+// launch's own: they come out of the exchange pool (exchange.h) with the same bookkeeping as a team's packet
+// slots, so no other launch or graph that may run at the same time shares them.  The workgroup that finishes
+// last clears them, so the next holder (or a replay of the graph) finds them zero.
 
 template <int NT, int LPR, int R>
-__global__ __launch_bounds__(NT) void k_softmax_stream(int32_t n, int32_t m, int32_t tiles_per_batch, uint32_t ntiles, uint32_t slot,
+__global__ __launch_bounds__(NT) void k_softmax_stream(int32_t n, int32_t m, int32_t tiles_per_batch, uint32_t ntiles, unsigned int* sched,
                                                        const half_t* inp, half_t* out) {
     using T = ColTile<NT, LPR, R>;
     constexpr int RPP = NT / LPR;
@@ -111,7 +111,7 @@ __global__ __launch_bounds__(NT) void k_softmax_stream(int32_t n, int32_t m, int
     const int8_t* stage = dyn + wave * (R * 1024) + lane * 16;
     const uint32_t stage_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) int8_t*)(dyn + wave * (R * 1024));
     const uint32_t G = gridDim.x;
-    unsigned int* ctr = &g_sm_sched[slot][0];
+    unsigned int* ctr = sched;
     const int rg = tid / LPR, cg = tid % LPR;
     auto issue = [&](uint32_t t) __attribute__((always_inline)) {
         const uint32_t b = t / tiles_per_batch, ct = t - b * tiles_per_batch;
@@ -163,11 +163,11 @@ __global__ __launch_bounds__(NT) void k_softmax_stream(int32_t n, int32_t m, int
         t = tn;
         tn = tnn;
     }
-    // every workgroup is past its last fetch when it signs off, so the last one to do so may clear the slot
+    // every workgroup is past its last fetch when it signs off, so the last one to do so may clear the counters
     if (tid == 0) {
-        if (atomicAdd(&g_sm_sched[slot][1], 1u) == G - 1) {
-            atomicExch(&g_sm_sched[slot][0], 0u);
-            atomicExch(&g_sm_sched[slot][1], 0u);
+        if (atomicAdd(sched + 1, 1u) == G - 1) {
+            atomicExch(sched, 0u);
+            atomicExch(sched + 1, 0u);
         }
     }
 }
@@ -330,10 +330,9 @@ static void launch_tile(int32_t batch, int32_t n, int32_t m, const half_t* inp, 
                        tiles, inp, out);
 }
 
-// launches that may be in flight together get different scheduling counters (one sequence for all instantiations)
-static unsigned g_sm_next_slot = 0;
-
-// persistent variant: one workgroup per compute unit, 16 bytes of LDS staging per element slot
+// persistent variant: one workgroup per compute unit, 16 bytes of LDS staging per element slot.  Returns kXchFull
+// (and launches nothing) when the call is recorded into a graph and the pool's capture reserve has no room
+// for the launch's counters: the caller then records a kernel that needs none.
 template <int NT, int LPR, int R>
 static int launch_stream(int32_t batch, int32_t n, int32_t m, const half_t* inp, half_t* out, hipStream_t st) {
     using T = ColTile<NT, LPR, R>;
@@ -345,9 +344,14 @@ static int launch_stream(int32_t batch, int32_t n, int32_t m, const half_t* inp,
     const int32_t tiles = (int32_t)ceil_div(m, LPR * 8);
     const int64_t ntiles = (int64_t)tiles * batch;
     const int cus = compute_units();
-    const unsigned slot = __atomic_fetch_add(&g_sm_next_slot, 1u, __ATOMIC_RELAXED) % kSmSlots;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(ntiles < cus ? ntiles : cus)), dim3(NT), smem, st, n, m, tiles, (uint32_t)ntiles, slot, inp, out);
-    return launch_status();
+    XchScope xs;
+    if (int rc = xs.begin(1, st)) return rc;
+    // the first team counter of the launch's range: eight bytes, all zero, used as two 32-bit counters
+    hipLaunchKernelGGL(kern, dim3((unsigned)(ntiles < cus ? ntiles : cus)), dim3(NT), smem, st, n, m, tiles, (uint32_t)ntiles,
+                       reinterpret_cast<unsigned int*>(xs.xl.counters), inp, out);
+    const int e = launch_status();
+    const int rc2 = xs.end();
+    return e ? e : rc2;
 }
 
 template <int NT, int LPR>
@@ -406,8 +410,10 @@ static int softmax_dispatch(int32_t batch, int32_t n, int32_t m, const void* inp
         }
         // several tiles per compute unit: the persistent kernel keeps loads in flight during the arithmetic
         if (n > 256 && n <= 1024 && m >= 64 && ceil_div(m, 64) * batch >= 2 * (int64_t)compute_units() &&
-            ceil_div(m, 64) * batch < (1ll << 31))
-            return n > 512 ? launch_stream<1024, 8, 8>(batch, n, m, x, y, st) : launch_stream<1024, 8, 4>(batch, n, m, x, y, st);
+            ceil_div(m, 64) * batch < (1ll << 31)) {
+            const int rc = n > 512 ? launch_stream<1024, 8, 8>(batch, n, m, x, y, st) : launch_stream<1024, 8, 4>(batch, n, m, x, y, st);
+            if (rc != kXchFull) return rc;
+        }
         if (n <= 64 * 8 && m >= 64) ok = launch_tile_r<512, 8>((int)ceil_div(n, 64), batch, n, m, x, y, st);
         else if (n <= 128 * 8 && m >= 64) ok = launch_tile_r<1024, 8>((int)ceil_div(n, 128), batch, n, m, x, y, st);
         else if (n <= 256 * 8 && m >= 32) ok = launch_tile_r<1024, 4>((int)ceil_div(n, 256), batch, n, m, x, y, st);

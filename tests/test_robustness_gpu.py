@@ -286,3 +286,41 @@ def test_captured_team_launch_between_eager_launches_on_another_stream(gpu):
         assert_bits_equal(to_np(ya), to_np(ref_a), "replays of round %d" % rnd)
         for o in outs:
             assert_bits_equal(to_np(o), to_np(ref_b), "eager launches of round %d" % rnd)
+
+
+def test_captured_many_tile_softmax_beside_eager_ones_on_another_stream(gpu):
+    """The many-tile softmax hands its tiles out from two counters in device memory.  They belong to the launch
+    (they come out of the exchange pool like a team's packet slots), so a recorded softmax may be replayed while
+    any number of eager ones run on a second stream: every result equals the single-stream result bit for bit."""
+    _name("captured many-tile softmax replayed beside 120 eager ones on a second stream")
+    from cpm_kernels_amd.library import cpmk
+    g = torch.Generator().manual_seed(46)
+    shape = (40, 1024, 1024)                # 640 column tiles: more than two per compute unit
+    xa = (torch.randn(shape, generator=g) * 3).half().to(gpu)
+    xb = (torch.randn(shape, generator=g) * 2 + 0.5).half().to(gpu)
+    ref_a, ref_b = torch.empty_like(xa), torch.empty_like(xb)
+    ck.softmax_forward(*shape, xa.data_ptr(), ref_a.data_ptr(), stream())
+    ck.softmax_forward(*shape, xb.data_ptr(), ref_b.data_ptr(), stream())
+    torch.cuda.synchronize()
+    left = cpmk.exchange_capture_slots_left()
+    ya = torch.zeros_like(xa)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ck.softmax_forward(*shape, xa.data_ptr(), ya.data_ptr(), stream())
+    assert cpmk.exchange_capture_slots_left() < left, "the recorded launch's counters come out of the capture reserve"
+    sa, sb = torch.cuda.Stream(), torch.cuda.Stream()
+    outs = [torch.zeros_like(xb) for _ in range(3)]
+    for rnd in range(3):
+        ya.fill_(0)
+        torch.cuda.synchronize()
+        for i in range(40):
+            with torch.cuda.stream(sb):
+                ck.softmax_forward(*shape, xb.data_ptr(), outs[i % 3].data_ptr(), sb.cuda_stream)
+            if i % 8 == 4:
+                with torch.cuda.stream(sa):
+                    graph.replay()
+        torch.cuda.synchronize()
+        cpmk.async_status()
+        assert_bits_equal(to_np(ya), to_np(ref_a), "replays of round %d" % rnd)
+        for o in outs:
+            assert_bits_equal(to_np(o), to_np(ref_b), "eager launches of round %d" % rnd)
