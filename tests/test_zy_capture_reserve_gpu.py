@@ -25,6 +25,10 @@ def test_recorded_launches_beyond_the_reserve_run_without_packets(gpu):
     ref_sm = torch.empty_like(xt); ref_sc = torch.empty((2, 128), dtype=torch.half, device=gpu); ref_q = torch.empty((2, 128, 4096), dtype=torch.int8, device=gpu)
     ck.softmax_forward(2, 4096, 128, xt.data_ptr(), ref_sm.data_ptr(), stream())
     ck.gemm_quantize_cols(2, 4096, 128, xt.data_ptr(), ref_sc.data_ptr(), ref_q.data_ptr(), True, stream())
+    # a softmax over many column tiles (640: more than two per compute unit), whose tile counters come out of the pool too
+    xm = (torch.randn(40, 1024, 1024, generator=g) * 3).half().to(gpu)
+    ref_many = torch.empty_like(xm); many = torch.zeros_like(xm)
+    ck.softmax_forward(40, 1024, 1024, xm.data_ptr(), ref_many.data_ptr(), stream())
     torch.cuda.synchronize()
     assert cpmk.exchange_capture_slots_left() <= 140 * 256
     ys = [torch.zeros_like(x) for _ in range(4)]
@@ -54,6 +58,7 @@ def test_recorded_launches_beyond_the_reserve_run_without_packets(gpu):
         ck.layernorm_forward(8, 4096, 512, x.data_ptr(), ys[3].data_ptr(), 1e-5, True, stream())
         ck.softmax_forward(2, 4096, 128, xt.data_ptr(), sm.data_ptr(), stream())
         ck.gemm_quantize_cols(2, 4096, 128, xt.data_ptr(), sc.data_ptr(), q.data_ptr(), True, stream())
+        ck.softmax_forward(40, 1024, 1024, xm.data_ptr(), many.data_ptr(), stream())
     last = record(without_packets)                             # the reserve is empty: recorded as kernels that need no packets
     for rep in range(2):
         for y in ys:
@@ -75,6 +80,8 @@ def test_recorded_launches_beyond_the_reserve_run_without_packets(gpu):
         assert_close_fp16(to_np(sm), to_np(ref_sm).astype(np.float64), rtol=1e-3, atol=1e-6, what="softmax without slots")
         assert_bits_equal(to_np(sc), to_np(ref_sc), "column scales without slots")
         assert_bits_equal(to_np(q), to_np(ref_q), "column int8 without slots")
+        # (one tile per workgroup instead of tiles from a counter: the same arithmetic on every column)
+        assert_bits_equal(to_np(many), to_np(ref_many), "many-tile softmax without counters")
     # eager launches are not affected
     y = torch.zeros_like(x)
     ck.layernorm_forward(8, 4096, 512, x.data_ptr(), y.data_ptr(), 1e-5, True, stream())
