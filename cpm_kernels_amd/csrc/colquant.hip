@@ -18,7 +18,7 @@ namespace cpmk {
 template <int NT, bool TRANSPOSED>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void k_col_quantize_team(int32_t n, int32_t m, int32_t tiles_per_batch, int32_t parts,
                                                           const half_t* __restrict__ mat, half_t* __restrict__ scale,
-                                                          int8_t* __restrict__ out, XchLaunch xl) {
+                                                          int8_t* __restrict__ out, uint32_t nteams, XchLaunch xl) {
     constexpr int LPR = 8, R = 8, COLS = 64, ROWS = NT / LPR * R;
     uint64_t* const xch = xl.region;
     const uint32_t tag = xl.tag;
@@ -26,7 +26,9 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     __shared__ float tot[COLS];
     __shared__ __attribute__((aligned(16))) int8_t tbuf[TRANSPOSED ? COLS * ROWS : 16];       // the transposed int8 tile on its way out
     const int tid = threadIdx.x, cg = tid % LPR, rg = tid / LPR;
-    const uint32_t part = blockIdx.x % parts, team = blockIdx.x / parts;
+    XchMember me;
+    if (!xch_member(blockIdx.x, parts, nteams, me)) return;
+    const uint32_t part = me.part, team = me.team;
     const uint32_t b = team / tiles_per_batch, ct = team - b * tiles_per_batch;
     const int32_t col0 = ct * COLS + cg * 8;
     const int32_t row0 = part * ROWS + rg * 8;           // this lane's first row
@@ -210,7 +212,7 @@ int cpmk_gemm_quantize_cols(int32_t batch, int32_t n, int32_t m, const void* mat
                          parts <= kColMaxParts && tiles * parts <= kXchSlots;
     if (team_ok) {
         // teams use one packet slot per (team, part): batches beyond the pool go out in several launches
-        const int64_t per_launch = parts > 1 ? kXchSlots / (tiles * parts) : ((1ll << 31) - 1) / (tiles * parts);
+        const int64_t per_launch = parts > 1 ? kXchSlots / (tiles * parts) : ((1ll << 31) - 8) / (tiles * parts);
         bool no_slots = false;
         for (int64_t b0 = 0; b0 < batch; b0 += per_launch) {
             const int64_t nb = batch - b0 < per_launch ? batch - b0 : per_launch;
@@ -224,13 +226,13 @@ int cpmk_gemm_quantize_cols(int32_t batch, int32_t n, int32_t m, const void* mat
                 if (rc != 0) return rc == kXchFull ? CPMK_ETOOBIG : rc;
             }
             if (out_transposed)
-                hipLaunchKernelGGL((k_col_quantize_team<512, true>), dim3((unsigned)(tiles * nb * parts)), dim3(512), 0, st, n, m,
+                hipLaunchKernelGGL((k_col_quantize_team<512, true>), dim3((unsigned)xch_team_grid(tiles * nb, parts)), dim3(512), 0, st, n, m,
                                    (int32_t)tiles, (int32_t)parts, (const half_t*)mat + b0 * n * m, (half_t*)scale + b0 * m,
-                                   (int8_t*)out + b0 * n * m, xs.xl);
+                                   (int8_t*)out + b0 * n * m, (uint32_t)(tiles * nb), xs.xl);
             else
-                hipLaunchKernelGGL((k_col_quantize_team<512, false>), dim3((unsigned)(tiles * nb * parts)), dim3(512), 0, st, n, m,
+                hipLaunchKernelGGL((k_col_quantize_team<512, false>), dim3((unsigned)xch_team_grid(tiles * nb, parts)), dim3(512), 0, st, n, m,
                                    (int32_t)tiles, (int32_t)parts, (const half_t*)mat + b0 * n * m, (half_t*)scale + b0 * m,
-                                   (int8_t*)out + b0 * n * m, xs.xl);
+                                   (int8_t*)out + b0 * n * m, (uint32_t)(tiles * nb), xs.xl);
             const int e = launch_status();
             const int rc2 = xs.end();
             if (e != 0 || rc2 != 0) return e ? e : rc2;

@@ -1,7 +1,7 @@
 // Exchange of per-column partial statistics between the workgroups of a team.
 //
 // A column reduction whose rows do not fit one workgroup's registers is split over the P
-// workgroups of a team (workgroups t*P .. t*P+P-1 of the launch, dispatched side by side).  Each
+// workgroups of a team (P workgroups that one XCD starts one after the other, see xch_member).  Each
 // posts its partials as 8-byte packets {value, launch tag} with device-scope atomic stores and
 // collects its team mates' packets by polling until the tag matches; a packet is valid as a
 // whole or not at all, so no fence and no separate flag is needed, and the packets of an older
@@ -26,13 +26,14 @@
 // or captured, is ever given it.  When the reserve is used up XchScope::begin says so (kXchFull)
 // and the caller records its kernel that needs no packets instead.
 //
-// Progress: a workgroup only ever waits for workgroups of its own team, whose indices differ by
-// less than the team size; the dispatcher starts the workgroups of a launch in index order (an
-// observed property of the hardware queue, not a documented one), so all members of the oldest
-// unfinished team are resident and that team completes.  Should a packet nevertheless not arrive
-// within about a second the wait gives up, the caller writes NaN (0 in an int8 output) and sets
-// the device's sticky status word and its mirror in pinned host memory.  Every launcher of the
-// library looks at the mirror before it returns (launch_status() in common.h), so the failure is
+// Progress: a workgroup only ever waits for workgroups of its own team, which are the next ones that its own
+// XCD starts for this launch (xch_member; that an XCD starts a launch's workgroups in index order is an observed
+// property of the hardware queue, not a documented one).  With several launches sharing the chip at most
+// (team size - 1) workgroups per launch and XCD can be waiting for a member that has not started, so the
+// oldest unfinished team of every XCD gets its members as soon as compute units are free there.  Should a
+// packet nevertheless not arrive within about a second the wait gives up, the caller writes NaN (0 in an int8
+// output) and sets the device's sticky status word and its mirror in pinned host memory.  Every launcher of
+// the library looks at the mirror before it returns (launch_status() in common.h), so the failure is
 // reported by the next call, whichever it is, like an asynchronous error of the runtime itself;
 // cpmk_async_status() reports and clears it: a visible failure instead of a hung GPU.
 #pragma once
@@ -184,6 +185,27 @@ __device__ inline bool xch_gather2(const uint64_t* team_slots, int parts, int q0
         __builtin_amdgcn_s_sleep(2);
     }
 }
+
+// Which team a workgroup belongs to.  The hardware deals the workgroups of a launch out to the chip's 8 XCDs
+// round robin (workgroup i runs on XCD i % 8), and every XCD starts its share on its own, in index order, as its
+// compute units become free: nothing orders the XCDs among each other.  A team therefore consists of workgroups of
+// ONE XCD that follow one another in that XCD's order -- workgroups 8s + x for `parts` consecutive s -- so a
+// member only ever waits for members that the same XCD starts next, whatever other launches keep the other XCDs
+// busy with (and its packets stay in that XCD's L2).  Teams go to the XCDs in turn: team t is the (t / 8)-th
+// team of XCD t % 8.  The grid holds whole teams on every XCD, xch_team_grid() workgroups; those of teams past
+// the last one find `false` here and leave at once.
+struct XchMember {
+    uint32_t team, part;
+};
+__device__ inline bool xch_member(uint32_t workgroup, uint32_t parts, uint32_t nteams, XchMember& m) {
+    const uint32_t x = workgroup & 7u, s = workgroup >> 3;
+    const uint32_t local = s / parts;
+    m.part = s - local * parts;
+    m.team = local * 8u + x;
+    return m.team < nteams;
+}
+// Host: workgroups to launch for `nteams` teams of `parts` members.
+inline int64_t xch_team_grid(int64_t nteams, int64_t parts) { return ceil_div(nteams, 8) * 8 * parts; }
 
 // To be called by the first wave of a workgroup once the whole workgroup has collected its
 // packets (i.e. after the barrier that follows the xch_wait calls): counts the team members that

@@ -113,7 +113,7 @@ __global__ __launch_bounds__(NT) void k_layernorm_team(int32_t n, int32_t m, int
                                                        const half_t* mat, half_t* out,
                                                        const half_t* __restrict__ alpha,
                                                        const half_t* __restrict__ beta, float eps, int rd_mean,
-                                                       int xcd_local, XchLaunch xl) {
+                                                       uint32_t nteams, XchLaunch xl) {
     constexpr int LPR = 8;
     using T = ColTile<NT, LPR, R>;
     static_assert(T::COLS * 2 == kXchVals, "slot layout");
@@ -124,12 +124,9 @@ __global__ __launch_bounds__(NT) void k_layernorm_team(int32_t n, int32_t m, int
     __shared__ half_t coef[2][NT];        // alpha and beta of this workgroup's rows (T::ROWS == NT)
     static_assert(T::ROWS == NT, "one affine coefficient pair per thread");
     const int tid = threadIdx.x;
-    // xcd_local (a launch of one round whose eighths hold whole teams): workgroup i runs on XCD i % 8, so
-    // renumbering puts the members of a team on one XCD and their packets stay in that XCD's L2 (1.4 % at
-    // 8 x 4096 x 512; with more rounds than one the same renumbering loses 3 %)
-    const uint32_t G = gridDim.x;
-    const uint32_t wid = xcd_local ? (blockIdx.x % 8) * (G / 8) + blockIdx.x / 8 : blockIdx.x;
-    const uint32_t part = wid % parts, team = wid / parts;
+    XchMember me;
+    if (!xch_member(blockIdx.x, parts, nteams, me)) return;
+    const uint32_t part = me.part, team = me.team;
     const uint32_t b = team / tiles_per_batch, ct = team - b * tiles_per_batch;
     const int32_t col0 = ct * T::COLS + (tid % LPR) * 8;
     const int32_t own0 = part * T::ROWS;                 // first row this workgroup normalises
@@ -352,18 +349,12 @@ static int layernorm_dispatch(int32_t batch, int32_t n, int32_t m, const void* m
                         if (rc != 0) return rc == kXchFull ? CPMK_ETOOBIG : rc;
                     }
                     const XchLaunch& xl = xs.xl;
-                    const dim3 grid((unsigned)(tiles * nb * parts));
+                    const dim3 grid((unsigned)xch_team_grid(tiles * nb, parts));
                     const half_t* xb = x + b0 * n * m;
                     half_t* yb = y + b0 * n * m;
-                    // Members of a team on one XCD when the launch is one round whose eighths hold whole teams.  With
-                    // the renumbering a team's members are 8 workgroup indices apart, so up to 8 * (parts - 1)
-                    // workgroups of a launch can be waiting for members that have not started when other launches
-                    // share the chip; kept to teams of at most four so that this stays a small part of the chip.
-                    const int64_t G = tiles * nb * parts;
-                    const int xcd_local = parts <= 4 && G % 8 == 0 && (G / 8) % parts == 0 && G <= compute_units() * (big ? 1 : 2);
                     auto go = [&](auto kern, int threads) {
                         hipLaunchKernelGGL(kern, grid, dim3(threads), 0, st, n, m, (int32_t)tiles, (int32_t)parts, xb, yb, al, be, eps,
-                                           rd_mean, xcd_local, xl);
+                                           rd_mean, (uint32_t)(tiles * nb), xl);
                     };
                     if (big) {
                         if (al != nullptr) go(k_layernorm_team<1024, 8, true>, 1024);

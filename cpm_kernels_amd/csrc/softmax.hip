@@ -179,7 +179,7 @@ __global__ __launch_bounds__(NT) void k_softmax_stream(int32_t n, int32_t m, int
 // which is the single-workgroup result up to two extra fp32 roundings.
 template <int NT, int R>
 __global__ __launch_bounds__(NT) void k_softmax_team(int32_t n, int32_t m, int32_t tiles_per_batch, int32_t parts,
-                                                     const half_t* inp, half_t* out, XchLaunch xl) {
+                                                     const half_t* inp, half_t* out, uint32_t nteams, XchLaunch xl) {
     constexpr int LPR = 8;
     using T = ColTile<NT, LPR, R>;
     static_assert(T::COLS * 2 == kXchVals, "slot layout");
@@ -188,7 +188,9 @@ __global__ __launch_bounds__(NT) void k_softmax_team(int32_t n, int32_t m, int32
     __shared__ float lds[(T::NW + 1) * T::COLS];
     __shared__ float tot[kXchVals];
     const int tid = threadIdx.x;
-    const uint32_t part = blockIdx.x % parts, team = blockIdx.x / parts;
+    XchMember me;
+    if (!xch_member(blockIdx.x, parts, nteams, me)) return;
+    const uint32_t part = me.part, team = me.team;
     const uint32_t b = team / tiles_per_batch, ct = team - b * tiles_per_batch;
     const int32_t col0 = ct * T::COLS + (tid % LPR) * 8;
     const int32_t own0 = part * T::ROWS;
@@ -396,11 +398,11 @@ static int softmax_dispatch(int32_t batch, int32_t n, int32_t m, const void* inp
                         break;
                     }
                     if (rc != 0) return rc == kXchFull ? CPMK_ETOOBIG : rc;
-                    const dim3 grid((unsigned)(tiles * nb * parts));
+                    const dim3 grid((unsigned)xch_team_grid(tiles * nb, parts));
                     const half_t* xb = x + b0 * n * m;
                     half_t* yb = y + b0 * n * m;
                     hipLaunchKernelGGL((k_softmax_team<1024, 8>), grid, dim3(1024), 0, st, n, m, (int32_t)tiles,
-                                       (int32_t)parts, xb, yb, xs.xl);
+                                       (int32_t)parts, xb, yb, (uint32_t)(tiles * nb), xs.xl);
                     const int e = launch_status();
                     const int rc2 = xs.end();
                     if (e != 0 || rc2 != 0) return e ? e : rc2;

@@ -265,7 +265,7 @@ __global__ __launch_bounds__(256) void k_col(ColArgs p) {
 constexpr int kColTeamMaxParts = 32;
 
 template <int KIND>
-__global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_batch, int32_t parts, XchLaunch xl) {
+__global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_batch, int32_t parts, uint32_t nteams, XchLaunch xl) {
     uint64_t* const xch = xl.region;
     const uint32_t tag = xl.tag;
     constexpr int NT = 512, LPR = 8, R = 8;
@@ -276,7 +276,9 @@ __global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_b
     __shared__ float lds[(T::NW + 1) * T::COLS * NV];
     __shared__ float tot[T::COLS * 2];
     const int tid = threadIdx.x, cg = tid % LPR, rg = tid / LPR;
-    const uint32_t part = blockIdx.x % parts, team = blockIdx.x / parts;
+    XchMember me;
+    if (!xch_member(blockIdx.x, parts, nteams, me)) return;
+    const uint32_t part = me.part, team = me.team;
     const uint32_t b = team / tiles_per_batch, ct = team - b * tiles_per_batch;
     const int32_t col0 = ct * T::COLS + cg * 8;
     const int32_t own0 = part * T::ROWS;
@@ -485,12 +487,14 @@ __global__ __launch_bounds__(256) void k_position_backward_team(int32_t query_le
                                                                 int32_t max_distance, const int32_t* __restrict__ mapping,
                                                                 const half_t* __restrict__ grad_out, half_t* __restrict__ grad,
                                                                 int bidirectional, int32_t parts, int32_t rows_per_part,
-                                                                XchLaunch xl) {
+                                                                uint32_t nteams, XchLaunch xl) {
     uint64_t* const xch = xl.region;
     const uint32_t tag = xl.tag;
     extern __shared__ float hist[];                       // num_buckets floats, then max_distance bucket numbers
     int32_t* lmap = reinterpret_cast<int32_t*>(hist + num_buckets);
-    const uint32_t part = blockIdx.x % parts, h = blockIdx.x / parts;
+    XchMember me;                                          // a head's parts are a team
+    if (!xch_member(blockIdx.x, parts, nteams, me)) return;
+    const uint32_t part = me.part, h = me.team;
     const int tid = threadIdx.x;
     for (int i = tid; i < num_buckets; i += 256) hist[i] = 0.0f;
     for (int i = tid; i < max_distance; i += 256) lmap[i] = mapping[i];
@@ -654,7 +658,7 @@ static int launch_col(int32_t batch, const ColArgs& p, void* stream, bool missin
                       parts <= kColTeamMaxParts && tiles * parts <= kXchSlots;
     if (wide) {
         // teams use one packet slot per (team, part): batches beyond the pool go out in several launches
-        const int64_t per_launch = parts > 1 ? kXchSlots / (tiles * parts) : ((1ll << 31) - 1) / (tiles * parts);
+        const int64_t per_launch = parts > 1 ? kXchSlots / (tiles * parts) : ((1ll << 31) - 8) / (tiles * parts);
         bool no_slots = false;
         for (int64_t b0 = 0; b0 < batch; b0 += per_launch) {
             const int64_t nb = batch - b0 < per_launch ? batch - b0 : per_launch;
@@ -668,8 +672,8 @@ static int launch_col(int32_t batch, const ColArgs& p, void* stream, bool missin
                 }
                 if (rc != 0) return rc == kXchFull ? CPMK_ETOOBIG : rc;
             }
-            hipLaunchKernelGGL((k_col_team<KIND>), dim3((unsigned)(tiles * nb * parts)), dim3(512), 0, (hipStream_t)stream, q,
-                               (int32_t)tiles, (int32_t)parts, xs.xl);
+            hipLaunchKernelGGL((k_col_team<KIND>), dim3((unsigned)xch_team_grid(tiles * nb, parts)), dim3(512), 0, (hipStream_t)stream, q,
+                               (int32_t)tiles, (int32_t)parts, (uint32_t)(tiles * nb), xs.xl);
             const int e = launch_status();
             const int rc2 = xs.end();
             if (e != 0 || rc2 != 0) return e ? e : rc2;
@@ -863,10 +867,10 @@ int cpmk_position_embedding_backward(int32_t query_len, int32_t key_len, int32_t
             const int rc = xs.begin((int64_t)num_heads * parts, (hipStream_t)stream);
             if (rc != 0 && rc != kXchFull) return rc;
             if (rc == 0) {      // (kXchFull: recorded into a graph and the capture reserve is used up: the kernel without packets below)
-                hipLaunchKernelGGL(k_position_backward_team, dim3((unsigned)(num_heads * parts)), dim3(256),
+                hipLaunchKernelGGL(k_position_backward_team, dim3((unsigned)xch_team_grid(num_heads, parts)), dim3(256),
                                    num_buckets * sizeof(float) + max_distance * sizeof(int32_t), (hipStream_t)stream, query_len, key_len,
                                    num_buckets, max_distance, (const int32_t*)position_mapping, (const half_t*)grad_out, (half_t*)grad,
-                                   bidirectional, (int32_t)parts, (int32_t)rpp, xs.xl);
+                                   bidirectional, (int32_t)parts, (int32_t)rpp, (uint32_t)num_heads, xs.xl);
                 const int e = launch_status();
                 const int rc2 = xs.end();
                 return e ? e : rc2;
