@@ -162,9 +162,17 @@ int XchScope::begin(int64_t slots, hipStream_t st) {
                 const hipError_t e = hipStreamWaitEvent(st, h.done, 0);
                 if (e != hipSuccess) return (int)e;
             }
+        // The new holder takes over what it overlaps.  Slots go out in rising order, so an earlier holder's range
+        // never starts below `first` unless it ends there too: what is left of a range that is only partly
+        // covered is its upper end, which stays on record with its event for whoever is given those slots next.
         for (size_t i = 0; i < d->held.size();) {
             Held& h = d->held[i];
             if (h.first < last && first < h.last) {
+                if (h.last > last && h.first >= first) {
+                    h.first = last;
+                    ++i;
+                    continue;
+                }
                 d->spare.push_back(h.done);
                 d->held[i] = d->held.back();
                 d->held.pop_back();
