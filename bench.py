@@ -599,6 +599,7 @@ def main():
         cl.ceil_read.argtypes = [VP, I64, VP, ctypes.c_int, VP]
         cl.ceil_read_span.argtypes = [VP, I32, VP, VP, VP]
         cl.ceil_empty.argtypes = [I32, I32, VP, VP]
+        cl.ceil_xcc_ids.argtypes = [VP, I32, I32, VP]
         cl.ceil_write.argtypes = [VP, I64, VP]
         cl.ceil_copy.argtypes = [VP, VP, I64, ctypes.c_int, VP]
         cl.ceil_copy_segments.argtypes = [VP, VP, I64, I32, I32, ctypes.c_int, VP]
@@ -665,6 +666,16 @@ def main():
         ms, how = graph_ms([(lambda i=i: dst_ln.copy_(srcs[i])) for i in range(10)], 60)
         ceil["runtime_memcpy_d2d_33.5MB"] = dict(gbs(2 * ln_bytes, ms), timing=how)
         del srcs, dst_ln
+        # the premise of the team kernels' layout (a team = workgroups 8s + x of one launch for consecutive s): workgroup i
+        # runs on XCD (i + k) % 8 with one k for the whole launch
+        ids = torch.full((2048,), -1, dtype=torch.int32, device=dev)
+        ok(cl.ceil_xcc_ids(ids.data_ptr(), 2048, 1024, st()))
+        torch.cuda.synchronize()
+        idl = ids.cpu().tolist()
+        off = idl[0] % 8
+        ceil["workgroup_to_xcd"] = {"xcds_seen": sorted(set(idl)), "first_workgroups": idl[:16], "k": off,
+                                    "workgroup_i_runs_on_xcd_(i+k)_mod_8": all(x == (i + off) % 8 for i, x in enumerate(idl)),
+                                    "launch": "2048 workgroups of 1024 threads, XCC_ID read by each"}
         # what one kernel launch costs between two others: a kernel that does nothing, in a graph like the per-kernel legs'
         ms, how = graph_ms([lambda: ok(cl.ceil_empty(256, 512, sink.data_ptr(), st()))], 640)
         ceil["empty_kernel (what a launch costs in the per-kernel legs)"] = {"us": round(ms * 1e3, 2), "timing": how}

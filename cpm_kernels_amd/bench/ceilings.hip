@@ -17,6 +17,7 @@
 //                       their start and end with the 100 MHz wall clock: last end - first start is the time the
 //                       memory system needs for those bytes, without what a kernel launch costs around it
 //   ceil_empty          a kernel that does nothing: what one launch costs between two others
+//   ceil_xcc_ids        which XCD each workgroup of a launch runs on
 //   ceil_copy_segments  a (rows, row_bytes) matrix copied in tiles of `seg` bytes x many rows, one
 //                       tile per 1024-thread workgroup, all loads of a tile before its stores: the
 //                       access pattern of the dim-1 kernels (layernorm, softmax) without arithmetic
@@ -105,6 +106,13 @@ __global__ __launch_bounds__(256) void k_read(const int4_t* __restrict__ p, int6
 
 __global__ void k_empty(int4_t* sink) {
     if (threadIdx.x == 0x7fffffff) sink[0] = int4_t{1, 2, 3, 4};      // never
+}
+
+// out[b] = the XCC (XCD) that workgroup b of the launch runs on, as the hardware register says
+__global__ void k_xcc_ids(int32_t* out) {
+    uint32_t xcc;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+    if (threadIdx.x == 0) out[blockIdx.x] = (int32_t)(xcc & 15u);
 }
 
 // 512 threads, NLD pieces of 16 bytes per thread: a share of NLD * 8 KB per workgroup; stamps[2b], [2b+1] = start, end of workgroup b
@@ -252,6 +260,13 @@ int ceil_read_span(const void* src, int32_t workgroups, void* sink, void* stamps
     if (workgroups < 1) return 1;
     hipLaunchKernelGGL(k_read_span<20>, dim3((unsigned)workgroups), dim3(512), 0, (hipStream_t)stream, (const char*)src, (int4_t*)sink,
                        (unsigned long long*)stamps);
+    return status();
+}
+
+// the XCD of each of `workgroups` workgroups of one launch (int32 each)
+int ceil_xcc_ids(void* out, int32_t workgroups, int32_t threads, void* stream) {
+    if (workgroups < 1 || threads < 1 || threads > 1024) return 1;
+    hipLaunchKernelGGL(k_xcc_ids, dim3((unsigned)workgroups), dim3((unsigned)threads), 0, (hipStream_t)stream, (int32_t*)out);
     return status();
 }
 

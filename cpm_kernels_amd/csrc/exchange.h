@@ -187,7 +187,7 @@ __device__ inline bool xch_gather2(const uint64_t* team_slots, int parts, int q0
 }
 
 // Which team a workgroup belongs to.  The hardware deals the workgroups of a launch out to the chip's 8 XCDs
-// round robin (workgroup i runs on XCD i % 8), and every XCD starts its share on its own, in index order, as its
+// round robin (workgroup i runs on XCD (i + k) % 8, k the same for the whole launch), and every XCD starts its share on its own, in index order, as its
 // compute units become free: nothing orders the XCDs among each other.  A team therefore consists of workgroups of
 // ONE XCD that follow one another in that XCD's order -- workgroups 8s + x for `parts` consecutive s -- so a
 // member only ever waits for members that the same XCD starts next, whatever other launches keep the other XCDs
