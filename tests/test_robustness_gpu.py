@@ -151,7 +151,7 @@ def test_results_do_not_depend_on_timing(gpu):
 
 
 def test_team_launches_overlapping_on_eight_streams(gpu):
-    """Team kernels of different kinds queued on eight streams at once, three rounds of them: each
+    """Team kernels of different kinds queued on eight streams at once, nine rounds of them: each
     launch gets packet slots of its own, so every result equals the single-stream result bit for
     bit and no wait runs out.  The reference's kernels keep no state between launches
     (cuda/layernorm.cu:6-71, cuda/softmax.cu:6-43), so callers may overlap them freely."""
@@ -183,7 +183,7 @@ def test_team_launches_overlapping_on_eight_streams(gpu):
     ref = [one(0, xs[i], tall[i], s0) for i in range(8)]
     torch.cuda.synchronize()
     streams = [torch.cuda.Stream() for _ in range(8)]
-    for rnd in range(3):
+    for rnd in range(9):
         got = []
         for i, st in enumerate(streams):
             with torch.cuda.stream(st):
