@@ -600,6 +600,7 @@ def main():
         cl.ceil_read_span.argtypes = [VP, I32, VP, VP, VP]
         cl.ceil_empty.argtypes = [I32, I32, VP, VP]
         cl.ceil_xcc_ids.argtypes = [VP, I32, I32, VP]
+        cl.ceil_read_gemv_pattern.argtypes = [VP, VP, ctypes.c_int, VP, VP, VP]
         cl.ceil_write.argtypes = [VP, I64, VP]
         cl.ceil_copy.argtypes = [VP, VP, I64, ctypes.c_int, VP]
         cl.ceil_copy_segments.argtypes = [VP, VP, I64, I32, I32, ctypes.c_int, VP]
@@ -698,6 +699,21 @@ def main():
                                                                in_kernel_span_frac_of_published_peak=round(piece / (span_us * 1e-6) / 1e9 / PEAK_HBM_GBS, 4),
                                                                note="span = last workgroup's end - first workgroup's start (wall clock stamps inside the kernel); the rest of "
                                                                     "the per-launch time is what a launch costs (see empty_kernel)")
+        # the decode GEMV's own loads without its arithmetic: the matrix in the MFMA operand layout (an instruction touches 64 bytes of
+        # 16 rows), alone and with the 128 KB of vectors that every workgroup reads alike; span and per-launch time as above
+        vecs = big2[:128 << 10]
+        for label, vp_, nt_ in (("matrix_only_nontemporal", None, 1), ("matrix_only_plain_loads", None, 0), ("with_the_vectors_nontemporal", vecs.data_ptr(), 1),
+                                ("with_the_vectors_plain_loads", vecs.data_ptr(), 0)):
+            for _ in range(3):
+                for i in range(8):
+                    ok(cl.ceil_read_gemv_pattern(big.data_ptr() + i * (128 << 20), vp_, nt_, sink.data_ptr(), stamps[i].data_ptr(), st()))
+            torch.cuda.synchronize()
+            sp = stamps.cpu().view(8, 256, 2)
+            span_us = float(((sp[:, :, 1].max(dim=1).values - sp[:, :, 0].min(dim=1).values).double().mean()) * 0.01)
+            ms, how = graph_ms([(lambda i=i: ok(cl.ceil_read_gemv_pattern(big.data_ptr() + i * (128 << 20), vp_, nt_, sink.data_ptr(), stamps[i].data_ptr(), st())))
+                                for i in range(8)], 80)
+            ceil["cold_read_42MB_gemv_access_pattern_" + label] = dict(gbs(piece, ms), timing=how, in_kernel_span_us=round(span_us, 2))
+        del vecs
         # the layernorm's traffic and pattern: [8*4096 rows, 1024 bytes] in 128-byte (and wider) column segments, ten buffers in turn
         for seg, nt_ in ((128, 0), (128, 1), (256, 1), (1024, 1)):
             ms, how = graph_ms([(lambda i=i: ok(cl.ceil_copy_segments(big.data_ptr() + i * (64 << 20), big2.data_ptr(), 8 * 4096, 1024, seg, nt_, st())))

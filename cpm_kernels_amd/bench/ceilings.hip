@@ -18,6 +18,7 @@
 //                       memory system needs for those bytes, without what a kernel launch costs around it
 //   ceil_empty          a kernel that does nothing: what one launch costs between two others
 //   ceil_xcc_ids        which XCD each workgroup of a launch runs on
+//   ceil_read_gemv_pattern  the decode GEMV's loads (matrix in the MFMA operand layout, the vectors every workgroup reads) without its arithmetic
 //   ceil_copy_segments  a (rows, row_bytes) matrix copied in tiles of `seg` bytes x many rows, one
 //                       tile per 1024-thread workgroup, all loads of a tile before its stores: the
 //                       access pattern of the dim-1 kernels (layernorm, softmax) without arithmetic
@@ -126,6 +127,48 @@ __global__ __launch_bounds__(512) void k_read_span(const char* __restrict__ src,
     int4_t a = {0, 0, 0, 0};
 #pragma unroll
     for (int i = 0; i < NLD; ++i) a += v[i];
+    if (a.x == 0x12345678 && a.y == 1) sink[0] = a;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        stamps[2 * blockIdx.x] = t0;
+        stamps[2 * blockIdx.x + 1] = wall_clock64();
+    }
+}
+
+// The decode GEMV's memory traffic without its arithmetic: 40 rows of 4096 bytes per workgroup, wave w bytes
+// [512w, 512w + 512) of every row, lane (r, q) 16 bytes of row 16g + r -- the MFMA operand layout, in which an
+// instruction touches 64 bytes of 16 rows -- and, if VEC, the 128 KB every workgroup reads alike (32 vectors),
+// requested behind the first 16 rows like the kernel does.  NTL: non-temporal matrix loads.  Stamps as k_read_span.
+template <int VEC, int NTL>
+__global__ __launch_bounds__(512) void k_read_gemv_pattern(const char* __restrict__ mat, const char* __restrict__ vec, int4_t* sink,
+                                                           unsigned long long* stamps) {
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, r = lane & 15, q = lane >> 4;
+    const unsigned long long t0 = wall_clock64();
+    const int row0 = blockIdx.x * 40;
+    int4_t v[3][8], u[VEC ? 16 : 1];
+    auto rows = [&](int g) __attribute__((always_inline)) {
+        const int row = row0 + min(g * 16 + r, 39);
+        const char* rp = mat + (uint32_t)row * 4096u + w * 512 + q * 16;
+#pragma unroll
+        for (int kb = 0; kb < 8; ++kb)
+            v[g][kb] = NTL ? __builtin_nontemporal_load(reinterpret_cast<const int4_t*>(rp + kb * 64)) : *reinterpret_cast<const int4_t*>(rp + kb * 64);
+    };
+    rows(0);
+    if (VEC) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) u[i] = *reinterpret_cast<const int4_t*>(vec + ((int64_t)i * 512 + tid) * 16);
+    }
+    rows(1);
+    rows(2);
+    int4_t a = {0, 0, 0, 0};
+#pragma unroll
+    for (int g = 0; g < 3; ++g)
+#pragma unroll
+        for (int kb = 0; kb < 8; ++kb) a += v[g][kb];
+    if (VEC) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) a += u[i];
+    }
     if (a.x == 0x12345678 && a.y == 1) sink[0] = a;
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -267,6 +310,20 @@ int ceil_read_span(const void* src, int32_t workgroups, void* sink, void* stamps
 int ceil_xcc_ids(void* out, int32_t workgroups, int32_t threads, void* stream) {
     if (workgroups < 1 || threads < 1 || threads > 1024) return 1;
     hipLaunchKernelGGL(k_xcc_ids, dim3((unsigned)workgroups), dim3((unsigned)threads), 0, (hipStream_t)stream, (int32_t*)out);
+    return status();
+}
+
+// 256 workgroups x 40 rows of 4096 bytes from src in the GEMV's access pattern; vec: 128 KB that every workgroup reads (or null)
+int ceil_read_gemv_pattern(const void* src, const void* vec, int nontemporal, void* sink, void* stamps, void* stream) {
+    const dim3 g(256), b(512);
+    hipStream_t st = (hipStream_t)stream;
+    if (vec != nullptr) {
+        if (nontemporal) hipLaunchKernelGGL((k_read_gemv_pattern<1, 1>), g, b, 0, st, (const char*)src, (const char*)vec, (int4_t*)sink, (unsigned long long*)stamps);
+        else hipLaunchKernelGGL((k_read_gemv_pattern<1, 0>), g, b, 0, st, (const char*)src, (const char*)vec, (int4_t*)sink, (unsigned long long*)stamps);
+    } else {
+        if (nontemporal) hipLaunchKernelGGL((k_read_gemv_pattern<0, 1>), g, b, 0, st, (const char*)src, (const char*)vec, (int4_t*)sink, (unsigned long long*)stamps);
+        else hipLaunchKernelGGL((k_read_gemv_pattern<0, 0>), g, b, 0, st, (const char*)src, (const char*)vec, (int4_t*)sink, (unsigned long long*)stamps);
+    }
     return status();
 }
 
