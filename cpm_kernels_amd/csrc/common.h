@@ -51,6 +51,19 @@ __device__ inline int32_t wave_sum_i32(int32_t v) {
     return v;
 }
 
+// Sum over the wave with data-parallel-primitive operands instead of cross-lane reads through the LDS crossbar:
+// six additions whose second operand comes from another lane (quad swaps, mirrors within 8 and 16 lanes, then the
+// last lane of a row of 16 broadcast to the next row, and lane 31 to the upper half).  The total is in LANE 63 only.
+__device__ inline int32_t wave_sum_i32_to_lane63(int32_t v) {
+    v += __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xf, 0xf, true);      // quad_perm [1,0,3,2]
+    v += __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xf, 0xf, true);      // quad_perm [2,3,0,1]
+    v += __builtin_amdgcn_update_dpp(0, v, 0x141, 0xf, 0xf, true);     // row_half_mirror
+    v += __builtin_amdgcn_update_dpp(0, v, 0x140, 0xf, 0xf, true);     // row_mirror
+    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);    // row_bcast15 into rows 1 and 3
+    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);    // row_bcast31 into rows 2 and 3
+    return v;
+}
+
 // Block-wide reductions for blocks of NWAVES*64 threads.  `red` is LDS scratch of at least
 // NWAVES floats.  Every thread returns the reduced value.  Contains two barriers so the
 // scratch can be reused by the next call.

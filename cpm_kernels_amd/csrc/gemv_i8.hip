@@ -396,6 +396,74 @@ __global__ __launch_bounds__(512) void k_gemv_direct(int32_t batch, int32_t dim_
     }
 }
 
+// One or two vectors (decode with a batch of one or two sequences): no matrix cores.  A wave reads whole rows --
+// instruction i of a row brings bytes [1024 i, 1024 i + 1024), 16 per lane, whole cache lines in address order,
+// the access pattern in which a one-round read of this size is 2 us quicker than in the MFMA operand layout of
+// the kernel above -- and multiplies them with v_dot4_i32_i8 against the vectors' bytes at the same positions,
+// which every lane keeps in registers (NV x PPL pieces of 16 bytes).  One workgroup per compute unit, wave w
+// takes rows w, w + 8, ... of the workgroup's share (G of them), all loads of a wave requested at once (G rows of
+// PPL pieces, at most 20 pieces = 80 registers); the per-lane sums of a (row, vector) pair are added over the wave,
+// and the outputs leave through LDS so that a vector's outputs are stored contiguously.
+template <int NV, int PPL, int G>
+__global__ __launch_bounds__(512) void k_gemv_rowwise(int32_t batch, int32_t dim_out, int32_t rpb,
+                                                      const half_t* __restrict__ scale_mat,
+                                                      const int8_t* __restrict__ mat,
+                                                      const half_t* __restrict__ scale_vec,
+                                                      const int8_t* __restrict__ vec,
+                                                      half_t* __restrict__ out) {
+    static_assert(G * PPL <= 20 && NV * PPL <= 20, "registers");
+    constexpr int DIN = PPL * 1024;
+    __shared__ int32_t part[8 * G * NV];           // [row of the share][vector]
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int32_t row0 = blockIdx.x * rpb;
+    int4_t wf[G][PPL];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        const int32_t row = min(row0 + min(g * 8 + w, rpb - 1), dim_out - 1);       // (rows past the share repeat its last row)
+        const int8_t* rp = mat + (uint32_t)row * (uint32_t)DIN + lane * 16;
+#pragma unroll
+        for (int i = 0; i < PPL; ++i) wf[g][i] = __builtin_nontemporal_load(reinterpret_cast<const int4_t*>(rp + i * 1024));
+    }
+    int4_t vf[NV][PPL];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int8_t* vp = vec + (uint32_t)min(v, batch - 1) * (uint32_t)DIN + lane * 16;
+#pragma unroll
+        for (int i = 0; i < PPL; ++i) vf[v][i] = *reinterpret_cast<const int4_t*>(vp + i * 1024);
+    }
+    // the outputs this thread will write and their scales (row fastest: a vector's outputs are contiguous)
+    const int nout = rpb * NV;
+    const int obb = tid / rpb, orr = tid - obb * rpb;
+    half_t osv = (half_t)0.0f, osm = (half_t)0.0f;
+    if (tid < nout) {
+        osv = scale_vec[min(obb, batch - 1)];
+        osm = scale_mat[min(row0 + orr, dim_out - 1)];
+    }
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        int32_t acc[NV];
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            acc[v] = 0;
+#pragma unroll
+            for (int i = 0; i < PPL; ++i)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[v] = __builtin_amdgcn_sdot4(wf[g][i][e], vf[v][i][e], acc[v], false);
+        }
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int32_t t = wave_sum_i32_to_lane63(acc[v]);
+            if (lane == 63) part[(g * 8 + w) * NV + v] = t;
+        }
+    }
+    __syncthreads();
+    if (tid < nout) {
+        const int32_t row = row0 + orr;
+        if (row < dim_out && obb < batch) out[(int64_t)obb * dim_out + row] = dequant(part[orr * NV + obb], (float)osv, (float)osm);
+    }
+}
+
 // Generic path (any dim_in % 4 == 0, any alignment): one wave per matrix row, dword loads,
 // v_dot4_i32_i8, up to 8 vectors per pass so the row is read from HBM once per 8 vectors.
 __global__ __launch_bounds__(256) void k_gemv_dot4(int32_t batch, int32_t dim_out, int32_t dim_in,
@@ -480,6 +548,46 @@ static bool launch_gemv_direct(int32_t batch, int32_t dim_out, int32_t dim_in, c
     return true;
 }
 
+// The row-wise kernel for one or two vectors: rows of 4 KB (up to 40 per compute unit) or 10 KB (up to 16 per
+// compute unit) -- the row lengths of the model this path serves; at least two rows per wave, below that the
+// matrix-core kernels are as quick.  ([10240, 4096] at one / two vectors: 7.8 / 8.5 us against 9.6 / 9.8 on the
+// matrix cores; with three or four vectors the dot products and their sums over the wave cost what the access
+// pattern saves.)
+static bool launch_gemv_rowwise(int32_t batch, int32_t dim_out, int32_t dim_in, const half_t* sm, const int8_t* mat,
+                                const half_t* sv, const int8_t* vec, half_t* out, hipStream_t st) {
+    if (batch > 2 || (dim_in != 4096 && dim_in != 10240) || (int64_t)dim_out * dim_in >= (1ll << 32)) return false;
+    const int nv = batch;
+    const int64_t rpb = ceil_div(dim_out, compute_units());
+    const int g = (int)ceil_div(rpb, 8);
+    const dim3 grid((unsigned)ceil_div(dim_out, rpb));
+    auto go = [&](auto kern) { hipLaunchKernelGGL(kern, grid, dim3(512), 0, st, batch, dim_out, (int32_t)rpb, sm, mat, sv, vec, out); };
+    auto pick = [&](auto nvc, auto pplc) {
+        constexpr int NV = decltype(nvc)::value, PPL = decltype(pplc)::value;
+        if constexpr (PPL == 4) {
+            if (g == 2) go(k_gemv_rowwise<NV, 4, 2>);
+            else if (g == 3) go(k_gemv_rowwise<NV, 4, 3>);
+            else if (g == 4) go(k_gemv_rowwise<NV, 4, 4>);
+            else go(k_gemv_rowwise<NV, 4, 5>);
+        } else {
+            go(k_gemv_rowwise<NV, 10, 2>);
+        }
+    };
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    using I4 = std::integral_constant<int, 4>;
+    if (dim_in == 4096 && g >= 2 && g <= 5) {
+        if (nv == 1) pick(I1{}, I4{});
+        else pick(I2{}, I4{});
+        return true;
+    }
+    if (dim_in == 10240 && g == 2) {
+        if (nv == 1) pick(I1{}, std::integral_constant<int, 10>{});
+        else pick(I2{}, std::integral_constant<int, 10>{});
+        return true;
+    }
+    return false;
+}
+
 template <int NB>
 static void launch_mfma(int32_t batch, int32_t dim_out, int32_t dim_in, const half_t* sm, const int8_t* mat,
                         const half_t* sv, const int8_t* vec, half_t* out, hipStream_t st) {
@@ -546,7 +654,8 @@ extern "C" int cpmk_gemv_broadcast_mat_int8(int32_t batch, int32_t dim_out, int3
         half_t* o = O + (int64_t)b0 * dim_out;
         const half_t* s = sv + b0;
         int derr = 0;
-        if (nb <= 16 ? launch_gemv_direct<1>(nb, dim_out, dim_in, sm, M, s, v, o, st, &derr)
+        if (launch_gemv_rowwise(nb, dim_out, dim_in, sm, M, s, v, o, st)) {
+        } else if (nb <= 16 ? launch_gemv_direct<1>(nb, dim_out, dim_in, sm, M, s, v, o, st, &derr)
                      : (nb <= 32 && launch_gemv_direct<2>(nb, dim_out, dim_in, sm, M, s, v, o, st, &derr))) {
             if (derr) return derr;
         } else if (dim_in % 256 == 0 && (int64_t)dim_out * dim_in < (1ll << 32) && (int64_t)nb * dim_in < (1ll << 32)) {

@@ -490,7 +490,11 @@ def test_north_star_fused_pipeline_bits(gpu):
                                                   (32, 4096, 8192), (5, 3333, 8192), (16, 100, 8192),
                                                   (32, 10240, 2048), (20, 7000, 2048), (3, 513, 2048), (32, 4096, 2048),
                                                   # and with more rows than one workgroup per compute unit holds
-                                                  (32, 5000, 10240), (32, 12500, 2048)])
+                                                  (32, 5000, 10240), (32, 12500, 2048),
+                                                  # one to four vectors (the row-wise kernel): rows of 4 KB at 40, 40 ragged, 20, 17 and 12 rows per
+                                                  # workgroup, rows of 10 KB at 16 rows (one and two vectors; three go to the chunked kernel)
+                                                  (1, 10240, 4096), (2, 10240, 4096), (4, 10239, 4096), (1, 5000, 4096), (2, 4097, 4096), (4, 3000, 4096),
+                                                  (3, 10240, 4096), (2, 4096, 10240), (1, 4001, 10240), (3, 4096, 10240)])
 def test_gemv_broadcast_mat_int8(gpu, batch, dim_out, dim_in):
     _name("gemv", batch, dim_out, dim_in)
     rng = np.random.default_rng(1002 + dim_out)
