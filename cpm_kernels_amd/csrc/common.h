@@ -64,6 +64,17 @@ __device__ inline int32_t wave_sum_i32_to_lane63(int32_t v) {
     return v;
 }
 
+// The same for an unsigned maximum, handed to every lane (as a wave-uniform value).
+__device__ inline uint32_t wave_max_u32_uniform(uint32_t v) {
+    v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xf, 0xf, true));
+    v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xf, 0xf, true));
+    v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x141, 0xf, 0xf, true));
+    v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x140, 0xf, 0xf, true));
+    v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x142, 0xa, 0xf, false));
+    v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x143, 0xc, 0xf, false));
+    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
+}
+
 // Block-wide reductions for blocks of NWAVES*64 threads.  `red` is LDS scratch of at least
 // NWAVES floats.  Every thread returns the reduced value.  Contains two barriers so the
 // scratch can be reused by the next call.

@@ -233,7 +233,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NV <= 8 ? 8
         ushort8_t um = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
         for (int i = 0; i < NV; ++i) um = absbits_max(um, cur[i]);
-        const uint32_t ub = wave_max_u32(absbits_max_of(um));
+        const uint32_t ub = wave_max_u32_uniform(absbits_max_of(um));
         float mx = (float)__builtin_bit_cast(half_t, (uint16_t)ub);
         if (ub > 0x7c00u) {      // (the same for the whole wave) a NaN in the row: the maximum that skips NaN elements
             half8_t hm;
