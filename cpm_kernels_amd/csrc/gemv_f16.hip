@@ -9,6 +9,11 @@
 
 namespace cpmk {
 
+constexpr int kShortLoads = 4;        // k_gemv_f16_short: loads in flight per lane when the grid still fills the chip
+constexpr int kShortMinGroups = 2048; // ... which it does from eight workgroups a compute unit on
+constexpr int kTransposeLoads = 8;    // k_gemv_f16_transpose: rows requested per lane before the first is used
+
+
 // One wave per (batch, row): 16-byte loads of the row and of the vector, wave reduction.
 // mat_bstride = 0 shares the matrix over the batch (then the rows of all vectors are done by one
 // wave, so the matrix is still read once).
@@ -54,34 +59,48 @@ __global__ __launch_bounds__(256) void k_gemv_f16_rows(int32_t batch, int32_t di
 }
 
 // Short rows (dim_in <= 256, the head dimension of attention scores over a key cache): LPRK lanes
-// per row, one 16-byte piece each, so a wave covers 64 / LPRK consecutive rows with one coalesced
-// load; the row sums are finished with LPRK-wide butterfly shuffles.  item = b * dim_out + row.
-template <int LPRK>
+// per row, one 16-byte piece each (LPRK >= dim_in / 8), so a wave covers 64 / LPRK consecutive rows
+// with one coalesced load, and U such loads (U * 1 KB of consecutive rows) are in flight per wave
+// before the first is used; the row sums are finished with LPRK-wide butterfly shuffles.  The matrix
+// is read once and bypasses the caches' retention; the vectors are shared by dim_out rows and stay.
+// item = b * dim_out + row.
+template <int LPRK, int U>
 __global__ __launch_bounds__(256) void k_gemv_f16_short(int64_t items, int32_t dim_out, int32_t dim_in,
                                                         const half_t* __restrict__ mat, const half_t* __restrict__ vec,
                                                         half_t* __restrict__ out) {
     constexpr int RPW = 64 / LPRK;
     const int lane = threadIdx.x & 63, pl = lane % LPRK;
-    const int64_t item = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * RPW + lane / LPRK;
-    const bool live = item < items;
-    const int64_t it = live ? item : items - 1;
-    const int64_t b = it / dim_out;
-    const half_t* mrow = mat + it * dim_in;
-    const half_t* v = vec + b * dim_in;
-    float acc = 0.0f;
-    for (int32_t i = pl; i < (dim_in >> 3); i += LPRK) {
-        const half8_t w = reinterpret_cast<const half8_t*>(mrow)[i];
-        const half8_t x = reinterpret_cast<const half8_t*>(v)[i];
+    const int64_t item0 = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * (U * RPW) + lane / LPRK;
+    const bool used = pl < (dim_in >> 3);
+    half8_t w[U], x[U];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) acc = __builtin_fmaf((float)w[e], (float)x[e], acc);
+    for (int u = 0; u < U; ++u) {
+        const int64_t item = item0 + u * RPW;
+        const int64_t it = item < items ? item : items - 1;
+        const int64_t b = it / dim_out;
+        if (used) {
+            w[u] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(mat + it * dim_in) + pl);
+            x[u] = reinterpret_cast<const half8_t*>(vec + b * dim_in)[pl];
+        }
     }
 #pragma unroll
-    for (int o = 1; o < LPRK; o <<= 1) acc += __shfl_xor(acc, o, kWave);
-    if (live && pl == 0) out[item] = (half_t)acc;
+    for (int u = 0; u < U; ++u) {
+        const int64_t item = item0 + u * RPW;
+        float acc = 0.0f;
+        if (used) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc = __builtin_fmaf((float)w[u][e], (float)x[u][e], acc);
+        }
+#pragma unroll
+        for (int o = 1; o < LPRK; o <<= 1) acc += __shfl_xor(acc, o, kWave);
+        if (item < items && pl == 0) out[item] = (half_t)acc;
+    }
 }
 
 // mat (batch, dim_in, dim_out): 256 threads = 32 row groups x 8 lanes of 8 adjacent columns; the
-// row groups stride over dim_in and are combined in LDS.  gridDim = (ceil(dim_out/64), batch).
+// row groups stride over dim_in and are combined in LDS.  A lane requests kTransposeLoads rows before it
+// uses the first (the sums still run in row order); the matrix is read once and bypasses the caches'
+// retention.  gridDim = (ceil(dim_out/64), batch).
 __global__ __launch_bounds__(256) void k_gemv_f16_transpose(int32_t dim_out, int32_t dim_in, const half_t* __restrict__ mat,
                                                             const half_t* __restrict__ vec, half_t* __restrict__ out,
                                                             int vec8) {
@@ -94,15 +113,33 @@ __global__ __launch_bounds__(256) void k_gemv_f16_transpose(int32_t dim_out, int
     float acc[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
-    for (int32_t i = rg; i < dim_in; i += 32) {
-        const float x = (float)v[i];
-        if (vec8) {
-            if (col0 < dim_out) {
-                const half8_t w = *reinterpret_cast<const half8_t*>(base + (int64_t)i * dim_out + col0);
+    if (vec8) {
+        if (col0 < dim_out) {
+            const half_t* col = base + col0;
+            int32_t i = rg;
+            for (; i + 32 * (kTransposeLoads - 1) < dim_in; i += 32 * kTransposeLoads) {
+                half8_t w[kTransposeLoads];
+                float x[kTransposeLoads];
+#pragma unroll
+                for (int u = 0; u < kTransposeLoads; ++u) {
+                    w[u] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(col + (int64_t)(i + 32 * u) * dim_out));
+                    x[u] = (float)v[i + 32 * u];
+                }
+#pragma unroll
+                for (int u = 0; u < kTransposeLoads; ++u)
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(x[u], (float)w[u][e], acc[e]);
+            }
+            for (; i < dim_in; i += 32) {
+                const half8_t w = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(col + (int64_t)i * dim_out));
+                const float x = (float)v[i];
 #pragma unroll
                 for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(x, (float)w[e], acc[e]);
             }
-        } else {
+        }
+    } else {
+        for (int32_t i = rg; i < dim_in; i += 32) {
+            const float x = (float)v[i];
 #pragma unroll
             for (int e = 0; e < 8; ++e)
                 if (col0 + e < dim_out) acc[e] = __builtin_fmaf(x, (float)base[(int64_t)i * dim_out + col0 + e], acc[e]);
@@ -140,8 +177,13 @@ int cpmk_gemv_fp16(int32_t batch, int32_t dim_out, int32_t dim_in, const void* m
         const hipStream_t st = (hipStream_t)stream;
         auto go = [&](auto lc) {
             constexpr int L = decltype(lc)::value;
-            hipLaunchKernelGGL((k_gemv_f16_short<L>), dim3((unsigned)ceil_div(items, 4 * (64 / L))), dim3(256), 0, st, items, dim_out,
-                               dim_in, (const half_t*)mat, (const half_t*)vec, (half_t*)out);
+            constexpr int per_wave = 64 / L;             // rows of one load
+            if (items >= (int64_t)kShortMinGroups * 4 * kShortLoads * per_wave)     // enough rows for several workgroups a compute unit
+                hipLaunchKernelGGL((k_gemv_f16_short<L, kShortLoads>), dim3((unsigned)ceil_div(items, 4 * kShortLoads * per_wave)), dim3(256), 0, st, items,
+                                   dim_out, dim_in, (const half_t*)mat, (const half_t*)vec, (half_t*)out);
+            else
+                hipLaunchKernelGGL((k_gemv_f16_short<L, 1>), dim3((unsigned)ceil_div(items, 4 * per_wave)), dim3(256), 0, st, items, dim_out,
+                                   dim_in, (const half_t*)mat, (const half_t*)vec, (half_t*)out);
         };
         if (p <= 1) go(std::integral_constant<int, 1>{});
         else if (p <= 2) go(std::integral_constant<int, 2>{});

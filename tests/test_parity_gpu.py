@@ -1002,7 +1002,10 @@ def test_gemm_fp16(gpu, case, aT, bT):
 
 @pytest.mark.parametrize("shape", [(4, 64, 256), (3, 33, 100), (2, 1000, 4096), (1, 7, 6),
                                    # short rows (lanes share a wave's rows) and rows of whole 256-byte chunks (matrix cores)
-                                   (5, 70, 64), (2, 1000, 128), (3, 9, 8), (40, 300, 512), (33, 1100, 1024), (130, 48, 384)])
+                                   (5, 70, 64), (2, 1000, 128), (3, 9, 8), (40, 300, 512), (33, 1100, 1024), (130, 48, 384),
+                                   # short rows in numbers that put several loads in flight per lane (ragged ends, waves that
+                                   # straddle two batch entries); a transposed product whose lanes leave the unrolled loop unevenly
+                                   (301, 1021, 64), (140, 1000, 128), (520, 1024, 24), (64, 64, 1000)])
 def test_gemv_fp16_family(gpu, shape):
     _name("gemv fp16", shape)
     batch, dim_out, dim_in = shape
