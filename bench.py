@@ -557,6 +557,8 @@ def main():
         vf = torch.randn(32, 4096, generator=gg).half().to(dev); of = torch.empty((32, 10240), dtype=torch.half, device=dev)
         ms, how = graph_ms([(lambda w_=w_: ck.gemv_broadcast_mat_fp16(32, 10240, 4096, w_.data_ptr(), vf.data_ptr(), of.data_ptr(), st())) for w_ in wf], max(3, reps // 8))
         hbm("gemv_broadcast_mat_fp16", 2 * 10240 * 4096 + 2 * 32 * 4096 + 2 * 32 * 10240, ms, how, "W fp16 [10240,4096] x 32 vectors", None)
+        ms, how = graph_ms([(lambda w_=w_: ck.gemv_broadcast_mat_fp16(1, 10240, 4096, w_.data_ptr(), vf.data_ptr(), of.data_ptr(), st())) for w_ in wf], max(3, reps // 8))
+        hbm("gemv_broadcast_mat_fp16 x 1", 2 * 10240 * 4096 + 2 * 4096 + 2 * 10240, ms, how, "W fp16 [10240,4096] x 1 vector (row-wise kernel, no matrix cores)", None)
         del wf
         kc = rot((2048, 1024, 64), 2)
         qf = torch.randn(2048, 64, generator=gg).half().to(dev); sc = torch.empty((2048, 1024), dtype=torch.half, device=dev)

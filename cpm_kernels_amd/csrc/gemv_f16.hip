@@ -157,6 +157,101 @@ __global__ __launch_bounds__(256) void k_gemv_f16_transpose(int32_t dim_out, int
     }
 }
 
+// One matrix for one or two vectors (decode with a batch of one or two sequences), rows of 4096 halves: no
+// matrix cores.  One workgroup of eight waves per compute unit; wave w takes rows w, w + 8, ... of the workgroup's
+// share, R of them.  A row is eight instructions of 1 KB in address order (16 bytes a lane); the loads of up to
+// three rows are in flight per wave (192 KB a compute unit), the next row's requested before a row is used.
+// Every lane keeps the vectors' halves at its positions in registers and multiplies with v_dot2_f32_f16 (fp32
+// sums, one chain per row and vector in a fixed order, so the result does not depend on timing); the lanes' sums
+// are added over the wave, and the outputs leave through LDS so that a vector's outputs are stored contiguously.
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+
+__device__ inline float wave_sum_f32_to_lane63(float v) {
+    auto from = [](float x, auto ctrl, auto rows, auto keep) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), decltype(ctrl)::value,
+                                                                     decltype(rows)::value, 0xf, decltype(keep)::value));
+    };
+    using std::integral_constant;
+    v += from(v, integral_constant<int, 0xB1>{}, integral_constant<int, 0xf>{}, integral_constant<bool, true>{});   // quad_perm [1,0,3,2]
+    v += from(v, integral_constant<int, 0x4E>{}, integral_constant<int, 0xf>{}, integral_constant<bool, true>{});   // quad_perm [2,3,0,1]
+    v += from(v, integral_constant<int, 0x141>{}, integral_constant<int, 0xf>{}, integral_constant<bool, true>{});  // row_half_mirror
+    v += from(v, integral_constant<int, 0x140>{}, integral_constant<int, 0xf>{}, integral_constant<bool, true>{});  // row_mirror
+    v += from(v, integral_constant<int, 0x142>{}, integral_constant<int, 0xa>{}, integral_constant<bool, false>{}); // row_bcast15 into rows 1 and 3
+    v += from(v, integral_constant<int, 0x143>{}, integral_constant<int, 0xc>{}, integral_constant<bool, false>{}); // row_bcast31 into rows 2 and 3
+    return v;                                                                                                       // the total: lane 63 only
+}
+
+template <int NV, int R>
+__global__ __launch_bounds__(512) void k_gemv_f16_rowwise(int32_t batch, int32_t dim_out, int32_t rpb, const half_t* __restrict__ mat,
+                                                          const half_t* __restrict__ vec, half_t* __restrict__ out) {
+    constexpr int PPL = 8, DIN = PPL * 512, D = R < 3 ? R : 3;
+    __shared__ float part[8 * R * NV];             // [row of the share][vector]
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int32_t row0 = blockIdx.x * rpb;
+    half8_t vf[NV][PPL];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const half_t* vp = vec + (uint32_t)min(v, batch - 1) * (uint32_t)DIN + lane * 8;
+#pragma unroll
+        for (int i = 0; i < PPL; ++i) vf[v][i] = *reinterpret_cast<const half8_t*>(vp + i * 512);
+    }
+    half8_t wf[D][PPL];
+    auto request = [&](int r, half8_t (&buf)[PPL]) {
+        const int32_t row = min(row0 + min(r * 8 + w, rpb - 1), dim_out - 1);       // (rows past the share repeat its last row)
+        const half_t* rp = mat + (uint32_t)row * (uint32_t)DIN + lane * 8;
+#pragma unroll
+        for (int i = 0; i < PPL; ++i) buf[i] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(rp + i * 512));
+    };
+#pragma unroll
+    for (int r = 0; r < D - 1; ++r) request(r, wf[r]);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        if (r + D - 1 < R) request(r + D - 1, wf[(r + D - 1) % D]);
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            float acc = 0.0f;
+#pragma unroll
+            for (int i = 0; i < PPL; ++i)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const half8_t a = wf[r % D][i], b = vf[v][i];
+                    acc = __builtin_amdgcn_fdot2(half2_t{a[2 * e], a[2 * e + 1]}, half2_t{b[2 * e], b[2 * e + 1]}, acc, false);
+                }
+            const float t = wave_sum_f32_to_lane63(acc);
+            if (lane == 63) part[(r * 8 + w) * NV + v] = t;
+        }
+    }
+    __syncthreads();
+    const int obb = tid / rpb, orr = tid - obb * rpb;
+    if (tid < rpb * NV) {
+        const int32_t row = row0 + orr;
+        if (row < dim_out && obb < batch) out[(int64_t)obb * dim_out + row] = (half_t)part[orr * NV + obb];
+    }
+}
+
+// Takes the call when the shape fits the row-wise kernel: rows of 4096 halves, one or two vectors, 9 to 40 rows
+// per compute unit ([10240, 4096] and [4096, 4096] among them).
+static bool launch_gemv_f16_rowwise(int32_t batch, int32_t dim_out, int32_t dim_in, const half_t* mat, const half_t* vec,
+                                    half_t* out, hipStream_t st) {
+    if (batch > 2 || dim_in != 4096 || (int64_t)dim_out * dim_in * 2 >= (1ll << 32) || !aligned16(mat) || !aligned16(vec)) return false;
+    const int64_t rpb = ceil_div(dim_out, compute_units());
+    const int r = (int)ceil_div(rpb, 8);
+    if (r < 2 || r > 5) return false;
+    const dim3 grid((unsigned)ceil_div(dim_out, rpb));
+    auto go = [&](auto kern) { hipLaunchKernelGGL(kern, grid, dim3(512), 0, st, batch, dim_out, (int32_t)rpb, mat, vec, out); };
+    auto pick = [&](auto nvc) {
+        constexpr int NV = decltype(nvc)::value;
+        if (r == 2) go(k_gemv_f16_rowwise<NV, 2>);
+        else if (r == 3) go(k_gemv_f16_rowwise<NV, 3>);
+        else if (r == 4) go(k_gemv_f16_rowwise<NV, 4>);
+        else go(k_gemv_f16_rowwise<NV, 5>);
+    };
+    if (batch == 1) pick(std::integral_constant<int, 1>{});
+    else pick(std::integral_constant<int, 2>{});
+    return true;
+}
+
 }  // namespace cpmk
 
 using namespace cpmk;
@@ -221,6 +316,8 @@ int cpmk_gemv_broadcast_mat_fp16(int32_t batch, int32_t dim_out, int32_t dim_in,
     if (batch < 0 || dim_out < 0 || dim_in < 0) return CPMK_EBADARG;
     if ((int64_t)batch * dim_out == 0) return 0;
     if (out == nullptr || (dim_in > 0 && any_null(mat, vec))) return CPMK_EBADARG;
+    if (launch_gemv_f16_rowwise(batch, dim_out, dim_in, (const half_t*)mat, (const half_t*)vec, (half_t*)out, (hipStream_t)stream))
+        return launch_status();
     {   // matrix cores when the rows are whole 256-byte chunks
         const int rc = gemv_f16_coalesced(batch, dim_out, dim_in, mat, vec, out, (hipStream_t)stream);
         if (rc >= 0) return rc;

@@ -117,8 +117,8 @@ __global__ __launch_bounds__(NW * 64) void k_gemv_mfma(int32_t batch, int32_t di
 //
 // F16: the same kernel on fp16 data (cpmk_gemv_broadcast_mat_fp16): dim_in is then the row length in
 // BYTES, a lane's 16 bytes are 8 halves of K for v_mfma_f32_16x16x32_f16 (the same lane -> byte
-// assignment as the int8 instruction), the accumulators are fp32 and leave without scales; the
-// waves add their partial sums in wave order, so the result does not depend on timing.
+// assignment as the int8 instruction), the accumulators are fp32 and leave without scales.
+// The matrix is read once and bypasses the caches' retention (the vectors, which every workgroup reads, stay).
 template <int NW, int RG, int NB, bool F16 = false>
 __global__ __launch_bounds__(NW * 64) void k_gemv_coalesced(int32_t batch, int32_t dim_out, int32_t dim_in, int32_t r4,
                                                             const half_t* __restrict__ scale_mat,
@@ -127,7 +127,6 @@ __global__ __launch_bounds__(NW * 64) void k_gemv_coalesced(int32_t batch, int32
                                                             const int8_t* __restrict__ vec,
                                                             half_t* __restrict__ out) {
     __shared__ __attribute__((aligned(16))) int8_t tbuf[NW][4096];
-    __shared__ int32_t part[RG * NB][256];
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int r = lane & 15, q = lane >> 4;      // MFMA layout
     const int x = lane & 15, y4 = lane >> 4;     // load layout
@@ -187,7 +186,7 @@ __global__ __launch_bounds__(NW * 64) void k_gemv_coalesced(int32_t batch, int32
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 wr[g][i] = int4_t{0, 0, 0, 0};
-                if (wok[g][i]) wr[g][i] = *reinterpret_cast<const int4_t*>(mat + (wo[g][i] + (uint32_t)c * 256u));
+                if (wok[g][i]) wr[g][i] = __builtin_nontemporal_load(reinterpret_cast<const int4_t*>(mat + (wo[g][i] + (uint32_t)c * 256u)));
             }
 #pragma unroll
         for (int t = 0; t < NB; ++t)
@@ -240,23 +239,36 @@ __global__ __launch_bounds__(NW * 64) void k_gemv_coalesced(int32_t batch, int32
         mac_chunk(wa, va);
     }
 
-    for (int idx = tid; idx < RG * NB * 256; idx += NW * 64) (&part[0][0])[idx] = 0;
-    __syncthreads();
-    // accumulator e of lane l: matrix row (l/16)*4 + e, vector l%16 of the 16x16 tile
+    // thread -> (vector, row) with the row fastest, so a vector's outputs are stored contiguously
     if constexpr (F16) {
-        float* fpart = reinterpret_cast<float*>(&part[0][0]);
-        for (int ww = 0; ww < NW; ++ww) {          // one wave after the other: a fixed order of summation
-            if (w == ww) {
+        // every wave leaves its partial sums in a slice of its own; the output threads add the NW slices in
+        // wave order, so the result does not depend on timing
+        __shared__ float fslice[NW * RG * NB * 256];
 #pragma unroll
-                for (int g = 0; g < RG; ++g)
+        for (int g = 0; g < RG; ++g)
 #pragma unroll
-                    for (int t = 0; t < NB; ++t)
+            for (int t = 0; t < NB; ++t)
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) fpart[(g * NB + t) * 256 + (q * 4 + e) * 16 + r] += acc[g][t][e];
+                for (int e = 0; e < 4; ++e) fslice[(w * RG * NB + g * NB + t) * 256 + (q * 4 + e) * 16 + r] = acc[g][t][e];
+        __syncthreads();
+#pragma unroll
+        for (int o = 0; o < NOUT; ++o) {
+            const int idx = tid + o * NW * 64;
+            if (idx < rpb * NB * 16) {
+                const int rr = idx % rpb, bb = idx / rpb;
+                const int g = rr >> 4, t = bb >> 4;
+                float s = 0.0f;
+#pragma unroll
+                for (int ww = 0; ww < NW; ++ww) s += fslice[(ww * RG * NB + g * NB + t) * 256 + (rr & 15) * 16 + (bb & 15)];
+                const int32_t row = row0 + rr;
+                if (row < dim_out && bb < batch) out[(int64_t)bb * dim_out + row] = (half_t)s;
             }
-            __syncthreads();
         }
     } else {
+        __shared__ int32_t part[RG * NB][256];
+        for (int idx = tid; idx < RG * NB * 256; idx += NW * 64) (&part[0][0])[idx] = 0;
+        __syncthreads();
+        // accumulator e of lane l: matrix row (l/16)*4 + e, vector l%16 of the 16x16 tile
 #pragma unroll
         for (int g = 0; g < RG; ++g)
 #pragma unroll
@@ -264,19 +276,15 @@ __global__ __launch_bounds__(NW * 64) void k_gemv_coalesced(int32_t batch, int32
 #pragma unroll
                 for (int e = 0; e < 4; ++e) atomicAdd(&part[g * NB + t][(q * 4 + e) * 16 + r], (int32_t)acc[g][t][e]);
         __syncthreads();
-    }
-    // thread -> (vector, row) with the row fastest, so a vector's outputs are stored contiguously
 #pragma unroll
-    for (int o = 0; o < NOUT; ++o) {
-        const int idx = tid + o * NW * 64;
-        if (idx < rpb * NB * 16) {
-            const int rr = idx % rpb, bb = idx / rpb;
-            const int g = rr >> 4, t = bb >> 4;
-            const int32_t s = part[g * NB + t][(rr & 15) * 16 + (bb & 15)];
-            const int32_t row = row0 + rr;
-            if (row < dim_out && bb < batch) {
-                if constexpr (F16) out[(int64_t)bb * dim_out + row] = (half_t)__builtin_bit_cast(float, s);
-                else out[(int64_t)bb * dim_out + row] = dequant(s, (float)osv[o], (float)osm[o]);
+        for (int o = 0; o < NOUT; ++o) {
+            const int idx = tid + o * NW * 64;
+            if (idx < rpb * NB * 16) {
+                const int rr = idx % rpb, bb = idx / rpb;
+                const int g = rr >> 4, t = bb >> 4;
+                const int32_t s = part[g * NB + t][(rr & 15) * 16 + (bb & 15)];
+                const int32_t row = row0 + rr;
+                if (row < dim_out && bb < batch) out[(int64_t)bb * dim_out + row] = dequant(s, (float)osv[o], (float)osm[o]);
             }
         }
     }

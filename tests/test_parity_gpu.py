@@ -1032,6 +1032,28 @@ def test_gemv_fp16_family(gpu, shape):
         assert_close_fp16(to_np(out), ref0, rtol=1e-3, atol=1e-3, what=fn.__name__)
 
 
+@pytest.mark.parametrize("shape", [(1, 10240, 4096), (2, 10240, 4096), (1, 4096, 4096), (2, 4096, 4096), (2, 5000, 4096),
+                                   (1, 7777, 4096), (2, 2305, 4096), (1, 2304, 4096), (3, 10240, 4096)])
+def test_gemv_broadcast_mat_fp16_one_or_two_vectors(gpu, shape):
+    """The decode shapes with one or two vectors (cuda/gemv.cu:137-164 serves them with the same kernel as any
+    other batch): rows of 4096 halves go to a kernel without matrix cores from 9 rows per compute unit on;
+    ragged last shares, the smallest and largest share, and the neighbours that stay on the matrix cores."""
+    _name("gemv broadcast fp16, few vectors", shape)
+    batch, dim_out, dim_in = shape
+    rng = np.random.default_rng(batch * 7 + dim_out)
+    vec = rng.standard_normal((batch, dim_in)).astype(np.float16)
+    mat = (rng.standard_normal((dim_out, dim_in)) / np.sqrt(dim_in)).astype(np.float16)
+    vd, md = to_gpu(vec), to_gpu(mat)
+    out = torch.full((batch, dim_out), float("nan"), dtype=torch.half, device=gpu)
+    ck.gemv_broadcast_mat_fp16(batch, dim_out, dim_in, md.data_ptr(), vd.data_ptr(), out.data_ptr(), stream())
+    ref = (vec.astype(np.float64) @ mat.astype(np.float64).T).astype(np.float16)
+    assert_close_fp16(to_np(out), ref, rtol=1e-3, atol=1e-3, what="gemv_broadcast_mat_fp16 %s" % (shape,))
+    # the same call again gives the same bits (fixed summation order)
+    out2 = torch.empty_like(out)
+    ck.gemv_broadcast_mat_fp16(batch, dim_out, dim_in, md.data_ptr(), vd.data_ptr(), out2.data_ptr(), stream())
+    assert_bits_equal(to_np(out2), to_np(out), "repeat")
+
+
 @pytest.mark.parametrize("shape", [(2, 64, 128), (3, 100, 77), (1, 4096, 33), (4, 24, 1)])
 def test_embedding_and_kv_copy(gpu, shape):
     """Pure data movement next to the path: gathers from the embedding table and the copy of a
