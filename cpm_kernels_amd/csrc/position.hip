@@ -39,7 +39,7 @@ constexpr int QC = 16384;
 __global__ __launch_bounds__(256) void k_position_forward(int32_t query_len, int32_t key_len, int32_t num_buckets,
                                                           int32_t max_distance, const int32_t* __restrict__ table,
                                                           const half_t* __restrict__ weight, half_t* out,
-                                                          int bidirectional) {
+                                                          int bidirectional, int vec8) {
     extern __shared__ half_t diag[];          // min(query_len, QC) + KR - 1 entries
     const int32_t k0 = blockIdx.x * KR;
     const int32_t h = blockIdx.y;
@@ -53,6 +53,20 @@ __global__ __launch_bounds__(256) void k_position_forward(int32_t query_len, int
     for (int32_t t = threadIdx.x; t < nd; t += 256)
         diag[t] = wh[bucket_of(rel_min + t, num_buckets, max_distance, table, bidirectional)];
     __syncthreads();
+    if (vec8) {
+        // 16-byte stores: the workgroup's rows are cut into pieces of eight queries and dealt to the threads
+        const int32_t nv = nq >> 3, items = (kend - k0) * nv;
+        for (int32_t it = threadIdx.x; it < items; it += 256) {
+            const int32_t kk = it / nv, qv = it - kk * nv;
+            const int32_t k = k0 + kk;
+            const half_t* d = diag + (qv * 8 + q0 - k - rel_min);
+            half8_t v;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = d[e];
+            *reinterpret_cast<half8_t*>(out + ((int64_t)h * key_len + k) * query_len + q0 + qv * 8) = v;
+        }
+        return;
+    }
     for (int32_t k = k0; k < kend; ++k) {
         half_t* orow = out + ((int64_t)h * key_len + k) * query_len + q0;
         const int32_t shift = q0 - k - rel_min;    // q - k - rel_min = (q - q0) + shift
@@ -97,13 +111,14 @@ int cpmk_position_embedding_forward(int32_t query_len, int32_t key_len, int32_t 
     if ((int64_t)query_len * key_len * num_heads == 0) return 0;
     if (any_null(position_mapping, weight, out)) return CPMK_EBADARG;
     const size_t smem = (size_t)((query_len < QC ? query_len : QC) + KR - 1) * sizeof(half_t);
+    const int vec8 = (query_len % 8 == 0) && aligned16(out);       // every row then starts on a 16-byte boundary
     // heads are the grid's y dimension (at most 65535): more go out in several launches
     for (int64_t h0 = 0; h0 < num_heads; h0 += 65535) {
         const int64_t nh = num_heads - h0 < 65535 ? num_heads - h0 : 65535;
         dim3 grid((unsigned)ceil_div(key_len, KR), (unsigned)nh, (unsigned)ceil_div(query_len, QC));
         hipLaunchKernelGGL(k_position_forward, grid, dim3(256), smem, (hipStream_t)stream, query_len, key_len,
                            num_buckets, max_distance, (const int32_t*)position_mapping,
-                           (const half_t*)weight + h0 * num_buckets, (half_t*)out + h0 * key_len * query_len, bidirectional);
+                           (const half_t*)weight + h0 * num_buckets, (half_t*)out + h0 * key_len * query_len, bidirectional, vec8);
         if (int e = launch_status()) return e;
     }
     return 0;

@@ -905,7 +905,7 @@ def test_position_embedding(gpu, cfg):
     rng = np.random.default_rng(1005)
     w = rand_half(rng, (heads, num_buckets))
     wd = to_gpu(w)
-    for (ql, kl) in ((128, 128), (77, 200), (1024, 16), (5, 3)):
+    for (ql, kl) in ((128, 128), (77, 200), (1024, 16), (5, 3), (136, 50)):
         out = torch.empty((heads, kl, ql), dtype=torch.half, device=gpu)
         ck.position_embedding_forward(ql, kl, num_buckets, max_distance, heads, table.data_ptr(), wd.data_ptr(),
                                       out.data_ptr(), bidi, stream())
