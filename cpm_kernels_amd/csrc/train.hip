@@ -272,7 +272,7 @@ __global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_b
     using T = ColTile<NT, LPR, R>;
     constexpr bool TWO = KIND != kLnFwdV && KIND != kLnFwdMV && KIND != kScaleRound;     // reads grad_in too
     constexpr bool IS_MAX = KIND == kScaleRound;
-    constexpr int NV = IS_MAX ? 1 : 2;
+    constexpr int NV = (KIND == kLnFwdMV || KIND == kLnBwdMV) ? 2 : 1;      // statistics per column
     __shared__ float lds[(T::NW + 1) * T::COLS * NV];
     __shared__ float tot[T::COLS * 2];
     const int tid = threadIdx.x, cg = tid % LPR, rg = tid / LPR;
@@ -301,8 +301,11 @@ __global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_b
         }
     }
     half8_t va[R], vg[TWO ? R : 1];
-    coltile_load<NT, LPR, R>(va, p.a + boff, own_n, p.m, col0, (half_t)0.0f);
-    if constexpr (TWO) coltile_load<NT, LPR, R>(vg, p.g + boff, own_n, p.m, col0, (half_t)0.0f);
+    // every input byte is read once: non-temporal loads; non-temporal stores too, except for the softmax
+    // gradient, where they measured 1-2 % slower
+    constexpr bool NTS = KIND != kSoftmaxBwd;
+    coltile_load<NT, LPR, R, true>(va, p.a + boff, own_n, p.m, col0, (half_t)0.0f);
+    if constexpr (TWO) coltile_load<NT, LPR, R, true>(vg, p.g + boff, own_n, p.m, col0, (half_t)0.0f);
     float mean[8], var[8], c3[8], sxv[R];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
@@ -322,7 +325,7 @@ __global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_b
         for (int e = 0; e < 8; ++e) {
             const float x = (float)va[q][e];
             const float gi = TWO ? (float)vg[TWO ? q : 0][e] : 0.0f;
-            if constexpr (KIND == kLnFwdV) s[8 + e] += x * x;
+            if constexpr (KIND == kLnFwdV) s[e] += x * x;
             else if constexpr (KIND == kLnFwdMV) { s[e] += x; s[8 + e] += x * x; }
             else if constexpr (KIND == kLnBwdV) s[e] += gi * c3[e] * x;
             else if constexpr (KIND == kLnBwdMV) { s[e] += gi * c3[e] * (x - mean[e]); s[8 + e] += -gi * var[e]; }
@@ -339,11 +342,13 @@ __global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_b
             const uint64_t deadline = wall_clock64() + kXchTimeoutTicks;
             float acc = 0.0f;
             bool ok = true;
-            for (int32_t q0 = 0; q0 < parts; q0 += 8) {
-                float x[8];
-                ok &= xch_gather<8>(team_slots, parts, q0, tid, tag, deadline, x);
+            // four parts per round trip: eight would push the kernels that can stay within 128 registers (two workgroups
+            // per compute unit) beyond them
+            for (int32_t q0 = 0; q0 < parts; q0 += 4) {
+                float x[4];
+                ok &= xch_gather<4>(team_slots, parts, q0, tid, tag, deadline, x);
 #pragma unroll
-                for (int j = 0; j < 8; ++j) acc = IS_MAX ? fmaxf(acc, x[j]) : acc + x[j];     // part order; absent parts are zeros
+                for (int j = 0; j < 4; ++j) acc = IS_MAX ? fmaxf(acc, x[j]) : acc + x[j];     // part order; absent parts are zeros
             }
             tot[tid] = ok ? acc : __builtin_nanf("");
             if (!ok) xch_flag(xl, kXchStatusTimeout);
@@ -358,7 +363,7 @@ __global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_b
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
         k0[e] = k1[e] = 0.0f;
-        if constexpr (KIND == kLnFwdV) k1[e] = rsqrtf(s[8 + e] / fn + p.eps);
+        if constexpr (KIND == kLnFwdV) k1[e] = rsqrtf(s[e] / fn + p.eps);
         else if constexpr (KIND == kLnFwdMV) { k0[e] = s[e] / fn; k1[e] = rsqrtf(s[8 + e] / fn - k0[e] * k0[e] + p.eps); }
         else if constexpr (KIND == kLnBwdMV) s[8 + e] -= 2.0f * s[e] * mean[e];        // local_grad_mean -= 2 * local_grad_var * local_mean
         else if constexpr (KIND == kScaleRound) k0[e] = (float)((double)s[e] / 127.0);     // float / double constant, as the reference writes it
@@ -400,7 +405,7 @@ __global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_b
                 else o = x * (gi - s[e]);
                 va[q][e] = round_f16(o);
             }
-        coltile_store<NT, LPR, R>(va, p.out + boff, own_n, p.m, col0);
+        coltile_store<NT, LPR, R, NTS>(va, p.out + boff, own_n, p.m, col0);
     }
     if (parts > 1 && tid < 64) xch_retire(xl, team, parts);
 }
