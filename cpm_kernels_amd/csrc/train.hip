@@ -554,6 +554,96 @@ __global__ __launch_bounds__(256) void k_position_backward_team(int32_t query_le
     if (tid < 64) xch_retire(xl, h, parts);
 }
 
+// The same team layout for query rows of whole 16-byte pieces: the bias depends on q - k only, so the sum over
+// a bucket is a sum over diagonals of grad_out.  A thread takes pieces of eight key rows x eight queries (eight
+// 16-byte non-temporal loads in flight, pieces dealt query-fastest so that a wave reads whole rows), adds the 64
+// values into the 15 diagonals that cross the piece -- element (row kk, query e) belongs to diagonal e - kk, a
+// register chosen at compile time -- and leaves the 15 sums in the piece's place in LDS.  Then a thread per
+// diagonal adds the pieces' contributions to it (two pieces per block of eight rows) in a fixed order: no
+// atomics up to here.  At the end the diagonals' sums go into the bucket histogram, and the parts' histograms
+// to part 0 as above.
+__global__ __launch_bounds__(256) void k_position_backward_diag(int32_t query_len, int32_t key_len, int32_t num_buckets,
+                                                                int32_t max_distance, const int32_t* __restrict__ mapping,
+                                                                const half_t* __restrict__ grad_out, half_t* __restrict__ grad,
+                                                                int bidirectional, int32_t parts, int32_t rows_per_part,
+                                                                uint32_t nteams, XchLaunch xl) {
+    uint64_t* const xch = xl.region;
+    const uint32_t tag = xl.tag;
+    extern __shared__ float psm[];
+    float* hist = psm;                                    // num_buckets
+    float* stage = psm + num_buckets;                     // 15 floats per piece of the part
+    XchMember me;
+    if (!xch_member(blockIdx.x, parts, nteams, me)) return;
+    const uint32_t part = me.part, h = me.team;
+    const int tid = threadIdx.x;
+    const int32_t k0 = part * rows_per_part, k1 = min(key_len, k0 + rows_per_part);
+    const int32_t rel_min = -(k1 - 1), nd = query_len + (k1 - k0) - 1;      // rel = q - k of the part's rows: rel_min + [0, nd)
+    for (int i = tid; i < num_buckets; i += 256) hist[i] = 0.0f;
+    const half_t* g = grad_out + (int64_t)h * key_len * query_len;
+    const int32_t ncp = query_len >> 3, nrb = (k1 - k0 + 7) >> 3;
+    for (int32_t pi = tid; pi < ncp * nrb; pi += 256) {
+        const int32_t rb = pi / ncp, cp = pi - rb * ncp;
+        const int32_t kr = k0 + rb * 8;
+        half8_t v[8];
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) {
+            const int32_t row = min(kr + kk, k1 - 1);      // (rows past the part's last repeat it and are left out below)
+            v[kk] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(g + (int64_t)row * query_len) + cp);
+        }
+        float d[15];
+#pragma unroll
+        for (int j = 0; j < 15; ++j) d[j] = 0.0f;
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) d[e - kk + 7] += (kr + kk < k1) ? (float)v[kk][e] : 0.0f;
+#pragma unroll
+        for (int j = 0; j < 15; ++j) stage[pi * 15 + j] = d[j];       // d[j]: diagonal rel = 8 cp - kr + j - 7
+    }
+    __syncthreads();
+    const int32_t half_b = num_buckets / 2;
+    for (int32_t r = tid; r < nd; r += 256) {
+        float sum = 0.0f;
+        for (int32_t rb = 0; rb < nrb; ++rb) {
+            const int32_t t = r + rel_min + k0 + 8 * rb + 7;          // = 8 cp + j of the pieces of this row block that hold the diagonal
+            const int32_t cp = t >> 3, j = t & 7;
+            if (j <= 6 && cp >= 1 && cp <= ncp) sum += stage[(rb * ncp + cp - 1) * 15 + j + 8];
+            if (cp >= 0 && cp < ncp) sum += stage[(rb * ncp + cp) * 15 + j];
+        }
+        int32_t rel = r + rel_min, off = 0;
+        if (rel < 0) {
+            if (bidirectional) { rel = -rel; off = half_b; }
+            else rel = 0;
+        }
+        if (rel >= max_distance) rel = max_distance - 1;
+        atomicAdd(&hist[mapping[rel] + off], sum);
+    }
+    __syncthreads();
+    if (parts == 1) {
+        for (int i = tid; i < num_buckets; i += 256) grad[(int64_t)h * num_buckets + i] = (half_t)hist[i];
+        return;
+    }
+    uint64_t* team_slots = xch + (size_t)h * parts * kXchVals;
+    for (int i = tid; i < num_buckets; i += 256) xch_post(team_slots + (size_t)part * kXchVals, i, hist[i], tag);
+    if (part == 0) {
+        const uint64_t deadline = wall_clock64() + kXchTimeoutTicks;
+        for (int i = tid; i < num_buckets; i += 256) {
+            float acc = 0.0f;
+            bool ok = true;
+            for (int32_t p0 = 0; p0 < parts; p0 += 8) {
+                float x[8];
+                ok &= xch_gather<8>(team_slots, parts, p0, i, tag, deadline, x);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc += x[j];
+            }
+            grad[(int64_t)h * num_buckets + i] = ok ? (half_t)acc : (half_t)__builtin_nanf("");
+            if (!ok) xch_flag(xl, kXchStatusTimeout);
+        }
+        __syncthreads();
+    }
+    if (tid < 64) xch_retire(xl, h, parts);
+}
+
 // ---------------------------------------------------------------------------------------
 // Embedding gradient in two stages over ids sorted per batch entry (cuda/embedding.cu:38-88):
 // stage 1 sums runs of equal ids inside one batch entry, writes complete runs to grad and the
@@ -871,6 +961,17 @@ int cpmk_position_embedding_backward(int32_t query_len, int32_t key_len, int32_t
             XchScope xs;
             const int rc = xs.begin((int64_t)num_heads * parts, (hipStream_t)stream);
             if (rc != 0 && rc != kXchFull) return rc;
+            const int64_t pieces = (query_len / 8) * ceil_div(rpp, 8);          // of eight key rows x eight queries, 15 floats each
+            const size_t smem = (size_t)(num_buckets + pieces * 15) * sizeof(float);
+            if (rc == 0 && query_len % 8 == 0 && smem <= 64 * 1024 && aligned16(grad_out)) {
+                hipLaunchKernelGGL(k_position_backward_diag, dim3((unsigned)xch_team_grid(num_heads, parts)), dim3(256), smem,
+                                   (hipStream_t)stream, query_len, key_len, num_buckets, max_distance, (const int32_t*)position_mapping,
+                                   (const half_t*)grad_out, (half_t*)grad, bidirectional, (int32_t)parts, (int32_t)rpp,
+                                   (uint32_t)num_heads, xs.xl);
+                const int e = launch_status();
+                const int rc2 = xs.end();
+                return e ? e : rc2;
+            }
             if (rc == 0) {      // (kXchFull: recorded into a graph and the capture reserve is used up: the kernel without packets below)
                 hipLaunchKernelGGL(k_position_backward_team, dim3((unsigned)xch_team_grid(num_heads, parts)), dim3(256),
                                    num_buckets * sizeof(float) + max_distance * sizeof(int32_t), (hipStream_t)stream, query_len, key_len,

@@ -232,7 +232,10 @@ def test_gemm_backward_quantisers(gpu, shape, bc):
 
 
 @pytest.mark.parametrize("cfg", [(32, 128, True, 12, 100, 90), (32, 128, False, 4, 64, 200), (64, 512, True, 3, 17, 9),
-                                 (32, 128, True, 16, 1024, 1024), (32, 128, False, 5, 333, 2500), (256, 128, True, 2, 70, 130)])
+                                 (32, 128, True, 16, 1024, 1024), (32, 128, False, 5, 333, 2500), (256, 128, True, 2, 70, 130),
+                                 # query rows of whole 16-byte pieces (sums over diagonals): the longest, ragged key rows, one-sided
+                                 (32, 128, True, 3, 4096, 130), (32, 128, True, 2, 520, 77), (32, 128, False, 2, 256, 300),
+                                 (128, 256, True, 9, 8, 4000)])
 def test_position_embedding_backward(gpu, cfg):
     _name("position_embedding_backward", cfg)
     import oracle
