@@ -456,6 +456,58 @@ __global__ __launch_bounds__(256) void k_round_scale_rows_wide(int64_t rows, int
     }
 }
 
+// The same for rows of at most 2048 columns, kept in registers: a wave takes U consecutive rows of P 16-byte pieces
+// per lane (P * U = 4 loads in flight per lane, the matrix read once and with the non-temporal hint), finds each
+// row's maximum over the wave with data-parallel-primitive operands and rounds from the registers.
+template <int P, int U>
+__global__ __launch_bounds__(256) void k_round_scale_rows_reg(int64_t rows, int32_t n, int32_t m, const half_t* __restrict__ mat,
+                                                              const half_t* __restrict__ scale_y, int8_t* __restrict__ out,
+                                                              half_t* __restrict__ scale_x, int bc) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row0 = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * U;
+    if (row0 >= rows) return;
+    half8_t xv[U][P], sv[U][P];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int64_t row = row0 + u < rows ? row0 + u : rows - 1;
+        const half_t* x = mat + row * m;
+        const half_t* sy = scale_y + (bc ? 0 : (row / n) * m);
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            const int32_t j = lane * 8 + p * 512;
+            xv[u][p] = sv[u][p] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+            if (j < m) {
+                xv[u][p] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(x + j));
+                sv[u][p] = *reinterpret_cast<const half8_t*>(sy + j);
+            }
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        float mx = 0.0f;
+#pragma unroll
+        for (int p = 0; p < P; ++p)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) mx = fmaxf(fabsf((float)xv[u][p][e] * (float)sv[u][p][e]), mx);
+        mx = __builtin_bit_cast(float, wave_max_u32_uniform(__builtin_bit_cast(uint32_t, mx)));      // (non-negative floats order as their bits)
+        const float s = (float)((double)mx / 127.0);
+        const int64_t row = row0 + u;
+        if (row < rows) {
+            if (lane == 0) scale_x[row] = (half_t)s;
+#pragma unroll
+            for (int p = 0; p < P; ++p) {
+                const int32_t j = lane * 8 + p * 512;
+                if (j < m) {
+                    int32_t t[8];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) t[e] = quant_i8((float)xv[u][p][e] * (float)sv[u][p][e], s);
+                    *reinterpret_cast<uint2_t*>(out + row * m + j) = uint2_t{pack4_i8(t[0], t[1], t[2], t[3]), pack4_i8(t[4], t[5], t[6], t[7])};
+                }
+            }
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------------------
 // Gradient of the relative-position bias: grad[h, bucket] = sum of grad_out[h, k, q] over the
 // (k, q) that map to the bucket.  One workgroup per head, a bucket histogram in LDS.
@@ -936,6 +988,17 @@ int cpmk_gemm_backward_round_scale(int32_t batch, int32_t n, int32_t m, const vo
     if (rows > 0x7fffffff) return CPMK_ETOOBIG;
     if (scale_x == nullptr || (m > 0 && any_null(mat, scale_y, out))) return CPMK_EBADARG;
     if (m % 8 == 0 && aligned16(mat) && aligned16(scale_y) && (reinterpret_cast<uintptr_t>(out) & 7u) == 0) {
+        if (m <= 2048) {      // rows that a wave holds in registers
+            auto go = [&](auto pc, auto uc) {
+                constexpr int P = decltype(pc)::value, U = decltype(uc)::value;
+                hipLaunchKernelGGL((k_round_scale_rows_reg<P, U>), dim3((unsigned)ceil_div(rows, 4 * U)), dim3(256), 0, (hipStream_t)stream, rows, n,
+                                   m, (const half_t*)mat, (const half_t*)scale_y, (int8_t*)out, (half_t*)scale_x, broad_cast_y);
+            };
+            if (m <= 512) go(std::integral_constant<int, 1>{}, std::integral_constant<int, 4>{});
+            else if (m <= 1024) go(std::integral_constant<int, 2>{}, std::integral_constant<int, 2>{});
+            else go(std::integral_constant<int, 4>{}, std::integral_constant<int, 1>{});
+            return launch_status();
+        }
         hipLaunchKernelGGL(k_round_scale_rows_wide, dim3((unsigned)ceil_div(rows, 4)), dim3(256), 0, (hipStream_t)stream, rows, n, m,
                            (const half_t*)mat, (const half_t*)scale_y, (int8_t*)out, (half_t*)scale_x, broad_cast_y);
         return launch_status();

@@ -207,7 +207,9 @@ def test_layernorm_training_kernels(gpu, shape):
     assert_close_fp16(to_np(grad), ot.layernorm_backward_mv(x, g, m_dev, v_dev), rtol=2e-3, atol=1e-3, what="backward_mv")
 
 
-@pytest.mark.parametrize("shape", COL_SHAPES + [(2, 256, 4096)])
+# (rows of at most 2048 columns stay in a wave's registers, one, two or four pieces a lane; ragged ends and waves
+# whose rows straddle two batch entries)
+@pytest.mark.parametrize("shape", COL_SHAPES + [(2, 256, 4096), (3, 37, 512), (2, 50, 1000), (1, 9, 2048), (2, 11, 1544)])
 @pytest.mark.parametrize("bc", [False, True])
 def test_gemm_backward_quantisers(gpu, shape, bc):
     _name("gemm_backward_round_scale / scale_round", shape, bc)
