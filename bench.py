@@ -45,7 +45,7 @@ PROFILES = os.path.join(ROOT, "profiles")
 OFFLINE_SOURCE = {"traffic": "profiles/hbm_traffic_counters.txt (offline rocprofv3 --pmc run of this bench, read at run time, not measured by this process)",
                   "mfma": "profiles/gemm_mfma_utilisation.txt (offline rocprofv3 --pmc run of this bench, read at run time, not measured by this process)"}
 # which row of profiles/hbm_traffic_counters.txt belongs to which workload (a substring of the kernel's name)
-TRAFFIC_KERNELS = {"gemm_fused": "k_gemm_dma<2, 4, 4, 2, 128, 1,", "gemv": "k_gemv_directILi2ELi3", "layernorm": "k_layernorm_teamILi1024ELi8ELb0", "softmax": "k_softmax_stream"}
+TRAFFIC_KERNELS = {"gemm_fused": "k_gemm_dma<2, 4, 4, 2, 128, 1,", "gemv": "k_gemv_coalescedILi8ELi3ELi2ELb0", "layernorm": "k_layernorm_teamILi1024ELi8ELb0", "softmax": "k_softmax_stream"}
 
 
 def offline_counters():
@@ -846,7 +846,7 @@ def main():
     # kernel, average launch time, algorithmic bytes, achieved rate, fraction of the published HBM peak, and
     # the HBM bytes the counters saw per launch (profiles/hbm_traffic_counters.txt).
     hbm_block = {}
-    for name, kernel in (("gemv_broadcast_mat_int8", "k_gemv_direct<2,3>"), ("layernorm_forward", "k_layernorm_team<1024,8,false>"),
+    for name, kernel in (("gemv_broadcast_mat_int8", "k_gemv_coalesced<8,3,2>"), ("layernorm_forward", "k_layernorm_team<1024,8,false>"),
                          ("softmax_forward", "k_softmax_stream<1024,8,8>")):
         c = components.get(name)
         if c is not None:

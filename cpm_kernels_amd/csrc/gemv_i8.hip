@@ -290,124 +290,9 @@ __global__ __launch_bounds__(NW * 64) void k_gemv_coalesced(int32_t batch, int32
     }
 }
 
-// One-round kernel for dim_in == 4096 and up to 32 vectors, at most 48 rows per workgroup.  Wave w owns
-// bytes [512w, 512w + 512) of K.  Its share of the vectors (NB*16 x 512 bytes) goes global -> LDS by
-// DMA, two vectors per instruction, fully coalesced, into the wave's own 16 KB region (16-byte
-// chunk c of a vector's piece at chunk slot c ^ (vector % 16), so that the MFMA-layout reads below
-// are bank-conflict free).  The wave requests all of its matrix bytes at once, straight in the
-// MFMA layout: lane (r, q) loads bytes [64kb + 16q, +16) of its K range of row 16g + r -- sixteen
-// half cache lines per instruction, the other halves by the instruction for the neighbouring kb.
-// No LDS transposes and no barrier until the final reduction: loads return in the order they
-// were issued, so s_waitcnt vmcnt tells when the vectors have landed, and the MFMAs follow the
-// matrix loads as they return.
-template <int NB, int RG>
-__global__ __launch_bounds__(512) void k_gemv_direct(int32_t batch, int32_t dim_out, int32_t rpb,
-                                                     const half_t* __restrict__ scale_mat,
-                                                     const int8_t* __restrict__ mat,
-                                                     const half_t* __restrict__ scale_vec,
-                                                     const int8_t* __restrict__ vec,
-                                                     half_t* __restrict__ out) {
-    constexpr int KB = 8, WK = KB * 64, DIN = 8 * WK;       // k-blocks and bytes of K per wave; dim_in
-    constexpr int REGION = NB * 16 * WK;                    // bytes of LDS per wave: its piece of every vector
-    extern __shared__ __attribute__((aligned(16))) int8_t vsm[];        // 8 * REGION bytes of vectors, then the cross-wave sums
-    int32_t* part = reinterpret_cast<int32_t*>(vsm + 8 * REGION);       // RG * NB * 256 words
-    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) int8_t*)vsm;
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int r = lane & 15, q = lane >> 4;
-    const int32_t row0 = blockIdx.x * rpb;
-    constexpr int NOUT = (RG * NB * 256 + 511) / 512;     // outputs per thread
-    // The first 16 rows of the matrix, then the vectors, then the other rows: the requests to memory are
-    // under way while the address unit works off the 128 KB of vectors, which come from L2.
-    int4_t wf[RG][KB];
-    auto load_rows = [&](auto gc) __attribute__((always_inline)) {
-        constexpr int g = decltype(gc)::value;
-        const int32_t row = min(row0 + min(g * 16 + r, rpb - 1), dim_out - 1);
-        const int8_t* rp = mat + (uint32_t)row * (uint32_t)DIN + w * WK + q * 16;
-        // (rows past the workgroup's share repeat its last row; switching those lanes off instead, and plain instead of
-        // non-temporal loads, each measured 0.5-0.7 us slower at 32 x [10240, 4096])
-#pragma unroll
-        for (int kb = 0; kb < KB; ++kb) wf[g][kb] = __builtin_nontemporal_load(reinterpret_cast<const int4_t*>(rp + kb * 64));
-    };
-    load_rows(std::integral_constant<int, 0>{});
-    __builtin_amdgcn_sched_barrier(0);
-    // the vectors: instruction j brings this wave's piece of vectors 2j and 2j + 1 (lanes 0-31 / 32-63)
-    {
-        const int p = lane & 31, hi = lane >> 5;
-#pragma unroll
-        for (int j = 0; j < NB * 8; ++j) {
-            const int v = 2 * j + hi;
-            const uint32_t voff = (uint32_t)min(v, batch - 1) * (uint32_t)DIN + (uint32_t)(w * WK) + (uint32_t)((p ^ (v & 15)) << 4);
-            lds_dma16(voff, vec, lds_base + w * REGION + j * 1024);
-        }
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    if constexpr (RG > 1) load_rows(std::integral_constant<int, 1>{});
-    if constexpr (RG > 2) load_rows(std::integral_constant<int, 2>{});
-    __builtin_amdgcn_sched_barrier(0);
-    // The outputs this thread will write (vector bb, row rr of the workgroup's share; the row runs fastest, so a
-    // vector's outputs are stored contiguously) and their scales.  Worked out and requested here, behind the
-    // last matrix load: the two divisions per output then run while the memory works, and the scales, needed
-    // last, are also the last loads to return.
-    int orr[NOUT], obb[NOUT];
-    half_t osv[NOUT], osm[NOUT];
-#pragma unroll
-    for (int o = 0; o < NOUT; ++o) {
-        const int idx = tid + o * 512;
-        obb[o] = idx / rpb;
-        orr[o] = idx - obb[o] * rpb;
-        osv[o] = scale_vec[min(obb[o], batch - 1)];
-        osm[o] = scale_mat[min(row0 + orr[o], dim_out - 1)];
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    for (int idx = tid; idx < RG * NB * 256; idx += 512) part[idx] = 0;
-    // the vectors (and the rows requested before them) have landed when only the later matrix loads and the scales are still under way
-    wait_vmcnt<(RG - 1) * KB + 2 * NOUT>();
-    __builtin_amdgcn_sched_barrier(0);
-    int4_t vf[NB][KB];
-#pragma unroll
-    for (int t = 0; t < NB; ++t) {
-        const int v = t * 16 + r;
-        const int8_t* vp = vsm + w * REGION + (v >> 1) * 1024 + (v & 1) * 512;
-#pragma unroll
-        for (int kb = 0; kb < KB; ++kb) vf[t][kb] = *reinterpret_cast<const int4_t*>(vp + (((kb * 4 + q) ^ (v & 15)) << 4));
-    }
-    __syncthreads();       // (part is zero)
-    // A row group's products are added to the workgroup's sums as soon as they exist, so that behind the last
-    // data only the last group's remain.  Accumulator e of lane l: matrix row (l/16)*4 + e, vector l%16 of the 16x16 tile.
-#pragma unroll
-    for (int g = 0; g < RG; ++g) {
-        int4_t acc[NB];
-#pragma unroll
-        for (int t = 0; t < NB; ++t) acc[t] = int4_t{0, 0, 0, 0};
-#pragma unroll
-        for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-            for (int t = 0; t < NB; ++t) acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[g][kb], vf[t][kb], acc[t], 0, 0, 0);
-#pragma unroll
-        for (int t = 0; t < NB; ++t)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) atomicAdd(&part[(g * NB + t) * 256 + (q * 4 + e) * 16 + r], (int32_t)acc[t][e]);
-        __builtin_amdgcn_sched_barrier(0);
-    }
-    __syncthreads();
-#pragma unroll
-    for (int o = 0; o < NOUT; ++o) {
-        const int idx = tid + o * 512;
-        if (idx < rpb * NB * 16) {
-            const int rr = orr[o], bb = obb[o];
-            const int g = rr >> 4, t = bb >> 4;
-            const int32_t s = part[(g * NB + t) * 256 + (rr & 15) * 16 + (bb & 15)];
-            const int32_t row = row0 + rr;
-            if (row < dim_out && bb < batch) out[(int64_t)bb * dim_out + row] = dequant(s, (float)osv[o], (float)osm[o]);
-        }
-    }
-}
-
 // One or two vectors (decode with a batch of one or two sequences): no matrix cores.  A wave reads whole rows --
 // instruction i of a row brings bytes [1024 i, 1024 i + 1024), 16 per lane, whole cache lines in address order,
-// the access pattern in which a one-round read of this size is 2 us quicker than in the MFMA operand layout of
-// the kernel above -- and multiplies them with v_dot4_i32_i8 against the vectors' bytes at the same positions,
+// the access pattern in which a one-round read of this size is quickest -- and multiplies them with v_dot4_i32_i8 against the vectors' bytes at the same positions,
 // which every lane keeps in registers (NV x PPL pieces of 16 bytes).  One workgroup per compute unit, wave w
 // takes rows w, w + 8, ... of the workgroup's share (G of them), all loads of a wave requested at once (G rows of
 // PPL pieces, at most 20 pieces = 80 registers); the per-lane sums of a (row, vector) pair are added over the wave,
@@ -528,34 +413,6 @@ static void launch_coalesced(int32_t batch, int32_t dim_out, int32_t dim_in, con
     go(std::integral_constant<int, 1>{});
 }
 
-// The one-round kernel: dim_in == 4096, at most 32 vectors, and 17 to 48 rows per compute unit, one workgroup
-// each.  Returns false when the shape does not qualify.  With at most 16 rows per compute unit the vectors outweigh
-// a workgroup's share of the matrix and the chunked kernel is quicker (32 x [4096, 4096]: 6.3 against 7.1 us; one
-// vector: 5.1 against 5.8).  The same kernel built for rows of 2048, 8192 and 10240 bytes (sixteen waves for the
-// long rows, the vectors straight into registers where the LDS cannot hold them) measured equal (2048) or slower
-// (32 x [4096, 8192]: 15.7 against 10.4 us; 32 x [4096, 10240]: 19.7 against 13.4) than the chunked kernel,
-// which therefore keeps every other row length.
-template <int NB>
-static bool launch_gemv_direct(int32_t batch, int32_t dim_out, int32_t dim_in, const half_t* sm, const int8_t* mat,
-                               const half_t* sv, const int8_t* vec, half_t* out, hipStream_t st, int* err) {
-    if (dim_in != 4096) return false;
-    const int64_t rpb = ceil_div(dim_out, compute_units());
-    if (rpb <= 16 || rpb > 48 || (int64_t)dim_out * dim_in >= (1ll << 32)) return false;
-    const int rg = (int)ceil_div(rpb, 16);
-    const dim3 grid((unsigned)ceil_div(dim_out, rpb));
-    auto go = [&](auto rgc) {
-        auto kern = k_gemv_direct<NB, decltype(rgc)::value>;
-        static std::atomic<bool> lds_enabled[64];
-        constexpr int smem = NB * 16 * 512 * 8 + decltype(rgc)::value * NB * 1024;
-        if (smem > 48 * 1024)
-            if (int e = enable_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_enabled)) { *err = e; return; }
-        hipLaunchKernelGGL(kern, grid, dim3(512), smem, st, batch, dim_out, (int32_t)rpb, sm, mat, sv, vec, out);
-    };
-    if (rg == 3) go(std::integral_constant<int, 3>{});
-    else go(std::integral_constant<int, 2>{});
-    return true;
-}
-
 // The row-wise kernel for one or two vectors: rows of 4 KB (up to 40 per compute unit) or 10 KB (up to 16 per
 // compute unit) -- the row lengths of the model this path serves; at least two rows per wave, below that the
 // matrix-core kernels are as quick.  ([10240, 4096] at one / two vectors: 7.8 / 8.5 us against 9.6 / 9.8 on the
@@ -661,11 +518,7 @@ extern "C" int cpmk_gemv_broadcast_mat_int8(int32_t batch, int32_t dim_out, int3
         const int8_t* v = V + (int64_t)b0 * dim_in;
         half_t* o = O + (int64_t)b0 * dim_out;
         const half_t* s = sv + b0;
-        int derr = 0;
         if (launch_gemv_rowwise(nb, dim_out, dim_in, sm, M, s, v, o, st)) {
-        } else if (nb <= 16 ? launch_gemv_direct<1>(nb, dim_out, dim_in, sm, M, s, v, o, st, &derr)
-                     : (nb <= 32 && launch_gemv_direct<2>(nb, dim_out, dim_in, sm, M, s, v, o, st, &derr))) {
-            if (derr) return derr;
         } else if (dim_in % 256 == 0 && (int64_t)dim_out * dim_in < (1ll << 32) && (int64_t)nb * dim_in < (1ll << 32)) {
             if (nb <= 16) launch_coalesced<1, 4>(nb, dim_out, dim_in, sm, M, s, v, o, st);
             else if (nb <= 32) launch_coalesced<2, 4>(nb, dim_out, dim_in, sm, M, s, v, o, st);

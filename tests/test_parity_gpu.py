@@ -481,7 +481,7 @@ def test_north_star_fused_pipeline_bits(gpu):
 # ---------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("batch,dim_out,dim_in", [(32, 10240, 4096), (16, 4444, 8888), (1, 48, 256), (33, 100, 4096),
                                                   (130, 64, 512), (5, 17, 12), (128, 1000, 1040), (8, 40, 16),
-                                                  # dim_in 4096: the one-round kernel at 40, 36, 25 (odd) and 20 rows per workgroup, ragged ends; 16, 2 and 1 rows (the chunked kernel)
+                                                  # dim_in 4096 at 40, 36, 25 (odd) and 20 rows per workgroup, ragged ends; 16, 2 and 1 rows
                                                   (32, 10239, 4096), (17, 9000, 4096), (3, 6145, 4096), (16, 5000, 4096),
                                                   (7, 257, 4096), (1, 256, 4096), (31, 4096, 4096), (32, 10241, 4096),
                                                   # other row lengths of whole 256-byte chunks (the chunked kernel): the decode shapes of a 4096 / 10240 FFN
