@@ -701,8 +701,9 @@ def main():
                                                                in_kernel_span_frac_of_published_peak=round(piece / (span_us * 1e-6) / 1e9 / PEAK_HBM_GBS, 4),
                                                                note="span = last workgroup's end - first workgroup's start (wall clock stamps inside the kernel); the rest of "
                                                                     "the per-launch time is what a launch costs (see empty_kernel)")
-        # the decode GEMV's own loads without its arithmetic: the matrix in the MFMA operand layout (an instruction touches 64 bytes of
-        # 16 rows), alone and with the 128 KB of vectors that every workgroup reads alike; span and per-launch time as above
+        # what loading a decode GEMV's matrix straight in the MFMA operand layout would cost (an instruction touches 64 bytes of
+        # 16 rows; the library's kernel reads 4 rows x 256 bytes per instruction instead and transposes in LDS), alone and with the
+        # 128 KB of vectors that every workgroup reads alike; span and per-launch time as above
         vecs = big2[:128 << 10]
         for label, vp_, nt_ in (("matrix_only_nontemporal", None, 1), ("matrix_only_plain_loads", None, 0), ("with_the_vectors_nontemporal", vecs.data_ptr(), 1),
                                 ("with_the_vectors_plain_loads", vecs.data_ptr(), 0)):

@@ -18,7 +18,7 @@
 //                       memory system needs for those bytes, without what a kernel launch costs around it
 //   ceil_empty          a kernel that does nothing: what one launch costs between two others
 //   ceil_xcc_ids        which XCD each workgroup of a launch runs on
-//   ceil_read_gemv_pattern  the decode GEMV's loads (matrix in the MFMA operand layout, the vectors every workgroup reads) without its arithmetic
+//   ceil_read_gemv_pattern  a decode GEMV's loads with the matrix straight in the MFMA operand layout (and the vectors every workgroup reads), no arithmetic
 //   ceil_copy_segments  a (rows, row_bytes) matrix copied in tiles of `seg` bytes x many rows, one
 //                       tile per 1024-thread workgroup, all loads of a tile before its stores: the
 //                       access pattern of the dim-1 kernels (layernorm, softmax) without arithmetic
@@ -135,10 +135,11 @@ __global__ __launch_bounds__(512) void k_read_span(const char* __restrict__ src,
     }
 }
 
-// The decode GEMV's memory traffic without its arithmetic: 40 rows of 4096 bytes per workgroup, wave w bytes
+// The memory traffic of a decode GEMV that loads its matrix straight in the MFMA operand layout (the library's kernel
+// does not: it reads 4 rows x 256 bytes per instruction), without the arithmetic: 40 rows of 4096 bytes per workgroup, wave w bytes
 // [512w, 512w + 512) of every row, lane (r, q) 16 bytes of row 16g + r -- the MFMA operand layout, in which an
 // instruction touches 64 bytes of 16 rows -- and, if VEC, the 128 KB every workgroup reads alike (32 vectors),
-// requested behind the first 16 rows like the kernel does.  NTL: non-temporal matrix loads.  Stamps as k_read_span.
+// requested behind the first 16 rows.  NTL: non-temporal matrix loads.  Stamps as k_read_span.
 template <int VEC, int NTL>
 __global__ __launch_bounds__(512) void k_read_gemv_pattern(const char* __restrict__ mat, const char* __restrict__ vec, int4_t* sink,
                                                            unsigned long long* stamps) {
