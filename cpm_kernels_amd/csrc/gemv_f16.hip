@@ -157,11 +157,12 @@ __global__ __launch_bounds__(256) void k_gemv_f16_transpose(int32_t dim_out, int
     }
 }
 
-// One matrix for one or two vectors (decode with a batch of one or two sequences), rows of 4096 halves: no
+// One matrix for one or two vectors (decode with a batch of one or two sequences), rows of PPL * 512 halves: no
 // matrix cores.  One workgroup of eight waves per compute unit; wave w takes rows w, w + 8, ... of the workgroup's
-// share, R of them.  A row is eight instructions of 1 KB in address order (16 bytes a lane); the loads of up to
-// three rows are in flight per wave (192 KB a compute unit), the next row's requested before a row is used.
-// Every lane keeps the vectors' halves at its positions in registers and multiplies with v_dot2_f32_f16 (fp32
+// share, R of them.  A row is PPL instructions of 1 KB in address order (16 bytes a lane); the loads of up to
+// three rows (two of the long ones) are in flight per wave, the next row's requested before a row is used.
+// Every lane keeps the vectors' halves at its positions in registers (in LDS, shared by the waves, when they
+// are more than 16 pieces) and multiplies with v_dot2_f32_f16 (fp32
 // sums, one chain per row and vector in a fixed order, so the result does not depend on timing); the lanes' sums
 // are added over the wave, and the outputs leave through LDS so that a vector's outputs are stored contiguously.
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
@@ -181,20 +182,35 @@ __device__ inline float wave_sum_f32_to_lane63(float v) {
     return v;                                                                                                       // the total: lane 63 only
 }
 
-template <int NV, int R>
+template <int NV, int PPL, int R>
 __global__ __launch_bounds__(512) void k_gemv_f16_rowwise(int32_t batch, int32_t dim_out, int32_t rpb, const half_t* __restrict__ mat,
                                                           const half_t* __restrict__ vec, half_t* __restrict__ out) {
-    constexpr int PPL = 8, DIN = PPL * 512, D = R < 3 ? R : 3;
+    constexpr int DIN = PPL * 512;
+    constexpr bool VLDS = NV * PPL > 16;           // the vectors' pieces in LDS instead of registers (rows of more than 4096 halves)
+    constexpr int D = VLDS ? (R < 2 ? R : 2) : (R < 3 ? R : 3);      // rows in flight per wave
     __shared__ float part[8 * R * NV];             // [row of the share][vector]
+    __shared__ __attribute__((aligned(16))) half8_t vlds[VLDS ? NV * PPL * 64 : 1];
     const int tid = threadIdx.x, lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int32_t row0 = blockIdx.x * rpb;
-    half8_t vf[NV][PPL];
+    // the vectors are requested first: they come from L2 and are there before the first row is
+    half8_t vf[VLDS ? 1 : NV][VLDS ? 1 : PPL];
+    constexpr int VPT = VLDS ? (NV * PPL * 64 + 511) / 512 : 1;     // pieces of the vectors a thread brings into LDS
+    half8_t vstage[VPT];
+    if constexpr (VLDS) {
 #pragma unroll
-    for (int v = 0; v < NV; ++v) {
-        const half_t* vp = vec + (uint32_t)min(v, batch - 1) * (uint32_t)DIN + lane * 8;
+        for (int j = 0; j < VPT; ++j) {
+            const int piece = tid + j * 512;       // piece = (v * PPL + i) * 64 + lane of the reader
+            const int v = piece / (PPL * 64), off = piece - v * (PPL * 64);
+            if (piece < NV * PPL * 64) vstage[j] = *reinterpret_cast<const half8_t*>(vec + (uint32_t)min(v, batch - 1) * (uint32_t)DIN + off * 8);
+        }
+    } else {
 #pragma unroll
-        for (int i = 0; i < PPL; ++i) vf[v][i] = *reinterpret_cast<const half8_t*>(vp + i * 512);
+        for (int v = 0; v < NV; ++v) {
+            const half_t* vp = vec + (uint32_t)min(v, batch - 1) * (uint32_t)DIN + lane * 8;
+#pragma unroll
+            for (int i = 0; i < PPL; ++i) vf[v][i] = *reinterpret_cast<const half8_t*>(vp + i * 512);
+        }
     }
     half8_t wf[D][PPL];
     auto request = [&](int r, half8_t (&buf)[PPL]) {
@@ -205,6 +221,12 @@ __global__ __launch_bounds__(512) void k_gemv_f16_rowwise(int32_t batch, int32_t
     };
 #pragma unroll
     for (int r = 0; r < D - 1; ++r) request(r, wf[r]);
+    if constexpr (VLDS) {
+#pragma unroll
+        for (int j = 0; j < VPT; ++j)
+            if (tid + j * 512 < NV * PPL * 64) vlds[tid + j * 512] = vstage[j];
+        __syncthreads();
+    }
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         if (r + D - 1 < R) request(r + D - 1, wf[(r + D - 1) % D]);
@@ -212,12 +234,15 @@ __global__ __launch_bounds__(512) void k_gemv_f16_rowwise(int32_t batch, int32_t
         for (int v = 0; v < NV; ++v) {
             float acc = 0.0f;
 #pragma unroll
-            for (int i = 0; i < PPL; ++i)
+            for (int i = 0; i < PPL; ++i) {
+                const half8_t a = wf[r % D][i];
+                half8_t b;
+                if constexpr (VLDS) b = vlds[(v * PPL + i) * 64 + lane];
+                else b = vf[v][i];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const half8_t a = wf[r % D][i], b = vf[v][i];
+                for (int e = 0; e < 4; ++e)
                     acc = __builtin_amdgcn_fdot2(half2_t{a[2 * e], a[2 * e + 1]}, half2_t{b[2 * e], b[2 * e + 1]}, acc, false);
-                }
+            }
             const float t = wave_sum_f32_to_lane63(acc);
             if (lane == 63) part[(r * 8 + w) * NV + v] = t;
         }
@@ -230,25 +255,34 @@ __global__ __launch_bounds__(512) void k_gemv_f16_rowwise(int32_t batch, int32_t
     }
 }
 
-// Takes the call when the shape fits the row-wise kernel: rows of 4096 halves, one or two vectors, 9 to 40 rows
-// per compute unit ([10240, 4096] and [4096, 4096] among them).
+// Takes the call when the shape fits the row-wise kernel: rows of 4096 or 10240 halves (the row lengths of the
+// model this path serves), one or two vectors, 9 to 40 rows per compute unit ([10240, 4096], [4096, 4096] and
+// [4096, 10240] among them).
 static bool launch_gemv_f16_rowwise(int32_t batch, int32_t dim_out, int32_t dim_in, const half_t* mat, const half_t* vec,
                                     half_t* out, hipStream_t st) {
-    if (batch > 2 || dim_in != 4096 || (int64_t)dim_out * dim_in * 2 >= (1ll << 32) || !aligned16(mat) || !aligned16(vec)) return false;
+    if (batch > 2 || (dim_in != 4096 && dim_in != 10240) || (int64_t)dim_out * dim_in * 2 >= (1ll << 32) || !aligned16(mat) || !aligned16(vec))
+        return false;
     const int64_t rpb = ceil_div(dim_out, compute_units());
     const int r = (int)ceil_div(rpb, 8);
     if (r < 2 || r > 5) return false;
     const dim3 grid((unsigned)ceil_div(dim_out, rpb));
     auto go = [&](auto kern) { hipLaunchKernelGGL(kern, grid, dim3(512), 0, st, batch, dim_out, (int32_t)rpb, mat, vec, out); };
-    auto pick = [&](auto nvc) {
-        constexpr int NV = decltype(nvc)::value;
-        if (r == 2) go(k_gemv_f16_rowwise<NV, 2>);
-        else if (r == 3) go(k_gemv_f16_rowwise<NV, 3>);
-        else if (r == 4) go(k_gemv_f16_rowwise<NV, 4>);
-        else go(k_gemv_f16_rowwise<NV, 5>);
+    auto pick = [&](auto nvc, auto pplc) {
+        constexpr int NV = decltype(nvc)::value, PPL = decltype(pplc)::value;
+        if (r == 2) go(k_gemv_f16_rowwise<NV, PPL, 2>);
+        else if (r == 3) go(k_gemv_f16_rowwise<NV, PPL, 3>);
+        else if (r == 4) go(k_gemv_f16_rowwise<NV, PPL, 4>);
+        else go(k_gemv_f16_rowwise<NV, PPL, 5>);
     };
-    if (batch == 1) pick(std::integral_constant<int, 1>{});
-    else pick(std::integral_constant<int, 2>{});
+    using I1 = std::integral_constant<int, 1>;
+    using I2 = std::integral_constant<int, 2>;
+    if (dim_in == 4096) {
+        if (batch == 1) pick(I1{}, std::integral_constant<int, 8>{});
+        else pick(I2{}, std::integral_constant<int, 8>{});
+    } else {
+        if (batch == 1) pick(I1{}, std::integral_constant<int, 20>{});
+        else pick(I2{}, std::integral_constant<int, 20>{});
+    }
     return true;
 }
 

@@ -1033,10 +1033,12 @@ def test_gemv_fp16_family(gpu, shape):
 
 
 @pytest.mark.parametrize("shape", [(1, 10240, 4096), (2, 10240, 4096), (1, 4096, 4096), (2, 4096, 4096), (2, 5000, 4096),
-                                   (1, 7777, 4096), (2, 2305, 4096), (1, 2304, 4096), (3, 10240, 4096)])
+                                   (1, 7777, 4096), (2, 2305, 4096), (1, 2304, 4096), (3, 10240, 4096),
+                                   # rows of 10240 halves (the vectors shared through LDS)
+                                   (1, 4096, 10240), (2, 4096, 10240), (1, 2305, 10240), (2, 7001, 10240), (1, 10240, 10240)])
 def test_gemv_broadcast_mat_fp16_one_or_two_vectors(gpu, shape):
     """The decode shapes with one or two vectors (cuda/gemv.cu:137-164 serves them with the same kernel as any
-    other batch): rows of 4096 halves go to a kernel without matrix cores from 9 rows per compute unit on;
+    other batch): rows of 4096 or 10240 halves go to a kernel without matrix cores from 9 rows per compute unit on;
     ragged last shares, the smallest and largest share, and the neighbours that stay on the matrix cores."""
     _name("gemv broadcast fp16, few vectors", shape)
     batch, dim_out, dim_in = shape
