@@ -971,7 +971,7 @@ F16_GEMM_CASES = [  # (batch, n, k, m) in the kernel's convention: out (batch, n
     # few rows (64 x 256 tiles) and many, ragged edges, one and several slabs of K
     (2, 64, 128, 264), (3, 40, 192, 1032), (2, 60, 128, 264), (2, 264, 320, 520), (1, 136, 64, 256), (2, 24, 64, 8),
     # one slab of K and several 256 x 256 tiles per workgroup (attention scores): whole tiles only, and ragged edges
-    (32, 512, 64, 768), (24, 520, 64, 776),
+    (32, 512, 64, 768), (24, 520, 64, 776), (40, 520, 128, 264), (36, 300, 192, 520),
     # several slabs of K and enough 256 x 256 tiles for every compute unit (the 16x16 MFMA form of the tile kernel)
     (48, 512, 256, 512), (50, 520, 320, 264),
     # more 128 x 128 tiles than compute units, at most two each (two workgroups per compute unit, two-stage ring)
