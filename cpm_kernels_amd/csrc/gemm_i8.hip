@@ -272,7 +272,10 @@ __device__ __forceinline__ void store_piece(int8_t* dst, int4_t v, int32_t left)
 // What the two forms of the tile function below share: the rows a wave's DMA instructions fetch, a slab's place in
 // the ring, what the last iterations of a tile fetch (the "tail"), and the priming of the ring at a tile's start.
 // BR x BC outputs per workgroup of NW waves, BKB bytes of K per slab, NST ring stages; LAY / F16 as in the tile functions.
-template <int BR, int BC, int BKB, int NW, int NST, int LAY, bool F16>
+// TSW: a (K, L) fp16 operand lands with the 32-byte units of every row of K exchanged among the four of a 128-byte
+// group (unit u of row k at u ^ (k & 3)), which is what keeps the transposing fragment reads of the 16x16 form free
+// of bank conflicts.  The DMA writes LDS in lane order, so the exchange happens in the choice of what a lane fetches.
+template <int BR, int BC, int BKB, int NW, int NST, int LAY, bool F16, bool TSW = false>
 struct SlabDma {
     static constexpr bool PT = (LAY & 1) != 0, QT = (LAY & 2) != 0;
     static constexpr int ESZ_IN = F16 ? 2 : 1;            // bytes per operand element
@@ -312,7 +315,9 @@ struct SlabDma {
             // a (K, L) operand: the instruction covers 1024 / (2 * B) rows of K, a lane one 16-byte piece of a row
             const int ppr = (q ? BC : BR) / EPP;                   // pieces per row of K
             const int dl = q ? dd - BR / RPI : dd;
-            const int kr = dl * (64 / ppr) + lane / ppr, pc = lane % ppr;
+            const int kr = dl * (64 / ppr) + lane / ppr;
+            const int pl = lane % ppr;                             // the piece's place in the row of K in LDS
+            const int pc = TSW ? ((((pl >> 1) ^ (kr & 3)) << 1) | (pl & 1)) : pl;      // ... and which piece of the row it is
             const int32_t L = q ? a.m : a.n;
             return ((uint32_t)kr * (uint32_t)L + (uint32_t)min((q ? oi : oj) + pc * EPP, L - EPP)) * (uint32_t)ESZ_IN;      // L % EPP == 0
         }
@@ -460,7 +465,8 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
     static_assert(KS >= 1, "k-steps of 64 bytes");
     constexpr int AR = TR * 2, AC = TC * 2;        // 16x16 MFMA tiles of a wave
     constexpr int NW = WR * WC, BR = WR * TR * 32, BC = WC * TC * 32;
-    using Dma = SlabDma<BR, BC, BKB, NW, NST, LAY, F16>;
+    constexpr bool TRP = PT && F16, TRQ = QT && F16;      // fragments of a (K, L) fp16 operand: transposing LDS reads
+    using Dma = SlabDma<BR, BC, BKB, NW, NST, LAY, F16, TRP || TRQ>;
     constexpr int STAGE = Dma::STAGE, CNT = Dma::CNT;      // bytes per ring stage; DMA instructions per wave and slab
     constexpr int RPW = 256 / BKB;                 // rows per 256-byte bank wrap
     const int tid = threadIdx.x, lane = tid & 63;
@@ -518,15 +524,35 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
     // its last MFMA of the second pass.
     constexpr int HC = AC / 2;
     int4_t fp[AR], fq[2][HC];
+    // Transposing reads (ds_read_b64_tr_b16): within 16 lanes, lane j hands in the address of four halves -- row of K
+    // k0 + j / 4, elements 4 (j % 4) .. + 3 of a block of 16 -- and lane i receives element i of rows k0 .. k0 + 3:
+    // four consecutive values of K for its own row of the MFMA operand, two reads per fragment instead of eight
+    // 2-byte ones.  Block u of row k lies at unit u ^ (k & 3) (SlabDma, TSW); the wave's first block is a multiple of
+    // four, so the exchange only touches the two low bits of the block's number: four lane-dependent offsets.
+    static_assert(!(TRP || TRQ) || ((TR * 2) % 4 == 0 && (TC * 2) % 4 == 0), "a wave's blocks start at a multiple of four");
+    int tro[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) tro[t] = ((t ^ (r16 >> 2)) << 5) + ((r16 & 3) << 3);
+    const int trk = q * 8 + (r16 >> 2);            // the row of K (within a k-step) this lane's first address names
+    auto tr_frag = [&](const int8_t* part, int rowlen, int ublock, int ks) __attribute__((always_inline)) {
+        // part: the operand's rows of K in the stage; rowlen: bytes per row of K; ublock: number of the block of 16 elements
+        const int8_t* p0 = part + (ks * 32 + trk) * rowlen + ((ublock & ~3) << 5) + tro[ublock & 3];
+        typedef short short4_t __attribute__((ext_vector_type(4)));
+        const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(uintptr_t)(lds_base + (uint32_t)(p0 - smem)));
+        const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(uintptr_t)(lds_base + (uint32_t)(p0 - smem) + 4 * rowlen));
+        return __builtin_bit_cast(int4_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    };
     auto lfragP = [&](auto ic, int stage, int ks) __attribute__((always_inline)) {
         constexpr int i = decltype(ic)::value;
-        if constexpr (PT) fp[i] = gather_k<F16, BR>(smem + stage * STAGE + offP0 + i * BLKP, ks);
+        if constexpr (TRP) fp[i] = tr_frag(smem + stage * STAGE, BR * 2, wr * TR * 2 + i, ks);
+        else if constexpr (PT) fp[i] = gather_k<F16, BR>(smem + stage * STAGE + offP0 + i * BLKP, ks);
         else fp[i] = *reinterpret_cast<const int4_t*>(smem + stage * STAGE + (offP0 ^ (ks << 6)) + i * BLKP);
     };
     auto lfragQ = [&](auto setc, auto jjc, int stage, int ks) __attribute__((always_inline)) {       // fragment jj of column half `set`
         constexpr int set = decltype(setc)::value, jj = decltype(jjc)::value;
         constexpr int j = set * HC + jj;
-        if constexpr (QT) fq[set][jj] = gather_k<F16, BC>(smem + stage * STAGE + offQ0 + j * BLKQ, ks);
+        if constexpr (TRQ) fq[set][jj] = tr_frag(smem + stage * STAGE + BR * BKB, BC * 2, wc * TC * 2 + j, ks);
+        else if constexpr (QT) fq[set][jj] = gather_k<F16, BC>(smem + stage * STAGE + offQ0 + j * BLKQ, ks);
         else fq[set][jj] = *reinterpret_cast<const int4_t*>(smem + stage * STAGE + (offQ0 ^ (ks << 6)) + j * BLKQ);
     };
     // One pass: the AR x HC MFMAs of column half `jh`, order pinned.  Between them the other set of column
