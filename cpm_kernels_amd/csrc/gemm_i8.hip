@@ -721,7 +721,8 @@ __device__ __forceinline__ bool gemm_dma_tile32(const GemmArgs& a, int8_t* smem,
     using acc_t = std::conditional_t<F16, float16_tv, int16_tv>;
     constexpr int KS = BKB / 32, CPR = BKB / 16;
     constexpr int NW = WR * WC, BR = WR * TR * 32, BC = WC * TC * 32;
-    using Dma = SlabDma<BR, BC, BKB, NW, NST, LAY, F16>;
+    constexpr bool TRP = PT && F16, TRQ = QT && F16;      // fragments of a (K, L) fp16 operand: transposing LDS reads
+    using Dma = SlabDma<BR, BC, BKB, NW, NST, LAY, F16, TRP || TRQ>;
     constexpr int STAGE = Dma::STAGE, CNT = Dma::CNT;      // bytes per ring stage; DMA instructions per wave and slab
     constexpr int NM = TR * TC;
     constexpr int RPW = 256 / BKB;                 // rows per 256-byte bank wrap
@@ -782,16 +783,40 @@ __device__ __forceinline__ bool gemm_dma_tile32(const GemmArgs& a, int8_t* smem,
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
     int4_t fp[2][TR], fq[2][TC];
+    // Transposing reads as in the 16x16 form.  Here a fragment is 32 rows x 8 values of K: the wave's four groups of
+    // 16 lanes are (rows 0-15 | 16-31) x (first | second half of the k-step's 16 values), so a group's block of 16
+    // rows is number 2 i + (group & 1) of the wave's, and its rows of K start at 8 (group >> 1).
+    static_assert(!(TRP || TRQ) || ((TR * 2) % 4 == 0 && (TC * 2) % 4 == 0), "a wave's blocks start at a multiple of four");
+    int tro[2];
+    {
+        const int jl = lane & 15, grp = lane >> 4;
+#pragma unroll
+        for (int t = 0; t < 2; ++t) tro[t] = (((2 * t + (grp & 1)) ^ (jl >> 2)) << 5) + ((jl & 3) << 3);
+    }
+    const int trk = (lane >> 5) * 8 + ((lane & 15) >> 2);
+    auto tr_frag = [&](const int8_t* part, int rowlen, int ublock0, auto ic, int ks) __attribute__((always_inline)) {
+        // part: the operand's rows of K in the stage; rowlen: bytes per row of K; ublock0: number of the wave's first block of 16 elements
+        constexpr int i = decltype(ic)::value;
+        const int8_t* p0 = part + (ks * 16 + trk) * rowlen + ((ublock0 + ((2 * i) & ~3)) << 5) + tro[i & 1];
+        typedef short short4_t __attribute__((ext_vector_type(4)));
+        const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(uintptr_t)(lds_base + (uint32_t)(p0 - smem)));
+        const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(uintptr_t)(lds_base + (uint32_t)(p0 - smem) + 4 * rowlen));
+        return __builtin_bit_cast(int4_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    };
     auto lfrag1 = [&](auto xc, auto bufc, int stage, int ks) __attribute__((always_inline)) {
         constexpr int x = decltype(xc)::value, buf = decltype(bufc)::value;
         if constexpr (x < TR) {
-            if constexpr (PT) {
+            if constexpr (TRP) {
+                fp[buf][x] = tr_frag(smem + stage * STAGE, BR * 2, wr * TR * 2, std::integral_constant<int, x>{}, ks);
+            } else if constexpr (PT) {
                 fp[buf][x] = gather_k32<F16, BR>(smem + stage * STAGE + offP[x], ks);
             } else {
                 fp[buf][x] = *reinterpret_cast<const int4_t*>(smem + stage * STAGE + (offP[x] ^ (ks << 5)));
             }
         } else {
-            if constexpr (QT) {
+            if constexpr (TRQ) {
+                fq[buf][x - TR] = tr_frag(smem + stage * STAGE + BR * BKB, BC * 2, wc * TC * 2, std::integral_constant<int, x - TR>{}, ks);
+            } else if constexpr (QT) {
                 fq[buf][x - TR] = gather_k32<F16, BC>(smem + stage * STAGE + offQ[x - TR], ks);
             } else {
                 fq[buf][x - TR] = *reinterpret_cast<const int4_t*>(smem + stage * STAGE + (offQ[x - TR] ^ (ks << 5)));
