@@ -231,30 +231,6 @@ __device__ __forceinline__ GemmItem gemm_item(uint32_t L, const DmaArgs& da) {
     return it;
 }
 
-// The 16 bytes of K one lane feeds to an MFMA, collected from a stage part that holds rows of K
-// with B elements each (an operand stored with K as the row index): eight 2-byte reads for fp16,
-// sixteen 1-byte reads for int8.  `p` points at the lane's element of the k-step's first row of K;
-// a k-step is 64 bytes of K (32 halves, 64 int8).
-template <bool F16, int B>
-__device__ __forceinline__ int4_t gather_k(const int8_t* p, int ks) {
-    if constexpr (F16) {
-        half8_t v;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = *reinterpret_cast<const half_t*>(p + (ks * 32 + e) * (B * 2));
-        return __builtin_bit_cast(int4_t, v);
-    } else {
-        uint32_t w[4];
-#pragma unroll
-        for (int d = 0; d < 4; ++d) {
-            uint32_t x = 0;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) x |= (uint32_t)(uint8_t)p[(ks * 64 + d * 4 + e) * B] << (8 * e);
-            w[d] = x;
-        }
-        return int4_t{(int32_t)w[0], (int32_t)w[1], (int32_t)w[2], (int32_t)w[3]};
-    }
-}
-
 // A 16-byte piece of an output row on its way to memory; `left` = elements from the piece's first to the end of
 // the row (a multiple of 4, at least 4).  int32 rows and fp16 rows of a multiple of 8 elements keep every piece
 // whole and 16-byte aligned.  fp16 rows of 8j + 4 elements are only 8-byte aligned from one row to the next and
@@ -272,9 +248,10 @@ __device__ __forceinline__ void store_piece(int8_t* dst, int4_t v, int32_t left)
 // What the two forms of the tile function below share: the rows a wave's DMA instructions fetch, a slab's place in
 // the ring, what the last iterations of a tile fetch (the "tail"), and the priming of the ring at a tile's start.
 // BR x BC outputs per workgroup of NW waves, BKB bytes of K per slab, NST ring stages; LAY / F16 as in the tile functions.
-// TSW: a (K, L) fp16 operand lands with the 32-byte units of every row of K exchanged among the four of a 128-byte
-// group (unit u of row k at u ^ (k & 3)), which is what keeps the transposing fragment reads of the 16x16 form free
-// of bank conflicts.  The DMA writes LDS in lane order, so the exchange happens in the choice of what a lane fetches.
+// TSW: a (K, L) operand lands with the units of every row of K exchanged within their 128-byte group -- fp16: unit
+// (32 bytes) u of row k at u ^ (k & 3); int8: unit (16 bytes) u at u ^ (k & 7) -- which is what keeps the transposing
+// fragment reads free of bank conflicts.  The DMA writes LDS in lane order, so the exchange happens in the choice of
+// what a lane fetches.
 template <int BR, int BC, int BKB, int NW, int NST, int LAY, bool F16, bool TSW = false>
 struct SlabDma {
     static constexpr bool PT = (LAY & 1) != 0, QT = (LAY & 2) != 0;
@@ -317,7 +294,7 @@ struct SlabDma {
             const int dl = q ? dd - BR / RPI : dd;
             const int kr = dl * (64 / ppr) + lane / ppr;
             const int pl = lane % ppr;                             // the piece's place in the row of K in LDS
-            const int pc = TSW ? ((((pl >> 1) ^ (kr & 3)) << 1) | (pl & 1)) : pl;      // ... and which piece of the row it is
+            const int pc = !TSW ? pl : F16 ? ((((pl >> 1) ^ (kr & 3)) << 1) | (pl & 1)) : (pl ^ (kr & 7));      // ... and which piece of the row it is
             const int32_t L = q ? a.m : a.n;
             return ((uint32_t)kr * (uint32_t)L + (uint32_t)min((q ? oi : oj) + pc * EPP, L - EPP)) * (uint32_t)ESZ_IN;      // L % EPP == 0
         }
@@ -450,8 +427,8 @@ struct StripOut {
 // LAY marks operands whose rows are K instead: bit 0 = the row operand is stored (K, n), bit 1 =
 // the column operand is stored (K, m).  Such an operand's part of a stage holds the slab's rows
 // of K (64 for fp16, 128 for int8) with the tile's BR (BC) elements each, DMA'd as they lie in
-// memory; a lane then collects its 16 bytes of K element by element (gather_k: 16 lanes read
-// contiguous bytes of one row, no bank conflicts) instead of with one 16-byte read.
+// memory (with the units of a row exchanged, SlabDma's TSW); a lane then gets its 16 bytes of K with two
+// transposing LDS reads instead of one 16-byte read.
 template <int WR, int WC, int TR, int TC, int BKB, int EPI, int NST, int LAY = 0>
 __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, int8_t* stg, uint32_t lds_base,
                                               const GemmItem cur_item, const GemmItem nxt_item, const bool have_slabs, int& ring) {
@@ -465,7 +442,7 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
     static_assert(KS >= 1, "k-steps of 64 bytes");
     constexpr int AR = TR * 2, AC = TC * 2;        // 16x16 MFMA tiles of a wave
     constexpr int NW = WR * WC, BR = WR * TR * 32, BC = WC * TC * 32;
-    constexpr bool TRP = PT && F16, TRQ = QT && F16;      // fragments of a (K, L) fp16 operand: transposing LDS reads
+    constexpr bool TRP = PT, TRQ = QT;             // fragments of a (K, L) operand: transposing LDS reads
     using Dma = SlabDma<BR, BC, BKB, NW, NST, LAY, F16, TRP || TRQ>;
     constexpr int STAGE = Dma::STAGE, CNT = Dma::CNT;      // bytes per ring stage; DMA instructions per wave and slab
     constexpr int RPW = 256 / BKB;                 // rows per 256-byte bank wrap
@@ -479,10 +456,10 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
     // fragment offsets of the wave's first block of 16 rows, k-step 0.  Step s reads logical chunk
     // 4s + q: xor (4s << 4) commutes with the swizzle; block i lies 16 rows further on, where the swizzle repeats.
     static_assert((16 / RPW) % CPR == 0, "the swizzle must repeat every 16 rows");
-    constexpr int BLKP = PT ? 16 * ESZ_IN : 16 * BKB, BLKQ = QT ? 16 * ESZ_IN : 16 * BKB;
+    constexpr int BLKP = 16 * BKB, BLKQ = 16 * BKB;        // (K-major operands; the others: tr_frag below)
     const int rp0 = wr * TR * 32 + r16, rq0 = wc * TC * 32 + r16;
-    const int offP0 = PT ? q * EPP * (BR * ESZ_IN) + rp0 * ESZ_IN : rp0 * BKB + ((q ^ swz(rp0)) << 4);
-    const int offQ0 = BR * BKB + (QT ? q * EPP * (BC * ESZ_IN) + rq0 * ESZ_IN : rq0 * BKB + ((q ^ swz(rq0)) << 4));
+    const int offP0 = rp0 * BKB + ((q ^ swz(rp0)) << 4);
+    const int offQ0 = BR * BKB + rq0 * BKB + ((q ^ swz(rq0)) << 4);
     // without slabs on their way the waits below count only loads: let the previous tile's stores finish first
     if (!have_slabs) wait_vmcnt<0>();
     Dma dma(a, lds_base, cur_item, nxt_item, wave, lane, ring);
@@ -524,35 +501,42 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
     // its last MFMA of the second pass.
     constexpr int HC = AC / 2;
     int4_t fp[AR], fq[2][HC];
-    // Transposing reads (ds_read_b64_tr_b16): within 16 lanes, lane j hands in the address of four halves -- row of K
-    // k0 + j / 4, elements 4 (j % 4) .. + 3 of a block of 16 -- and lane i receives element i of rows k0 .. k0 + 3:
-    // four consecutive values of K for its own row of the MFMA operand, two reads per fragment instead of eight
-    // 2-byte ones.  Block u of row k lies at unit u ^ (k & 3) (SlabDma, TSW); the wave's first block is a multiple of
-    // four, so the exchange only touches the two low bits of the block's number: four lane-dependent offsets.
-    static_assert(!(TRP || TRQ) || ((TR * 2) % 4 == 0 && (TC * 2) % 4 == 0), "a wave's blocks start at a multiple of four");
-    int tro[4];
-#pragma unroll
-    for (int t = 0; t < 4; ++t) tro[t] = ((t ^ (r16 >> 2)) << 5) + ((r16 & 3) << 3);
-    const int trk = q * 8 + (r16 >> 2);            // the row of K (within a k-step) this lane's first address names
+    // Transposing reads.  fp16 (ds_read_b64_tr_b16): within 16 lanes, lane j hands in the address of four halves -- row
+    // of K k0 + j / 4, elements 4 (j % 4) .. + 3 of a block of 16 -- and lane i receives element i of rows k0 .. k0 + 3:
+    // four consecutive values of K for its own row of the MFMA operand.  int8 (ds_read_b64_tr_b8): lane j hands in
+    // eight bytes -- row of K k0 + j / 2, elements 8 (j % 2) .. + 7 -- and lane i receives element i of rows k0 .. k0 + 7.
+    // Two reads per fragment either way, instead of eight 2-byte or sixteen 1-byte ones.  Block u (16 elements) of
+    // row k lies at unit u ^ (k & 3) resp. u ^ (k & 7) (SlabDma, TSW): an exclusive-or of the block's offset with a
+    // lane's constant.
+    constexpr int ULOG = F16 ? 5 : 4;              // log2 of a block's bytes
+    const int trx = F16 ? (r16 >> 2) << 5 : (r16 >> 1) << 4;                  // the exchange, as an offset
+    const int trb = F16 ? (r16 & 3) << 3 : (r16 & 1) << 3;                    // the lane's eight bytes within the block
+    const int trk = F16 ? q * 8 + (r16 >> 2) : q * 16 + (r16 >> 1);            // the row of K (within a k-step) this lane's first address names
     auto tr_frag = [&](const int8_t* part, int rowlen, int ublock, int ks) __attribute__((always_inline)) {
         // part: the operand's rows of K in the stage; rowlen: bytes per row of K; ublock: number of the block of 16 elements
-        const int8_t* p0 = part + (ks * 32 + trk) * rowlen + ((ublock & ~3) << 5) + tro[ublock & 3];
-        typedef short short4_t __attribute__((ext_vector_type(4)));
-        const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(uintptr_t)(lds_base + (uint32_t)(p0 - smem)));
-        const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(uintptr_t)(lds_base + (uint32_t)(p0 - smem) + 4 * rowlen));
-        return __builtin_bit_cast(int4_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        const uint32_t p0 = lds_base + (uint32_t)(part - smem) + (ks * (F16 ? 32 : 64) + trk) * rowlen + ((ublock << ULOG) ^ trx) + trb;
+        const uint32_t p1 = p0 + (F16 ? 4 : 8) * rowlen;
+        if constexpr (F16) {
+            typedef short short4_t __attribute__((ext_vector_type(4)));
+            const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(uintptr_t)p0);
+            const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(uintptr_t)p1);
+            return __builtin_bit_cast(int4_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        } else {
+            typedef int int2_tv __attribute__((ext_vector_type(2)));
+            const int2_tv lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) int2_tv*)(uintptr_t)p0);
+            const int2_tv hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) int2_tv*)(uintptr_t)p1);
+            return int4_t{lo.x, lo.y, hi.x, hi.y};
+        }
     };
     auto lfragP = [&](auto ic, int stage, int ks) __attribute__((always_inline)) {
         constexpr int i = decltype(ic)::value;
-        if constexpr (TRP) fp[i] = tr_frag(smem + stage * STAGE, BR * 2, wr * TR * 2 + i, ks);
-        else if constexpr (PT) fp[i] = gather_k<F16, BR>(smem + stage * STAGE + offP0 + i * BLKP, ks);
+        if constexpr (TRP) fp[i] = tr_frag(smem + stage * STAGE, BR * ESZ_IN, wr * TR * 2 + i, ks);
         else fp[i] = *reinterpret_cast<const int4_t*>(smem + stage * STAGE + (offP0 ^ (ks << 6)) + i * BLKP);
     };
     auto lfragQ = [&](auto setc, auto jjc, int stage, int ks) __attribute__((always_inline)) {       // fragment jj of column half `set`
         constexpr int set = decltype(setc)::value, jj = decltype(jjc)::value;
         constexpr int j = set * HC + jj;
-        if constexpr (TRQ) fq[set][jj] = tr_frag(smem + stage * STAGE + BR * BKB, BC * 2, wc * TC * 2 + j, ks);
-        else if constexpr (QT) fq[set][jj] = gather_k<F16, BC>(smem + stage * STAGE + offQ0 + j * BLKQ, ks);
+        if constexpr (TRQ) fq[set][jj] = tr_frag(smem + stage * STAGE + BR * BKB, BC * ESZ_IN, wc * TC * 2 + j, ks);
         else fq[set][jj] = *reinterpret_cast<const int4_t*>(smem + stage * STAGE + (offQ0 ^ (ks << 6)) + j * BLKQ);
     };
     // One pass: the AR x HC MFMAs of column half `jh`, order pinned.  Between them the other set of column
@@ -681,29 +665,6 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
     return ahead;
 }
 
-// The same for k-steps of 32 bytes (the 32x32 MFMAs): the 16 bytes of K one lane feeds to an MFMA, collected from a stage part that holds rows of K
-// with B elements each (an operand stored with K as the row index): eight 2-byte reads for fp16,
-// sixteen 1-byte reads for int8.  `p` points at the lane's element of the k-step's first row.
-template <bool F16, int B>
-__device__ __forceinline__ int4_t gather_k32(const int8_t* p, int ks) {
-    if constexpr (F16) {
-        half8_t v;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = *reinterpret_cast<const half_t*>(p + (ks * 16 + e) * (B * 2));
-        return __builtin_bit_cast(int4_t, v);
-    } else {
-        uint32_t w[4];
-#pragma unroll
-        for (int d = 0; d < 4; ++d) {
-            uint32_t x = 0;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) x |= (uint32_t)(uint8_t)p[(ks * 32 + d * 4 + e) * B] << (8 * e);
-            w[d] = x;
-        }
-        return int4_t{(int32_t)w[0], (int32_t)w[1], (int32_t)w[2], (int32_t)w[3]};
-    }
-}
-
 // The same tile with v_mfma_i32_32x32x32_i8 / v_mfma_f32_32x32x16_f16 (k-steps of 32 bytes, a wave owns
 // TR x TC tiles of 32x32, lane l holds output row l%32; both operands' fragments double buffered,
 // the barrier before the last k-step).  Used where a wave's share of a k-step is too small for the
@@ -716,8 +677,8 @@ __device__ __forceinline__ bool gemm_dma_tile32(const GemmArgs& a, int8_t* smem,
     constexpr bool FUSED = EPI == kEpiDequant, F16 = EPI == kEpiF16;
     constexpr bool PT = (LAY & 1) != 0, QT = (LAY & 2) != 0;
     static_assert(LAY == 0 || BKB == 128, "transposed operands: 128 bytes of K per slab");
+    static_assert(LAY == 0 || F16, "int8 operands stored (K, rows) run on the 16x16 form");
     constexpr int ESZ_IN = F16 ? 2 : 1;            // bytes per operand element
-    constexpr int EPP = 16 / ESZ_IN;               // elements per 16-byte piece
     using acc_t = std::conditional_t<F16, float16_tv, int16_tv>;
     constexpr int KS = BKB / 32, CPR = BKB / 16;
     constexpr int NW = WR * WC, BR = WR * TR * 32, BC = WC * TC * 32;
@@ -738,12 +699,12 @@ __device__ __forceinline__ bool gemm_dma_tile32(const GemmArgs& a, int8_t* smem,
 #pragma unroll
     for (int i = 0; i < TR; ++i) {
         const int r = wr * TR * 32 + i * 32 + lrow;
-        offP[i] = PT ? lk * EPP * (BR * ESZ_IN) + r * ESZ_IN : r * BKB + ((lk ^ swz(r)) << 4);
+        offP[i] = r * BKB + ((lk ^ swz(r)) << 4);          // (K-major operands; the others: tr_frag below)
     }
 #pragma unroll
     for (int j = 0; j < TC; ++j) {
         const int r = wc * TC * 32 + j * 32 + lrow;
-        offQ[j] = BR * BKB + (QT ? lk * EPP * (BC * ESZ_IN) + r * ESZ_IN : r * BKB + ((lk ^ swz(r)) << 4));
+        offQ[j] = BR * BKB + r * BKB + ((lk ^ swz(r)) << 4);
     }
     // without slabs on their way the waits below count only loads: let the previous tile's stores finish first
     if (!have_slabs) wait_vmcnt<0>();
@@ -808,16 +769,12 @@ __device__ __forceinline__ bool gemm_dma_tile32(const GemmArgs& a, int8_t* smem,
         if constexpr (x < TR) {
             if constexpr (TRP) {
                 fp[buf][x] = tr_frag(smem + stage * STAGE, BR * 2, wr * TR * 2, std::integral_constant<int, x>{}, ks);
-            } else if constexpr (PT) {
-                fp[buf][x] = gather_k32<F16, BR>(smem + stage * STAGE + offP[x], ks);
             } else {
                 fp[buf][x] = *reinterpret_cast<const int4_t*>(smem + stage * STAGE + (offP[x] ^ (ks << 5)));
             }
         } else {
             if constexpr (TRQ) {
                 fq[buf][x - TR] = tr_frag(smem + stage * STAGE + BR * BKB, BC * 2, wc * TC * 2, std::integral_constant<int, x - TR>{}, ks);
-            } else if constexpr (QT) {
-                fq[buf][x - TR] = gather_k32<F16, BC>(smem + stage * STAGE + offQ[x - TR], ks);
             } else {
                 fq[buf][x - TR] = *reinterpret_cast<const int4_t*>(smem + stage * STAGE + (offQ[x - TR] ^ (ks << 5)));
             }
