@@ -1137,7 +1137,7 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
         if (small > cus && small <= 2 * cus) return launch_dma<2, 2, 2, 1, 128, EPI, 2, 0, 32>(a, batch, st, 2);
         return launch_dma<2, 2, 2, 1, 128, EPI, kRingSmall, 0, 32>(a, batch, st);
     }
-    // an operand stored (K, rows): the tile kernel reads it as it lies and gathers the fragments byte by byte in LDS
+    // an operand stored (K, rows): the tile kernel reads it as it lies and takes the fragments with transposing LDS reads
     if (!(p_kmajor && q_kmajor) && wide && k > 0 && (k % 128 == 0) && aligned16(A) && aligned16(B) && (p_kmajor || n % 16 == 0) &&
         (q_kmajor || m % 16 == 0) && (int64_t)n * k < (1ll << 32) && (int64_t)m * k < (1ll << 32)) {
         constexpr int EPI = FUSED ? kEpiDequant : kEpiInt32;
@@ -1270,7 +1270,7 @@ static int gemm_f16_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, in
         if (mid > cus && mid <= 2 * cus) return launch_dma<2, 2, 2, 2, 128, kEpiF16, 2, 0, 32>(a, batch, st, 2);
         return launch_dma<2, 2, 2, 2, 128, kEpiF16, kRingSmall, 0, 32>(a, batch, st);
     }
-    // an operand stored (K, rows): the tile kernel reads it as it lies, with 2-byte LDS reads for the fragments
+    // an operand stored (K, rows): the tile kernel reads it as it lies, with transposing LDS reads for the fragments
     if (!(p_kmajor && q_kmajor) && wide && k > 0 && (k % 64 == 0) && aligned16(A) && aligned16(B) && (p_kmajor || n % 8 == 0) &&
         (q_kmajor || m % 8 == 0) && (int64_t)n * k * 2 < (1ll << 32) && (int64_t)m * k * 2 < (1ll << 32)) {
         const int lay = (p_kmajor ? 0 : 1) | (q_kmajor ? 0 : 2);
