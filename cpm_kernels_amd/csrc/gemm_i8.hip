@@ -263,6 +263,7 @@ struct SlabDma {
     static constexpr int RPI = 1024 / BKB;                // rows per DMA instruction
     static constexpr int NDMA = (BR + BC) / RPI;
     static_assert(NDMA % NW == 0, "stage must split evenly over the waves");
+    static_assert(!TSW || ((BR * ESZ_IN) % 128 == 0 && (BC * ESZ_IN) % 128 == 0), "the exchange of units stays inside whole 128-byte groups of a row of K");
     static constexpr int CNT = NDMA / NW;                 // DMA instructions per wave and slab
 
     const GemmArgs& a;
