@@ -678,12 +678,11 @@ __device__ __forceinline__ bool gemm_dma_tile32(const GemmArgs& a, int8_t* smem,
     constexpr bool FUSED = EPI == kEpiDequant, F16 = EPI == kEpiF16;
     constexpr bool PT = (LAY & 1) != 0, QT = (LAY & 2) != 0;
     static_assert(LAY == 0 || BKB == 128, "transposed operands: 128 bytes of K per slab");
-    static_assert(LAY == 0 || F16, "int8 operands stored (K, rows) run on the 16x16 form");
     constexpr int ESZ_IN = F16 ? 2 : 1;            // bytes per operand element
     using acc_t = std::conditional_t<F16, float16_tv, int16_tv>;
     constexpr int KS = BKB / 32, CPR = BKB / 16;
     constexpr int NW = WR * WC, BR = WR * TR * 32, BC = WC * TC * 32;
-    constexpr bool TRP = PT && F16, TRQ = QT && F16;      // fragments of a (K, L) fp16 operand: transposing LDS reads
+    constexpr bool TRP = PT, TRQ = QT;             // fragments of a (K, L) operand: transposing LDS reads
     using Dma = SlabDma<BR, BC, BKB, NW, NST, LAY, F16, TRP || TRQ>;
     constexpr int STAGE = Dma::STAGE, CNT = Dma::CNT;      // bytes per ring stage; DMA instructions per wave and slab
     constexpr int NM = TR * TC;
@@ -745,37 +744,42 @@ __device__ __forceinline__ bool gemm_dma_tile32(const GemmArgs& a, int8_t* smem,
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
     int4_t fp[2][TR], fq[2][TC];
-    // Transposing reads as in the 16x16 form.  Here a fragment is 32 rows x 8 values of K: the wave's four groups of
-    // 16 lanes are (rows 0-15 | 16-31) x (first | second half of the k-step's 16 values), so a group's block of 16
-    // rows is number 2 i + (group & 1) of the wave's, and its rows of K start at 8 (group >> 1).
-    static_assert(!(TRP || TRQ) || ((TR * 2) % 4 == 0 && (TC * 2) % 4 == 0), "a wave's blocks start at a multiple of four");
-    int tro[2];
-    {
-        const int jl = lane & 15, grp = lane >> 4;
-#pragma unroll
-        for (int t = 0; t < 2; ++t) tro[t] = (((2 * t + (grp & 1)) ^ (jl >> 2)) << 5) + ((jl & 3) << 3);
-    }
-    const int trk = (lane >> 5) * 8 + ((lane & 15) >> 2);
+    // Transposing reads as in the 16x16 form.  Here a fragment is 32 rows x 16 bytes of K: the wave's four groups of
+    // 16 lanes are (rows 0-15 | 16-31) x (first | second half of the k-step's 32 bytes), so a group's block of 16
+    // rows is number 2 i + (group & 1) of the wave's, and its rows of K start at 8 (fp16) or 16 (int8) times group >> 1.
+    constexpr int ULOG = F16 ? 5 : 4;              // log2 of a block's bytes
+    const int trj = lane & 15, trg = lane >> 4;
+    const int trx = F16 ? (trj >> 2) << 5 : (trj >> 1) << 4;                  // the exchange, as an offset
+    const int trb = F16 ? (trj & 3) << 3 : (trj & 1) << 3;                    // the lane's eight bytes within the block
+    const int trk = F16 ? (trg >> 1) * 8 + (trj >> 2) : (trg >> 1) * 16 + (trj >> 1);      // the row of K (within a k-step) of the lane's first address
     auto tr_frag = [&](const int8_t* part, int rowlen, int ublock0, auto ic, int ks) __attribute__((always_inline)) {
         // part: the operand's rows of K in the stage; rowlen: bytes per row of K; ublock0: number of the wave's first block of 16 elements
         constexpr int i = decltype(ic)::value;
-        const int8_t* p0 = part + (ks * 16 + trk) * rowlen + ((ublock0 + ((2 * i) & ~3)) << 5) + tro[i & 1];
-        typedef short short4_t __attribute__((ext_vector_type(4)));
-        const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(uintptr_t)(lds_base + (uint32_t)(p0 - smem)));
-        const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(uintptr_t)(lds_base + (uint32_t)(p0 - smem) + 4 * rowlen));
-        return __builtin_bit_cast(int4_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        const uint32_t p0 = lds_base + (uint32_t)(part - smem) + (ks * (F16 ? 16 : 32) + trk) * rowlen + (((ublock0 + 2 * i + (trg & 1)) << ULOG) ^ trx) + trb;
+        const uint32_t p1 = p0 + (F16 ? 4 : 8) * rowlen;
+        if constexpr (F16) {
+            typedef short short4_t __attribute__((ext_vector_type(4)));
+            const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(uintptr_t)p0);
+            const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4_t*)(uintptr_t)p1);
+            return __builtin_bit_cast(int4_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        } else {
+            typedef int int2_tv __attribute__((ext_vector_type(2)));
+            const int2_tv lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) int2_tv*)(uintptr_t)p0);
+            const int2_tv hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) int2_tv*)(uintptr_t)p1);
+            return int4_t{lo.x, lo.y, hi.x, hi.y};
+        }
     };
     auto lfrag1 = [&](auto xc, auto bufc, int stage, int ks) __attribute__((always_inline)) {
         constexpr int x = decltype(xc)::value, buf = decltype(bufc)::value;
         if constexpr (x < TR) {
             if constexpr (TRP) {
-                fp[buf][x] = tr_frag(smem + stage * STAGE, BR * 2, wr * TR * 2, std::integral_constant<int, x>{}, ks);
+                fp[buf][x] = tr_frag(smem + stage * STAGE, BR * ESZ_IN, wr * TR * 2, std::integral_constant<int, x>{}, ks);
             } else {
                 fp[buf][x] = *reinterpret_cast<const int4_t*>(smem + stage * STAGE + (offP[x] ^ (ks << 5)));
             }
         } else {
             if constexpr (TRQ) {
-                fq[buf][x - TR] = tr_frag(smem + stage * STAGE + BR * BKB, BC * 2, wc * TC * 2, std::integral_constant<int, x - TR>{}, ks);
+                fq[buf][x - TR] = tr_frag(smem + stage * STAGE + BR * BKB, BC * ESZ_IN, wc * TC * 2, std::integral_constant<int, x - TR>{}, ks);
             } else {
                 fq[buf][x - TR] = *reinterpret_cast<const int4_t*>(smem + stage * STAGE + (offQ[x - TR] ^ (ks << 5)));
             }
@@ -1142,10 +1146,13 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
     if (!(p_kmajor && q_kmajor) && wide && k > 0 && (k % 128 == 0) && aligned16(A) && aligned16(B) && (p_kmajor || n % 16 == 0) &&
         (q_kmajor || m % 16 == 0) && (int64_t)n * k < (1ll << 32) && (int64_t)m * k < (1ll << 32)) {
         constexpr int EPI = FUSED ? kEpiDequant : kEpiInt32;
+        // 256x256 tiles when they give most compute units a tile, else 128x128 (as for K-major operands)
+        const int64_t big = ceil_div(n, 256) * ceil_div(m, 256) * batch;
+        const bool large = big * 4 >= compute_units() * 3 && n > 128 && m > 128;
         switch ((p_kmajor ? 0 : 1) | (q_kmajor ? 0 : 2)) {
-            case 1: return launch_dma<2, 4, 4, 2, 128, EPI, 2, 1, 16>(a, batch, st);
-            case 2: return launch_dma<2, 4, 4, 2, 128, EPI, 2, 2, 16>(a, batch, st);
-            default: return launch_dma<2, 4, 4, 2, 128, EPI, 2, 3, 16>(a, batch, st);
+            case 1: return large ? launch_dma<2, 4, 4, 2, 128, EPI, 2, 1, 16>(a, batch, st) : launch_dma<2, 2, 2, 2, 128, EPI, kRingSmall, 1, 32>(a, batch, st);
+            case 2: return large ? launch_dma<2, 4, 4, 2, 128, EPI, 2, 2, 16>(a, batch, st) : launch_dma<2, 2, 2, 2, 128, EPI, kRingSmall, 2, 32>(a, batch, st);
+            default: return large ? launch_dma<2, 4, 4, 2, 128, EPI, 2, 3, 16>(a, batch, st) : launch_dma<2, 2, 2, 2, 128, EPI, kRingSmall, 3, 32>(a, batch, st);
         }
     }
     if (fast) {
@@ -1276,10 +1283,19 @@ static int gemm_f16_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, in
         (q_kmajor || m % 8 == 0) && (int64_t)n * k * 2 < (1ll << 32) && (int64_t)m * k * 2 < (1ll << 32)) {
         const int lay = (p_kmajor ? 0 : 1) | (q_kmajor ? 0 : 2);
         const bool low = n <= 64;                // 64 x 256 tiles for few output rows (attention: probabilities x values)
+        // else 256x256 tiles when they give most compute units a tile, else 128x128 (as for K-major operands)
+        const int64_t big = ceil_div(n, 256) * ceil_div(m, 256) * batch;
+        const bool large = big * 4 >= compute_units() * 3 && n > 128 && m > 128;
         switch (lay) {
-            case 1: return low ? launch_dma<1, 4, 2, 2, 128, kEpiF16, 3, 1, 32>(a, batch, st) : launch_dma<2, 4, 4, 2, 128, kEpiF16, 2, 1, 16>(a, batch, st);
-            case 2: return low ? launch_dma<1, 4, 2, 2, 128, kEpiF16, 3, 2, 32>(a, batch, st) : launch_dma<2, 4, 4, 2, 128, kEpiF16, 2, 2, 16>(a, batch, st);
-            default: return low ? launch_dma<1, 4, 2, 2, 128, kEpiF16, 3, 3, 32>(a, batch, st) : launch_dma<2, 4, 4, 2, 128, kEpiF16, 2, 3, 16>(a, batch, st);
+            case 1:
+                if (low) return launch_dma<1, 4, 2, 2, 128, kEpiF16, 3, 1, 32>(a, batch, st);
+                return large ? launch_dma<2, 4, 4, 2, 128, kEpiF16, 2, 1, 16>(a, batch, st) : launch_dma<2, 2, 2, 2, 128, kEpiF16, kRingSmall, 1, 32>(a, batch, st);
+            case 2:
+                if (low) return launch_dma<1, 4, 2, 2, 128, kEpiF16, 3, 2, 32>(a, batch, st);
+                return large ? launch_dma<2, 4, 4, 2, 128, kEpiF16, 2, 2, 16>(a, batch, st) : launch_dma<2, 2, 2, 2, 128, kEpiF16, kRingSmall, 2, 32>(a, batch, st);
+            default:
+                if (low) return launch_dma<1, 4, 2, 2, 128, kEpiF16, 3, 3, 32>(a, batch, st);
+                return large ? launch_dma<2, 4, 4, 2, 128, kEpiF16, 2, 3, 16>(a, batch, st) : launch_dma<2, 2, 2, 2, 128, kEpiF16, kRingSmall, 3, 32>(a, batch, st);
         }
     }
     for (int64_t r0 = 0; r0 < n; r0 += 65535ll * 64) {        // (rows beyond the grid's y dimension: several launches)

@@ -322,7 +322,9 @@ def test_gemm_int8_tile_kernels(gpu, case):
 
 # int8 operands with the contraction index as the row (the other three aT/bT combinations) on the tile kernel:
 # k % 128 == 0 and row lengths that are multiples of 16; ragged tiles, one to several slabs, batch broadcast.
-LAYOUT_CASES = [(1, 512, 256, 768), (2, 272, 128, 528), (1, 48, 384, 1040), (3, 1040, 640, 16), (1, 2304, 1024, 2064), (2, 2048, 256, 2560)]
+# (few 256 x 256 tiles: 128 x 128 tiles on the 32x32 form; enough of them for most compute units: the 16x16 form)
+LAYOUT_CASES = [(1, 512, 256, 768), (2, 272, 128, 528), (1, 48, 384, 1040), (3, 1040, 640, 16), (1, 2304, 1024, 2064), (2, 2048, 256, 2560),
+                (1, 4096, 256, 3088), (2, 3072, 128, 2064)]
 
 
 @pytest.mark.parametrize("case", LAYOUT_CASES)
