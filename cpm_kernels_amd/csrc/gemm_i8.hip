@@ -20,7 +20,7 @@
 //                  as whole 128-byte lines.
 //                  With template parameter LAY it also takes operands stored with K as the row index
 //                  (rows of whole 16-byte pieces), gathering the MFMA fragments element by element.
-//   k_gemm_kmajor  both operands K-major, k % 16 == 0: register-staged 64-byte K slabs.
+//   k_gemm_kmajor  both operands K-major, k % 16 == 0 (16-byte loads) or any k % 4 == 0 (4-byte loads): register-staged 64-byte K slabs.
 //   k_gemm_generic any layout and size: LDS tiles + v_dot4_i32_i8.
 // The tile kernel also serves the fp16 product of kernels/gemm.py:188-256 (cpmk_gemm_fp16): the
 // same bytes of K per lane feed v_mfma_f32_16x16x32_f16 / v_mfma_f32_32x32x16_f16, with fp32 accumulators.
@@ -50,7 +50,8 @@ constexpr int BK = 64;   // bytes of K per LDS stage
 // consecutive rows reading the same logical chunk then cover all 64 banks exactly once.
 __device__ inline int lds_off(int r, int c) { return r * BK + ((c ^ ((r >> 2) & 3)) << 4); }
 
-template <int WAVES_R, int WAVES_C, int TR, int TC, bool FUSED>
+// DW: rows that are only 4-byte aligned (k % 16 != 0): a 16-byte piece comes as four dwords, each zero past the end of K.
+template <int WAVES_R, int WAVES_C, int TR, int TC, bool FUSED, bool DW = false>
 __global__ __launch_bounds__(WAVES_R* WAVES_C * 64) void k_gemm_kmajor(GemmArgs a) {
     constexpr int NT = WAVES_R * WAVES_C * 64;
     constexpr int BR = WAVES_R * TR * 32;   // output rows per workgroup
@@ -84,22 +85,29 @@ __global__ __launch_bounds__(WAVES_R* WAVES_C * 64) void k_gemm_kmajor(GemmArgs 
 
     // global -> register staging: chunk id q = tid + s*NT -> row q/4, chunk q%4
     int4_t gp[CH_P], gq[CH_Q];
+    auto piece = [&](const int8_t* rowp, int32_t kc) __attribute__((always_inline)) {      // bytes [kc, kc + 16) of a row, zeros past K
+        int4_t v = {0, 0, 0, 0};
+        if constexpr (DW) {
+#pragma unroll
+            for (int d = 0; d < 4; ++d)
+                if (kc + 4 * d < K) v[d] = *reinterpret_cast<const int32_t*>(rowp + kc + 4 * d);
+        } else {
+            if (kc < K) v = *reinterpret_cast<const int4_t*>(rowp + kc);
+        }
+        return v;
+    };
     auto gload = [&](int32_t k0) {
 #pragma unroll
         for (int s = 0; s < CH_P; ++s) {
             const int q = tid + s * NT, r = q >> 2, c = q & 3;
-            const int32_t row = j0 + r, kc = k0 + c * 16;
-            int4_t v = {0, 0, 0, 0};
-            if (row < a.n && kc < K) v = *reinterpret_cast<const int4_t*>(P + (int64_t)row * K + kc);
-            gp[s] = v;
+            const int32_t row = j0 + r;
+            gp[s] = row < a.n ? piece(P + (int64_t)row * K, k0 + c * 16) : int4_t{0, 0, 0, 0};
         }
 #pragma unroll
         for (int s = 0; s < CH_Q; ++s) {
             const int q = tid + s * NT, r = q >> 2, c = q & 3;
-            const int32_t row = i0 + r, kc = k0 + c * 16;
-            int4_t v = {0, 0, 0, 0};
-            if (row < a.m && kc < K) v = *reinterpret_cast<const int4_t*>(Q + (int64_t)row * K + kc);
-            gq[s] = v;
+            const int32_t row = i0 + r;
+            gq[s] = row < a.m ? piece(Q + (int64_t)row * K, k0 + c * 16) : int4_t{0, 0, 0, 0};
         }
     };
     auto sstore = [&](int buf) {
@@ -1026,13 +1034,13 @@ __global__ __launch_bounds__(256) void k_gemm_generic(GemmArgs a, int p_kmajor, 
     }
 }
 
-template <int WAVES_R, int WAVES_C, int TR, int TC, bool FUSED>
+template <int WAVES_R, int WAVES_C, int TR, int TC, bool FUSED, bool DW = false>
 static int launch_kmajor(GemmArgs& a, int batch, hipStream_t st) {
     constexpr int BR = WAVES_R * TR * 32, BC = WAVES_C * TC * 32;
     constexpr int smem = 2 * (BR + BC) * BK;
     a.tiles_r = (int32_t)ceil_div(a.n, BR);
     a.tiles_c = (int32_t)ceil_div(a.m, BC);
-    auto kern = k_gemm_kmajor<WAVES_R, WAVES_C, TR, TC, FUSED>;
+    auto kern = k_gemm_kmajor<WAVES_R, WAVES_C, TR, TC, FUSED, DW>;
     static std::atomic<bool> lds_enabled[64];
     if (smem > 48 * 1024)
         if (int e = enable_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_enabled)) return e;
@@ -1159,6 +1167,13 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
         const int64_t t256 = ceil_div(n, 256) * ceil_div(m, 128) * batch;
         if (t256 >= 256) return launch_kmajor<2, 2, 4, 2, FUSED>(a, batch, st);
         return launch_kmajor<2, 2, 2, 2, FUSED>(a, batch, st);
+    }
+    // K-major rows that are only 4-byte aligned (k % 16 != 0; k % 4 == 0 always): the same kernel on 4-byte loads
+    if (p_kmajor && q_kmajor && k > 0 && batch <= 65535 && (reinterpret_cast<uintptr_t>(A) & 3u) == 0 && (reinterpret_cast<uintptr_t>(B) & 3u) == 0 &&
+        (FUSED ? (reinterpret_cast<uintptr_t>(out) & 1u) == 0 : (reinterpret_cast<uintptr_t>(out) & 3u) == 0)) {
+        const int64_t t256 = ceil_div(n, 256) * ceil_div(m, 128) * batch;
+        if (t256 >= 256) return launch_kmajor<2, 2, 4, 2, FUSED, true>(a, batch, st);
+        return launch_kmajor<2, 2, 2, 2, FUSED, true>(a, batch, st);
     }
     // output rows are the grid's y dimension (65535 tiles of 64 rows): taller products go out in several launches
     for (int64_t r0 = 0; r0 < n; r0 += 65535ll * 64) {
