@@ -39,6 +39,7 @@ struct GemmArgs {
     int32_t n, m, k;
     int32_t bc_row, bc_col;
     int32_t tiles_r, tiles_c;
+    int32_t edge_in;      // bit 0 / 1: the last row / column tile starts at n - BR / m - BC instead of reaching past the end
 };
 
 // ---------------------------------------------------------------------------------------
@@ -236,6 +237,11 @@ __device__ __forceinline__ GemmItem gemm_item(uint32_t L, const DmaArgs& da) {
     const uint32_t tin = t - g * group_sz;
     it.j0 = (int32_t)((g * GRP + tin % rows_in_group) * BR + (h & 1) * (BR / 2));
     it.i0 = (int32_t)((tin / rows_in_group) * BC);
+    // An operand stored (K, rows) whose rows are not whole 16-byte pieces cannot be read past the matrix's edge piece by
+    // piece: its last tile then lies inside the matrix and overlaps its neighbour, whose outputs it computes again
+    // (the same bits, stored twice).
+    if (da.g.edge_in & 1) it.j0 = min(it.j0, da.g.n - BR);
+    if (da.g.edge_in & 2) it.i0 = min(it.i0, da.g.m - BC);
     return it;
 }
 
@@ -1125,6 +1131,7 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
     a.strideQ = batchA == 1 ? 0 : (int64_t)m * k;
     a.n = n; a.m = m; a.k = k; a.bc_row = bcr; a.bc_col = bcc;
     a.tiles_r = a.tiles_c = 0;
+    a.edge_in = 0;
     // the tile kernel stores 16-byte pieces of output rows (8-byte halves where fp16 rows are not whole pieces: m % 8 == 4)
     const bool wide = aligned16(out);
     const bool p_kmajor = !bT, q_kmajor = aT != 0;
@@ -1151,12 +1158,16 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
         return launch_dma<2, 2, 2, 1, 128, EPI, kRingSmall, 0, 32>(a, batch, st);
     }
     // an operand stored (K, rows): the tile kernel reads it as it lies and takes the fragments with transposing LDS reads
-    if (!(p_kmajor && q_kmajor) && wide && k > 0 && (k % 128 == 0) && aligned16(A) && aligned16(B) && (p_kmajor || n % 16 == 0) &&
-        (q_kmajor || m % 16 == 0) && (int64_t)n * k < (1ll << 32) && (int64_t)m * k < (1ll << 32)) {
+    // (rows of such an operand that are not whole 16-byte pieces: tiles that stay inside the matrix, which takes a matrix of
+    // at least one tile)
+    const bool in_p = !p_kmajor && n % 16 != 0, in_q = !q_kmajor && m % 16 != 0;
+    if (!(p_kmajor && q_kmajor) && wide && k > 0 && (k % 128 == 0) && aligned16(A) && aligned16(B) && (!in_p || n >= 128) &&
+        (!in_q || m >= 128) && (int64_t)n * k < (1ll << 32) && (int64_t)m * k < (1ll << 32)) {
         constexpr int EPI = FUSED ? kEpiDequant : kEpiInt32;
         // 256x256 tiles when they give most compute units a tile, else 128x128 (as for K-major operands)
         const int64_t big = ceil_div(n, 256) * ceil_div(m, 256) * batch;
-        const bool large = big * 4 >= compute_units() * 3 && n > 128 && m > 128;
+        const bool large = big * 4 >= compute_units() * 3 && n > 128 && m > 128 && (!in_p || n >= 256) && (!in_q || m >= 256);
+        a.edge_in = (in_p ? 1 : 0) | (in_q ? 2 : 0);
         switch ((p_kmajor ? 0 : 1) | (q_kmajor ? 0 : 2)) {
             case 1: return large ? launch_dma<2, 4, 4, 2, 128, EPI, 2, 1, 16>(a, batch, st) : launch_dma<2, 2, 2, 2, 128, EPI, kRingSmall, 1, 32>(a, batch, st);
             case 2: return large ? launch_dma<2, 4, 4, 2, 128, EPI, 2, 2, 16>(a, batch, st) : launch_dma<2, 2, 2, 2, 128, EPI, kRingSmall, 2, 32>(a, batch, st);
@@ -1276,6 +1287,7 @@ static int gemm_f16_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, in
     a.strideQ = batchA == 1 ? 0 : (int64_t)m * k * 2;
     a.n = n; a.m = m; a.k = k * 2; a.bc_row = 0; a.bc_col = 0;
     a.tiles_r = a.tiles_c = 0;
+    a.edge_in = 0;
     const bool wide = aligned16(out) && m % 4 == 0;       // the tile kernel stores 16-byte pieces of output rows (8-byte halves where m % 8 == 4)
     const bool p_kmajor = !bT, q_kmajor = aT != 0;
     if (p_kmajor && q_kmajor && wide && k > 0 && (k % 64 == 0) && aligned16(A) && aligned16(B) &&
@@ -1294,13 +1306,18 @@ static int gemm_f16_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, in
         return launch_dma<2, 2, 2, 2, 128, kEpiF16, kRingSmall, 0, 32>(a, batch, st);
     }
     // an operand stored (K, rows): the tile kernel reads it as it lies, with transposing LDS reads for the fragments
-    if (!(p_kmajor && q_kmajor) && wide && k > 0 && (k % 64 == 0) && aligned16(A) && aligned16(B) && (p_kmajor || n % 8 == 0) &&
-        (q_kmajor || m % 8 == 0) && (int64_t)n * k * 2 < (1ll << 32) && (int64_t)m * k * 2 < (1ll << 32)) {
+    // (rows of such an operand that are not whole 16-byte pieces, but whole 8-byte ones: tiles that stay inside the matrix,
+    // which takes a matrix of at least one tile)
+    const bool in_p = !p_kmajor && n % 8 != 0, in_q = !q_kmajor && m % 8 != 0;
+    const bool low = n <= 64;                // 64 x 256 tiles for few output rows (attention: probabilities x values)
+    if (!(p_kmajor && q_kmajor) && wide && k > 0 && (k % 64 == 0) && aligned16(A) && aligned16(B) &&
+        (!in_p || (n % 4 == 0 && n >= 128)) && (!in_q || (m % 4 == 0 && m >= (low ? 256 : 128))) &&
+        (int64_t)n * k * 2 < (1ll << 32) && (int64_t)m * k * 2 < (1ll << 32)) {
         const int lay = (p_kmajor ? 0 : 1) | (q_kmajor ? 0 : 2);
-        const bool low = n <= 64;                // 64 x 256 tiles for few output rows (attention: probabilities x values)
         // else 256x256 tiles when they give most compute units a tile, else 128x128 (as for K-major operands)
         const int64_t big = ceil_div(n, 256) * ceil_div(m, 256) * batch;
-        const bool large = big * 4 >= compute_units() * 3 && n > 128 && m > 128;
+        const bool large = big * 4 >= compute_units() * 3 && n > 128 && m > 128 && (!in_p || n >= 256) && (!in_q || m >= 256);
+        a.edge_in = (in_p ? 1 : 0) | (in_q ? 2 : 0);
         switch (lay) {
             case 1:
                 if (low) return launch_dma<1, 4, 2, 2, 128, kEpiF16, 3, 1, 32>(a, batch, st);

@@ -324,7 +324,9 @@ def test_gemm_int8_tile_kernels(gpu, case):
 # k % 128 == 0 and row lengths that are multiples of 16; ragged tiles, one to several slabs, batch broadcast.
 # (few 256 x 256 tiles: 128 x 128 tiles on the 32x32 form; enough of them for most compute units: the 16x16 form)
 LAYOUT_CASES = [(1, 512, 256, 768), (2, 272, 128, 528), (1, 48, 384, 1040), (3, 1040, 640, 16), (1, 2304, 1024, 2064), (2, 2048, 256, 2560),
-                (1, 4096, 256, 3088), (2, 3072, 128, 2064)]
+                (1, 4096, 256, 3088), (2, 3072, 128, 2064),
+                # rows of a (K, rows) operand that are not whole 16-byte pieces (edge tiles that stay inside the matrix): small and large tiles
+                (1, 500, 256, 1004), (3, 500, 128, 7996), (2, 132, 128, 260)]
 
 
 @pytest.mark.parametrize("case", LAYOUT_CASES)
@@ -976,6 +978,9 @@ F16_GEMM_CASES = [  # (batch, n, k, m) in the kernel's convention: out (batch, n
     (32, 512, 64, 768), (24, 520, 64, 776), (40, 520, 128, 264), (36, 300, 192, 520),
     # several slabs of K and enough 256 x 256 tiles for every compute unit (the 16x16 MFMA form of the tile kernel)
     (48, 512, 256, 512), (50, 520, 320, 264),
+    # rows of a (K, rows) operand that are whole 8-byte but not whole 16-byte pieces (the reference's 500 x 7996 of tests/test_gemm.py:56):
+    # edge tiles that stay inside the matrix, small and large tiles, and the 64 x 256 tiles of few output rows
+    (2, 500, 128, 1004), (3, 500, 128, 7996), (2, 132, 64, 260), (4, 48, 192, 1004),
     # more 128 x 128 tiles than compute units, at most two each (two workgroups per compute unit, two-stage ring)
     (24, 512, 128, 512),
     # output rows of 8j + 4 halves on the tile kernels (8-byte stores): 128 x 128 tiles, and 256 x 256 on every compute unit
