@@ -1136,10 +1136,16 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
     const bool wide = aligned16(out);
     const bool p_kmajor = !bT, q_kmajor = aT != 0;
     const bool fast = p_kmajor && q_kmajor && k > 0 && (k % 16 == 0) && aligned16(A) && aligned16(B);
-    if (fast && wide && (k % 128 == 0) && (int64_t)n * k < (1ll << 32) && (int64_t)m * k < (1ll << 32)) {
+    if (fast && wide && (k % 64 == 0) && (int64_t)n * k < (1ll << 32) && (int64_t)m * k < (1ll << 32)) {
         // 256x256 tiles when they give most compute units a tile, else 128x128
         const int64_t big = ceil_div(n, 256) * ceil_div(m, 256) * batch;
         constexpr int EPI = FUSED ? kEpiDequant : kEpiInt32;
+        if (k % 128 != 0) {
+            // a depth of whole 64-byte but not whole 128-byte slabs (1600, 4544 ...): the same kernels on 64-byte slabs and
+            // a ring of four stages -- twice the barriers per byte of K, 5-10 % behind the 128-byte form
+            if (big * 4 >= compute_units() * 3 && n > 128 && m > 128) return launch_dma<2, 4, 4, 2, 64, EPI, 4, 0, 16>(a, batch, st);
+            return launch_dma<2, 2, 2, 2, 64, EPI, kRingSmall, 0, 32>(a, batch, st);
+        }
         // (a dimension of at most 128 would leave half or more of every 256-wide tile empty)
         if (big * 4 >= compute_units() * 3 && n > 128 && m > 128) return launch_dma<2, 4, 4, 2, 128, EPI, kRingBig, 0, 16>(a, batch, st);
         // 128x128 tiles, or 128x64 when even those leave a quarter of the compute units idle
@@ -1290,16 +1296,19 @@ static int gemm_f16_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, in
     a.edge_in = 0;
     const bool wide = aligned16(out) && m % 4 == 0;       // the tile kernel stores 16-byte pieces of output rows (8-byte halves where m % 8 == 4)
     const bool p_kmajor = !bT, q_kmajor = aT != 0;
-    if (p_kmajor && q_kmajor && wide && k > 0 && (k % 64 == 0) && aligned16(A) && aligned16(B) &&
+    if (p_kmajor && q_kmajor && wide && k > 0 && (k % 32 == 0) && aligned16(A) && aligned16(B) &&
         (int64_t)n * k * 2 < (1ll << 32) && (int64_t)m * k * 2 < (1ll << 32)) {
         const int64_t big = ceil_div(n, 256) * ceil_div(m, 256) * batch;
+        const bool whole128 = k % 64 == 0;       // the depth is whole 128-byte slabs (else whole 64-byte ones: 96, 160 ...)
         if (big * 4 >= compute_units() * 3 && n > 128 && m > 128) {
-            if (k >= 256) return launch_dma<2, 4, 4, 2, 128, kEpiF16, 2, 0, 16>(a, batch, st);
-            // Products of a few slabs -- attention scores, K = 64 -- are all prologue and epilogue, bound by the stores:
+            if (whole128 && k >= 256) return launch_dma<2, 4, 4, 2, 128, kEpiF16, 2, 0, 16>(a, batch, st);
+            // Products of a few slabs -- attention scores, K = 64 -- are all prologue and epilogue, bound by the stores (and
+            // depths of whole 64-byte slabs only need this form anyway):
             // the 32x32 form is quicker there, and waves of 64 rows x 128 columns, whose row segments are 256 bytes,
             // store 5-15 % faster than waves of 128 x 64 (slabs of 64 bytes make room for their wider output strips)
             return launch_dma<4, 2, 2, 4, 64, kEpiF16, 2, 0, 32>(a, batch, st);
         }
+        if (!whole128) return launch_dma<2, 2, 2, 2, 64, kEpiF16, kRingSmall, 0, 32>(a, batch, st);
         // (as for int8: more 128x128 tiles than compute units but at most two each -> two workgroups per compute unit)
         const int64_t mid = ceil_div(n, 128) * ceil_div(m, 128) * batch, cus = compute_units();
         if (mid > cus && mid <= 2 * cus) return launch_dma<2, 2, 2, 2, 128, kEpiF16, 2, 0, 32>(a, batch, st, 2);

@@ -308,6 +308,8 @@ TILE_CASES = [  # (batch, kernel n = output rows, k, kernel m = output columns)
     (1, 128, 128, 64), (1, 132, 128, 72), (1, 100, 256, 60), (3, 260, 384, 520), (1, 512, 128, 4096),
     (1, 520, 1152, 1032), (1, 1024, 896, 1028), (1, 640, 2048, 644), (4, 384, 512, 392), (1, 4100, 128, 2056),
     (1, 8, 128, 8), (1, 4, 256, 260), (2, 2816, 256, 2304), (1, 4096, 256, 3076), (2, 500, 1024, 1996), (1, 2052, 128, 4100),
+    # depths of whole 64-byte but not whole 128-byte slabs: large and small tiles, one slab to many
+    (1, 4096, 192, 3328), (1, 520, 448, 1032), (2, 132, 64, 72), (1, 2304, 1600, 2064), (3, 260, 320, 516),
 ]
 
 
@@ -978,6 +980,8 @@ F16_GEMM_CASES = [  # (batch, n, k, m) in the kernel's convention: out (batch, n
     (32, 512, 64, 768), (24, 520, 64, 776), (40, 520, 128, 264), (36, 300, 192, 520),
     # several slabs of K and enough 256 x 256 tiles for every compute unit (the 16x16 MFMA form of the tile kernel)
     (48, 512, 256, 512), (50, 520, 320, 264),
+    # depths of whole 64-byte but not whole 128-byte slabs (96, 160, 224 halves): large and small tiles
+    (32, 512, 96, 768), (2, 264, 160, 520), (3, 40, 224, 1032),
     # rows of a (K, rows) operand that are whole 8-byte but not whole 16-byte pieces (the reference's 500 x 7996 of tests/test_gemm.py:56):
     # edge tiles that stay inside the matrix, small and large tiles, and the 64 x 256 tiles of few output rows
     (2, 500, 128, 1004), (3, 500, 128, 7996), (2, 132, 64, 260), (4, 48, 192, 1004),
