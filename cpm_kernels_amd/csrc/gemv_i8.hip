@@ -27,7 +27,9 @@ namespace cpmk {
 // in piece j lane (r = l%16, q = l/16) reads bytes [j*64 + q*16, +16) of row r -- the four
 // lanes of a row read one contiguous 64-byte sector per instruction.  The vector operand uses
 // the same lane -> k assignment, which is all the MFMA needs.
-template <int NW, int RG, int NB>
+// DW: rows that are only 4-byte aligned (dim_in % 16 != 0): a lane's 16 bytes come as four dwords, each zero past the
+// end of k.
+template <int NW, int RG, int NB, bool DW = false>
 __global__ __launch_bounds__(NW * 64) void k_gemv_mfma(int32_t batch, int32_t dim_out, int32_t dim_in,
                                                        const half_t* __restrict__ scale_mat,
                                                        const int8_t* __restrict__ mat,
@@ -46,31 +48,33 @@ __global__ __launch_bounds__(NW * 64) void k_gemv_mfma(int32_t batch, int32_t di
         for (int t = 0; t < NB; ++t) acc[g][t] = int4_t{0, 0, 0, 0};
 
     const int nchunks = (dim_in + 255) >> 8;
+    auto piece = [&](const int8_t* rowp, int32_t k0) __attribute__((always_inline)) {      // bytes [k0, k0 + 16) of a row, zeros past dim_in
+        int4_t v = {0, 0, 0, 0};
+        if constexpr (DW) {
+#pragma unroll
+            for (int d = 0; d < 4; ++d)
+                if (k0 + 4 * d < dim_in) v[d] = *reinterpret_cast<const int32_t*>(rowp + k0 + 4 * d);
+        } else {
+            if (k0 < dim_in) v = *reinterpret_cast<const int4_t*>(rowp + k0);
+        }
+        return v;
+    };
     for (int c = w; c < nchunks; c += NW) {
         const int32_t kb = c * 256 + q * 16;
         int4_t wv[RG][4], vv[NB][4];
 #pragma unroll
         for (int g = 0; g < RG; ++g) {
             const int32_t row = row0 + g * 16 + r;
-            const int8_t* p = mat + (int64_t)row * dim_in + kb;
+            const int8_t* p = mat + (int64_t)min(row, dim_out - 1) * dim_in;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                int4_t v = {0, 0, 0, 0};
-                if (row < dim_out && kb + j * 64 < dim_in)
-                    v = *reinterpret_cast<const int4_t*>(p + j * 64);
-                wv[g][j] = v;
-            }
+            for (int j = 0; j < 4; ++j) wv[g][j] = row < dim_out ? piece(p, kb + j * 64) : int4_t{0, 0, 0, 0};
         }
 #pragma unroll
         for (int t = 0; t < NB; ++t) {
             const int32_t b = t * 16 + r;
-            const int8_t* p = vec + (int64_t)b * dim_in + kb;
+            const int8_t* p = vec + (int64_t)min(b, batch - 1) * dim_in;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                int4_t v = {0, 0, 0, 0};
-                if (b < batch && kb + j * 64 < dim_in) v = *reinterpret_cast<const int4_t*>(p + j * 64);
-                vv[t][j] = v;
-            }
+            for (int j = 0; j < 4; ++j) vv[t][j] = b < batch ? piece(p, kb + j * 64) : int4_t{0, 0, 0, 0};
         }
 #pragma unroll
         for (int j = 0; j < 4; ++j)
@@ -453,16 +457,16 @@ static bool launch_gemv_rowwise(int32_t batch, int32_t dim_out, int32_t dim_in, 
     return false;
 }
 
-template <int NB>
+template <int NB, bool DW = false>
 static void launch_mfma(int32_t batch, int32_t dim_out, int32_t dim_in, const half_t* sm, const int8_t* mat,
                         const half_t* sv, const int8_t* vec, half_t* out, hipStream_t st) {
     // 32 rows per workgroup halves the L2 traffic for the vectors; keep 16 when that
     // would leave compute units without a workgroup.
     if (dim_out >= 32 * 256) {
-        hipLaunchKernelGGL((k_gemv_mfma<8, 2, NB>), dim3((unsigned)ceil_div(dim_out, 32)), dim3(512), 0, st,
+        hipLaunchKernelGGL((k_gemv_mfma<8, 2, NB, DW>), dim3((unsigned)ceil_div(dim_out, 32)), dim3(512), 0, st,
                            batch, dim_out, dim_in, sm, mat, sv, vec, out);
     } else {
-        hipLaunchKernelGGL((k_gemv_mfma<8, 1, NB>), dim3((unsigned)ceil_div(dim_out, 16)), dim3(512), 0, st,
+        hipLaunchKernelGGL((k_gemv_mfma<8, 1, NB, DW>), dim3((unsigned)ceil_div(dim_out, 16)), dim3(512), 0, st,
                            batch, dim_out, dim_in, sm, mat, sv, vec, out);
     }
 }
@@ -508,6 +512,21 @@ extern "C" int cpmk_gemv_broadcast_mat_int8(int32_t batch, int32_t dim_out, int3
     half_t* O = (half_t*)out;
     const bool fast = dim_in > 0 && (dim_in % 16 == 0) && aligned16(mat) && aligned16(vec);
     if (!fast) {
+        if (dim_in > 0 && (reinterpret_cast<uintptr_t>(mat) & 3u) == 0 && (reinterpret_cast<uintptr_t>(vec) & 3u) == 0) {
+            // rows that are only 4-byte aligned (dim_in % 16 != 0, e.g. the 8888 of the reference's tests/test_gemv.py:12):
+            // the matrix-core kernel on 4-byte loads, up to 128 vectors per pass over the matrix
+            for (int32_t b0 = 0; b0 < batch; b0 += 128) {
+                const int32_t nb = batch - b0 < 128 ? batch - b0 : 128;
+                const int8_t* v = V + (int64_t)b0 * dim_in;
+                half_t* o = O + (int64_t)b0 * dim_out;
+                if (nb <= 16) launch_mfma<1, true>(nb, dim_out, dim_in, sm, M, sv + b0, v, o, st);
+                else if (nb <= 32) launch_mfma<2, true>(nb, dim_out, dim_in, sm, M, sv + b0, v, o, st);
+                else if (nb <= 64) launch_mfma<4, true>(nb, dim_out, dim_in, sm, M, sv + b0, v, o, st);
+                else launch_mfma<8, true>(nb, dim_out, dim_in, sm, M, sv + b0, v, o, st);
+                if (int e = launch_status()) return e;
+            }
+            return 0;
+        }
         hipLaunchKernelGGL(k_gemv_dot4, dim3((unsigned)ceil_div(dim_out, 4)), dim3(256), 0, st, batch, dim_out,
                            dim_in, sm, M, sv, V, O);
         return launch_status();
