@@ -253,6 +253,7 @@ __device__ __forceinline__ void wait_vmcnt() {
 
 // fp16 broadcast-matrix GEMV on the MFMA kernel of gemv_i8.hip (0, a HIP error code, or -1: shape not eligible)
 int gemv_f16_coalesced(int32_t batch, int32_t dim_out, int32_t dim_in, const void* mat, const void* vec, void* out, hipStream_t st);
+int gemv_f16_mfma(int32_t batch, int32_t dim_out, int32_t dim_in, const void* mat, const void* vec, void* out, hipStream_t st);
 
 // Compute units of the current device (cached per device ordinal; 256 if the query fails).  The cache
 // is atomic: host threads that make their first call together each ask the runtime and store the

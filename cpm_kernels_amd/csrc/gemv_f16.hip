@@ -356,6 +356,10 @@ int cpmk_gemv_broadcast_mat_fp16(int32_t batch, int32_t dim_out, int32_t dim_in,
         const int rc = gemv_f16_coalesced(batch, dim_out, dim_in, mat, vec, out, (hipStream_t)stream);
         if (rc >= 0) return rc;
     }
+    if (dim_in >= 128) {   // other row lengths: the predicated matrix-core kernel (short rows stay on the wave-per-row kernel below)
+        const int rc = gemv_f16_mfma(batch, dim_out, dim_in, mat, vec, out, (hipStream_t)stream);
+        if (rc >= 0) return rc;
+    }
     const int vec8 = (dim_in % 8 == 0) && aligned16(mat) && aligned16(vec);
     constexpr int NB = 8;               // vectors per pass over a matrix row
     const int64_t passes = ceil_div(batch, NB);

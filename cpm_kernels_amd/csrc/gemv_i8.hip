@@ -29,23 +29,28 @@ namespace cpmk {
 // the same lane -> k assignment, which is all the MFMA needs.
 // DW: rows that are only 4-byte aligned (dim_in % 16 != 0): a lane's 16 bytes come as four dwords, each zero past the
 // end of k.
-template <int NW, int RG, int NB, bool DW = false>
+// F16: the same on fp16 data (cpmk_gemv_broadcast_mat_fp16 with rows that are not whole 256-byte chunks): dim_in is the
+// row length in BYTES, a lane's 16 bytes are 8 halves of K for v_mfma_f32_16x16x32_f16, the accumulators are fp32 and
+// leave without scales; the waves' partial sums are added in wave order.
+template <int NW, int RG, int NB, bool DW = false, bool F16 = false>
 __global__ __launch_bounds__(NW * 64) void k_gemv_mfma(int32_t batch, int32_t dim_out, int32_t dim_in,
                                                        const half_t* __restrict__ scale_mat,
                                                        const int8_t* __restrict__ mat,
                                                        const half_t* __restrict__ scale_vec,
                                                        const int8_t* __restrict__ vec,
                                                        half_t* __restrict__ out) {
-    __shared__ int32_t part[RG * NB][256];   // cross-wave sums (LDS integer atomics)
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int r = lane & 15, q = lane >> 4;
     const int32_t row0 = blockIdx.x * (RG * 16);
 
-    int4_t acc[RG][NB];
+    using acc_t = std::conditional_t<F16, float4_t, int4_t>;
+    acc_t acc[RG][NB];
 #pragma unroll
     for (int g = 0; g < RG; ++g)
 #pragma unroll
-        for (int t = 0; t < NB; ++t) acc[g][t] = int4_t{0, 0, 0, 0};
+        for (int t = 0; t < NB; ++t)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[g][t][e] = 0;
 
     const int nchunks = (dim_in + 255) >> 8;
     auto piece = [&](const int8_t* rowp, int32_t k0) __attribute__((always_inline)) {      // bytes [k0, k0 + 16) of a row, zeros past dim_in
@@ -81,10 +86,37 @@ __global__ __launch_bounds__(NW * 64) void k_gemv_mfma(int32_t batch, int32_t di
 #pragma unroll
             for (int g = 0; g < RG; ++g)
 #pragma unroll
-                for (int t = 0; t < NB; ++t)
-                    acc[g][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wv[g][j], vv[t][j], acc[g][t], 0, 0, 0);
+                for (int t = 0; t < NB; ++t) {
+                    if constexpr (F16)
+                        acc[g][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, wv[g][j]), __builtin_bit_cast(half8_t, vv[t][j]),
+                                                                           acc[g][t], 0, 0, 0);
+                    else
+                        acc[g][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wv[g][j], vv[t][j], acc[g][t], 0, 0, 0);
+                }
     }
 
+    if constexpr (F16) {
+        // every wave leaves its partial sums in a slice of its own; the output threads add the NW slices in wave order
+        __shared__ float fslice[NW * RG * NB * 256];
+#pragma unroll
+        for (int g = 0; g < RG; ++g)
+#pragma unroll
+            for (int t = 0; t < NB; ++t)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) fslice[(w * RG * NB + g * NB + t) * 256 + (q * 4 + e) * 16 + r] = acc[g][t][e];
+        __syncthreads();
+        for (int idx = tid; idx < RG * NB * 256; idx += NW * 64) {
+            const int rr = idx % (RG * 16), bb = idx / (RG * 16);
+            const int g = rr >> 4, t = bb >> 4;
+            float sum = 0.0f;
+#pragma unroll
+            for (int ww = 0; ww < NW; ++ww) sum += fslice[(ww * RG * NB + g * NB + t) * 256 + (rr & 15) * 16 + (bb & 15)];
+            const int32_t row = row0 + rr;
+            if (row < dim_out && bb < batch) out[(int64_t)bb * dim_out + row] = (half_t)sum;
+        }
+        return;
+    }
+    __shared__ int32_t part[RG * NB][256];   // cross-wave sums (LDS integer atomics)
     for (int idx = tid; idx < RG * NB * 256; idx += NW * 64) (&part[0][0])[idx] = 0;
     __syncthreads();
     // accumulator e of lane l: matrix row (l/16)*4 + e, vector l%16 of the 16x16 tile
@@ -93,7 +125,7 @@ __global__ __launch_bounds__(NW * 64) void k_gemv_mfma(int32_t batch, int32_t di
 #pragma unroll
         for (int t = 0; t < NB; ++t)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) atomicAdd(&part[g * NB + t][(q * 4 + e) * 16 + r], acc[g][t][e]);
+            for (int e = 0; e < 4; ++e) atomicAdd(&part[g * NB + t][(q * 4 + e) * 16 + r], (int32_t)acc[g][t][e]);
     __syncthreads();
 
     // part[tile][row_in_tile*16 + b_in_tile]; thread -> (b, row) with row fastest so a
@@ -469,6 +501,36 @@ static void launch_mfma(int32_t batch, int32_t dim_out, int32_t dim_in, const ha
         hipLaunchKernelGGL((k_gemv_mfma<8, 1, NB, DW>), dim3((unsigned)ceil_div(dim_out, 16)), dim3(512), 0, st,
                            batch, dim_out, dim_in, sm, mat, sv, vec, out);
     }
+}
+
+// fp16 matrix with rows that are not whole 256-byte chunks, on the predicated MFMA kernel: rows of whole 16-byte pieces,
+// or (DW) of whole dwords.  Returns -1 when the buffers are not aligned for it.
+int gemv_f16_mfma(int32_t batch, int32_t dim_out, int32_t dim_in, const void* mat, const void* vec, void* out, hipStream_t st) {
+    const int64_t row_bytes = (int64_t)dim_in * 2;
+    if (dim_in <= 0 || row_bytes % 4 != 0 || row_bytes > 0x7fffffff || (reinterpret_cast<uintptr_t>(mat) & 3u) || (reinterpret_cast<uintptr_t>(vec) & 3u)) return -1;
+    const bool dw = row_bytes % 16 != 0 || !aligned16(mat) || !aligned16(vec);
+    const int8_t* M = (const int8_t*)mat;
+    for (int32_t b0 = 0; b0 < batch; b0 += 32) {           // (the fp32 slices of 32 vectors x 32 rows x 8 waves fill 64 KB of LDS)
+        const int32_t nb = batch - b0 < 32 ? batch - b0 : 32;
+        const int8_t* v = (const int8_t*)vec + (int64_t)b0 * row_bytes;
+        half_t* o = (half_t*)out + (int64_t)b0 * dim_out;
+        auto go = [&](auto nbc, auto dwc) {
+            constexpr int NB = decltype(nbc)::value;
+            constexpr bool DW = decltype(dwc)::value;
+            if (dim_out >= 32 * 256)
+                hipLaunchKernelGGL((k_gemv_mfma<8, 2, NB, DW, true>), dim3((unsigned)ceil_div(dim_out, 32)), dim3(512), 0, st, nb, dim_out,
+                                   (int32_t)row_bytes, nullptr, M, nullptr, v, o);
+            else
+                hipLaunchKernelGGL((k_gemv_mfma<8, 1, NB, DW, true>), dim3((unsigned)ceil_div(dim_out, 16)), dim3(512), 0, st, nb, dim_out,
+                                   (int32_t)row_bytes, nullptr, M, nullptr, v, o);
+        };
+        using I1 = std::integral_constant<int, 1>;
+        using I2 = std::integral_constant<int, 2>;
+        if (nb <= 16) { if (dw) go(I1{}, std::true_type{}); else go(I1{}, std::false_type{}); }
+        else { if (dw) go(I2{}, std::true_type{}); else go(I2{}, std::false_type{}); }
+        if (int e = launch_status()) return e;
+    }
+    return 0;
 }
 
 // fp16 matrix (dim_out, dim_in) shared by `batch` fp16 vectors on the MFMA kernel above.  Returns -1 when

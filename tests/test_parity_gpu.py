@@ -1016,7 +1016,10 @@ def test_gemm_fp16(gpu, case, aT, bT):
                                    (5, 70, 64), (2, 1000, 128), (3, 9, 8), (40, 300, 512), (33, 1100, 1024), (130, 48, 384),
                                    # short rows in numbers that put several loads in flight per lane (ragged ends, waves that
                                    # straddle two batch entries); a transposed product whose lanes leave the unrolled loop unevenly
-                                   (301, 1021, 64), (140, 1000, 128), (520, 1024, 24), (64, 64, 1000)])
+                                   (301, 1021, 64), (140, 1000, 128), (520, 1024, 24), (64, 64, 1000),
+                                   # rows of 128 halves and more that are not whole 256-byte chunks (the predicated matrix-core kernel for the
+                                   # shared matrix): whole 16-byte pieces, whole dwords only, more than 32 vectors
+                                   (5, 300, 200), (40, 1000, 2050), (3, 70, 130), (2, 600, 4544)])
 def test_gemv_fp16_family(gpu, shape):
     _name("gemv fp16", shape)
     batch, dim_out, dim_in = shape
