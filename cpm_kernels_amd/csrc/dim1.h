@@ -30,35 +30,70 @@ struct ColTile {
 // NTL / NTS: non-temporal loads / stores.  Only for tiles whose row segments are whole 128-byte cache
 // lines (LPR == 8) and for data that is not read again soon: a segment shorter than a line is completed
 // by a neighbouring workgroup, so it has to allocate in L2.
-template <int NT, int LPR, int R, bool NTL = false>
+//
+// UA: rows that are not whole 16-byte pieces, or buffers that are not 16-byte aligned (m % 8 != 0): the eight columns
+// of a piece come and go one by one, each checked against m.
+template <int NT, int LPR, int R, bool NTL = false, bool UA = false>
 __device__ inline void coltile_load(half8_t (&v)[R], const half_t* base, int32_t n, int32_t m, int32_t col0,
                                     half_t fill) {
     constexpr int RPP = NT / LPR;
     const int rg = threadIdx.x / LPR;
     const uint32_t off0 = (uint32_t)rg * (uint32_t)m + (uint32_t)col0, stride = (uint32_t)RPP * (uint32_t)m;
+    const bool pairs = UA && (m & 1) == 0 && (reinterpret_cast<uintptr_t>(base) & 3u) == 0;
 #pragma unroll
     for (int p = 0; p < R; ++p) {
         const int32_t row = p * RPP + rg;
         half8_t x;
 #pragma unroll
         for (int e = 0; e < 8; ++e) x[e] = fill;
-        if (row < n && col0 < m) {
-            const half8_t* src = reinterpret_cast<const half8_t*>(base + (off0 + p * stride));
-            x = NTL ? __builtin_nontemporal_load(src) : *src;
+        if constexpr (UA) {
+            if (row < n) {
+                if (pairs) {        // even m, 4-byte aligned buffer: two columns per access
+#pragma unroll
+                    for (int e = 0; e < 8; e += 2)
+                        if (col0 + e < m) {
+                            const half2_t t = *reinterpret_cast<const half2_t*>(base + (off0 + p * stride + e));
+                            x[e] = t[0];
+                            x[e + 1] = t[1];
+                        }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (col0 + e < m) x[e] = base[off0 + p * stride + e];
+                }
+            }
+        } else {
+            if (row < n && col0 < m) {
+                const half8_t* src = reinterpret_cast<const half8_t*>(base + (off0 + p * stride));
+                x = NTL ? __builtin_nontemporal_load(src) : *src;
+            }
         }
         v[p] = x;
     }
 }
 
-template <int NT, int LPR, int R, bool NTS = false>
+template <int NT, int LPR, int R, bool NTS = false, bool UA = false>
 __device__ inline void coltile_store(const half8_t (&v)[R], half_t* base, int32_t n, int32_t m, int32_t col0) {
     constexpr int RPP = NT / LPR;
     const int rg = threadIdx.x / LPR;
     const uint32_t off0 = (uint32_t)rg * (uint32_t)m + (uint32_t)col0, stride = (uint32_t)RPP * (uint32_t)m;
+    const bool pairs = UA && (m & 1) == 0 && (reinterpret_cast<uintptr_t>(base) & 3u) == 0;
 #pragma unroll
     for (int p = 0; p < R; ++p) {
         const int32_t row = p * RPP + rg;
-        if (row < n && col0 < m) {
+        if constexpr (UA) {
+            if (row < n) {
+                if (pairs) {
+#pragma unroll
+                    for (int e = 0; e < 8; e += 2)
+                        if (col0 + e < m) *reinterpret_cast<half2_t*>(base + (off0 + p * stride + e)) = half2_t{v[p][e], v[p][e + 1]};
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (col0 + e < m) base[off0 + p * stride + e] = v[p][e];
+                }
+            }
+        } else if (row < n && col0 < m) {
             half8_t* dst = reinterpret_cast<half8_t*>(base + (off0 + p * stride));
             if (NTS) __builtin_nontemporal_store(v[p], dst);
             else *dst = v[p];

@@ -25,7 +25,9 @@ __device__ inline half8_t affine8(half8_t y, half_t a, half_t b, bool has_beta) 
 // Single pass: the whole (n x LPR*8) column tile lives in registers.  Tiles of whole cache lines (LPR == 8) are
 // read and written with the non-temporal hint: every byte is touched once (8 x 4096 x 512 through the team
 // kernel: 17.2 -> 15.2 us).
-template <int NT, int LPR, int R, bool AFF>
+// MODE 0: 16-byte accesses, non-temporal where a tile's row segments are whole cache lines; 1: 16-byte accesses without
+// the hint (rows that do not start on 128-byte boundaries); 2: any m and alignment, element by element (dim1.h).
+template <int NT, int LPR, int R, bool AFF, int MODE = 0>
 __global__ __launch_bounds__(NT) void k_layernorm_tile(int32_t n, int32_t m, int32_t tiles_per_batch,
                                                        const half_t* mat, half_t* out,
                                                        const half_t* __restrict__ alpha,
@@ -53,7 +55,7 @@ __global__ __launch_bounds__(NT) void k_layernorm_tile(int32_t n, int32_t m, int
         }
     }
     half8_t v[R];
-    coltile_load<NT, LPR, R, LPR == 8>(v, mat + boff, n, m, col0, (half_t)0.0f);
+    coltile_load<NT, LPR, R, LPR == 8 && MODE == 0, MODE == 2>(v, mat + boff, n, m, col0, (half_t)0.0f);
     if constexpr (AFF) {
 #pragma unroll
         for (int i = 0; i < CPT; ++i) {
@@ -99,7 +101,7 @@ __global__ __launch_bounds__(NT) void k_layernorm_tile(int32_t n, int32_t m, int
         if constexpr (AFF) y = affine8(y, coef[0][p * T::RPP + rg], coef[1][p * T::RPP + rg], beta != nullptr);
         v[p] = y;
     }
-    coltile_store<NT, LPR, R, LPR == 8>(v, out + boff, n, m, col0);
+    coltile_store<NT, LPR, R, LPR == 8 && MODE == 0, MODE == 2>(v, out + boff, n, m, col0);
 }
 
 // Tall columns.  A register tile holds T::ROWS rows of 64 columns (128-byte row segments, whole
@@ -108,7 +110,7 @@ __global__ __launch_bounds__(NT) void k_layernorm_tile(int32_t n, int32_t m, int
 // each keeps its own rows in registers, posts its partial column sums, adds up the team's
 // partials in part order (so the result does not depend on timing) and normalises its rows.
 // A workgroup reads and writes only its own rows: out may alias mat.
-template <int NT, int R, bool AFF>
+template <int NT, int R, bool AFF, int MODE = 0>
 __global__ __launch_bounds__(NT) void k_layernorm_team(int32_t n, int32_t m, int32_t tiles_per_batch, int32_t parts,
                                                        const half_t* mat, half_t* out,
                                                        const half_t* __restrict__ alpha,
@@ -146,7 +148,7 @@ __global__ __launch_bounds__(NT) void k_layernorm_team(int32_t n, int32_t m, int
         if (beta != nullptr) cb = beta[row];
     }
     half8_t v[R];
-    coltile_load<NT, LPR, R, true>(v, mat + boff, own_n, m, col0, (half_t)0.0f);
+    coltile_load<NT, LPR, R, MODE == 0, MODE == 2>(v, mat + boff, own_n, m, col0, (half_t)0.0f);
     if constexpr (AFF) {
         coef[0][tid] = ca;
         coef[1][tid] = cb;
@@ -208,7 +210,7 @@ __global__ __launch_bounds__(NT) void k_layernorm_team(int32_t n, int32_t m, int
         if constexpr (AFF) y = affine8(y, coef[0][p * T::RPP + rg], coef[1][p * T::RPP + rg], beta != nullptr);
         v[p] = y;
     }
-    coltile_store<NT, LPR, R, true>(v, out + boff, own_n, m, col0);
+    coltile_store<NT, LPR, R, MODE == 0, MODE == 2>(v, out + boff, own_n, m, col0);
     if (tid < 64) xch_retire(xl, team, parts);     // after the barrier above: this workgroup holds all it needs
 }
 
@@ -277,26 +279,26 @@ __global__ __launch_bounds__(256) void k_layernorm_rows(int32_t n, const half_t*
     for (int32_t i = threadIdx.x; i < n; i += 256) o[i] = round_f16(((float)p[i] - mean) * rstd);
 }
 
-template <int LPR, int R>
+template <int LPR, int R, int MODE = 0>
 static void launch_tile(int32_t batch, int32_t n, int32_t m, const half_t* mat, half_t* out, const half_t* alpha,
                         const half_t* beta, float eps, int rd_mean, hipStream_t st) {
     constexpr int NT = 1024;
     const int32_t tiles = (int32_t)ceil_div(m, LPR * 8);
     if (alpha != nullptr)
-        hipLaunchKernelGGL((k_layernorm_tile<NT, LPR, R, true>), dim3((unsigned)((int64_t)tiles * batch)), dim3(NT), 0, st, n,
+        hipLaunchKernelGGL((k_layernorm_tile<NT, LPR, R, true, MODE>), dim3((unsigned)((int64_t)tiles * batch)), dim3(NT), 0, st, n,
                            m, tiles, mat, out, alpha, beta, eps, rd_mean);
     else
-        hipLaunchKernelGGL((k_layernorm_tile<NT, LPR, R, false>), dim3((unsigned)((int64_t)tiles * batch)), dim3(NT), 0, st, n,
+        hipLaunchKernelGGL((k_layernorm_tile<NT, LPR, R, false, MODE>), dim3((unsigned)((int64_t)tiles * batch)), dim3(NT), 0, st, n,
                            m, tiles, mat, out, alpha, beta, eps, rd_mean);
 }
 
-template <int LPR>
+template <int LPR, int MODE = 0>
 static bool launch_tile_r(int r, int32_t batch, int32_t n, int32_t m, const half_t* mat, half_t* out,
                           const half_t* alpha, const half_t* beta, float eps, int rd_mean, hipStream_t st) {
-    if (r <= 1) launch_tile<LPR, 1>(batch, n, m, mat, out, alpha, beta, eps, rd_mean, st);
-    else if (r <= 2) launch_tile<LPR, 2>(batch, n, m, mat, out, alpha, beta, eps, rd_mean, st);
-    else if (r <= 4) launch_tile<LPR, 4>(batch, n, m, mat, out, alpha, beta, eps, rd_mean, st);
-    else if (r <= 8) launch_tile<LPR, 8>(batch, n, m, mat, out, alpha, beta, eps, rd_mean, st);
+    if (r <= 1) launch_tile<LPR, 1, MODE>(batch, n, m, mat, out, alpha, beta, eps, rd_mean, st);
+    else if (r <= 2) launch_tile<LPR, 2, MODE>(batch, n, m, mat, out, alpha, beta, eps, rd_mean, st);
+    else if (r <= 4) launch_tile<LPR, 4, MODE>(batch, n, m, mat, out, alpha, beta, eps, rd_mean, st);
+    else if (r <= 8) launch_tile<LPR, 8, MODE>(batch, n, m, mat, out, alpha, beta, eps, rd_mean, st);
     else return false;
     return true;
 }
@@ -318,10 +320,15 @@ static int layernorm_dispatch(int32_t batch, int32_t n, int32_t m, const void* m
         hipLaunchKernelGGL(k_layernorm_rows, dim3((unsigned)batch), dim3(256), 0, st, n, x, y, eps, rd_mean);
         return launch_status();
     }
-    if (m % 8 == 0 && aligned16(mat) && aligned16(out) && (int64_t)n * m < (1ll << 31)) {
+    // rows of whole 16-byte pieces in 16-byte aligned buffers: 16-byte accesses; any other width or alignment: the same
+    // kernels (64-column tiles only) moving their tiles element by element
+    const bool wide = m % 8 == 0 && aligned16(mat) && aligned16(out);
+    // the 128-byte row segments of the 64-column tiles are whole cache lines: the non-temporal hint pays there only
+    const bool lines = m % 64 == 0 && (reinterpret_cast<uintptr_t>(mat) & 127u) == 0 && (reinterpret_cast<uintptr_t>(out) & 127u) == 0;
+    if ((int64_t)n * m < (1ll << 31) && (wide || m > 1)) {
         // widest row segment whose tile still fits the register budget (at most 8 pieces per lane)
         bool ok = false;
-        if (n > 128 * 8 && m >= 64) {
+        if (n > 128 * 8 && (m >= 64 || !wide)) {
             // tall columns: 64-column tiles, the rows split over a team of workgroups
             const int64_t tiles = ceil_div(m, 64);
             // 1024 rows a part (one 1024-thread workgroup per compute unit) while those parts fit the chip in
@@ -356,13 +363,19 @@ static int layernorm_dispatch(int32_t batch, int32_t n, int32_t m, const void* m
                         hipLaunchKernelGGL(kern, grid, dim3(threads), 0, st, n, m, (int32_t)tiles, (int32_t)parts, xb, yb, al, be, eps,
                                            rd_mean, (uint32_t)(tiles * nb), xl);
                     };
-                    if (big) {
-                        if (al != nullptr) go(k_layernorm_team<1024, 8, true>, 1024);
-                        else go(k_layernorm_team<1024, 8, false>, 1024);
-                    } else {
-                        if (al != nullptr) go(k_layernorm_team<512, 8, true>, 512);
-                        else go(k_layernorm_team<512, 8, false>, 512);
-                    }
+                    auto pick = [&](auto modec) {
+                        constexpr int MODE = decltype(modec)::value;
+                        if (big) {
+                            if (al != nullptr) go(k_layernorm_team<1024, 8, true, MODE>, 1024);
+                            else go(k_layernorm_team<1024, 8, false, MODE>, 1024);
+                        } else {
+                            if (al != nullptr) go(k_layernorm_team<512, 8, true, MODE>, 512);
+                            else go(k_layernorm_team<512, 8, false, MODE>, 512);
+                        }
+                    };
+                    if (!wide) pick(std::integral_constant<int, 2>{});
+                    else if (lines) pick(std::integral_constant<int, 0>{});
+                    else pick(std::integral_constant<int, 1>{});
                     const int e = launch_status();
                     const int rc2 = xs.end();
                     if (e != 0 || rc2 != 0) return e ? e : rc2;
@@ -370,7 +383,9 @@ static int layernorm_dispatch(int32_t batch, int32_t n, int32_t m, const void* m
                 if (!no_slots) return 0;
             }
         }
-        if (n <= 128 * 8 && m >= 64) ok = launch_tile_r<8>((int)ceil_div(n, 128), batch, n, m, x, y, al, be, eps, rd_mean, st);
+        if (!wide) ok = n <= 128 * 8 && launch_tile_r<8, 2>((int)ceil_div(n, 128), batch, n, m, x, y, al, be, eps, rd_mean, st);
+        else if (n <= 128 * 8 && m >= 64 && !lines) ok = launch_tile_r<8, 1>((int)ceil_div(n, 128), batch, n, m, x, y, al, be, eps, rd_mean, st);
+        else if (n <= 128 * 8 && m >= 64) ok = launch_tile_r<8>((int)ceil_div(n, 128), batch, n, m, x, y, al, be, eps, rd_mean, st);
         else if (n <= 256 * 8 && m >= 32) ok = launch_tile_r<4>((int)ceil_div(n, 256), batch, n, m, x, y, al, be, eps, rd_mean, st);
         else ok = launch_tile_r<2>((int)ceil_div(n, 512), batch, n, m, x, y, al, be, eps, rd_mean, st);
         if (ok) return launch_status();
