@@ -65,7 +65,9 @@ __device__ __forceinline__ void softmax_cols(half8_t (&v)[R], float* lds) {
 // multiply-add and one exp2 per element, and a 16-byte piece whose 8 inputs are all -inf for
 // every lane of the wave (whole rows masked out, as in causal attention) is skipped -- its
 // exponentials are exactly 0.
-template <int NT, int LPR, int R>
+// MODE 0: 16-byte accesses, non-temporal where a tile's row segments are whole cache lines; 1: 16-byte accesses without
+// the hint (rows that do not start on 128-byte boundaries); 2: any m and alignment, element by element (dim1.h).
+template <int NT, int LPR, int R, int MODE = 0>
 __global__ __launch_bounds__(NT) void k_softmax_tile(int32_t n, int32_t m, int32_t tiles_per_batch,
                                                      const half_t* inp, half_t* out) {
     using T = ColTile<NT, LPR, R>;
@@ -76,10 +78,10 @@ __global__ __launch_bounds__(NT) void k_softmax_tile(int32_t n, int32_t m, int32
     const int64_t boff = (int64_t)b * n * m;
 
     half8_t v[R];
-    coltile_load<NT, LPR, R, LPR == 8>(v, inp + boff, n, m, col0, (half_t)(-__builtin_inff()));
+    coltile_load<NT, LPR, R, LPR == 8 && MODE == 0, MODE == 2>(v, inp + boff, n, m, col0, (half_t)(-__builtin_inff()));
 
     softmax_cols<NT, LPR, R>(v, lds);
-    coltile_store<NT, LPR, R, LPR == 8>(v, out + boff, n, m, col0);
+    coltile_store<NT, LPR, R, LPR == 8 && MODE == 0, MODE == 2>(v, out + boff, n, m, col0);
 }
 
 // The same for many tiles per compute unit: persistent workgroups, each wave fetching its share
@@ -177,7 +179,7 @@ __global__ __launch_bounds__(NT) void k_softmax_stream(int32_t n, int32_t m, int
 // -1e6 like M itself) and the exponentials and their sum s_p relative to m_p, posts (m_p, s_p),
 // and rescales by exp(m_p - M) / S with M = max_p m_p and S = sum_p s_p exp(m_p - M) + 1e-10,
 // which is the single-workgroup result up to two extra fp32 roundings.
-template <int NT, int R>
+template <int NT, int R, int MODE = 0>
 __global__ __launch_bounds__(NT) void k_softmax_team(int32_t n, int32_t m, int32_t tiles_per_batch, int32_t parts,
                                                      const half_t* inp, half_t* out, uint32_t nteams, XchLaunch xl) {
     constexpr int LPR = 8;
@@ -198,7 +200,7 @@ __global__ __launch_bounds__(NT) void k_softmax_team(int32_t n, int32_t m, int32
     const int64_t boff = (int64_t)b * n * m + (int64_t)own0 * m;
 
     half8_t v[R];
-    coltile_load<NT, LPR, R, true>(v, inp + boff, own_n, m, col0, (half_t)(-__builtin_inff()));
+    coltile_load<NT, LPR, R, MODE == 0, MODE == 2>(v, inp + boff, own_n, m, col0, (half_t)(-__builtin_inff()));
 
     half8_t hm = v[0];
 #pragma unroll
@@ -278,7 +280,7 @@ __global__ __launch_bounds__(NT) void k_softmax_team(int32_t n, int32_t m, int32
     for (int p = 0; p < R; ++p)
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[p][e] = round_f16(ex[p][e] * f[e]);
-    coltile_store<NT, LPR, R, true>(v, out + boff, own_n, m, col0);
+    coltile_store<NT, LPR, R, MODE == 0, MODE == 2>(v, out + boff, own_n, m, col0);
     if (tid < 64) xch_retire(xl, team, parts);     // after the barrier above: this workgroup holds all it needs
 }
 
@@ -325,10 +327,10 @@ __global__ __launch_bounds__(256) void k_softmax_rows(int32_t n, const half_t* i
     for (int32_t i = threadIdx.x; i < n; i += 256) o[i] = round_f16(exp_shift((float)p[i], mx) * s);
 }
 
-template <int NT, int LPR, int R>
+template <int NT, int LPR, int R, int MODE>
 static void launch_tile(int32_t batch, int32_t n, int32_t m, const half_t* inp, half_t* out, hipStream_t st) {
     const int32_t tiles = (int32_t)ceil_div(m, LPR * 8);
-    hipLaunchKernelGGL((k_softmax_tile<NT, LPR, R>), dim3((unsigned)((int64_t)tiles * batch)), dim3(NT), 0, st, n, m,
+    hipLaunchKernelGGL((k_softmax_tile<NT, LPR, R, MODE>), dim3((unsigned)((int64_t)tiles * batch)), dim3(NT), 0, st, n, m,
                        tiles, inp, out);
 }
 
@@ -356,13 +358,13 @@ static int launch_stream(int32_t batch, int32_t n, int32_t m, const half_t* inp,
     return e ? e : rc2;
 }
 
-template <int NT, int LPR>
+template <int NT, int LPR, int MODE>
 static bool launch_tile_r(int r, int32_t batch, int32_t n, int32_t m, const half_t* inp, half_t* out,
                           hipStream_t st) {
-    if (r <= 1) launch_tile<NT, LPR, 1>(batch, n, m, inp, out, st);
-    else if (r <= 2) launch_tile<NT, LPR, 2>(batch, n, m, inp, out, st);
-    else if (r <= 4) launch_tile<NT, LPR, 4>(batch, n, m, inp, out, st);
-    else if (r <= 8) launch_tile<NT, LPR, 8>(batch, n, m, inp, out, st);
+    if (r <= 1) launch_tile<NT, LPR, 1, MODE>(batch, n, m, inp, out, st);
+    else if (r <= 2) launch_tile<NT, LPR, 2, MODE>(batch, n, m, inp, out, st);
+    else if (r <= 4) launch_tile<NT, LPR, 4, MODE>(batch, n, m, inp, out, st);
+    else if (r <= 8) launch_tile<NT, LPR, 8, MODE>(batch, n, m, inp, out, st);
     else return false;
     return true;
 }
@@ -380,7 +382,17 @@ static int softmax_dispatch(int32_t batch, int32_t n, int32_t m, const void* inp
         hipLaunchKernelGGL(k_softmax_rows, dim3((unsigned)batch), dim3(256), 0, st, n, x, y);
         return launch_status();
     }
-    if (m % 8 == 0 && aligned16(inp) && aligned16(out) && (int64_t)n * m < (1ll << 31)) {
+    // rows of whole 16-byte pieces in 16-byte aligned buffers: 16-byte accesses, with the non-temporal hint where the
+    // 128-byte row segments of the 64-column tiles are whole cache lines; any other width or alignment: the same kernels
+    // moving their tiles element by element
+    const bool wide = m % 8 == 0 && aligned16(inp) && aligned16(out);
+    const bool lines = wide && m % 64 == 0 && (reinterpret_cast<uintptr_t>(inp) & 127u) == 0 && (reinterpret_cast<uintptr_t>(out) & 127u) == 0;
+    auto with_mode = [&](auto&& f) {       // f(integral_constant<int, MODE>)
+        if (!wide) return f(std::integral_constant<int, 2>{});
+        if (lines) return f(std::integral_constant<int, 0>{});
+        return f(std::integral_constant<int, 1>{});
+    };
+    if ((int64_t)n * m < (1ll << 31)) {
         bool ok = false;
         if (n > kSoftmaxTeamMin && m >= 64) {
             const int64_t tiles = ceil_div(m, 64);
@@ -401,8 +413,11 @@ static int softmax_dispatch(int32_t batch, int32_t n, int32_t m, const void* inp
                     const dim3 grid((unsigned)xch_team_grid(tiles * nb, parts));
                     const half_t* xb = x + b0 * n * m;
                     half_t* yb = y + b0 * n * m;
-                    hipLaunchKernelGGL((k_softmax_team<1024, 8>), grid, dim3(1024), 0, st, n, m, (int32_t)tiles,
-                                       (int32_t)parts, xb, yb, (uint32_t)(tiles * nb), xs.xl);
+                    with_mode([&](auto mc) {
+                        hipLaunchKernelGGL((k_softmax_team<1024, 8, decltype(mc)::value>), grid, dim3(1024), 0, st, n, m, (int32_t)tiles,
+                                           (int32_t)parts, xb, yb, (uint32_t)(tiles * nb), xs.xl);
+                        return true;
+                    });
                     const int e = launch_status();
                     const int rc2 = xs.end();
                     if (e != 0 || rc2 != 0) return e ? e : rc2;
@@ -411,15 +426,19 @@ static int softmax_dispatch(int32_t batch, int32_t n, int32_t m, const void* inp
             }
         }
         // several tiles per compute unit: the persistent kernel keeps loads in flight during the arithmetic
-        if (n > 256 && n <= 1024 && m >= 64 && ceil_div(m, 64) * batch >= 2 * (int64_t)compute_units() &&
+        if (lines && n > 256 && n <= 1024 && m >= 64 && ceil_div(m, 64) * batch >= 2 * (int64_t)compute_units() &&
             ceil_div(m, 64) * batch < (1ll << 31)) {
             const int rc = n > 512 ? launch_stream<1024, 8, 8>(batch, n, m, x, y, st) : launch_stream<1024, 8, 4>(batch, n, m, x, y, st);
             if (rc != kXchFull) return rc;
         }
-        if (n <= 64 * 8 && m >= 64) ok = launch_tile_r<512, 8>((int)ceil_div(n, 64), batch, n, m, x, y, st);
-        else if (n <= 128 * 8 && m >= 64) ok = launch_tile_r<1024, 8>((int)ceil_div(n, 128), batch, n, m, x, y, st);
-        else if (n <= 256 * 8 && m >= 32) ok = launch_tile_r<1024, 4>((int)ceil_div(n, 256), batch, n, m, x, y, st);
-        else if (n <= 512 * 8) ok = launch_tile_r<1024, 2>((int)ceil_div(n, 512), batch, n, m, x, y, st);
+        ok = with_mode([&](auto mc) {
+            constexpr int MODE = decltype(mc)::value;
+            if (n <= 64 * 8 && m >= 64) return launch_tile_r<512, 8, MODE>((int)ceil_div(n, 64), batch, n, m, x, y, st);
+            if (n <= 128 * 8 && m >= 64) return launch_tile_r<1024, 8, MODE>((int)ceil_div(n, 128), batch, n, m, x, y, st);
+            if (n <= 256 * 8 && m >= 32) return launch_tile_r<1024, 4, MODE>((int)ceil_div(n, 256), batch, n, m, x, y, st);
+            if (n <= 512 * 8) return launch_tile_r<1024, 2, MODE>((int)ceil_div(n, 512), batch, n, m, x, y, st);
+            return false;
+        });
         if (ok) return launch_status();
     }
     // the batch is the grid's y dimension (at most 65535): larger batches go out in several launches
