@@ -15,7 +15,9 @@ namespace cpmk {
 // consecutive rows rg*8 .. rg*8+7, so that its int8 results are 8 contiguous bytes in either
 // output layout.
 // (two 512-thread workgroups share a compute unit: at most 128 registers per lane)
-template <int NT, bool TRANSPOSED>
+// NTH: the tile's 128-byte row segments are whole cache lines (m % 64 == 0, the matrix on a 128-byte boundary): the input is
+// read with the non-temporal hint.  Elsewhere a line is shared with the neighbouring tile and has to stay in L2 for it.
+template <int NT, bool TRANSPOSED, bool NTH>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void k_col_quantize_team(int32_t n, int32_t m, int32_t tiles_per_batch, int32_t parts,
                                                           const half_t* __restrict__ mat, half_t* __restrict__ scale,
                                                           int8_t* __restrict__ out, uint32_t nteams, XchLaunch xl) {
@@ -41,7 +43,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         for (int e = 0; e < 8; ++e) v[p][e] = (half_t)0.0f;
         if (row0 + p < n && col0 < m) {
             const half8_t* src = reinterpret_cast<const half8_t*>(mat + boff + ((uint32_t)(row0 + p) * (uint32_t)m + (uint32_t)col0));
-            v[p] = __builtin_nontemporal_load(src);        // read once; the int8 output below is what the next kernel wants in cache
+            v[p] = NTH ? __builtin_nontemporal_load(src) : *src;        // read once; the int8 output below is what the next kernel wants in cache
         }
     }
     // |x| maxima of the lane's 8 columns as integers; a NaN among them (rare) repeats the maximum in
@@ -225,14 +227,18 @@ int cpmk_gemm_quantize_cols(int32_t batch, int32_t n, int32_t m, const void* mat
                 }
                 if (rc != 0) return rc == kXchFull ? CPMK_ETOOBIG : rc;
             }
-            if (out_transposed)
-                hipLaunchKernelGGL((k_col_quantize_team<512, true>), dim3((unsigned)xch_team_grid(tiles * nb, parts)), dim3(512), 0, st, n, m,
-                                   (int32_t)tiles, (int32_t)parts, (const half_t*)mat + b0 * n * m, (half_t*)scale + b0 * m,
-                                   (int8_t*)out + b0 * n * m, (uint32_t)(tiles * nb), xs.xl);
-            else
-                hipLaunchKernelGGL((k_col_quantize_team<512, false>), dim3((unsigned)xch_team_grid(tiles * nb, parts)), dim3(512), 0, st, n, m,
-                                   (int32_t)tiles, (int32_t)parts, (const half_t*)mat + b0 * n * m, (half_t*)scale + b0 * m,
-                                   (int8_t*)out + b0 * n * m, (uint32_t)(tiles * nb), xs.xl);
+            const bool lines = m % 64 == 0 && (reinterpret_cast<uintptr_t>(mat) & 127u) == 0;
+            auto go = [&](auto kern) {
+                hipLaunchKernelGGL(kern, dim3((unsigned)xch_team_grid(tiles * nb, parts)), dim3(512), 0, st, n, m, (int32_t)tiles, (int32_t)parts,
+                                   (const half_t*)mat + b0 * n * m, (half_t*)scale + b0 * m, (int8_t*)out + b0 * n * m, (uint32_t)(tiles * nb), xs.xl);
+            };
+            if (out_transposed) {
+                if (lines) go(k_col_quantize_team<512, true, true>);
+                else go(k_col_quantize_team<512, true, false>);
+            } else {
+                if (lines) go(k_col_quantize_team<512, false, true>);
+                else go(k_col_quantize_team<512, false, false>);
+            }
             const int e = launch_status();
             const int rc2 = xs.end();
             if (e != 0 || rc2 != 0) return e ? e : rc2;

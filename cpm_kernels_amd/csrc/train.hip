@@ -264,7 +264,8 @@ __global__ __launch_bounds__(256) void k_col(ColArgs p) {
 // accesses; k_col above serves everything else.
 constexpr int kColTeamMaxParts = 32;
 
-template <int KIND>
+// NTH: the tile's row segments are whole cache lines (m % 64 == 0, buffers on 128-byte boundaries): non-temporal accesses.
+template <int KIND, bool NTH>
 __global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_batch, int32_t parts, uint32_t nteams, XchLaunch xl) {
     uint64_t* const xch = xl.region;
     const uint32_t tag = xl.tag;
@@ -303,9 +304,9 @@ __global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_b
     half8_t va[R], vg[TWO ? R : 1];
     // every input byte is read once: non-temporal loads; non-temporal stores too, except for the softmax
     // gradient, where they measured 1-2 % slower
-    constexpr bool NTS = KIND != kSoftmaxBwd;
-    coltile_load<NT, LPR, R, true>(va, p.a + boff, own_n, p.m, col0, (half_t)0.0f);
-    if constexpr (TWO) coltile_load<NT, LPR, R, true>(vg, p.g + boff, own_n, p.m, col0, (half_t)0.0f);
+    constexpr bool NTS = NTH && KIND != kSoftmaxBwd;
+    coltile_load<NT, LPR, R, NTH>(va, p.a + boff, own_n, p.m, col0, (half_t)0.0f);
+    if constexpr (TWO) coltile_load<NT, LPR, R, NTH>(vg, p.g + boff, own_n, p.m, col0, (half_t)0.0f);
     float mean[8], var[8], c3[8], sxv[R];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
@@ -803,6 +804,8 @@ static int launch_col(int32_t batch, const ColArgs& p, void* stream, bool missin
                       (p.out_mean == nullptr || aligned16(p.out_mean)) && (p.out_var == nullptr || aligned16(p.out_var)) &&
                       (p.out_i8 == nullptr || (reinterpret_cast<uintptr_t>(p.out_i8) & 7u) == 0) && (int64_t)p.n * p.m < (1ll << 31) &&
                       parts <= kColTeamMaxParts && tiles * parts <= kXchSlots;
+    auto on_line = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 127u) == 0; };
+    const bool lines = p.m % 64 == 0 && on_line(p.a) && on_line(p.g) && on_line(p.out);      // (a null pointer counts as aligned)
     if (wide) {
         // teams use one packet slot per (team, part): batches beyond the pool go out in several launches
         const int64_t per_launch = parts > 1 ? kXchSlots / (tiles * parts) : ((1ll << 31) - 8) / (tiles * parts);
@@ -819,8 +822,12 @@ static int launch_col(int32_t batch, const ColArgs& p, void* stream, bool missin
                 }
                 if (rc != 0) return rc == kXchFull ? CPMK_ETOOBIG : rc;
             }
-            hipLaunchKernelGGL((k_col_team<KIND>), dim3((unsigned)xch_team_grid(tiles * nb, parts)), dim3(512), 0, (hipStream_t)stream, q,
-                               (int32_t)tiles, (int32_t)parts, (uint32_t)(tiles * nb), xs.xl);
+            if (lines)
+                hipLaunchKernelGGL((k_col_team<KIND, true>), dim3((unsigned)xch_team_grid(tiles * nb, parts)), dim3(512), 0, (hipStream_t)stream, q,
+                                   (int32_t)tiles, (int32_t)parts, (uint32_t)(tiles * nb), xs.xl);
+            else
+                hipLaunchKernelGGL((k_col_team<KIND, false>), dim3((unsigned)xch_team_grid(tiles * nb, parts)), dim3(512), 0, (hipStream_t)stream, q,
+                                   (int32_t)tiles, (int32_t)parts, (uint32_t)(tiles * nb), xs.xl);
             const int e = launch_status();
             const int rc2 = xs.end();
             if (e != 0 || rc2 != 0) return e ? e : rc2;
