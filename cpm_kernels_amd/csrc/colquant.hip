@@ -17,7 +17,9 @@ namespace cpmk {
 // (two 512-thread workgroups share a compute unit: at most 128 registers per lane)
 // NTH: the tile's 128-byte row segments are whole cache lines (m % 64 == 0, the matrix on a 128-byte boundary): the input is
 // read with the non-temporal hint.  Elsewhere a line is shared with the neighbouring tile and has to stay in L2 for it.
-template <int NT, bool TRANSPOSED, bool NTH>
+// UA: any m and alignment: the eight columns of a piece are read (and the scales and, not transposed, the int8 values
+// written) one by one, each checked against m.
+template <int NT, bool TRANSPOSED, bool NTH, bool UA = false>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void k_col_quantize_team(int32_t n, int32_t m, int32_t tiles_per_batch, int32_t parts,
                                                           const half_t* __restrict__ mat, half_t* __restrict__ scale,
                                                           int8_t* __restrict__ out, uint32_t nteams, XchLaunch xl) {
@@ -41,7 +43,14 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     for (int p = 0; p < R; ++p) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[p][e] = (half_t)0.0f;
-        if (row0 + p < n && col0 < m) {
+        if constexpr (UA) {
+            if (row0 + p < n) {
+                const half_t* src = mat + boff + ((uint32_t)(row0 + p) * (uint32_t)m + (uint32_t)col0);
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (col0 + e < m) v[p][e] = src[e];
+            }
+        } else if (row0 + p < n && col0 < m) {
             const half8_t* src = reinterpret_cast<const half8_t*>(mat + boff + ((uint32_t)(row0 + p) * (uint32_t)m + (uint32_t)col0));
             v[p] = NTH ? __builtin_nontemporal_load(src) : *src;        // read once; the int8 output below is what the next kernel wants in cache
         }
@@ -92,7 +101,15 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         s[e] = (float)sh[e];
         y[e] = 1.0f / s[e];
     }
-    if (part == 0 && rg == 0 && col0 < m) *reinterpret_cast<half8_t*>(scale + (int64_t)b * m + col0) = sh;
+    if (part == 0 && rg == 0) {
+        if constexpr (UA) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (col0 + e < m) scale[(int64_t)b * m + col0 + e] = sh[e];
+        } else if (col0 < m) {
+            *reinterpret_cast<half8_t*>(scale + (int64_t)b * m + col0) = sh;
+        }
+    }
 
     uint32_t q[R][2];       // [row p][columns 0-3 | 4-7], one byte each
     bool normal = true;
@@ -125,9 +142,16 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         if constexpr (!TRANSPOSED) {
 #pragma unroll
             for (int p = 0; p < R; ++p)
-                if (row0 + p < n)
-                    *reinterpret_cast<uint2_t*>(out + boff + ((uint32_t)(row0 + p) * (uint32_t)m + (uint32_t)col0)) =
-                        uint2_t{q[p][0], q[p][1]};
+                if (row0 + p < n) {
+                    int8_t* dst = out + boff + ((uint32_t)(row0 + p) * (uint32_t)m + (uint32_t)col0);
+                    if constexpr (UA) {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            if (col0 + e < m) dst[e] = (int8_t)(q[p][e >> 2] >> (8 * (e & 3)));
+                    } else {
+                        *reinterpret_cast<uint2_t*>(dst) = uint2_t{q[p][0], q[p][1]};
+                    }
+                }
         }
     }
     if constexpr (TRANSPOSED) {
@@ -209,8 +233,10 @@ int cpmk_gemm_quantize_cols(int32_t batch, int32_t n, int32_t m, const void* mat
     // (16384 rows; far fewer workgroups than are resident at once, which is what progress needs)
     constexpr int64_t kColMaxParts = 32;
     const int64_t tiles = ceil_div(m, 64), parts = ceil_div(n, 512);
-    const bool team_ok = (m % 8 == 0) && (!out_transposed || n % 8 == 0) && aligned16(mat) && aligned16(scale) &&
-                         ((reinterpret_cast<uintptr_t>(out) & 7u) == 0) && (int64_t)n * m < (1ll << 31) &&
+    // rows of whole 16-byte pieces in aligned buffers: 16-byte accesses; any other width or alignment: the same kernel moving
+    // its columns one by one (the transposed output runs along n either way)
+    const bool wide = (m % 8 == 0) && aligned16(mat) && aligned16(scale) && ((reinterpret_cast<uintptr_t>(out) & 7u) == 0);
+    const bool team_ok = (!out_transposed || (n % 8 == 0 && (reinterpret_cast<uintptr_t>(out) & 7u) == 0)) && (int64_t)n * m < (1ll << 31) &&
                          parts <= kColMaxParts && tiles * parts <= kXchSlots;
     if (team_ok) {
         // teams use one packet slot per (team, part): batches beyond the pool go out in several launches
@@ -233,10 +259,12 @@ int cpmk_gemm_quantize_cols(int32_t batch, int32_t n, int32_t m, const void* mat
                                    (const half_t*)mat + b0 * n * m, (half_t*)scale + b0 * m, (int8_t*)out + b0 * n * m, (uint32_t)(tiles * nb), xs.xl);
             };
             if (out_transposed) {
-                if (lines) go(k_col_quantize_team<512, true, true>);
+                if (!wide) go(k_col_quantize_team<512, true, false, true>);
+                else if (lines) go(k_col_quantize_team<512, true, true>);
                 else go(k_col_quantize_team<512, true, false>);
             } else {
-                if (lines) go(k_col_quantize_team<512, false, true>);
+                if (!wide) go(k_col_quantize_team<512, false, false, true>);
+                else if (lines) go(k_col_quantize_team<512, false, true>);
                 else go(k_col_quantize_team<512, false, false>);
             }
             const int e = launch_status();
