@@ -1203,67 +1203,78 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
 }
 
 // ---------------------------------------------------------------------------------------
-// fp16 product (fp32 accumulation), any layout and size: 64x64 output tile, 16 halves of K per
-// stage, 256 threads each computing a 4x4 block.  The K-major, k % 64 == 0 case runs on the
-// tile kernel above with the fp16 MFMA instead.
+// fp16 product (fp32 accumulation), any layout, size and alignment: 64x64 output tile, 32 halves of K per
+// stage, four waves of one 32x32 MFMA tile each.  Shapes that are whole slabs and pieces run on the tile
+// kernel above instead.
 // ---------------------------------------------------------------------------------------
+// V: halves per global access (4, 2 or 1: what the contiguous dimension of both operands and the alignment of the buffers allow).
+template <int V>
 __global__ __launch_bounds__(256) void k_gemm_f16_generic(GemmArgs a, int p_kmajor, int q_kmajor, int32_t row_base) {
-    constexpr int T = 64, GK = 16, LD = GK + 2;
-    __shared__ half_t sP[T * LD];
-    __shared__ half_t sQ[T * LD];
+    // Element-wise guarded loads bring a 64 x 32 piece of each operand into LDS with K contiguous (zeros past the edges,
+    // so any size, layout and alignment works); each of the four waves then owns a 32 x 32 quarter of the tile and
+    // multiplies with v_mfma_f32_32x32x16_f16.
+    constexpr int T = 64, GK = 32, LD = GK + 4;        // rows of 72 bytes: 8-byte aligned fragment reads, spread over the banks
+    __shared__ __attribute__((aligned(16))) half_t sP[T * LD];
+    __shared__ __attribute__((aligned(16))) half_t sQ[T * LD];
     const int b = blockIdx.z;
     const int32_t k = a.k >> 1;                        // a.k is the row length in bytes
     const half_t* P = reinterpret_cast<const half_t*>(a.P + (int64_t)b * a.strideP);
     const half_t* Q = reinterpret_cast<const half_t*>(a.Q + (int64_t)b * a.strideQ);
     const int32_t j0 = row_base + blockIdx.y * T, i0 = blockIdx.x * T;
-    const int tid = threadIdx.x, ty = tid >> 4, tx = tid & 15;
-    float acc[4][4];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wr = wave >> 1, wc = wave & 1;
+    const int lrow = lane & 31, lk = lane >> 5;
+    float16_tv acc;
 #pragma unroll
-    for (int r = 0; r < 4; ++r)
+    for (int e = 0; e < 16; ++e) acc[e] = 0.0f;
+    typedef _Float16 halfV_t __attribute__((ext_vector_type(V > 1 ? V : 2)));
+    // V halves of one operand's piece: along K for a K-major operand (one row), along the rows for one stored (K, rows)
+    auto stage = [&](half_t* sm, const half_t* G, int kmajor, int32_t r0, int32_t L, int32_t k0, int q) __attribute__((always_inline)) {
+        int r, kk;
+        if (kmajor) { r = q / (GK / V); kk = (q % (GK / V)) * V; } else { r = (q % (T / V)) * V; kk = q / (T / V); }
+        const int32_t row = r0 + r, kg = k0 + kk;
+        half_t v[V];
 #pragma unroll
-        for (int c = 0; c < 4; ++c) acc[r][c] = 0.0f;
+        for (int e = 0; e < V; ++e) v[e] = (half_t)0.0f;
+        if (row < L && kg < k) {            // (L and k are multiples of V where the access runs along them)
+            const half_t* src = kmajor ? G + ((int64_t)row * k + kg) : G + ((int64_t)kg * L + row);
+            if constexpr (V > 1) {
+                const halfV_t t = *reinterpret_cast<const halfV_t*>(src);
+#pragma unroll
+                for (int e = 0; e < V; ++e) v[e] = t[e];
+            } else {
+                v[0] = *src;
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < V; ++e) sm[kmajor ? r * LD + kk + e : (r + e) * LD + kk] = v[e];
+    };
     for (int32_t k0 = 0; k0 < k; k0 += GK) {
 #pragma unroll
-        for (int s = 0; s < T * GK / 256; ++s) {
-            const int q = tid + s * 256;
-            int r, kk;
-            if (p_kmajor) { r = q / GK; kk = q % GK; } else { r = q % T; kk = q / T; }
-            const int32_t row = j0 + r, kg = k0 + kk;
-            half_t v = (half_t)0.0f;
-            if (row < a.n && kg < k) v = p_kmajor ? P[(int64_t)row * k + kg] : P[(int64_t)kg * a.n + row];
-            sP[r * LD + kk] = v;
-            if (q_kmajor) { r = q / GK; kk = q % GK; } else { r = q % T; kk = q / T; }
-            const int32_t col = i0 + r;
-            const int32_t kg2 = k0 + kk;
-            v = (half_t)0.0f;
-            if (col < a.m && kg2 < k) v = q_kmajor ? Q[(int64_t)col * k + kg2] : Q[(int64_t)kg2 * a.m + col];
-            sQ[r * LD + kk] = v;
+        for (int s = 0; s < T * GK / V / 256; ++s) {
+            stage(sP, P, p_kmajor, j0, a.n, k0, tid + s * 256);
+            stage(sQ, Q, q_kmajor, i0, a.m, k0, tid + s * 256);
         }
         __syncthreads();
 #pragma unroll
-        for (int kk = 0; kk < GK; ++kk) {
-            float pa[4], qb[4];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) pa[r] = (float)sP[(ty * 4 + r) * LD + kk];
-#pragma unroll
-            for (int c = 0; c < 4; ++c) qb[c] = (float)sQ[(tx + c * 16) * LD + kk];
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-#pragma unroll
-                for (int c = 0; c < 4; ++c) acc[r][c] = __builtin_fmaf(pa[r], qb[c], acc[r][c]);
+        for (int ks = 0; ks < GK / 16; ++ks) {
+            // lane (lrow, lk): the 8 halves k = 16 ks + 8 lk .. + 7 of its row / column, as two 8-byte reads
+            const half_t* pp = sP + (wr * 32 + lrow) * LD + ks * 16 + lk * 8;
+            const half_t* qp = sQ + (wc * 32 + lrow) * LD + ks * 16 + lk * 8;
+            const half4_t p0 = *reinterpret_cast<const half4_t*>(pp), p1 = *reinterpret_cast<const half4_t*>(pp + 4);
+            const half4_t q0 = *reinterpret_cast<const half4_t*>(qp), q1 = *reinterpret_cast<const half4_t*>(qp + 4);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_shufflevector(p0, p1, 0, 1, 2, 3, 4, 5, 6, 7),
+                                                         __builtin_shufflevector(q0, q1, 0, 1, 2, 3, 4, 5, 6, 7), acc, 0, 0, 0);
         }
         __syncthreads();
     }
+    // accumulator register e of lane l: output row (e / 4) * 8 + (l / 32) * 4 + e % 4, column l % 32 of the wave's quarter
     const int64_t obase = (int64_t)b * a.n * a.m;
+    const int32_t col = i0 + wc * 32 + lrow;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const int32_t row = j0 + ty * 4 + r;
-        if (row >= a.n) continue;
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const int32_t col = i0 + tx + c * 16;
-            if (col < a.m) reinterpret_cast<half_t*>(a.out)[obase + (int64_t)row * a.m + col] = (half_t)acc[r][c];
-        }
+    for (int e = 0; e < 16; ++e) {
+        const int32_t row = j0 + wr * 32 + (e >> 2) * 8 + lk * 4 + (e & 3);
+        if (row < a.n && col < a.m) reinterpret_cast<half_t*>(a.out)[obase + (int64_t)row * a.m + col] = (half_t)acc[e];
     }
 }
 
@@ -1342,7 +1353,15 @@ static int gemm_f16_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, in
     for (int64_t r0 = 0; r0 < n; r0 += 65535ll * 64) {        // (rows beyond the grid's y dimension: several launches)
         const int64_t nr = n - r0 < 65535ll * 64 ? n - r0 : 65535ll * 64;
         dim3 grid((unsigned)ceil_div(m, 64), (unsigned)ceil_div(nr, 64), (unsigned)batch);
-        hipLaunchKernelGGL(k_gemm_f16_generic, grid, dim3(256), 0, st, a, (int)p_kmajor, (int)q_kmajor, (int32_t)r0);
+        // the widest access both operands allow: their contiguous dimension a multiple of it, their buffers aligned to it
+        const int32_t cp = p_kmajor ? k : n, cq = q_kmajor ? k : m;
+        const uintptr_t al = reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B);
+        if (cp % 4 == 0 && cq % 4 == 0 && (al & 7u) == 0)
+            hipLaunchKernelGGL(k_gemm_f16_generic<4>, grid, dim3(256), 0, st, a, (int)p_kmajor, (int)q_kmajor, (int32_t)r0);
+        else if (cp % 2 == 0 && cq % 2 == 0 && (al & 3u) == 0)
+            hipLaunchKernelGGL(k_gemm_f16_generic<2>, grid, dim3(256), 0, st, a, (int)p_kmajor, (int)q_kmajor, (int32_t)r0);
+        else
+            hipLaunchKernelGGL(k_gemm_f16_generic<1>, grid, dim3(256), 0, st, a, (int)p_kmajor, (int)q_kmajor, (int32_t)r0);
         if (int e = launch_status()) return e;
     }
     return 0;
