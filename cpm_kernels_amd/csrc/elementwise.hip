@@ -84,7 +84,24 @@ __global__ __launch_bounds__(256) void k_mask(int64_t total, int32_t n, int32_t 
     const int64_t row = e0 / m;
     const int32_t j = (int32_t)(e0 - row * m);
     const int8_t* mp = mask + (row / n) * m + j;
-    if (vec) {
+    if (vec == 2) {
+        // rows that are not whole 16-byte pieces (m >= 8): the tensor is still one contiguous run, so its elements go
+        // eight at a time; the eight may run over the end of a row, and each looks up its own mask byte
+        if (e0 + 8 <= total) {
+            half8_t v = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(x + e0));
+            const int8_t* m0 = mask + (row / n) * m + j;                   // this row's mask bytes from column j on
+            const int8_t* m1 = mask + ((row + 1) / n) * m + (j - m);       // the next row's, addressed by the same index
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if ((j + e < m ? m0 : m1)[e] == 0) v[e] = value;
+            __builtin_nontemporal_store(v, reinterpret_cast<half8_t*>(out + e0));
+        } else {
+            for (int64_t i = e0; i < total; ++i) {
+                const int64_t r2 = i / m;
+                out[i] = (mask[(r2 / n) * m + (i - r2 * m)] == 0) ? value : x[i];
+            }
+        }
+    } else if (vec) {
         half8_t v = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(x + e0));
         const uint2_t mk = *reinterpret_cast<const uint2_t*>(mp);
 #pragma unroll
@@ -169,8 +186,9 @@ int cpmk_mask(int32_t batch, int32_t n, int32_t m, const void* inp, const void* 
     const int64_t total = (int64_t)batch * n * m;
     if (total == 0) return 0;
     if (any_null(inp, mask, out)) return CPMK_EBADARG;
-    const int vec = (m % 8 == 0) && aligned16(inp) && aligned16(out) && ((reinterpret_cast<uintptr_t>(mask) & 7u) == 0);
-    const int64_t g = ceil_div(vec ? total / 8 : total, 256);
+    int vec = (m % 8 == 0) && aligned16(inp) && aligned16(out) && ((reinterpret_cast<uintptr_t>(mask) & 7u) == 0);
+    if (!vec && m >= 8 && aligned16(inp) && aligned16(out)) vec = 2;
+    const int64_t g = ceil_div(vec ? ceil_div(total, 8) : total, 256);
     hipLaunchKernelGGL(k_mask, dim3((unsigned)g), dim3(256), 0, (hipStream_t)stream, total, n, m, (const half_t*)inp,
                        (const int8_t*)mask, (half_t)value, (half_t*)out, vec);
     return launch_status();
