@@ -40,6 +40,7 @@ __device__ inline void coltile_load(half8_t (&v)[R], const half_t* base, int32_t
     const int rg = threadIdx.x / LPR;
     const uint32_t off0 = (uint32_t)rg * (uint32_t)m + (uint32_t)col0, stride = (uint32_t)RPP * (uint32_t)m;
     const bool pairs = UA && (m & 1) == 0 && (reinterpret_cast<uintptr_t>(base) & 3u) == 0;
+    const bool quads = UA && (m & 3) == 0 && (reinterpret_cast<uintptr_t>(base) & 7u) == 0;
 #pragma unroll
     for (int p = 0; p < R; ++p) {
         const int32_t row = p * RPP + rg;
@@ -48,7 +49,15 @@ __device__ inline void coltile_load(half8_t (&v)[R], const half_t* base, int32_t
         for (int e = 0; e < 8; ++e) x[e] = fill;
         if constexpr (UA) {
             if (row < n) {
-                if (pairs) {        // even m, 4-byte aligned buffer: two columns per access
+                if (quads) {        // m % 4 == 0, 8-byte aligned buffer: four columns per access
+#pragma unroll
+                    for (int e = 0; e < 8; e += 4)
+                        if (col0 + e < m) {
+                            const half4_t t = *reinterpret_cast<const half4_t*>(base + (off0 + p * stride + e));
+#pragma unroll
+                            for (int d = 0; d < 4; ++d) x[e + d] = t[d];
+                        }
+                } else if (pairs) {        // even m, 4-byte aligned buffer: two columns per access
 #pragma unroll
                     for (int e = 0; e < 8; e += 2)
                         if (col0 + e < m) {
@@ -78,12 +87,18 @@ __device__ inline void coltile_store(const half8_t (&v)[R], half_t* base, int32_
     const int rg = threadIdx.x / LPR;
     const uint32_t off0 = (uint32_t)rg * (uint32_t)m + (uint32_t)col0, stride = (uint32_t)RPP * (uint32_t)m;
     const bool pairs = UA && (m & 1) == 0 && (reinterpret_cast<uintptr_t>(base) & 3u) == 0;
+    const bool quads = UA && (m & 3) == 0 && (reinterpret_cast<uintptr_t>(base) & 7u) == 0;
 #pragma unroll
     for (int p = 0; p < R; ++p) {
         const int32_t row = p * RPP + rg;
         if constexpr (UA) {
             if (row < n) {
-                if (pairs) {
+                if (quads) {
+#pragma unroll
+                    for (int e = 0; e < 8; e += 4)
+                        if (col0 + e < m)
+                            *reinterpret_cast<half4_t*>(base + (off0 + p * stride + e)) = half4_t{v[p][e], v[p][e + 1], v[p][e + 2], v[p][e + 3]};
+                } else if (pairs) {
 #pragma unroll
                     for (int e = 0; e < 8; e += 2)
                         if (col0 + e < m) *reinterpret_cast<half2_t*>(base + (off0 + p * stride + e)) = half2_t{v[p][e], v[p][e + 1]};
