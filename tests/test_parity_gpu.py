@@ -43,7 +43,9 @@ def adversarial_rows(rng, n, m):
 
 QUANT_SHAPES = [(1, 512, 4096), (3, 17, 1000), (2, 5, 7), (1, 1, 8), (2, 64, 48), (1, 9, 8200), (4, 33, 16),
                 (1, 2100, 128), (1, 3, 20480), (2, 4096, 192), (1, 1032, 72), (3, 520, 8),
-                (1, 10240, 192), (2, 16384, 64), (1, 16392, 64)]
+                (1, 10240, 192), (2, 16384, 64), (1, 16392, 64),
+                # tall columns in widths that are not whole 16-byte pieces (the team kernel, one column at a time)
+                (2, 4096, 500), (1, 1040, 77), (1, 2100, 36)]
 
 
 @pytest.mark.parametrize("shape", QUANT_SHAPES)
@@ -531,7 +533,10 @@ def test_gemv_broadcast_mat_int8(gpu, batch, dim_out, dim_in):
 # layernorm / softmax / gelu (tolerance ops)
 # ---------------------------------------------------------------------------------------------
 LN_SHAPES = [(8, 4096, 512), (16, 768, 512), (4, 1024, 512), (3, 100, 40), (2, 33, 24), (2, 777, 123), (5, 4096, 1),
-             (1, 5000, 64), (2, 2048, 32), (1, 1536, 8), (2, 64, 72), (2, 1100, 64), (1, 8192, 128), (1, 9000, 64)]
+             (1, 5000, 64), (2, 2048, 32), (1, 1536, 8), (2, 64, 72), (2, 1100, 64), (1, 8192, 128), (1, 9000, 64),
+             # widths that are not whole 16-byte pieces (8-byte, 4-byte, 2-byte accesses) on the tile and team kernels, and
+             # widths whose rows do not start on cache-line boundaries (no non-temporal hint)
+             (2, 4096, 500), (1, 3000, 77), (1, 4096, 38), (3, 640, 500), (2, 2048, 1000), (2, 900, 200)]
 
 
 @pytest.mark.parametrize("shape", LN_SHAPES)
@@ -747,7 +752,9 @@ SOFTMAX_SHAPES = [(1, 2, 32), (4, 128, 128), (4, 128, 16), (4, 123, 16), (16, 10
                   (3, 512, 64), (2, 2000, 48), (2, 4096, 16), (1, 5000, 24), (6, 333, 1), (2, 64, 200), (2, 2100, 64),
                   (1, 4096, 192), (1, 8192, 64), (1, 9000, 64),
                   # several tiles per compute unit: the persistent kernel (ragged rows, ragged last column tile)
-                  (40, 700, 1024), (64, 300, 520), (33, 1024, 1000), (600, 257, 64), (20, 1500, 1024), (70, 2048, 264)]
+                  (40, 700, 1024), (64, 300, 520), (33, 1024, 1000), (600, 257, 64), (20, 1500, 1024), (70, 2048, 264),
+                  # widths that are not whole 16-byte pieces on the tile and team kernels
+                  (2, 2100, 500), (1, 3000, 77), (3, 1024, 1004), (2, 500, 38), (3, 1500, 250)]
 
 
 @pytest.mark.parametrize("shape", SOFTMAX_SHAPES)
