@@ -264,8 +264,9 @@ __global__ __launch_bounds__(256) void k_col(ColArgs p) {
 // accesses; k_col above serves everything else.
 constexpr int kColTeamMaxParts = 32;
 
-// NTH: the tile's row segments are whole cache lines (m % 64 == 0, buffers on 128-byte boundaries): non-temporal accesses.
-template <int KIND, bool NTH>
+// MODE 0: 16-byte accesses with the non-temporal hint (the tile's row segments are whole cache lines: m % 64 == 0, buffers on
+// 128-byte boundaries); 1: 16-byte accesses without it; 2: any m and alignment, the columns of a piece one by one.
+template <int KIND, int MODE>
 __global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_batch, int32_t parts, uint32_t nteams, XchLaunch xl) {
     uint64_t* const xch = xl.region;
     const uint32_t tag = xl.tag;
@@ -291,8 +292,29 @@ __global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_b
     // order, and behind the tiles they would hold the sums back until the last piece had arrived.
     half8_t hv = {0, 0, 0, 0, 0, 0, 0, 0}, hm = {0, 0, 0, 0, 0, 0, 0, 0};
     half_t sxh[R];
-    if (live && (KIND == kLnBwdV || KIND == kLnBwdMV)) hv = *reinterpret_cast<const half8_t*>(p.var + (int64_t)b * p.m + col0);
-    if (live && KIND == kLnBwdMV) hm = *reinterpret_cast<const half8_t*>(p.mean + (int64_t)b * p.m + col0);
+    constexpr bool NTH = MODE == 0, UA = MODE == 2;
+    auto load8 = [&](const half_t* src) __attribute__((always_inline)) {       // eight per-column values of this lane's columns
+        half8_t r = {0, 0, 0, 0, 0, 0, 0, 0};
+        if constexpr (UA) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (col0 + e < p.m) r[e] = src[e];
+        } else {
+            r = *reinterpret_cast<const half8_t*>(src);
+        }
+        return r;
+    };
+    auto store8 = [&](half_t* dst, half8_t r) __attribute__((always_inline)) {
+        if constexpr (UA) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (col0 + e < p.m) dst[e] = r[e];
+        } else {
+            *reinterpret_cast<half8_t*>(dst) = r;
+        }
+    };
+    if (live && (KIND == kLnBwdV || KIND == kLnBwdMV)) hv = load8(p.var + (int64_t)b * p.m + col0);
+    if (live && KIND == kLnBwdMV) hm = load8(p.mean + (int64_t)b * p.m + col0);
 #pragma unroll
     for (int q = 0; q < R; ++q) {
         sxh[q] = (half_t)0.0f;
@@ -305,8 +327,8 @@ __global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_b
     // every input byte is read once: non-temporal loads; non-temporal stores too, except for the softmax
     // gradient, where they measured 1-2 % slower
     constexpr bool NTS = NTH && KIND != kSoftmaxBwd;
-    coltile_load<NT, LPR, R, NTH>(va, p.a + boff, own_n, p.m, col0, (half_t)0.0f);
-    if constexpr (TWO) coltile_load<NT, LPR, R, NTH>(vg, p.g + boff, own_n, p.m, col0, (half_t)0.0f);
+    coltile_load<NT, LPR, R, NTH, UA>(va, p.a + boff, own_n, p.m, col0, (half_t)0.0f);
+    if constexpr (TWO) coltile_load<NT, LPR, R, NTH, UA>(vg, p.g + boff, own_n, p.m, col0, (half_t)0.0f);
     float mean[8], var[8], c3[8], sxv[R];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
@@ -373,9 +395,9 @@ __global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_b
         half8_t h0, h1;
 #pragma unroll
         for (int e = 0; e < 8; ++e) { h0[e] = (half_t)k0[e]; h1[e] = (half_t)k1[e]; }
-        if (KIND == kLnFwdV || KIND == kLnFwdMV) *reinterpret_cast<half8_t*>(p.out_var + (int64_t)b * p.m + col0) = h1;
-        if (KIND == kLnFwdMV) *reinterpret_cast<half8_t*>(p.out_mean + (int64_t)b * p.m + col0) = h0;
-        if (KIND == kScaleRound) *reinterpret_cast<half8_t*>(p.out_var + (int64_t)b * p.m + col0) = h0;
+        if (KIND == kLnFwdV || KIND == kLnFwdMV) store8(p.out_var + (int64_t)b * p.m + col0, h1);
+        if (KIND == kLnFwdMV) store8(p.out_mean + (int64_t)b * p.m + col0, h0);
+        if (KIND == kScaleRound) store8(p.out_var + (int64_t)b * p.m + col0, h0);
     }
     if constexpr (KIND == kScaleRound) {
         if (live) {
@@ -386,8 +408,14 @@ __global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_b
                     int32_t t[8];
 #pragma unroll
                     for (int e = 0; e < 8; ++e) t[e] = quant_i8((float)va[q][e] * sxv[q], k0[e]);
-                    *reinterpret_cast<uint2_t*>(p.out_i8 + boff + ((uint32_t)lrow * (uint32_t)p.m + (uint32_t)col0)) =
-                        uint2_t{pack4_i8(t[0], t[1], t[2], t[3]), pack4_i8(t[4], t[5], t[6], t[7])};
+                    int8_t* dst = p.out_i8 + boff + ((uint32_t)lrow * (uint32_t)p.m + (uint32_t)col0);
+                    if constexpr (UA) {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            if (col0 + e < p.m) dst[e] = (int8_t)t[e];
+                    } else {
+                        *reinterpret_cast<uint2_t*>(dst) = uint2_t{pack4_i8(t[0], t[1], t[2], t[3]), pack4_i8(t[4], t[5], t[6], t[7])};
+                    }
                 }
             }
         }
@@ -406,7 +434,7 @@ __global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_b
                 else o = x * (gi - s[e]);
                 va[q][e] = round_f16(o);
             }
-        coltile_store<NT, LPR, R, NTS>(va, p.out + boff, own_n, p.m, col0);
+        coltile_store<NT, LPR, R, NTS, UA>(va, p.out + boff, own_n, p.m, col0);
     }
     if (parts > 1 && tid < 64) xch_retire(xl, team, parts);
 }
@@ -797,13 +825,13 @@ static int launch_col(int32_t batch, const ColArgs& p, void* stream, bool missin
     if (batch < 0 || p.n < 0 || p.m < 0) return CPMK_EBADARG;
     if ((int64_t)batch * p.n * p.m == 0) return 0;
     if (missing) return CPMK_EBADARG;       // (a null buffer, found by the caller, in a call that has work to do)
-    // register-resident team kernel when every access can be 16 bytes wide (8 for the int8 output)
     const int64_t tiles = ceil_div(p.m, 64), parts = ceil_div(p.n, 512);
-    const bool wide = p.m % 8 == 0 && aligned16(p.a) && (p.g == nullptr || aligned16(p.g)) && (p.out == nullptr || aligned16(p.out)) &&
-                      (p.mean == nullptr || aligned16(p.mean)) && (p.var == nullptr || aligned16(p.var)) &&
-                      (p.out_mean == nullptr || aligned16(p.out_mean)) && (p.out_var == nullptr || aligned16(p.out_var)) &&
-                      (p.out_i8 == nullptr || (reinterpret_cast<uintptr_t>(p.out_i8) & 7u) == 0) && (int64_t)p.n * p.m < (1ll << 31) &&
-                      parts <= kColTeamMaxParts && tiles * parts <= kXchSlots;
+    // 16-byte accesses when every row and buffer allows them, else the same kernel moving its columns one by one
+    const bool vec16 = p.m % 8 == 0 && aligned16(p.a) && (p.g == nullptr || aligned16(p.g)) && (p.out == nullptr || aligned16(p.out)) &&
+                       (p.mean == nullptr || aligned16(p.mean)) && (p.var == nullptr || aligned16(p.var)) &&
+                       (p.out_mean == nullptr || aligned16(p.out_mean)) && (p.out_var == nullptr || aligned16(p.out_var)) &&
+                       (p.out_i8 == nullptr || (reinterpret_cast<uintptr_t>(p.out_i8) & 7u) == 0);
+    const bool wide = (int64_t)p.n * p.m < (1ll << 31) && parts <= kColTeamMaxParts && tiles * parts <= kXchSlots;
     auto on_line = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 127u) == 0; };
     const bool lines = p.m % 64 == 0 && on_line(p.a) && on_line(p.g) && on_line(p.out);      // (a null pointer counts as aligned)
     if (wide) {
@@ -822,12 +850,13 @@ static int launch_col(int32_t batch, const ColArgs& p, void* stream, bool missin
                 }
                 if (rc != 0) return rc == kXchFull ? CPMK_ETOOBIG : rc;
             }
-            if (lines)
-                hipLaunchKernelGGL((k_col_team<KIND, true>), dim3((unsigned)xch_team_grid(tiles * nb, parts)), dim3(512), 0, (hipStream_t)stream, q,
-                                   (int32_t)tiles, (int32_t)parts, (uint32_t)(tiles * nb), xs.xl);
-            else
-                hipLaunchKernelGGL((k_col_team<KIND, false>), dim3((unsigned)xch_team_grid(tiles * nb, parts)), dim3(512), 0, (hipStream_t)stream, q,
-                                   (int32_t)tiles, (int32_t)parts, (uint32_t)(tiles * nb), xs.xl);
+            auto go = [&](auto kern) {
+                hipLaunchKernelGGL(kern, dim3((unsigned)xch_team_grid(tiles * nb, parts)), dim3(512), 0, (hipStream_t)stream, q, (int32_t)tiles,
+                                   (int32_t)parts, (uint32_t)(tiles * nb), xs.xl);
+            };
+            if (!vec16) go(k_col_team<KIND, 2>);
+            else if (lines) go(k_col_team<KIND, 0>);
+            else go(k_col_team<KIND, 1>);
             const int e = launch_status();
             const int rc2 = xs.end();
             if (e != 0 || rc2 != 0) return e ? e : rc2;

@@ -161,7 +161,8 @@ class GEMMInt8(torch.autograd.Function):
             # formed directly in the layout its operand came in, from operands with the contraction index
             # contiguous: no product on the general kernel and no transposition of a result.
             in_aT, in_bT = ctx.layout
-            qB_t = _transposed_copy_i8(quantized_B)                     # (bB, K, N)
+            qB_t = _rows_padded_i8(_transposed_copy_i8(quantized_B))    # (bB, K, N)
+            quant_G_a = _rows_padded_i8(quant_G_a)                      # both contracted over N
             if in_aT:       # grad_A (b, K, M) = qB_t x quant_G_a^T, scaled per column m
                 grad_A = gemm_and_scale(qB_t, None, quant_G_a, scale_G_a, False, True)
             else:           # grad_A (b, M, K) = quant_G_a x qB_t^T, scaled per row m
@@ -171,9 +172,9 @@ class GEMMInt8(torch.autograd.Function):
             quant_G_b = torch.empty((batch, m, n), dtype=torch.int8, device=grad_f.device)
             gemm_backward_scale_round(batch, m, n, grad_f.data_ptr(), scale_A.data_ptr(), quant_G_b.data_ptr(),
                                       scale_G_b.data_ptr(), scale_A.size(0) == 1, st)
-            qG_t = _transposed_copy_i8(quant_G_b)                       # (b, N, M)
+            qG_t = _rows_padded_i8(_transposed_copy_i8(quant_G_b))      # (b, N, M)
             del quant_G_b
-            qA_t = _transposed_copy_i8(quantized_A)                     # (bA, K, M)
+            qA_t = _rows_padded_i8(_transposed_copy_i8(quantized_A))    # (bA, K, M); both contracted over M
             if in_bT:       # grad_B (b, N, K) = qG_t x qA_t^T, scaled per row n
                 grad_B = gemm_and_scale(qG_t, scale_G_b, qA_t, None, False, True)
             else:           # grad_B (b, K, N) = qA_t x qG_t^T, scaled per column n
@@ -214,6 +215,19 @@ def _transposed_copy_i8(x: torch.Tensor) -> torch.Tensor:
     out = torch.empty((x.size(0), x.size(2), x.size(1)), dtype=torch.int8, device=x.device)
     transpose_i8(x.size(0), x.size(1), x.size(2), x.data_ptr(), out.data_ptr(), cur_stream())
     return out
+
+
+def _rows_padded_i8(x: torch.Tensor) -> torch.Tensor:
+    """A (b, r, k) operand that is contracted over k, with its rows lengthened by zeros to a multiple of 128
+    bytes when k is not a multiple of 64: padded on both operands of a product the zeros add nothing, and the
+    tile kernel's whole-slab path applies whatever k is (at k = 500 it is several times faster than the kernels
+    for ragged rows, and the copy costs two passes over the operand)."""
+    k = x.size(2)
+    if k % 64 == 0 or k < 128:
+        return x
+    padded = torch.zeros((x.size(0), x.size(1), (k + 127) // 128 * 128), dtype=torch.int8, device=x.device)
+    padded[:, :, :k].copy_(x)
+    return padded
 
 
 def _transposed_copy(x: torch.Tensor) -> torch.Tensor:

@@ -100,11 +100,14 @@ def test_bmm_backward(gpu, case, aT, bT, mode):
 @pytest.mark.parametrize("aT", [False, True])
 @pytest.mark.parametrize("bT", [False, True])
 @pytest.mark.parametrize("fused", [False, True])
-def test_bmm_int8_backward_bits(gpu, aT, bT, fused):
+# (the second case: M and N of at least 128 that are not multiples of 64 -- the fused backward then contracts over
+# rows lengthened with zeros)
+@pytest.mark.parametrize("dims", [(2, 24, 32, 20), (2, 200, 32, 132)])
+def test_bmm_int8_backward_bits(gpu, aT, bT, fused, dims):
     """Every step of GEMMInt8.backward restated with the oracle: bit-identical gradients."""
-    _name("bmm int8 backward bits", aT, bT, fused)
+    _name("bmm int8 backward bits", aT, bT, fused, dims)
     from cpm_kernels_amd.torch.gemm import bmm
-    batch, M, K, N = 2, 24, 32, 20
+    batch, M, K, N = dims
     rng = np.random.default_rng(aT * 2 + bT)
     A = (rng.standard_normal((batch, M, K)) / 2).astype(np.float16)          # logical (M, K)
     B = (rng.standard_normal((batch, N, K)) / 2).astype(np.float16)          # logical (N, K) = B^T

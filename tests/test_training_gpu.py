@@ -138,7 +138,8 @@ def test_gelu_backward(gpu, shape):
     assert_close_fp16(to_np(grad), ot.gelu_backward(g, x), rtol=1e-3, atol=1e-5, what="gelu_backward")
 
 
-COL_SHAPES = [(2, 64, 64), (3, 17, 100), (1, 1024, 96), (2, 5, 7), (1, 3000, 33)]
+# (widths that are not whole 16-byte pieces: multiples of 4, of 2, odd -- the register tiles then move 8, 4 or 2 bytes at a time)
+COL_SHAPES = [(2, 64, 64), (3, 17, 100), (1, 1024, 96), (2, 5, 7), (1, 3000, 33), (2, 700, 500), (1, 1100, 250), (2, 513, 1)]
 
 
 @pytest.mark.parametrize("shape", COL_SHAPES)
@@ -152,6 +153,54 @@ def test_softmax_backward(gpu, shape):
     grad = _empty((b, n, m), gpu)
     ck.softmax_backward(b, n, m, dev(out).data_ptr(), dev(g).data_ptr(), grad.data_ptr(), stream())
     assert_close_fp16(to_np(grad), ot.softmax_backward(out, g), rtol=2e-3, atol=1e-5, what="softmax_backward")
+
+
+def test_column_kernels_on_buffers_off_16_byte_boundaries(gpu):
+    """Every buffer starts 2 bytes (the int8 output 1 byte) past a 16-byte boundary: the register tiles fall back to
+    narrower accesses and must give the same bits as on aligned buffers."""
+    _name("column kernels, misaligned buffers")
+    b, n, m = 2, 600, 72
+    rng = np.random.default_rng(77)
+    x = rand_half(rng, (b, n, m)); g = rand_half(rng, (b, n, m))
+    sx = np.abs(rand_half(rng, (b, n), 0.02)) + np.float16(1e-3)
+
+    def off(arr, dtype=torch.half):
+        t = torch.from_numpy(arr).to(gpu)
+        buf = torch.zeros(t.numel() + 8, dtype=dtype, device=gpu)
+        v = buf[1:1 + t.numel()].view(t.shape)
+        v.copy_(t)
+        return v
+
+    def blank(shape, dtype=torch.half):
+        numel = int(np.prod(shape))
+        return torch.zeros(numel + 8, dtype=dtype, device=gpu)[1:1 + numel].view(shape)
+
+    xa, ga = to_gpu(x), to_gpu(g)
+    xo, go = off(x), off(g)
+    assert xo.data_ptr() % 16 == 2
+    for name, call in (
+        ("softmax_backward", lambda a, c, o: ck.softmax_backward(b, n, m, a.data_ptr(), c.data_ptr(), o.data_ptr(), stream())),
+    ):
+        o1, o2 = _empty((b, n, m), gpu), blank((b, n, m))
+        call(xa, ga, o1); call(xo, go, o2)
+        assert_bits_equal(to_np(o2.contiguous()), to_np(o1), name)
+    out1, var1 = _empty((b, n, m), gpu), _empty((b, m), gpu)
+    out2, var2 = blank((b, n, m)), blank((b, m))
+    ck.layernorm_forward_v(b, n, m, xa.data_ptr(), out1.data_ptr(), var1.data_ptr(), 1e-5, stream())
+    ck.layernorm_forward_v(b, n, m, xo.data_ptr(), out2.data_ptr(), var2.data_ptr(), 1e-5, stream())
+    assert_bits_equal(to_np(out2.contiguous()), to_np(out1), "forward_v out")
+    assert_bits_equal(to_np(var2.contiguous()), to_np(var1), "forward_v var")
+    gr1, gr2 = _empty((b, n, m), gpu), blank((b, n, m))
+    ck.layernorm_backward_v(b, n, m, xa.data_ptr(), ga.data_ptr(), var1.data_ptr(), gr1.data_ptr(), stream())
+    ck.layernorm_backward_v(b, n, m, xo.data_ptr(), go.data_ptr(), var2.data_ptr(), gr2.data_ptr(), stream())
+    assert_bits_equal(to_np(gr2.contiguous()), to_np(gr1), "backward_v")
+    q1, s1 = _empty((b, n, m), gpu, torch.int8), _empty((b, m), gpu)
+    q2, s2 = blank((b, n, m), torch.int8), blank((b, m))
+    sxa, sxo = to_gpu(sx), off(sx)
+    ck.gemm_backward_scale_round(b, n, m, xa.data_ptr(), sxa.data_ptr(), q1.data_ptr(), s1.data_ptr(), False, stream())
+    ck.gemm_backward_scale_round(b, n, m, xo.data_ptr(), sxo.data_ptr(), q2.data_ptr(), s2.data_ptr(), False, stream())
+    assert_bits_equal(to_np(q2.contiguous()), to_np(q1), "scale_round int8")
+    assert_bits_equal(to_np(s2.contiguous()), to_np(s1), "scale_round scale_y")
 
 
 def test_softmax_backward_more_teams_than_packet_slots(gpu):
