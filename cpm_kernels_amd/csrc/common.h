@@ -255,6 +255,9 @@ __device__ __forceinline__ void wait_vmcnt() {
 int gemv_f16_coalesced(int32_t batch, int32_t dim_out, int32_t dim_in, const void* mat, const void* vec, void* out, hipStream_t st);
 int gemv_f16_mfma(int32_t batch, int32_t dim_out, int32_t dim_in, const void* mat, const void* vec, void* out, hipStream_t st);
 
+// Column scales (cu_gemm_calc_scale_transpose) on the register-tile team kernel of train.hip: 0, an error code, or -1 (shape not taken)
+int col_absmax_team(int32_t batch, int32_t n, int32_t m, const void* mat, void* out, void* stream);
+
 // Compute units of the current device (cached per device ordinal; 256 if the query fails).  The cache
 // is atomic: host threads that make their first call together each ask the runtime and store the
 // same value.

@@ -205,15 +205,21 @@ struct RowsArgs {
 };
 
 // (the launcher counts on 8 resident workgroups per compute unit up to NV = 8, 4 beyond)
-template <int NV, bool QUANT>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NV <= 8 ? 8 : 4))) void k_rows(RowsArgs a) {
+// UA: rows that are not whole 16-byte pieces, or buffers off 16-byte boundaries: the eight elements of a piece move
+// four (m % 4 == 0, 8-byte aligned inputs, 4-byte aligned outputs), two (even m, 4- and 2-byte aligned) or one at a time.
+template <int NV, bool QUANT, bool UA = false>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(UA ? (NV <= 4 ? 8 : NV <= 8 ? 4 : 2) : (NV <= 8 ? 8 : 4)))) void k_rows(RowsArgs a) {
     const int lane = threadIdx.x & 63;
     const int64_t nw = (int64_t)gridDim.x * 4;
     const int64_t rows = a.rows0 + a.rows1;
     const int32_t m = a.m;
     int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= rows) return;
-    const int m8 = m >> 3;
+    const int m8 = UA ? (m + 7) >> 3 : m >> 3;
+    const uintptr_t in_bits = reinterpret_cast<uintptr_t>(a.mat0) | reinterpret_cast<uintptr_t>(a.mat1);
+    const uintptr_t out_bits = reinterpret_cast<uintptr_t>(a.out0) | reinterpret_cast<uintptr_t>(a.out1);
+    const bool quads = UA && (m & 3) == 0 && (in_bits & 7u) == 0 && (out_bits & 3u) == 0;
+    const bool pairs = UA && (m & 1) == 0 && (in_bits & 3u) == 0 && (out_bits & 1u) == 0;
     half8_t cur[NV];
     auto load = [&](half8_t (&v)[NV], int64_t r) __attribute__((always_inline)) {
         const half_t* mat = r < a.rows0 ? a.mat0 + r * m : a.mat1 + (r - a.rows0) * m;
@@ -223,7 +229,49 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NV <= 8 ? 8
             const int j = lane + i * 64;
 #pragma unroll
             for (int e = 0; e < 8; ++e) v[i][e] = (half_t)0.0f;
-            if (j < m8) v[i] = __builtin_nontemporal_load(p8 + j);
+            if constexpr (!UA) {
+                if (j < m8) v[i] = __builtin_nontemporal_load(p8 + j);
+            } else if (quads) {
+#pragma unroll
+                for (int e = 0; e < 8; e += 4)
+                    if (j * 8 + e < m) {
+                        const half4_t t = *reinterpret_cast<const half4_t*>(mat + j * 8 + e);
+#pragma unroll
+                        for (int d = 0; d < 4; ++d) v[i][e + d] = t[d];
+                    }
+            } else if (pairs) {
+#pragma unroll
+                for (int e = 0; e < 8; e += 2)
+                    if (j * 8 + e < m) {
+                        const half2_t t = *reinterpret_cast<const half2_t*>(mat + j * 8 + e);
+                        v[i][e] = t[0];
+                        v[i][e + 1] = t[1];
+                    }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (j * 8 + e < m) v[i][e] = mat[j * 8 + e];
+            }
+        }
+    };
+    // piece j (eight int8 in w) of the output row at `orow`
+    auto store = [&](int8_t* orow, int j, uint2_t w) __attribute__((always_inline)) {
+        if constexpr (!UA) {
+            reinterpret_cast<uint2_t*>(orow)[j] = w;
+        } else if (quads) {
+            *reinterpret_cast<uint32_t*>(orow + j * 8) = w.x;
+            if (j * 8 + 4 < m) *reinterpret_cast<uint32_t*>(orow + j * 8 + 4) = w.y;
+        } else {
+            const uint64_t bits = (uint64_t)w.x | ((uint64_t)w.y << 32);
+            if (pairs) {
+#pragma unroll
+                for (int e = 0; e < 8; e += 2)
+                    if (j * 8 + e < m) *reinterpret_cast<uint16_t*>(orow + j * 8 + e) = (uint16_t)(bits >> (8 * e));
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (j * 8 + e < m) orow[j * 8 + e] = (int8_t)(bits >> (8 * e));
+            }
         }
     };
     load(cur, row);
@@ -256,7 +304,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NV <= 8 ? 8
         if (lane == 0) (second ? a.scale1 : a.scale0)[lrow] = sh;
         if (QUANT) {
             const float s = (float)sh, y = 1.0f / s;
-            uint2_t* o8 = reinterpret_cast<uint2_t*>((second ? a.out1 : a.out0) + lrow * m);
+            int8_t* const orow = (second ? a.out1 : a.out0) + lrow * m;
             if (scale_is_normal(sh)) {       // (the same for the whole wave) the short rounding sequence
 #pragma unroll
                 for (int i = 0; i < NV; ++i) {
@@ -270,7 +318,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NV <= 8 ? 8
                     uint2_t w;
                     w.x = pack4_i8((int32_t)q[0], (int32_t)q[1], (int32_t)q[2], (int32_t)q[3]);
                     w.y = pack4_i8((int32_t)q[4], (int32_t)q[5], (int32_t)q[6], (int32_t)q[7]);
-                    if (j < m8) o8[j] = w;
+                    if (j < m8) store(orow, j, w);
                 }
             } else {
 #pragma unroll
@@ -283,7 +331,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NV <= 8 ? 8
                         uint2_t w;
                         w.x = pack4_i8(q[0], q[1], q[2], q[3]);
                         w.y = pack4_i8(q[4], q[5], q[6], q[7]);
-                        o8[j] = w;
+                        store(orow, j, w);
                     }
                 }
             }
@@ -314,14 +362,14 @@ static unsigned rows_grid(int64_t rows, int cus, int nv) {
     return (unsigned)best;
 }
 
-template <bool QUANT>
+template <bool QUANT, bool UA = false>
 static void launch_rows(const RowsArgs& ra, int nv, hipStream_t st) {
     const dim3 g(rows_grid(ra.rows0 + ra.rows1, compute_units(), nv));
-    if (nv <= 1) hipLaunchKernelGGL((k_rows<1, QUANT>), g, dim3(256), 0, st, ra);
-    else if (nv <= 2) hipLaunchKernelGGL((k_rows<2, QUANT>), g, dim3(256), 0, st, ra);
-    else if (nv <= 4) hipLaunchKernelGGL((k_rows<4, QUANT>), g, dim3(256), 0, st, ra);
-    else if (nv <= 8) hipLaunchKernelGGL((k_rows<8, QUANT>), g, dim3(256), 0, st, ra);
-    else hipLaunchKernelGGL((k_rows<16, QUANT>), g, dim3(256), 0, st, ra);
+    if (nv <= 1) hipLaunchKernelGGL((k_rows<1, QUANT, UA>), g, dim3(256), 0, st, ra);
+    else if (nv <= 2) hipLaunchKernelGGL((k_rows<2, QUANT, UA>), g, dim3(256), 0, st, ra);
+    else if (nv <= 4) hipLaunchKernelGGL((k_rows<4, QUANT, UA>), g, dim3(256), 0, st, ra);
+    else if (nv <= 8) hipLaunchKernelGGL((k_rows<8, QUANT, UA>), g, dim3(256), 0, st, ra);
+    else hipLaunchKernelGGL((k_rows<16, QUANT, UA>), g, dim3(256), 0, st, ra);
 }
 
 static int check3(int32_t batch, int32_t n, int32_t m) {
@@ -342,9 +390,10 @@ static int row_absmax(int64_t rows, int32_t m, const void* mat, void* out, hipSt
         else hipLaunchKernelGGL((k_row_absmax<256, false>), dim3((unsigned)rows), dim3(256), 0, st, rows, m, p, o);
     } else {
         const int nv = (int)ceil_div(m, 512);
-        if (vec && nv <= 16) {
+        if (nv <= 16) {
             const RowsArgs ra = {p, o, nullptr, rows, nullptr, nullptr, nullptr, 0, m};
-            launch_rows<false>(ra, nv, st);
+            if (vec) launch_rows<false>(ra, nv, st);
+            else launch_rows<false, true>(ra, nv, st);
             return launch_status();
         }
         if (!grid_fits(ceil_div(rows, 4))) return CPMK_ETOOBIG;
@@ -420,6 +469,10 @@ int cpmk_gemm_calc_scale_transpose(int32_t batch, int32_t n, int32_t m, const vo
     if (int e = check3(batch, n, m)) return e;
     if (batch == 0 || m == 0) return 0;
     if (any_null(out) || (n > 0 && mat == nullptr)) return CPMK_EBADARG;
+    if (n > 0) {        // columns in registers, tall ones shared by a team of workgroups
+        const int rc = col_absmax_team(batch, n, m, mat, out, stream);
+        if (rc >= 0) return rc;
+    }
     const bool vec = (m % 8 == 0) && aligned16(mat);
     for (int64_t b0 = 0; b0 < batch; b0 += 65535) {       // (grid y: at most 65535 batch entries per launch)
         const int64_t nb = batch - b0 < 65535 ? batch - b0 : 65535;
@@ -484,9 +537,10 @@ int cpmk_gemm_quantize(int32_t batch, int32_t n, int32_t m, const void* mat, voi
         if (rows == 0) return 0;
         if (any_null(scale) || (m > 0 && any_null(mat, out))) return CPMK_EBADARG;
         const bool vec = (m % 8 == 0) && aligned16(mat) && ((reinterpret_cast<uintptr_t>(out) & 7u) == 0);
-        if (vec && m <= 64 * 8 * 16) {
+        if (m > 0 && m <= 64 * 8 * 16) {
             const RowsArgs ra = {(const half_t*)mat, (half_t*)scale, (int8_t*)out, rows, nullptr, nullptr, nullptr, 0, m};
-            launch_rows<true>(ra, (int)ceil_div(m, 512), st);
+            if (vec) launch_rows<true>(ra, (int)ceil_div(m, 512), st);
+            else launch_rows<true, true>(ra, (int)ceil_div(m, 512), st);
             return launch_status();
         }
         if (int e = cpmk_gemm_calc_scale(batch, n, m, mat, scale, stream)) return e;
@@ -501,12 +555,14 @@ int cpmk_gemm_quantize_pair(int64_t rows0, const void* mat0, void* scale0, void*
     if (rows0 < 0 || rows1 < 0 || m < 0 || rows0 > 0x7fffffff || rows1 > 0x7fffffff) return CPMK_EBADARG;
     if (m == 0 || rows0 + rows1 == 0) return 0;
     if ((rows0 > 0 && any_null(mat0, scale0, out0)) || (rows1 > 0 && any_null(mat1, scale1, out1))) return CPMK_EBADARG;
-    const bool vec = (m % 8 == 0) && m <= 64 * 8 * 16 && (rows0 == 0 || (aligned16(mat0) && (reinterpret_cast<uintptr_t>(out0) & 7u) == 0)) &&
+    const bool vec = (m % 8 == 0) && (rows0 == 0 || (aligned16(mat0) && (reinterpret_cast<uintptr_t>(out0) & 7u) == 0)) &&
                      (rows1 == 0 || (aligned16(mat1) && (reinterpret_cast<uintptr_t>(out1) & 7u) == 0));
-    if (vec) {
-        const RowsArgs ra = {(const half_t*)mat0, (half_t*)scale0, (int8_t*)out0, rows0,
-                             (const half_t*)mat1, (half_t*)scale1, (int8_t*)out1, rows1, m};
-        launch_rows<true>(ra, (int)ceil_div(m, 512), (hipStream_t)stream);
+    if (m <= 64 * 8 * 16) {
+        // (an absent tensor's pointers count as aligned in the kernel's choice of access width)
+        const RowsArgs ra = {rows0 ? (const half_t*)mat0 : nullptr, (half_t*)scale0, rows0 ? (int8_t*)out0 : nullptr, rows0,
+                             rows1 ? (const half_t*)mat1 : nullptr, (half_t*)scale1, rows1 ? (int8_t*)out1 : nullptr, rows1, m};
+        if (vec) launch_rows<true>(ra, (int)ceil_div(m, 512), (hipStream_t)stream);
+        else launch_rows<true, true>(ra, (int)ceil_div(m, 512), (hipStream_t)stream);
         return launch_status();
     }
     if (rows0 > 0)

@@ -176,7 +176,8 @@ __global__ __launch_bounds__(256) void k_ln_backward(int64_t batch, int64_t n, i
 // Reductions over dim 1 of (batch, n, m) followed by an elementwise pass.  Workgroup = 64
 // columns x 4 row groups; gridDim = (ceil(m/64), batch).
 // ---------------------------------------------------------------------------------------
-enum : int { kLnFwdV = 0, kLnFwdMV = 1, kLnBwdV = 2, kLnBwdMV = 3, kSoftmaxBwd = 4, kScaleRound = 5 };
+// (kColAbsmax: the column scales alone, cu_gemm_calc_scale_transpose; only the team kernel below knows it)
+enum : int { kLnFwdV = 0, kLnFwdMV = 1, kLnBwdV = 2, kLnBwdMV = 3, kSoftmaxBwd = 4, kScaleRound = 5, kColAbsmax = 6 };
 
 struct ColArgs {
     int32_t n, m;
@@ -272,8 +273,8 @@ __global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_b
     const uint32_t tag = xl.tag;
     constexpr int NT = 512, LPR = 8, R = 8;
     using T = ColTile<NT, LPR, R>;
-    constexpr bool TWO = KIND != kLnFwdV && KIND != kLnFwdMV && KIND != kScaleRound;     // reads grad_in too
-    constexpr bool IS_MAX = KIND == kScaleRound;
+    constexpr bool TWO = KIND != kLnFwdV && KIND != kLnFwdMV && KIND != kScaleRound && KIND != kColAbsmax;     // reads grad_in too
+    constexpr bool IS_MAX = KIND == kScaleRound || KIND == kColAbsmax;
     constexpr int NV = (KIND == kLnFwdMV || KIND == kLnBwdMV) ? 2 : 1;      // statistics per column
     __shared__ float lds[(T::NW + 1) * T::COLS * NV];
     __shared__ float tot[T::COLS * 2];
@@ -353,6 +354,7 @@ __global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_b
             else if constexpr (KIND == kLnBwdV) s[e] += gi * c3[e] * x;
             else if constexpr (KIND == kLnBwdMV) { s[e] += gi * c3[e] * (x - mean[e]); s[8 + e] += -gi * var[e]; }
             else if constexpr (KIND == kSoftmaxBwd) s[e] += x * gi;
+            else if constexpr (KIND == kColAbsmax) s[e] = fmaxf(s[e], fabsf(x));
             else s[e] = fmaxf(s[e], fabsf(x * sxv[q]));
         }
     if (parts == 1) {
@@ -398,8 +400,15 @@ __global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_b
         if (KIND == kLnFwdV || KIND == kLnFwdMV) store8(p.out_var + (int64_t)b * p.m + col0, h1);
         if (KIND == kLnFwdMV) store8(p.out_mean + (int64_t)b * p.m + col0, h0);
         if (KIND == kScaleRound) store8(p.out_var + (int64_t)b * p.m + col0, h0);
+        if constexpr (KIND == kColAbsmax) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) h0[e] = scale_from_absmax(s[e]);
+            store8(p.out_var + (int64_t)b * p.m + col0, h0);
+        }
     }
-    if constexpr (KIND == kScaleRound) {
+    if constexpr (KIND == kColAbsmax) {
+        // the scales are all there is to write
+    } else if constexpr (KIND == kScaleRound) {
         if (live) {
 #pragma unroll
             for (int q = 0; q < R; ++q) {
@@ -488,13 +497,45 @@ __global__ __launch_bounds__(256) void k_round_scale_rows_wide(int64_t rows, int
 // The same for rows of at most 2048 columns, kept in registers: a wave takes U consecutive rows of P 16-byte pieces
 // per lane (P * U = 4 loads in flight per lane, the matrix read once and with the non-temporal hint), finds each
 // row's maximum over the wave with data-parallel-primitive operands and rounds from the registers.
-template <int P, int U>
+// UA: rows that are not whole 16-byte pieces or buffers off 16-byte boundaries -- the eight columns of a piece then
+// move four (m % 4 == 0, 8-byte aligned buffers), two (even m, 4-byte aligned) or one at a time.
+template <int P, int U, bool UA>
 __global__ __launch_bounds__(256) void k_round_scale_rows_reg(int64_t rows, int32_t n, int32_t m, const half_t* __restrict__ mat,
                                                               const half_t* __restrict__ scale_y, int8_t* __restrict__ out,
                                                               half_t* __restrict__ scale_x, int bc) {
     const int lane = threadIdx.x & 63;
     const int64_t row0 = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * U;
     if (row0 >= rows) return;
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(mat) | reinterpret_cast<uintptr_t>(scale_y);
+    const bool quads = UA && (m & 3) == 0 && (bits & 7u) == 0 && (reinterpret_cast<uintptr_t>(out) & 3u) == 0;
+    const bool pairs = UA && (m & 1) == 0 && (bits & 3u) == 0 && (reinterpret_cast<uintptr_t>(out) & 1u) == 0;
+    auto load8 = [&](const half_t* src, int32_t j, bool nt) __attribute__((always_inline)) {
+        half8_t r = {0, 0, 0, 0, 0, 0, 0, 0};
+        if constexpr (!UA) {
+            r = nt ? __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(src + j)) : *reinterpret_cast<const half8_t*>(src + j);
+        } else if (quads) {
+#pragma unroll
+            for (int e = 0; e < 8; e += 4)
+                if (j + e < m) {
+                    const half4_t t = *reinterpret_cast<const half4_t*>(src + j + e);
+#pragma unroll
+                    for (int d = 0; d < 4; ++d) r[e + d] = t[d];
+                }
+        } else if (pairs) {
+#pragma unroll
+            for (int e = 0; e < 8; e += 2)
+                if (j + e < m) {
+                    const half2_t t = *reinterpret_cast<const half2_t*>(src + j + e);
+                    r[e] = t[0];
+                    r[e + 1] = t[1];
+                }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (j + e < m) r[e] = src[j + e];
+        }
+        return r;
+    };
     half8_t xv[U][P], sv[U][P];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -506,8 +547,8 @@ __global__ __launch_bounds__(256) void k_round_scale_rows_reg(int64_t rows, int3
             const int32_t j = lane * 8 + p * 512;
             xv[u][p] = sv[u][p] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
             if (j < m) {
-                xv[u][p] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(x + j));
-                sv[u][p] = *reinterpret_cast<const half8_t*>(sy + j);
+                xv[u][p] = load8(x, j, true);
+                sv[u][p] = load8(sy, j, false);
             }
         }
     }
@@ -530,7 +571,21 @@ __global__ __launch_bounds__(256) void k_round_scale_rows_reg(int64_t rows, int3
                     int32_t t[8];
 #pragma unroll
                     for (int e = 0; e < 8; ++e) t[e] = quant_i8((float)xv[u][p][e] * (float)sv[u][p][e], s);
-                    *reinterpret_cast<uint2_t*>(out + row * m + j) = uint2_t{pack4_i8(t[0], t[1], t[2], t[3]), pack4_i8(t[4], t[5], t[6], t[7])};
+                    int8_t* dst = out + row * m + j;
+                    if constexpr (!UA) {
+                        *reinterpret_cast<uint2_t*>(dst) = uint2_t{pack4_i8(t[0], t[1], t[2], t[3]), pack4_i8(t[4], t[5], t[6], t[7])};
+                    } else if (quads) {
+                        *reinterpret_cast<uint32_t*>(dst) = pack4_i8(t[0], t[1], t[2], t[3]);
+                        if (j + 4 < m) *reinterpret_cast<uint32_t*>(dst + 4) = pack4_i8(t[4], t[5], t[6], t[7]);
+                    } else if (pairs) {
+#pragma unroll
+                        for (int e = 0; e < 8; e += 2)
+                            if (j + e < m) *reinterpret_cast<uint16_t*>(dst + e) = (uint16_t)((t[e] & 0xff) | ((t[e + 1] & 0xff) << 8));
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            if (j + e < m) dst[e] = (int8_t)t[e];
+                    }
                 }
             }
         }
@@ -863,14 +918,24 @@ static int launch_col(int32_t batch, const ColArgs& p, void* stream, bool missin
         }
         if (!no_slots) return 0;
     }
-    // the batch is the grid's y dimension (at most 65535): larger batches go out in several launches
-    for (int64_t b0 = 0; b0 < batch; b0 += 65535) {
-        const int64_t nb = batch - b0 < 65535 ? batch - b0 : 65535;
-        hipLaunchKernelGGL((k_col<KIND>), dim3((unsigned)ceil_div(p.m, 64), (unsigned)nb), dim3(256), 0, (hipStream_t)stream,
-                           col_args_from(p, b0));
-        if (int e = launch_status()) return e;
+    if constexpr (KIND == kColAbsmax) {
+        return -1;      // (the caller has a kernel of its own for what the team kernel does not take)
+    } else {
+        // the batch is the grid's y dimension (at most 65535): larger batches go out in several launches
+        for (int64_t b0 = 0; b0 < batch; b0 += 65535) {
+            const int64_t nb = batch - b0 < 65535 ? batch - b0 : 65535;
+            hipLaunchKernelGGL((k_col<KIND>), dim3((unsigned)ceil_div(p.m, 64), (unsigned)nb), dim3(256), 0, (hipStream_t)stream,
+                               col_args_from(p, b0));
+            if (int e = launch_status()) return e;
+        }
+        return 0;
     }
-    return 0;
+}
+
+// Column scales of (batch, n, m) on the team kernel: 0, an error code, or -1 when the shape is not one it takes.
+int col_absmax_team(int32_t batch, int32_t n, int32_t m, const void* mat, void* out, void* stream) {
+    ColArgs p = {n, m, (const half_t*)mat, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, (half_t*)out, 0.0f, 0};
+    return launch_col<kColAbsmax>(batch, p, stream, false);
 }
 
 }  // namespace cpmk
@@ -1023,18 +1088,23 @@ int cpmk_gemm_backward_round_scale(int32_t batch, int32_t n, int32_t m, const vo
     if (rows == 0) return 0;
     if (rows > 0x7fffffff) return CPMK_ETOOBIG;
     if (scale_x == nullptr || (m > 0 && any_null(mat, scale_y, out))) return CPMK_EBADARG;
-    if (m % 8 == 0 && aligned16(mat) && aligned16(scale_y) && (reinterpret_cast<uintptr_t>(out) & 7u) == 0) {
-        if (m <= 2048) {      // rows that a wave holds in registers
-            auto go = [&](auto pc, auto uc) {
-                constexpr int P = decltype(pc)::value, U = decltype(uc)::value;
-                hipLaunchKernelGGL((k_round_scale_rows_reg<P, U>), dim3((unsigned)ceil_div(rows, 4 * U)), dim3(256), 0, (hipStream_t)stream, rows, n,
-                                   m, (const half_t*)mat, (const half_t*)scale_y, (int8_t*)out, (half_t*)scale_x, broad_cast_y);
+    const bool vec16 = m % 8 == 0 && aligned16(mat) && aligned16(scale_y) && (reinterpret_cast<uintptr_t>(out) & 7u) == 0;
+    if (m > 0 && m <= 2048) {      // rows that a wave holds in registers
+        auto go = [&](auto pc, auto uc) {
+            constexpr int P = decltype(pc)::value, U = decltype(uc)::value;
+            auto run = [&](auto kern) {
+                hipLaunchKernelGGL(kern, dim3((unsigned)ceil_div(rows, 4 * U)), dim3(256), 0, (hipStream_t)stream, rows, n, m, (const half_t*)mat,
+                                   (const half_t*)scale_y, (int8_t*)out, (half_t*)scale_x, broad_cast_y);
             };
-            if (m <= 512) go(std::integral_constant<int, 1>{}, std::integral_constant<int, 4>{});
-            else if (m <= 1024) go(std::integral_constant<int, 2>{}, std::integral_constant<int, 2>{});
-            else go(std::integral_constant<int, 4>{}, std::integral_constant<int, 1>{});
-            return launch_status();
-        }
+            if (vec16) run(k_round_scale_rows_reg<P, U, false>);
+            else run(k_round_scale_rows_reg<P, U, true>);
+        };
+        if (m <= 512) go(std::integral_constant<int, 1>{}, std::integral_constant<int, 4>{});
+        else if (m <= 1024) go(std::integral_constant<int, 2>{}, std::integral_constant<int, 2>{});
+        else go(std::integral_constant<int, 4>{}, std::integral_constant<int, 1>{});
+        return launch_status();
+    }
+    if (vec16) {
         hipLaunchKernelGGL(k_round_scale_rows_wide, dim3((unsigned)ceil_div(rows, 4)), dim3(256), 0, (hipStream_t)stream, rows, n, m,
                            (const half_t*)mat, (const half_t*)scale_y, (int8_t*)out, (half_t*)scale_x, broad_cast_y);
         return launch_status();

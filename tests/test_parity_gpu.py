@@ -45,7 +45,9 @@ QUANT_SHAPES = [(1, 512, 4096), (3, 17, 1000), (2, 5, 7), (1, 1, 8), (2, 64, 48)
                 (1, 2100, 128), (1, 3, 20480), (2, 4096, 192), (1, 1032, 72), (3, 520, 8),
                 (1, 10240, 192), (2, 16384, 64), (1, 16392, 64),
                 # tall columns in widths that are not whole 16-byte pieces (the team kernel, one column at a time)
-                (2, 4096, 500), (1, 1040, 77), (1, 2100, 36)]
+                (2, 4096, 500), (1, 1040, 77), (1, 2100, 36),
+                # rows in registers moving 4 or 2 bytes or one element at a time, up to the longest such rows
+                (3, 33, 250), (2, 9, 8190), (1, 5, 8191), (2, 40, 4100)]
 
 
 @pytest.mark.parametrize("shape", QUANT_SHAPES)

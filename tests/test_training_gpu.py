@@ -201,6 +201,13 @@ def test_column_kernels_on_buffers_off_16_byte_boundaries(gpu):
     ck.gemm_backward_scale_round(b, n, m, xo.data_ptr(), sxo.data_ptr(), q2.data_ptr(), s2.data_ptr(), False, stream())
     assert_bits_equal(to_np(q2.contiguous()), to_np(q1), "scale_round int8")
     assert_bits_equal(to_np(s2.contiguous()), to_np(s1), "scale_round scale_y")
+    sy = np.abs(rand_half(rng, (b, m), 0.02)) + np.float16(1e-3)
+    r1, r2 = _empty((b, n), gpu), blank((b, n))
+    sya, syo = to_gpu(sy), off(sy)
+    ck.gemm_backward_round_scale(b, n, m, xa.data_ptr(), sya.data_ptr(), q1.data_ptr(), r1.data_ptr(), False, stream())
+    ck.gemm_backward_round_scale(b, n, m, xo.data_ptr(), syo.data_ptr(), q2.data_ptr(), r2.data_ptr(), False, stream())
+    assert_bits_equal(to_np(q2.contiguous()), to_np(q1), "round_scale int8")
+    assert_bits_equal(to_np(r2.contiguous()), to_np(r1), "round_scale scale_x")
 
 
 def test_softmax_backward_more_teams_than_packet_slots(gpu):
