@@ -87,15 +87,32 @@ __global__ __launch_bounds__(256) void k_col_absmax(int32_t n, int32_t m,
 
 // ---------------------------------------------------------------------------------------
 // rounding: out = int8(rint(x / scale)).  MODE 0: scale per row (index = element / m),
-// MODE 1: scale per (batch, column) (index = b*m + j).  VEC: 16 elements per thread.
+// MODE 1: scale per (batch, column) (index = b*m + j).  W elements per thread: 16 (m % 16 == 0, 16-byte aligned
+// buffers), 4 (m % 4 == 0, 8-byte aligned input and scales, 4-byte aligned output) or 1.
 // ---------------------------------------------------------------------------------------
-template <int MODE, bool VEC>
+template <int MODE, int W>
 __global__ __launch_bounds__(256) void k_round(int64_t total, int32_t n, int32_t m,
                                                const half_t* __restrict__ mat,
                                                const half_t* __restrict__ scale,
                                                int8_t* __restrict__ out) {
     const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (VEC) {
+    if constexpr (W == 4) {
+        const int64_t e0 = gid * 4;
+        if (e0 >= total) return;
+        const int64_t row = e0 / m;            // m % 4 == 0: the 4 elements share a row
+        const half4_t a = __builtin_nontemporal_load(reinterpret_cast<const half4_t*>(mat + e0));
+        int32_t q[4];
+        if (MODE == 0) {
+            const float sr = (float)scale[row], y = 1.0f / sr;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) q[e] = quant_i8_rcp((float)a[e], sr, y);
+        } else {
+            const half4_t sv = *reinterpret_cast<const half4_t*>(scale + (row / n) * m + (e0 - row * m));
+#pragma unroll
+            for (int e = 0; e < 4; ++e) q[e] = quant_i8((float)a[e], (float)sv[e]);
+        }
+        *reinterpret_cast<uint32_t*>(out + e0) = pack4_i8(q[0], q[1], q[2], q[3]);
+    } else if constexpr (W == 16) {
         const int64_t e0 = gid * 16;
         if (e0 >= total) return;
         const int64_t row = e0 / m;            // m % 16 == 0: the 16 elements share a row
@@ -148,16 +165,18 @@ __global__ __launch_bounds__(256) void k_round(int64_t total, int32_t n, int32_t
 // ---------------------------------------------------------------------------------------
 // dequantisation: out = fp16((f32(acc) * sx) * sy)
 // MODE 0: both scales (cu_gemm_scale), MODE 1: scale_x only, MODE 2: scale_y only.
-// VEC: 8 elements per thread (two 16-byte loads, one 16-byte store), m % 8 == 0.
+// W elements per thread: 8 (two 16-byte loads, one 16-byte store; m % 8 == 0), 4 (m % 4 == 0, 8-byte aligned
+// output and column scales) or 1.
 // ---------------------------------------------------------------------------------------
-template <int MODE, bool VEC>
+template <int MODE, int W>
 __global__ __launch_bounds__(256) void k_dequant(int64_t total, int32_t n, int32_t m,
                                                  const int32_t* __restrict__ mat,
                                                  const half_t* __restrict__ scale_x,
                                                  const half_t* __restrict__ scale_y,
                                                  half_t* __restrict__ out, int bcx, int bcy) {
     const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    const int64_t e0 = VEC ? gid * 8 : gid;
+    constexpr bool VEC = W == 8;
+    const int64_t e0 = gid * W;
     if (e0 >= total) return;
     const int64_t row = e0 / m;                // = b*n + i
     const int32_t j0 = (int32_t)(e0 - row * m);
@@ -180,6 +199,18 @@ __global__ __launch_bounds__(256) void k_dequant(int64_t total, int32_t n, int32
             else o[e] = round_f16((float)acc * (float)syv[e]);
         }
         *reinterpret_cast<half8_t*>(out + e0) = o;
+    } else if (W == 4) {
+        const int4_t a0 = __builtin_nontemporal_load(reinterpret_cast<const int4_t*>(mat + e0));
+        half4_t syv = {0, 0, 0, 0};
+        if (MODE != 1) syv = *reinterpret_cast<const half4_t*>(sy);
+        half4_t o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if (MODE == 0) o[e] = dequant(a0[e], sx, (float)syv[e]);
+            else if (MODE == 1) o[e] = round_f16(sx * (float)a0[e]);
+            else o[e] = round_f16((float)a0[e] * (float)syv[e]);
+        }
+        *reinterpret_cast<half4_t*>(out + e0) = o;
     } else {
         const int32_t acc = mat[e0];
         if (MODE == 0) out[e0] = dequant(acc, sx, (float)sy[0]);
@@ -410,16 +441,21 @@ static int round_launch(int32_t batch, int32_t n, int32_t m, const void* mat, co
     const int64_t total = (int64_t)batch * n * m;
     if (total == 0) return 0;
     if (any_null(mat, scale, out)) return CPMK_EBADARG;
+    auto low = [](const void* q, uintptr_t mask) { return (reinterpret_cast<uintptr_t>(q) & mask) == 0; };
     const bool vec = (m % 16 == 0) && aligned16(mat) && aligned16(out) && (MODE == 0 || aligned16(scale));
+    const bool quads = (m % 4 == 0) && low(mat, 7) && low(out, 3) && (MODE == 0 || low(scale, 7));
     const half_t* p = (const half_t*)mat;
     const half_t* s = (const half_t*)scale;
     int8_t* o = (int8_t*)out;
     if (vec) {
         const int64_t g = ceil_div(total / 16, 256);
-        hipLaunchKernelGGL((k_round<MODE, true>), dim3((unsigned)g), dim3(256), 0, st, total, n, m, p, s, o);
+        hipLaunchKernelGGL((k_round<MODE, 16>), dim3((unsigned)g), dim3(256), 0, st, total, n, m, p, s, o);
+    } else if (quads) {
+        const int64_t g = ceil_div(total / 4, 256);
+        hipLaunchKernelGGL((k_round<MODE, 4>), dim3((unsigned)g), dim3(256), 0, st, total, n, m, p, s, o);
     } else {
         const int64_t g = ceil_div(total, 256);
-        hipLaunchKernelGGL((k_round<MODE, false>), dim3((unsigned)g), dim3(256), 0, st, total, n, m, p, s, o);
+        hipLaunchKernelGGL((k_round<MODE, 1>), dim3((unsigned)g), dim3(256), 0, st, total, n, m, p, s, o);
     }
     return launch_status();
 }
@@ -430,16 +466,16 @@ static int dequant_launch(int32_t batch, int32_t n, int32_t m, const void* mat, 
     const int64_t total = (int64_t)batch * n * m;
     if (total == 0) return 0;
     if (any_null(mat, out) || (MODE != 2 && sx == nullptr) || (MODE != 1 && sy == nullptr)) return CPMK_EBADARG;
+    auto low = [](const void* q, uintptr_t mask) { return (reinterpret_cast<uintptr_t>(q) & mask) == 0; };
     const bool vec = (m % 8 == 0) && aligned16(mat) && aligned16(out) && (MODE == 1 || aligned16(sy));
-    if (vec) {
-        const int64_t g = ceil_div(total / 8, 256);
-        hipLaunchKernelGGL((k_dequant<MODE, true>), dim3((unsigned)g), dim3(256), 0, st, total, n, m,
-                           (const int32_t*)mat, (const half_t*)sx, (const half_t*)sy, (half_t*)out, bcx, bcy);
-    } else {
-        const int64_t g = ceil_div(total, 256);
-        hipLaunchKernelGGL((k_dequant<MODE, false>), dim3((unsigned)g), dim3(256), 0, st, total, n, m,
-                           (const int32_t*)mat, (const half_t*)sx, (const half_t*)sy, (half_t*)out, bcx, bcy);
-    }
+    const bool quads = (m % 4 == 0) && aligned16(mat) && low(out, 7) && (MODE == 1 || low(sy, 7));
+    auto go = [&](auto kern, int w) {
+        hipLaunchKernelGGL(kern, dim3((unsigned)ceil_div(total / w, 256)), dim3(256), 0, st, total, n, m, (const int32_t*)mat,
+                           (const half_t*)sx, (const half_t*)sy, (half_t*)out, bcx, bcy);
+    };
+    if (vec) go(k_dequant<MODE, 8>, 8);
+    else if (quads) go(k_dequant<MODE, 4>, 4);
+    else go(k_dequant<MODE, 1>, 1);
     return launch_status();
 }
 

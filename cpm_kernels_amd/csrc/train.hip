@@ -419,9 +419,14 @@ __global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_b
                     for (int e = 0; e < 8; ++e) t[e] = quant_i8((float)va[q][e] * sxv[q], k0[e]);
                     int8_t* dst = p.out_i8 + boff + ((uint32_t)lrow * (uint32_t)p.m + (uint32_t)col0);
                     if constexpr (UA) {
+                        if ((p.m & 3) == 0 && (reinterpret_cast<uintptr_t>(p.out_i8) & 3u) == 0) {       // whole dwords
+                            *reinterpret_cast<uint32_t*>(dst) = pack4_i8(t[0], t[1], t[2], t[3]);
+                            if (col0 + 4 < p.m) *reinterpret_cast<uint32_t*>(dst + 4) = pack4_i8(t[4], t[5], t[6], t[7]);
+                        } else {
 #pragma unroll
-                        for (int e = 0; e < 8; ++e)
-                            if (col0 + e < p.m) dst[e] = (int8_t)t[e];
+                            for (int e = 0; e < 8; ++e)
+                                if (col0 + e < p.m) dst[e] = (int8_t)t[e];
+                        }
                     } else {
                         *reinterpret_cast<uint2_t*>(dst) = uint2_t{pack4_i8(t[0], t[1], t[2], t[3]), pack4_i8(t[4], t[5], t[6], t[7])};
                     }

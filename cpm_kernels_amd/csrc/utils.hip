@@ -46,22 +46,38 @@ __global__ __launch_bounds__(256) void k_transpose_wide(int32_t n, int32_t m, co
     }
 }
 
-// (batch, n, m) -> (batch, m, n) of bytes: 64x64 tile through LDS, 16-byte global accesses where
-// the shape allows (WIDE: n % 16 == 0, m % 16 == 0, aligned pointers), single bytes otherwise.
-template <bool WIDE>
+// (batch, n, m) -> (batch, m, n) of bytes: 64x64 tile through LDS.  IN / OUT: bytes per global load / store -- 16 where
+// the rows of that side are whole 16-byte pieces on 16-byte boundaries (m % 16 == 0 for the loads, n % 16 == 0 for the
+// stores), 4 where they are whole dwords, else single bytes; the two sides choose independently.
+template <int IN, int OUT>
 __global__ __launch_bounds__(256) void k_transpose_i8(int32_t n, int32_t m, const int8_t* __restrict__ in, int8_t* __restrict__ out) {
     __shared__ __attribute__((aligned(16))) int8_t tile[64][68];        // pitch 68: dword-aligned rows, 17 banks apart
     const int64_t boff = (int64_t)blockIdx.z * n * m;
     const int32_t r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
-    if (WIDE) {
+    if constexpr (IN == 16) {
         const int pc = threadIdx.x & 3, rr = threadIdx.x >> 2;          // 4 pieces of 16 bytes x 64 rows
         if (r0 + rr < n && c0 + pc * 16 < m) {
             const uint4_t v = *reinterpret_cast<const uint4_t*>(in + boff + (int64_t)(r0 + rr) * m + c0 + pc * 16);
             uint32_t* dst = reinterpret_cast<uint32_t*>(&tile[rr][pc * 16]);
             dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
         }
-        __syncthreads();
+    } else if constexpr (IN == 4) {
+        const int pc = threadIdx.x & 15, rr = threadIdx.x >> 4;         // 16 dwords x 16 rows per pass
+#pragma unroll
+        for (int ps = 0; ps < 4; ++ps) {
+            const int r = ps * 16 + rr;
+            if (r0 + r < n && c0 + pc * 4 < m)
+                *reinterpret_cast<uint32_t*>(&tile[r][pc * 4]) = *reinterpret_cast<const uint32_t*>(in + boff + (int64_t)(r0 + r) * m + c0 + pc * 4);
+        }
+    } else {
+        const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+        for (int r = ty; r < 64; r += 4)
+            if (r0 + r < n && c0 + tx < m) tile[r][tx] = in[boff + (int64_t)(r0 + r) * m + c0 + tx];
+    }
+    __syncthreads();
+    if constexpr (OUT == 16) {
         // row rr of the transposed tile = column rr of the tile; this thread's 16 bytes are its rows pc*16 .. pc*16+15
+        const int pc = threadIdx.x & 3, rr = threadIdx.x >> 2;
         if (c0 + rr < m && r0 + pc * 16 < n) {
             uint32_t w[4];
 #pragma unroll
@@ -73,11 +89,20 @@ __global__ __launch_bounds__(256) void k_transpose_i8(int32_t n, int32_t m, cons
             }
             *reinterpret_cast<uint4_t*>(out + boff + (int64_t)(c0 + rr) * n + r0 + pc * 16) = uint4_t{w[0], w[1], w[2], w[3]};
         }
+    } else if constexpr (OUT == 4) {
+        const int pc = threadIdx.x & 15, rr = threadIdx.x >> 4;
+#pragma unroll
+        for (int ps = 0; ps < 4; ++ps) {
+            const int c = ps * 16 + rr;
+            if (c0 + c < m && r0 + pc * 4 < n) {
+                uint32_t x = 0;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) x |= (uint32_t)(uint8_t)tile[pc * 4 + e][c] << (8 * e);
+                *reinterpret_cast<uint32_t*>(out + boff + (int64_t)(c0 + c) * n + r0 + pc * 4) = x;
+            }
+        }
     } else {
         const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-        for (int r = ty; r < 64; r += 4)
-            if (r0 + r < n && c0 + tx < m) tile[r][tx] = in[boff + (int64_t)(r0 + r) * m + c0 + tx];
-        __syncthreads();
         for (int c = ty; c < 64; c += 4)
             if (c0 + c < m && r0 + tx < n) out[boff + (int64_t)(c0 + c) * n + r0 + tx] = tile[tx][c];
     }
@@ -161,14 +186,22 @@ int cpmk_transpose_i8(int32_t batch, int32_t n, int32_t m, const void* inp, void
     if ((int64_t)batch * n * m == 0) return 0;
     if (any_null(inp, out)) return CPMK_EBADARG;
     if (ceil_div(n, 64) > 65535) return CPMK_ETOOBIG;
-    const bool wide = n % 16 == 0 && m % 16 == 0 && aligned16(inp) && aligned16(out);
+    // bytes per access on each side: what the row length and the buffer's alignment allow (a batch entry is n * m bytes
+    // on, which keeps the alignment of either side whenever that side's rows do)
+    auto width = [](int32_t row, const void* q) {
+        const uintptr_t a = reinterpret_cast<uintptr_t>(q);
+        return row % 16 == 0 && (a & 15u) == 0 ? 16 : row % 4 == 0 && (a & 3u) == 0 ? 4 : 1;
+    };
+    const int win = width(m, inp), wout = width(n, out);
     for (int64_t b0 = 0; b0 < batch; b0 += 65535) {       // (grid z: at most 65535 batch entries per launch)
         const int64_t nb = batch - b0 < 65535 ? batch - b0 : 65535;
         const dim3 grid((unsigned)ceil_div(m, 64), (unsigned)ceil_div(n, 64), (unsigned)nb);
         const int8_t* src = (const int8_t*)inp + b0 * n * m;
         int8_t* dst = (int8_t*)out + b0 * n * m;
-        if (wide) hipLaunchKernelGGL(k_transpose_i8<true>, grid, dim3(256), 0, (hipStream_t)stream, n, m, src, dst);
-        else hipLaunchKernelGGL(k_transpose_i8<false>, grid, dim3(256), 0, (hipStream_t)stream, n, m, src, dst);
+        auto go = [&](auto kern) { hipLaunchKernelGGL(kern, grid, dim3(256), 0, (hipStream_t)stream, n, m, src, dst); };
+        if (win == 16) { if (wout == 16) go(k_transpose_i8<16, 16>); else if (wout == 4) go(k_transpose_i8<16, 4>); else go(k_transpose_i8<16, 1>); }
+        else if (win == 4) { if (wout == 16) go(k_transpose_i8<4, 16>); else if (wout == 4) go(k_transpose_i8<4, 4>); else go(k_transpose_i8<4, 1>); }
+        else { if (wout == 16) go(k_transpose_i8<1, 16>); else if (wout == 4) go(k_transpose_i8<1, 4>); else go(k_transpose_i8<1, 1>); }
         if (int e = launch_status()) return e;
     }
     return 0;

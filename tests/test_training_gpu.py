@@ -349,7 +349,9 @@ def test_transpose(gpu, shape):
 
 
 @pytest.mark.parametrize("shape", [(2, 64, 64), (3, 17, 100), (1, 1000, 3), (2, 5, 7), (1, 4096, 512), (4, 1, 9),
-                                   (2, 80, 48), (1, 208, 144), (3, 16, 1040), (1, 10240, 4096)])
+                                   (2, 80, 48), (1, 208, 144), (3, 16, 1040), (1, 10240, 4096),
+                                   # every pairing of 16-byte, 4-byte and single-byte accesses on the two sides
+                                   (2, 4096, 500), (2, 500, 4096), (1, 36, 100), (1, 48, 7), (1, 7, 48), (1, 100, 33)])
 def test_transpose_i8(gpu, shape):
     _name("transpose_i8", shape)
     b, n, m = shape
