@@ -51,7 +51,10 @@ constexpr int BK = 64;   // bytes of K per LDS stage
 // consecutive rows reading the same logical chunk then cover all 64 banks exactly once.
 __device__ inline int lds_off(int r, int c) { return r * BK + ((c ^ ((r >> 2) & 3)) << 4); }
 
-// DW: rows that are only 4-byte aligned (k % 16 != 0): a 16-byte piece comes as four dwords, each zero past the end of K.
+// DW: rows that are only 4-byte aligned (k % 16 != 0): a whole 16-byte piece still comes in one load (global loads of
+// four dwords need dword alignment only), the piece across the end of K as single dwords, zero past the end.
+struct __attribute__((aligned(4))) Int4Dword { int32_t x, y, z, w; };
+
 template <int WAVES_R, int WAVES_C, int TR, int TC, bool FUSED, bool DW = false>
 __global__ __launch_bounds__(WAVES_R* WAVES_C * 64) void k_gemm_kmajor(GemmArgs a) {
     constexpr int NT = WAVES_R * WAVES_C * 64;
@@ -89,9 +92,14 @@ __global__ __launch_bounds__(WAVES_R* WAVES_C * 64) void k_gemm_kmajor(GemmArgs 
     auto piece = [&](const int8_t* rowp, int32_t kc) __attribute__((always_inline)) {      // bytes [kc, kc + 16) of a row, zeros past K
         int4_t v = {0, 0, 0, 0};
         if constexpr (DW) {
+            if (kc + 16 <= K) {
+                const Int4Dword t = *reinterpret_cast<const Int4Dword*>(rowp + kc);
+                v = int4_t{t.x, t.y, t.z, t.w};
+            } else {
 #pragma unroll
-            for (int d = 0; d < 4; ++d)
-                if (kc + 4 * d < K) v[d] = *reinterpret_cast<const int32_t*>(rowp + kc + 4 * d);
+                for (int d = 0; d < 3; ++d)
+                    if (kc + 4 * d < K) v[d] = *reinterpret_cast<const int32_t*>(rowp + kc + 4 * d);
+            }
         } else {
             if (kc < K) v = *reinterpret_cast<const int4_t*>(rowp + kc);
         }

@@ -27,8 +27,8 @@ namespace cpmk {
 // in piece j lane (r = l%16, q = l/16) reads bytes [j*64 + q*16, +16) of row r -- the four
 // lanes of a row read one contiguous 64-byte sector per instruction.  The vector operand uses
 // the same lane -> k assignment, which is all the MFMA needs.
-// DW: rows that are only 4-byte aligned (dim_in % 16 != 0): a lane's 16 bytes come as four dwords, each zero past the
-// end of k.
+// DW: rows that are only 4-byte aligned (dim_in % 16 != 0): a lane's 16 bytes still come in one load where they lie
+// inside the row, as single dwords (zero past the end of k) across its end.
 // F16: the same on fp16 data (cpmk_gemv_broadcast_mat_fp16 with rows that are not whole 256-byte chunks): dim_in is the
 // row length in BYTES, a lane's 16 bytes are 8 halves of K for v_mfma_f32_16x16x32_f16, the accumulators are fp32 and
 // leave without scales; the waves' partial sums are added in wave order.
@@ -56,9 +56,15 @@ __global__ __launch_bounds__(NW * 64) void k_gemv_mfma(int32_t batch, int32_t di
     auto piece = [&](const int8_t* rowp, int32_t k0) __attribute__((always_inline)) {      // bytes [k0, k0 + 16) of a row, zeros past dim_in
         int4_t v = {0, 0, 0, 0};
         if constexpr (DW) {
+            if (k0 + 16 <= dim_in) {       // (a global load of four dwords needs dword alignment only)
+                struct __attribute__((aligned(4))) Int4Dword { int32_t x, y, z, w; };
+                const Int4Dword t = *reinterpret_cast<const Int4Dword*>(rowp + k0);
+                v = int4_t{t.x, t.y, t.z, t.w};
+            } else {
 #pragma unroll
-            for (int d = 0; d < 4; ++d)
-                if (k0 + 4 * d < dim_in) v[d] = *reinterpret_cast<const int32_t*>(rowp + k0 + 4 * d);
+                for (int d = 0; d < 3; ++d)
+                    if (k0 + 4 * d < dim_in) v[d] = *reinterpret_cast<const int32_t*>(rowp + k0 + 4 * d);
+            }
         } else {
             if (k0 < dim_in) v = *reinterpret_cast<const int4_t*>(rowp + k0);
         }
