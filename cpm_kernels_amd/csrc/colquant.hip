@@ -17,8 +17,9 @@ namespace cpmk {
 // (two 512-thread workgroups share a compute unit: at most 128 registers per lane)
 // NTH: the tile's 128-byte row segments are whole cache lines (m % 64 == 0, the matrix on a 128-byte boundary): the input is
 // read with the non-temporal hint.  Elsewhere a line is shared with the neighbouring tile and has to stay in L2 for it.
-// UA: any m and alignment: the eight columns of a piece are read (and the scales and, not transposed, the int8 values
-// written) one by one, each checked against m.
+// UA: any m and alignment: a piece inside its row still moves whole, at whatever address it lies (global accesses need
+// no alignment); the piece across a row's end is read (and its scales and, not transposed, its int8 values are
+// written) in at most three narrower accesses.
 template <int NT, bool TRANSPOSED, bool NTH, bool UA = false>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void k_col_quantize_team(int32_t n, int32_t m, int32_t tiles_per_batch, int32_t parts,
                                                           const half_t* __restrict__ mat, half_t* __restrict__ scale,
@@ -46,9 +47,11 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
         if constexpr (UA) {
             if (row0 + p < n) {
                 const half_t* src = mat + boff + ((uint32_t)(row0 + p) * (uint32_t)m + (uint32_t)col0);
-#pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    if (col0 + e < m) v[p][e] = src[e];
+                if (col0 + 8 <= m) {
+                    v[p] = load_half8_any(src);
+                } else if (col0 < m) {
+                    v[p] = load_half8_head_any(src, m & 7, v[p]);
+                }
             }
         } else if (row0 + p < n && col0 < m) {
             const half8_t* src = reinterpret_cast<const half8_t*>(mat + boff + ((uint32_t)(row0 + p) * (uint32_t)m + (uint32_t)col0));
@@ -103,9 +106,11 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     }
     if (part == 0 && rg == 0) {
         if constexpr (UA) {
-#pragma unroll
-            for (int e = 0; e < 8; ++e)
-                if (col0 + e < m) scale[(int64_t)b * m + col0 + e] = sh[e];
+            if (col0 + 8 <= m) {
+                store_half8_any(scale + (int64_t)b * m + col0, sh);
+            } else if (col0 < m) {
+                store_half8_head_any(scale + (int64_t)b * m + col0, m & 7, sh);
+            }
         } else if (col0 < m) {
             *reinterpret_cast<half8_t*>(scale + (int64_t)b * m + col0) = sh;
         }
@@ -145,9 +150,11 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
                 if (row0 + p < n) {
                     int8_t* dst = out + boff + ((uint32_t)(row0 + p) * (uint32_t)m + (uint32_t)col0);
                     if constexpr (UA) {
-#pragma unroll
-                        for (int e = 0; e < 8; ++e)
-                            if (col0 + e < m) dst[e] = (int8_t)(q[p][e >> 2] >> (8 * (e & 3)));
+                        if (col0 + 8 <= m) {
+                            store_byte8_any(dst, q[p][0], q[p][1]);
+                        } else {
+                            store_byte8_head_any(dst, m & 7, q[p][0], q[p][1]);
+                        }
                     } else {
                         *reinterpret_cast<uint2_t*>(dst) = uint2_t{q[p][0], q[p][1]};
                     }

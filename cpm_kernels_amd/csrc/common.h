@@ -12,6 +12,7 @@ typedef _Float16 half_t;
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+
 typedef float float4_t __attribute__((ext_vector_type(4)));
 typedef int32_t int4_t __attribute__((ext_vector_type(4)));
 typedef int32_t int2_t __attribute__((ext_vector_type(2)));
@@ -19,6 +20,55 @@ typedef int32_t int16_tv __attribute__((ext_vector_type(16)));
 typedef float float16_tv __attribute__((ext_vector_type(16)));
 typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
+
+// Wide accesses at addresses that are not multiples of their size: global loads and stores of this target need no
+// alignment (the compiler itself emits 16-byte accesses for data declared with alignment 1); an access that crosses
+// a cache line costs a second request.  Eight halves at any half's address, eight bytes at any address:
+struct __attribute__((packed, aligned(2))) Half8Any { uint32_t x, y, z, w; };
+struct __attribute__((packed, aligned(1))) Byte8Any { uint32_t x, y; };
+__device__ __forceinline__ half8_t load_half8_any(const half_t* p) { return __builtin_bit_cast(half8_t, *reinterpret_cast<const Half8Any*>(p)); }
+__device__ __forceinline__ void store_half8_any(half_t* p, half8_t v) { *reinterpret_cast<Half8Any*>(p) = __builtin_bit_cast(Half8Any, v); }
+__device__ __forceinline__ void store_byte8_any(int8_t* p, uint32_t lo, uint32_t hi) { *reinterpret_cast<Byte8Any*>(p) = Byte8Any{lo, hi}; }
+
+// The first t (1..7, the same for the whole wave) of eight halves at p, at any address, in at most three accesses
+// (8, 4 and 2 bytes); the other elements of the result keep `r`'s values.
+struct __attribute__((packed, aligned(2))) Half4Any { uint32_t x, y; };
+struct __attribute__((packed, aligned(2))) Half2Any { uint32_t x; };
+__device__ __forceinline__ half8_t load_half8_head_any(const half_t* p, int t, half8_t r) {
+    if (t & 4) {
+        const half4_t q = __builtin_bit_cast(half4_t, *reinterpret_cast<const Half4Any*>(p));
+        r[0] = q[0]; r[1] = q[1]; r[2] = q[2]; r[3] = q[3];
+    }
+    if (t & 2) {
+        const half2_t q = __builtin_bit_cast(half2_t, *reinterpret_cast<const Half2Any*>(p + (t & 4)));
+        if (t & 4) { r[4] = q[0]; r[5] = q[1]; } else { r[0] = q[0]; r[1] = q[1]; }
+    }
+    if (t & 1) {
+        const half_t h = p[t & 6];
+        if ((t & 6) == 0) r[0] = h;
+        else if ((t & 6) == 2) r[2] = h;
+        else if ((t & 6) == 4) r[4] = h;
+        else r[6] = h;
+    }
+    return r;
+}
+__device__ __forceinline__ void store_half8_head_any(half_t* p, int t, half8_t v) {
+    if (t & 4) *reinterpret_cast<Half4Any*>(p) = __builtin_bit_cast(Half4Any, half4_t{v[0], v[1], v[2], v[3]});
+    if (t & 2) {
+        const half2_t q = (t & 4) ? half2_t{v[4], v[5]} : half2_t{v[0], v[1]};
+        *reinterpret_cast<Half2Any*>(p + (t & 4)) = __builtin_bit_cast(Half2Any, q);
+    }
+    if (t & 1) p[t & 6] = (t & 6) == 0 ? v[0] : (t & 6) == 2 ? v[2] : (t & 6) == 4 ? v[4] : v[6];
+}
+// the first t (1..7) of the eight bytes lo | hi << 32 to p, at any address
+struct __attribute__((packed, aligned(1))) Byte4Any { uint32_t x; };
+struct __attribute__((packed, aligned(1))) Byte2Any { uint16_t x; };
+__device__ __forceinline__ void store_byte8_head_any(int8_t* p, int t, uint32_t lo, uint32_t hi) {
+    if (t & 4) *reinterpret_cast<Byte4Any*>(p) = Byte4Any{lo};
+    const uint32_t rest = (t & 4) ? hi : lo;
+    if (t & 2) *reinterpret_cast<Byte2Any*>(p + (t & 4)) = Byte2Any{(uint16_t)rest};
+    if (t & 1) p[t & 6] = (int8_t)((t & 2) ? rest >> 16 : rest);
+}
 
 constexpr int kWave = 64;
 

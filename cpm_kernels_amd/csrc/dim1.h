@@ -31,53 +31,49 @@ struct ColTile {
 // lines (LPR == 8) and for data that is not read again soon: a segment shorter than a line is completed
 // by a neighbouring workgroup, so it has to allocate in L2.
 //
-// UA: rows that are not whole 16-byte pieces, or buffers that are not 16-byte aligned (m % 8 != 0): the eight columns
-// of a piece come and go one by one, each checked against m.
+// UA: rows that are not whole 16-byte pieces, or buffers that are not 16-byte aligned.  A piece inside its row still
+// moves as one 16-byte access (global accesses need no alignment; one that crosses a cache line costs a second
+// request), the piece across a row's end in at most three narrower ones.
 template <int NT, int LPR, int R, bool NTL = false, bool UA = false>
 __device__ inline void coltile_load(half8_t (&v)[R], const half_t* base, int32_t n, int32_t m, int32_t col0,
                                     half_t fill) {
     constexpr int RPP = NT / LPR;
     const int rg = threadIdx.x / LPR;
     const uint32_t off0 = (uint32_t)rg * (uint32_t)m + (uint32_t)col0, stride = (uint32_t)RPP * (uint32_t)m;
-    const bool pairs = UA && (m & 1) == 0 && (reinterpret_cast<uintptr_t>(base) & 3u) == 0;
-    const bool quads = UA && (m & 3) == 0 && (reinterpret_cast<uintptr_t>(base) & 7u) == 0;
+    if constexpr (UA) {
+        if (col0 + 8 <= m) {        // the lane's pieces lie inside their rows
 #pragma unroll
-    for (int p = 0; p < R; ++p) {
-        const int32_t row = p * RPP + rg;
-        half8_t x;
+            for (int p = 0; p < R; ++p) {
+                half8_t x;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) x[e] = fill;
-        if constexpr (UA) {
-            if (row < n) {
-                if (quads) {        // m % 4 == 0, 8-byte aligned buffer: four columns per access
-#pragma unroll
-                    for (int e = 0; e < 8; e += 4)
-                        if (col0 + e < m) {
-                            const half4_t t = *reinterpret_cast<const half4_t*>(base + (off0 + p * stride + e));
-#pragma unroll
-                            for (int d = 0; d < 4; ++d) x[e + d] = t[d];
-                        }
-                } else if (pairs) {        // even m, 4-byte aligned buffer: two columns per access
-#pragma unroll
-                    for (int e = 0; e < 8; e += 2)
-                        if (col0 + e < m) {
-                            const half2_t t = *reinterpret_cast<const half2_t*>(base + (off0 + p * stride + e));
-                            x[e] = t[0];
-                            x[e + 1] = t[1];
-                        }
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e)
-                        if (col0 + e < m) x[e] = base[off0 + p * stride + e];
-                }
+                for (int e = 0; e < 8; ++e) x[e] = fill;
+                if (p * RPP + rg < n) x = load_half8_any(base + (off0 + p * stride));
+                v[p] = x;
             }
-        } else {
+        } else {                    // ... or across their ends (the first m % 8 columns of the piece), or past them
+            const bool tail = col0 < m;
+#pragma unroll
+            for (int p = 0; p < R; ++p) {
+                half8_t x;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[e] = fill;
+                if (tail && p * RPP + rg < n) x = load_half8_head_any(base + (off0 + p * stride), m & 7, x);
+                v[p] = x;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int p = 0; p < R; ++p) {
+            const int32_t row = p * RPP + rg;
+            half8_t x;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[e] = fill;
             if (row < n && col0 < m) {
                 const half8_t* src = reinterpret_cast<const half8_t*>(base + (off0 + p * stride));
                 x = NTL ? __builtin_nontemporal_load(src) : *src;
             }
+            v[p] = x;
         }
-        v[p] = x;
     }
 }
 
@@ -86,32 +82,25 @@ __device__ inline void coltile_store(const half8_t (&v)[R], half_t* base, int32_
     constexpr int RPP = NT / LPR;
     const int rg = threadIdx.x / LPR;
     const uint32_t off0 = (uint32_t)rg * (uint32_t)m + (uint32_t)col0, stride = (uint32_t)RPP * (uint32_t)m;
-    const bool pairs = UA && (m & 1) == 0 && (reinterpret_cast<uintptr_t>(base) & 3u) == 0;
-    const bool quads = UA && (m & 3) == 0 && (reinterpret_cast<uintptr_t>(base) & 7u) == 0;
+    if constexpr (UA) {
+        if (col0 + 8 <= m) {
 #pragma unroll
-    for (int p = 0; p < R; ++p) {
-        const int32_t row = p * RPP + rg;
-        if constexpr (UA) {
-            if (row < n) {
-                if (quads) {
+            for (int p = 0; p < R; ++p)
+                if (p * RPP + rg < n) store_half8_any(base + (off0 + p * stride), v[p]);
+        } else if (col0 < m) {
 #pragma unroll
-                    for (int e = 0; e < 8; e += 4)
-                        if (col0 + e < m)
-                            *reinterpret_cast<half4_t*>(base + (off0 + p * stride + e)) = half4_t{v[p][e], v[p][e + 1], v[p][e + 2], v[p][e + 3]};
-                } else if (pairs) {
+            for (int p = 0; p < R; ++p)
+                if (p * RPP + rg < n) store_half8_head_any(base + (off0 + p * stride), m & 7, v[p]);
+        }
+    } else {
 #pragma unroll
-                    for (int e = 0; e < 8; e += 2)
-                        if (col0 + e < m) *reinterpret_cast<half2_t*>(base + (off0 + p * stride + e)) = half2_t{v[p][e], v[p][e + 1]};
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e)
-                        if (col0 + e < m) base[off0 + p * stride + e] = v[p][e];
-                }
+        for (int p = 0; p < R; ++p) {
+            const int32_t row = p * RPP + rg;
+            if (row < n && col0 < m) {
+                half8_t* dst = reinterpret_cast<half8_t*>(base + (off0 + p * stride));
+                if (NTS) __builtin_nontemporal_store(v[p], dst);
+                else *dst = v[p];
             }
-        } else if (row < n && col0 < m) {
-            half8_t* dst = reinterpret_cast<half8_t*>(base + (off0 + p * stride));
-            if (NTS) __builtin_nontemporal_store(v[p], dst);
-            else *dst = v[p];
         }
     }
 }

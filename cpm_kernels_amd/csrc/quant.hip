@@ -236,8 +236,9 @@ struct RowsArgs {
 };
 
 // (the launcher counts on 8 resident workgroups per compute unit up to NV = 8, 4 beyond)
-// UA: rows that are not whole 16-byte pieces, or buffers off 16-byte boundaries: the eight elements of a piece move
-// four (m % 4 == 0, 8-byte aligned inputs, 4-byte aligned outputs), two (even m, 4- and 2-byte aligned) or one at a time.
+// UA: rows that are not whole 16-byte pieces, or buffers off 16-byte boundaries: a piece inside its row still comes in one
+// 16-byte load and leaves in one 8-byte store (global accesses need no alignment), the piece across a row's end in at
+// most three narrower accesses each way.
 template <int NV, bool QUANT, bool UA = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(UA ? (NV <= 4 ? 8 : NV <= 8 ? 4 : 2) : (NV <= 8 ? 8 : 4)))) void k_rows(RowsArgs a) {
     const int lane = threadIdx.x & 63;
@@ -247,14 +248,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(UA ? (NV <=
     int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= rows) return;
     const int m8 = UA ? (m + 7) >> 3 : m >> 3;
-    const uintptr_t in_bits = reinterpret_cast<uintptr_t>(a.mat0) | reinterpret_cast<uintptr_t>(a.mat1);
-    const uintptr_t out_bits = reinterpret_cast<uintptr_t>(a.out0) | reinterpret_cast<uintptr_t>(a.out1);
-    const bool quads = UA && (m & 3) == 0 && (in_bits & 7u) == 0 && (out_bits & 3u) == 0;
-    const bool pairs = UA && (m & 1) == 0 && (in_bits & 3u) == 0 && (out_bits & 1u) == 0;
     half8_t cur[NV];
     auto load = [&](half8_t (&v)[NV], int64_t r) __attribute__((always_inline)) {
         const half_t* mat = r < a.rows0 ? a.mat0 + r * m : a.mat1 + (r - a.rows0) * m;
         const half8_t* p8 = reinterpret_cast<const half8_t*>(mat);
+        // the one piece across the row's end (piece m / 8, if m % 8 != 0) comes element by element, to the lane that owns it
+        half8_t tailv = {0, 0, 0, 0, 0, 0, 0, 0};
+        const int jt = m >> 3;
+        if constexpr (UA) {
+            if ((m & 7) != 0 && (jt & 63) == lane) tailv = load_half8_head_any(mat + jt * 8, m & 7, tailv);
+        }
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int j = lane + i * 64;
@@ -262,26 +265,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(UA ? (NV <=
             for (int e = 0; e < 8; ++e) v[i][e] = (half_t)0.0f;
             if constexpr (!UA) {
                 if (j < m8) v[i] = __builtin_nontemporal_load(p8 + j);
-            } else if (quads) {
-#pragma unroll
-                for (int e = 0; e < 8; e += 4)
-                    if (j * 8 + e < m) {
-                        const half4_t t = *reinterpret_cast<const half4_t*>(mat + j * 8 + e);
-#pragma unroll
-                        for (int d = 0; d < 4; ++d) v[i][e + d] = t[d];
-                    }
-            } else if (pairs) {
-#pragma unroll
-                for (int e = 0; e < 8; e += 2)
-                    if (j * 8 + e < m) {
-                        const half2_t t = *reinterpret_cast<const half2_t*>(mat + j * 8 + e);
-                        v[i][e] = t[0];
-                        v[i][e + 1] = t[1];
-                    }
             } else {
-#pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    if (j * 8 + e < m) v[i][e] = mat[j * 8 + e];
+                if (j * 8 + 8 <= m) v[i] = load_half8_any(mat + j * 8);
+                else if (j == jt) v[i] = tailv;
             }
         }
     };
@@ -289,20 +275,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(UA ? (NV <=
     auto store = [&](int8_t* orow, int j, uint2_t w) __attribute__((always_inline)) {
         if constexpr (!UA) {
             reinterpret_cast<uint2_t*>(orow)[j] = w;
-        } else if (quads) {
-            *reinterpret_cast<uint32_t*>(orow + j * 8) = w.x;
-            if (j * 8 + 4 < m) *reinterpret_cast<uint32_t*>(orow + j * 8 + 4) = w.y;
+        } else if (j * 8 + 8 <= m) {
+            store_byte8_any(orow + j * 8, w.x, w.y);
         } else {
-            const uint64_t bits = (uint64_t)w.x | ((uint64_t)w.y << 32);
-            if (pairs) {
-#pragma unroll
-                for (int e = 0; e < 8; e += 2)
-                    if (j * 8 + e < m) *reinterpret_cast<uint16_t*>(orow + j * 8 + e) = (uint16_t)(bits >> (8 * e));
-            } else {
-#pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    if (j * 8 + e < m) orow[j * 8 + e] = (int8_t)(bits >> (8 * e));
-            }
+            store_byte8_head_any(orow + j * 8, m & 7, w.x, w.y);       // (callers pass j < ceil(m / 8))
         }
     };
     load(cur, row);
@@ -594,9 +570,8 @@ int cpmk_gemm_quantize_pair(int64_t rows0, const void* mat0, void* scale0, void*
     const bool vec = (m % 8 == 0) && (rows0 == 0 || (aligned16(mat0) && (reinterpret_cast<uintptr_t>(out0) & 7u) == 0)) &&
                      (rows1 == 0 || (aligned16(mat1) && (reinterpret_cast<uintptr_t>(out1) & 7u) == 0));
     if (m <= 64 * 8 * 16) {
-        // (an absent tensor's pointers count as aligned in the kernel's choice of access width)
-        const RowsArgs ra = {rows0 ? (const half_t*)mat0 : nullptr, (half_t*)scale0, rows0 ? (int8_t*)out0 : nullptr, rows0,
-                             rows1 ? (const half_t*)mat1 : nullptr, (half_t*)scale1, rows1 ? (int8_t*)out1 : nullptr, rows1, m};
+        const RowsArgs ra = {(const half_t*)mat0, (half_t*)scale0, (int8_t*)out0, rows0,
+                             (const half_t*)mat1, (half_t*)scale1, (int8_t*)out1, rows1, m};
         if (vec) launch_rows<true>(ra, (int)ceil_div(m, 512), (hipStream_t)stream);
         else launch_rows<true, true>(ra, (int)ceil_div(m, 512), (hipStream_t)stream);
         return launch_status();

@@ -266,7 +266,8 @@ __global__ __launch_bounds__(256) void k_col(ColArgs p) {
 constexpr int kColTeamMaxParts = 32;
 
 // MODE 0: 16-byte accesses with the non-temporal hint (the tile's row segments are whole cache lines: m % 64 == 0, buffers on
-// 128-byte boundaries); 1: 16-byte accesses without it; 2: any m and alignment, the columns of a piece one by one.
+// 128-byte boundaries); 1: 16-byte accesses without it; 2: any m and alignment (pieces inside a row still whole, at whatever
+// address they lie; the piece across a row's end in at most three narrower accesses).
 template <int KIND, int MODE>
 __global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_batch, int32_t parts, uint32_t nteams, XchLaunch xl) {
     uint64_t* const xch = xl.region;
@@ -297,9 +298,8 @@ __global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_b
     auto load8 = [&](const half_t* src) __attribute__((always_inline)) {       // eight per-column values of this lane's columns
         half8_t r = {0, 0, 0, 0, 0, 0, 0, 0};
         if constexpr (UA) {
-#pragma unroll
-            for (int e = 0; e < 8; ++e)
-                if (col0 + e < p.m) r[e] = src[e];
+            if (col0 + 8 <= p.m) r = load_half8_any(src);
+            else if (col0 < p.m) r = load_half8_head_any(src, p.m & 7, r);
         } else {
             r = *reinterpret_cast<const half8_t*>(src);
         }
@@ -307,9 +307,8 @@ __global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_b
     };
     auto store8 = [&](half_t* dst, half8_t r) __attribute__((always_inline)) {
         if constexpr (UA) {
-#pragma unroll
-            for (int e = 0; e < 8; ++e)
-                if (col0 + e < p.m) dst[e] = r[e];
+            if (col0 + 8 <= p.m) store_half8_any(dst, r);
+            else if (col0 < p.m) store_half8_head_any(dst, p.m & 7, r);
         } else {
             *reinterpret_cast<half8_t*>(dst) = r;
         }
@@ -419,13 +418,10 @@ __global__ __launch_bounds__(512) void k_col_team(ColArgs p, int32_t tiles_per_b
                     for (int e = 0; e < 8; ++e) t[e] = quant_i8((float)va[q][e] * sxv[q], k0[e]);
                     int8_t* dst = p.out_i8 + boff + ((uint32_t)lrow * (uint32_t)p.m + (uint32_t)col0);
                     if constexpr (UA) {
-                        if ((p.m & 3) == 0 && (reinterpret_cast<uintptr_t>(p.out_i8) & 3u) == 0) {       // whole dwords
-                            *reinterpret_cast<uint32_t*>(dst) = pack4_i8(t[0], t[1], t[2], t[3]);
-                            if (col0 + 4 < p.m) *reinterpret_cast<uint32_t*>(dst + 4) = pack4_i8(t[4], t[5], t[6], t[7]);
+                        if (col0 + 8 <= p.m) {
+                            store_byte8_any(dst, pack4_i8(t[0], t[1], t[2], t[3]), pack4_i8(t[4], t[5], t[6], t[7]));
                         } else {
-#pragma unroll
-                            for (int e = 0; e < 8; ++e)
-                                if (col0 + e < p.m) dst[e] = (int8_t)t[e];
+                            store_byte8_head_any(dst, p.m & 7, pack4_i8(t[0], t[1], t[2], t[3]), pack4_i8(t[4], t[5], t[6], t[7]));
                         }
                     } else {
                         *reinterpret_cast<uint2_t*>(dst) = uint2_t{pack4_i8(t[0], t[1], t[2], t[3]), pack4_i8(t[4], t[5], t[6], t[7])};
@@ -502,8 +498,9 @@ __global__ __launch_bounds__(256) void k_round_scale_rows_wide(int64_t rows, int
 // The same for rows of at most 2048 columns, kept in registers: a wave takes U consecutive rows of P 16-byte pieces
 // per lane (P * U = 4 loads in flight per lane, the matrix read once and with the non-temporal hint), finds each
 // row's maximum over the wave with data-parallel-primitive operands and rounds from the registers.
-// UA: rows that are not whole 16-byte pieces or buffers off 16-byte boundaries -- the eight columns of a piece then
-// move four (m % 4 == 0, 8-byte aligned buffers), two (even m, 4-byte aligned) or one at a time.
+// UA: rows that are not whole 16-byte pieces or buffers off 16-byte boundaries -- a piece inside its row still comes in
+// one 16-byte load and leaves in one 8-byte store (global accesses need no alignment), the piece across a row's end
+// in at most three narrower accesses each way.
 template <int P, int U, bool UA>
 __global__ __launch_bounds__(256) void k_round_scale_rows_reg(int64_t rows, int32_t n, int32_t m, const half_t* __restrict__ mat,
                                                               const half_t* __restrict__ scale_y, int8_t* __restrict__ out,
@@ -511,33 +508,14 @@ __global__ __launch_bounds__(256) void k_round_scale_rows_reg(int64_t rows, int3
     const int lane = threadIdx.x & 63;
     const int64_t row0 = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * U;
     if (row0 >= rows) return;
-    const uintptr_t bits = reinterpret_cast<uintptr_t>(mat) | reinterpret_cast<uintptr_t>(scale_y);
-    const bool quads = UA && (m & 3) == 0 && (bits & 7u) == 0 && (reinterpret_cast<uintptr_t>(out) & 3u) == 0;
-    const bool pairs = UA && (m & 1) == 0 && (bits & 3u) == 0 && (reinterpret_cast<uintptr_t>(out) & 1u) == 0;
     auto load8 = [&](const half_t* src, int32_t j, bool nt) __attribute__((always_inline)) {
         half8_t r = {0, 0, 0, 0, 0, 0, 0, 0};
         if constexpr (!UA) {
             r = nt ? __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(src + j)) : *reinterpret_cast<const half8_t*>(src + j);
-        } else if (quads) {
-#pragma unroll
-            for (int e = 0; e < 8; e += 4)
-                if (j + e < m) {
-                    const half4_t t = *reinterpret_cast<const half4_t*>(src + j + e);
-#pragma unroll
-                    for (int d = 0; d < 4; ++d) r[e + d] = t[d];
-                }
-        } else if (pairs) {
-#pragma unroll
-            for (int e = 0; e < 8; e += 2)
-                if (j + e < m) {
-                    const half2_t t = *reinterpret_cast<const half2_t*>(src + j + e);
-                    r[e] = t[0];
-                    r[e + 1] = t[1];
-                }
+        } else if (j + 8 <= m) {
+            r = load_half8_any(src + j);
         } else {
-#pragma unroll
-            for (int e = 0; e < 8; ++e)
-                if (j + e < m) r[e] = src[j + e];
+            r = load_half8_head_any(src + j, m & 7, r);       // (callers pass j < m)
         }
         return r;
     };
@@ -579,17 +557,10 @@ __global__ __launch_bounds__(256) void k_round_scale_rows_reg(int64_t rows, int3
                     int8_t* dst = out + row * m + j;
                     if constexpr (!UA) {
                         *reinterpret_cast<uint2_t*>(dst) = uint2_t{pack4_i8(t[0], t[1], t[2], t[3]), pack4_i8(t[4], t[5], t[6], t[7])};
-                    } else if (quads) {
-                        *reinterpret_cast<uint32_t*>(dst) = pack4_i8(t[0], t[1], t[2], t[3]);
-                        if (j + 4 < m) *reinterpret_cast<uint32_t*>(dst + 4) = pack4_i8(t[4], t[5], t[6], t[7]);
-                    } else if (pairs) {
-#pragma unroll
-                        for (int e = 0; e < 8; e += 2)
-                            if (j + e < m) *reinterpret_cast<uint16_t*>(dst + e) = (uint16_t)((t[e] & 0xff) | ((t[e + 1] & 0xff) << 8));
+                    } else if (j + 8 <= m) {
+                        store_byte8_any(dst, pack4_i8(t[0], t[1], t[2], t[3]), pack4_i8(t[4], t[5], t[6], t[7]));
                     } else {
-#pragma unroll
-                        for (int e = 0; e < 8; ++e)
-                            if (j + e < m) dst[e] = (int8_t)t[e];
+                        store_byte8_head_any(dst, m & 7, pack4_i8(t[0], t[1], t[2], t[3]), pack4_i8(t[4], t[5], t[6], t[7]));
                     }
                 }
             }
