@@ -90,10 +90,19 @@ __global__ __launch_bounds__(256) void k_mask(int64_t total, int32_t n, int32_t 
         if (e0 + 8 <= total) {
             half8_t v = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(x + e0));
             const int8_t* m0 = mask + (row / n) * m + j;                   // this row's mask bytes from column j on
-            const int8_t* m1 = mask + ((row + 1) / n) * m + (j - m);       // the next row's, addressed by the same index
+            if (j + 8 <= m) {       // the eight share a row: their mask bytes in one load (global loads need no alignment)
+                const Byte8Any mk = *reinterpret_cast<const Byte8Any*>(m0);
 #pragma unroll
-            for (int e = 0; e < 8; ++e)
-                if ((j + e < m ? m0 : m1)[e] == 0) v[e] = value;
+                for (int e = 0; e < 8; ++e) {
+                    const uint32_t byte = ((e < 4 ? mk.x : mk.y) >> ((e & 3) * 8)) & 0xffu;
+                    if (byte == 0) v[e] = value;
+                }
+            } else {
+                const int8_t* m1 = mask + ((row + 1) / n) * m + (j - m);       // the next row's, addressed by the same index
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if ((j + e < m ? m0 : m1)[e] == 0) v[e] = value;
+            }
             __builtin_nontemporal_store(v, reinterpret_cast<half8_t*>(out + e0));
         } else {
             for (int64_t i = e0; i < total; ++i) {

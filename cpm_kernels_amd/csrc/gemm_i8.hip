@@ -1236,12 +1236,16 @@ __global__ __launch_bounds__(256) void k_gemm_f16_generic(GemmArgs a, int p_kmaj
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc[e] = 0.0f;
     typedef _Float16 halfV_t __attribute__((ext_vector_type(V > 1 ? V : 2)));
-    // V halves of one operand's piece: along K for a K-major operand (one row), along the rows for one stored (K, rows)
-    auto stage = [&](half_t* sm, const half_t* G, int kmajor, int32_t r0, int32_t L, int32_t k0, int q) __attribute__((always_inline)) {
-        int r, kk;
+    // V halves of one operand's piece: along K for a K-major operand (one row), along the rows for one stored (K, rows).
+    // A stage's pieces are requested one stage ahead into registers, so that their latency passes under the products.
+    constexpr int S = T * GK / V / 256;       // accesses per thread, operand and stage
+    auto place = [&](int kmajor, int q, int& r, int& kk) __attribute__((always_inline)) {
         if (kmajor) { r = q / (GK / V); kk = (q % (GK / V)) * V; } else { r = (q % (T / V)) * V; kk = q / (T / V); }
+    };
+    auto fetch = [&](half_t (&v)[V], const half_t* G, int kmajor, int32_t r0, int32_t L, int32_t k0, int q) __attribute__((always_inline)) {
+        int r, kk;
+        place(kmajor, q, r, kk);
         const int32_t row = r0 + r, kg = k0 + kk;
-        half_t v[V];
 #pragma unroll
         for (int e = 0; e < V; ++e) v[e] = (half_t)0.0f;
         if (row < L && kg < k) {            // (L and k are multiples of V where the access runs along them)
@@ -1254,16 +1258,30 @@ __global__ __launch_bounds__(256) void k_gemm_f16_generic(GemmArgs a, int p_kmaj
                 v[0] = *src;
             }
         }
+    };
+    auto put = [&](half_t* sm, const half_t (&v)[V], int kmajor, int q) __attribute__((always_inline)) {
+        int r, kk;
+        place(kmajor, q, r, kk);
 #pragma unroll
         for (int e = 0; e < V; ++e) sm[kmajor ? r * LD + kk + e : (r + e) * LD + kk] = v[e];
     };
+    half_t rp[S][V], rq[S][V];
+    auto fetch_all = [&](int32_t k0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int s = 0; s < S; ++s) {
+            fetch(rp[s], P, p_kmajor, j0, a.n, k0, tid + s * 256);
+            fetch(rq[s], Q, q_kmajor, i0, a.m, k0, tid + s * 256);
+        }
+    };
+    fetch_all(0);
     for (int32_t k0 = 0; k0 < k; k0 += GK) {
 #pragma unroll
-        for (int s = 0; s < T * GK / V / 256; ++s) {
-            stage(sP, P, p_kmajor, j0, a.n, k0, tid + s * 256);
-            stage(sQ, Q, q_kmajor, i0, a.m, k0, tid + s * 256);
+        for (int s = 0; s < S; ++s) {
+            put(sP, rp[s], p_kmajor, tid + s * 256);
+            put(sQ, rq[s], q_kmajor, tid + s * 256);
         }
         __syncthreads();
+        if (k0 + GK < k) fetch_all(k0 + GK);
 #pragma unroll
         for (int ks = 0; ks < GK / 16; ++ks) {
             // lane (lrow, lk): the 8 halves k = 16 ks + 8 lk .. + 7 of its row / column, as two 8-byte reads
