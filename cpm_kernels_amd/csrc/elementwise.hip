@@ -41,12 +41,34 @@ __global__ __launch_bounds__(256) void k_ln_affine(int64_t total, int32_t n, int
                                                    const half_t* __restrict__ alpha,
                                                    const half_t* __restrict__ beta, half_t* out, int vec) {
     const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    const int64_t e0 = vec ? gid * 8 : gid * 2;       // m % 2 == 0 (vec: m % 8 == 0)
+    const int64_t e0 = vec ? gid * 8 : gid * 2;       // m % 2 == 0 (vec 1: m % 8 == 0)
     if (e0 >= total) return;
     const int32_t ch = (int32_t)((e0 / m) % n);
     const half_t a = alpha[ch];
     const half_t b = HAS_BETA ? beta[ch] : (half_t)0.0f;
-    if (vec) {
+    if (vec == 2) {
+        // rows that are not whole 16-byte pieces (m >= 8), or buffers off 16-byte boundaries: the tensor is still one
+        // contiguous run, so its elements go eight at a time at whatever address they start; the eight may run over
+        // the end of a row into the next channel
+        if (e0 + 8 <= total) {
+            const int32_t left = m - (int32_t)(e0 % m);       // elements of this row from e0 on
+            const int32_t ch1 = ch + 1 == n ? 0 : ch + 1;
+            const half_t a1 = alpha[ch1];
+            const half_t b1 = HAS_BETA ? beta[ch1] : (half_t)0.0f;
+            half8_t v = load_half8_any(x + e0);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const half_t ae = e < left ? a : a1, be = e < left ? b : b1;
+                v[e] = HAS_BETA ? __builtin_fmaf16(v[e], ae, be) : (half_t)(v[e] * ae);
+            }
+            store_half8_any(out + e0, v);
+        } else {
+            for (int64_t i = e0; i < total; ++i) {
+                const int32_t c = (int32_t)((i / m) % n);
+                out[i] = HAS_BETA ? __builtin_fmaf16(x[i], alpha[c], beta[c]) : (half_t)(x[i] * alpha[c]);
+            }
+        }
+    } else if (vec) {
         half8_t v = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(x + e0));
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] = HAS_BETA ? __builtin_fmaf16(v[e], a, b) : (half_t)(v[e] * a);
@@ -150,8 +172,8 @@ static int ln_affine(int32_t batch, int32_t n, int32_t m, const void* inp, const
     const int64_t total = (int64_t)batch * n * m;
     if (total == 0) return 0;
     if (any_null(inp, alpha, out)) return CPMK_EBADARG;
-    const int vec = (m % 8 == 0) && aligned16(inp) && aligned16(out);
-    const int64_t g = ceil_div(total / (vec ? 8 : 2), 256);
+    const int vec = (m % 8 == 0) && aligned16(inp) && aligned16(out) ? 1 : m >= 8 ? 2 : 0;
+    const int64_t g = ceil_div(vec ? ceil_div(total, 8) : total / 2, 256);
     if (beta)
         hipLaunchKernelGGL((k_ln_affine<true>), dim3((unsigned)g), dim3(256), 0, st, total, n, m, (const half_t*)inp,
                            (const half_t*)alpha, (const half_t*)beta, (half_t*)out, vec);

@@ -32,12 +32,13 @@ __device__ inline half_t ew_apply(int op, half_t x, half_t a, half_t b) {
 
 // The tensor is seen as rows x cols: BC 0: one row; BC 1: rows = batch, cols = n, a/b indexed by the
 // column; BC 2: rows = batch*n, cols = m, a/b indexed by row % n.  blockIdx.x = row * chunks + chunk;
-// a thread handles V adjacent elements (8 = 16-byte accesses when cols % 8 == 0 and everything is
-// 16-byte aligned, else 2: element counts are even, the reference asserts it).
-template <int OP, int BC, int V>
+// a thread handles 8 adjacent elements of a row.  ANY false: cols % 8 == 0 and everything 16-byte aligned; true: any
+// row length and alignment -- eight elements inside the row still move as one 16-byte access at whatever address they
+// start, the piece across the row's end in narrower ones.
+template <int OP, int BC, bool ANY>
 __global__ __launch_bounds__(256) void k_ew(int64_t cols, uint32_t chunks, int64_t n, const half_t* x, const half_t* __restrict__ a,
                                             const half_t* __restrict__ b, half_t* out) {
-    typedef half_t vec_t __attribute__((ext_vector_type(V)));
+    constexpr int V = 8;
     // BC 1: the rows of one chunk of columns run side by side, so a/b are fetched from HBM once
     const uint32_t rows = gridDim.x / chunks;
     const uint32_t chunk = BC == 1 ? blockIdx.x / rows : blockIdx.x % chunks;
@@ -45,8 +46,14 @@ __global__ __launch_bounds__(256) void k_ew(int64_t cols, uint32_t chunks, int64
     const int64_t c = ((int64_t)chunk * 256 + threadIdx.x) * V;
     if (c >= cols) return;
     const int64_t i = row * cols + c;
-    const vec_t v = *reinterpret_cast<const vec_t*>(x + i);
-    vec_t av, bv;
+    const int t = !ANY || cols - c >= V ? V : (int)(cols - c);        // elements of this piece inside the row
+    const half8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    auto get = [&](const half_t* p) __attribute__((always_inline)) {
+        if constexpr (!ANY) return *reinterpret_cast<const half8_t*>(p);
+        else return t == V ? load_half8_any(p) : load_half8_head_any(p, t, zero);
+    };
+    const half8_t v = get(x + i);
+    half8_t av = zero, bv = zero;
     if (BC == 2) {
         const int64_t k = row % n;
         const half_t a1 = a[k], b1 = b ? b[k] : (half_t)0.0f;
@@ -54,15 +61,15 @@ __global__ __launch_bounds__(256) void k_ew(int64_t cols, uint32_t chunks, int64
         for (int e = 0; e < V; ++e) { av[e] = a1; bv[e] = b1; }
     } else {
         const int64_t k = BC == 0 ? i : c;
-        av = *reinterpret_cast<const vec_t*>(a + k);
-#pragma unroll
-        for (int e = 0; e < V; ++e) bv[e] = (half_t)0.0f;
-        if (b) bv = *reinterpret_cast<const vec_t*>(b + k);
+        av = get(a + k);
+        if (b) bv = get(b + k);
     }
-    vec_t r;
+    half8_t r;
 #pragma unroll
     for (int e = 0; e < V; ++e) r[e] = ew_apply(OP, v[e], av[e], bv[e]);
-    *reinterpret_cast<vec_t*>(out + i) = r;
+    if constexpr (!ANY) *reinterpret_cast<half8_t*>(out + i) = r;
+    else if (t == V) store_half8_any(out + i, r);
+    else store_half8_head_any(out + i, t, r);
 }
 
 template <int V>
@@ -822,15 +829,14 @@ static int launch_ew(int64_t rows, int64_t cols, int64_t n, const void* x, const
     if (cols % 2) return CPMK_EALIGN;
     if (any_null(x, a, out) || ((OP == kFma || OP == kSubDiv) && b == nullptr)) return CPMK_EBADARG;
     const bool wide = cols % 8 == 0 && aligned16(x) && aligned16(out) && (BC == 2 || (aligned16(a) && (!b || aligned16(b))));
-    const int v = wide ? 8 : 2;
-    const int64_t chunks = ceil_div(cols, 256 * v);
+    const int64_t chunks = ceil_div(cols, 256 * 8);
     if (rows * chunks > 0x7fffffffll) return CPMK_ETOOBIG;
     const dim3 grid((unsigned)(rows * chunks));
     if (wide)
-        hipLaunchKernelGGL((k_ew<OP, BC, 8>), grid, dim3(256), 0, (hipStream_t)stream, cols, (uint32_t)chunks, n, (const half_t*)x,
+        hipLaunchKernelGGL((k_ew<OP, BC, false>), grid, dim3(256), 0, (hipStream_t)stream, cols, (uint32_t)chunks, n, (const half_t*)x,
                            (const half_t*)a, (const half_t*)b, (half_t*)out);
     else
-        hipLaunchKernelGGL((k_ew<OP, BC, 2>), grid, dim3(256), 0, (hipStream_t)stream, cols, (uint32_t)chunks, n, (const half_t*)x,
+        hipLaunchKernelGGL((k_ew<OP, BC, true>), grid, dim3(256), 0, (hipStream_t)stream, cols, (uint32_t)chunks, n, (const half_t*)x,
                            (const half_t*)a, (const half_t*)b, (half_t*)out);
     return launch_status();
 }

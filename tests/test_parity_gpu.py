@@ -955,7 +955,8 @@ def test_position_embedding_config5_size(gpu):
 # ---------------------------------------------------------------------------------------------
 # elementwise helpers
 # ---------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("shape", [(8, 4096, 512), (3, 33, 10), (2, 5, 1232)])
+# (rows that are not whole 16-byte pieces: pieces of eight that run over a row's end into the next channel; rows under eight)
+@pytest.mark.parametrize("shape", [(8, 4096, 512), (3, 33, 10), (2, 5, 1232), (2, 7, 500), (1, 3, 6), (3, 4, 14)])
 def test_elementwise(gpu, shape):
     _name("elementwise", shape)
     b, n, m = shape
