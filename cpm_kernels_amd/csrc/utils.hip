@@ -5,104 +5,103 @@
 
 namespace cpmk {
 
-// (batch, n, m) -> (batch, m, n) through a 64x64 LDS tile: each wave reads 128-byte row pieces
-// and writes 128-byte row pieces of the transposed tensor.
+// (batch, n, m) -> (batch, m, n) through a 64x64 LDS tile.  IN / OUT: eight halves per global load / store where a
+// piece of eight lies inside its row (a 16-byte access at whatever address it starts: global accesses need no
+// alignment), single halves for the piece across a row's end; the scalar form (IN = OUT = false) for rows under eight.
+template <bool IN, bool OUT>
 __global__ __launch_bounds__(256) void k_transpose(int32_t n, int32_t m, const half_t* __restrict__ in, half_t* __restrict__ out) {
-    __shared__ half_t tile[64][66];
-    const int64_t boff = (int64_t)blockIdx.z * n * m;
-    const int32_t r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
-    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-    for (int r = ty; r < 64; r += 4)
-        if (r0 + r < n && c0 + tx < m) tile[r][tx] = in[boff + (int64_t)(r0 + r) * m + c0 + tx];
-    __syncthreads();
-    for (int c = ty; c < 64; c += 4)
-        if (c0 + c < m && r0 + tx < n) out[boff + (int64_t)(c0 + c) * n + r0 + tx] = tile[tx][c];
-}
-
-// The same with 16-byte global accesses (n % 8 == 0, m % 8 == 0, 16-byte aligned pointers): a row
-// of the tile is read by eight lanes, a row of the transposed tile is written by eight lanes; the
-// transposition itself is eight 2-byte LDS reads per lane.
-__global__ __launch_bounds__(256) void k_transpose_wide(int32_t n, int32_t m, const half_t* __restrict__ in, half_t* __restrict__ out) {
-    __shared__ half_t tile[64][72];                     // pitch 144 bytes: 16-byte aligned rows, odd multiple of 16 bytes
+    __shared__ __attribute__((aligned(16))) half_t tile[64][72];    // pitch 144 bytes: 16-byte aligned rows, odd multiple of 16 bytes
     const int64_t boff = (int64_t)blockIdx.z * n * m;
     const int32_t r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
     const int pc = threadIdx.x & 7, rr = threadIdx.x >> 3;          // 8 pieces x 32 rows per pass
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    if constexpr (IN) {
 #pragma unroll
-    for (int ps = 0; ps < 2; ++ps) {
-        const int r = ps * 32 + rr;
-        if (r0 + r < n && c0 + pc * 8 < m)
-            *reinterpret_cast<half8_t*>(&tile[r][pc * 8]) = *reinterpret_cast<const half8_t*>(in + boff + (int64_t)(r0 + r) * m + c0 + pc * 8);
-    }
-    __syncthreads();
-#pragma unroll
-    for (int ps = 0; ps < 2; ++ps) {
-        const int c = ps * 32 + rr;                     // row of the transposed tile
-        if (c0 + c < m && r0 + pc * 8 < n) {
-            half8_t v;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) v[e] = tile[pc * 8 + e][c];
-            *reinterpret_cast<half8_t*>(out + boff + (int64_t)(c0 + c) * n + r0 + pc * 8) = v;
-        }
-    }
-}
-
-// (batch, n, m) -> (batch, m, n) of bytes: 64x64 tile through LDS.  IN / OUT: bytes per global load / store -- 16 where
-// the rows of that side are whole 16-byte pieces on 16-byte boundaries (m % 16 == 0 for the loads, n % 16 == 0 for the
-// stores), 4 where they are whole dwords, else single bytes; the two sides choose independently.
-template <int IN, int OUT>
-__global__ __launch_bounds__(256) void k_transpose_i8(int32_t n, int32_t m, const int8_t* __restrict__ in, int8_t* __restrict__ out) {
-    __shared__ __attribute__((aligned(16))) int8_t tile[64][68];        // pitch 68: dword-aligned rows, 17 banks apart
-    const int64_t boff = (int64_t)blockIdx.z * n * m;
-    const int32_t r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
-    if constexpr (IN == 16) {
-        const int pc = threadIdx.x & 3, rr = threadIdx.x >> 2;          // 4 pieces of 16 bytes x 64 rows
-        if (r0 + rr < n && c0 + pc * 16 < m) {
-            const uint4_t v = *reinterpret_cast<const uint4_t*>(in + boff + (int64_t)(r0 + rr) * m + c0 + pc * 16);
-            uint32_t* dst = reinterpret_cast<uint32_t*>(&tile[rr][pc * 16]);
-            dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
-        }
-    } else if constexpr (IN == 4) {
-        const int pc = threadIdx.x & 15, rr = threadIdx.x >> 4;         // 16 dwords x 16 rows per pass
-#pragma unroll
-        for (int ps = 0; ps < 4; ++ps) {
-            const int r = ps * 16 + rr;
-            if (r0 + r < n && c0 + pc * 4 < m)
-                *reinterpret_cast<uint32_t*>(&tile[r][pc * 4]) = *reinterpret_cast<const uint32_t*>(in + boff + (int64_t)(r0 + r) * m + c0 + pc * 4);
+        for (int ps = 0; ps < 2; ++ps) {
+            const int r = ps * 32 + rr;
+            const int32_t c = c0 + pc * 8;
+            if (r0 + r < n && c < m) {
+                const half_t* src = in + boff + (int64_t)(r0 + r) * m + c;
+                half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+                if (c + 8 <= m) v = load_half8_any(src);
+                else v = load_half8_head_any(src, m - c, v);
+                *reinterpret_cast<half8_t*>(&tile[r][pc * 8]) = v;
+            }
         }
     } else {
-        const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
         for (int r = ty; r < 64; r += 4)
             if (r0 + r < n && c0 + tx < m) tile[r][tx] = in[boff + (int64_t)(r0 + r) * m + c0 + tx];
     }
     __syncthreads();
-    if constexpr (OUT == 16) {
-        // row rr of the transposed tile = column rr of the tile; this thread's 16 bytes are its rows pc*16 .. pc*16+15
-        const int pc = threadIdx.x & 3, rr = threadIdx.x >> 2;
-        if (c0 + rr < m && r0 + pc * 16 < n) {
-            uint32_t w[4];
+    if constexpr (OUT) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                uint32_t x = 0;
+        for (int ps = 0; ps < 2; ++ps) {
+            const int c = ps * 32 + rr;                     // row of the transposed tile
+            const int32_t r = r0 + pc * 8;
+            if (c0 + c < m && r < n) {
+                half8_t v;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) x |= (uint32_t)(uint8_t)tile[pc * 16 + q * 4 + e][rr] << (8 * e);
-                w[q] = x;
-            }
-            *reinterpret_cast<uint4_t*>(out + boff + (int64_t)(c0 + rr) * n + r0 + pc * 16) = uint4_t{w[0], w[1], w[2], w[3]};
-        }
-    } else if constexpr (OUT == 4) {
-        const int pc = threadIdx.x & 15, rr = threadIdx.x >> 4;
-#pragma unroll
-        for (int ps = 0; ps < 4; ++ps) {
-            const int c = ps * 16 + rr;
-            if (c0 + c < m && r0 + pc * 4 < n) {
-                uint32_t x = 0;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) x |= (uint32_t)(uint8_t)tile[pc * 4 + e][c] << (8 * e);
-                *reinterpret_cast<uint32_t*>(out + boff + (int64_t)(c0 + c) * n + r0 + pc * 4) = x;
+                for (int e = 0; e < 8; ++e) v[e] = tile[pc * 8 + e][c];
+                half_t* dst = out + boff + (int64_t)(c0 + c) * n + r;
+                if (r + 8 <= n) store_half8_any(dst, v);
+                else store_half8_head_any(dst, n - r, v);
             }
         }
     } else {
-        const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+        for (int c = ty; c < 64; c += 4)
+            if (c0 + c < m && r0 + tx < n) out[boff + (int64_t)(c0 + c) * n + r0 + tx] = tile[tx][c];
+    }
+}
+
+// (batch, n, m) -> (batch, m, n) of bytes: 64x64 tile through LDS.  IN / OUT: sixteen bytes per global load / store where
+// a piece of sixteen lies inside its row (at whatever address it starts: global accesses need no alignment), single
+// bytes for the piece across a row's end; the scalar form (false) for rows under sixteen bytes.
+struct __attribute__((packed, aligned(1))) Byte16Any { uint32_t x, y, z, w; };
+
+template <bool IN, bool OUT>
+__global__ __launch_bounds__(256) void k_transpose_i8(int32_t n, int32_t m, const int8_t* __restrict__ in, int8_t* __restrict__ out) {
+    __shared__ __attribute__((aligned(16))) int8_t tile[64][68];        // pitch 68: dword-aligned rows, 17 banks apart
+    const int64_t boff = (int64_t)blockIdx.z * n * m;
+    const int32_t r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+    const int pc = threadIdx.x & 3, rr = threadIdx.x >> 2;          // 4 pieces of 16 bytes x 64 rows
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    if constexpr (IN) {
+        const int32_t c = c0 + pc * 16;
+        if (r0 + rr < n && c < m) {
+            const int8_t* src = in + boff + (int64_t)(r0 + rr) * m + c;
+            if (c + 16 <= m) {
+                const Byte16Any v = *reinterpret_cast<const Byte16Any*>(src);
+                uint32_t* dst = reinterpret_cast<uint32_t*>(&tile[rr][pc * 16]);
+                dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
+            } else {
+                for (int e = 0; e < m - c; ++e) tile[rr][pc * 16 + e] = src[e];
+            }
+        }
+    } else {
+        for (int r = ty; r < 64; r += 4)
+            if (r0 + r < n && c0 + tx < m) tile[r][tx] = in[boff + (int64_t)(r0 + r) * m + c0 + tx];
+    }
+    __syncthreads();
+    if constexpr (OUT) {
+        // row rr of the transposed tile = column rr of the tile; this thread's 16 bytes are its rows pc*16 .. pc*16+15
+        const int32_t r = r0 + pc * 16;
+        if (c0 + rr < m && r < n) {
+            int8_t* dst = out + boff + (int64_t)(c0 + rr) * n + r;
+            if (r + 16 <= n) {
+                uint32_t w[4];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    uint32_t x = 0;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) x |= (uint32_t)(uint8_t)tile[pc * 16 + q * 4 + e][rr] << (8 * e);
+                    w[q] = x;
+                }
+                *reinterpret_cast<Byte16Any*>(dst) = Byte16Any{w[0], w[1], w[2], w[3]};
+            } else {
+                for (int e = 0; e < n - r; ++e) dst[e] = tile[pc * 16 + e][rr];
+            }
+        }
+    } else {
         for (int c = ty; c < 64; c += 4)
             if (c0 + c < m && r0 + tx < n) out[boff + (int64_t)(c0 + c) * n + r0 + tx] = tile[tx][c];
     }
@@ -166,15 +165,16 @@ int cpmk_transpose(int32_t batch, int32_t n, int32_t m, const void* inp, void* o
     if ((int64_t)batch * n * m == 0) return 0;
     if (any_null(inp, out)) return CPMK_EBADARG;
     if (ceil_div(n, 64) > 65535) return CPMK_ETOOBIG;
-    const bool wide = n % 8 == 0 && m % 8 == 0 && aligned16(inp) && aligned16(out);
+    const bool win = m >= 8, wout = n >= 8;       // pieces of eight on a side whose rows hold at least one
     // the batch is the grid's z dimension (at most 65535): larger batches go out in several launches
     for (int64_t b0 = 0; b0 < batch; b0 += 65535) {
         const int64_t nb = batch - b0 < 65535 ? batch - b0 : 65535;
         const dim3 grid((unsigned)ceil_div(m, 64), (unsigned)ceil_div(n, 64), (unsigned)nb);
         const half_t* src = (const half_t*)inp + b0 * n * m;
         half_t* dst = (half_t*)out + b0 * n * m;
-        if (wide) hipLaunchKernelGGL(k_transpose_wide, grid, dim3(256), 0, (hipStream_t)stream, n, m, src, dst);
-        else hipLaunchKernelGGL(k_transpose, grid, dim3(256), 0, (hipStream_t)stream, n, m, src, dst);
+        auto go = [&](auto kern) { hipLaunchKernelGGL(kern, grid, dim3(256), 0, (hipStream_t)stream, n, m, src, dst); };
+        if (win) { if (wout) go(k_transpose<true, true>); else go(k_transpose<true, false>); }
+        else { if (wout) go(k_transpose<false, true>); else go(k_transpose<false, false>); }
         if (int e = launch_status()) return e;
     }
     return 0;
@@ -186,22 +186,15 @@ int cpmk_transpose_i8(int32_t batch, int32_t n, int32_t m, const void* inp, void
     if ((int64_t)batch * n * m == 0) return 0;
     if (any_null(inp, out)) return CPMK_EBADARG;
     if (ceil_div(n, 64) > 65535) return CPMK_ETOOBIG;
-    // bytes per access on each side: what the row length and the buffer's alignment allow (a batch entry is n * m bytes
-    // on, which keeps the alignment of either side whenever that side's rows do)
-    auto width = [](int32_t row, const void* q) {
-        const uintptr_t a = reinterpret_cast<uintptr_t>(q);
-        return row % 16 == 0 && (a & 15u) == 0 ? 16 : row % 4 == 0 && (a & 3u) == 0 ? 4 : 1;
-    };
-    const int win = width(m, inp), wout = width(n, out);
+    const bool win = m >= 16, wout = n >= 16;       // pieces of sixteen on a side whose rows hold at least one
     for (int64_t b0 = 0; b0 < batch; b0 += 65535) {       // (grid z: at most 65535 batch entries per launch)
         const int64_t nb = batch - b0 < 65535 ? batch - b0 : 65535;
         const dim3 grid((unsigned)ceil_div(m, 64), (unsigned)ceil_div(n, 64), (unsigned)nb);
         const int8_t* src = (const int8_t*)inp + b0 * n * m;
         int8_t* dst = (int8_t*)out + b0 * n * m;
         auto go = [&](auto kern) { hipLaunchKernelGGL(kern, grid, dim3(256), 0, (hipStream_t)stream, n, m, src, dst); };
-        if (win == 16) { if (wout == 16) go(k_transpose_i8<16, 16>); else if (wout == 4) go(k_transpose_i8<16, 4>); else go(k_transpose_i8<16, 1>); }
-        else if (win == 4) { if (wout == 16) go(k_transpose_i8<4, 16>); else if (wout == 4) go(k_transpose_i8<4, 4>); else go(k_transpose_i8<4, 1>); }
-        else { if (wout == 16) go(k_transpose_i8<1, 16>); else if (wout == 4) go(k_transpose_i8<1, 4>); else go(k_transpose_i8<1, 1>); }
+        if (win) { if (wout) go(k_transpose_i8<true, true>); else go(k_transpose_i8<true, false>); }
+        else { if (wout) go(k_transpose_i8<false, true>); else go(k_transpose_i8<false, false>); }
         if (int e = launch_status()) return e;
     }
     return 0;

@@ -337,7 +337,7 @@ def test_embedding_backward(gpu, shape):
 
 
 @pytest.mark.parametrize("shape", [(2, 64, 64), (3, 17, 100), (1, 1000, 3), (2, 5, 7), (1, 4096, 512), (4, 1, 9),
-                                   (2, 72, 40), (1, 200, 136), (3, 8, 1032)])
+                                   (2, 72, 40), (1, 200, 136), (3, 8, 1032), (2, 4096, 500), (1, 501, 4090), (1, 77, 33)])
 def test_transpose(gpu, shape):
     _name("transpose", shape)
     b, n, m = shape
