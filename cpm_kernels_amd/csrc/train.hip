@@ -128,18 +128,54 @@ __global__ __launch_bounds__(256) void k_gelu_backward(int64_t total, const half
 // Sums over everything but one index (fp32 accumulation, one workgroup per output).
 // ---------------------------------------------------------------------------------------
 // grad[j] = sum_b grad_out[b, j]                                            cu_arith_batch_add_backward
-__global__ __launch_bounds__(256) void k_batch_add_backward(int64_t batch, int64_t n, const half_t* __restrict__ grad_out,
+// A lane owns eight adjacent columns: one 16-byte load per row at whatever address the piece starts (global loads need
+// no alignment), eight rows requested at a time, the sums in fp32; the piece across the end of the row in narrower
+// accesses.  With few columns the rows are dealt to `rgs` (a power of two up to 64) groups of 256 / rgs lanes, whose
+// sums are added in group order.
+__global__ __launch_bounds__(256) void k_batch_add_backward(int64_t batch, int64_t n, int rgs, const half_t* __restrict__ grad_out,
                                                             half_t* __restrict__ grad) {
-    // 64 columns per workgroup, 4 row groups
-    __shared__ float red[4][64];
-    const int c = threadIdx.x & 63, rg = threadIdx.x >> 6;
-    const int64_t col = (int64_t)blockIdx.x * 64 + c;
-    float s = 0.0f;
-    if (col < n)
-        for (int64_t i = rg; i < batch; i += 4) s += (float)grad_out[i * n + col];
-    red[rg][c] = s;
-    __syncthreads();
-    if (rg == 0 && col < n) grad[col] = round_f16(red[0][c] + red[1][c] + red[2][c] + red[3][c]);
+    __shared__ float red[2048];                 // [row group][column of the workgroup]
+    const int cgs = 256 / rgs, cg = threadIdx.x % cgs, rg = threadIdx.x / cgs;
+    const int64_t col = ((int64_t)blockIdx.x * cgs + cg) * 8;
+    const int t = col >= n ? 0 : n - col >= 8 ? 8 : (int)(n - col);
+    const half8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    float s[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    if (t > 0) {
+        for (int64_t i0 = rg; i0 < batch; i0 += 8 * rgs) {
+            half8_t v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                v[u] = zero;
+                const int64_t i = i0 + (int64_t)u * rgs;
+                if (i < batch) {
+                    const half_t* src = grad_out + i * n + col;
+                    v[u] = t == 8 ? load_half8_any(src) : load_half8_head_any(src, t, zero);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) s[e] += (float)v[u][e];
+        }
+    }
+    if (rgs > 1) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) red[rg * (cgs * 8) + cg * 8 + e] = s[e];
+        __syncthreads();
+        if (rg != 0) return;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            float a = s[e];
+            for (int g = 1; g < rgs; ++g) a += red[g * (cgs * 8) + cg * 8 + e];
+            s[e] = a;
+        }
+    }
+    if (t == 0) return;
+    half8_t r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r[e] = round_f16(s[e]);
+    if (t == 8) store_half8_any(grad + col, r);
+    else store_half8_head_any(grad + col, t, r);
 }
 
 // grad[i] = sum_{b, j} (WITH_X ? x[b,i,j] : 1) * grad_out[b,i,j]            cu_arith_ln_mul_backward / _ln_add_backward
@@ -149,8 +185,11 @@ __global__ __launch_bounds__(256) void k_ln_backward(int64_t batch, int64_t n, i
     __shared__ float red[4];
     const int64_t ch = blockIdx.x;
     float s = 0.0f;
-    if (vec) {         // m % 8 == 0, 16-byte aligned: the (b, j) pairs of this channel in pieces of 8
-        const uint32_t m8 = (uint32_t)(m >> 3), db = 256u / m8, dj = 256u % m8;      // one step of 256 pieces, as rows and remainder
+    if (vec) {         // m >= 8: the (b, j) pairs of this channel in pieces of 8, at whatever address a piece starts (global
+                       // loads need no alignment); the piece across a row's end in narrower loads, zeros beyond it
+        const uint32_t m8 = (uint32_t)((m + 7) >> 3), db = 256u / m8, dj = 256u % m8;      // one step of 256 pieces, as rows and remainder
+        const int tail = (int)(m & 7);
+        const half8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
         uint32_t b = threadIdx.x / m8, j8 = threadIdx.x % m8;
         for (; b < (uint32_t)batch; b += db, j8 += dj) {
             if (j8 >= m8) {
@@ -158,9 +197,10 @@ __global__ __launch_bounds__(256) void k_ln_backward(int64_t batch, int64_t n, i
                 if (++b >= (uint32_t)batch) break;
             }
             const int64_t o = ((int64_t)b * n + ch) * m + ((int64_t)j8 << 3);
-            const half8_t gv = *reinterpret_cast<const half8_t*>(grad_out + o);
+            const bool whole = tail == 0 || j8 + 1 < m8;
+            const half8_t gv = whole ? load_half8_any(grad_out + o) : load_half8_head_any(grad_out + o, tail, zero);
             if (WITH_X) {
-                const half8_t xv = *reinterpret_cast<const half8_t*>(x + o);
+                const half8_t xv = whole ? load_half8_any(x + o) : load_half8_head_any(x + o, tail, zero);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) s += (float)xv[e] * (float)gv[e];
             } else {
@@ -983,8 +1023,11 @@ int cpmk_arith_batch_add_backward(int32_t batch, int32_t n, const void* grad_out
     if (batch < 0 || n < 0) return CPMK_EBADARG;
     if (n == 0) return 0;
     if (grad == nullptr || (batch > 0 && grad_out == nullptr)) return CPMK_EBADARG;
-    hipLaunchKernelGGL(k_batch_add_backward, dim3((unsigned)ceil_div(n, 64)), dim3(256), 0, (hipStream_t)stream, (int64_t)batch,
-                       (int64_t)n, (const half_t*)grad_out, (half_t*)grad);
+    // enough lanes for the whole chip: with few columns, more row groups per workgroup
+    int rgs = 1;
+    while (rgs < 64 && ceil_div(n, 8) * rgs < 131072 && rgs * 2 <= batch) rgs *= 2;
+    hipLaunchKernelGGL(k_batch_add_backward, dim3((unsigned)ceil_div(n, (256 / rgs) * 8)), dim3(256), 0, (hipStream_t)stream, (int64_t)batch,
+                       (int64_t)n, rgs, (const half_t*)grad_out, (half_t*)grad);
     return launch_status();
 }
 int cpmk_arith_ln_mul_backward(int32_t batch, int32_t n, int32_t m, const void* inp, const void* grad_out, void* grad, void* stream) {
@@ -993,8 +1036,7 @@ int cpmk_arith_ln_mul_backward(int32_t batch, int32_t n, int32_t m, const void* 
     if (n == 0) return 0;
     if (grad == nullptr || ((int64_t)batch * m > 0 && any_null(inp, grad_out))) return CPMK_EBADARG;
     hipLaunchKernelGGL((k_ln_backward<true>), dim3((unsigned)n), dim3(256), 0, (hipStream_t)stream, (int64_t)batch, (int64_t)n,
-                       (int64_t)m, (const half_t*)inp, (const half_t*)grad_out, (half_t*)grad,
-                       (int)(m % 8 == 0 && aligned16(inp) && aligned16(grad_out)));
+                       (int64_t)m, (const half_t*)inp, (const half_t*)grad_out, (half_t*)grad, (int)(m >= 8));
     return launch_status();
 }
 int cpmk_arith_ln_add_backward(int32_t batch, int32_t n, int32_t m, const void* grad_out, void* grad, void* stream) {
@@ -1003,8 +1045,7 @@ int cpmk_arith_ln_add_backward(int32_t batch, int32_t n, int32_t m, const void* 
     if (n == 0) return 0;
     if (grad == nullptr || ((int64_t)batch * m > 0 && grad_out == nullptr)) return CPMK_EBADARG;
     hipLaunchKernelGGL((k_ln_backward<false>), dim3((unsigned)n), dim3(256), 0, (hipStream_t)stream, (int64_t)batch, (int64_t)n,
-                       (int64_t)m, (const half_t*)nullptr, (const half_t*)grad_out, (half_t*)grad,
-                       (int)(m % 8 == 0 && aligned16(grad_out)));
+                       (int64_t)m, (const half_t*)nullptr, (const half_t*)grad_out, (half_t*)grad, (int)(m >= 8));
     return launch_status();
 }
 

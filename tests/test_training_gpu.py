@@ -52,7 +52,8 @@ def assert_fp16_equal_nan_ok(actual, expected, what):
     assert_bits_equal(np.where(both_nan, np.float16(0), a), np.where(both_nan, np.float16(0), e), what)
 
 
-@pytest.mark.parametrize("shape", [(3, 64), (16, 4096), (1, 2), (5, 1026)])
+# (the last three: many rows of few columns -- the rows dealt to groups of lanes --, a ragged last piece, a wide tensor)
+@pytest.mark.parametrize("shape", [(3, 64), (16, 4096), (1, 2), (5, 1026), (1000, 72), (130, 5002), (8, 1 << 21)])
 def test_arith_batch_family(gpu, shape):
     _name("arith batch_*", shape)
     b, n = shape
