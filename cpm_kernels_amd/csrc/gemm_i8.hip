@@ -459,7 +459,6 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
     constexpr bool PT = (LAY & 1) != 0, QT = (LAY & 2) != 0;
     static_assert(LAY == 0 || BKB == 128, "transposed operands: 128 bytes of K per slab");
     constexpr int ESZ_IN = F16 ? 2 : 1;            // bytes per operand element
-    constexpr int EPP = 16 / ESZ_IN;               // elements per 16-byte piece
     using acc_t = std::conditional_t<F16, float4_t, int4_t>;
     constexpr int KS = BKB / 64, CPR = BKB / 16;
     static_assert(KS >= 1, "k-steps of 64 bytes");
