@@ -447,6 +447,10 @@ struct StripOut {
 // lets the compiler keep the accumulators in place and the MFMA/memory interleave as written.
 // Returns true if the next tile's first slabs are on their way.
 //
+// LAY bit 2 (K-major operands only): the depth is whole 16-byte pieces but not whole slabs.  The slabs of the ring cover
+// the whole ones; the rest of every row (less than a slab) goes from memory straight into the fragment registers
+// before the K loop starts -- a lane's 16 bytes of a k-step are the same bytes in memory as in the stage -- with zeros
+// past the end of K.
 // LAY marks operands whose rows are K instead: bit 0 = the row operand is stored (K, n), bit 1 =
 // the column operand is stored (K, m).  Such an operand's part of a stage holds the slab's rows
 // of K (64 for fp16, 128 for int8) with the tile's BR (BC) elements each, DMA'd as they lie in
@@ -457,7 +461,7 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
                                               const GemmItem cur_item, const GemmItem nxt_item, const bool have_slabs, int& ring) {
     constexpr bool FUSED = EPI == kEpiDequant, F16 = EPI == kEpiF16;
     constexpr bool PT = (LAY & 1) != 0, QT = (LAY & 2) != 0;
-    static_assert(LAY == 0 || BKB == 128, "transposed operands: 128 bytes of K per slab");
+    static_assert((LAY & 3) == 0 || BKB == 128, "transposed operands: 128 bytes of K per slab");
     constexpr int ESZ_IN = F16 ? 2 : 1;            // bytes per operand element
     using acc_t = std::conditional_t<F16, float4_t, int4_t>;
     constexpr int KS = BKB / 64, CPR = BKB / 16;
@@ -517,6 +521,41 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
         for (int j = 0; j < AC; ++j)
 #pragma unroll
             for (int e = 0; e < 4; ++e) acc[i][j][e] = 0;
+    if constexpr ((LAY & 4) != 0) {
+        const int32_t K1 = nk * BKB, rem = K - K1;
+        if (rem > 0) {
+            const int8_t* Pr = a.P + (int64_t)b * a.strideP + K1;
+            const int8_t* Qr = a.Q + (int64_t)b * a.strideQ + K1;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                if (ks * 64 < rem) {
+                    const int32_t kc = ks * 64 + q * 16;
+                    int4_t rp[AR], rq[AC];
+#pragma unroll
+                    for (int i = 0; i < AR; ++i) {
+                        const int32_t row = min(j0 + wr * TR * 32 + i * 16 + r16, a.n - 1);
+                        rp[i] = int4_t{0, 0, 0, 0};
+                        if (kc < rem) rp[i] = *reinterpret_cast<const int4_t*>(Pr + (int64_t)row * K + kc);
+                    }
+#pragma unroll
+                    for (int j = 0; j < AC; ++j) {
+                        const int32_t col = min(i0 + wc * TC * 32 + j * 16 + r16, a.m - 1);
+                        rq[j] = int4_t{0, 0, 0, 0};
+                        if (kc < rem) rq[j] = *reinterpret_cast<const int4_t*>(Qr + (int64_t)col * K + kc);
+                    }
+#pragma unroll
+                    for (int i = 0; i < AR; ++i)
+#pragma unroll
+                        for (int j = 0; j < AC; ++j) {
+                            if constexpr (F16)
+                                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, rq[j]), __builtin_bit_cast(half8_t, rp[i]), acc[i][j], 0, 0, 0);
+                            else
+                                acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(rq[j], rp[i], acc[i][j], 0, 0, 0);
+                        }
+                }
+            }
+        }
+    }
     // Fragments: all AR of the row operand, and the column operand's in two sets of AC/2 -- a k-step is two
     // passes over the wave's rows, one per half of its columns, and while one set is multiplied the
     // other is read.  A row fragment's register is refilled with the next k-step's right after
@@ -698,7 +737,7 @@ __device__ __forceinline__ bool gemm_dma_tile32(const GemmArgs& a, int8_t* smem,
                                               const GemmItem cur_item, const GemmItem nxt_item, const bool have_slabs, int& ring) {
     constexpr bool FUSED = EPI == kEpiDequant, F16 = EPI == kEpiF16;
     constexpr bool PT = (LAY & 1) != 0, QT = (LAY & 2) != 0;
-    static_assert(LAY == 0 || BKB == 128, "transposed operands: 128 bytes of K per slab");
+    static_assert((LAY & 3) == 0 || BKB == 128, "transposed operands: 128 bytes of K per slab");
     constexpr int ESZ_IN = F16 ? 2 : 1;            // bytes per operand element
     using acc_t = std::conditional_t<F16, float16_tv, int16_tv>;
     constexpr int KS = BKB / 32, CPR = BKB / 16;
@@ -764,6 +803,41 @@ __device__ __forceinline__ bool gemm_dma_tile32(const GemmArgs& a, int8_t* smem,
         for (int j = 0; j < TC; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+    if constexpr ((LAY & 4) != 0) {       // (the depth beyond the last whole slab, as in the 16x16 form)
+        const int32_t K1 = nk * BKB, rem = K - K1;
+        if (rem > 0) {
+            const int8_t* Pr = a.P + (int64_t)b * a.strideP + K1;
+            const int8_t* Qr = a.Q + (int64_t)b * a.strideQ + K1;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                if (ks * 32 < rem) {
+                    const int32_t kc = ks * 32 + lk * 16;
+                    int4_t rp[TR], rq[TC];
+#pragma unroll
+                    for (int i = 0; i < TR; ++i) {
+                        const int32_t row = min(j0 + wr * TR * 32 + i * 32 + lrow, a.n - 1);
+                        rp[i] = int4_t{0, 0, 0, 0};
+                        if (kc < rem) rp[i] = *reinterpret_cast<const int4_t*>(Pr + (int64_t)row * K + kc);
+                    }
+#pragma unroll
+                    for (int j = 0; j < TC; ++j) {
+                        const int32_t col = min(i0 + wc * TC * 32 + j * 32 + lrow, a.m - 1);
+                        rq[j] = int4_t{0, 0, 0, 0};
+                        if (kc < rem) rq[j] = *reinterpret_cast<const int4_t*>(Qr + (int64_t)col * K + kc);
+                    }
+#pragma unroll
+                    for (int i = 0; i < TR; ++i)
+#pragma unroll
+                        for (int j = 0; j < TC; ++j) {
+                            if constexpr (F16)
+                                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, rq[j]), __builtin_bit_cast(half8_t, rp[i]), acc[i][j], 0, 0, 0);
+                            else
+                                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(rq[j], rp[i], acc[i][j], 0, 0, 0);
+                        }
+                }
+            }
+        }
+    }
     int4_t fp[2][TR], fq[2][TC];
     // Transposing reads as in the 16x16 form.  Here a fragment is 32 rows x 16 bytes of K: the wave's four groups of
     // 16 lanes are (rows 0-15 | 16-31) x (first | second half of the k-step's 32 bytes), so a group's block of 16
@@ -1170,6 +1244,14 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
         if (small > cus && small <= 2 * cus) return launch_dma<2, 2, 2, 1, 128, EPI, 2, 0, 32>(a, batch, st, 2);
         return launch_dma<2, 2, 2, 1, 128, EPI, kRingSmall, 0, 32>(a, batch, st);
     }
+    // a depth of whole 16-byte pieces that is not whole 64-byte slabs (4000, 4048 ...): the tile kernels on 64-byte slabs,
+    // the rest of the depth straight from memory into the fragments
+    if (fast && wide && k > 64 && (int64_t)n * k < (1ll << 32) && (int64_t)m * k < (1ll << 32)) {
+        constexpr int EPI = FUSED ? kEpiDequant : kEpiInt32;
+        const int64_t big = ceil_div(n, 256) * ceil_div(m, 256) * batch;
+        if (big * 4 >= compute_units() * 3 && n > 128 && m > 128) return launch_dma<2, 4, 4, 2, 64, EPI, 4, 4, 16>(a, batch, st);
+        return launch_dma<2, 2, 2, 2, 64, EPI, kRingSmall, 4, 32>(a, batch, st);
+    }
     // an operand stored (K, rows): the tile kernel reads it as it lies and takes the fragments with transposing LDS reads
     // (rows of such an operand that are not whole 16-byte pieces: tiles that stay inside the matrix, which takes a matrix of
     // at least one tile)
@@ -1349,6 +1431,14 @@ static int gemm_f16_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, in
         const int64_t mid = ceil_div(n, 128) * ceil_div(m, 128) * batch, cus = compute_units();
         if (mid > cus && mid <= 2 * cus) return launch_dma<2, 2, 2, 2, 128, kEpiF16, 2, 0, 32>(a, batch, st, 2);
         return launch_dma<2, 2, 2, 2, 128, kEpiF16, kRingSmall, 0, 32>(a, batch, st);
+    }
+    // a depth of whole 16-byte pieces that is not whole 64-byte slabs (K = 40, 72, 1000 ...): the same kernels, the rest of
+    // the depth straight from memory into the fragments
+    if (p_kmajor && q_kmajor && wide && k > 32 && (k % 8 == 0) && aligned16(A) && aligned16(B) &&
+        (int64_t)n * k * 2 < (1ll << 32) && (int64_t)m * k * 2 < (1ll << 32)) {
+        const int64_t big = ceil_div(n, 256) * ceil_div(m, 256) * batch;
+        if (big * 4 >= compute_units() * 3 && n > 128 && m > 128) return launch_dma<4, 2, 2, 4, 64, kEpiF16, 2, 4, 32>(a, batch, st);
+        return launch_dma<2, 2, 2, 2, 64, kEpiF16, kRingSmall, 4, 32>(a, batch, st);
     }
     // an operand stored (K, rows): the tile kernel reads it as it lies, with transposing LDS reads for the fragments
     // (rows of such an operand that are not whole 16-byte pieces, but whole 8-byte ones: tiles that stay inside the matrix,

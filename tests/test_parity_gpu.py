@@ -314,6 +314,9 @@ TILE_CASES = [  # (batch, kernel n = output rows, k, kernel m = output columns)
     (1, 8, 128, 8), (1, 4, 256, 260), (2, 2816, 256, 2304), (1, 4096, 256, 3076), (2, 500, 1024, 1996), (1, 2052, 128, 4100),
     # depths of whole 64-byte but not whole 128-byte slabs: large and small tiles, one slab to many
     (1, 4096, 192, 3328), (1, 520, 448, 1032), (2, 132, 64, 72), (1, 2304, 1600, 2064), (3, 260, 320, 516),
+    # depths of whole 16-byte pieces that are not whole slabs (the rest of the depth goes straight into the fragments):
+    # one slab + 16 bytes, + 48 bytes, many slabs, large and small tiles, ragged edges
+    (1, 132, 80, 72), (2, 260, 112, 516), (1, 4096, 208, 3328), (1, 2304, 1008, 2064), (3, 100, 144, 60), (1, 520, 4000, 1032),
 ]
 
 
@@ -992,6 +995,8 @@ F16_GEMM_CASES = [  # (batch, n, k, m) in the kernel's convention: out (batch, n
     (48, 512, 256, 512), (50, 520, 320, 264),
     # depths of whole 64-byte but not whole 128-byte slabs (96, 160, 224 halves): large and small tiles
     (32, 512, 96, 768), (2, 264, 160, 520), (3, 40, 224, 1032),
+    # depths of whole 16-byte pieces (8 halves) that are not whole slabs: one slab + 8 halves, + 24, many slabs, large and small tiles
+    (2, 264, 40, 520), (3, 40, 56, 1032), (32, 512, 72, 768), (2, 300, 1000, 260), (40, 520, 104, 264),
     # rows of a (K, rows) operand that are whole 8-byte but not whole 16-byte pieces (the reference's 500 x 7996 of tests/test_gemm.py:56):
     # edge tiles that stay inside the matrix, small and large tiles, and the 64 x 256 tiles of few output rows
     (2, 500, 128, 1004), (3, 500, 128, 7996), (2, 132, 64, 260), (4, 48, 192, 1004),
