@@ -1292,17 +1292,17 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
 }
 
 // ---------------------------------------------------------------------------------------
-// fp16 product (fp32 accumulation), any layout, size and alignment: 64x64 output tile, 32 halves of K per
+// fp16 product (fp32 accumulation), any layout, size and alignment: 64x64 output tile, 64 halves of K per
 // stage, four waves of one 32x32 MFMA tile each.  Shapes that are whole slabs and pieces run on the tile
 // kernel above instead.
 // ---------------------------------------------------------------------------------------
 // V: halves per global access (4, 2 or 1: what the contiguous dimension of both operands and the alignment of the buffers allow).
 template <int V>
 __global__ __launch_bounds__(256) void k_gemm_f16_generic(GemmArgs a, int p_kmajor, int q_kmajor, int32_t row_base) {
-    // Element-wise guarded loads bring a 64 x 32 piece of each operand into LDS with K contiguous (zeros past the edges,
+    // Guarded loads bring a 64 x 64 piece of each operand into LDS with K contiguous (zeros past the edges,
     // so any size, layout and alignment works); each of the four waves then owns a 32 x 32 quarter of the tile and
     // multiplies with v_mfma_f32_32x32x16_f16.
-    constexpr int T = 64, GK = 32, LD = GK + 4;        // rows of 72 bytes: 8-byte aligned fragment reads, spread over the banks
+    constexpr int T = 64, GK = 64, LD = GK + 4;        // rows of 136 bytes: 8-byte aligned fragment reads, spread over the banks
     __shared__ __attribute__((aligned(16))) half_t sP[T * LD];
     __shared__ __attribute__((aligned(16))) half_t sQ[T * LD];
     const int b = blockIdx.z;
