@@ -4,6 +4,16 @@
 
 namespace cpmk {
 
+// Eight halves of a flat tensor: on 16-byte boundaries with the non-temporal hint (WIDE 1), at any address without it
+// (WIDE 2: global accesses need no alignment).
+__device__ __forceinline__ half8_t flat_load8(const half_t* p, int wide) {
+    return wide == 1 ? __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(p)) : load_half8_any(p);
+}
+__device__ __forceinline__ void flat_store8(half_t* p, half8_t v, int wide) {
+    if (wide == 1) __builtin_nontemporal_store(v, reinterpret_cast<half8_t*>(p));
+    else store_half8_any(p, v);
+}
+
 // cuda/gelu.cu:14 evaluates 0.5 * x * (1 + tanh(c * x * (1 + 0.044715 x^2))), c = sqrt(2/pi), partly in
 // double.  With u = c x (1 + 0.044715 x^2) the same function is x / (1 + exp(-2u)), which needs
 // one exp2 and one reciprocal in fp32 and, unlike 1 + tanh(u), does not cancel for negative x.
@@ -22,10 +32,10 @@ __global__ __launch_bounds__(256) void k_gelu(int64_t total, const half_t* mat, 
     if (vec) {
         const int64_t e0 = gid * 8;
         if (e0 + 8 <= total) {
-            half8_t v = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(mat + e0));
+            half8_t v = flat_load8(mat + e0, vec);
 #pragma unroll
             for (int e = 0; e < 8; ++e) v[e] = gelu1(v[e]);
-            __builtin_nontemporal_store(v, reinterpret_cast<half8_t*>(out + e0));
+            flat_store8(out + e0, v, vec);
         } else {
             for (int64_t i = e0; i < total; ++i) out[i] = gelu1(mat[i]);
         }
@@ -86,9 +96,9 @@ __global__ __launch_bounds__(256) void k_add(int64_t total, const half_t* x, con
     if (vec) {
         const int64_t e0 = gid * 8;
         if (e0 + 8 <= total) {
-            half8_t a = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(x + e0));
-            half8_t b = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(y + e0));
-            __builtin_nontemporal_store(a + b, reinterpret_cast<half8_t*>(out + e0));
+            half8_t a = flat_load8(x + e0, vec);
+            half8_t b = flat_load8(y + e0, vec);
+            flat_store8(out + e0, a + b, vec);
         } else {
             for (int64_t i = e0; i < total; ++i) out[i] = x[i] + y[i];
         }
@@ -110,7 +120,8 @@ __global__ __launch_bounds__(256) void k_mask(int64_t total, int32_t n, int32_t 
         // rows that are not whole 16-byte pieces (m >= 8): the tensor is still one contiguous run, so its elements go
         // eight at a time; the eight may run over the end of a row, and each looks up its own mask byte
         if (e0 + 8 <= total) {
-            half8_t v = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(x + e0));
+            const int wide = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0 ? 1 : 2;
+            half8_t v = flat_load8(x + e0, wide);
             const int8_t* m0 = mask + (row / n) * m + j;                   // this row's mask bytes from column j on
             if (j + 8 <= m) {       // the eight share a row: their mask bytes in one load (global loads need no alignment)
                 const Byte8Any mk = *reinterpret_cast<const Byte8Any*>(m0);
@@ -125,7 +136,7 @@ __global__ __launch_bounds__(256) void k_mask(int64_t total, int32_t n, int32_t 
                 for (int e = 0; e < 8; ++e)
                     if ((j + e < m ? m0 : m1)[e] == 0) v[e] = value;
             }
-            __builtin_nontemporal_store(v, reinterpret_cast<half8_t*>(out + e0));
+            flat_store8(out + e0, v, wide);
         } else {
             for (int64_t i = e0; i < total; ++i) {
                 const int64_t r2 = i / m;
@@ -158,8 +169,8 @@ int cpmk_gelu_forward(int32_t batch, int32_t n, const void* mat, void* out, void
     const int64_t total = (int64_t)batch * n;
     if (total == 0) return 0;
     if (any_null(mat, out)) return CPMK_EBADARG;
-    const int vec = aligned16(mat) && aligned16(out);
-    const int64_t g = ceil_div(vec ? ceil_div(total, 8) : total, 256);
+    const int vec = aligned16(mat) && aligned16(out) ? 1 : 2;       // (2: buffers off 16-byte boundaries)
+    const int64_t g = ceil_div(ceil_div(total, 8), 256);
     hipLaunchKernelGGL(k_gelu, dim3((unsigned)g), dim3(256), 0, (hipStream_t)stream, total, (const half_t*)mat,
                        (half_t*)out, vec);
     return launch_status();
@@ -203,8 +214,8 @@ int cpmk_arith_element_add(int32_t batch, int32_t n, const void* x, const void* 
     const int64_t total = (int64_t)batch * n;
     if (total == 0) return 0;
     if (any_null(x, y, out)) return CPMK_EBADARG;
-    const int vec = aligned16(x) && aligned16(y) && aligned16(out);
-    const int64_t g = ceil_div(vec ? ceil_div(total, 8) : total, 256);
+    const int vec = aligned16(x) && aligned16(y) && aligned16(out) ? 1 : 2;       // (2: buffers off 16-byte boundaries)
+    const int64_t g = ceil_div(ceil_div(total, 8), 256);
     hipLaunchKernelGGL(k_add, dim3((unsigned)g), dim3(256), 0, (hipStream_t)stream, total, (const half_t*)x,
                        (const half_t*)y, (half_t*)out, vec);
     return launch_status();
@@ -218,7 +229,7 @@ int cpmk_mask(int32_t batch, int32_t n, int32_t m, const void* inp, const void* 
     if (total == 0) return 0;
     if (any_null(inp, mask, out)) return CPMK_EBADARG;
     int vec = (m % 8 == 0) && aligned16(inp) && aligned16(out) && ((reinterpret_cast<uintptr_t>(mask) & 7u) == 0);
-    if (!vec && m >= 8 && aligned16(inp) && aligned16(out)) vec = 2;
+    if (!vec && m >= 8) vec = 2;
     const int64_t g = ceil_div(vec ? ceil_div(total, 8) : total, 256);
     hipLaunchKernelGGL(k_mask, dim3((unsigned)g), dim3(256), 0, (hipStream_t)stream, total, n, m, (const half_t*)inp,
                        (const int8_t*)mask, (half_t)value, (half_t*)out, vec);
