@@ -3,7 +3,10 @@ Pointers that are only 4-byte aligned: torch hands out 256-byte aligned tensors,
 view into a larger buffer need not be, and the reference asks for nothing beyond the alignment of
 its half2 / char4 accesses.  Every 16-byte fast path must step aside for such pointers: each
 function is run on aligned tensors and again with every operand moved 4 bytes off, and the two
-results must agree (to the bit for the exact kernels)."""
+results must agree (to the bit for the exact kernels).  The dim-1 and elementwise kernels are also run
+on buffers that start on an odd element (2 bytes off), which they take as well."""
+import sys
+
 import numpy as np
 import pytest
 import torch
@@ -18,13 +21,16 @@ def _name(*a):
     print("case", *a, flush=True)
 
 
+SHIFT_BYTES = 4
+
+
 def shifted(t):
-    """The same values at an address 4 bytes past a 256-byte boundary."""
-    e = 4 // t.element_size()
+    """The same values at an address SHIFT_BYTES (4 unless a test says otherwise) past a 256-byte boundary."""
+    e = max(1, SHIFT_BYTES // t.element_size())
     buf = torch.empty(t.numel() + 64, dtype=t.dtype, device=t.device)
     v = buf[e:e + t.numel()].view(t.shape)
     v.copy_(t)
-    assert v.data_ptr() % 16 == 4
+    assert v.data_ptr() % 16 == e * t.element_size()
     return v
 
 
@@ -72,9 +78,13 @@ def test_quantised_gemm_path_unaligned(gpu):
          exact=False, what="gemv_broadcast_mat_fp16")
 
 
-@pytest.mark.parametrize("shape", [(3, 512, 128), (2, 2048, 64), (4, 100, 72)])
-def test_dim1_and_elementwise_unaligned(gpu, shape):
-    _name("layernorm / softmax / elementwise, 4-byte aligned pointers", shape)
+# (shift 2: buffers that start on an odd element, which the reference's half2 kernels would not take; the kernels here
+# move their 16-byte pieces at any address)
+@pytest.mark.parametrize("shift", [4, 2])
+@pytest.mark.parametrize("shape", [(3, 512, 128), (2, 2048, 64), (4, 100, 72), (2, 600, 250)])
+def test_dim1_and_elementwise_unaligned(gpu, shape, shift, monkeypatch):
+    _name("layernorm / softmax / elementwise, pointers off 16-byte boundaries", shape, shift)
+    monkeypatch.setattr(sys.modules[__name__], "SHIFT_BYTES", shift)
     b, n, m = shape
     g = torch.Generator().manual_seed(32 + n)
     x = (torch.randn(b, n, m, generator=g) * 2).half().to(gpu)
