@@ -447,10 +447,10 @@ struct StripOut {
 // lets the compiler keep the accumulators in place and the MFMA/memory interleave as written.
 // Returns true if the next tile's first slabs are on their way.
 //
-// LAY bit 2 (K-major operands only): the depth is whole 16-byte pieces but not whole slabs.  The slabs of the ring cover
-// the whole ones; the rest of every row (less than a slab) goes from memory straight into the fragment registers
-// before the K loop starts -- a lane's 16 bytes of a k-step are the same bytes in memory as in the stage -- with zeros
-// past the end of K.
+// LAY bit 2: the depth is not whole slabs (any multiple of 4 bytes).  The slabs of the ring cover the whole ones; the
+// rest of the depth (less than a slab) goes from memory straight into the fragment registers before the K loop starts
+// -- a lane's 16 bytes of a k-step are the same bytes in memory as in the stage -- with zeros past the end of K.  (An
+// operand stored (K, rows) beside it: the 32x32 form only, which gathers such a fragment element by element.)
 // LAY marks operands whose rows are K instead: bit 0 = the row operand is stored (K, n), bit 1 =
 // the column operand is stored (K, m).  Such an operand's part of a stage holds the slab's rows
 // of K (64 for fp16, 128 for int8) with the tile's BR (BC) elements each, DMA'd as they lie in
@@ -526,23 +526,30 @@ __device__ __forceinline__ bool gemm_dma_tile(const GemmArgs& a, int8_t* smem, i
         if (rem > 0) {
             const int8_t* Pr = a.P + (int64_t)b * a.strideP + K1;
             const int8_t* Qr = a.Q + (int64_t)b * a.strideQ + K1;
+            // bytes [kc, kc + 16) of the rest of a row, zeros from byte `rem` on: the piece may start at any address and
+            // end inside (rows of K that are whole dwords, not whole 16-byte pieces)
+            struct __attribute__((packed, aligned(1))) Piece16 { uint32_t x, y, z, w; };
+            // (without branches -- a load under a condition would be waited for before the next one is issued: the 16 bytes
+            // that end where the piece or K ends, moved down by the dwords that lie beyond K)
+            auto piece = [&](const int8_t* rest, int32_t kc) __attribute__((always_inline)) {
+                const int32_t over = min(max(kc + 16 - rem, 0), 16);        // bytes of the piece beyond K: 0, 4 ... 16
+                const Piece16 t = *reinterpret_cast<const Piece16*>(rest + min(kc - over, rem - 16));       // (inside the row: at least one slab precedes `rest`)
+                const int32_t w[8] = {(int32_t)t.x, (int32_t)t.y, (int32_t)t.z, (int32_t)t.w, 0, 0, 0, 0};
+                const int sh = over >> 2;
+                int4_t v;
+#pragma unroll
+                for (int d = 0; d < 4; ++d) v[d] = sh == 0 ? w[d] : sh == 1 ? w[d + 1] : sh == 2 ? w[d + 2] : sh == 3 ? w[d + 3] : 0;
+                return v;
+            };
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 if (ks * 64 < rem) {
                     const int32_t kc = ks * 64 + q * 16;
                     int4_t rp[AR], rq[AC];
 #pragma unroll
-                    for (int i = 0; i < AR; ++i) {
-                        const int32_t row = min(j0 + wr * TR * 32 + i * 16 + r16, a.n - 1);
-                        rp[i] = int4_t{0, 0, 0, 0};
-                        if (kc < rem) rp[i] = *reinterpret_cast<const int4_t*>(Pr + (int64_t)row * K + kc);
-                    }
+                    for (int i = 0; i < AR; ++i) rp[i] = piece(Pr + (int64_t)min(j0 + wr * TR * 32 + i * 16 + r16, a.n - 1) * K, kc);
 #pragma unroll
-                    for (int j = 0; j < AC; ++j) {
-                        const int32_t col = min(i0 + wc * TC * 32 + j * 16 + r16, a.m - 1);
-                        rq[j] = int4_t{0, 0, 0, 0};
-                        if (kc < rem) rq[j] = *reinterpret_cast<const int4_t*>(Qr + (int64_t)col * K + kc);
-                    }
+                    for (int j = 0; j < AC; ++j) rq[j] = piece(Qr + (int64_t)min(i0 + wc * TC * 32 + j * 16 + r16, a.m - 1) * K, kc);
 #pragma unroll
                     for (int i = 0; i < AR; ++i)
 #pragma unroll
@@ -803,36 +810,86 @@ __device__ __forceinline__ bool gemm_dma_tile32(const GemmArgs& a, int8_t* smem,
         for (int j = 0; j < TC; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
-    if constexpr ((LAY & 4) != 0) {       // (the depth beyond the last whole slab, as in the 16x16 form)
-        const int32_t K1 = nk * BKB, rem = K - K1;
+    if constexpr ((LAY & 4) != 0) {
+        // The depth beyond the last whole slab, as in the 16x16 form.  Here either operand may also be stored (K, rows): its
+        // fragment -- a lane's 8 (fp16) or 16 (int8) consecutive values of K for its own row -- is then gathered element
+        // by element, adjacent lanes reading adjacent elements of a row of K.  K-major pieces may start at any address
+        // and end inside the piece (rows of K that are whole dwords, not whole 16-byte pieces).
+        const int32_t K1 = nk * BKB, rem = K - K1;           // bytes
         if (rem > 0) {
-            const int8_t* Pr = a.P + (int64_t)b * a.strideP + K1;
-            const int8_t* Qr = a.Q + (int64_t)b * a.strideQ + K1;
+            constexpr int EPP = 16 / ESZ_IN;
+            struct __attribute__((packed, aligned(1))) Piece16 { uint32_t x, y, z, w; };
+            const int8_t* Pr = a.P + (int64_t)b * a.strideP;
+            const int8_t* Qr = a.Q + (int64_t)b * a.strideQ;
+            // a K-major operand's piece: bytes [kc, kc + 16) of the rest of row `row`, zeros from byte `rem` on
+            // (both without branches -- a load under a condition would be waited for before the next one is issued.  The
+            // piece: the 16 bytes that end where the piece or K ends, moved down by the dwords that lie beyond K.)
+            auto piece = [&](const int8_t* base, int32_t row, int32_t kc) __attribute__((always_inline)) {
+                const int32_t over = min(max(kc + 16 - rem, 0), 16);        // bytes of the piece beyond K: 0, 4 ... 16
+                const Piece16 t = *reinterpret_cast<const Piece16*>(base + (int64_t)row * K + K1 + min(kc - over, rem - 16));      // (inside the row: at least one slab precedes)
+                const int32_t w[8] = {(int32_t)t.x, (int32_t)t.y, (int32_t)t.z, (int32_t)t.w, 0, 0, 0, 0};
+                const int sh = over >> 2;
+                int4_t v;
+#pragma unroll
+                for (int d = 0; d < 4; ++d) v[d] = sh == 0 ? w[d] : sh == 1 ? w[d + 1] : sh == 2 ? w[d + 2] : sh == 3 ? w[d + 3] : 0;
+                return v;
+            };
+            // a (K, L) operand's piece: elements [ke, ke + EPP) of the rest of K for element `row` of the rows of K
+            auto gather = [&](const int8_t* base, int32_t L, int32_t row, int32_t ke) __attribute__((always_inline)) {
+                const int32_t kel0 = K1 / ESZ_IN, krem = rem / ESZ_IN;
+                if constexpr (F16) {
+                    half8_t h;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const half_t x = reinterpret_cast<const half_t*>(base)[(int64_t)(kel0 + min(ke + e, krem - 1)) * L + row];
+                        h[e] = ke + e < krem ? x : (half_t)0.0f;
+                    }
+                    return __builtin_bit_cast(int4_t, h);
+                } else {
+                    int4_t v = {0, 0, 0, 0};
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const uint32_t x = (uint8_t)base[(int64_t)(kel0 + min(ke + e, krem - 1)) * L + row];
+                        v[e >> 2] |= (int32_t)((ke + e < krem ? x : 0u) << (8 * (e & 3)));
+                    }
+                    return v;
+                }
+            };
+            // every k-step's pieces are requested before the first product: one trip to memory, not one per k-step
+            int4_t rp[KS][TR], rq[KS][TC];
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const int32_t kc = ks * 32 + lk * 16;
+#pragma unroll
+                for (int i = 0; i < TR; ++i) {
+                    const int32_t row = min(j0 + wr * TR * 32 + i * 32 + lrow, a.n - 1);
+                    rp[ks][i] = int4_t{0, 0, 0, 0};
+                    if (ks * 32 < rem) {
+                        if constexpr (PT) rp[ks][i] = gather(Pr, a.n, row, kc / ESZ_IN);
+                        else rp[ks][i] = piece(Pr, row, kc);
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < TC; ++j) {
+                    const int32_t col = min(i0 + wc * TC * 32 + j * 32 + lrow, a.m - 1);
+                    rq[ks][j] = int4_t{0, 0, 0, 0};
+                    if (ks * 32 < rem) {
+                        if constexpr (QT) rq[ks][j] = gather(Qr, a.m, col, kc / ESZ_IN);
+                        else rq[ks][j] = piece(Qr, col, kc);
+                    }
+                }
+            }
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 if (ks * 32 < rem) {
-                    const int32_t kc = ks * 32 + lk * 16;
-                    int4_t rp[TR], rq[TC];
-#pragma unroll
-                    for (int i = 0; i < TR; ++i) {
-                        const int32_t row = min(j0 + wr * TR * 32 + i * 32 + lrow, a.n - 1);
-                        rp[i] = int4_t{0, 0, 0, 0};
-                        if (kc < rem) rp[i] = *reinterpret_cast<const int4_t*>(Pr + (int64_t)row * K + kc);
-                    }
-#pragma unroll
-                    for (int j = 0; j < TC; ++j) {
-                        const int32_t col = min(i0 + wc * TC * 32 + j * 32 + lrow, a.m - 1);
-                        rq[j] = int4_t{0, 0, 0, 0};
-                        if (kc < rem) rq[j] = *reinterpret_cast<const int4_t*>(Qr + (int64_t)col * K + kc);
-                    }
 #pragma unroll
                     for (int i = 0; i < TR; ++i)
 #pragma unroll
                         for (int j = 0; j < TC; ++j) {
                             if constexpr (F16)
-                                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, rq[j]), __builtin_bit_cast(half8_t, rp[i]), acc[i][j], 0, 0, 0);
+                                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, rq[ks][j]), __builtin_bit_cast(half8_t, rp[ks][i]), acc[i][j], 0, 0, 0);
                             else
-                                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(rq[j], rp[i], acc[i][j], 0, 0, 0);
+                                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(rq[ks][j], rp[ks][i], acc[i][j], 0, 0, 0);
                         }
                 }
             }
@@ -1244,9 +1301,10 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
         if (small > cus && small <= 2 * cus) return launch_dma<2, 2, 2, 1, 128, EPI, 2, 0, 32>(a, batch, st, 2);
         return launch_dma<2, 2, 2, 1, 128, EPI, kRingSmall, 0, 32>(a, batch, st);
     }
-    // a depth of whole 16-byte pieces that is not whole 64-byte slabs (4000, 4048 ...): the tile kernels on 64-byte slabs,
-    // the rest of the depth straight from memory into the fragments
-    if (fast && wide && k > 64 && (int64_t)n * k < (1ll << 32) && (int64_t)m * k < (1ll << 32)) {
+    // a depth that is not whole 64-byte slabs (4000, 4048, 4100 ...): the tile kernels on 64-byte slabs, the rest of the
+    // depth straight from memory into the fragments (k % 4 == 0 is the reference's precondition: rows of whole dwords)
+    if (p_kmajor && q_kmajor && wide && k > 64 && (k % 4 == 0) && (reinterpret_cast<uintptr_t>(A) & 3u) == 0 &&
+        (reinterpret_cast<uintptr_t>(B) & 3u) == 0 && (int64_t)n * k < (1ll << 32) && (int64_t)m * k < (1ll << 32)) {
         constexpr int EPI = FUSED ? kEpiDequant : kEpiInt32;
         const int64_t big = ceil_div(n, 256) * ceil_div(m, 256) * batch;
         if (big * 4 >= compute_units() * 3 && n > 128 && m > 128) return launch_dma<2, 4, 4, 2, 64, EPI, 4, 4, 16>(a, batch, st);
@@ -1432,9 +1490,9 @@ static int gemm_f16_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, in
         if (mid > cus && mid <= 2 * cus) return launch_dma<2, 2, 2, 2, 128, kEpiF16, 2, 0, 32>(a, batch, st, 2);
         return launch_dma<2, 2, 2, 2, 128, kEpiF16, kRingSmall, 0, 32>(a, batch, st);
     }
-    // a depth of whole 16-byte pieces that is not whole 64-byte slabs (K = 40, 72, 1000 ...): the same kernels, the rest of
-    // the depth straight from memory into the fragments
-    if (p_kmajor && q_kmajor && wide && k > 32 && (k % 8 == 0) && aligned16(A) && aligned16(B) &&
+    // a depth that is not whole 64-byte slabs (K = 40, 72, 500, 1000 ...): the same kernels, the rest of the depth straight
+    // from memory into the fragments
+    if (p_kmajor && q_kmajor && wide && k > 32 && (reinterpret_cast<uintptr_t>(A) & 3u) == 0 && (reinterpret_cast<uintptr_t>(B) & 3u) == 0 &&
         (int64_t)n * k * 2 < (1ll << 32) && (int64_t)m * k * 2 < (1ll << 32)) {
         const int64_t big = ceil_div(n, 256) * ceil_div(m, 256) * batch;
         if (big * 4 >= compute_units() * 3 && n > 128 && m > 128) return launch_dma<4, 2, 2, 4, 64, kEpiF16, 2, 4, 32>(a, batch, st);
@@ -1464,6 +1522,15 @@ static int gemm_f16_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, in
                 if (low) return launch_dma<1, 4, 2, 2, 128, kEpiF16, 3, 3, 32>(a, batch, st);
                 return large ? launch_dma<2, 4, 4, 2, 128, kEpiF16, 2, 3, 16>(a, batch, st) : launch_dma<2, 2, 2, 2, 128, kEpiF16, kRingSmall, 3, 32>(a, batch, st);
         }
+    }
+    // one operand stored (K, rows) and a depth that is not whole slabs (attention: probabilities x values over 500 keys):
+    // the 32x32 form of the tile kernel, the rest of the depth straight from memory into the fragments
+    if (p_kmajor != q_kmajor && wide && k > 64 && (k % 64 != 0) && aligned16(A) && aligned16(B) &&
+        (!in_p || (n % 4 == 0 && n >= 128)) && (!in_q || (m % 4 == 0 && m >= (low ? 256 : 128))) &&
+        (int64_t)n * k * 2 < (1ll << 32) && (int64_t)m * k * 2 < (1ll << 32)) {
+        a.edge_in = (in_p ? 1 : 0) | (in_q ? 2 : 0);
+        if (!p_kmajor) return low ? launch_dma<1, 4, 2, 2, 128, kEpiF16, 3, 5, 32>(a, batch, st) : launch_dma<2, 2, 2, 2, 128, kEpiF16, kRingSmall, 5, 32>(a, batch, st);
+        return low ? launch_dma<1, 4, 2, 2, 128, kEpiF16, 3, 6, 32>(a, batch, st) : launch_dma<2, 2, 2, 2, 128, kEpiF16, kRingSmall, 6, 32>(a, batch, st);
     }
     for (int64_t r0 = 0; r0 < n; r0 += 65535ll * 64) {        // (rows beyond the grid's y dimension: several launches)
         const int64_t nr = n - r0 < 65535ll * 64 ? n - r0 : 65535ll * 64;

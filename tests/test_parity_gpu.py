@@ -317,6 +317,8 @@ TILE_CASES = [  # (batch, kernel n = output rows, k, kernel m = output columns)
     # depths of whole 16-byte pieces that are not whole slabs (the rest of the depth goes straight into the fragments):
     # one slab + 16 bytes, + 48 bytes, many slabs, large and small tiles, ragged edges
     (1, 132, 80, 72), (2, 260, 112, 516), (1, 4096, 208, 3328), (1, 2304, 1008, 2064), (3, 100, 144, 60), (1, 520, 4000, 1032),
+    # ... and depths of whole dwords only (rows that start 4, 8 or 12 bytes into a 16-byte piece)
+    (1, 520, 4100, 1032), (2, 260, 100, 516), (1, 4096, 212, 3328), (3, 132, 72, 72), (1, 300, 1000, 260),
 ]
 
 
@@ -997,6 +999,8 @@ F16_GEMM_CASES = [  # (batch, n, k, m) in the kernel's convention: out (batch, n
     (32, 512, 96, 768), (2, 264, 160, 520), (3, 40, 224, 1032),
     # depths of whole 16-byte pieces (8 halves) that are not whole slabs: one slab + 8 halves, + 24, many slabs, large and small tiles
     (2, 264, 40, 520), (3, 40, 56, 1032), (32, 512, 72, 768), (2, 300, 1000, 260), (40, 520, 104, 264),
+    # any even depth beyond a slab, also beside an operand stored (K, rows) (probabilities x values over 500 keys: few and many output rows)
+    (4, 64, 500, 500), (2, 132, 200, 260), (3, 40, 100, 1004), (2, 264, 250, 520), (2, 48, 66, 264), (3, 300, 130, 136),
     # rows of a (K, rows) operand that are whole 8-byte but not whole 16-byte pieces (the reference's 500 x 7996 of tests/test_gemm.py:56):
     # edge tiles that stay inside the matrix, small and large tiles, and the 64 x 256 tiles of few output rows
     (2, 500, 128, 1004), (3, 500, 128, 7996), (2, 132, 64, 260), (4, 48, 192, 1004),
