@@ -32,8 +32,9 @@ def _gemm_shapes(seed, count):
             k = 128 * int(rng.integers(1, 9))
             n = _near(rng, [64, 128, 256, 512, 768], 40, lo=4, step=4)
             m = _near(rng, [64, 128, 256, 512, 1024], 40, lo=4, step=int(rng.choice([4, 8])))
-        elif kind == 2:     # register-staged kernel: k % 16 == 0 but not % 128
-            k = 16 * int(rng.integers(1, 40))
+        elif kind == 2:     # depths that are not whole slabs: whole 16-byte pieces, or whole dwords only (under one slab: the
+                            # register-staged kernel; beyond: the tile kernels, the rest of the depth straight into the fragments)
+            k = int(rng.choice([16, 4])) * int(rng.integers(1, 40))
             n = _near(rng, [32, 128, 300], 30, lo=4, step=4)
             m = _near(rng, [32, 128, 300], 30, lo=4, step=4)
         else:               # stored (K, rows) layouts on the tile kernel: rows in whole 16-byte pieces
@@ -116,9 +117,14 @@ def _f16_gemm_shapes(seed, count):
     rng = np.random.default_rng(seed)
     out = []
     for _ in range(count):
-        kind = int(rng.integers(0, 3))
+        kind = int(rng.integers(0, 4))
         if kind == 0:       # even sizes only (kernels/gemm.py:200): the generic kernel
             n, k, m = (2 * int(rng.integers(1, 80)) for _ in range(3))
+        elif kind == 3:     # any even depth beyond a slab on the tile kernels (the rest of the depth straight into the fragments),
+                            # output rows of whole 8-byte pieces
+            k = 2 * int(rng.integers(17, 300))
+            n = _near(rng, [24, 64, 136, 264, 520], 24, lo=8, step=int(rng.choice([4, 8])))
+            m = _near(rng, [64, 256, 520], 24, lo=8, step=int(rng.choice([4, 8])))
         elif kind == 1:     # tile kernel: k % 64 == 0, output rows of whole 16-byte pieces
             k = 64 * int(rng.integers(1, 8))
             n = _near(rng, [24, 64, 136, 264, 520], 24, lo=8, step=8)
