@@ -1327,6 +1327,15 @@ static int gemm_dispatch(int32_t m, int32_t k, int32_t n, int32_t batchA, int32_
             default: return large ? launch_dma<2, 4, 4, 2, 128, EPI, 2, 3, 16>(a, batch, st) : launch_dma<2, 2, 2, 2, 128, EPI, kRingSmall, 3, 32>(a, batch, st);
         }
     }
+    // one operand stored (K, rows) and a depth beyond one slab that is not whole slabs: the 32x32 form of the tile kernel,
+    // the rest of the depth straight from memory into the fragments
+    if (p_kmajor != q_kmajor && wide && k > 128 && (k % 4 == 0) && aligned16(A) && aligned16(B) && (!in_p || n >= 128) &&
+        (!in_q || m >= 128) && (int64_t)n * k < (1ll << 32) && (int64_t)m * k < (1ll << 32)) {
+        constexpr int EPI = FUSED ? kEpiDequant : kEpiInt32;
+        a.edge_in = (in_p ? 1 : 0) | (in_q ? 2 : 0);
+        if (!p_kmajor) return launch_dma<2, 2, 2, 2, 128, EPI, kRingSmall, 5, 32>(a, batch, st);
+        return launch_dma<2, 2, 2, 2, 128, EPI, kRingSmall, 6, 32>(a, batch, st);
+    }
     if (fast) {
         const int64_t t256 = ceil_div(n, 256) * ceil_div(m, 128) * batch;
         if (t256 >= 256) return launch_kmajor<2, 2, 4, 2, FUSED>(a, batch, st);

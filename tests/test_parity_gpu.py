@@ -337,7 +337,9 @@ def test_gemm_int8_tile_kernels(gpu, case):
 LAYOUT_CASES = [(1, 512, 256, 768), (2, 272, 128, 528), (1, 48, 384, 1040), (3, 1040, 640, 16), (1, 2304, 1024, 2064), (2, 2048, 256, 2560),
                 (1, 4096, 256, 3088), (2, 3072, 128, 2064),
                 # rows of a (K, rows) operand that are not whole 16-byte pieces (edge tiles that stay inside the matrix): small and large tiles
-                (1, 500, 256, 1004), (3, 500, 128, 7996), (2, 132, 128, 260)]
+                (1, 500, 256, 1004), (3, 500, 128, 7996), (2, 132, 128, 260),
+                # one operand stored (K, rows) and a depth beyond a slab that is not whole slabs (whole 16-byte pieces, whole dwords only)
+                (1, 512, 200, 768), (2, 272, 500, 528), (1, 500, 132, 1004), (2, 132, 1000, 260)]
 
 
 @pytest.mark.parametrize("case", LAYOUT_CASES)
