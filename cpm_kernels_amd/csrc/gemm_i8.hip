@@ -855,42 +855,55 @@ __device__ __forceinline__ bool gemm_dma_tile32(const GemmArgs& a, int8_t* smem,
                     return v;
                 }
             };
-            // every k-step's pieces are requested before the first product: one trip to memory, not one per k-step
-            int4_t rp[KS][TR], rq[KS][TC];
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
+            auto load_ks = [&](int4_t (&rp)[TR], int4_t (&rq)[TC], int ks) __attribute__((always_inline)) {
                 const int32_t kc = ks * 32 + lk * 16;
 #pragma unroll
                 for (int i = 0; i < TR; ++i) {
                     const int32_t row = min(j0 + wr * TR * 32 + i * 32 + lrow, a.n - 1);
-                    rp[ks][i] = int4_t{0, 0, 0, 0};
+                    rp[i] = int4_t{0, 0, 0, 0};
                     if (ks * 32 < rem) {
-                        if constexpr (PT) rp[ks][i] = gather(Pr, a.n, row, kc / ESZ_IN);
-                        else rp[ks][i] = piece(Pr, row, kc);
+                        if constexpr (PT) rp[i] = gather(Pr, a.n, row, kc / ESZ_IN);
+                        else rp[i] = piece(Pr, row, kc);
                     }
                 }
 #pragma unroll
                 for (int j = 0; j < TC; ++j) {
                     const int32_t col = min(i0 + wc * TC * 32 + j * 32 + lrow, a.m - 1);
-                    rq[ks][j] = int4_t{0, 0, 0, 0};
+                    rq[j] = int4_t{0, 0, 0, 0};
                     if (ks * 32 < rem) {
-                        if constexpr (QT) rq[ks][j] = gather(Qr, a.m, col, kc / ESZ_IN);
-                        else rq[ks][j] = piece(Qr, col, kc);
+                        if constexpr (QT) rq[j] = gather(Qr, a.m, col, kc / ESZ_IN);
+                        else rq[j] = piece(Qr, col, kc);
                     }
                 }
-            }
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
+            };
+            auto mac_ks = [&](const int4_t (&rp)[TR], const int4_t (&rq)[TC], int ks) __attribute__((always_inline)) {
                 if (ks * 32 < rem) {
 #pragma unroll
                     for (int i = 0; i < TR; ++i)
 #pragma unroll
                         for (int j = 0; j < TC; ++j) {
                             if constexpr (F16)
-                                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, rq[ks][j]), __builtin_bit_cast(half8_t, rp[ks][i]), acc[i][j], 0, 0, 0);
+                                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, rq[j]), __builtin_bit_cast(half8_t, rp[i]), acc[i][j], 0, 0, 0);
                             else
-                                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(rq[ks][j], rp[ks][i], acc[i][j], 0, 0, 0);
+                                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(rq[j], rp[i], acc[i][j], 0, 0, 0);
                         }
+                }
+            };
+            if constexpr (PT || QT) {
+                // gathered fragments are many small loads: every k-step's are requested before the first product -- one trip
+                // to memory, not one per k-step
+                int4_t rp[KS][TR], rq[KS][TC];
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) load_ks(rp[ks], rq[ks], ks);
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) mac_ks(rp[ks], rq[ks], ks);
+            } else {
+                // (K-major operands only: a k-step at a time, which keeps the wide accumulator tiles of this form in registers)
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    int4_t rp[TR], rq[TC];
+                    load_ks(rp, rq, ks);
+                    mac_ks(rp, rq, ks);
                 }
             }
         }
